@@ -1,0 +1,132 @@
+// Dense fp32 GEMM for gfx950:  C[m,n] = alpha * op(A) * op(B) + beta * C, row-major.
+//
+// The mean-field path only has tall-and-skinny products (m = nodes or graphs,
+// n and k = label types / hidden sizes <= 256), which are HBM-bound: every A
+// element is used n times from LDS, every B element lives in L2.  The kernel is
+// a classic LDS-tiled register-blocked SGEMM: a 64 x 64 output tile per 256-lane
+// workgroup, 4 x 4 outputs per lane, K walked in steps of 16 through two LDS
+// tiles.  Edges are handled by bounds-checked tile loads (zeros) and stores.
+// Bound: HBM for the shapes above; algorithmic bytes 4(mk + kn + mn).
+#include "gnnhip_internal.h"
+
+namespace gnnhip {
+namespace {
+
+constexpr int BM = 64, BN = 64, BK = 16, kBlock = 256;
+
+template <bool TA, bool TB>
+__global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
+    int m, int n, int k, float alpha, const float* __restrict__ A, int lda,
+    const float* __restrict__ B, int ldb, float beta, float* C, int ldc)
+{
+    __shared__ float As[BK][BM + 4];     // As[p][i] = op(A)[row0 + i][k0 + p]
+    __shared__ float Bs[BK][BN + 4];     // Bs[p][j] = op(B)[k0 + p][col0 + j]
+
+    const int tid = threadIdx.x;
+    const int tx = tid & 15;             // output columns tx*4 .. tx*4+3
+    const int ty = tid >> 4;             // output rows    ty*4 .. ty*4+3
+    const long long row0 = (long long)blockIdx.x * BM;
+    const int col0 = blockIdx.y * BN;
+
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+    for (int k0 = 0; k0 < k; k0 += BK) {
+        // each lane loads 4 elements of each tile
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int idx = tid + e * kBlock;        // 0 .. 1023
+            {
+                // A tile: choose the fast index to follow memory
+                int i, p;
+                if (TA) { i = idx & (BM - 1); p = idx >> 6; }       // stored A is [k][m]: i contiguous
+                else    { p = idx & (BK - 1); i = idx >> 4; }       // stored A is [m][k]: p contiguous
+                const long long gi = row0 + i;
+                const int gp = k0 + p;
+                float v = 0.f;
+                if (gi < m && gp < k) v = TA ? A[(size_t)gp * lda + gi] : A[(size_t)gi * lda + gp];
+                As[p][i] = v;
+            }
+            {
+                int j, p;
+                if (TB) { p = idx & (BK - 1); j = idx >> 4; }       // stored B is [n][k]: p contiguous
+                else    { j = idx & (BN - 1); p = idx >> 6; }       // stored B is [k][n]: j contiguous
+                const int gj = col0 + j;
+                const int gp = k0 + p;
+                float v = 0.f;
+                if (gj < n && gp < k) v = TB ? B[(size_t)gj * ldb + gp] : B[(size_t)gp * ldb + gj];
+                Bs[p][j] = v;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int p = 0; p < BK; ++p) {
+            const float4 a = *reinterpret_cast<const float4*>(&As[p][ty * 4]);
+            const float4 b = *reinterpret_cast<const float4*>(&Bs[p][tx * 4]);
+            const float av[4] = {a.x, a.y, a.z, a.w};
+            const float bv[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * bv[j];
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const long long gi = row0 + ty * 4 + i;
+        if (gi >= m) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int gj = col0 + tx * 4 + j;
+            if (gj >= n) continue;
+            float* dst = C + (size_t)gi * ldc + gj;
+            const float r = alpha * acc[i][j];
+            *dst = (beta == 0.f) ? r : r + beta * (*dst);
+        }
+    }
+}
+
+}  // namespace
+
+int gemm_dispatch(int transA, int transB, int m, int n, int k, float alpha, const float* A, int lda,
+                  const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s)
+{
+    dim3 grid(ceil_div_u((size_t)m, BM), ceil_div_u((size_t)n, BN));
+    dim3 block(kBlock);
+    if (!transA && !transB)
+        hipLaunchKernelGGL((sgemm_tile_kernel<false, false>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+    else if (transA && !transB)
+        hipLaunchKernelGGL((sgemm_tile_kernel<true, false>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+    else if (!transA && transB)
+        hipLaunchKernelGGL((sgemm_tile_kernel<false, true>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+    else
+        hipLaunchKernelGGL((sgemm_tile_kernel<true, true>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+    GNNHIP_LAUNCH_CHECK("sgemm_tile");
+    return GNNHIP_OK;
+}
+
+}  // namespace gnnhip
+
+using namespace gnnhip;
+
+extern "C" int gnnhip_gemm_f32(int transA, int transB, int m, int n, int k, float alpha, const float* A, int lda,
+                               const float* B, int ldb, float beta, float* C, int ldc, void* stream)
+{
+    GNNHIP_REQUIRE(m >= 0 && n >= 0 && k >= 0, "negative dimension in gemm (m=%d n=%d k=%d)", m, n, k);
+    GNNHIP_REQUIRE((transA == 0 || transA == 1) && (transB == 0 || transB == 1), "trans flags must be 0 or 1");
+    if (m == 0 || n == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(C != nullptr && ldc >= n, "bad output in gemm (ldc=%d n=%d)", ldc, n);
+    if (k > 0) {
+        GNNHIP_REQUIRE(A && B, "null operand in gemm");
+        GNNHIP_REQUIRE(lda >= (transA ? m : k), "lda=%d too small", lda);
+        GNNHIP_REQUIRE(ldb >= (transB ? k : n), "ldb=%d too small", ldb);
+    }
+    GNNHIP_REQUIRE(ceil_div_u((size_t)n, 64) <= 65535u, "n=%d too wide for the gemm grid", n);
+    if (int rc = require_ready()) return rc;
+    return gemm_dispatch(transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, as_stream(stream));
+}

@@ -1,0 +1,136 @@
+// Internal helpers shared by the gfx950 kernels: status handling, launch
+// geometry and wave64 reduction primitives (DPP inside a 16-lane row, then two
+// cross-row exchanges).
+#ifndef GNNHIP_INTERNAL_H
+#define GNNHIP_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "gnnhip.h"
+
+namespace gnnhip {
+
+constexpr int kWave = 64;            // CDNA wavefront width
+constexpr int kNumCU = 256;          // MI355X compute units
+constexpr int kNumXCD = 8;           // accelerator complex dies, one L2 each
+
+int set_error(int code, const char* fmt, ...);
+bool runtime_ready();
+int require_ready();
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+#define GNNHIP_REQUIRE(cond, ...)                                         \
+    do {                                                                  \
+        if (!(cond)) return ::gnnhip::set_error(GNNHIP_EINVAL, __VA_ARGS__); \
+    } while (0)
+
+#define GNNHIP_HIP(call)                                                            \
+    do {                                                                            \
+        hipError_t e__ = (call);                                                    \
+        if (e__ != hipSuccess)                                                      \
+            return ::gnnhip::set_error(GNNHIP_EHIP, "%s failed: %s", #call,         \
+                                       hipGetErrorString(e__));                     \
+    } while (0)
+
+#define GNNHIP_LAUNCH_CHECK(name)                                                   \
+    do {                                                                            \
+        hipError_t e__ = hipGetLastError();                                         \
+        if (e__ != hipSuccess)                                                      \
+            return ::gnnhip::set_error(GNNHIP_EHIP, "launch of %s failed: %s", name, \
+                                       hipGetErrorString(e__));                     \
+    } while (0)
+
+inline unsigned ceil_div_u(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---------------------------------------------------------------- wave64 primitives
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov_f(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_mov_i(int v)
+{
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
+}
+
+// DPP controls: quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror.
+// Each is an involution that pairs lanes, so both partners combine the same two
+// operands and every lane ends with bit-identical results.
+constexpr int kDppXor1 = 0xB1;
+constexpr int kDppXor2 = 0x4E;
+constexpr int kDppHalfMirror = 0x141;   // lane i <-> 7-i inside each group of 8
+constexpr int kDppMirror = 0x140;       // lane i <-> 15-i inside each row of 16
+
+// Every lane of the wavefront receives the sum over all 64 lanes.
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v += dpp_mov_f<kDppXor1>(v);
+    v += dpp_mov_f<kDppXor2>(v);
+    v += dpp_mov_f<kDppHalfMirror>(v);
+    v += dpp_mov_f<kDppMirror>(v);
+    v += __shfl_xor(v, 16, kWave);
+    v += __shfl_xor(v, 32, kWave);
+    return v;
+}
+
+__device__ __forceinline__ int wave_sum_i(int v)
+{
+    v += dpp_mov_i<kDppXor1>(v);
+    v += dpp_mov_i<kDppXor2>(v);
+    v += dpp_mov_i<kDppHalfMirror>(v);
+    v += dpp_mov_i<kDppMirror>(v);
+    v += __shfl_xor(v, 16, kWave);
+    v += __shfl_xor(v, 32, kWave);
+    return v;
+}
+
+// max with "a < b ? b : a" so that a NaN in b never replaces a (the reference's
+// strict comparison never selects a NaN that is not first in the row).
+__device__ __forceinline__ float max_keep(float a, float b) { return a < b ? b : a; }
+
+__device__ __forceinline__ float wave_max(float v)
+{
+    v = max_keep(v, dpp_mov_f<kDppXor1>(v));
+    v = max_keep(v, dpp_mov_f<kDppXor2>(v));
+    v = max_keep(v, dpp_mov_f<kDppHalfMirror>(v));
+    v = max_keep(v, dpp_mov_f<kDppMirror>(v));
+    v = max_keep(v, __shfl_xor(v, 16, kWave));
+    v = max_keep(v, __shfl_xor(v, 32, kWave));
+    return v;
+}
+
+// (value, index) arg-max with the lowest index winning ties.
+__device__ __forceinline__ void argmax_combine(float& v, int& i, float ov, int oi)
+{
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+}
+
+__device__ __forceinline__ void wave_argmax(float& v, int& i)
+{
+    argmax_combine(v, i, dpp_mov_f<kDppXor1>(v), dpp_mov_i<kDppXor1>(i));
+    argmax_combine(v, i, dpp_mov_f<kDppXor2>(v), dpp_mov_i<kDppXor2>(i));
+    argmax_combine(v, i, dpp_mov_f<kDppHalfMirror>(v), dpp_mov_i<kDppHalfMirror>(i));
+    argmax_combine(v, i, dpp_mov_f<kDppMirror>(v), dpp_mov_i<kDppMirror>(i));
+    argmax_combine(v, i, __shfl_xor(v, 16, kWave), __shfl_xor(i, 16, kWave));
+    argmax_combine(v, i, __shfl_xor(v, 32, kWave), __shfl_xor(i, 32, kWave));
+}
+
+// Device memory from the library's pool (released with pool_release).
+int pool_acquire(void** p, size_t bytes);
+int pool_release(void* p);
+
+// Grow-only scratch owned by the library, one buffer per stream, so that calls
+// ordered on one stream reuse it safely and calls on different streams never
+// share it.  The pointer stays valid until a later call on the same stream asks
+// for more bytes.
+int stream_scratch(hipStream_t s, size_t bytes, void** p);
+
+}  // namespace gnnhip
+
+#endif

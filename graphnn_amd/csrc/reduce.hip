@@ -1,0 +1,319 @@
+// Row, jagged and global reductions for gfx950, built on the wave64 DPP/shuffle
+// primitives of gnnhip_internal.h: row softmax, jagged softmax, global
+// sum/mean/max, dense and CSR row arg-max, cross-entropy and in-top-k.
+// One wavefront owns one row (or segment): 64 lanes stride the row with
+// coalesced loads and combine with a DPP butterfly, replacing the thread-0
+// serial loops of cunn_SoftMax_updateOutput_kernel
+// (src/tensor/gpu_dense_tensor.cu:298-370) and the 256-lane shared-memory tree
+// of MatColReduceKernel (include/tensor/gpu_reduce_kernel.h:57-99).
+// All of these are HBM-bound: 8 bytes per element for the in-place softmaxes,
+// 4 bytes per element for the reductions.
+#include "gnnhip_internal.h"
+
+namespace gnnhip {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+// ---- softmax of one contiguous run by one wavefront (all 64 lanes call this)
+__device__ __forceinline__ void wave_softmax_inplace(float* x, long long len, int lane)
+{
+    if (len <= 0) return;
+    float mx = x[0];                                  // reference scan starts at element 0
+    for (long long j = lane; j < len; j += kWave) mx = max_keep(mx, x[j]);
+    mx = wave_max(mx);
+    float s = 0.f;
+    for (long long j = lane; j < len; j += kWave) {
+        const float e = expf(x[j] - mx);
+        x[j] = e;
+        s += e;
+    }
+    s = wave_sum(s);
+    for (long long j = lane; j < len; j += kWave) x[j] = x[j] / s;
+}
+
+__global__ __launch_bounds__(kBlock) void row_softmax_kernel(float* x, int rows, int cols)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    for (long long r = (long long)blockIdx.x * kWavesPerBlock + wave; r < rows; r += (long long)gridDim.x * kWavesPerBlock)
+        wave_softmax_inplace(x + (size_t)r * cols, cols, lane);
+}
+
+// ---- exclusive scan of lens[nseg] into off[nseg+1] by one workgroup of 1024 lanes
+constexpr int kScanBlock = 1024;
+__global__ __launch_bounds__(kScanBlock) void exclusive_scan_kernel(const int* __restrict__ lens, int nseg, int* __restrict__ off)
+{
+    __shared__ int wave_tot[kScanBlock / kWave];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid / kWave;
+    const int chunk = (nseg + kScanBlock - 1) / kScanBlock;
+    const int lo = min(tid * chunk, nseg), hi = min(lo + chunk, nseg);
+    int local = 0;
+    for (int i = lo; i < hi; ++i) local += lens[i];
+    // inclusive scan across the wavefront
+    int incl = local;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int o = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += o;
+    }
+    if (lane == kWave - 1) wave_tot[wave] = incl;
+    __syncthreads();
+    int wave_base = 0;
+    for (int w = 0; w < wave; ++w) wave_base += wave_tot[w];
+    int run = wave_base + incl - local;               // exclusive prefix of this lane's chunk
+    for (int i = lo; i < hi; ++i) { off[i] = run; run += lens[i]; }
+    if (tid == kScanBlock - 1) off[nseg] = run;
+}
+
+__global__ __launch_bounds__(kBlock) void jagged_softmax_kernel(float* x, const int* __restrict__ off, int nseg)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    for (long long s = (long long)blockIdx.x * kWavesPerBlock + wave; s < nseg; s += (long long)gridDim.x * kWavesPerBlock) {
+        const int a = off[s], b = off[s + 1];
+        wave_softmax_inplace(x + a, b - a, lane);
+    }
+}
+
+// ---- global reductions: stage 1 writes one partial per workgroup, stage 2 combines
+// them in index order, so the result does not depend on scheduling.
+template <bool IS_MAX>
+__device__ __forceinline__ float block_combine(float v, float* sh)
+{
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    v = IS_MAX ? wave_max(v) : wave_sum(v);
+    if (lane == 0) sh[wave] = v;
+    __syncthreads();
+    float r = sh[0];
+    for (int w = 1; w < kWavesPerBlock; ++w) r = IS_MAX ? max_keep(r, sh[w]) : r + sh[w];
+    __syncthreads();
+    return r;
+}
+
+template <bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void reduce_partial_kernel(const float* __restrict__ x, size_t n, float* __restrict__ partial)
+{
+    __shared__ float sh[kWavesPerBlock];
+    const size_t per = (n + gridDim.x - 1) / gridDim.x;
+    const size_t lo = (size_t)blockIdx.x * per;
+    const size_t hi = lo + per < n ? lo + per : n;
+    float v = IS_MAX ? -INFINITY : 0.f;
+    if (IS_MAX && lo < hi) v = x[lo];
+    for (size_t i = lo + threadIdx.x; i < hi; i += kBlock) v = IS_MAX ? max_keep(v, x[i]) : v + x[i];
+    v = block_combine<IS_MAX>(v, sh);
+    if (threadIdx.x == 0) partial[blockIdx.x] = v;
+}
+
+template <bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void reduce_final_kernel(const float* __restrict__ partial, int np, float scale_div, float* __restrict__ out)
+{
+    __shared__ float sh[kWavesPerBlock];
+    float v = IS_MAX ? partial[0] : 0.f;
+    for (int i = threadIdx.x; i < np; i += kBlock) v = IS_MAX ? max_keep(v, partial[i]) : v + partial[i];
+    v = block_combine<IS_MAX>(v, sh);
+    if (threadIdx.x == 0) out[0] = (scale_div != 0.f) ? v / scale_div : v;
+}
+
+// ---- arg-max of each dense row, first index among ties
+__global__ __launch_bounds__(kBlock) void row_argmax_kernel(const float* __restrict__ x, int rows, int cols, int* __restrict__ out)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    for (long long r = (long long)blockIdx.x * kWavesPerBlock + wave; r < rows; r += (long long)gridDim.x * kWavesPerBlock) {
+        const float* p = x + (size_t)r * cols;
+        const float first = p[0];
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int j = lane; j < cols; j += kWave) {
+            const float v = p[j];
+            argmax_combine(bv, bi, (v != v) ? -INFINITY : v, j);     // a NaN that is not first never wins
+        }
+        wave_argmax(bv, bi);
+        if (first != first) bi = 0;                                    // a NaN in column 0 is never displaced
+        if (lane == 0) out[r] = bi;
+    }
+}
+
+// ---- CSR rows are short (one-hot labels): one lane per row, reference scan order
+__global__ __launch_bounds__(kBlock) void csr_row_argmax_kernel(const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
+                                                                const float* __restrict__ val, int rows, int* __restrict__ out)
+{
+    for (long long r = (long long)blockIdx.x * kBlock + threadIdx.x; r < rows; r += (long long)gridDim.x * kBlock) {
+        const int a = row_ptr[r], b = row_ptr[r + 1];
+        int best = 0;
+        float cur = 0.f;
+        for (int j = a; j < b; ++j)
+            if (j == a || val[j] > cur) { cur = val[j]; best = col_idx[j]; }
+        out[r] = best;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void cross_entropy_kernel(const float* __restrict__ prob, int rows, int cols,
+                                                               const int* __restrict__ lrow_ptr, const int* __restrict__ lcol,
+                                                               const float* __restrict__ lval, float* __restrict__ out)
+{
+    for (long long r = (long long)blockIdx.x * kBlock + threadIdx.x; r < rows; r += (long long)gridDim.x * kBlock) {
+        float loss = 0.f;
+        for (int k = lrow_ptr[r]; k < lrow_ptr[r + 1]; ++k) {
+            float t = prob[(size_t)cols * r + lcol[k]];
+            if (fabs((double)t) < 1e-8) t = (float)1e-8;
+            loss = (float)((double)loss - log((double)t) * (double)lval[k]);
+        }
+        out[r] = loss;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void in_top_k_kernel(const float* __restrict__ pred, const int* __restrict__ label,
+                                                          int rows, int cols, int k, int* __restrict__ out)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    for (long long r = (long long)blockIdx.x * kWavesPerBlock + wave; r < rows; r += (long long)gridDim.x * kWavesPerBlock) {
+        const float* p = pred + (size_t)r * cols;
+        const int target = label[r];
+        const float pt = p[target];
+        int cnt = 0;
+        for (int j = lane; j < cols; j += kWave)
+            if (j != target && p[j] > pt) cnt += 1;
+        cnt = wave_sum_i(cnt);
+        if (lane == 0) out[r] = cnt < k ? 1 : 0;
+    }
+}
+
+inline unsigned wave_rows_grid(long long rows)
+{
+    long long b = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (b < 1) b = 1;
+    if (b > kNumCU * 16) b = kNumCU * 16;
+    return (unsigned)b;
+}
+
+inline unsigned lane_rows_grid(long long rows)
+{
+    long long b = (rows + kBlock - 1) / kBlock;
+    if (b < 1) b = 1;
+    if (b > kNumCU * 16) b = kNumCU * 16;
+    return (unsigned)b;
+}
+
+}  // namespace
+
+int row_softmax_dispatch(float* x, int rows, int cols, hipStream_t s)
+{
+    hipLaunchKernelGGL(row_softmax_kernel, dim3(wave_rows_grid(rows)), dim3(kBlock), 0, s, x, rows, cols);
+    GNNHIP_LAUNCH_CHECK("row_softmax");
+    return GNNHIP_OK;
+}
+
+int row_argmax_dispatch(const float* x, int rows, int cols, int* out, hipStream_t s)
+{
+    hipLaunchKernelGGL(row_argmax_kernel, dim3(wave_rows_grid(rows)), dim3(kBlock), 0, s, x, rows, cols, out);
+    GNNHIP_LAUNCH_CHECK("row_argmax");
+    return GNNHIP_OK;
+}
+
+}  // namespace gnnhip
+
+using namespace gnnhip;
+
+extern "C" {
+
+int gnnhip_row_softmax_f32(float* x, int rows, int cols, void* stream)
+{
+    GNNHIP_REQUIRE(rows >= 0 && cols >= 0, "negative shape in row_softmax");
+    if (rows == 0 || cols == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(x != nullptr, "null tensor in row_softmax");
+    if (int rc = require_ready()) return rc;
+    return row_softmax_dispatch(x, rows, cols, as_stream(stream));
+}
+
+int gnnhip_jagged_softmax_f32(float* x, const int* lens, int nseg, void* stream)
+{
+    GNNHIP_REQUIRE(nseg >= 0, "negative segment count");
+    if (nseg == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(x && lens, "null tensor in jagged_softmax");
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    void* off = nullptr;
+    if (int rc = stream_scratch(s, sizeof(int) * ((size_t)nseg + 1), &off)) return rc;
+    hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(kScanBlock), 0, s, lens, nseg, static_cast<int*>(off));
+    GNNHIP_LAUNCH_CHECK("exclusive_scan");
+    hipLaunchKernelGGL(jagged_softmax_kernel, dim3(wave_rows_grid(nseg)), dim3(kBlock), 0, s, x, static_cast<const int*>(off), nseg);
+    GNNHIP_LAUNCH_CHECK("jagged_softmax");
+    return GNNHIP_OK;
+}
+
+int gnnhip_reduce_f32(int op, const float* x, size_t n, float* out, void* stream)
+{
+    GNNHIP_REQUIRE(op == GNNHIP_REDUCE_SUM || op == GNNHIP_REDUCE_MEAN || op == GNNHIP_REDUCE_MAX, "unknown reduce op %d", op);
+    GNNHIP_REQUIRE(out != nullptr, "null output in reduce");
+    GNNHIP_REQUIRE(n > 0 && x != nullptr, "empty input in reduce");
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    size_t nb = (n + 16383) / 16384;                   // >= 16K elements per workgroup
+    if (nb > 1024) nb = 1024;
+    void* partial = nullptr;
+    if (int rc = stream_scratch(s, sizeof(float) * 1024, &partial)) return rc;
+    float* pp = static_cast<float*>(partial);
+    const float div = (op == GNNHIP_REDUCE_MEAN) ? (float)n : 0.f;
+    if (op == GNNHIP_REDUCE_MAX) {
+        hipLaunchKernelGGL((reduce_partial_kernel<true>), dim3((unsigned)nb), dim3(kBlock), 0, s, x, n, pp);
+        hipLaunchKernelGGL((reduce_final_kernel<true>), dim3(1), dim3(kBlock), 0, s, pp, (int)nb, 0.f, out);
+    } else {
+        hipLaunchKernelGGL((reduce_partial_kernel<false>), dim3((unsigned)nb), dim3(kBlock), 0, s, x, n, pp);
+        hipLaunchKernelGGL((reduce_final_kernel<false>), dim3(1), dim3(kBlock), 0, s, pp, (int)nb, div, out);
+    }
+    GNNHIP_LAUNCH_CHECK("reduce");
+    return GNNHIP_OK;
+}
+
+int gnnhip_row_argmax_f32(const float* x, int rows, int cols, int* out, void* stream)
+{
+    GNNHIP_REQUIRE(rows >= 0 && cols >= 1, "bad shape in row_argmax (rows=%d cols=%d)", rows, cols);
+    if (rows == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(x && out, "null tensor in row_argmax");
+    if (int rc = require_ready()) return rc;
+    return row_argmax_dispatch(x, rows, cols, out, as_stream(stream));
+}
+
+int gnnhip_csr_row_argmax_f32(const int* row_ptr, const int* col_idx, const float* val, int rows, int* out, void* stream)
+{
+    GNNHIP_REQUIRE(rows >= 0, "negative row count");
+    if (rows == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(row_ptr && out, "null tensor in csr_row_argmax");
+    if (int rc = require_ready()) return rc;
+    hipLaunchKernelGGL(csr_row_argmax_kernel, dim3(lane_rows_grid(rows)), dim3(kBlock), 0, as_stream(stream),
+                       row_ptr, col_idx, val, rows, out);
+    GNNHIP_LAUNCH_CHECK("csr_row_argmax");
+    return GNNHIP_OK;
+}
+
+int gnnhip_cross_entropy_f32(const float* prob, int rows, int cols, const int* lrow_ptr, const int* lcol,
+                             const float* lval, float* out, void* stream)
+{
+    GNNHIP_REQUIRE(rows >= 0 && cols >= 1, "bad shape in cross_entropy");
+    if (rows == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(prob && lrow_ptr && out, "null tensor in cross_entropy");
+    if (int rc = require_ready()) return rc;
+    hipLaunchKernelGGL(cross_entropy_kernel, dim3(lane_rows_grid(rows)), dim3(kBlock), 0, as_stream(stream),
+                       prob, rows, cols, lrow_ptr, lcol, lval, out);
+    GNNHIP_LAUNCH_CHECK("cross_entropy");
+    return GNNHIP_OK;
+}
+
+int gnnhip_in_top_k_f32(const float* pred, const int* label, int rows, int cols, int k, int* out, void* stream)
+{
+    GNNHIP_REQUIRE(rows >= 0 && cols >= 1, "bad shape in in_top_k");
+    if (rows == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(pred && label && out, "null tensor in in_top_k");
+    if (int rc = require_ready()) return rc;
+    hipLaunchKernelGGL(in_top_k_kernel, dim3(wave_rows_grid(rows)), dim3(kBlock), 0, as_stream(stream),
+                       pred, label, rows, cols, k, out);
+    GNNHIP_LAUNCH_CHECK("in_top_k");
+    return GNNHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,265 @@
+// Runtime of the gfx950 backend: device selection, error text, the size-keyed
+// device-memory pool and the copy entry points.
+//
+// The pool follows the policy of graphnn's MemHolder<GPU>
+// (src/util/mem_holder.cpp:15-97): recycle parks a block under its byte size,
+// malloc hands out the smallest parked block that is large enough, and only
+// free() gives memory back to the driver.  Per-level activations therefore stay
+// resident in HBM from batch to batch.
+#include "gnnhip_internal.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+
+namespace gnnhip {
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+struct Runtime {
+    std::mutex mu;
+    bool ready = false;
+    int device = -1;
+    std::multimap<size_t, void*> parked;           // size -> free block
+    std::unordered_map<void*, size_t> live;        // block handed out -> size
+    std::unordered_map<void*, size_t> all;         // every driver allocation -> size
+    size_t bytes_in_use = 0;
+    size_t bytes_parked = 0;
+    size_t n_driver_allocs = 0;
+    std::unordered_map<hipStream_t, std::pair<void*, size_t>> scratch;   // per-stream library scratch
+};
+
+Runtime& rt()
+{
+    static Runtime r;
+    return r;
+}
+
+constexpr size_t kAllocGranule = 256;   // keeps every block 256-byte aligned in size as well as address
+
+}  // namespace
+
+int set_error(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+bool runtime_ready() { return rt().ready; }
+
+int require_ready()
+{
+    if (!rt().ready) return set_error(GNNHIP_ENOTINIT, "gnnhip_init has not been called");
+    return GNNHIP_OK;
+}
+
+int pool_acquire(void** p, size_t bytes)
+{
+    if (!p) return set_error(GNNHIP_EINVAL, "null output pointer");
+    *p = nullptr;
+    Runtime& r = rt();
+    std::lock_guard<std::mutex> lock(r.mu);
+    if (!r.ready) return set_error(GNNHIP_ENOTINIT, "gnnhip_init has not been called");
+    if (bytes == 0) bytes = 1;
+    size_t want = (bytes + kAllocGranule - 1) / kAllocGranule * kAllocGranule;
+    auto it = r.parked.lower_bound(want);
+    if (it != r.parked.end()) {
+        void* q = it->second;
+        size_t sz = it->first;
+        r.parked.erase(it);
+        r.bytes_parked -= sz;
+        r.live[q] = sz;
+        r.bytes_in_use += sz;
+        *p = q;
+        return GNNHIP_OK;
+    }
+    void* q = nullptr;
+    hipError_t e = hipMalloc(&q, want);
+    if (e != hipSuccess || q == nullptr) {
+        (void)hipGetLastError();
+        return set_error(GNNHIP_ENOMEM, "hipMalloc of %zu bytes failed: %s", want, hipGetErrorString(e));
+    }
+    r.all[q] = want;
+    r.live[q] = want;
+    r.bytes_in_use += want;
+    r.n_driver_allocs += 1;
+    *p = q;
+    return GNNHIP_OK;
+}
+
+int pool_release(void* p)
+{
+    if (!p) return GNNHIP_OK;
+    Runtime& r = rt();
+    std::lock_guard<std::mutex> lock(r.mu);
+    auto it = r.live.find(p);
+    if (it == r.live.end()) return set_error(GNNHIP_EINVAL, "pointer %p was not handed out by gnnhip_malloc", p);
+    size_t sz = it->second;
+    r.live.erase(it);
+    r.bytes_in_use -= sz;
+    r.parked.emplace(sz, p);
+    r.bytes_parked += sz;
+    return GNNHIP_OK;
+}
+
+int stream_scratch(hipStream_t s, size_t bytes, void** p)
+{
+    Runtime& r = rt();
+    std::lock_guard<std::mutex> lock(r.mu);
+    if (!r.ready) return set_error(GNNHIP_ENOTINIT, "gnnhip_init has not been called");
+    auto& slot = r.scratch[s];
+    if (slot.second < bytes) {
+        size_t want = (bytes + 65535) / 65536 * 65536;
+        if (want < slot.second * 2) want = slot.second * 2;
+        void* q = nullptr;
+        hipError_t e = hipMalloc(&q, want);
+        if (e != hipSuccess || !q) {
+            (void)hipGetLastError();
+            return set_error(GNNHIP_ENOMEM, "hipMalloc of %zu scratch bytes failed: %s", want, hipGetErrorString(e));
+        }
+        if (slot.first) {
+            // kernels queued earlier on this stream may still read the old buffer
+            (void)hipStreamSynchronize(s);
+            (void)hipFree(slot.first);
+        }
+        slot.first = q;
+        slot.second = want;
+    }
+    *p = slot.first;
+    return GNNHIP_OK;
+}
+
+}  // namespace gnnhip
+
+using namespace gnnhip;
+
+extern "C" {
+
+const char* gnnhip_last_error(void) { return g_err; }
+
+const char* gnnhip_version(void) { return "gnnhip 0.1 (gfx950)"; }
+
+int gnnhip_init(int device_id)
+{
+    Runtime& r = rt();
+    std::lock_guard<std::mutex> lock(r.mu);
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return set_error(GNNHIP_EHIP, "no HIP device visible (%s)", hipGetErrorString(e));
+    }
+    if (device_id < 0 || device_id >= count)
+        return set_error(GNNHIP_EINVAL, "device_id %d out of range [0,%d)", device_id, count);
+    if (r.ready && r.device != device_id)
+        return set_error(GNNHIP_EINVAL, "already initialised on device %d", r.device);
+    GNNHIP_HIP(hipSetDevice(device_id));
+    r.device = device_id;
+    r.ready = true;
+    return GNNHIP_OK;
+}
+
+int gnnhip_shutdown(void)
+{
+    Runtime& r = rt();
+    std::lock_guard<std::mutex> lock(r.mu);
+    if (!r.ready) return GNNHIP_OK;
+    (void)hipDeviceSynchronize();
+    for (auto& kv : r.all) (void)hipFree(kv.first);
+    for (auto& kv : r.scratch) (void)hipFree(kv.second.first);
+    r.scratch.clear();
+    r.all.clear();
+    r.live.clear();
+    r.parked.clear();
+    r.bytes_in_use = r.bytes_parked = 0;
+    r.ready = false;
+    r.device = -1;
+    return GNNHIP_OK;
+}
+
+int gnnhip_malloc(void** device_ptr, size_t bytes) { return pool_acquire(device_ptr, bytes); }
+
+int gnnhip_recycle(void* device_ptr) { return pool_release(device_ptr); }
+
+int gnnhip_free(void* device_ptr)
+{
+    if (!device_ptr) return GNNHIP_OK;
+    Runtime& r = rt();
+    std::lock_guard<std::mutex> lock(r.mu);
+    auto it = r.all.find(device_ptr);
+    if (it == r.all.end())
+        return set_error(GNNHIP_EINVAL, "pointer %p is not owned by the gnnhip pool", device_ptr);
+    size_t sz = it->second;
+    auto lv = r.live.find(device_ptr);
+    if (lv != r.live.end()) {
+        r.live.erase(lv);
+        r.bytes_in_use -= sz;
+    } else {
+        auto range = r.parked.equal_range(sz);
+        for (auto p = range.first; p != range.second; ++p) {
+            if (p->second == device_ptr) {
+                r.parked.erase(p);
+                r.bytes_parked -= sz;
+                break;
+            }
+        }
+    }
+    r.all.erase(it);
+    GNNHIP_HIP(hipFree(device_ptr));
+    return GNNHIP_OK;
+}
+
+int gnnhip_pool_stats(size_t* bytes_in_use, size_t* bytes_parked, size_t* n_driver_allocs)
+{
+    Runtime& r = rt();
+    std::lock_guard<std::mutex> lock(r.mu);
+    if (bytes_in_use) *bytes_in_use = r.bytes_in_use;
+    if (bytes_parked) *bytes_parked = r.bytes_parked;
+    if (n_driver_allocs) *n_driver_allocs = r.n_driver_allocs;
+    return GNNHIP_OK;
+}
+
+int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream)
+{
+    if (bytes == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(dst_device && src_host, "null pointer in memcpy_h2d");
+    if (int rc = require_ready()) return rc;
+    // Pageable source: the runtime stages the bytes before returning, so the host buffer may be reused at once.
+    GNNHIP_HIP(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    return GNNHIP_OK;
+}
+
+int gnnhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream)
+{
+    if (bytes == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(dst_host && src_device, "null pointer in memcpy_d2h");
+    if (int rc = require_ready()) return rc;
+    GNNHIP_HIP(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
+    GNNHIP_HIP(hipStreamSynchronize(as_stream(stream)));
+    return GNNHIP_OK;
+}
+
+int gnnhip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream)
+{
+    if (bytes == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(dst_device && src_device, "null pointer in memcpy_d2d");
+    if (int rc = require_ready()) return rc;
+    GNNHIP_HIP(hipMemcpyAsync(dst_device, src_device, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+    return GNNHIP_OK;
+}
+
+int gnnhip_stream_sync(void* stream)
+{
+    if (int rc = require_ready()) return rc;
+    GNNHIP_HIP(hipStreamSynchronize(as_stream(stream)));
+    return GNNHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,277 @@
+"""Thin torch-pointer helpers over the C ABI (used by the tests, the smoke check and the bench).
+
+torch supplies device memory and the stream; all arithmetic happens in libgnnhip.so.
+Every helper validates dtype / device / contiguity on the host before a pointer
+reaches a kernel, and raises GnnHipError on a non-zero status.
+"""
+import ctypes
+
+import torch
+
+from ._lib import check, load_library
+
+UNARY = {
+    "set": 0, "truncate": 1, "scale": 2, "add": 3, "abs": 4, "inv": 5, "relu": 6, "sigmoid": 7,
+    "tanh": 8, "log": 9, "invsqrt": 10, "exp": 11, "square": 12, "sqrt": 13,
+}
+REDUCE = {"sum": 0, "mean": 1, "max": 2}
+
+_initialised = False
+
+
+def init(device_id=0):
+    global _initialised
+    lib = load_library()
+    check(lib.gnnhip_init(int(device_id)))
+    _initialised = True
+    return lib
+
+
+def _lib():
+    if not _initialised:
+        init(torch.cuda.current_device())
+    return load_library()
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _f32(t, name):
+    if t is None:
+        return None
+    if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()):
+        raise ValueError("%s must be a contiguous float32 CUDA tensor" % name)
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _i32(t, name):
+    if t is None:
+        return None
+    if not (t.is_cuda and t.dtype == torch.int32 and t.is_contiguous()):
+        raise ValueError("%s must be a contiguous int32 CUDA tensor" % name)
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _check_csr(row_ptr, col_idx, val, rows, name):
+    if row_ptr.numel() != rows + 1:
+        raise ValueError("%s.row_ptr must have rows+1 = %d entries" % (name, rows + 1))
+    if col_idx.numel() != val.numel():
+        raise ValueError("%s: col_idx and val differ in length" % name)
+
+
+def spmm(row_ptr, col_idx, val, B, m, alpha=1.0, beta=0.0, out=None):
+    """out[m,n] = alpha * A * B + beta * out, A CSR with m rows and B.shape[0] columns."""
+    k, n = B.shape
+    _check_csr(row_ptr, col_idx, val, m, "A")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=B.device)
+    elif tuple(out.shape) != (m, n):
+        raise ValueError("out has the wrong shape")
+    check(_lib().gnnhip_spmm_csr_f32(m, k, n, alpha, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"),
+                                     _f32(val, "val"), _f32(B, "B"), n, beta, _f32(out, "out"), n, _stream()))
+    return out
+
+
+def gemm(A, B, transA=False, transB=False, alpha=1.0, beta=0.0, out=None):
+    m = A.shape[1] if transA else A.shape[0]
+    k = A.shape[0] if transA else A.shape[1]
+    kb = B.shape[1] if transB else B.shape[0]
+    n = B.shape[0] if transB else B.shape[1]
+    if k != kb:
+        raise ValueError("mat dim doesn't match")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=A.device)
+    elif tuple(out.shape) != (m, n):
+        raise ValueError("out has the wrong shape")
+    check(_lib().gnnhip_gemm_f32(int(transA), int(transB), m, n, k, alpha, _f32(A, "A"), A.shape[1],
+                                 _f32(B, "B"), B.shape[1], beta, _f32(out, "out"), n, _stream()))
+    return out
+
+
+def s2v_input(X, W_n2l):
+    N, K = X.shape
+    if W_n2l.shape[0] != K:
+        raise ValueError("X and W_n2l disagree on the label width")
+    C = W_n2l.shape[1]
+    msg = torch.empty((N, C), dtype=torch.float32, device=X.device)
+    h0 = torch.empty_like(msg)
+    check(_lib().gnnhip_s2v_input_f32(N, K, C, _f32(X, "X"), _f32(W_n2l, "W_n2l"), _f32(msg, "msg"),
+                                      _f32(h0, "h0"), _stream()))
+    return msg, h0
+
+
+def s2v_level(row_ptr, col_idx, val, h_in, W, msg=None, bias=None, out=None):
+    N, C = h_in.shape
+    _check_csr(row_ptr, col_idx, val, N, "A")
+    if tuple(W.shape) != (C, C):
+        raise ValueError("W must be [C,C]")
+    if msg is not None and tuple(msg.shape) != (N, C):
+        raise ValueError("msg must be [N,C]")
+    if bias is not None and bias.numel() != C:
+        raise ValueError("bias must have C entries")
+    if out is None:
+        out = torch.empty_like(h_in)
+    check(_lib().gnnhip_s2v_level_f32(N, C, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"), _f32(val, "val"),
+                                      _f32(h_in, "h_in"), _f32(W, "W"), _f32(msg, "msg"), _f32(bias, "bias"),
+                                      _f32(out, "out"), _stream()))
+    return out
+
+
+def s2v_readout(s_row_ptr, s_col_idx, s_val, h, W_h1, W_h2, B):
+    N, C = h.shape
+    H, Q = W_h1.shape[1], W_h2.shape[1]
+    _check_csr(s_row_ptr, s_col_idx, s_val, B, "S")
+    if W_h1.shape[0] != C or W_h2.shape[0] != H:
+        raise ValueError("readout weight shapes do not chain")
+    dev = h.device
+    pool = torch.empty((B, C), dtype=torch.float32, device=dev)
+    hidden = torch.empty((B, H), dtype=torch.float32, device=dev)
+    logits = torch.empty((B, Q), dtype=torch.float32, device=dev)
+    probs = torch.empty((B, Q), dtype=torch.float32, device=dev)
+    pred = torch.empty((B,), dtype=torch.int32, device=dev)
+    check(_lib().gnnhip_s2v_readout_f32(B, N, C, H, Q, _i32(s_row_ptr, "s_row_ptr"), _i32(s_col_idx, "s_col_idx"),
+                                        _f32(s_val, "s_val"), _f32(h, "h"), _f32(W_h1, "W_h1"), _f32(W_h2, "W_h2"),
+                                        _f32(pool, "pool"), _f32(hidden, "hidden"), _f32(logits, "logits"),
+                                        _f32(probs, "probs"), _i32(pred, "pred"), _stream()))
+    return pool, hidden, logits, probs, pred
+
+
+class ForwardBuffers:
+    """Caller-owned activations of one forward; allocated once and reused across calls."""
+
+    def __init__(self, N, B, C, H, Q, device):
+        f = dict(dtype=torch.float32, device=device)
+        self.msg = torch.empty((N, C), **f)
+        self.h_a = torch.empty((N, C), **f)
+        self.h_b = torch.empty((N, C), **f)
+        self.pool = torch.empty((B, C), **f)
+        self.hidden = torch.empty((B, H), **f)
+        self.logits = torch.empty((B, Q), **f)
+        self.probs = torch.empty((B, Q), **f)
+        self.pred = torch.empty((B,), dtype=torch.int32, device=device)
+        self.which = ctypes.c_int(0)
+
+    @property
+    def h_final(self):
+        return self.h_a if self.which.value == 0 else self.h_b
+
+
+def s2v_forward(a_csr, s_csr, X, W_n2l, W_conv, W_h1, W_h2, L, bufs=None):
+    """Whole forward.  a_csr / s_csr are (row_ptr, col_idx, val) triples of int32/int32/float32 device tensors."""
+    N, K = X.shape
+    C, H, Q = W_n2l.shape[1], W_h1.shape[1], W_h2.shape[1]
+    B = s_csr[0].numel() - 1
+    _check_csr(a_csr[0], a_csr[1], a_csr[2], N, "A")
+    _check_csr(s_csr[0], s_csr[1], s_csr[2], B, "S")
+    if W_n2l.shape[0] != K or tuple(W_conv.shape) != (C, C) or W_h1.shape[0] != C or W_h2.shape[0] != H:
+        raise ValueError("weight shapes do not chain")
+    if bufs is None:
+        bufs = ForwardBuffers(N, B, C, H, Q, X.device)
+    check(_lib().gnnhip_s2v_forward_f32(
+        N, B, K, C, H, Q, L,
+        _i32(a_csr[0], "a_row_ptr"), _i32(a_csr[1], "a_col_idx"), _f32(a_csr[2], "a_val"),
+        _i32(s_csr[0], "s_row_ptr"), _i32(s_csr[1], "s_col_idx"), _f32(s_csr[2], "s_val"),
+        _f32(X, "X"), _f32(W_n2l, "W_n2l"), _f32(W_conv, "W_conv"), _f32(W_h1, "W_h1"), _f32(W_h2, "W_h2"),
+        _f32(bufs.msg, "msg"), _f32(bufs.h_a, "h_a"), _f32(bufs.h_b, "h_b"), _f32(bufs.pool, "pool"),
+        _f32(bufs.hidden, "hidden"), _f32(bufs.logits, "logits"), _f32(bufs.probs, "probs"),
+        _i32(bufs.pred, "pred"), ctypes.byref(bufs.which), _stream()))
+    return bufs
+
+
+def unary(op, x, a0=0.0, a1=0.0):
+    check(_lib().gnnhip_unary_f32(UNARY[op], _f32(x, "x"), x.numel(), a0, a1, _stream()))
+    return x
+
+
+def relu(x, out=None):
+    if out is None:
+        out = torch.empty_like(x)
+    check(_lib().gnnhip_relu_f32(_f32(x, "x"), _f32(out, "out"), x.numel(), _stream()))
+    return out
+
+
+def axpy(a, x, y):
+    if x.numel() != y.numel():
+        raise ValueError("shape doesn't match in Axpy")
+    check(_lib().gnnhip_axpy_f32(x.numel(), a, _f32(x, "x"), _f32(y, "y"), _stream()))
+    return y
+
+
+def axpby(a, x, b, y):
+    if x.numel() != y.numel():
+        raise ValueError("shape doesn't match in Axpby")
+    check(_lib().gnnhip_axpby_f32(x.numel(), a, _f32(x, "x"), b, _f32(y, "y"), _stream()))
+    return y
+
+
+def add(a, b, out=None):
+    if a.numel() != b.numel():
+        raise ValueError("no broadcasting is supported")
+    if out is None:
+        out = torch.empty_like(a)
+    check(_lib().gnnhip_add_f32(a.numel(), _f32(a, "a"), _f32(b, "b"), _f32(out, "out"), _stream()))
+    return out
+
+
+def row_softmax(x):
+    rows, cols = x.shape
+    check(_lib().gnnhip_row_softmax_f32(_f32(x, "x"), rows, cols, _stream()))
+    return x
+
+
+def jagged_softmax(x, lens):
+    check(_lib().gnnhip_jagged_softmax_f32(_f32(x, "x"), _i32(lens, "lens"), lens.numel(), _stream()))
+    return x
+
+
+def reduce(op, x):
+    out = torch.empty((1,), dtype=torch.float32, device=x.device)
+    check(_lib().gnnhip_reduce_f32(REDUCE[op], _f32(x, "x"), x.numel(), _f32(out, "out"), _stream()))
+    return out
+
+
+def row_argmax(x):
+    rows, cols = x.shape
+    out = torch.empty((rows,), dtype=torch.int32, device=x.device)
+    check(_lib().gnnhip_row_argmax_f32(_f32(x, "x"), rows, cols, _i32(out, "out"), _stream()))
+    return out
+
+
+def csr_row_argmax(row_ptr, col_idx, val):
+    rows = row_ptr.numel() - 1
+    out = torch.empty((rows,), dtype=torch.int32, device=row_ptr.device)
+    check(_lib().gnnhip_csr_row_argmax_f32(_i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"), _f32(val, "val"),
+                                           rows, _i32(out, "out"), _stream()))
+    return out
+
+
+def cross_entropy(prob, l_row_ptr, l_col_idx, l_val):
+    rows, cols = prob.shape
+    _check_csr(l_row_ptr, l_col_idx, l_val, rows, "label")
+    out = torch.empty((rows, 1), dtype=torch.float32, device=prob.device)
+    check(_lib().gnnhip_cross_entropy_f32(_f32(prob, "prob"), rows, cols, _i32(l_row_ptr, "l_row_ptr"),
+                                          _i32(l_col_idx, "l_col_idx"), _f32(l_val, "l_val"), _f32(out, "out"),
+                                          _stream()))
+    return out
+
+
+def in_top_k(pred, label, k=1):
+    rows, cols = pred.shape
+    if label.numel() != rows:
+        raise ValueError("# instances doesn't match")
+    out = torch.empty((rows,), dtype=torch.int32, device=pred.device)
+    check(_lib().gnnhip_in_top_k_f32(_f32(pred, "pred"), _i32(label, "label"), rows, cols, k, _i32(out, "out"),
+                                     _stream()))
+    return out
+
+
+def cast_i32_f32(src):
+    dst = torch.empty(src.shape, dtype=torch.float32, device=src.device)
+    check(_lib().gnnhip_cast_i32_f32(_i32(src, "src"), _f32(dst, "dst"), src.numel(), _stream()))
+    return dst
+
+
+def memset0(t):
+    check(_lib().gnnhip_memset0(ctypes.c_void_p(t.data_ptr()), t.numel() * t.element_size(), _stream()))
+    return t

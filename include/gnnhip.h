@@ -1,0 +1,181 @@
+/*
+ * gnnhip — C ABI of the gfx950 (MI355X) backend for graphnn's structure2vec
+ * mean-field forward.  Plain pointers and sizes only; every pointer named
+ * "device" is HIP device memory, every matrix is row-major fp32, every CSR
+ * index is int32 (reference layout: include/tensor/t_data.h:123-165).
+ *
+ * Conventions
+ *   - every entry returns GNNHIP_OK (0) or a negative GNNHIP_E* code and never
+ *     throws; gnnhip_last_error() gives the text for the calling thread.
+ *   - `stream` is a hipStream_t passed as void*; NULL means the HIP null stream.
+ *     Calls are asynchronous on that stream except where stated.
+ *   - the library keeps no caller pointer after the call's work on the stream
+ *     has finished; outputs are caller-allocated.
+ *
+ * Each declaration cites the reference interface it stands in for
+ * (paths relative to the graphnn source tree).
+ */
+#ifndef GNNHIP_H
+#define GNNHIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GNNHIP_OK            0
+#define GNNHIP_EINVAL       -1   /* bad argument (null pointer, negative size, bad op code) */
+#define GNNHIP_ENOMEM       -2   /* device allocation failed */
+#define GNNHIP_EHIP         -3   /* a HIP runtime call failed */
+#define GNNHIP_ENOTINIT     -4   /* gnnhip_init has not been called */
+#define GNNHIP_EUNSUPPORTED -5   /* shape outside what the kernels handle */
+
+/* unary functor codes — include/tensor/gpu_unary_functor.h:17-327 */
+enum {
+    GNNHIP_UNARY_SET = 0, GNNHIP_UNARY_TRUNCATE = 1, GNNHIP_UNARY_SCALE = 2, GNNHIP_UNARY_ADD = 3,
+    GNNHIP_UNARY_ABS = 4, GNNHIP_UNARY_INV = 5, GNNHIP_UNARY_RELU = 6, GNNHIP_UNARY_SIGMOID = 7,
+    GNNHIP_UNARY_TANH = 8, GNNHIP_UNARY_LOG = 9, GNNHIP_UNARY_INVSQRT = 10, GNNHIP_UNARY_EXP = 11,
+    GNNHIP_UNARY_SQUARE = 12, GNNHIP_UNARY_SQRT = 13, GNNHIP_UNARY__COUNT = 14
+};
+
+/* reduction codes — include/tensor/gpu_reduce_kernel.h:12-55 */
+enum { GNNHIP_REDUCE_SUM = 0, GNNHIP_REDUCE_MEAN = 1, GNNHIP_REDUCE_MAX = 2 };
+
+const char* gnnhip_last_error(void);
+const char* gnnhip_version(void);
+
+/* ---- runtime: GpuHandle::Init / Destroy (include/tensor/gpu_handle.h:38-59,
+ *      src/tensor/gpu_handle.cu:17-70).  No vendor BLAS/SPARSE handles exist. */
+int gnnhip_init(int device_id);
+int gnnhip_shutdown(void);
+
+/* ---- pooled device memory: MemHolder<GPU>::MallocArr / Recycle / ForceDel
+ *      (include/util/mem_holder.h:20-51, src/util/mem_holder.cpp:15-97).
+ *      malloc takes the smallest parked block >= bytes or allocates; recycle
+ *      parks the block for reuse; free returns it to the driver. */
+int gnnhip_malloc(void** device_ptr, size_t bytes);
+int gnnhip_recycle(void* device_ptr);
+int gnnhip_free(void* device_ptr);
+int gnnhip_pool_stats(size_t* bytes_in_use, size_t* bytes_parked, size_t* n_driver_allocs);
+
+/* ---- copies: DTensor<GPU>::CopyFrom / AsScalar / Zeros
+ *      (src/tensor/gpu_dense_tensor.cu:97-150), SpTensor<GPU>::CopyFrom
+ *      (src/tensor/gpu_sparse_tensor.cu:55-73).  d2h blocks until the data
+ *      is in host memory (the reference's only synchronisation point). */
+int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream);
+int gnnhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
+int gnnhip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream);
+int gnnhip_memset0(void* device_ptr, size_t bytes, void* stream);
+int gnnhip_stream_sync(void* stream);
+
+/* ---- C[m,n] = alpha * A * B + beta * C, A CSR [m,k], B dense [k,n].
+ *      DTensor<GPU>::MM(SpTensor, DTensor, Trans::N, Trans::N) + CSRMMKernel
+ *      (src/tensor/gpu_dense_tensor.cu:227-239,257-270).  beta == 0 overwrites C. */
+int gnnhip_spmm_csr_f32(int m, int k, int n, float alpha, const int* row_ptr, const int* col_idx,
+                        const float* val, const float* B, int ldb, float beta, float* C, int ldc,
+                        void* stream);
+
+/* ---- C[m,n] = alpha * op(A) * op(B) + beta * C, all dense row-major.
+ *      DTensor<GPU>::MM(DTensor, DTensor) (src/tensor/gpu_dense_tensor.cu:192-224).
+ *      transA/transB: 0 = N, 1 = T.  lda/ldb/ldc are row strides of the stored matrices. */
+int gnnhip_gemm_f32(int transA, int transB, int m, int n, int k, float alpha, const float* A, int lda,
+                    const float* B, int ldb, float beta, float* C, int ldc, void* stream);
+
+/* ---- one mean-field level in a single pass:
+ *      h_out = ReLU((A * h_in) * W + bias + msg)
+ *      replaces MatMul(sparse) + MatMul(dense) + ElewiseAdd + ReLU
+ *      (examples/graph_classification/src/kernel_mean_field.cpp:35-42,
+ *       src/nn/matmul.cpp:13-33, src/nn/elewise_add.cpp:13-33, src/nn/relu.cu:9-13;
+ *       bias as in src/nn/fully_connected.cpp:28-39).  msg and bias may be NULL.
+ *      A is [N,N] CSR, h_in/h_out/msg are [N,C], W is [C,C]; h_out must not alias h_in. */
+int gnnhip_s2v_level_f32(int N, int C, const int* row_ptr, const int* col_idx, const float* val,
+                         const float* h_in, const float* W, const float* msg, const float* bias,
+                         float* h_out, void* stream);
+
+/* ---- msg = X * W_n2l and h0 = ReLU(msg) in one pass
+ *      (examples/graph_classification/src/kernel_mean_field.cpp:31-32: MatMul + ReLU).  X [N,K], W_n2l [K,C]. */
+int gnnhip_s2v_input_f32(int N, int K, int C, const float* X, const float* W_n2l,
+                         float* msg, float* h0, void* stream);
+
+/* ---- readout: pool = S * h ; hidden = ReLU(pool * W_h1) ; logits = hidden * W_h2 ;
+ *      probs = softmax(logits) ; pred = row argmax(logits)
+ *      (examples/graph_classification/src/kernel_mean_field.cpp:44-49 and the softmax of
+ *      src/nn/cross_entropy.cpp:45-47).
+ *      S is [B,N] CSR.  pool [B,C], hidden [B,H], logits/probs [B,Q], pred int[B];
+ *      probs and pred may be NULL. */
+int gnnhip_s2v_readout_f32(int B, int N, int C, int H, int Q,
+                           const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                           const float* h, const float* W_h1, const float* W_h2,
+                           float* pool, float* hidden, float* logits, float* probs, int* pred,
+                           void* stream);
+
+/* ---- whole forward = input + L levels + readout, device-resident.
+ *      h_a / h_b are [N,C] ping-pong buffers; *which_h (host int, may be NULL)
+ *      receives 0 if the final embedding is in h_a, 1 if in h_b.
+ *      Op sequence of examples/graph_classification/src/kernel_mean_field.cpp:31-49 scheduled by
+ *      FactorGraph::SequentialForward (src/nn/factor_graph.cpp:75-144). */
+int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L,
+                           const int* a_row_ptr, const int* a_col_idx, const float* a_val,
+                           const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                           const float* X, const float* W_n2l, const float* W_conv,
+                           const float* W_h1, const float* W_h2,
+                           float* msg, float* h_a, float* h_b,
+                           float* pool, float* hidden, float* logits, float* probs, int* pred,
+                           int* which_h, void* stream);
+
+/* ---- UnaryEngine<GPU>::Exec<Functor> (include/tensor/gpu_unary_functor.h:331-384):
+ *      in-place x[i] = f(x[i]); a0/a1 are the functor's constructor arguments. */
+int gnnhip_unary_f32(int op, float* x, size_t n, float a0, float a1, void* stream);
+
+/* ---- out = ReLU(in) without the intermediate copy: ReLUAct(GPU) (src/nn/relu.cu:9-13) */
+int gnnhip_relu_f32(const float* in, float* out, size_t n, void* stream);
+
+/* ---- y += a*x : DTensor<GPU>::Axpy (src/tensor/gpu_dense_tensor.cu:489-496);
+ *      y = a*x + b*y : Axpby. */
+int gnnhip_axpy_f32(size_t n, float a, const float* x, float* y, void* stream);
+int gnnhip_axpby_f32(size_t n, float a, const float* x, float b, float* y, void* stream);
+
+/* ---- out = a + b (the ElewiseAdd of two operands without the copy, src/nn/elewise_add.cpp:13-33) */
+int gnnhip_add_f32(size_t n, const float* a, const float* b, float* out, void* stream);
+
+/* ---- row softmax in place: DTensor<GPU>::Softmax (src/tensor/gpu_dense_tensor.cu:298-370) */
+int gnnhip_row_softmax_f32(float* x, int rows, int cols, void* stream);
+
+/* ---- softmax over consecutive segments of a column vector; lens is a device int[nseg]:
+ *      DTensor<GPU>::JaggedSoftmax (src/tensor/gpu_dense_tensor.cu:372-450).
+ *      Segment offsets come from an exclusive scan of lens done on the device. */
+int gnnhip_jagged_softmax_f32(float* x, const int* lens, int nseg, void* stream);
+
+/* ---- global sum / mean / max into out[0] (device):
+ *      DTensor<GPU>::Sum / Mean (src/tensor/gpu_dense_tensor.cu:466-481),
+ *      MatColReduceKernel (include/tensor/gpu_reduce_kernel.h:57-99) */
+int gnnhip_reduce_f32(int op, const float* x, size_t n, float* out, void* stream);
+
+/* ---- per-row arg-max, first index among ties (the CPU rule,
+ *      src/tensor/cpu_dense_tensor.cpp:176-196; GPU call site gpu_dense_tensor.cu:184-190) */
+int gnnhip_row_argmax_f32(const float* x, int rows, int cols, int* out, void* stream);
+
+/* ---- per-CSR-row column of the largest stored value, empty row -> 0:
+ *      SpTensor<GPU>::ArgMax (src/tensor/gpu_sparse_tensor.cu:82-122; CPU rule
+ *      src/tensor/cpu_sparse_tensor.cpp:86-103) */
+int gnnhip_csr_row_argmax_f32(const int* row_ptr, const int* col_idx, const float* val, int rows,
+                              int* out, void* stream);
+
+/* ---- out[r] = -sum_k log(p[r, lcol[k]]) * lval[k], |p| < 1e-8 clamped to 1e-8:
+ *      CalcCrossEntropy (src/nn/cross_entropy.cu:9-49; clamp of src/nn/cross_entropy.cpp:18-19) */
+int gnnhip_cross_entropy_f32(const float* prob, int rows, int cols, const int* lrow_ptr,
+                             const int* lcol, const float* lval, float* out, void* stream);
+
+/* ---- out[r] = (#{j != label[r] : p[r,j] > p[r,label[r]]}) < k :
+ *      IsInTopK (src/nn/in_top_k.cu:9-51) */
+int gnnhip_in_top_k_f32(const float* pred, const int* label, int rows, int cols, int k, int* out,
+                        void* stream);
+
+/* ---- dst[i] = (float)src[i] : TypeCastCopy (src/tensor/gpu_binary_functor.cu:7-31) */
+int gnnhip_cast_i32_f32(const int* src, float* dst, size_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

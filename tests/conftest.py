@@ -1,0 +1,219 @@
+import ctypes
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+# --------------------------------------------------------------------------- oracle binding
+_ORACLE_PATH = os.path.join(ROOT, "oracle", "liboracle.so")
+_REF_PATH = os.path.join(ROOT, "oracle", "_ref", "libref_graph.so")
+
+
+def _ptr(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+class Oracle:
+    """ctypes view of oracle/liboracle.so (the CPU restatement; checker only)."""
+
+    def __init__(self):
+        if not os.path.exists(_ORACLE_PATH):
+            import subprocess
+            subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle"), "liboracle.so"])
+        self.lib = ctypes.CDLL(_ORACLE_PATH)
+        self.lib.orc_sum.restype = ctypes.c_float
+        self.lib.orc_mean.restype = ctypes.c_float
+        self.lib.orc_max.restype = ctypes.c_float
+
+    # ---- CSR builders
+    def csr_node2node(self, N, ex, ey, average=False):
+        E = len(ex)
+        ex = np.ascontiguousarray(ex, dtype=np.int32)
+        ey = np.ascontiguousarray(ey, dtype=np.int32)
+        rp = np.zeros(N + 1, np.int32); ci = np.zeros(E, np.int32); v = np.zeros(E, np.float32)
+        self.lib.orc_csr_node2node(N, E, _ptr(ex), _ptr(ey), int(average), _ptr(rp), _ptr(ci), _ptr(v))
+        return rp, ci, v
+
+    def csr_subgraph(self, B, sid, nid, average=False):
+        N = len(sid)
+        sid = np.ascontiguousarray(sid, dtype=np.int32)
+        nid = np.ascontiguousarray(nid, dtype=np.int32)
+        rp = np.zeros(B + 1, np.int32); ci = np.zeros(N, np.int32); v = np.zeros(N, np.float32)
+        self.lib.orc_csr_subgraph(B, N, _ptr(sid), _ptr(nid), int(average), _ptr(rp), _ptr(ci), _ptr(v))
+        return rp, ci, v
+
+    # ---- tensor ops
+    def spmm(self, rp, ci, v, Bm, m, alpha=1.0, beta=0.0, C=None):
+        Bm = np.ascontiguousarray(Bm, np.float32)
+        n = Bm.shape[1]
+        out = np.zeros((m, n), np.float32) if C is None else np.array(C, dtype=np.float32, copy=True)
+        self.lib.orc_spmm_csr(m, n, ctypes.c_float(alpha), _ptr(rp), _ptr(ci), _ptr(v), _ptr(Bm), n,
+                              ctypes.c_float(beta), _ptr(out), n)
+        return out
+
+    def spmm_T(self, rp, ci, v, Bm, m, k, alpha=1.0, beta=0.0, C=None):
+        Bm = np.ascontiguousarray(Bm, np.float32)
+        n = Bm.shape[1]
+        out = np.zeros((k, n), np.float32) if C is None else np.array(C, dtype=np.float32, copy=True)
+        self.lib.orc_spmm_csr_T(m, n, k, ctypes.c_float(alpha), _ptr(rp), _ptr(ci), _ptr(v), _ptr(Bm), n,
+                                ctypes.c_float(beta), _ptr(out), n)
+        return out
+
+    def gemm(self, A, Bm, transA=False, transB=False, alpha=1.0, beta=0.0, C=None):
+        A = np.ascontiguousarray(A, np.float32); Bm = np.ascontiguousarray(Bm, np.float32)
+        m = A.shape[1] if transA else A.shape[0]
+        k = A.shape[0] if transA else A.shape[1]
+        n = Bm.shape[0] if transB else Bm.shape[1]
+        out = np.zeros((m, n), np.float32) if C is None else np.array(C, dtype=np.float32, copy=True)
+        self.lib.orc_gemm(int(transA), int(transB), m, n, k, ctypes.c_float(alpha), _ptr(A), A.shape[1],
+                          _ptr(Bm), Bm.shape[1], ctypes.c_float(beta), _ptr(out), n)
+        return out
+
+    def axpy(self, a, x, y):
+        y = np.array(y, np.float32, copy=True); x = np.ascontiguousarray(x, np.float32)
+        self.lib.orc_axpy(ctypes.c_size_t(x.size), ctypes.c_float(a), _ptr(x), _ptr(y))
+        return y
+
+    def axpby(self, a, x, b, y):
+        y = np.array(y, np.float32, copy=True); x = np.ascontiguousarray(x, np.float32)
+        self.lib.orc_axpby(ctypes.c_size_t(x.size), ctypes.c_float(a), _ptr(x), ctypes.c_float(b), _ptr(y))
+        return y
+
+    def unary(self, op, x, a0=0.0, a1=0.0):
+        x = np.array(x, np.float32, copy=True)
+        self.lib.orc_unary(int(op), _ptr(x), ctypes.c_size_t(x.size), ctypes.c_float(a0), ctypes.c_float(a1))
+        return x
+
+    def row_softmax(self, x):
+        x = np.array(x, np.float32, copy=True)
+        self.lib.orc_row_softmax(_ptr(x), x.shape[0], x.shape[1])
+        return x
+
+    def jagged_softmax(self, x, lens):
+        x = np.array(x, np.float32, copy=True); lens = np.ascontiguousarray(lens, np.int32)
+        self.lib.orc_jagged_softmax(_ptr(x), _ptr(lens), len(lens))
+        return x
+
+    def sum(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        return float(self.lib.orc_sum(_ptr(x), ctypes.c_size_t(x.size)))
+
+    def mean(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        return float(self.lib.orc_mean(_ptr(x), ctypes.c_size_t(x.size)))
+
+    def max(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        return float(self.lib.orc_max(_ptr(x), ctypes.c_size_t(x.size)))
+
+    def row_argmax(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.zeros(x.shape[0], np.int32)
+        self.lib.orc_row_argmax(_ptr(x), x.shape[0], x.shape[1], _ptr(out))
+        return out
+
+    def csr_row_argmax(self, rp, ci, v):
+        out = np.zeros(len(rp) - 1, np.int32)
+        self.lib.orc_csr_row_argmax(_ptr(rp), _ptr(ci), _ptr(v), len(rp) - 1, _ptr(out))
+        return out
+
+    def cross_entropy(self, prob, rp, ci, v):
+        prob = np.ascontiguousarray(prob, np.float32)
+        out = np.zeros(prob.shape[0], np.float32)
+        self.lib.orc_cross_entropy(_ptr(prob), prob.shape[0], prob.shape[1], _ptr(rp), _ptr(ci), _ptr(v), _ptr(out))
+        return out
+
+    def in_top_k(self, pred, label, k=1):
+        pred = np.ascontiguousarray(pred, np.float32); label = np.ascontiguousarray(label, np.int32)
+        out = np.zeros(pred.shape[0], np.int32)
+        self.lib.orc_in_top_k(_ptr(pred), _ptr(label), pred.shape[0], pred.shape[1], k, _ptr(out))
+        return out
+
+    def cast(self, src):
+        src = np.ascontiguousarray(src, np.int32)
+        dst = np.zeros(src.shape, np.float32)
+        self.lib.orc_cast_i32_f32(_ptr(src), _ptr(dst), ctypes.c_size_t(src.size))
+        return dst
+
+    def level(self, rp, ci, v, h_in, W, msg=None, bias=None):
+        h_in = np.ascontiguousarray(h_in, np.float32); W = np.ascontiguousarray(W, np.float32)
+        N, C = h_in.shape
+        tmp = np.zeros((N, C), np.float32); out = np.zeros((N, C), np.float32)
+        msg_p = _ptr(np.ascontiguousarray(msg, np.float32)) if msg is not None else None
+        bias_a = np.ascontiguousarray(bias, np.float32) if bias is not None else None
+        self.lib.orc_s2v_level(N, C, _ptr(rp), _ptr(ci), _ptr(v), _ptr(h_in), _ptr(W), msg_p,
+                               _ptr(bias_a) if bias_a is not None else None, _ptr(tmp), _ptr(out))
+        return out
+
+    def forward(self, a_csr, s_csr, X, w, L, label_csr=None):
+        X = np.ascontiguousarray(X, np.float32)
+        N, K = X.shape
+        C, H, Q = w.W_n2l.shape[1], w.W_h1.shape[1], w.W_h2.shape[1]
+        B = len(s_csr[0]) - 1
+        f = np.float32
+        out = dict(msg=np.zeros((N, C), f), h=np.zeros((L + 1, N, C), f), pool=np.zeros((B, C), f),
+                   hidden=np.zeros((B, H), f), logits=np.zeros((B, Q), f), probs=np.zeros((B, Q), f),
+                   loss_rows=np.zeros(B, f), pred=np.zeros(B, np.int32), truth=np.zeros(B, np.int32),
+                   hit=np.zeros(B, np.int32), scalars=np.zeros(2, f))
+        Ws = [np.ascontiguousarray(a, f) for a in (w.W_n2l, w.W_conv, w.W_h1, w.W_h2)]
+        lab = [(_ptr(a) if label_csr is not None else None) for a in (label_csr or (None, None, None))]
+        self.lib.orc_s2v_forward(N, B, K, C, H, Q, L, _ptr(a_csr[0]), _ptr(a_csr[1]), _ptr(a_csr[2]),
+                                 _ptr(s_csr[0]), _ptr(s_csr[1]), _ptr(s_csr[2]), _ptr(X),
+                                 _ptr(Ws[0]), _ptr(Ws[1]), _ptr(Ws[2]), _ptr(Ws[3]), lab[0], lab[1], lab[2],
+                                 _ptr(out["msg"]), _ptr(out["h"]), _ptr(out["pool"]), _ptr(out["hidden"]),
+                                 _ptr(out["logits"]), _ptr(out["probs"]), _ptr(out["loss_rows"]),
+                                 _ptr(out["pred"]), _ptr(out["truth"]), _ptr(out["hit"]), _ptr(out["scalars"]))
+        return out
+
+
+@pytest.fixture(scope="session")
+def oracle():
+    return Oracle()
+
+
+@pytest.fixture(scope="session")
+def ref_graph():
+    """The reference's own GraphStruct compiled into oracle/_ref (None when not built)."""
+    if not os.path.exists(_REF_PATH):
+        return None
+    return ctypes.CDLL(_REF_PATH)
+
+
+def max_rel(a, b, floor=None):
+    """Parity metric for fp32 tensors: max_i |a_i - b_i| / max(|a_i|, |b_i|, floor).
+
+    The floor defaults to 1% of the reference tensor's largest magnitude.  A fixed
+    tiny floor is not usable: post-ReLU activations are sums with cancellation, so an
+    element that is 1e-5 of the tensor's scale legitimately differs by parts in 1e-2
+    between two correct fp32 summation orders.  With this floor the 1e-4 bound reads
+    "relative 1e-4 on every element that matters, absolute 1e-6 x scale on the rest".
+    """
+    a = np.asarray(a, np.float64); b = np.asarray(b, np.float64)
+    if a.size == 0:
+        return 0.0
+    if floor is None:
+        floor = max(1e-2 * float(np.max(np.abs(b))), 1e-30)
+    return float(np.max(np.abs(a - b) / np.maximum(np.maximum(np.abs(a), np.abs(b)), floor)))
+
+
+PARITY_TOL = 1e-4     # the north-star tolerance for fp32 activations and logits
+
+
+@pytest.fixture(scope="session")
+def gpu():
+    """torch CUDA device + initialised gnnhip library; GPU tests fail loudly without either."""
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a HIP device"
+    from graphnn_amd import ops
+    ops.init(0)
+    return torch.device("cuda:0")

@@ -1,0 +1,500 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle on identical seeded inputs.
+
+Bit-exact for integer / index outputs and for single-rounding element-wise ops;
+PARITY_TOL = 1e-4 (see conftest.max_rel for the floor) for fp32 sums.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from conftest import PARITY_TOL, max_rel
+from graphnn_amd import batching, synth
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _t(a, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _n(t):
+    return t.detach().cpu().numpy()
+
+
+def _csr_t(csr, dev):
+    return tuple(_t(a, dev) for a in csr)
+
+
+def _random_csr(rng, m, k, nnz, unit=False, sort_cols=False):
+    rows = np.sort(rng.integers(0, m, nnz))
+    rp = np.zeros(m + 1, np.int32)
+    np.cumsum(np.bincount(rows, minlength=m), out=rp[1:])
+    ci = rng.integers(0, max(k, 1), nnz).astype(np.int32)
+    if sort_cols:
+        order = np.lexsort((ci, rows))
+        ci = ci[order]
+    v = np.ones(nnz, np.float32) if unit else rng.standard_normal(nnz).astype(np.float32)
+    return rp, ci, v
+
+
+# ------------------------------------------------------------------ SpMM
+def test_spmm_known_answer(gpu, oracle):
+    from graphnn_amd import ops
+    g = json.load(open(os.path.join(GOLDEN, "sparse_mm_known_answer.json")))
+    csr = (np.array(g["row_ptr"], np.int32), np.array(g["col_idx"], np.int32), np.array(g["val"], np.float32))
+    B = np.array(g["b_for_normal"], np.float32)
+    got = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), g["a_rows"]))
+    assert np.array_equal(got, np.array(g["expected_A_b"], np.float32))
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 7, 16, 32, 64, 100, 128, 256, 300, 512, 1100])
+def test_spmm_widths_random_values(gpu, oracle, n):
+    from graphnn_amd import ops
+    rng = np.random.default_rng(100 + n)
+    m, k = 517, 389                        # not multiples of any group count
+    csr = _random_csr(rng, m, k, 4000)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    C0 = rng.standard_normal((m, n)).astype(np.float32)
+    want = oracle.spmm(*csr, B, m)
+    got = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m))
+    assert max_rel(got, want) < PARITY_TOL
+    want2 = oracle.spmm(*csr, B, m, alpha=0.5, beta=-2.0, C=C0)
+    got2 = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m, alpha=0.5, beta=-2.0, out=_t(C0, gpu)))
+    assert max_rel(got2, want2) < PARITY_TOL
+
+
+@pytest.mark.parametrize("n", [2, 64, 128, 256])
+def test_spmm_unit_weights_bit_exact(gpu, oracle, n):
+    """unit edge weights and row-order accumulation: same additions in the same order as the oracle"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(200 + n)
+    m = 3001
+    csr = _random_csr(rng, m, m, 30000, unit=True, sort_cols=True)
+    B = rng.standard_normal((m, n)).astype(np.float32)
+    got = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m))
+    assert np.array_equal(got, oracle.spmm(*csr, B, m))
+
+
+def test_spmm_edge_cases(gpu, oracle):
+    from graphnn_amd import ops
+    import torch
+    rng = np.random.default_rng(3)
+    n = 64
+    # all rows empty; beta = 0 must overwrite NaN garbage
+    rp = np.zeros(11, np.int32)
+    ci = np.zeros(0, np.int32); v = np.zeros(0, np.float32)
+    B = rng.standard_normal((5, n)).astype(np.float32)
+    out = torch.full((10, n), float("nan"), device=gpu)
+    got = _n(ops.spmm(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(B, gpu), 10, out=out))
+    assert np.array_equal(got, np.zeros((10, n), np.float32))
+    # identity
+    m = 300
+    eye = (np.arange(m + 1, dtype=np.int32), np.arange(m, dtype=np.int32), np.ones(m, np.float32))
+    X = rng.standard_normal((m, n)).astype(np.float32)
+    assert np.array_equal(_n(ops.spmm(*_csr_t(eye, gpu), _t(X, gpu), m)), X)
+    # single row, single column
+    one = (np.array([0, 3], np.int32), np.array([0, 0, 0], np.int32), np.array([1, 2, 3], np.float32))
+    X1 = rng.standard_normal((1, 4)).astype(np.float32)
+    assert max_rel(_n(ops.spmm(*_csr_t(one, gpu), _t(X1, gpu), 1)), oracle.spmm(*one, X1, 1)) < PARITY_TOL
+    # operand validation happens on the host
+    with pytest.raises(ValueError):
+        ops.spmm(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(B, gpu), 12)
+
+
+@pytest.mark.parametrize("n", [64, 128, 6])
+def test_spmm_long_rows(gpu, oracle, n):
+    """rows far longer than the per-group limit take the whole-workgroup path (hub vertices)"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(4)
+    m, k = 70, 5000
+    lens = rng.integers(0, 12, m)
+    lens[3] = 5000; lens[4] = 2049; lens[40] = 9000; lens[69] = 2048
+    rp = np.zeros(m + 1, np.int32); np.cumsum(lens, out=rp[1:])
+    nnz = int(rp[-1])
+    ci = rng.integers(0, k, nnz).astype(np.int32)
+    v = rng.standard_normal(nnz).astype(np.float32)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    want = oracle.spmm(rp, ci, v, B, m)
+    got = _n(ops.spmm(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(B, gpu), m))
+    assert max_rel(got, want) < PARITY_TOL
+    # twice the same input: identical bits (no atomics, fixed combination order)
+    got_again = _n(ops.spmm(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(B, gpu), m))
+    assert np.array_equal(got, got_again)
+
+
+# ------------------------------------------------------------------ GEMM
+@pytest.mark.parametrize("shape", [(1, 1, 1), (7, 5, 3), (64, 64, 16), (65, 63, 17), (300, 2, 32), (1000, 64, 38), (33, 130, 70)])
+def test_gemm_all_transposes(gpu, oracle, shape):
+    from graphnn_amd import ops
+    m, n, k = shape
+    rng = np.random.default_rng(sum(shape))
+    for ta in (False, True):
+        for tb in (False, True):
+            A = rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32)
+            B = rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32)
+            C0 = rng.standard_normal((m, n)).astype(np.float32)
+            got = _n(ops.gemm(_t(A, gpu), _t(B, gpu), ta, tb))
+            assert max_rel(got, oracle.gemm(A, B, ta, tb)) < PARITY_TOL, (ta, tb)
+            got2 = _n(ops.gemm(_t(A, gpu), _t(B, gpu), ta, tb, alpha=1.5, beta=-0.5, out=_t(C0, gpu)))
+            assert max_rel(got2, oracle.gemm(A, B, ta, tb, alpha=1.5, beta=-0.5, C=C0)) < PARITY_TOL, (ta, tb)
+
+
+def test_gemm_reference_test_shape(gpu, oracle):
+    """10x20 . (30x20)^T with |delta ASum| <= 1e-4 (test/gpu_tensor_test.cpp:131-149)"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(5)
+    A = rng.standard_normal((10, 20)).astype(np.float32); B = rng.standard_normal((30, 20)).astype(np.float32)
+    got = _n(ops.gemm(_t(A, gpu), _t(B, gpu), False, True))
+    want = oracle.gemm(A, B, False, True)
+    assert abs(float(np.abs(got).sum()) - float(np.abs(want).sum())) <= 1e-4 * 30
+    with pytest.raises(ValueError):
+        ops.gemm(_t(A, gpu), _t(B, gpu), False, False)
+
+
+# ------------------------------------------------------------------ element-wise engine
+EXACT_UNARY = [("set", 0, 3.5, 0.0), ("truncate", 1, -0.5, 0.75), ("scale", 2, -1.75, 0.0), ("add", 3, 0.125, 0.0),
+               ("abs", 4, 0, 0), ("relu", 6, 0, 0), ("square", 12, 0, 0)]
+CLOSE_UNARY = [("inv", 5), ("sigmoid", 7), ("tanh", 8), ("exp", 11)]
+POS_UNARY = [("log", 9), ("invsqrt", 10), ("sqrt", 13)]
+
+
+@pytest.mark.parametrize("n,offset", [(1, 0), (3, 0), (1024, 0), (100003, 0), (4099, 1), (4099, 3)])
+def test_unary_engine(gpu, oracle, n, offset):
+    """offset > 0 gives a pointer that is not 16-byte aligned (a row view), exercising the scalar path"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(n + offset)
+    base = (rng.standard_normal(n + offset) * 2).astype(np.float32)
+    base[offset::7] = -0.0
+    x = base[offset:]
+    for name, code, a0, a1 in EXACT_UNARY:
+        buf = _t(base, gpu)
+        ops.unary(name, buf[offset:], a0, a1)
+        got = _n(buf)
+        assert np.array_equal(got[offset:].view(np.uint32), oracle.unary(code, x, a0, a1).view(np.uint32)), name
+        assert np.array_equal(got[:offset], base[:offset])
+    for name, code in CLOSE_UNARY:
+        buf = _t(base, gpu)
+        ops.unary(name, buf[offset:])
+        assert np.allclose(_n(buf)[offset:], oracle.unary(code, x), rtol=2e-6, atol=1e-7), name
+    pos = np.abs(base) + np.float32(0.01)
+    for name, code in POS_UNARY:
+        buf = _t(pos, gpu)
+        ops.unary(name, buf[offset:])
+        assert np.allclose(_n(buf)[offset:], oracle.unary(code, pos[offset:]), rtol=2e-6, atol=1e-7), name
+
+
+def test_relu_keeps_negative_zero_and_nan(gpu):
+    from graphnn_amd import ops
+    x = np.array([-1.0, -0.0, 0.0, 2.0, np.nan, -np.inf, np.inf, -1e-45], np.float32)
+    got = _n(ops.relu(_t(x, gpu)))
+    assert np.array_equal(got[[0, 2, 3, 5, 6, 7]], np.array([0, 0, 2, 0, np.inf, 0], np.float32))
+    assert got[1] == 0 and np.signbit(got[1]) and np.isnan(got[4])
+
+
+@pytest.mark.parametrize("n", [1, 5, 4096, 250001])
+def test_axpy_add_cast(gpu, oracle, n):
+    from graphnn_amd import ops
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float32); y = rng.standard_normal(n).astype(np.float32)
+    assert np.array_equal(_n(ops.axpy(1.0, _t(x, gpu), _t(y, gpu))), oracle.axpy(1.0, x, y))      # one rounded add
+    assert np.array_equal(_n(ops.add(_t(x, gpu), _t(y, gpu))), x + y)
+    assert np.allclose(_n(ops.axpy(0.3, _t(x, gpu), _t(y, gpu))), oracle.axpy(0.3, x, y), rtol=1e-6, atol=1e-7)
+    assert np.allclose(_n(ops.axpby(0.3, _t(x, gpu), -1.5, _t(y, gpu))), oracle.axpby(0.3, x, -1.5, y), rtol=1e-6, atol=1e-7)
+    ints = rng.integers(-2**30, 2**30, n).astype(np.int32)
+    assert np.array_equal(_n(ops.cast_i32_f32(_t(ints, gpu))), oracle.cast(ints))
+    with pytest.raises(ValueError):
+        ops.axpy(1.0, _t(x, gpu), _t(np.zeros(n + 1, np.float32), gpu))
+
+
+@pytest.mark.parametrize("n,offset", [(1, 0), (15, 1), (16, 0), (1000, 3), (1 << 20, 5)])
+def test_memset0(gpu, n, offset):
+    import torch
+    from graphnn_amd import ops
+    buf = torch.full((n + offset + 7,), 7, dtype=torch.uint8, device=gpu)
+    ops.memset0(buf[offset:offset + n])
+    got = _n(buf)
+    assert np.all(got[offset:offset + n] == 0) and np.all(got[:offset] == 7) and np.all(got[offset + n:] == 7)
+
+
+# ------------------------------------------------------------------ softmax family
+@pytest.mark.parametrize("rows,cols", [(20, 200), (256, 2), (7, 1), (3, 64), (5, 65), (2, 5000)])
+def test_row_softmax(gpu, oracle, rows, cols):
+    from graphnn_amd import ops
+    rng = np.random.default_rng(rows * cols)
+    x = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
+    got = _n(ops.row_softmax(_t(x, gpu)))
+    want = oracle.row_softmax(x)
+    assert float(np.abs(got - want).sum()) <= 1e-4              # the reference's own bound (gpu_tensor_test.cpp:151-166)
+    assert max_rel(got, want) < PARITY_TOL
+    assert np.allclose(got.sum(axis=1), 1.0, atol=1e-5)
+
+
+def test_jagged_softmax(gpu, oracle):
+    from graphnn_amd import ops
+    rng = np.random.default_rng(6)
+    x = (1.0 + rng.random(10)).astype(np.float32)
+    lens = np.array([2, 3, 5], np.int32)                        # gpu_tensor_test.cpp:182-209, bound 1e-5
+    got = _n(ops.jagged_softmax(_t(x, gpu), _t(lens, gpu)))
+    assert float(np.abs(got - oracle.jagged_softmax(x, lens)).sum()) <= 1e-5
+    # ragged: empty segments, length-1 segments, one long segment, > 1024 segments (several scan chunks)
+    lens2 = rng.integers(0, 40, 3000).astype(np.int32)
+    lens2[[0, 17, 2999]] = 0
+    lens2[5] = 1
+    lens2[1234] = 20000
+    total = int(lens2.sum())
+    x2 = (rng.standard_normal(total) * 2).astype(np.float32)
+    got2 = _n(ops.jagged_softmax(_t(x2, gpu), _t(lens2, gpu)))
+    want2 = oracle.jagged_softmax(x2, lens2)
+    assert max_rel(got2, want2) < PARITY_TOL
+    sums = np.add.reduceat(got2.astype(np.float64), np.concatenate([[0], np.cumsum(lens2)[:-1]])[lens2 > 0])
+    assert np.allclose(sums, 1.0, atol=1e-4)
+
+
+# ------------------------------------------------------------------ reductions and index ops
+@pytest.mark.parametrize("n", [1, 63, 256, 4000, 16385, 3_000_001])
+def test_reduce(gpu, oracle, n):
+    from graphnn_amd import ops
+    rng = np.random.default_rng(n)
+    x = (1.0 + rng.random(n)).astype(np.float32)                # U(1,2): the reference's Mean test distribution
+    xd = _t(x, gpu)
+    ref64 = x.astype(np.float64)
+    assert abs(float(_n(ops.reduce("sum", xd))[0]) - ref64.sum()) <= 1e-5 * ref64.sum()
+    assert abs(float(_n(ops.reduce("mean", xd))[0]) - ref64.mean()) <= 1e-5     # gpu_tensor_test.cpp:168-180
+    assert float(_n(ops.reduce("max", xd))[0]) == oracle.max(x)
+    ints = rng.integers(-50, 50, min(n, 100000)).astype(np.float32)
+    assert float(_n(ops.reduce("sum", _t(ints, gpu)))[0]) == float(ints.astype(np.float64).sum())   # exact in fp32
+
+
+def test_row_argmax(gpu, oracle):
+    from graphnn_amd import ops
+    rng = np.random.default_rng(7)
+    big = rng.standard_normal((10, 1023)).astype(np.float32)     # gpu_tensor_test.cpp:111-129
+    assert np.array_equal(_n(ops.row_argmax(_t(big, gpu))), oracle.row_argmax(big))
+    ties = np.array([[1, 3, 3, 2], [5, 5, 5, 5], [-1, -2, -0.5, -0.5], [0.0, -0.0, 0.0, 0.0]], np.float32)
+    assert list(_n(ops.row_argmax(_t(ties, gpu)))) == [1, 0, 2, 0]
+    withnan = np.array([[np.nan, 9, 1], [1, np.nan, 3], [2, 5, np.nan], [-np.inf, np.nan, -np.inf]], np.float32)
+    assert np.array_equal(_n(ops.row_argmax(_t(withnan, gpu))), oracle.row_argmax(withnan))
+    # many rows with heavy ties: small integer values
+    tied = rng.integers(0, 3, (5000, 130)).astype(np.float32)
+    assert np.array_equal(_n(ops.row_argmax(_t(tied, gpu))), oracle.row_argmax(tied))
+    two = rng.standard_normal((256, 2)).astype(np.float32)
+    assert np.array_equal(_n(ops.row_argmax(_t(two, gpu))), oracle.row_argmax(two))
+
+
+def test_label_ops(gpu, oracle):
+    from graphnn_amd import ops
+    rng = np.random.default_rng(8)
+    B, Q = 1000, 6
+    # general CSR label rows: 0..3 entries per row
+    lens = rng.integers(0, 4, B)
+    rp = np.zeros(B + 1, np.int32); np.cumsum(lens, out=rp[1:])
+    nnz = int(rp[-1])
+    ci = rng.integers(0, Q, nnz).astype(np.int32)
+    v = rng.integers(0, 3, nnz).astype(np.float32)              # ties between stored values
+    assert np.array_equal(_n(ops.csr_row_argmax(_t(rp, gpu), _t(ci, gpu), _t(v, gpu))), oracle.csr_row_argmax(rp, ci, v))
+    prob = oracle.row_softmax(rng.standard_normal((B, Q)).astype(np.float32) * 4)
+    prob[3, :] = 0.0                                             # exercises the 1e-8 clamp
+    got = _n(ops.cross_entropy(_t(prob, gpu), _t(rp, gpu), _t(ci, gpu), _t(v, gpu)))[:, 0]
+    assert np.allclose(got, oracle.cross_entropy(prob, rp, ci, v), rtol=1e-6, atol=1e-7)
+    label = rng.integers(0, Q, B).astype(np.int32)
+    pred = rng.integers(0, 4, (B, Q)).astype(np.float32)         # ties
+    for k in (1, 2, 3):
+        assert np.array_equal(_n(ops.in_top_k(_t(pred, gpu), _t(label, gpu), k)), oracle.in_top_k(pred, label, k))
+    wide = rng.standard_normal((50, 300)).astype(np.float32)
+    wl = rng.integers(0, 300, 50).astype(np.int32)
+    assert np.array_equal(_n(ops.in_top_k(_t(wide, gpu), _t(wl, gpu), 5)), oracle.in_top_k(wide, wl, 5))
+
+
+# ------------------------------------------------------------------ fused stages
+def _small_problem(seed, B, K, C, H, Q, lo=3, hi=40):
+    batch = synth.molecule_batch(seed, B, K, Q, size_mode="uniform", size_lo=lo, size_hi=hi)
+    w = synth.make_weights(synth.Stream(seed), K, C, H, Q)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    return batch, w, a, s
+
+
+@pytest.mark.parametrize("C", [16, 32, 64, 48, 128])
+@pytest.mark.parametrize("K", [7, 38, 64])
+def test_input_stage(gpu, oracle, C, K):
+    from graphnn_amd import ops
+    batch, w, a, s = _small_problem(10 + C + K, 9, K, C, 8, 2)
+    X = batch.one_hot()
+    X += (np.random.default_rng(C).standard_normal(X.shape) * 0.01).astype(np.float32)    # dense, not just one-hot
+    msg, h0 = ops.s2v_input(_t(X, gpu), _t(w.W_n2l, gpu))
+    want = oracle.gemm(X, w.W_n2l)
+    assert max_rel(_n(msg), want) < PARITY_TOL
+    assert np.array_equal(_n(h0), np.maximum(_n(msg), 0))       # ReLU of what was stored, exactly
+
+
+@pytest.mark.parametrize("C", [16, 32, 64, 48, 128])
+@pytest.mark.parametrize("with_msg,with_bias", [(True, False), (True, True), (False, False)])
+def test_level_stage(gpu, oracle, C, with_msg, with_bias):
+    from graphnn_amd import ops
+    batch, w, a, s = _small_problem(20 + C, 40, 5, C, 8, 2)
+    rng = np.random.default_rng(C)
+    N = batch.num_nodes
+    h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
+    msg = rng.standard_normal((N, C)).astype(np.float32) if with_msg else None
+    bias = rng.standard_normal(C).astype(np.float32) if with_bias else None
+    want = oracle.level(*a, h_in, w.W_conv, msg, bias)
+    got = _n(ops.s2v_level(*_csr_t(a, gpu), _t(h_in, gpu), _t(w.W_conv, gpu),
+                           _t(msg, gpu) if with_msg else None, _t(bias, gpu) if with_bias else None))
+    assert max_rel(got, want) < PARITY_TOL
+    assert np.all(got >= 0)
+
+
+def test_level_stage_hub_rows_and_weights(gpu, oracle):
+    """one vertex with thousands of in-neighbours (whole-workgroup gather) and non-unit edge weights"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(9)
+    N, C = 5000, 64
+    lens = rng.integers(0, 6, N); lens[17] = 4000; lens[4999] = 1500; lens[2048] = 1025
+    rp = np.zeros(N + 1, np.int32); np.cumsum(lens, out=rp[1:])
+    nnz = int(rp[-1])
+    ci = rng.integers(0, N, nnz).astype(np.int32)
+    v = (rng.random(nnz) * 0.1).astype(np.float32)
+    h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
+    W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
+    msg = rng.standard_normal((N, C)).astype(np.float32)
+    want = oracle.level(rp, ci, v, h_in, W, msg, None)
+    got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu)))
+    assert max_rel(got, want) < PARITY_TOL
+
+
+@pytest.mark.parametrize("C,H,Q", [(64, 32, 2), (16, 8, 3), (32, 100, 70), (48, 16, 2), (128, 64, 5)])
+def test_readout_stage(gpu, oracle, C, H, Q):
+    from graphnn_amd import ops
+    batch, w, a, s = _small_problem(30 + C, 33, 5, C, H, Q, lo=1, hi=300)
+    rng = np.random.default_rng(C + H)
+    h = np.maximum(rng.standard_normal((batch.num_nodes, C)), 0).astype(np.float32)
+    pool, hidden, logits, probs, pred = (_n(t) for t in ops.s2v_readout(*_csr_t(s, gpu), _t(h, gpu), _t(w.W_h1, gpu),
+                                                                        _t(w.W_h2, gpu), batch.num_graphs))
+    w_pool = oracle.spmm(*s, h, batch.num_graphs)
+    w_hidden = np.maximum(oracle.gemm(w_pool, w.W_h1), 0)
+    w_logits = oracle.gemm(w_hidden, w.W_h2)
+    assert max_rel(pool, w_pool) < PARITY_TOL
+    assert max_rel(hidden, w_hidden) < PARITY_TOL
+    assert max_rel(logits, w_logits) < PARITY_TOL
+    assert max_rel(probs, oracle.row_softmax(w_logits)) < PARITY_TOL
+    assert np.array_equal(pred, oracle.row_argmax(logits))      # arg-max of the logits the device produced: exact
+
+
+# ------------------------------------------------------------------ whole forward, configurations 1 and 2
+def _forward_case(gpu, oracle, config_id, B=None):
+    from graphnn_amd import ops
+    batch, w, cfg = synth.make_config(config_id, B=B)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    lab = batch.label_csr()
+    want = oracle.forward(a, s, X, w, cfg["L"], lab)
+    bufs = ops.s2v_forward(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+                           _t(w.W_h1, gpu), _t(w.W_h2, gpu), cfg["L"])
+    got = dict(msg=_n(bufs.msg), h_final=_n(bufs.h_final), pool=_n(bufs.pool), hidden=_n(bufs.hidden),
+               logits=_n(bufs.logits), probs=_n(bufs.probs), pred=_n(bufs.pred))
+    return batch, cfg, a, s, X, w, lab, want, got, bufs
+
+
+@pytest.mark.parametrize("config_id", [1, 2])
+def test_forward_matches_reference_path(gpu, oracle, config_id):
+    from graphnn_amd import ops
+    batch, cfg, a, s, X, w, lab, want, got, bufs = _forward_case(gpu, oracle, config_id)
+    assert max_rel(got["msg"], want["msg"]) < PARITY_TOL
+    assert max_rel(got["h_final"], want["h"][cfg["L"]]) < PARITY_TOL
+    for key in ("pool", "hidden", "logits", "probs"):
+        assert max_rel(got[key], want[key]) < PARITY_TOL, key
+    # argmax predictions bit-exact with the reference path
+    assert np.array_equal(got["pred"], want["pred"])
+    # loss / accuracy tail of the graph, operator by operator on the device
+    lab_d = _csr_t(lab, gpu)
+    loss_rows = ops.cross_entropy(bufs.probs, *lab_d)
+    truth = ops.csr_row_argmax(*lab_d)
+    hit = ops.in_top_k(bufs.logits, truth, 1)
+    loss = float(_n(ops.reduce("mean", loss_rows))[0])
+    acc = float(_n(ops.reduce("mean", ops.cast_i32_f32(hit)))[0])
+    assert np.array_equal(_n(truth), want["truth"])
+    assert np.array_equal(_n(hit), want["hit"])
+    assert np.allclose(_n(loss_rows)[:, 0], want["loss_rows"], rtol=1e-4)
+    assert abs(loss - want["scalars"][0]) <= 1e-4 * abs(want["scalars"][0])
+    assert abs(acc - want["scalars"][1]) <= 1e-6
+
+
+def test_forward_every_level_matches(gpu, oracle):
+    """level by level through the per-level entry point, against each of the oracle's stored h_l"""
+    from graphnn_amd import ops
+    batch, w, cfg = synth.make_config(2, B=64)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    want = oracle.forward(a, s, X, w, cfg["L"], batch.label_csr())
+    a_d = _csr_t(a, gpu)
+    msg, h = ops.s2v_input(_t(X, gpu), _t(w.W_n2l, gpu))
+    assert max_rel(_n(h), want["h"][0]) < PARITY_TOL
+    Wc = _t(w.W_conv, gpu)
+    for lv in range(cfg["L"]):
+        h = ops.s2v_level(*a_d, h, Wc, msg)
+        assert max_rel(_n(h), want["h"][lv + 1]) < PARITY_TOL, lv
+
+
+def test_forward_unfused_operator_route_agrees(gpu, oracle):
+    """the same forward built from the general operators (the route FactorGraph takes op by op)"""
+    from graphnn_amd import ops
+    batch, cfg, a, s, X, w, lab, want, got, bufs = _forward_case(gpu, oracle, 1)
+    a_d, s_d = _csr_t(a, gpu), _csr_t(s, gpu)
+    Wn, Wc, W1, W2 = (_t(m, gpu) for m in (w.W_n2l, w.W_conv, w.W_h1, w.W_h2))
+    msg = ops.gemm(_t(X, gpu), Wn)
+    h = ops.relu(msg)
+    for _ in range(cfg["L"]):
+        pool = ops.spmm(*a_d, h, batch.num_nodes)
+        lin = ops.gemm(pool, Wc)
+        merged = ops.add(lin, msg)
+        h = ops.relu(merged)
+    y = ops.spmm(*s_d, h, batch.num_graphs)
+    hidden = ops.relu(ops.gemm(y, W1))
+    logits = ops.gemm(hidden, W2)
+    probs = ops.row_softmax(logits.clone())
+    assert max_rel(_n(logits), want["logits"]) < PARITY_TOL
+    assert max_rel(_n(probs), want["probs"]) < PARITY_TOL
+    assert max_rel(_n(logits), got["logits"]) < PARITY_TOL
+    assert np.array_equal(_n(ops.row_argmax(logits)), want["pred"])
+
+
+def test_forward_is_deterministic_and_reuses_buffers(gpu, oracle):
+    from graphnn_amd import ops
+    batch, cfg, a, s, X, w, lab, want, got, bufs = _forward_case(gpu, oracle, 1)
+    args = (_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu), _t(w.W_h1, gpu), _t(w.W_h2, gpu))
+    for _ in range(3):
+        ops.s2v_forward(*args, cfg["L"], bufs=bufs)
+        assert np.array_equal(_n(bufs.logits), got["logits"])
+        assert np.array_equal(_n(bufs.h_final), got["h_final"])
+
+
+# ------------------------------------------------------------------ pool allocator
+def test_pool_recycles_blocks(gpu):
+    import ctypes
+    from graphnn_amd import _lib as binding
+    lib = binding.load_library()
+    used0, parked0, allocs0 = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    lib.gnnhip_pool_stats(ctypes.byref(used0), ctypes.byref(parked0), ctypes.byref(allocs0))
+    p = ctypes.c_void_p(); q = ctypes.c_void_p()
+    assert lib.gnnhip_malloc(ctypes.byref(p), 1 << 20) == 0
+    assert lib.gnnhip_recycle(p) == 0
+    assert lib.gnnhip_malloc(ctypes.byref(q), (1 << 20) - 4096) == 0     # smallest parked block that is large enough
+    assert q.value == p.value
+    used, parked, allocs = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    lib.gnnhip_pool_stats(ctypes.byref(used), ctypes.byref(parked), ctypes.byref(allocs))
+    assert allocs.value == allocs0.value + 1
+    # h2d / d2h round trip through the library's own copies
+    src = np.arange(1000, dtype=np.float32); dst = np.zeros_like(src)
+    P = lambda arr: arr.ctypes.data_as(ctypes.c_void_p)
+    assert lib.gnnhip_memcpy_h2d(q, P(src), src.nbytes, None) == 0
+    assert lib.gnnhip_memcpy_d2h(P(dst), q, src.nbytes, None) == 0
+    assert np.array_equal(src, dst)
+    assert lib.gnnhip_free(q) == 0
+    assert lib.gnnhip_recycle(q) == -1                                   # no longer owned by the pool

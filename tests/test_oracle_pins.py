@@ -1,0 +1,405 @@
+"""Pins the CPU oracle (oracle/s2v_oracle.c) before anything is compared with it.
+
+Each oracle function is checked against something that does not share its code:
+brute force in float64, closed forms, invariants, the reference's own known-answer
+matrix, the reference's own GraphStruct container (oracle/_ref, when built) and,
+when libmkl_rt can be loaded, Intel MKL called with the argument pattern graphnn's
+CPU tensors use (mkl_scsrmm "GLNC", cblas_sgemm row-major).
+"""
+import ctypes
+import json
+import os
+
+import numpy as np
+import pytest
+
+from conftest import max_rel
+from graphnn_amd import batching, synth
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _rng(seed):
+    return np.random.default_rng(seed)
+
+
+# ------------------------------------------------------------------ CSR builders
+def _random_graph(rng, N, E, B):
+    ex = rng.integers(0, N, E).astype(np.int32)
+    ey = rng.integers(0, N, E).astype(np.int32)
+    sid = np.sort(rng.integers(0, B, N)).astype(np.int32)
+    nid = np.arange(N, dtype=np.int32)
+    return ex, ey, sid, nid
+
+
+def test_csr_node2node_bruteforce(oracle):
+    rng = _rng(1)
+    for N, E in [(1, 0), (5, 7), (40, 200), (64, 64)]:
+        ex, ey, _, _ = _random_graph(rng, N, E, 1)
+        rp, ci, v = oracle.csr_node2node(N, ex, ey)
+        # invariants
+        assert rp[0] == 0 and rp[N] == E and np.all(np.diff(rp) >= 0)
+        # brute force: row y holds the sources of edges into y, in edge order
+        for y in range(N):
+            want = [int(ex[e]) for e in range(E) if ey[e] == y]
+            assert list(ci[rp[y]:rp[y + 1]]) == want
+        assert np.all(v == 1.0)
+        # dense adjacency counts (duplicates accumulate)
+        dense = np.zeros((N, N), np.int64)
+        for e in range(E):
+            dense[ey[e], ex[e]] += 1
+        rebuilt = np.zeros((N, N), np.int64)
+        for y in range(N):
+            for t in range(rp[y], rp[y + 1]):
+                rebuilt[y, ci[t]] += 1
+        assert np.array_equal(dense, rebuilt)
+
+
+def test_csr_average_values(oracle):
+    rng = _rng(2)
+    ex, ey, sid, nid = _random_graph(rng, 30, 90, 4)
+    rp, ci, v = oracle.csr_node2node(30, ex, ey, average=True)
+    for y in range(30):
+        d = rp[y + 1] - rp[y]
+        if d:
+            assert np.all(v[rp[y]:rp[y + 1]] == np.float32(1.0 / d))
+    rp, ci, v = oracle.csr_subgraph(4, sid, nid, average=True)
+    for g in range(4):
+        d = rp[g + 1] - rp[g]
+        if d:
+            assert np.all(v[rp[g]:rp[g + 1]] == np.float32(1.0 / d))
+
+
+def test_csr_subgraph_contiguous(oracle):
+    b = synth.molecule_batch(7, 12, 5)
+    rp, ci, v = oracle.csr_subgraph(b.num_graphs, b.subg_id, b.node_idx)
+    assert np.array_equal(ci, np.arange(b.num_nodes))            # identity permutation
+    assert np.array_equal(rp, np.concatenate([[0], np.cumsum(b.graph_sizes)]))
+    assert np.all(v == 1.0)
+
+
+def test_csr_undirected_batch_is_symmetric_and_sorted(oracle):
+    b = synth.molecule_batch(11, 20, 7)
+    rp, ci, _ = oracle.csr_node2node(b.num_nodes, b.edge_x, b.edge_y)
+    assert rp[-1] == b.num_edges
+    dense = np.zeros((b.num_nodes, b.num_nodes), np.int32)
+    for y in range(b.num_nodes):
+        row = ci[rp[y]:rp[y + 1]]
+        assert np.all(np.diff(row) > 0)                           # ascending, no duplicates
+        dense[y, row] = 1
+    assert np.array_equal(dense, dense.T)
+    # block diagonal: no edge leaves its graph
+    off = np.concatenate([[0], np.cumsum(b.graph_sizes)])
+    gid = np.repeat(np.arange(b.num_graphs), b.graph_sizes)
+    rows = np.repeat(np.arange(b.num_nodes), np.diff(rp))
+    assert np.array_equal(gid[rows], gid[ci])
+    assert off[-1] == b.num_nodes
+
+
+def test_csr_against_reference_graphstruct(oracle, ref_graph):
+    if ref_graph is None:
+        pytest.skip("oracle/_ref/libref_graph.so not built (reference tree absent)")
+    rng = _rng(3)
+    for N, E, B in [(1, 0, 1), (9, 20, 3), (200, 1000, 17)]:
+        ex, ey, sid, nid = _random_graph(rng, N, E, B)
+        # AddNode order need not be sorted by subgraph: shuffle it
+        perm = rng.permutation(N)
+        sid, nid = sid[perm].copy(), nid[perm].copy()
+        P = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+        arp = np.zeros(N + 1, np.int32); aci = np.zeros(E, np.int32)
+        srp = np.zeros(B + 1, np.int32); sci = np.zeros(N, np.int32)
+        rc = ref_graph.ref_graph_to_csr(B, N, E, P(sid), P(nid), P(ex), P(ey), P(arp), P(aci), P(srp), P(sci))
+        assert rc == 0
+        rp, ci, _ = oracle.csr_node2node(N, ex, ey)
+        assert np.array_equal(rp, arp) and np.array_equal(ci, aci)
+        rp, ci, _ = oracle.csr_subgraph(B, sid, nid)
+        assert np.array_equal(rp, srp) and np.array_equal(ci, sci)
+
+
+def test_host_batching_matches_oracle(oracle):
+    """the product's numpy CSR builders are bit-exact with the oracle (and thereby with GraphStruct)"""
+    rng = _rng(4)
+    for avg in (False, True):
+        for N, E, B in [(1, 0, 1), (50, 300, 6), (1000, 5000, 40)]:
+            ex, ey, sid, nid = _random_graph(rng, N, E, B)
+            for got, want in zip(batching.node2node_csr(N, ex, ey, avg), oracle.csr_node2node(N, ex, ey, avg)):
+                assert got.dtype == want.dtype and np.array_equal(got, want)
+            for got, want in zip(batching.subgraph_csr(B, sid, nid, avg), oracle.csr_subgraph(B, sid, nid, avg)):
+                assert got.dtype == want.dtype and np.array_equal(got, want)
+
+
+# ------------------------------------------------------------------ SpMM / GEMM
+def _random_csr(rng, m, k, nnz):
+    rows = np.sort(rng.integers(0, m, nnz))
+    rp = np.zeros(m + 1, np.int32)
+    np.cumsum(np.bincount(rows, minlength=m), out=rp[1:])
+    ci = rng.integers(0, max(k, 1), nnz).astype(np.int32)
+    v = rng.standard_normal(nnz).astype(np.float32)
+    return rp, ci, v
+
+
+def _dense_of(rp, ci, v, m, k):
+    A = np.zeros((m, k), np.float64)
+    for i in range(m):
+        for t in range(rp[i], rp[i + 1]):
+            A[i, ci[t]] += float(v[t])
+    return A
+
+
+def test_spmm_known_answer(oracle):
+    g = json.load(open(os.path.join(GOLDEN, "sparse_mm_known_answer.json")))
+    rp = np.array(g["row_ptr"], np.int32); ci = np.array(g["col_idx"], np.int32); v = np.array(g["val"], np.float32)
+    got = oracle.spmm(rp, ci, v, np.array(g["b_for_normal"], np.float32), g["a_rows"])
+    assert np.array_equal(got, np.array(g["expected_A_b"], np.float32))
+    got_t = oracle.spmm_T(rp, ci, v, np.array(g["b_for_transpose"], np.float32), g["a_rows"], g["a_cols"])
+    assert np.array_equal(got_t, np.array(g["expected_At_b"], np.float32))
+
+
+def test_spmm_bruteforce_identity_duplicates(oracle):
+    rng = _rng(5)
+    m, k, n = 37, 23, 11
+    rp, ci, v = _random_csr(rng, m, k, 300)            # 300 entries over 37x23: duplicates certain
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    C0 = rng.standard_normal((m, n)).astype(np.float32)
+    want = 0.5 * _dense_of(rp, ci, v, m, k) @ B.astype(np.float64) + 2.0 * C0
+    got = oracle.spmm(rp, ci, v, B, m, alpha=0.5, beta=2.0, C=C0)
+    assert max_rel(got, want, 1.0) < 1e-5
+    # identity
+    n_id = 19
+    rp_i = np.arange(n_id + 1, dtype=np.int32); ci_i = np.arange(n_id, dtype=np.int32); v_i = np.ones(n_id, np.float32)
+    X = rng.standard_normal((n_id, 8)).astype(np.float32)
+    assert np.array_equal(oracle.spmm(rp_i, ci_i, v_i, X, n_id), X)
+    # beta = 0 ignores what was in C, even NaN
+    Cn = np.full((m, n), np.nan, np.float32)
+    assert np.all(np.isfinite(oracle.spmm(rp, ci, v, B, m, C=Cn)))
+    # empty rows give zeros
+    rp_e = np.zeros(5, np.int32)
+    assert np.array_equal(oracle.spmm(rp_e, ci[:0], v[:0], B, 4), np.zeros((4, n), np.float32))
+    # transpose
+    Bt = rng.standard_normal((m, n)).astype(np.float32)
+    want_t = _dense_of(rp, ci, v, m, k).T @ Bt.astype(np.float64)
+    assert max_rel(oracle.spmm_T(rp, ci, v, Bt, m, k), want_t, 1.0) < 1e-5
+
+
+def test_gemm_bruteforce_all_transposes(oracle):
+    rng = _rng(6)
+    m, n, k = 13, 9, 21
+    for ta in (False, True):
+        for tb in (False, True):
+            A = rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32)
+            B = rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32)
+            C0 = rng.standard_normal((m, n)).astype(np.float32)
+            opA = A.T if ta else A
+            opB = B.T if tb else B
+            want = 1.5 * opA.astype(np.float64) @ opB.astype(np.float64) - 0.5 * C0
+            got = oracle.gemm(A, B, ta, tb, alpha=1.5, beta=-0.5, C=C0)
+            assert max_rel(got, want, 1.0) < 1e-5, (ta, tb)
+    # the reference's own GEMM test shape: 10x20 . (30x20)^T, |delta ASum| <= 1e-4 (test/gpu_tensor_test.cpp:131-149)
+    A = rng.standard_normal((10, 20)).astype(np.float32); B = rng.standard_normal((30, 20)).astype(np.float32)
+    got = oracle.gemm(A, B, False, True)
+    want = A.astype(np.float64) @ B.astype(np.float64).T
+    assert abs(np.abs(got).sum() - np.abs(want).sum()) <= 1e-4 * 30
+
+
+# ------------------------------------------------------------------ MKL (the reference's arithmetic dependency)
+def _load_mkl():
+    os.environ.setdefault("MKL_THREADING_LAYER", "SEQUENTIAL")
+    for name in ("libmkl_rt.so.1", "libmkl_rt.so", "/opt/conda/lib/libmkl_rt.so.1", "/opt/conda/lib/libmkl_rt.so"):
+        try:
+            return ctypes.CDLL(name)
+        except OSError:
+            continue
+    return None
+
+
+def test_spmm_and_gemm_against_mkl(oracle):
+    mkl = _load_mkl()
+    if mkl is None:
+        pytest.skip("libmkl_rt not loadable on this host")
+    rng = _rng(7)
+    P = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    ci_t, cf = ctypes.c_int, ctypes.c_float
+    # mkl_scsrmm('N', m, n, k, alpha, "GLNC", val, col_idx, row_ptr, row_ptr + 1, B, ldb, beta, C, ldc)
+    # as called by DTensor<CPU>::MM(SpTensor...) (src/tensor/cpu_dense_tensor.cpp:221-224)
+    m, k, n = 101, 77, 64
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    for trans, rows_out in ((b"N", m), (b"T", k)):
+        rp, ci, v = _random_csr(rng, m, k, 900)
+        if trans == b"T":
+            # MKL's transposed kernel does not accumulate repeated (row, col) coordinates
+            # (observed with oneMKL 2021.4), so the 'T' comparison uses a duplicate-free matrix;
+            # the 'N' orientation, the one the forward uses, is compared with duplicates present.
+            key = np.unique(np.repeat(np.arange(m), np.diff(rp)).astype(np.int64) * k + ci)
+            rows_u, ci = key // k, (key % k).astype(np.int32)
+            rp = np.zeros(m + 1, np.int32); np.cumsum(np.bincount(rows_u, minlength=m), out=rp[1:])
+            v = v[:len(key)].copy()
+        Bm = B if trans == b"N" else rng.standard_normal((m, n)).astype(np.float32)
+        C = np.zeros((rows_out, n), np.float32)
+        mm, nn, kk, al, be, ld = ci_t(m), ci_t(n), ci_t(k), cf(1.25), cf(0.0), ci_t(n)
+        pe = rp[1:]
+        mkl.mkl_scsrmm(ctypes.c_char_p(trans), ctypes.byref(mm), ctypes.byref(nn), ctypes.byref(kk), ctypes.byref(al),
+                       ctypes.c_char_p(b"GLNC"), P(v), P(ci), P(rp), P(pe), P(Bm), ctypes.byref(ld), ctypes.byref(be),
+                       P(C), ctypes.byref(ld))
+        got = oracle.spmm(rp, ci, v, Bm, m, alpha=1.25) if trans == b"N" else oracle.spmm_T(rp, ci, v, Bm, m, k, alpha=1.25)
+        assert max_rel(got, C, 1.0) < 1e-5, trans
+    # cblas_sgemm(CblasRowMajor=101, NoTrans=111 / Trans=112, ...) (cpu_dense_tensor.cpp:206-210)
+    for ta in (False, True):
+        for tb in (False, True):
+            M, N, K = 33, 17, 40
+            A = rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+            Bd = rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+            C = np.zeros((M, N), np.float32)
+            mkl.cblas_sgemm(101, 112 if ta else 111, 112 if tb else 111, M, N, K, cf(1.0), P(A), A.shape[1],
+                            P(Bd), Bd.shape[1], cf(0.0), P(C), N)
+            assert max_rel(oracle.gemm(A, Bd, ta, tb), C, 1.0) < 1e-5, (ta, tb)
+
+
+# ------------------------------------------------------------------ element-wise
+def test_unary_closed_forms(oracle):
+    x = np.array([-2.5, -0.0, 0.0, 0.3, 1.0, 4.0, np.nan], np.float32)
+    relu = oracle.unary(6, x)
+    assert np.array_equal(relu[:6], np.array([0.0, -0.0, 0.0, 0.3, 1.0, 4.0], np.float32))
+    assert np.signbit(relu[1]) and np.isnan(relu[6])             # -0.0 and NaN pass through
+    assert np.array_equal(oracle.unary(0, x, 3.0), np.full(7, 3.0, np.float32))
+    assert np.array_equal(oracle.unary(1, x[:6], -1.0, 1.0), np.clip(x[:6], -1.0, 1.0))
+    assert np.array_equal(oracle.unary(2, x[:6], 2.0), x[:6] * np.float32(2.0))
+    assert np.array_equal(oracle.unary(3, x[:6], 2.0), x[:6] + np.float32(2.0))
+    assert np.array_equal(oracle.unary(4, x[:6]), np.abs(x[:6]))
+    assert np.array_equal(oracle.unary(12, x[:6]), x[:6] * x[:6])
+    pos = np.array([0.25, 1.0, 9.0], np.float32)
+    assert np.array_equal(oracle.unary(13, pos), np.array([0.5, 1.0, 3.0], np.float32))
+    assert np.array_equal(oracle.unary(5, pos), np.float32(1.0) / pos)
+    assert np.allclose(oracle.unary(10, pos), 1.0 / np.sqrt(pos.astype(np.float64)), rtol=1e-6)
+    y = np.linspace(-3, 3, 13).astype(np.float32)
+    assert np.allclose(oracle.unary(7, y), 1.0 / (1.0 + np.exp(-y.astype(np.float64))), rtol=1e-6)
+    assert np.allclose(oracle.unary(8, y), np.tanh(y.astype(np.float64)), rtol=2e-6, atol=1e-7)
+    assert np.allclose(oracle.unary(11, y), np.exp(y.astype(np.float64)), rtol=1e-6)
+    assert np.allclose(oracle.unary(9, pos), np.log(pos.astype(np.float64)), rtol=1e-6, atol=1e-7)
+
+
+def test_axpy_axpby_exact(oracle):
+    rng = _rng(8)
+    x = rng.standard_normal(1001).astype(np.float32); y = rng.standard_normal(1001).astype(np.float32)
+    assert np.array_equal(oracle.axpy(1.0, x, y), x + y)         # single rounded add
+    assert np.array_equal(oracle.axpy(-1.0, x, y), y - x)
+    a, b = np.float32(0.75), np.float32(-1.5)
+    assert np.array_equal(oracle.axpby(0.75, x, -1.5, y), a * x + b * y)
+    assert np.array_equal(oracle.cast(np.array([-3, 0, 7, 2**24 + 1], np.int32)),
+                          np.array([-3, 0, 7, 2**24 + 1], np.int32).astype(np.float32))
+
+
+# ------------------------------------------------------------------ softmax family
+def test_softmax_properties(oracle):
+    rng = _rng(9)
+    x = rng.standard_normal((20, 200)).astype(np.float32)        # the reference's test shape
+    p = oracle.row_softmax(x)
+    assert np.allclose(p.sum(axis=1), 1.0, atol=1e-5)
+    assert np.all(p > 0)
+    assert max_rel(oracle.row_softmax(x + np.float32(5.0)), p, 1e-6) < 1e-4     # shift invariance
+    e = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True))
+    assert np.abs(p - e / e.sum(axis=1, keepdims=True)).sum() <= 1e-4          # ASum(diff) <= 1e-4
+    two = rng.standard_normal((50, 2)).astype(np.float32)
+    sig = 1.0 / (1.0 + np.exp(-(two[:, 0].astype(np.float64) - two[:, 1])))
+    assert np.allclose(oracle.row_softmax(two)[:, 0], sig, rtol=1e-6)
+    big = np.array([[1000.0, 1000.0, -1000.0]], np.float32)                     # no overflow
+    assert np.allclose(oracle.row_softmax(big), [[0.5, 0.5, 0.0]])
+
+
+def test_jagged_softmax_equals_per_segment(oracle):
+    rng = _rng(10)
+    x = (1.0 + rng.random(10)).astype(np.float32)                 # U(1,2), lens {2,3,5}: the reference's test
+    lens = np.array([2, 3, 5], np.int32)
+    got = oracle.jagged_softmax(x, lens)
+    off = 0
+    for ln in lens:
+        seg = x[off:off + ln].astype(np.float64)
+        e = np.exp(seg - seg.max())
+        assert np.abs(got[off:off + ln] - e / e.sum()).sum() <= 1e-5
+        assert np.array_equal(got[off:off + ln], oracle.row_softmax(x[off:off + ln][None, :])[0])
+        off += ln
+    # ragged with empty segments
+    lens2 = np.array([0, 4, 0, 1, 5, 0], np.int32)
+    g2 = oracle.jagged_softmax(x, lens2)
+    assert np.isclose(g2[0:4].sum(), 1.0, atol=1e-6) and g2[4] == 1.0 and np.isclose(g2[5:].sum(), 1.0, atol=1e-6)
+
+
+# ------------------------------------------------------------------ reductions, arg-max, CE, top-k
+def test_reductions(oracle):
+    ints = np.arange(1, 1001, dtype=np.float32)
+    assert oracle.sum(ints) == 500500.0 and oracle.mean(ints) == 500.5 and oracle.max(ints) == 1000.0
+    rng = _rng(11)
+    x = (1.0 + rng.random((20, 200))).astype(np.float32)          # U(1,2) 20x200: reference Mean test, tol 1e-5
+    assert abs(oracle.mean(x) - x.astype(np.float64).mean()) <= 1e-5
+
+
+def test_argmax_rules(oracle):
+    x = np.array([[1, 3, 3, 2], [5, 5, 5, 5], [-1, -2, -0.5, -0.5], [0.0, -0.0, 0.0, 0.0]], np.float32)
+    assert list(oracle.row_argmax(x)) == [1, 0, 2, 0]             # first index among ties
+    rng = _rng(12)
+    big = rng.standard_normal((10, 1023)).astype(np.float32)       # reference ArgMax test shape
+    assert np.array_equal(oracle.row_argmax(big), big.argmax(axis=1).astype(np.int32))
+    withnan = np.array([[np.nan, 9, 1], [1, np.nan, 3], [2, 5, np.nan]], np.float32)
+    assert list(oracle.row_argmax(withnan)) == [0, 2, 1]          # strict '>' never selects a later NaN
+    # CSR rows: first largest stored value wins, empty row -> 0
+    rp = np.array([0, 1, 1, 4, 6], np.int32)
+    ci = np.array([2, 0, 3, 1, 4, 0], np.int32)
+    v = np.array([1.0, 0.5, 0.9, 0.9, -2.0, -1.0], np.float32)
+    assert list(oracle.csr_row_argmax(rp, ci, v)) == [2, 0, 3, 0]
+
+
+def test_cross_entropy_and_top_k(oracle):
+    prob = np.array([[0.25, 0.75], [1.0, 0.0], [0.5, 0.5]], np.float32)
+    rp = np.array([0, 1, 2, 3], np.int32); ci = np.array([1, 1, 0], np.int32); v = np.ones(3, np.float32)
+    got = oracle.cross_entropy(prob, rp, ci, v)
+    want = np.array([-np.log(0.75), -np.log(1e-8), -np.log(0.5)])
+    assert np.allclose(got, want, rtol=1e-6)
+    # weighted multi-entry label row
+    rp2 = np.array([0, 2], np.int32); ci2 = np.array([0, 1], np.int32); v2 = np.array([0.25, 0.75], np.float32)
+    got2 = oracle.cross_entropy(prob[:1], rp2, ci2, v2)
+    assert np.isclose(got2[0], -(0.25 * np.log(0.25) + 0.75 * np.log(0.75)), rtol=1e-6)
+    pred = np.array([[0.1, 0.9, 0.0], [0.3, 0.3, 0.4], [0.2, 0.2, 0.2]], np.float32)
+    label = np.array([1, 0, 2], np.int32)
+    assert list(oracle.in_top_k(pred, label, 1)) == [1, 0, 1]     # ties do not count against the target
+    assert list(oracle.in_top_k(pred, label, 2)) == [1, 1, 1]
+
+
+# ------------------------------------------------------------------ level and forward compose the pinned ops
+def _forward_float64(a_csr, s_csr, X, w, L):
+    N = X.shape[0]; B = len(s_csr[0]) - 1
+    A = _dense_of(*a_csr, N, N); S = _dense_of(*s_csr, B, N)
+    msg = X.astype(np.float64) @ w.W_n2l.astype(np.float64)
+    h = np.maximum(msg, 0)
+    hs = [h]
+    for _ in range(L):
+        h = np.maximum(A @ h @ w.W_conv.astype(np.float64) + msg, 0)
+        hs.append(h)
+    pool = S @ h
+    hidden = np.maximum(pool @ w.W_h1.astype(np.float64), 0)
+    logits = hidden @ w.W_h2.astype(np.float64)
+    e = np.exp(logits - logits.max(axis=1, keepdims=True))
+    return dict(msg=msg, h=np.stack(hs), pool=pool, hidden=hidden, logits=logits, probs=e / e.sum(axis=1, keepdims=True))
+
+
+def test_forward_against_float64_dense_model(oracle):
+    batch, w, cfg = synth.make_config(1, B=12)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    got = oracle.forward(a, s, X, w, cfg["L"], batch.label_csr())
+    want = _forward_float64(a, s, X, w, cfg["L"])
+    for key in ("msg", "h", "pool", "hidden", "logits", "probs"):
+        assert max_rel(got[key], want[key]) < 1e-4, key
+    assert np.array_equal(got["pred"], want["logits"].argmax(axis=1))
+    assert np.array_equal(got["truth"], batch.graph_label)
+    assert np.array_equal(got["hit"], (got["pred"] == batch.graph_label).astype(np.int32))
+    lp = -np.log(want["probs"][np.arange(batch.num_graphs), batch.graph_label])
+    assert np.allclose(got["loss_rows"], lp, rtol=1e-4)
+    assert np.isclose(got["scalars"][0], lp.mean(), rtol=1e-4)
+    assert np.isclose(got["scalars"][1], got["hit"].mean(), rtol=1e-6)
+    # the level with bias: (pool * W + b) + msg, then ReLU
+    rng = _rng(13)
+    bias = rng.standard_normal(cfg["C"]).astype(np.float32)
+    lvl = oracle.level(*a, got["h"][0], w.W_conv, got["msg"], bias)
+    A = _dense_of(*a, batch.num_nodes, batch.num_nodes)
+    want_lvl = np.maximum(A @ got["h"][0].astype(np.float64) @ w.W_conv.astype(np.float64) + bias + got["msg"], 0)
+    assert max_rel(lvl, want_lvl) < 1e-4
