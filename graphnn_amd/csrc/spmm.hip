@@ -256,7 +256,7 @@ extern "C" int gnnhip_spmm_csr_f32(int m, int k, int n, float alpha, const int* 
     if (m == 0 || n == 0) return GNNHIP_OK;
     GNNHIP_REQUIRE(row_ptr && C, "null row_ptr or output in spmm");
     GNNHIP_REQUIRE(ldb >= n && ldc >= n, "leading dimension smaller than n in spmm (ldb=%d ldc=%d n=%d)", ldb, ldc, n);
-    GNNHIP_REQUIRE(k == 0 || (col_idx && val && B), "null operand in spmm");
+    GNNHIP_REQUIRE(k == 0 || B, "null dense operand in spmm");   // col_idx / val may be null when A has no entries
     if (int rc = require_ready()) return rc;
     return spmm_dispatch(m, n, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, as_stream(stream));
 }
