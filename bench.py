@@ -108,7 +108,7 @@ def cpu_baseline(host, budget_s=12.0):
         orc.forward(host["a"], host["s"], host["X"], host["w"], cfg["L"], None)
         reps += 1
         el = time.perf_counter() - t0
-        if el >= budget_s or reps >= 2000:
+        if el >= budget_s or reps >= 100000:
             break
     return dict(value=batch.num_graphs * reps / el, unit="graphs/s", cores=threads, kind="port",
                 sample="%d forwards of the same configuration-2 batch in %.1f s (gcc -O3 -mavx2, OpenMP over rows)" % (reps, el))
@@ -121,6 +121,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-spmm", action="store_true", help="skip the configuration-3 SpMM roofline leg")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch one element-wise copy kernel of known size (1 GiB read, 1 GiB written) "
+                         "so hardware counters collected over this run can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -168,6 +171,14 @@ def main():
         }
     else:
         out["roofline"] = None
+
+    if args.calibrate:
+        n = 1 << 28
+        src = torch.ones(n, device=dev, dtype=torch.float32)
+        dst = torch.empty_like(src)
+        ops.relu(src, dst)              # map1_kernel<FReLU>: reads 4n bytes, writes 4n bytes
+        torch.cuda.synchronize()
+        out["calibration"] = {"kernel": "map1_kernel<FReLU>", "bytes_read": 4 * n, "bytes_written": 4 * n}
 
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline(host)
     print(json.dumps(out))

@@ -23,6 +23,11 @@
 // Workgroups are persistent over tiles so W is loaded into LDS once per group.
 #include "gnnhip_internal.h"
 
+// Phase markers for a timing build of this file; they expand to nothing in the library.
+#ifndef GNNHIP_PHASE_MARK
+#define GNNHIP_PHASE_MARK(i)
+#endif
+
 namespace gnnhip {
 namespace {
 
@@ -35,6 +40,38 @@ __device__ __forceinline__ void f4_fma(float4& a, float s, const float4& x)
     a.x += s * x.x; a.y += s * x.y; a.z += s * x.z; a.w += s * x.w;
 }
 __device__ __forceinline__ float relu_ref(float v) { return v < 0.f ? 0.f : v; }
+
+// Copy N4 float4s (a compile-time count) from global to LDS.  All of a lane's loads are
+// issued before the first LDS store, so the copy costs one memory round trip.
+template <int N4>
+__device__ __forceinline__ void copy_to_lds_fixed(float* dst, const float* __restrict__ src, int tid)
+{
+    constexpr int FULL = N4 / kBlock, REM = N4 % kBlock;
+    const float4* s4 = reinterpret_cast<const float4*>(src);
+    float4* d4 = reinterpret_cast<float4*>(dst);
+    float4 r[FULL + 1];
+#pragma unroll
+    for (int i = 0; i < FULL; ++i) r[i] = s4[tid + i * kBlock];
+    if (REM && tid < REM) r[FULL] = s4[tid + FULL * kBlock];
+#pragma unroll
+    for (int i = 0; i < FULL; ++i) d4[tid + i * kBlock] = r[i];
+    if (REM && tid < REM) d4[tid + FULL * kBlock] = r[FULL];
+}
+
+// Run-time count: four loads in flight per lane.
+__device__ __forceinline__ void copy_to_lds(float* dst, const float* __restrict__ src, int n4, int tid)
+{
+    const float4* s4 = reinterpret_cast<const float4*>(src);
+    float4* d4 = reinterpret_cast<float4*>(dst);
+    int base = 0;
+    for (; base + 4 * kBlock <= n4; base += 4 * kBlock) {
+        const float4 r0 = s4[base + tid], r1 = s4[base + tid + kBlock];
+        const float4 r2 = s4[base + tid + 2 * kBlock], r3 = s4[base + tid + 3 * kBlock];
+        d4[base + tid] = r0; d4[base + tid + kBlock] = r1;
+        d4[base + tid + 2 * kBlock] = r2; d4[base + tid + 3 * kBlock] = r3;
+    }
+    for (int idx = base + tid; idx < n4; idx += kBlock) d4[idx] = s4[idx];
+}
 
 // acc[r] += tile[row(r)][0..kdim) * Ws[0..kdim)[4tx..4tx+3]
 template <int C, int RT>
@@ -77,8 +114,7 @@ __global__ __launch_bounds__(kBlock) void s2v_input_kernel(
     float* tile = smem + (size_t)K * C;            // [R][ldt]
     const int tid = threadIdx.x, tx = tid % G, ty = tid / G;
 
-    for (int i = tid; i < K * C / 4; i += kBlock)
-        reinterpret_cast<float4*>(Ws)[i] = reinterpret_cast<const float4*>(Wn2l)[i];
+    copy_to_lds(Ws, Wn2l, K * C / 4, tid);
 
     const int ntiles = (N + R - 1) / R;
     for (int tile_id = blockIdx.x; tile_id < ntiles; tile_id += gridDim.x) {
@@ -87,9 +123,18 @@ __global__ __launch_bounds__(kBlock) void s2v_input_kernel(
         __syncthreads();                           // previous tile consumed; Ws visible on the first pass
         // rows of X are contiguous in memory: copy rows*K floats, coalesced
         const float* src = X + (size_t)row0 * K;
-        for (int i = tid; i < R * K; i += kBlock) {
-            const int r = i / K, c = i - r * K;
-            tile[(size_t)r * ldt + c] = (r < rows) ? src[i] : 0.f;
+        for (int base = 0; base < R * K; base += 4 * kBlock) {
+            float xv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i = base + tid + u * kBlock;
+                xv[u] = (i < rows * K) ? src[i] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i = base + tid + u * kBlock;
+                if (i < R * K) { const int r = i / K; tile[(size_t)r * ldt + (i - r * K)] = xv[u]; }
+            }
         }
         __syncthreads();
 
@@ -113,53 +158,110 @@ __global__ __launch_bounds__(kBlock) void s2v_input_kernel(
 }
 
 // ---------------------------------------------------------------- level
-template <int C, int RT>
+// Wave-autonomous: each wavefront owns tiles of 16 rows and never synchronises with
+// another wavefront.  Per tile:
+//   1. gather-sum: G = C/4 lanes per row gather float4 slices of the neighbours' rows
+//      (64/G rows at a time) and park the sums in a wave-private LDS tile [16][C+4];
+//   2. contraction on the matrix cores: out^T = W^T * tile^T with
+//      v_mfma_f32_16x16x4_f32, W^T held in registers for the lifetime of the wavefront.
+//      Lane (q = lane/16, t = lane%16) feeds k = (C/4) q + s at step s, and the output
+//      columns of block jb are permuted so that the lane ends up owning row t,
+//      columns (C/4) q .. (C/4) q + C/4 - 1: contiguous float4s for the epilogue;
+//   3. epilogue: + bias + msg, ReLU, float4 stores.
+typedef float mfma_f4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWaveLongRow = 256;   // entries; longer rows are gathered by all groups of the wavefront together
+
+template <int C>
 __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
     int N, const int* __restrict__ row_ptr, const int* __restrict__ col_idx, const float* __restrict__ val,
     const float* __restrict__ h_in, const float* __restrict__ W, const float* __restrict__ msg,
     const float* __restrict__ bias, float* __restrict__ h_out)
 {
-    constexpr int G = C / 4, P = kBlock / G, R = RT * P, LDT = C + 4;
-    extern __shared__ float smem[];
-    float* Ws = smem;                              // [C][C]
-    float* tile = Ws + C * C;                      // [R][LDT]   gathered A*h rows
-    float* red = tile + R * LDT;                   // [P][C]     partial sums for long rows
-    __shared__ int lr_list[R];
-    __shared__ int lr_count;
+    constexpr int G = C / 4;             // lanes per gathered row
+    constexpr int RPR = kWave / G;       // rows gathered per round
+    constexpr int ROUNDS = 16 / RPR;     // rounds per tile
+    constexpr int KS = C / 4;            // contraction steps
+    constexpr int NJB = C / 16;          // 16-column output blocks
+    constexpr int LDT = C + 4;
+    constexpr int kWavesPerBlock = kBlock / kWave;
 
-    const int tid = threadIdx.x, tx = tid % G, ty = tid / G;
+    __shared__ float lds[kWavesPerBlock][16 * LDT + RPR * C];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    float* tile = lds[wave];             // [16][LDT]
+    float* red = tile + 16 * LDT;        // [RPR][C]
+    const int q = lane >> 4, t = lane & 15;
+    const int grp = lane / G, tx = lane % G;
 
-    for (int i = tid; i < C * C / 4; i += kBlock)
-        reinterpret_cast<float4*>(Ws)[i] = reinterpret_cast<const float4*>(W)[i];
-
-    const int ntiles = (N + R - 1) / R;
-    for (int tile_id = blockIdx.x; tile_id < ntiles; tile_id += gridDim.x) {
-        const long long row0 = (long long)tile_id * R;
-        const int rows = (int)min((long long)R, (long long)N - row0);
-        if (tid == 0) lr_count = 0;
-        __syncthreads();                           // previous tile consumed, counter reset, Ws visible
-
-        // ---- phase 1: gather-sum, group ty owns local rows ty + r*P
+    GNNHIP_PHASE_MARK(0);
+    // W^T operand: wreg[jb][s] = W[KS q + s][KS (t/4) + 4 jb + t%4]
+    float wreg[NJB][KS];
 #pragma unroll
-        for (int r = 0; r < RT; ++r) {
-            const int lr = ty + r * P;
-            int start = 0, end = 0;
-            if (lr < rows) { start = row_ptr[row0 + lr]; end = row_ptr[row0 + lr + 1]; }
-            if (end - start > kLongRow) {
-                if (tx == 0) lr_list[atomicAdd(&lr_count, 1)] = lr;
-                end = start;
+    for (int jb = 0; jb < NJB; ++jb)
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+            wreg[jb][s] = W[(size_t)(KS * q + s) * C + KS * (t >> 2) + 4 * jb + (t & 3)];
+    GNNHIP_PHASE_MARK(1);
+
+    const long long ntiles = ((long long)N + 15) / 16;
+    const long long wave_stride = (long long)gridDim.x * kWavesPerBlock;
+    for (long long tile_id = (long long)blockIdx.x * kWavesPerBlock + wave; tile_id < ntiles; tile_id += wave_stride) {
+        const long long row0 = tile_id * 16;
+        // one coalesced load of the 17 row pointers of this tile
+        int rp = 0;
+        if (lane <= 16) rp = row_ptr[min(row0 + lane, (long long)N)];
+
+        int st[ROUNDS], en[ROUNDS], c0[ROUNDS];
+        float v0[ROUNDS];
+        bool is_long[ROUNDS];
+#pragma unroll
+        for (int rd = 0; rd < ROUNDS; ++rd) {
+            const int lr = rd * RPR + grp;
+            st[rd] = __shfl(rp, lr, kWave);
+            en[rd] = __shfl(rp, lr + 1, kWave);
+            is_long[rd] = (en[rd] - st[rd] > kWaveLongRow);
+            if (is_long[rd]) en[rd] = st[rd];
+            c0[rd] = 0;
+            v0[rd] = 0.f;
+            if (st[rd] + tx < en[rd]) { c0[rd] = col_idx[st[rd] + tx]; v0[rd] = val[st[rd] + tx]; }
+        }
+
+        // ---- gather-sum; the first four neighbours of every row of the tile are fetched together
+        float4 x[ROUNDS][4];
+        float vv[ROUNDS][4];
+#pragma unroll
+        for (int rd = 0; rd < ROUNDS; ++rd) {
+            const int cnt = en[rd] - st[rd];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int cj = __shfl(c0[rd], u & (G - 1), G);
+                vv[rd][u] = __shfl(v0[rd], u & (G - 1), G);
+                x[rd][u] = (u < cnt && u < G) ? *reinterpret_cast<const float4*>(h_in + (size_t)cj * C + tx * 4) : f4_zero();
             }
+        }
+#pragma unroll
+        for (int rd = 0; rd < ROUNDS; ++rd) {
+            const int lr = rd * RPR + grp;
+            const int cnt_all = en[rd] - st[rd];
             float4 acc = f4_zero();
-            for (int base = start; base < end; base += G) {
-                const int t = base + tx;
-                int c = 0;
-                float v = 0.f;
-                if (t < end) { c = col_idx[t]; v = val[t]; }
-                const int cnt = min(G, end - base);
-                for (int j = 0; j < cnt; j += 4) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (u < cnt_all && u < G) f4_fma(acc, vv[rd][u], x[rd][u]);
+            // the rest of the row: entries 4.. of the first batch, then further batches of G
+            for (int base = st[rd]; base < en[rd]; base += G) {
+                int c = c0[rd];
+                float v = v0[rd];
+                int j0 = (G > 4) ? 4 : G;          // the first batch has had its first min(4, G) entries consumed
+                if (base != st[rd]) {
+                    c = 0; v = 0.f; j0 = 0;
+                    if (base + tx < en[rd]) { c = col_idx[base + tx]; v = val[base + tx]; }
+                }
+                const int cnt = min(G, en[rd] - base);
+                for (int j = j0; j < cnt; j += 4) {
                     int cj[4];
                     float vj[4];
-                    float4 x[4];
+                    float4 xx[4];
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
                         cj[u] = __shfl(c, (j + u) & (G - 1), G);
@@ -167,65 +269,85 @@ __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
                     }
 #pragma unroll
                     for (int u = 0; u < 4; ++u)
-                        x[u] = (j + u < cnt) ? *reinterpret_cast<const float4*>(h_in + (size_t)cj[u] * C + tx * 4) : f4_zero();
+                        xx[u] = (j + u < cnt) ? *reinterpret_cast<const float4*>(h_in + (size_t)cj[u] * C + tx * 4) : f4_zero();
 #pragma unroll
                     for (int u = 0; u < 4; ++u)
-                        if (j + u < cnt) f4_fma(acc, vj[u], x[u]);
+                        if (j + u < cnt) f4_fma(acc, vj[u], xx[u]);
                 }
             }
-            *reinterpret_cast<float4*>(tile + (size_t)lr * LDT + tx * 4) = acc;
+            *reinterpret_cast<float4*>(tile + lr * LDT + tx * 4) = acc;
         }
-        __syncthreads();
 
-        // ---- phase 1b: rows too long for one group, entries split over all P groups
-        const int nlong = lr_count;
-        for (int li = 0; li < nlong; ++li) {
-            const int lr = lr_list[li];
-            const int ls = row_ptr[row0 + lr], le = row_ptr[row0 + lr + 1];
-            float4 acc = f4_zero();
-            int t = ls + ty;
-            for (; t + 3 * P < le; t += 4 * P) {
-                int c4[4];
-                float v4[4];
-                float4 x[4];
+        // ---- rows too long for one group: every group of the wavefront takes a share of the entries
 #pragma unroll
-                for (int u = 0; u < 4; ++u) { c4[u] = col_idx[t + u * P]; v4[u] = val[t + u * P]; }
+        for (int rd = 0; rd < ROUNDS; ++rd) {
+            unsigned long long pending = __ballot(is_long[rd] && tx == 0);
+            while (pending) {
+                const int src_lane = __ffsll((long long)pending) - 1;
+                pending &= pending - 1;
+                const int lr = rd * RPR + src_lane / G;
+                const int ls = __shfl(rp, lr, kWave), le = __shfl(rp, lr + 1, kWave);
+                float4 acc = f4_zero();
+                int e = ls + grp;
+                for (; e + 3 * RPR < le; e += 4 * RPR) {
+                    int c4[4];
+                    float v4[4];
+                    float4 xx[4];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const float4*>(h_in + (size_t)c4[u] * C + tx * 4);
+                    for (int u = 0; u < 4; ++u) { c4[u] = col_idx[e + u * RPR]; v4[u] = val[e + u * RPR]; }
 #pragma unroll
-                for (int u = 0; u < 4; ++u) f4_fma(acc, v4[u], x[u]);
-            }
-            for (; t < le; t += P)
-                f4_fma(acc, val[t], *reinterpret_cast<const float4*>(h_in + (size_t)col_idx[t] * C + tx * 4));
-            *reinterpret_cast<float4*>(red + (size_t)ty * C + tx * 4) = acc;
-            __syncthreads();
-            if (ty == 0) {
-                float4 s = f4_zero();
-                for (int g = 0; g < P; ++g) {
-                    const float4 p = *reinterpret_cast<const float4*>(red + (size_t)g * C + tx * 4);
-                    s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
+                    for (int u = 0; u < 4; ++u) xx[u] = *reinterpret_cast<const float4*>(h_in + (size_t)c4[u] * C + tx * 4);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) f4_fma(acc, v4[u], xx[u]);
                 }
-                *reinterpret_cast<float4*>(tile + (size_t)lr * LDT + tx * 4) = s;
+                for (; e < le; e += RPR)
+                    f4_fma(acc, val[e], *reinterpret_cast<const float4*>(h_in + (size_t)col_idx[e] * C + tx * 4));
+                *reinterpret_cast<float4*>(red + grp * C + tx * 4) = acc;
+                __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+                if (grp == 0) {
+                    float4 sum = f4_zero();
+                    for (int g = 0; g < RPR; ++g) {
+                        const float4 p = *reinterpret_cast<const float4*>(red + g * C + tx * 4);
+                        sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
+                    }
+                    *reinterpret_cast<float4*>(tile + lr * LDT + tx * 4) = sum;
+                }
+                __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
             }
-            __syncthreads();
         }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        GNNHIP_PHASE_MARK(2);
 
-        // ---- phase 2: tile * W
-        float4 acc[RT];
+        // ---- contraction: lane (q, t) supplies tile[t][KS q + s] at step s
+        float areg[KS];
 #pragma unroll
-        for (int r = 0; r < RT; ++r) acc[r] = f4_zero();
-        tile_times_w<C, RT>(tile, LDT, C, Ws, ty, tx, acc);
+        for (int s4 = 0; s4 < KS / 4; ++s4) {
+            const float4 a = *reinterpret_cast<const float4*>(tile + t * LDT + KS * q + 4 * s4);
+            areg[4 * s4 + 0] = a.x; areg[4 * s4 + 1] = a.y; areg[4 * s4 + 2] = a.z; areg[4 * s4 + 3] = a.w;
+        }
+        GNNHIP_PHASE_MARK(3);
+        mfma_f4 acc[NJB];
+#pragma unroll
+        for (int jb = 0; jb < NJB; ++jb) {
+            acc[jb] = mfma_f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; ++s)
+                acc[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(wreg[jb][s], areg[s], acc[jb], 0, 0, 0);
+        }
+        GNNHIP_PHASE_MARK(4);
 
-        // ---- phase 3: + bias + msg, ReLU, store
-        float4 b4 = f4_zero();
-        if (bias) b4 = *reinterpret_cast<const float4*>(bias + tx * 4);
+        // ---- epilogue: lane owns row t, columns KS q + 4 jb + {0..3}
+        const long long row = row0 + t;
+        if (row < N) {
 #pragma unroll
-        for (int r = 0; r < RT; ++r) {
-            const int lr = ty + r * P;
-            if (lr < rows) {
-                const size_t off = ((size_t)row0 + lr) * C + tx * 4;
-                float4 v = acc[r];
-                if (bias) { v.x += b4.x; v.y += b4.y; v.z += b4.z; v.w += b4.w; }
+            for (int jb = 0; jb < NJB; ++jb) {
+                const int cbase = KS * q + 4 * jb;
+                const size_t off = (size_t)row * C + cbase;
+                float4 v = make_float4(acc[jb][0], acc[jb][1], acc[jb][2], acc[jb][3]);
+                if (bias) {
+                    const float4 b4 = *reinterpret_cast<const float4*>(bias + cbase);
+                    v.x += b4.x; v.y += b4.y; v.z += b4.z; v.w += b4.w;
+                }
                 if (msg) {
                     const float4 mm = *reinterpret_cast<const float4*>(msg + off);
                     v.x += mm.x; v.y += mm.y; v.z += mm.z; v.w += mm.w;
@@ -234,6 +356,8 @@ __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
                     make_float4(relu_ref(v.x), relu_ref(v.y), relu_ref(v.z), relu_ref(v.w));
             }
         }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");     // the tile is rewritten by the next iteration
+        GNNHIP_PHASE_MARK(5);
     }
 }
 
@@ -280,6 +404,7 @@ __global__ __launch_bounds__(kBlock) void s2v_readout_kernel(
         // hidden = ReLU(pool * W_h1)
         for (int j = tid; j < H; j += kBlock) {
             float s = 0.f;
+#pragma unroll 16
             for (int c = 0; c < C; ++c) s += pl[c] * Wh1[(size_t)c * H + j];
             s = relu_ref(s);
             hid[j] = s;
@@ -289,6 +414,7 @@ __global__ __launch_bounds__(kBlock) void s2v_readout_kernel(
         // logits = hidden * W_h2
         for (int q = tid; q < Q; q += kBlock) {
             float s = 0.f;
+#pragma unroll 8
             for (int j = 0; j < H; ++j) s += hid[j] * Wh2[(size_t)j * Q + q];
             lg[q] = s;
             logits[(size_t)g * Q + q] = s;
@@ -339,15 +465,15 @@ int launch_input(int N, int K, const float* X, const float* Wn2l, float* msg, fl
     return GNNHIP_OK;
 }
 
-template <int C, int RT>
+template <int C>
 int launch_level(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
                  const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
 {
-    constexpr int P = kBlock / (C / 4), R = RT * P;
-    const size_t smem = sizeof(float) * ((size_t)C * C + (size_t)R * (C + 4) + (size_t)P * C);
-    const int ntiles = (N + R - 1) / R;
-    const int grid = ntiles < kNumCU * 4 ? ntiles : kNumCU * 4;
-    hipLaunchKernelGGL((s2v_level_kernel<C, RT>), dim3(grid), dim3(kBlock), smem, s,
+    constexpr int kWavesPerBlock = kBlock / kWave;
+    const long long ntiles = ((long long)N + 15) / 16;
+    long long blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > kNumCU * 8) blocks = kNumCU * 8;          // persistent beyond this
+    hipLaunchKernelGGL((s2v_level_kernel<C>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
                        N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out);
     GNNHIP_LAUNCH_CHECK("s2v_level");
     return GNNHIP_OK;
@@ -393,14 +519,10 @@ int level_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const f
 {
     if (!(aligned16(h_in) && aligned16(W) && aligned16(h_out) && (!msg || aligned16(msg)) && (!bias || aligned16(bias))))
         return GNNHIP_EUNSUPPORTED;
-    const bool small = small_batch(N);
     switch (C) {
-    case 16: return small ? launch_level<16, 1>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s)
-                          : launch_level<16, 4>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
-    case 32: return small ? launch_level<32, 1>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s)
-                          : launch_level<32, 4>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
-    case 64: return small ? launch_level<64, 1>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s)
-                          : launch_level<64, 4>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    case 16: return launch_level<16>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    case 32: return launch_level<32>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    case 64: return launch_level<64>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
     }
     return GNNHIP_EUNSUPPORTED;
 }
