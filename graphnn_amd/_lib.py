@@ -4,7 +4,8 @@ import os
 from ctypes import POINTER, c_char_p, c_float, c_int, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "lib", "libgnnhip.so")
+# GNNHIP_LIBRARY overrides the in-tree location (e.g. an instrumented build of the same ABI)
+_LIB_PATH = os.environ.get("GNNHIP_LIBRARY") or os.path.join(_HERE, "lib", "libgnnhip.so")
 _lib = None
 
 
@@ -40,6 +41,7 @@ SIGNATURES = {
     "gnnhip_s2v_input_f32": [_I, _I, _I, _P, _P, _P, _P, _P],
     "gnnhip_s2v_readout_f32": [_I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_s2v_forward_f32": [_I] * 7 + [_P] * 11 + [_P] * 8 + [POINTER(c_int), _P],
+    "gnnhip_s2v_forward_batched_f32": [_I] * 8 + [_P] * 11 + [_P] * 7 + [_P, _P],
     "gnnhip_unary_f32": [_I, _P, _Z, _F, _F, _P],
     "gnnhip_relu_f32": [_P, _P, _Z, _P],
     "gnnhip_axpy_f32": [_Z, _F, _P, _P, _P],

@@ -121,6 +121,21 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i)
     argmax_combine(v, i, __shfl_xor(v, 32, kWave), __shfl_xor(i, 32, kWave));
 }
 
+// ---------------------------------------------------------------- small vector helpers
+typedef float mfma_f4 __attribute__((ext_vector_type(4)));   // accumulator of v_mfma_f32_16x16x4_f32
+
+__device__ __forceinline__ float4 f4_zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+__device__ __forceinline__ void f4_fma(float4& a, float s, const float4& x)
+{
+    a.x += s * x.x; a.y += s * x.y; a.z += s * x.z; a.w += s * x.w;
+}
+// ReLU exactly as the reference writes it: `if (x < 0) x = 0`, so -0.0 and NaN pass through.
+__device__ __forceinline__ float relu_ref(float v) { return v < 0.f ? 0.f : v; }
+__device__ __forceinline__ float4 relu_ref4(const float4& v)
+{
+    return make_float4(relu_ref(v.x), relu_ref(v.y), relu_ref(v.z), relu_ref(v.w));
+}
+
 // Device memory from the library's pool (released with pool_release).
 int pool_acquire(void** p, size_t bytes);
 int pool_release(void* p);

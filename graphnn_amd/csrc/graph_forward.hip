@@ -1,0 +1,452 @@
+// Graph-resident structure2vec forward for batches of small graphs (gfx950).
+//
+// When a batch is block diagonal — graph g owns the contiguous node range
+// [s_row_ptr[g], s_row_ptr[g+1]) and no edge leaves its graph, which is what
+// graphnn's GetBatch produces (examples/graph_classification/include/nn_common.h:36-105)
+// — every graph is an independent problem whose embeddings fit in LDS.  One
+// workgroup then runs the whole forward of one graph:
+//
+//   msg = X W_n2l, h = ReLU(msg)                      (matrix cores, msg to HBM once)
+//   L times:  agg = A_g h   (neighbour rows read from LDS)
+//             h   = ReLU(agg W + msg)                  (matrix cores, h stays in LDS)
+//   pool = sum_i s_val_i h_i ; hidden = ReLU(pool W_h1) ; logits = hidden W_h2 ;
+//   probs = softmax(logits) ; pred = argmax(logits)
+//
+// replacing L + 2 launches and 2 L round trips of the [N,C] activations through
+// HBM by one launch that reads the inputs once and writes msg, the final
+// embedding and the per-graph outputs once.  The graph's CSR slice is staged in
+// LDS and reused by all L levels.
+//
+// Work split inside the workgroup (4, 8 or 16 wavefronts): gathers split rows (C/4
+// lanes per row); the contraction splits (16-column block) x (16-row tile):
+// wavefront w owns column block w % (C/16) and every (WAVES / (C/16))-th tile, so it
+// keeps only its own 16 columns of W^T in registers.  MFMA operand layout as in level.hip.
+#include "gnnhip_internal.h"
+
+// Phase markers for a timing build of this file; they expand to nothing in the library.
+#ifndef GNNHIP_PHASE_MARK
+#define GNNHIP_PHASE_MARK(i)
+#endif
+
+namespace gnnhip {
+namespace {
+
+constexpr int kEdgeCapMax = 4096;       // CSR entries of one graph staged in LDS (fewer if LDS is short); larger graphs read them from L2
+constexpr size_t kLdsLimit = 160 * 1024;
+constexpr int kReadoutCap = 8192;       // floats of W_h1 and W_h2 staged in LDS; larger layers are read from L2
+
+// LDS carve-up, in floats:
+//   h[n16][C+4] | agg[n16][C+4] (shared with the staged X rows and the pooling partials) | rp[n16+4] | pool[C] | hid[H] | lg[Q]
+//   | W_h1, W_h2 (when small) | col[ecap] | val[ecap]
+struct GraphLds {
+    // the agg buffer also holds the staged X rows (n x K) and the pooling partials (waves x C)
+    __host__ __device__ static size_t agg_floats(int n16, int C, int K, int block)
+    {
+        size_t a = (size_t)n16 * (C + 4);
+        const size_t p = (size_t)(block / 64) * C, x = (size_t)n16 * K;
+        if (p > a) a = p;
+        if (x > a) a = x;
+        return (a + 3) / 4 * 4;
+    }
+    static size_t fixed_floats(int n16, int C, int K, int H, int Q, int block)
+    {
+        const size_t wro = ((size_t)C * H + (size_t)H * Q <= (size_t)kReadoutCap) ? (size_t)C * H + (size_t)H * Q : 0;
+        size_t f = (size_t)n16 * (C + 4) + agg_floats(n16, C, K, block) + (size_t)(n16 + 4) + C + H + Q + wro;
+        return (f + 3) / 4 * 4;
+    }
+    // entries of the edge cache that still fit under the LDS limit
+    static int edge_cap(int n16, int C, int K, int H, int Q, int block)
+    {
+        const size_t fixed = fixed_floats(n16, C, K, H, Q, block) * sizeof(float);
+        if (fixed >= kLdsLimit) return -1;
+        size_t cap = (kLdsLimit - fixed) / (2 * sizeof(float));
+        if (cap > (size_t)kEdgeCapMax) cap = kEdgeCapMax;
+        return (int)(cap / 4 * 4);
+    }
+};
+
+// WAVES wavefronts per workgroup (4, 8 or 16): chosen by the host so that the largest graph's
+// (column block x row tile) tasks spread over the wavefronts.
+template <int C, int KSX, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
+    int B, int K, int H, int Q, int L, int n16max, int ecap,
+    const int* __restrict__ a_row_ptr, const int* __restrict__ a_col_idx, const float* __restrict__ a_val,
+    const int* __restrict__ s_row_ptr, const int* __restrict__ s_col_idx, const float* __restrict__ s_val,
+    const float* __restrict__ X, const float* __restrict__ Wn2l, const float* __restrict__ Wc,
+    const float* __restrict__ Wh1, const float* __restrict__ Wh2,
+    float* __restrict__ msg, float* __restrict__ h_final, float* __restrict__ pool, float* __restrict__ hidden,
+    float* __restrict__ logits, float* __restrict__ probs, int* __restrict__ pred, int* __restrict__ status)
+{
+    constexpr int kBlock = WAVES * kWave;
+    constexpr int kWavesPerBlock = WAVES;
+    constexpr int G = C / 4;             // lanes per row in gathers
+    constexpr int P = kBlock / G;        // rows per gather round
+    constexpr int KS = C / 4;            // contraction steps of a level
+    constexpr int NJB = C / 16;          // column blocks
+    constexpr int TS = kWavesPerBlock / NJB;   // wavefronts sharing one column block, splitting tiles
+    constexpr int LDT = C + 4;
+    constexpr int kMsgTiles = (WAVES >= 16) ? 2 : 4;   // msg tiles a wavefront keeps in registers across the levels
+
+    extern __shared__ float smem[];
+    const bool ro_staged = ((size_t)C * H + (size_t)H * Q <= (size_t)kReadoutCap);
+    const size_t agg_fl = GraphLds::agg_floats(n16max, C, K, kBlock);
+    float* hbuf = smem;                                  // [n16max][LDT]
+    float* agg = hbuf + (size_t)n16max * LDT;            // [n16max][LDT]; doubles as part[P][C] in the readout
+    float* part = agg;
+    int* l_rp = reinterpret_cast<int*>(agg + agg_fl);    // [n16max + 1] row pointers relative to the graph's first entry
+    float* pl = reinterpret_cast<float*>(l_rp + n16max + 4);   // [C]
+    float* hid = pl + C;                                 // [H]
+    float* lg = hid + H;                                 // [Q]
+    float* w1s = lg + Q;                                 // W_h1 transposed, [H][C], when staged
+    float* w2s = w1s + (size_t)C * H;                    // W_h2 transposed, [Q][H], when staged
+    float* tail = ro_staged ? (w2s + (size_t)H * Q) : w1s;
+    tail = smem + ((size_t)(tail - smem) + 3) / 4 * 4;
+    int* e_col = reinterpret_cast<int*>(tail);           // [ecap] neighbour index local to the graph
+    float* e_val = tail + ecap;                          // [ecap]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid / kWave;
+    const int q = lane >> 4, t = lane & 15;
+    const int jb = wave % NJB, tsplit = wave / NJB;
+    const int gi = tid / G, tx = tid % G;
+
+    GNNHIP_PHASE_MARK(0);
+    // this wavefront's 16 columns of W^T, level contraction: wreg[s] = Wc[KS q + s][16 jb + t]
+    float wreg[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) wreg[s] = Wc[(size_t)(KS * q + s) * C + 16 * jb + t];
+
+    if (ro_staged) {
+        // coalesced reads; the transposed layout lets a wavefront read one output's weights contiguously
+        for (int i = tid; i < C * H; i += kBlock) w1s[(i % H) * C + i / H] = Wh1[i];
+        for (int i = tid; i < H * Q; i += kBlock) w2s[(i % Q) * H + i / Q] = Wh2[i];
+    }
+    // (the staged copies become visible to all lanes at the first barrier of the graph loop)
+    GNNHIP_PHASE_MARK(1);
+    for (int g = blockIdx.x; g < B; g += gridDim.x) {
+        const int node0 = s_row_ptr[g];
+        const int n = s_row_ptr[g + 1] - node0;
+        if (n > n16max || n < 0) {                      // host promised max_graph_nodes; refuse instead of overrunning LDS
+            if (tid == 0 && status) atomicOr(status, 1);
+            continue;
+        }
+        const int ntile = (n + 15) >> 4;
+        // this wavefront's 16 columns of W_n2l^T for the input stage: k = KSX q + s, zero beyond K.
+        // Loaded per graph (from L2) so the registers are free during the levels.
+        float wx[KSX];
+#pragma unroll
+        for (int s = 0; s < KSX; ++s) {
+            const int k = KSX * q + s;
+            wx[s] = Wn2l[(size_t)min(k, K - 1) * C + 16 * jb + t];
+            if (k >= K) wx[s] = 0.f;
+        }
+        const int e0 = a_row_ptr[node0];
+        const int ne = a_row_ptr[node0 + n] - e0;
+        const bool staged = (ne <= ecap);
+
+        // ---- stage the graph's CSR slice (L uses) and check the block-diagonal promise
+        for (int i = tid; i <= n; i += kBlock) l_rp[i] = a_row_ptr[node0 + i] - e0;
+        if (staged) {
+            for (int i = tid; i < ne; i += kBlock) {
+                const int c = a_col_idx[e0 + i] - node0;
+                if (c < 0 || c >= n) { if (status) atomicOr(status, 2); }
+                e_col[i] = min(max(c, 0), n - 1);
+                e_val[i] = a_val[e0 + i];
+            }
+        }
+        for (int i = tid; i < n; i += kBlock)
+            if (s_col_idx[node0 + i] != node0 + i) { if (status) atomicOr(status, 4); }
+        // the graph's rows of X, contiguous in memory, parked in the (still unused) agg buffer
+        float* xs = agg;
+        {
+            const float* xg = X + (size_t)node0 * K;
+            const int nx = n * K;
+            int base = 0;
+            for (; base + 4 * kBlock <= nx; base += 4 * kBlock) {
+                const float x0 = xg[base + tid], x1 = xg[base + tid + kBlock];
+                const float x2 = xg[base + tid + 2 * kBlock], x3 = xg[base + tid + 3 * kBlock];
+                xs[base + tid] = x0; xs[base + tid + kBlock] = x1;
+                xs[base + tid + 2 * kBlock] = x2; xs[base + tid + 3 * kBlock] = x3;
+            }
+            for (int i = base + tid; i < nx; i += kBlock) xs[i] = xg[i];
+        }
+        __syncthreads();
+
+        GNNHIP_PHASE_MARK(2);
+        // ---- input stage: msg tile = X tile * W_n2l on the matrix cores
+        float4 mreg[kMsgTiles];            // this wavefront's msg values for its first kMsgTiles tiles, kept for all levels
+#pragma unroll
+        for (int i = 0; i < kMsgTiles; ++i) mreg[i] = f4_zero();
+        {
+            int ti = 0;
+            for (int tl = tsplit; tl < ntile; tl += TS, ++ti) {
+                const int lr = tl * 16 + t;
+                const bool valid = lr < n;
+                // every lane reads a valid LDS slot (row and k clamped); wx is zero beyond K and
+                // rows beyond n are zeroed below, so the clamped values cannot reach a result
+                const float* xrow = xs + min(lr, n - 1) * K;
+                float xreg[KSX];
+#pragma unroll
+                for (int s = 0; s < KSX; ++s) xreg[s] = xrow[min(KSX * q + s, K - 1)];
+                mfma_f4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < KSX; ++s) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wx[s], xreg[s], acc, 0, 0, 0);
+                float4 v = make_float4(acc[0], acc[1], acc[2], acc[3]);      // row lr, columns 16 jb + 4 q + {0..3}
+                if (!valid) v = f4_zero();
+                if (valid) *reinterpret_cast<float4*>(msg + (size_t)(node0 + lr) * C + 16 * jb + 4 * q) = v;
+                *reinterpret_cast<float4*>(hbuf + (size_t)lr * LDT + 16 * jb + 4 * q) = relu_ref4(v);
+#pragma unroll
+                for (int i = 0; i < kMsgTiles; ++i) if (i == ti) mreg[i] = v;
+            }
+        }
+        __syncthreads();
+        GNNHIP_PHASE_MARK(3);
+
+        for (int lv = 0; lv < L; ++lv) {
+            // ---- gather-sum from LDS: agg[i] = sum_e val_e * h[col_e]
+            for (int r0 = 0; r0 < ntile * 16; r0 += P) {
+                const int lr = r0 + gi;
+                float4 acc = f4_zero();
+                if (lr < n) {
+                    const int st = l_rp[lr], en = l_rp[lr + 1];
+                    if (staged) {
+                        int e = st;
+                        for (; e + 1 < en; e += 2) {
+                            const int ca = e_col[e], cb = e_col[e + 1];
+                            const float va = e_val[e], vb = e_val[e + 1];
+                            const float4 xa = *reinterpret_cast<const float4*>(hbuf + (size_t)ca * LDT + tx * 4);
+                            const float4 xb = *reinterpret_cast<const float4*>(hbuf + (size_t)cb * LDT + tx * 4);
+                            f4_fma(acc, va, xa);
+                            f4_fma(acc, vb, xb);
+                        }
+                        if (e < en) f4_fma(acc, e_val[e], *reinterpret_cast<const float4*>(hbuf + (size_t)e_col[e] * LDT + tx * 4));
+                    } else {
+                        for (int e = st; e < en; ++e) {
+                            int c = a_col_idx[e0 + e] - node0;
+                            if (c < 0 || c >= n) { if (status) atomicOr(status, 2); c = min(max(c, 0), n - 1); }
+                            f4_fma(acc, a_val[e0 + e], *reinterpret_cast<const float4*>(hbuf + (size_t)c * LDT + tx * 4));
+                        }
+                    }
+                }
+                if (lr < ntile * 16) *reinterpret_cast<float4*>(agg + (size_t)lr * LDT + tx * 4) = acc;
+            }
+            __syncthreads();
+            if (lv == 0) { GNNHIP_PHASE_MARK(4); }
+
+            // ---- contraction + epilogue; h is rewritten in place (the gather above was its last reader)
+            int ti = 0;
+            for (int tl = tsplit; tl < ntile; tl += TS, ++ti) {
+                const int lr = tl * 16 + t;
+                const bool valid = lr < n;
+                float4 mm = f4_zero();
+                if (ti < kMsgTiles) {
+#pragma unroll
+                    for (int i = 0; i < kMsgTiles; ++i) if (i == ti) mm = mreg[i];
+                } else if (valid) {
+                    mm = *reinterpret_cast<const float4*>(msg + (size_t)(node0 + lr) * C + 16 * jb + 4 * q);
+                }
+                float areg[KS];
+#pragma unroll
+                for (int s4 = 0; s4 < KS / 4; ++s4) {
+                    const float4 a = *reinterpret_cast<const float4*>(agg + (size_t)lr * LDT + KS * q + 4 * s4);
+                    areg[4 * s4 + 0] = a.x; areg[4 * s4 + 1] = a.y; areg[4 * s4 + 2] = a.z; areg[4 * s4 + 3] = a.w;
+                }
+                mfma_f4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < KS; ++s) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wreg[s], areg[s], acc, 0, 0, 0);
+                float4 v = make_float4(acc[0] + mm.x, acc[1] + mm.y, acc[2] + mm.z, acc[3] + mm.w);
+                v = relu_ref4(v);
+                *reinterpret_cast<float4*>(hbuf + (size_t)lr * LDT + 16 * jb + 4 * q) = v;
+                if (lv == L - 1 && valid)
+                    *reinterpret_cast<float4*>(h_final + (size_t)(node0 + lr) * C + 16 * jb + 4 * q) = v;
+            }
+            __syncthreads();
+            if (lv == 0) { GNNHIP_PHASE_MARK(5); }
+        }
+        GNNHIP_PHASE_MARK(6);
+        if (L == 0) {
+            // the embedding is h0
+            for (int i = tid; i < n * G; i += kBlock) {
+                const int lr = i / G, f = i % G;
+                *reinterpret_cast<float4*>(h_final + (size_t)(node0 + lr) * C + f * 4) =
+                    *reinterpret_cast<const float4*>(hbuf + (size_t)lr * LDT + f * 4);
+            }
+        }
+
+        // ---- readout: weighted sum-pool over the graph's rows, then the two small dense layers,
+        // one wavefront per output element (64 lanes stride the contraction, DPP reduction)
+        {
+            float4 acc = f4_zero();
+            for (int lr = gi; lr < n; lr += P)
+                f4_fma(acc, s_val[node0 + lr], *reinterpret_cast<const float4*>(hbuf + (size_t)lr * LDT + tx * 4));
+            // combine the row groups of this wavefront, then one partial per wavefront goes to LDS
+#pragma unroll
+            for (int off = G; off < kWave; off <<= 1) {
+                acc.x += __shfl_xor(acc.x, off, kWave); acc.y += __shfl_xor(acc.y, off, kWave);
+                acc.z += __shfl_xor(acc.z, off, kWave); acc.w += __shfl_xor(acc.w, off, kWave);
+            }
+            if (lane < G) *reinterpret_cast<float4*>(part + (size_t)wave * C + tx * 4) = acc;
+        }
+        __syncthreads();
+        if (tid < C) {
+            float s = 0.f;
+#pragma unroll
+            for (int p = 0; p < kWavesPerBlock; ++p) s += part[(size_t)p * C + tid];
+            pl[tid] = s;
+            pool[(size_t)g * C + tid] = s;
+        }
+        __syncthreads();
+        for (int j = wave; j < H; j += kWavesPerBlock) {
+            float s = 0.f;
+            if (ro_staged) {
+                for (int c = lane; c < C; c += kWave) s += pl[c] * w1s[j * C + c];
+            } else {
+                for (int c = lane; c < C; c += kWave) s += pl[c] * Wh1[(size_t)c * H + j];
+            }
+            s = relu_ref(wave_sum(s));
+            if (lane == 0) { hid[j] = s; hidden[(size_t)g * H + j] = s; }
+        }
+        __syncthreads();
+        for (int qq = wave; qq < Q; qq += kWavesPerBlock) {
+            float s = 0.f;
+            if (ro_staged) {
+                for (int j = lane; j < H; j += kWave) s += hid[j] * w2s[qq * H + j];
+            } else {
+                for (int j = lane; j < H; j += kWave) s += hid[j] * Wh2[(size_t)j * Q + qq];
+            }
+            s = wave_sum(s);
+            if (lane == 0) { lg[qq] = s; logits[(size_t)g * Q + qq] = s; }
+        }
+        __syncthreads();
+        if (tid < kWave) {
+            const float first = lg[0];
+            float mx = first;
+            float bv = -INFINITY;
+            int bi = 0x7fffffff;
+            for (int qq = tid; qq < Q; qq += kWave) {
+                const float v = lg[qq];
+                mx = max_keep(mx, v);
+                argmax_combine(bv, bi, (v != v) ? -INFINITY : v, qq);
+            }
+            mx = wave_max(mx);
+            wave_argmax(bv, bi);
+            if (first != first) bi = 0;
+            if (pred && tid == 0) pred[g] = bi;
+            if (probs) {
+                float s = 0.f;
+                for (int qq = tid; qq < Q; qq += kWave) {
+                    const float e = expf(lg[qq] - mx);
+                    lg[qq] = e;
+                    s += e;
+                }
+                s = wave_sum(s);
+                for (int qq = tid; qq < Q; qq += kWave) probs[(size_t)g * Q + qq] = lg[qq] / s;
+            }
+        }
+        GNNHIP_PHASE_MARK(7);
+        __syncthreads();          // LDS is reused by the next graph of this workgroup
+    }
+}
+
+template <int C, int KSX, int WAVES>
+int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
+                         const int* a_row_ptr, const int* a_col_idx, const float* a_val,
+                         const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                         const float* X, const float* Wn2l, const float* Wc, const float* Wh1, const float* Wh2,
+                         float* msg, float* h_final, float* pool, float* hidden, float* logits, float* probs,
+                         int* pred, int* status, hipStream_t s)
+{
+    constexpr int kBlock = WAVES * kWave;
+    const int ecap = GraphLds::edge_cap(n16max, C, K, H, Q, kBlock);
+    if (ecap < 0) return GNNHIP_EUNSUPPORTED;
+    const size_t smem = sizeof(float) * (GraphLds::fixed_floats(n16max, C, K, H, Q, kBlock) + 2 * (size_t)ecap);
+    static size_t configured = 0;           // largest dynamic LDS size this kernel has been allowed so far
+    if (smem > 64 * 1024 && smem > configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) { (void)hipGetLastError(); return GNNHIP_EUNSUPPORTED; }
+        configured = smem;
+    }
+    const int grid = B < kNumCU * 4 ? B : kNumCU * 4;
+    hipLaunchKernelGGL((s2v_graph_forward_kernel<C, KSX, WAVES>), dim3(grid), dim3(kBlock), smem, s,
+                       B, K, H, Q, L, n16max, ecap, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val,
+                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status);
+    GNNHIP_LAUNCH_CHECK("s2v_graph_forward");
+    return GNNHIP_OK;
+}
+
+template <int C, int WAVES>
+int dispatch_ksx(int B, int K, int H, int Q, int L, int n16max,
+                 const int* a_row_ptr, const int* a_col_idx, const float* a_val,
+                 const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                 const float* X, const float* Wn2l, const float* Wc, const float* Wh1, const float* Wh2,
+                 float* msg, float* h_final, float* pool, float* hidden, float* logits, float* probs,
+                 int* pred, int* status, hipStream_t s)
+{
+#define GNNHIP_GF_ARGS B, K, H, Q, L, n16max, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
+                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, s
+    if (K <= 16) return launch_graph_forward<C, 4, WAVES>(GNNHIP_GF_ARGS);
+    if (K <= 32) return launch_graph_forward<C, 8, WAVES>(GNNHIP_GF_ARGS);
+    if (K <= 48) return launch_graph_forward<C, 12, WAVES>(GNNHIP_GF_ARGS);
+    if (K <= 64) return launch_graph_forward<C, 16, WAVES>(GNNHIP_GF_ARGS);
+    return GNNHIP_EUNSUPPORTED;
+#undef GNNHIP_GF_ARGS
+}
+
+template <int C>
+int dispatch_waves(int B, int K, int H, int Q, int L, int n16max,
+                   const int* a_row_ptr, const int* a_col_idx, const float* a_val,
+                   const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                   const float* X, const float* Wn2l, const float* Wc, const float* Wh1, const float* Wh2,
+                   float* msg, float* h_final, float* pool, float* hidden, float* logits, float* probs,
+                   int* pred, int* status, hipStream_t s)
+{
+#define GNNHIP_GF_ARGS B, K, H, Q, L, n16max, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
+                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, s
+    const int tasks = (C / 16) * (n16max / 16);         // (column block x row tile) tasks of the largest graph
+    if (tasks <= 4) return dispatch_ksx<C, 4>(GNNHIP_GF_ARGS);
+    if (tasks <= 8) return dispatch_ksx<C, 8>(GNNHIP_GF_ARGS);
+    return dispatch_ksx<C, 16>(GNNHIP_GF_ARGS);
+#undef GNNHIP_GF_ARGS
+}
+
+}  // namespace
+}  // namespace gnnhip
+
+using namespace gnnhip;
+
+extern "C" int gnnhip_s2v_forward_batched_f32(int N, int B, int K, int C, int H, int Q, int L, int max_graph_nodes,
+                                              const int* a_row_ptr, const int* a_col_idx, const float* a_val,
+                                              const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                                              const float* X, const float* W_n2l, const float* W_conv,
+                                              const float* W_h1, const float* W_h2,
+                                              float* msg, float* h_final, float* pool, float* hidden, float* logits,
+                                              float* probs, int* pred, int* status, void* stream)
+{
+    GNNHIP_REQUIRE(N >= 1 && B >= 1 && K >= 1 && C >= 1 && H >= 1 && Q >= 1 && L >= 0 && max_graph_nodes >= 1,
+                   "bad shape in s2v_forward_batched (N=%d B=%d K=%d C=%d H=%d Q=%d L=%d max_graph_nodes=%d)",
+                   N, B, K, C, H, Q, L, max_graph_nodes);
+    GNNHIP_REQUIRE(a_row_ptr && a_col_idx && a_val && s_row_ptr && s_col_idx && s_val && X && W_n2l && W_conv && W_h1 && W_h2,
+                   "null input in s2v_forward_batched");
+    GNNHIP_REQUIRE(msg && h_final && pool && hidden && logits, "null output in s2v_forward_batched");
+    if (int rc = require_ready()) return rc;
+    if (!(C == 16 || C == 32 || C == 64) || K > 64)
+        return set_error(GNNHIP_EUNSUPPORTED, "graph-resident forward supports hidden 16/32/64 and at most 64 label types (C=%d K=%d)", C, K);
+    if (!(aligned16(msg) && aligned16(h_final)))
+        return set_error(GNNHIP_EUNSUPPORTED, "msg and h_final must be 16-byte aligned");
+    const int n16 = (max_graph_nodes + 15) / 16 * 16;
+    if (GraphLds::edge_cap(n16, C, K, H, Q, 256) < 0)
+        return set_error(GNNHIP_EUNSUPPORTED, "a graph of %d nodes does not fit the 160 KB of LDS", max_graph_nodes);
+    hipStream_t s = as_stream(stream);
+    int rc;
+#define GNNHIP_GF_ARGS B, K, H, Q, L, n16, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
+                       X, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, s
+    switch (C) {
+    case 16: rc = dispatch_waves<16>(GNNHIP_GF_ARGS); break;
+    case 32: rc = dispatch_waves<32>(GNNHIP_GF_ARGS); break;
+    default: rc = dispatch_waves<64>(GNNHIP_GF_ARGS); break;
+    }
+#undef GNNHIP_GF_ARGS
+    if (rc == GNNHIP_EUNSUPPORTED) return set_error(rc, "graph-resident forward could not be configured for this shape");
+    return rc;
+}

@@ -34,12 +34,6 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kLongRow = 1024;      // level kernel: longer rows are gathered by the whole workgroup
 
-__device__ __forceinline__ float4 f4_zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
-__device__ __forceinline__ void f4_fma(float4& a, float s, const float4& x)
-{
-    a.x += s * x.x; a.y += s * x.y; a.z += s * x.z; a.w += s * x.w;
-}
-__device__ __forceinline__ float relu_ref(float v) { return v < 0.f ? 0.f : v; }
 
 // Copy N4 float4s (a compile-time count) from global to LDS.  All of a lane's loads are
 // issued before the first LDS store, so the copy costs one memory round trip.
@@ -168,8 +162,6 @@ __global__ __launch_bounds__(kBlock) void s2v_input_kernel(
 //      columns of block jb are permuted so that the lane ends up owning row t,
 //      columns (C/4) q .. (C/4) q + C/4 - 1: contiguous float4s for the epilogue;
 //   3. epilogue: + bias + msg, ReLU, float4 stores.
-typedef float mfma_f4 __attribute__((ext_vector_type(4)));
-
 constexpr int kWaveLongRow = 256;   // entries; longer rows are gathered by all groups of the wavefront together
 
 template <int C>

@@ -124,6 +124,25 @@ int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L,
                            float* pool, float* hidden, float* logits, float* probs, int* pred,
                            int* which_h, void* stream);
 
+/* ---- the same forward for block-diagonal batches of small graphs, in ONE launch with the
+ *      embeddings resident in LDS: the op sequence of
+ *      examples/graph_classification/src/kernel_mean_field.cpp:31-49 on a batch laid out by GetBatch
+ *      (examples/graph_classification/include/nn_common.h:36-105), i.e. graph g owns the contiguous
+ *      nodes [s_row_ptr[g], s_row_ptr[g+1]), s_col_idx[i] == i, and no entry of A joins two graphs.
+ *      max_graph_nodes (host int) bounds the largest graph.  h_final [N,C] receives the last-level
+ *      embedding.  status (device int, may be NULL; caller zeroes it) gets bit 0 set if a graph
+ *      exceeds max_graph_nodes, bit 1 if an edge leaves its graph, bit 2 if S is not the identity
+ *      layout; results are then unspecified but no access goes out of bounds.
+ *      Returns GNNHIP_EUNSUPPORTED (nothing launched) for shapes it does not cover
+ *      (hidden not in {16,32,64}, more than 64 label types, graph too large for LDS). */
+int gnnhip_s2v_forward_batched_f32(int N, int B, int K, int C, int H, int Q, int L, int max_graph_nodes,
+                                   const int* a_row_ptr, const int* a_col_idx, const float* a_val,
+                                   const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                                   const float* X, const float* W_n2l, const float* W_conv,
+                                   const float* W_h1, const float* W_h2,
+                                   float* msg, float* h_final, float* pool, float* hidden, float* logits,
+                                   float* probs, int* pred, int* status, void* stream);
+
 /* ---- UnaryEngine<GPU>::Exec<Functor> (include/tensor/gpu_unary_functor.h:331-384):
  *      in-place x[i] = f(x[i]); a0/a1 are the functor's constructor arguments. */
 int gnnhip_unary_f32(int op, float* x, size_t n, float a0, float a1, void* stream);

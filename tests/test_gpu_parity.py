@@ -498,3 +498,106 @@ def test_pool_recycles_blocks(gpu):
     assert np.array_equal(src, dst)
     assert lib.gnnhip_free(q) == 0
     assert lib.gnnhip_recycle(q) == -1                                   # no longer owned by the pool
+
+
+# ------------------------------------------------------------------ graph-resident (one-launch) forward
+def _batched_case(gpu, oracle, batch, w, L):
+    from graphnn_amd import ops
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    want = oracle.forward(a, s, X, w, L, batch.label_csr())
+    bufs = ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+                                   _t(w.W_h1, gpu), _t(w.W_h2, gpu), L, int(batch.graph_sizes.max()))
+    return want, bufs
+
+
+def _assert_batched_matches(want, bufs, L):
+    assert int(_n(bufs.status)[0]) == 0
+    assert max_rel(_n(bufs.msg), want["msg"]) < PARITY_TOL
+    assert max_rel(_n(bufs.h_final), want["h"][L]) < PARITY_TOL
+    for key in ("pool", "hidden", "logits", "probs"):
+        assert max_rel(_n(getattr(bufs, key)), want[key]) < PARITY_TOL, key
+    assert np.array_equal(_n(bufs.pred), want["pred"])
+
+
+@pytest.mark.parametrize("config_id", [1, 2])
+def test_batched_forward_matches_reference_path(gpu, oracle, config_id):
+    batch, w, cfg = synth.make_config(config_id)
+    want, bufs = _batched_case(gpu, oracle, batch, w, cfg["L"])
+    _assert_batched_matches(want, bufs, cfg["L"])
+
+
+@pytest.mark.parametrize("C,K,H,Q,L", [(16, 7, 8, 3, 2), (32, 20, 16, 2, 3), (64, 64, 32, 5, 1), (64, 3, 100, 70, 0),
+                                       (32, 48, 8, 2, 5), (16, 33, 4, 2, 1)])
+def test_batched_forward_shapes(gpu, oracle, C, K, H, Q, L):
+    seed = 1000 + C + K + L
+    batch = synth.molecule_batch(seed, 37, K, Q, size_mode="uniform", size_lo=1, size_hi=70)
+    w = synth.make_weights(synth.Stream(seed), K, C, H, Q)
+    want, bufs = _batched_case(gpu, oracle, batch, w, L)
+    _assert_batched_matches(want, bufs, L)
+
+
+def test_batched_forward_large_and_dense_graphs(gpu, oracle):
+    """a 200-node graph (more than 64 KB of LDS) next to a complete graph whose edge list is not staged in LDS"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(77)
+    sizes = np.array([200, 100, 1, 17], np.int64)
+    off = np.concatenate([[0], np.cumsum(sizes)])
+    N, B, K, C, H, Q, L = int(off[-1]), 4, 9, 64, 32, 2, 3
+    ex, ey = [], []
+    for g, n in enumerate(sizes):
+        if g == 1:                                   # complete graph: 9,900 directed edges
+            a, b = np.meshgrid(np.arange(n), np.arange(n), indexing="ij")
+            m = a != b
+            ex.append(off[g] + a[m]); ey.append(off[g] + b[m])
+        elif n > 1:                                  # ring plus chords
+            i = np.arange(n)
+            for step in (1, 7):
+                ex += [off[g] + i, off[g] + (i + step) % n]; ey += [off[g] + (i + step) % n, off[g] + i]
+    ex = np.concatenate(ex).astype(np.int32); ey = np.concatenate(ey).astype(np.int32)
+    order = np.lexsort((ey, ex)); ex, ey = ex[order], ey[order]
+    a = batching.node2node_csr(N, ex, ey)
+    s = batching.subgraph_csr(B, np.repeat(np.arange(B), sizes).astype(np.int32), np.arange(N, dtype=np.int32))
+    a = (a[0], a[1], (rng.random(a[1].size) * 0.05).astype(np.float32))           # non-unit edge weights
+    s = (s[0], s[1], (rng.random(N) * 0.5).astype(np.float32))                    # weighted pooling
+    X = rng.standard_normal((N, K)).astype(np.float32)
+    w = synth.make_weights(synth.Stream(5), K, C, H, Q)
+    want = oracle.forward(a, s, X, w, L, None)
+    bufs = ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+                                   _t(w.W_h1, gpu), _t(w.W_h2, gpu), L, 200)
+    _assert_batched_matches(want, bufs, L)
+    # the general multi-launch forward gives the same answer on this batch
+    gen = ops.s2v_forward(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+                          _t(w.W_h1, gpu), _t(w.W_h2, gpu), L)
+    assert max_rel(_n(gen.logits), _n(bufs.logits)) < PARITY_TOL
+
+
+def test_batched_forward_reports_broken_promises(gpu, oracle):
+    from graphnn_amd import ops
+    from graphnn_amd._lib import GnnHipError
+    batch, w, cfg = synth.make_config(1, B=8)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    dev_w = (_t(w.W_n2l, gpu), _t(w.W_conv, gpu), _t(w.W_h1, gpu), _t(w.W_h2, gpu))
+    nmax = int(batch.graph_sizes.max())
+    # a graph larger than promised: bit 0, nothing overruns
+    assert nmax > 16                                          # the promise is checked at 16-row granularity
+    bufs = ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), *dev_w, cfg["L"], 16)
+    assert int(_n(bufs.status)[0]) & 1
+    # an edge that joins two graphs: bit 1
+    bad_col = a[1].copy()
+    bad_col[0] = batch.num_nodes - 1
+    bufs = ops.s2v_forward_batched((_t(a[0], gpu), _t(bad_col, gpu), _t(a[2], gpu)), _csr_t(s, gpu), _t(X, gpu), *dev_w,
+                                   cfg["L"], nmax)
+    assert int(_n(bufs.status)[0]) & 2
+    # a pooling matrix that is not the identity layout: bit 2
+    bad_s = s[1].copy(); bad_s[[0, 1]] = bad_s[[1, 0]]
+    bufs = ops.s2v_forward_batched(_csr_t(a, gpu), (_t(s[0], gpu), _t(bad_s, gpu), _t(s[2], gpu)), _t(X, gpu), *dev_w,
+                                   cfg["L"], nmax)
+    assert int(_n(bufs.status)[0]) & 4
+    # shapes outside the kernel's range are refused without launching
+    with pytest.raises(GnnHipError) as err:
+        ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), *dev_w, cfg["L"], 5000)
+    assert err.value.code == -5
