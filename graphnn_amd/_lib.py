@@ -55,6 +55,11 @@ SIGNATURES = {
     "gnnhip_cross_entropy_f32": [_P, _I, _I, _P, _P, _P, _P, _P],
     "gnnhip_in_top_k_f32": [_P, _P, _I, _I, _I, _P, _P],
     "gnnhip_cast_i32_f32": [_P, _P, _Z, _P],
+    "gnnhip_spmm_csr_t_f32": [_I, _I, _I, _F, _P, _P, _P, _P, _I, _F, _P, _I, _P],
+    "gnnhip_csr_axpy_f32": [_I, _I, _F, _P, _P, _P, _P, _P],
+    "gnnhip_relu_deriv_f32": [_Z, _P, _P, _P, _P],
+    "gnnhip_mul_f32": [_Z, _P, _P, _P],
+    "gnnhip_row_scale_f32": [_I, _I, _P, _P, _P],
     "gnnhip_last_error": [],
     "gnnhip_version": [],
 }

@@ -93,7 +93,7 @@ __device__ __forceinline__ float block_combine(float v, float* sh)
     return r;
 }
 
-template <bool IS_MAX>
+template <bool IS_MAX, bool SQUARE = false>
 __global__ __launch_bounds__(kBlock) void reduce_partial_kernel(const float* __restrict__ x, size_t n, float* __restrict__ partial)
 {
     __shared__ float sh[kWavesPerBlock];
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(kBlock) void reduce_partial_kernel(const float* __r
     const size_t hi = lo + per < n ? lo + per : n;
     float v = IS_MAX ? -INFINITY : 0.f;
     if (IS_MAX && lo < hi) v = x[lo];
-    for (size_t i = lo + threadIdx.x; i < hi; i += kBlock) v = IS_MAX ? max_keep(v, x[i]) : v + x[i];
+    for (size_t i = lo + threadIdx.x; i < hi; i += kBlock) v = IS_MAX ? max_keep(v, x[i]) : v + (SQUARE ? x[i] * x[i] : x[i]);
     v = block_combine<IS_MAX>(v, sh);
     if (threadIdx.x == 0) partial[blockIdx.x] = v;
 }
@@ -248,7 +248,8 @@ int gnnhip_jagged_softmax_f32(float* x, const int* lens, int nseg, void* stream)
 
 int gnnhip_reduce_f32(int op, const float* x, size_t n, float* out, void* stream)
 {
-    GNNHIP_REQUIRE(op == GNNHIP_REDUCE_SUM || op == GNNHIP_REDUCE_MEAN || op == GNNHIP_REDUCE_MAX, "unknown reduce op %d", op);
+    GNNHIP_REQUIRE(op == GNNHIP_REDUCE_SUM || op == GNNHIP_REDUCE_MEAN || op == GNNHIP_REDUCE_MAX || op == GNNHIP_REDUCE_SUMSQ,
+                   "unknown reduce op %d", op);
     GNNHIP_REQUIRE(out != nullptr, "null output in reduce");
     GNNHIP_REQUIRE(n > 0 && x != nullptr, "empty input in reduce");
     if (int rc = require_ready()) return rc;
@@ -262,6 +263,9 @@ int gnnhip_reduce_f32(int op, const float* x, size_t n, float* out, void* stream
     if (op == GNNHIP_REDUCE_MAX) {
         hipLaunchKernelGGL((reduce_partial_kernel<true>), dim3((unsigned)nb), dim3(kBlock), 0, s, x, n, pp);
         hipLaunchKernelGGL((reduce_final_kernel<true>), dim3(1), dim3(kBlock), 0, s, pp, (int)nb, 0.f, out);
+    } else if (op == GNNHIP_REDUCE_SUMSQ) {
+        hipLaunchKernelGGL((reduce_partial_kernel<false, true>), dim3((unsigned)nb), dim3(kBlock), 0, s, x, n, pp);
+        hipLaunchKernelGGL((reduce_final_kernel<false>), dim3(1), dim3(kBlock), 0, s, pp, (int)nb, 0.f, out);
     } else {
         hipLaunchKernelGGL((reduce_partial_kernel<false>), dim3((unsigned)nb), dim3(kBlock), 0, s, x, n, pp);
         hipLaunchKernelGGL((reduce_final_kernel<false>), dim3(1), dim3(kBlock), 0, s, pp, (int)nb, div, out);

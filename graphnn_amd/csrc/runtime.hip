@@ -99,6 +99,8 @@ int pool_release(void* p)
     if (!p) return GNNHIP_OK;
     Runtime& r = rt();
     std::lock_guard<std::mutex> lock(r.mu);
+    // after gnnhip_shutdown every block is already gone; late owners (static destructors) are told so
+    if (!r.ready) return set_error(GNNHIP_ENOTINIT, "gnnhip is shut down; the block was released with the pool");
     auto it = r.live.find(p);
     if (it == r.live.end()) return set_error(GNNHIP_EINVAL, "pointer %p was not handed out by gnnhip_malloc", p);
     size_t sz = it->second;
@@ -193,6 +195,7 @@ int gnnhip_free(void* device_ptr)
     if (!device_ptr) return GNNHIP_OK;
     Runtime& r = rt();
     std::lock_guard<std::mutex> lock(r.mu);
+    if (!r.ready) return set_error(GNNHIP_ENOTINIT, "gnnhip is shut down; the block was released with the pool");
     auto it = r.all.find(device_ptr);
     if (it == r.all.end())
         return set_error(GNNHIP_EINVAL, "pointer %p is not owned by the gnnhip pool", device_ptr);
@@ -231,8 +234,10 @@ int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void
     if (bytes == 0) return GNNHIP_OK;
     GNNHIP_REQUIRE(dst_device && src_host, "null pointer in memcpy_h2d");
     if (int rc = require_ready()) return rc;
-    // Pageable source: the runtime stages the bytes before returning, so the host buffer may be reused at once.
+    // Ordered after earlier work on the stream; returns once the host buffer has been read, so the
+    // caller may overwrite it at once (the reference's blocking cudaMemcpy gives callers the same promise).
     GNNHIP_HIP(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    GNNHIP_HIP(hipStreamSynchronize(as_stream(stream)));
     return GNNHIP_OK;
 }
 

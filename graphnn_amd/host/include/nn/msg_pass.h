@@ -1,0 +1,116 @@
+// Message-passing operands: CSR matrices built from the batch GraphStruct on the host and
+// copied to the device (interface of graphnn's include/nn/msg_pass.h; construction rules of
+// src/nn/msg_pass.cpp:46-67 and :156-177).  Row i of the node-to-node matrix lists the
+// in-neighbours of node i in edge order; row g of the subgraph matrix lists the nodes of
+// graph g in AddNode order; values are 1, or 1/row length when `average` is set.
+#ifndef MSG_PASS_H
+#define MSG_PASS_H
+
+#include "nn/factor.h"
+#include "util/graph_struct.h"
+
+namespace gnn
+{
+
+template<typename mode, typename Dtype>
+class IMsgPass : public Factor
+{
+public:
+    static std::string StrType() { return "IMsgPass"; }
+
+    IMsgPass(std::string _name, bool _average) : Factor(_name, PropErr::N), average(_average) {}
+
+    virtual void Forward(std::vector< std::shared_ptr<Variable> >& operands,
+                         std::vector< std::shared_ptr<Variable> >& outputs, Phase) override
+    {
+        ASSERT(operands.size() == 1, "unexpected input size for " << StrType());
+        ASSERT(outputs.size() == 1, "unexpected output size for " << StrType());
+        auto* gv = dynamic_cast<GraphVar*>(operands[0].get());
+        ASSERT(gv && gv->graph, "message passing needs a bound GraphVar");
+        auto& out = detail::sparse_var<mode, Dtype>(outputs[0], "IMsgPass").value;
+        InitCPUWeight(gv->graph);
+        out.CopyFrom(cpu_weight);          // host -> device (or host -> host) copy of the three CSR arrays
+    }
+
+    // layout facts about the last batch, gathered while the CSR was built (used to choose kernels)
+    bool block_diagonal = false;           // node2node: no edge joins two subgraphs
+    bool contiguous_subgraphs = false;     // subgraph: graph g owns one contiguous, ascending node range
+    int max_subgraph_nodes = 0;
+
+protected:
+    virtual void InitCPUWeight(GraphStruct* graph) = 0;
+    SpTensor<CPU, Dtype> cpu_weight;
+    bool average;
+};
+
+template<typename mode, typename Dtype>
+class Node2NodeMsgPass : public IMsgPass<mode, Dtype>
+{
+public:
+    static std::string StrType() { return "Node2NodeMsgPass"; }
+    using OutType = std::shared_ptr< SpTensorVar<mode, Dtype> >;
+    OutType CreateOutVar() { return std::make_shared< SpTensorVar<mode, Dtype> >(fmt::sprintf("%s:out_0", this->name)); }
+    Node2NodeMsgPass(std::string _name, bool _average = false) : IMsgPass<mode, Dtype>(_name, _average) {}
+
+protected:
+    virtual void InitCPUWeight(GraphStruct* graph) override
+    {
+        auto& w = this->cpu_weight;
+        w.Reshape({graph->num_nodes, graph->num_nodes});
+        w.ResizeSp((int)graph->num_edges, (int)graph->num_nodes + 1);
+        int* rp = w.data->row_ptr;
+        int* ci = w.data->col_idx;
+        Dtype* va = w.data->val;
+        int nnz = 0;
+        for (unsigned i = 0; i < graph->num_nodes; ++i) {
+            rp[i] = nnz;
+            const auto& in = graph->in_edges->head[i];
+            const Dtype weight = this->average ? (Dtype)(1.0 / (double)in.size()) : (Dtype)1.0;
+            for (size_t j = 0; j < in.size(); ++j) { ci[nnz] = in[j].second; va[nnz] = weight; ++nnz; }
+        }
+        rp[graph->num_nodes] = nnz;
+        ASSERT(nnz == (int)graph->num_edges, "edge count does not match the in-edge lists");
+    }
+};
+
+template<typename mode, typename Dtype>
+class SubgraphMsgPass : public IMsgPass<mode, Dtype>
+{
+public:
+    static std::string StrType() { return "SubgraphMsgPass"; }
+    using OutType = std::shared_ptr< SpTensorVar<mode, Dtype> >;
+    OutType CreateOutVar() { return std::make_shared< SpTensorVar<mode, Dtype> >(fmt::sprintf("%s:out_0", this->name)); }
+    SubgraphMsgPass(std::string _name, bool _average = false) : IMsgPass<mode, Dtype>(_name, _average) {}
+
+protected:
+    virtual void InitCPUWeight(GraphStruct* graph) override
+    {
+        auto& w = this->cpu_weight;
+        w.Reshape({graph->num_subgraph, graph->num_nodes});
+        w.ResizeSp((int)graph->num_nodes, (int)graph->num_subgraph + 1);
+        int* rp = w.data->row_ptr;
+        int* ci = w.data->col_idx;
+        Dtype* va = w.data->val;
+        int nnz = 0, biggest = 0;
+        bool contiguous = true;
+        for (unsigned g = 0; g < graph->num_subgraph; ++g) {
+            rp[g] = nnz;
+            const auto& nodes = graph->subgraph->head[g];
+            const Dtype weight = this->average ? (Dtype)(1.0 / (double)nodes.size()) : (Dtype)1.0;
+            for (size_t j = 0; j < nodes.size(); ++j) {
+                contiguous = contiguous && nodes[j] == nnz;
+                ci[nnz] = nodes[j];
+                va[nnz] = weight;
+                ++nnz;
+            }
+            biggest = std::max(biggest, (int)nodes.size());
+        }
+        rp[graph->num_subgraph] = nnz;
+        ASSERT(nnz == (int)graph->num_nodes, "node count does not match the subgraph lists");
+        this->contiguous_subgraphs = contiguous;
+        this->max_subgraph_nodes = biggest;
+    }
+};
+
+}  // namespace gnn
+#endif

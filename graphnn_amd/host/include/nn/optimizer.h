@@ -1,0 +1,95 @@
+// Parameter updates on the device (include/nn/optimizer.h, src/nn/optimizer.cpp:16-92):
+// plain SGD and momentum SGD over the full (dense) gradients of a ParamSet.
+#ifndef OPTIMIZER_H
+#define OPTIMIZER_H
+
+#include <cmath>
+#include "nn/param_set.h"
+
+namespace gnn
+{
+
+template<typename mode, typename Dtype>
+class IOptimizer
+{
+public:
+    IOptimizer(ParamSet<mode, Dtype>* _param_set, Dtype _init_lr, Dtype _l2_penalty = 0)
+        : param_set(_param_set), init_lr(_init_lr), l2_penalty(_l2_penalty), cur_lr(_init_lr),
+          clip_threshold(5), clipping_enabled(true), cur_iter(0) {}
+    virtual ~IOptimizer() {}
+    virtual void Update() = 0;
+
+    // factor that brings the global gradient norm down to clip_threshold (1 when it already is)
+    Dtype ClipGradients()
+    {
+        if (!clipping_enabled) return 1.0;
+        Dtype sq = 0;
+        for (auto& kv : param_set->params) {
+            const Dtype n2 = kv.second->grad.Norm2();
+            sq += n2 * n2;
+        }
+        const Dtype norm = std::sqrt(sq);
+        return norm > clip_threshold ? clip_threshold / norm : (Dtype)1.0;
+    }
+
+    ParamSet<mode, Dtype>* param_set;
+    Dtype init_lr;
+    Dtype l2_penalty;
+    Dtype cur_lr;
+    Dtype clip_threshold;
+    bool clipping_enabled;
+    int cur_iter;
+};
+
+template<typename mode, typename Dtype>
+class SGDOptimizer : public IOptimizer<mode, Dtype>
+{
+public:
+    SGDOptimizer(ParamSet<mode, Dtype>* m, Dtype _init_lr, Dtype _l2_penalty = 0) : IOptimizer<mode, Dtype>(m, _init_lr, _l2_penalty) {}
+    // w <- (1 - lr * l2) w - lr * g
+    virtual void Update() override
+    {
+        for (auto& kv : this->param_set->params) {
+            auto& p = kv.second;
+            auto g = p->grad.Full();
+            p->value.Axpby(-this->cur_lr, g, 1 - this->cur_lr * this->l2_penalty);
+            p->grad.RowSpZeros();
+        }
+    }
+};
+
+template<typename mode, typename Dtype>
+class MomentumSGDOptimizer : public IOptimizer<mode, Dtype>
+{
+public:
+    MomentumSGDOptimizer(ParamSet<mode, Dtype>* m, Dtype _init_lr, Dtype _momentum = 0.9, Dtype _l2_penalty = 0)
+        : IOptimizer<mode, Dtype>(m, _init_lr, _l2_penalty), momentum(_momentum) {}
+
+    // g <- g + l2 * w ;  v <- momentum * v + lr * g ;  w <- w - v     (plain SGD when momentum == 0)
+    virtual void Update() override
+    {
+        for (auto& kv : this->param_set->params) {
+            auto& p = kv.second;
+            auto g = p->grad.Full();
+            if (momentum > 0) {
+                auto& v = acc_grad_dict[kv.first];
+                if (!v) {
+                    v = std::make_shared< DTensor<mode, Dtype> >(p->grad.shape);
+                    v->Zeros();
+                }
+                g.Axpy(this->l2_penalty, p->value);
+                v->Axpby(this->cur_lr, g, momentum);
+                p->value.Axpy(-1.0, *v);
+            } else {
+                p->value.Axpby(-this->cur_lr, g, 1 - this->cur_lr * this->l2_penalty);
+            }
+            p->grad.RowSpZeros();
+        }
+    }
+
+    Dtype momentum;
+    std::map<std::string, std::shared_ptr< DTensor<mode, Dtype> > > acc_grad_dict;
+};
+
+}  // namespace gnn
+#endif

@@ -1,0 +1,104 @@
+// Device CSR tensor (interface of graphnn's include/tensor/gpu_sparse_tensor.h) and the
+// sparse-operand methods of the dense tensor.
+#ifndef GPU_CSR_SPARSE_TENSOR_H
+#define GPU_CSR_SPARSE_TENSOR_H
+
+#include "tensor/gpu_dense_tensor.h"
+#include "tensor/cpu_sparse_tensor.h"
+
+namespace gnn
+{
+
+template<typename Dtype>
+class TensorTemplate<GPU, CSR_SPARSE, Dtype> : public Tensor
+{
+public:
+    TensorTemplate() : data(std::make_shared< SparseData<GPU, Dtype> >()) {}
+    virtual ~TensorTemplate() {}
+
+    virtual void Reshape(std::vector<size_t> l) override
+    {
+        ASSERT(l.size() == 2, "only support sparse matrix");
+        shape.Reshape(l);
+    }
+    virtual MatType GetMatType() override { return MatType::sparse; }
+    virtual MatMode GetMatMode() override { return MatMode::gpu; }
+
+    void ResizeSp(int newNNZ, int newNPtr)
+    {
+        data->Reserve(newNNZ, newNPtr);
+        data->nnz = newNNZ;
+        data->len_ptr = newNPtr;
+    }
+    // three host-to-device copies, ordered on the layer's stream
+    void CopyFrom(SpTensor<CPU, Dtype>& src)
+    {
+        shape = src.shape;
+        ResizeSp(src.data->nnz, src.data->len_ptr);
+        void* s = GpuHandle::Stream();
+        GNN_HIP(gnnhip_memcpy_h2d(data->val, src.data->val, sizeof(Dtype) * (size_t)data->nnz, s));
+        GNN_HIP(gnnhip_memcpy_h2d(data->col_idx, src.data->col_idx, sizeof(int) * (size_t)data->nnz, s));
+        GNN_HIP(gnnhip_memcpy_h2d(data->row_ptr, src.data->row_ptr, sizeof(int) * (size_t)data->len_ptr, s));
+    }
+    void CopyFrom(SpTensor<GPU, Dtype>& src)
+    {
+        shape = src.shape;
+        ResizeSp(src.data->nnz, src.data->len_ptr);
+        void* s = GpuHandle::Stream();
+        GNN_HIP(gnnhip_memcpy_d2d(data->val, src.data->val, sizeof(Dtype) * (size_t)data->nnz, s));
+        GNN_HIP(gnnhip_memcpy_d2d(data->col_idx, src.data->col_idx, sizeof(int) * (size_t)data->nnz, s));
+        GNN_HIP(gnnhip_memcpy_d2d(data->row_ptr, src.data->row_ptr, sizeof(int) * (size_t)data->len_ptr, s));
+    }
+    void ShallowCopy(SpTensor<GPU, Dtype>& src) { shape = src.shape; data = src.data; }
+
+    void ArgMax(DTensor<GPU, int>& dst, uint axis = 0)
+    {
+        ASSERT(axis == 0, "not supported for axis > 0 in GPU Sparse Tensor");
+        dst.Reshape({shape[0]});
+        GNN_HIP(gnnhip_csr_row_argmax_f32(data->row_ptr, data->col_idx, data->val, (int)shape[0], dst.data->ptr,
+                                          GpuHandle::Stream()));
+    }
+
+    std::shared_ptr< SparseData<GPU, Dtype> > data;
+};
+
+// dense <- alpha * op(sparse) * dense + beta * dense
+inline void TensorTemplate<GPU, DENSE, float>::MM(SpTensor<GPU, float>& a, DTensor<GPU, float>& b,
+                                                  Trans transA, Trans transB, float alpha, float beta)
+{
+    ASSERT(transB == Trans::N, "the dense operand of a sparse product cannot be transposed");
+    size_t m, n, k;
+    GetDims(a.rows(), a.cols(), transA, b.rows(), b.cols(), transB, m, n, k);
+    Reshape({m, n});
+    if (transA == Trans::N) {
+        GNN_HIP(gnnhip_spmm_csr_f32((int)m, (int)k, (int)n, alpha, a.data->row_ptr, a.data->col_idx, a.data->val,
+                                    b.data->ptr, (int)b.cols(), beta, data->ptr, (int)n, GpuHandle::Stream()));
+    } else {
+        GNN_HIP(gnnhip_spmm_csr_t_f32((int)a.rows(), (int)a.cols(), (int)n, alpha, a.data->row_ptr, a.data->col_idx,
+                                      a.data->val, b.data->ptr, (int)b.cols(), beta, data->ptr, (int)n,
+                                      GpuHandle::Stream()));
+    }
+}
+
+// dense += a * sparse
+inline void TensorTemplate<GPU, DENSE, float>::Axpy(float a, SpTensor<GPU, float>& x)
+{
+    ASSERT(shape == x.shape, "shape doesn't match in Axpy");
+    GNN_HIP(gnnhip_csr_axpy_f32((int)x.rows(), (int)x.cols(), a, x.data->row_ptr, x.data->col_idx, x.data->val,
+                                data->ptr, GpuHandle::Stream()));
+}
+
+// ---- host <- device CSR copy declared in cpu_sparse_tensor.h
+template<typename Dtype>
+void TensorTemplate<CPU, CSR_SPARSE, Dtype>::CopyFrom(SpTensor<GPU, Dtype>& src)
+{
+    shape = src.shape;
+    ResizeSp(src.data->nnz, src.data->len_ptr);
+    void* s = GpuHandle::Stream();
+    GNN_HIP(gnnhip_memcpy_d2h(data->val, src.data->val, sizeof(Dtype) * (size_t)data->nnz, s));
+    GNN_HIP(gnnhip_memcpy_d2h(data->col_idx, src.data->col_idx, sizeof(int) * (size_t)data->nnz, s));
+    GNN_HIP(gnnhip_memcpy_d2h(data->row_ptr, src.data->row_ptr, sizeof(int) * (size_t)data->len_ptr, s));
+}
+
+}  // namespace gnn
+#endif

@@ -1,0 +1,63 @@
+// CPU-only check of the host layer: GraphStruct + the message-pass factors scheduled by
+// FactorGraph build the CSR operands of a batch; the arrays are written out for a bit-exact
+// comparison with the oracle.  Needs no GPU (mode = CPU end to end).
+//
+//   host_csr_check <in.bin> <out.bin> <average 0|1>
+//   in.bin : int32 B, N, E, then subg_id[N], node_idx[N], edge_x[E], edge_y[E]
+//   out.bin: int32 a_row_ptr[N+1], a_col[E], fp32 a_val[E], int32 s_row_ptr[B+1], s_col[N], fp32 s_val[N],
+//            int32 flags {contiguous_subgraphs, max_subgraph_nodes}
+#include <cstdio>
+#include <vector>
+#include "tensor/tensor_all.h"
+#include "nn/nn_all.h"
+
+using namespace gnn;
+
+int main(int argc, char** argv)
+{
+    ASSERT(argc == 4, "usage: host_csr_check in.bin out.bin average");
+    FILE* f = fopen(argv[1], "rb");
+    ASSERT(f, "cannot open input");
+    int hdr[3];
+    ASSERT(fread(hdr, sizeof(int), 3, f) == 3, "short header");
+    const int B = hdr[0], N = hdr[1], E = hdr[2];
+    std::vector<int> sid(N), nid(N), ex(E), ey(E);
+    ASSERT(fread(sid.data(), 4, N, f) == (size_t)N && fread(nid.data(), 4, N, f) == (size_t)N, "short read");
+    ASSERT(fread(ex.data(), 4, E, f) == (size_t)E && fread(ey.data(), 4, E, f) == (size_t)E, "short read");
+    fclose(f);
+    const bool average = atoi(argv[3]) != 0;
+
+    GraphStruct g;
+    // a first, larger batch leaves stale capacity behind; the second Resize must not leak it
+    g.Resize(B + 3, N + 5);
+    for (int i = 0; i < N + 5; ++i) g.AddNode(i % (B + 3), i);
+    g.AddEdge(0, N + 4, 0);
+    g.Resize(B, N);
+    for (int i = 0; i < N; ++i) g.AddNode(sid[i], nid[i]);
+    for (int e = 0; e < E; ++e) g.AddEdge(e, ex[e], ey[e]);
+
+    FactorGraph fg;
+    auto gv = add_const<GraphVar>(fg, "graph", true);
+    auto a = af< Node2NodeMsgPass<CPU, float> >(fg, {gv}, average);
+    auto s = af< SubgraphMsgPass<CPU, float> >(fg, {gv}, average);
+    std::map<std::string, void*> feed;
+    feed["graph"] = &g;
+    fg.FeedForward({a, s}, feed, Phase::TEST);
+    ASSERT(fg.LastPlanFactorCount() == 2, "both builders must run");
+    // requesting only one target must run only its builder
+    fg.FeedForward({s}, feed, Phase::TEST);
+    ASSERT(fg.LastPlanFactorCount() == 1, "dependency pruning failed");
+
+    FILE* o = fopen(argv[2], "wb");
+    ASSERT(o, "cannot open output");
+    auto& ad = *a->value.data;
+    auto& sd = *s->value.data;
+    ASSERT(ad.nnz == E && ad.len_ptr == N + 1 && sd.nnz == N && sd.len_ptr == B + 1, "unexpected CSR sizes");
+    fwrite(ad.row_ptr, 4, N + 1, o); fwrite(ad.col_idx, 4, E, o); fwrite(ad.val, 4, E, o);
+    fwrite(sd.row_ptr, 4, B + 1, o); fwrite(sd.col_idx, 4, N, o); fwrite(sd.val, 4, N, o);
+    auto* sf = dynamic_cast<SubgraphMsgPass<CPU, float>*>(fg.factor_list[1].get());
+    int flags[2] = {sf->contiguous_subgraphs ? 1 : 0, sf->max_subgraph_nodes};
+    fwrite(flags, 4, 2, o);
+    fclose(o);
+    return 0;
+}

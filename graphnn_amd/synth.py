@@ -273,3 +273,30 @@ def make_config(config_id, B=None):
     batch = molecule_batch(seed, cfg["B"], cfg["K"], cfg["Q"], size_mode=cfg["size_mode"], **kw)
     weights = make_weights(Stream(seed), cfg["K"], cfg["C"], cfg["H"], cfg["Q"])
     return batch, weights, cfg
+
+
+def write_graphnn_txt(batch, graph_path, train_idx_path=None, test_idx_path=None, test_fraction=0.2):
+    """Write a batch as a dataset in graphnn's txt layout (examples/graph_classification/data/README.md:1-9):
+    first line the number of graphs; per graph a line `n label`, then one line per node
+    `tag m nbr_1 .. nbr_m` with neighbour indices local to the graph.  Optionally writes index files
+    (one graph index per line) splitting the graphs into train / test."""
+    offsets = np.concatenate([[0], np.cumsum(batch.graph_sizes)])
+    # adjacency of node x = destinations of its out-edges, which are stored grouped by x and ascending
+    deg = np.bincount(batch.edge_x, minlength=batch.num_nodes)
+    starts = np.concatenate([[0], np.cumsum(deg)])
+    lines = [str(batch.num_graphs)]
+    for g in range(batch.num_graphs):
+        n, o = int(batch.graph_sizes[g]), int(offsets[g])
+        lines.append("%d %d" % (n, int(batch.graph_label[g])))
+        for j in range(n):
+            nb = batch.edge_y[starts[o + j]:starts[o + j + 1]] - o
+            lines.append(" ".join([str(int(batch.node_label[o + j])), str(nb.size)] + [str(int(v)) for v in nb]))
+    with open(graph_path, "w") as f:
+        f.write("\n".join(lines) + "\n")
+    if train_idx_path and test_idx_path:
+        n_test = max(1, int(round(batch.num_graphs * test_fraction)))
+        idx = np.arange(batch.num_graphs)
+        with open(test_idx_path, "w") as f:
+            f.write("\n".join(str(int(i)) for i in idx[:n_test]) + "\n")
+        with open(train_idx_path, "w") as f:
+            f.write("\n".join(str(int(i)) for i in idx[n_test:]) + "\n")

@@ -40,7 +40,7 @@ enum {
 };
 
 /* reduction codes — include/tensor/gpu_reduce_kernel.h:12-55 */
-enum { GNNHIP_REDUCE_SUM = 0, GNNHIP_REDUCE_MEAN = 1, GNNHIP_REDUCE_MAX = 2 };
+enum { GNNHIP_REDUCE_SUM = 0, GNNHIP_REDUCE_MEAN = 1, GNNHIP_REDUCE_MAX = 2, GNNHIP_REDUCE_SUMSQ = 3 };
 
 const char* gnnhip_last_error(void);
 const char* gnnhip_version(void);
@@ -61,8 +61,9 @@ int gnnhip_pool_stats(size_t* bytes_in_use, size_t* bytes_parked, size_t* n_driv
 
 /* ---- copies: DTensor<GPU>::CopyFrom / AsScalar / Zeros
  *      (src/tensor/gpu_dense_tensor.cu:97-150), SpTensor<GPU>::CopyFrom
- *      (src/tensor/gpu_sparse_tensor.cu:55-73).  d2h blocks until the data
- *      is in host memory (the reference's only synchronisation point). */
+ *      (src/tensor/gpu_sparse_tensor.cu:55-73).  h2d returns once the host buffer
+ *      has been read (it may be overwritten at once); d2h blocks until the data is in
+ *      host memory; d2d and memset0 are asynchronous on the stream. */
 int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream);
 int gnnhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
 int gnnhip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream);
@@ -166,7 +167,7 @@ int gnnhip_row_softmax_f32(float* x, int rows, int cols, void* stream);
  *      Segment offsets come from an exclusive scan of lens done on the device. */
 int gnnhip_jagged_softmax_f32(float* x, const int* lens, int nseg, void* stream);
 
-/* ---- global sum / mean / max into out[0] (device):
+/* ---- global sum / mean / max / sum of squares into out[0] (device):
  *      DTensor<GPU>::Sum / Mean (src/tensor/gpu_dense_tensor.cu:466-481),
  *      MatColReduceKernel (include/tensor/gpu_reduce_kernel.h:57-99) */
 int gnnhip_reduce_f32(int op, const float* x, size_t n, float* out, void* stream);
@@ -193,6 +194,33 @@ int gnnhip_in_top_k_f32(const float* pred, const int* label, int rows, int cols,
 
 /* ---- dst[i] = (float)src[i] : TypeCastCopy (src/tensor/gpu_binary_functor.cu:7-31) */
 int gnnhip_cast_i32_f32(const int* src, float* dst, size_t n, void* stream);
+
+/* ================= backward pass of the same path ================= */
+
+/* ---- C[k,n] = alpha * A^T * B + beta * C, A CSR [m,k], B dense [m,n]:
+ *      DTensor<GPU>::MM(SpTensor, DTensor, Trans::T, Trans::N) (src/tensor/gpu_dense_tensor.cu:271-294,
+ *      the cuSPARSE csrmm(T) + two geam route), used by MatMul::Backward (src/nn/matmul.cpp:35-76).
+ *      Accumulates with fp32 atomics: the order of additions into one output row is not fixed. */
+int gnnhip_spmm_csr_t_f32(int m, int k, int n, float alpha, const int* row_ptr, const int* col_idx,
+                          const float* val, const float* B, int ldb, float beta, float* C, int ldc,
+                          void* stream);
+
+/* ---- dense[r, col[t]] += a * val[t] : DTensor<GPU>::Axpy(a, SpTensor) + SpAxpyKernel
+ *      (src/tensor/gpu_dense_tensor.cu:578-609), the label term of CrossEntropy::Backward
+ *      (src/nn/cross_entropy.cpp:52-78). */
+int gnnhip_csr_axpy_f32(int rows, int cols, float a, const int* row_ptr, const int* col_idx, const float* val,
+                        float* dense, void* stream);
+
+/* ---- dst[i] += grad[i] where out[i] > 0 : ReLUDeriv(GPU) + ReLUDerivKernel (src/nn/relu.cu:18-37) */
+int gnnhip_relu_deriv_f32(size_t n, const float* out, const float* grad, float* dst, void* stream);
+
+/* ---- y[i] *= x[i] : DTensor<GPU>::ElewiseMul(DTensor) with equal shapes
+ *      (src/tensor/gpu_dense_tensor.cu:611-628, include/tensor/gpu_binary_functor.h:40-95) */
+int gnnhip_mul_f32(size_t n, const float* x, float* y, void* stream);
+
+/* ---- y[r, :] *= scale[r] : the column-broadcast case of DTensor<GPU>::ElewiseMul
+ *      (BCastEleWiseMulKernel, src/tensor/gpu_dense_tensor.cu:654-713) */
+int gnnhip_row_scale_f32(int rows, int cols, const float* scale, float* y, void* stream);
 
 #ifdef __cplusplus
 }

@@ -51,7 +51,7 @@ def test_argument_validation_needs_no_gpu():
     assert lib.gnnhip_spmm_csr_f32(4, 4, 8, f(1), None, None, None, None, 8, f(0), None, 8, None) == -1
     assert lib.gnnhip_gemm_f32(2, 0, 1, 1, 1, f(1), None, 1, None, 1, f(0), None, 1, None) == -1
     assert lib.gnnhip_unary_f32(99, None, 10, f(0), f(0), None) == -1
-    assert lib.gnnhip_reduce_f32(7, None, 10, None, None) == -1
+    assert lib.gnnhip_reduce_f32(9, None, 10, None, None) == -1
     assert lib.gnnhip_row_argmax_f32(None, 3, 0, None, None) == -1
     assert lib.gnnhip_s2v_forward_f32(0, 1, 1, 1, 1, 1, 1, *([None] * 19), None, None) == -1
     x = np.zeros(8, np.float32)
