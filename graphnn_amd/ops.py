@@ -14,7 +14,7 @@ UNARY = {
     "set": 0, "truncate": 1, "scale": 2, "add": 3, "abs": 4, "inv": 5, "relu": 6, "sigmoid": 7,
     "tanh": 8, "log": 9, "invsqrt": 10, "exp": 11, "square": 12, "sqrt": 13,
 }
-REDUCE = {"sum": 0, "mean": 1, "max": 2}
+REDUCE = {"sum": 0, "mean": 1, "max": 2, "sumsq": 3}
 
 _initialised = False
 
@@ -314,3 +314,47 @@ def cast_i32_f32(src):
 def memset0(t):
     check(_lib().gnnhip_memset0(ctypes.c_void_p(t.data_ptr()), t.numel() * t.element_size(), _stream()))
     return t
+
+
+# ---- backward-pass entry points
+def spmm_t(row_ptr, col_idx, val, B, m, k, alpha=1.0, beta=0.0, out=None):
+    """out[k,n] = alpha * A^T * B + beta * out, A CSR [m,k], B [m,n]"""
+    n = B.shape[1]
+    _check_csr(row_ptr, col_idx, val, m, "A")
+    if B.shape[0] != m:
+        raise ValueError("mat dim doesn't match")
+    if out is None:
+        out = torch.zeros((k, n), dtype=torch.float32, device=B.device)
+    check(_lib().gnnhip_spmm_csr_t_f32(m, k, n, alpha, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"),
+                                       _f32(val, "val"), _f32(B, "B"), n, beta, _f32(out, "out"), n, _stream()))
+    return out
+
+
+def csr_axpy(a, row_ptr, col_idx, val, dense):
+    rows, cols = dense.shape
+    _check_csr(row_ptr, col_idx, val, rows, "x")
+    check(_lib().gnnhip_csr_axpy_f32(rows, cols, a, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"), _f32(val, "val"),
+                                     _f32(dense, "dense"), _stream()))
+    return dense
+
+
+def relu_deriv(dst, out, grad):
+    if not (dst.numel() == out.numel() == grad.numel()):
+        raise ValueError("shape mismatch in ReLUDeriv")
+    check(_lib().gnnhip_relu_deriv_f32(dst.numel(), _f32(out, "out"), _f32(grad, "grad"), _f32(dst, "dst"), _stream()))
+    return dst
+
+
+def mul(x, y):
+    if x.numel() != y.numel():
+        raise ValueError("shape mismatch in ElewiseMul")
+    check(_lib().gnnhip_mul_f32(x.numel(), _f32(x, "x"), _f32(y, "y"), _stream()))
+    return y
+
+
+def row_scale(scale, y):
+    rows, cols = y.shape
+    if scale.numel() != rows:
+        raise ValueError("one factor per row is needed")
+    check(_lib().gnnhip_row_scale_f32(rows, cols, _f32(scale, "scale"), _f32(y, "y"), _stream()))
+    return y

@@ -601,3 +601,49 @@ def test_batched_forward_reports_broken_promises(gpu, oracle):
     with pytest.raises(GnnHipError) as err:
         ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), *dev_w, cfg["L"], 5000)
     assert err.value.code == -5
+
+
+# ------------------------------------------------------------------ backward-pass kernels
+@pytest.mark.parametrize("n", [2, 7, 64, 128])
+def test_spmm_transposed(gpu, oracle, n):
+    from graphnn_amd import ops
+    rng = np.random.default_rng(300 + n)
+    m, k = 411, 233
+    csr = _random_csr(rng, m, k, 3000)                       # duplicates present
+    B = rng.standard_normal((m, n)).astype(np.float32)
+    C0 = rng.standard_normal((k, n)).astype(np.float32)
+    got = _n(ops.spmm_t(*_csr_t(csr, gpu), _t(B, gpu), m, k))
+    assert max_rel(got, oracle.spmm_T(*csr, B, m, k)) < PARITY_TOL
+    got2 = _n(ops.spmm_t(*_csr_t(csr, gpu), _t(B, gpu), m, k, alpha=0.5, beta=2.0, out=_t(C0, gpu)))
+    assert max_rel(got2, oracle.spmm_T(*csr, B, m, k, alpha=0.5, beta=2.0, C=C0)) < PARITY_TOL
+    # the reference's own SparseMM case (A^T B), test/gpu_tensor_test.cpp:311-336
+    g = json.load(open(os.path.join(GOLDEN, "sparse_mm_known_answer.json")))
+    kc = (np.array(g["row_ptr"], np.int32), np.array(g["col_idx"], np.int32), np.array(g["val"], np.float32))
+    got3 = _n(ops.spmm_t(*_csr_t(kc, gpu), _t(np.array(g["b_for_transpose"], np.float32), gpu), g["a_rows"], g["a_cols"]))
+    assert np.array_equal(got3, np.array(g["expected_At_b"], np.float32))
+
+
+def test_gradient_elementwise_kernels(gpu):
+    from graphnn_amd import ops
+    rng = np.random.default_rng(31)
+    n = 10007
+    out = rng.standard_normal(n).astype(np.float32); out[::5] = 0.0
+    grad = rng.standard_normal(n).astype(np.float32)
+    dst = rng.standard_normal(n).astype(np.float32)
+    got = _n(ops.relu_deriv(_t(dst, gpu), _t(out, gpu), _t(grad, gpu)))
+    assert np.array_equal(got, np.where(out > 0, dst + grad, dst))
+    x = rng.standard_normal(n).astype(np.float32); y = rng.standard_normal(n).astype(np.float32)
+    assert np.array_equal(_n(ops.mul(_t(x, gpu), _t(y, gpu))), x * y)
+    M = rng.standard_normal((37, 5)).astype(np.float32); s = rng.standard_normal(37).astype(np.float32)
+    assert np.array_equal(_n(ops.row_scale(_t(s, gpu), _t(M, gpu))), M * s[:, None])
+    # dense += a * sparse, duplicates in a row accumulate in order
+    rp = np.array([0, 2, 2, 5], np.int32); ci = np.array([1, 1, 0, 3, 0], np.int32); v = np.array([1, 2, 3, 4, 5], np.float32)
+    D = np.zeros((3, 4), np.float32)
+    want = D.copy()
+    for r in range(3):
+        for t in range(rp[r], rp[r + 1]):
+            want[r, ci[t]] += np.float32(-0.5) * v[t]
+    assert np.array_equal(_n(ops.csr_axpy(-0.5, _t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(D, gpu))), want)
+    big = (rng.random(300001) * 2 - 1).astype(np.float32)
+    ss = float(_n(ops.reduce("sumsq", _t(big, gpu)))[0])
+    assert abs(ss - float((big.astype(np.float64) ** 2).sum())) <= 1e-5 * ss
