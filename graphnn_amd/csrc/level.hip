@@ -29,6 +29,11 @@
 #endif
 
 namespace gnnhip {
+
+// level_wide.hip
+int level_wide_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
+                        const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s);
+
 namespace {
 
 constexpr int kBlock = 256;
@@ -492,7 +497,7 @@ inline bool small_batch(int N) { return N <= 32 * 1024; }
 
 // ---- dispatchers used by the C entry points and by forward.hip.
 // Return GNNHIP_EUNSUPPORTED (without setting an error text) when the shape has no fused kernel.
-bool fused_hidden_supported(int C) { return C == 16 || C == 32 || C == 64; }
+bool fused_hidden_supported(int C) { return C == 16 || C == 32 || C == 64 || C == 128 || C == 256; }
 
 int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s)
 {
@@ -515,6 +520,8 @@ int level_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const f
     case 16: return launch_level<16>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
     case 32: return launch_level<32>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
     case 64: return launch_level<64>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    case 128:
+    case 256: return level_wide_dispatch(N, C, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
     }
     return GNNHIP_EUNSUPPORTED;
 }

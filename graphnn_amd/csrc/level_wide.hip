@@ -1,0 +1,424 @@
+// Fused mean-field level for wide hidden sizes (C = 128 or 256):
+//     h_out = ReLU((A * h_in) * W + bias + msg)
+// the operator chain MatMul(sparse) -> MatMul -> ElewiseAdd -> ReLU of
+// examples/graph_classification/src/kernel_mean_field.cpp:35-42 in one launch.
+//
+// At C = 256 the C x C contraction is 2 N C^2 = 131 kflop per node against
+// 3 KB of activation traffic per node: on FP32 matrix cores (157 TFLOP/s) the
+// contraction takes about twice as long as the HBM traffic, so this kernel is
+// organised around keeping the matrix pipes fed.
+//
+// One persistent workgroup of 8 wavefronts per compute unit.  W never moves
+// after start-up: wavefront w keeps the W^T operand of its C/8 output columns
+// in registers (C = 256: 128 registers per lane, half of the register file of
+// the compute unit across the 8 wavefronts).  Per pass over 64 rows:
+//   1. gather-sum  wavefront w sums the neighbour rows of 8 rows, the whole
+//                  wavefront across the C columns of a row, six row loads in
+//                  flight, and parks the sums in an LDS tile [64][C+4];
+//   2. contraction v_mfma_f32_16x16x4_f32, out^T = W^T * tile^T: the lane
+//                  (q = lane/16, t = lane%16) feeds k = (C/4) q + s at step s, so
+//                  four steps of its tile operand are one 128-bit LDS read, and it
+//                  ends up owning row t, four consecutive columns per block;
+//   3. epilogue    + bias + msg, ReLU, 128-bit stores (issued at the top of the
+//                  next 16-row block).
+// The tile is double-buffered and the gather of pass p+1 is spread, one batch
+// of six row loads per 16-row block, over the contraction of pass p; the CSR
+// indices are fetched one batch (columns, weights) or one pass (row pointers)
+// further ahead still.  Only a wavefront whose 8 rows hold more than 24 entries
+// gathers in the open.
+//
+// What shaped the code (measured on MI355X):
+//   * While a wavefront streams FP32 matrix instructions, every other
+//     instruction issued on that SIMD, by either wavefront and of any kind
+//     (vector, scalar, LDS, memory), gets about one issue slot per matrix
+//     instruction (14 ns) instead of one per 2 ns.  The budget is therefore one
+//     non-matrix instruction per matrix instruction; beyond it the matrix pipe
+//     idles.  Hence: CSR indices through scalar loads (no broadcast
+//     instructions), buffer addressing (a gathered row costs one scalar shift
+//     and one load; rows past N are dropped by the descriptor's size, not by a
+//     predicate), msg/bias added after the contraction in 8 + 8 adds.
+//   * Vector memory operations retire in order, so any wait for a load also
+//     waits for every store issued before it.  Stores are therefore issued
+//     right before a contraction, never right before a wait.
+//   * The loads of a batch and their uses sit under separate (uniform)
+//     conditions; the compiler then assumes a path on which loads are still in
+//     flight and waits at the top of the next block.  One explicit wait after
+//     the contraction removes that.
+#include "gnnhip_internal.h"
+
+// Phase accounting for a timing build of this file; expands to nothing in the library.
+#ifndef GNNHIP_PHASE_ACC
+#define GNNHIP_PHASE_ACC(i)
+#define GNNHIP_PHASE_INIT
+#define GNNHIP_PHASE_FINI
+#endif
+
+
+namespace gnnhip {
+namespace {
+
+constexpr int kTileRows = 64;                    // rows per pass
+constexpr int kInFlight = 6;                     // row gathers in flight per wavefront
+constexpr int kWaitVmcnt0 = 0x0F70;              // s_waitcnt operand: vmcnt(0), other counters unconstrained
+
+template <int VEC> struct VecT;
+template <> struct VecT<2> { using type = float2; };
+template <> struct VecT<4> { using type = float4; };
+
+// Buffer addressing: the memory instruction takes a 128-bit descriptor (base, size), a per-lane 32-bit
+// offset and a scalar 32-bit offset, so a gathered row costs one scalar shift and no per-lane address
+// arithmetic, and lanes whose offset lies past the size are dropped by the hardware (no predication).
+using rsrc_t = __amdgpu_buffer_rsrc_t;
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+constexpr int kRsrcWord3 = 0x00020000;           // raw buffer of 32-bit data on gfx9-family hardware
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, unsigned bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, kRsrcWord3);
+}
+__device__ __forceinline__ float4 buf_load4(rsrc_t r, int voff, int soff)
+{
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+    return make_float4(__uint_as_float(v[0]), __uint_as_float(v[1]), __uint_as_float(v[2]), __uint_as_float(v[3]));
+}
+__device__ __forceinline__ float2 buf_load2(rsrc_t r, int voff, int soff)
+{
+    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+    return make_float2(__uint_as_float(v[0]), __uint_as_float(v[1]));
+}
+__device__ __forceinline__ void buf_store4(rsrc_t r, int voff, int soff, const float4& x)
+{
+    const u32x4 v = {__float_as_uint(x.x), __float_as_uint(x.y), __float_as_uint(x.z), __float_as_uint(x.w)};
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, soff, 0);
+}
+template <int VEC> struct BufLoad;
+template <> struct BufLoad<4> { static __device__ __forceinline__ float4 get(rsrc_t r, int v, int s) { return buf_load4(r, v, s); } };
+template <> struct BufLoad<2> { static __device__ __forceinline__ float2 get(rsrc_t r, int v, int s) { return buf_load2(r, v, s); } };
+
+template <int VEC>
+__device__ __forceinline__ void vec_fma(float (&acc)[VEC], float a, const typename VecT<VEC>::type& x)
+{
+    const float* p = reinterpret_cast<const float*>(&x);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = fmaf(a, p[i], acc[i]);
+}
+
+// Everything that steers the gather (row pointers, column indices, edge weights) is uniform
+// across the wavefront and is fetched with scalar loads: the values land in scalar registers, cost
+// no vector instruction to broadcast, and are counted apart from vector memory operations, so
+// waiting for them never waits for a store.  That matters because on this hardware the FP32 matrix
+// instructions and ordinary vector instructions do not overlap: every vector instruction issued by
+// either wavefront of a SIMD takes time away from its matrix pipe.
+template <int C, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
+    int N, int tiles_per_block, const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
+    const float* __restrict__ val, const float* __restrict__ h_in, const float* __restrict__ W,
+    const float* __restrict__ msg, const float* __restrict__ bias, float* __restrict__ h_out)
+{
+    constexpr int KS = C / 4;                    // contraction steps
+    constexpr int kWideBlock = WAVES * kWave;
+    constexpr int CW = C / WAVES;                // output columns per wavefront
+    constexpr int NB = CW / 16;                  // 16-column blocks per wavefront
+    constexpr int VEC = C / kWave;               // gathered floats per lane
+    constexpr int LDT = C + 4;                   // LDS row stride: rows 0..7 start in distinct 16-byte bank groups
+    constexpr int RPW = kTileRows / WAVES;       // rows gathered per wavefront per pass
+    using vec_t = typename VecT<VEC>::type;
+
+    extern __shared__ float tiles[];             // two tiles [kTileRows][LDT]: one read by the matrix cores,
+                                                 // the other being filled for the next pass
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int q = lane >> 4, t = lane & 15;
+    const int col0 = wave * CW;
+    const int gather_off = (wave * RPW) * LDT + lane * VEC;
+    float* bias_lds = tiles + 2 * kTileRows * LDT;      // [C], read in the epilogue without a trip to memory
+    if (bias)
+        for (int i = threadIdx.x; i < C; i += kWideBlock) bias_lds[i] = bias[i];
+
+    // W^T operand: wreg[jb][s] = W[KS q + s][col0 + 16 jb + t]
+    float wreg[NB][KS];
+#pragma unroll
+    for (int jb = 0; jb < NB; ++jb)
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+            wreg[jb][s] = W[(size_t)(KS * q + s) * C + col0 + 16 * jb + t];
+
+    const int ntiles = (int)(((long long)N + kTileRows - 1) / kTileRows);
+    const int tile_begin = (int)min((long long)blockIdx.x * tiles_per_block, (long long)ntiles);
+    const int tile_end = (int)min((long long)ntiles, (long long)tile_begin + tiles_per_block);
+    if (tile_begin >= tile_end) return;
+
+    // ---- loaders.  The 9 row pointers of a pass sit in lanes 0..8 of one vector register; columns
+    //      and weights of a batch are uniform and come through scalar loads (weights as bit patterns
+    //      so that selecting them stays on the scalar unit).
+    auto load_rowptrs = [&](int tile_id) {
+        const long long r0 = (long long)tile_id * kTileRows + wave * RPW;
+        int v = 0;
+        if (lane <= RPW) v = row_ptr[min(r0 + lane, (long long)N)];
+        return v;
+    };
+    const int* val_bits = reinterpret_cast<const int*>(val);
+    // entries [s, s + kInFlight) of the CSR arrays.  What lies past the end of the wavefront's rows is
+    // loaded but never added, so the batch is read as it lies; only at the very end of the arrays do
+    // the indices have to be clamped.  No selection on the loaded values here: a scalar load followed
+    // at once by a use of its result is a full trip to the scalar cache each.
+    const int nnz = row_ptr[N];
+    auto load_cols = [&](int s, int (&c)[kInFlight]) {
+        if (s + kInFlight <= nnz) {
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) c[u] = col_idx[s + u];
+        } else {
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) c[u] = col_idx[min(s + u, nnz - 1)];
+        }
+    };
+    auto load_weights = [&](int s, int (&a)[kInFlight]) {
+        if (s + kInFlight <= nnz) {
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) a[u] = val_bits[s + u];
+        } else {
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) a[u] = val_bits[min(s + u, nnz - 1)];
+        }
+    };
+    const rsrc_t h_rsrc = make_rsrc(h_in, (unsigned)((size_t)N * C * 4));
+    auto issue = [&](const int (&c)[kInFlight], vec_t (&x)[kInFlight]) {
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u)
+            x[u] = BufLoad<VEC>::get(h_rsrc, lane * (VEC * 4), c[u] * (C * 4));     // N C 4 < 2^32 (host-checked)
+    };
+
+    // ---- state of the gather of one pass: entries [e, ee) of the wavefront's 8 rows, taken in order;
+    //      a row goes to LDS when its last entry has been added
+    int e = 0, ee = 0, lr = 0, row_end = 0, rpv = 0;
+    float* dstp = nullptr;
+    float acc[VEC];
+    auto begin = [&](int rp_lanes, int eb, int eend, float* dst) {
+        rpv = rp_lanes;
+        e = eb; ee = eend; lr = 0;
+        row_end = __builtin_amdgcn_readlane(rpv, 1);
+        dstp = dst;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+    };
+    auto flush_row = [&]() {
+        *reinterpret_cast<vec_t*>(dstp) = *reinterpret_cast<vec_t*>(acc);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+        dstp += LDT;
+        ++lr;
+        row_end = __builtin_amdgcn_readlane(rpv, min(lr + 1, RPW));
+    };
+    auto consume = [&](const int (&a)[kInFlight], const vec_t (&x)[kInFlight]) {
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) {
+            if (e + u < ee) {
+                while (e + u >= row_end) flush_row();          // rows ending here (possibly empty ones)
+                vec_fma<VEC>(acc, __int_as_float(a[u]), x[u]);
+            }
+        }
+        e += kInFlight;
+    };
+    auto finish = [&]() { while (lr < RPW) flush_row(); };      // the open row and empty rows after it
+
+    // Output of the last finished 16-row block, stored at the top of the following block (or at the end
+    // of the pass): a store then has a whole contraction between its issue and the next wait on
+    // vector memory.  msg and h_out are addressed through descriptors that cover the rows of the
+    // current pass only, so rows past N fall outside and need no predicate.
+    float4 outv[NB];
+    int out_rt = -1;                             // block of this pass held in outv, -1: none
+#pragma unroll
+    for (int jb = 0; jb < NB; ++jb) outv[jb] = f4_zero();
+    const int lane_off = (t * C + col0 + 4 * q) * 4;              // byte offset of this lane inside a 16-row block
+    rsrc_t msg_rsrc = make_rsrc(msg, 0), out_rsrc = make_rsrc(h_out, 0);
+    auto store_pending = [&]() {
+        if (out_rt >= 0) {
+#pragma unroll
+            for (int jb = 0; jb < NB; ++jb) buf_store4(out_rsrc, lane_off + out_rt * (16 * C * 4) + 64 * jb, 0, outv[jb]);
+        }
+        out_rt = -1;
+    };
+
+    GNNHIP_PHASE_INIT
+    int cC[kInFlight], aC[kInFlight];            // columns / weights of the next batch to issue / to sum
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) { cC[u] = 0; aC[u] = 0; }
+
+    // ---- first pass: its gather has nothing to hide behind
+    int rp_next = load_rowptrs(tile_begin);      // row pointers of the next pass to gather
+    int ebN = __builtin_amdgcn_readlane(rp_next, 0), eeN = __builtin_amdgcn_readlane(rp_next, RPW);
+    begin(rp_next, ebN, eeN, tiles + gather_off);
+    while (e < ee) {
+        vec_t x[kInFlight];
+        load_cols(e, cC);
+        load_weights(e, aC);
+        issue(cC, x);
+        consume(aC, x);
+    }
+    finish();
+    ebN = eeN = 0;
+    if (tile_begin + 1 < tile_end) {
+        rp_next = load_rowptrs(tile_begin + 1);
+        ebN = __builtin_amdgcn_readlane(rp_next, 0);
+        eeN = __builtin_amdgcn_readlane(rp_next, RPW);
+        if (ebN < eeN) { load_cols(ebN, cC); load_weights(ebN, aC); }
+    }
+    __syncthreads();
+    GNNHIP_PHASE_ACC(0);
+
+    for (int tile_id = tile_begin; tile_id < tile_end; ++tile_id) {
+        const long long row0 = (long long)tile_id * kTileRows;
+        const int parity = (tile_id - tile_begin) & 1;
+        const float* cur = tiles + parity * (kTileRows * LDT);
+        const bool has_next = tile_id + 1 < tile_end;
+        const bool has_next2 = tile_id + 2 < tile_end;
+        begin(rp_next, ebN, eeN, tiles + (parity ^ 1) * (kTileRows * LDT) + gather_off);   // empty when !has_next
+        {
+            const long long left = (long long)N - row0;
+            const unsigned bytes = (unsigned)(min(left, (long long)kTileRows) * (C * 4));
+            out_rsrc = make_rsrc(h_out + (size_t)row0 * C, bytes);
+            msg_rsrc = make_rsrc(msg ? msg + (size_t)row0 * C : nullptr, msg ? bytes : 0u);   // no msg: every load reads 0
+        }
+        if (has_next2) rp_next = load_rowptrs(tile_id + 2);
+
+        // ---- contraction and epilogue, one 16-row block at a time; each block also carries one batch
+        //      of the next pass's gather, issued before its matrix instructions and summed after them
+#pragma unroll 1
+        for (int rt = 0; rt < kTileRows / 16; ++rt) {
+            // msg is asked for now and added after the contraction (as the accumulators' initial value it
+            // would have to arrive before the first matrix instruction)
+            float4 mm[NB];
+            mfma_f4 acc_m[NB];
+#pragma unroll
+            for (int jb = 0; jb < NB; ++jb) {
+                mm[jb] = buf_load4(msg_rsrc, lane_off + rt * (16 * C * 4) + 64 * jb, 0);
+                acc_m[jb] = mfma_f4{0.f, 0.f, 0.f, 0.f};
+            }
+            vec_t x[kInFlight];
+            const bool batch = e < ee;
+            if (batch) issue(cC, x);
+            store_pending();
+            // where the follower of this batch starts: inside this pass, or (after the last block) at the
+            // first entry of the next pass; its columns travel while the matrix cores work
+            int ns = 0, nend = 0;
+            if (rt < kTileRows / 16 - 1) {
+                if (e + kInFlight < ee) { ns = e + kInFlight; nend = ee; }
+            } else if (e + kInFlight >= ee) {
+                ns = ebN; nend = eeN;                     // both zero when there is no next pass
+            }
+            if (ns < nend) load_cols(ns, cC);
+            GNNHIP_PHASE_ACC(1);
+
+            const float* src = cur + (rt * 16 + t) * LDT + KS * q;
+            // the tile operand is read two 128-bit words (eight contraction steps) ahead of its use
+            float4 b_cur[2], b_nxt[2];
+            b_cur[0] = *reinterpret_cast<const float4*>(src);
+            b_cur[1] = *reinterpret_cast<const float4*>(src + 4);
+#pragma unroll
+            for (int s8 = 0; s8 < KS / 8; ++s8) {
+                if (s8 + 1 < KS / 8) {
+                    b_nxt[0] = *reinterpret_cast<const float4*>(src + 8 * (s8 + 1));
+                    b_nxt[1] = *reinterpret_cast<const float4*>(src + 8 * (s8 + 1) + 4);
+                }
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const float4 b = b_cur[h];
+                    const int s0 = 8 * s8 + 4 * h;
+#pragma unroll
+                    for (int jb = 0; jb < NB; ++jb) acc_m[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(wreg[jb][s0 + 0], b.x, acc_m[jb], 0, 0, 0);
+#pragma unroll
+                    for (int jb = 0; jb < NB; ++jb) acc_m[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(wreg[jb][s0 + 1], b.y, acc_m[jb], 0, 0, 0);
+#pragma unroll
+                    for (int jb = 0; jb < NB; ++jb) acc_m[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(wreg[jb][s0 + 2], b.z, acc_m[jb], 0, 0, 0);
+#pragma unroll
+                    for (int jb = 0; jb < NB; ++jb) acc_m[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(wreg[jb][s0 + 3], b.w, acc_m[jb], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);            // keeps the read-ahead where it is written
+                b_cur[0] = b_nxt[0]; b_cur[1] = b_nxt[1];
+            }
+            GNNHIP_PHASE_ACC(2);
+            // One unconditional wait for everything this block asked for (gathered rows, msg).  The loads
+            // and their uses sit under separate conditions; without this the compiler has to assume a
+            // path on which they are still in flight and waits at the top of the next block instead,
+            // where the wait also covers the stores issued just before it.
+            __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
+            if (batch) consume(aC, x);
+            if (ns < nend) load_weights(ns, aC);
+            if (rt == 0) {                                // the row pointers asked for at the top have arrived
+                ebN = eeN = 0;
+                if (has_next2) {
+                    ebN = __builtin_amdgcn_readlane(rp_next, 0);
+                    eeN = __builtin_amdgcn_readlane(rp_next, RPW);
+                }
+            }
+            GNNHIP_PHASE_ACC(3);
+#pragma unroll
+            for (int jb = 0; jb < NB; ++jb) {
+                acc_m[jb][0] += mm[jb].x; acc_m[jb][1] += mm[jb].y; acc_m[jb][2] += mm[jb].z; acc_m[jb][3] += mm[jb].w;
+            }
+#pragma unroll
+            for (int jb = 0; jb < NB; ++jb) {
+                float4 v = make_float4(acc_m[jb][0], acc_m[jb][1], acc_m[jb][2], acc_m[jb][3]);
+                if (bias) {
+                    const float4 b4 = *reinterpret_cast<const float4*>(bias_lds + col0 + 16 * jb + 4 * q);
+                    v.x += b4.x; v.y += b4.y; v.z += b4.z; v.w += b4.w;
+                }
+                outv[jb] = make_float4(relu_ref(v.x), relu_ref(v.y), relu_ref(v.z), relu_ref(v.w));
+            }
+            out_rt = rt;
+            GNNHIP_PHASE_ACC(4);
+        }
+        if (e < ee) {                                     // more than four batches: finish in the open
+            while (e < ee) {
+                vec_t x[kInFlight];
+                load_cols(e, cC);
+                load_weights(e, aC);
+                issue(cC, x);
+                consume(aC, x);
+            }
+            if (ebN < eeN) { load_cols(ebN, cC); load_weights(ebN, aC); }
+        }
+        if (has_next) finish();
+        store_pending();
+        GNNHIP_PHASE_ACC(5);
+        __syncthreads();                                  // the tile just filled is complete, the other one is free
+        GNNHIP_PHASE_ACC(6);
+    }
+    GNNHIP_PHASE_FINI
+}
+
+template <int C, int WAVES>
+int launch_level_wide(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
+                      const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
+{
+    if ((unsigned long long)N * C * 4ull >= (1ull << 32)) return GNNHIP_EUNSUPPORTED;   // 32-bit buffer offsets
+    const long long ntiles = ((long long)N + kTileRows - 1) / kTileRows;
+    const long long per = (ntiles + kNumCU - 1) / kNumCU;            // contiguous run of tiles per workgroup
+    const long long blocks = (ntiles + per - 1) / per;
+    const size_t smem = sizeof(float) * (2 * kTileRows * (C + 4) + C);
+    static bool attr_set = false;                                    // more than 64 KB of LDS has to be asked for
+    if (!attr_set) {
+        GNNHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&s2v_level_wide_kernel<C, WAVES>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((s2v_level_wide_kernel<C, WAVES>), dim3((unsigned)blocks), dim3(WAVES * kWave), smem, s,
+                       N, (int)per, row_ptr, col_idx, val, h_in, W, msg, bias, h_out);
+    GNNHIP_LAUNCH_CHECK("s2v_level_wide");
+    return GNNHIP_OK;
+}
+
+}  // namespace
+
+int level_wide_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
+                        const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
+{
+    switch (C) {
+    case 128: return launch_level_wide<128, 8>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    case 256: return launch_level_wide<256, 8>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    }
+    return GNNHIP_EUNSUPPORTED;
+}
+
+}  // namespace gnnhip

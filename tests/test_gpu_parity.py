@@ -332,7 +332,7 @@ def test_input_stage(gpu, oracle, C, K):
     assert np.array_equal(_n(h0), np.maximum(_n(msg), 0))       # ReLU of what was stored, exactly
 
 
-@pytest.mark.parametrize("C", [16, 32, 64, 48, 128])
+@pytest.mark.parametrize("C", [16, 32, 64, 48, 128, 256])
 @pytest.mark.parametrize("with_msg,with_bias", [(True, False), (True, True), (False, False)])
 def test_level_stage(gpu, oracle, C, with_msg, with_bias):
     from graphnn_amd import ops
@@ -359,6 +359,26 @@ def test_level_stage_hub_rows_and_weights(gpu, oracle):
     nnz = int(rp[-1])
     ci = rng.integers(0, N, nnz).astype(np.int32)
     v = (rng.random(nnz) * 0.1).astype(np.float32)
+    h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
+    W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
+    msg = rng.standard_normal((N, C)).astype(np.float32)
+    want = oracle.level(rp, ci, v, h_in, W, msg, None)
+    got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu)))
+    assert max_rel(got, want) < PARITY_TOL
+
+
+@pytest.mark.parametrize("C", [128, 256])
+def test_wide_level_ragged_rows_and_weights(gpu, oracle, C):
+    """wide-hidden kernel: empty rows, rows longer than one 64-entry index batch, a row count that is
+    not a multiple of the 64-row pass, non-unit weights"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(90 + C)
+    N = 64 * 300 + 37                                   # more passes than compute units take one each
+    lens = rng.integers(0, 7, N); lens[5] = 700; lens[6] = 0; lens[7] = 0; lens[N - 1] = 130; lens[64:72] = 0
+    rp = np.zeros(N + 1, np.int32); np.cumsum(lens, out=rp[1:])
+    nnz = int(rp[-1])
+    ci = rng.integers(0, N, nnz).astype(np.int32)
+    v = (rng.random(nnz) * 0.5).astype(np.float32)
     h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
     W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
     msg = rng.standard_normal((N, C)).astype(np.float32)
