@@ -35,12 +35,12 @@ SIGNATURES = {
     "gnnhip_memcpy_d2d": [_P, _P, _Z, _P],
     "gnnhip_memset0": [_P, _Z, _P],
     "gnnhip_stream_sync": [_P],
-    "gnnhip_spmm_csr_f32": [_I, _I, _I, _F, _P, _P, _P, _P, _I, _F, _P, _I, _P],
+    "gnnhip_spmm_csr_f32": [_I, _I, _I, _I, _F, _P, _P, _P, _P, _I, _F, _P, _I, _P],
     "gnnhip_gemm_f32": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P],
-    "gnnhip_s2v_level_f32": [_I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P],
+    "gnnhip_s2v_level_f32": [_I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_s2v_input_f32": [_I, _I, _I, _P, _P, _P, _P, _P],
     "gnnhip_s2v_readout_f32": [_I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
-    "gnnhip_s2v_forward_f32": [_I] * 7 + [_P] * 11 + [_P] * 8 + [POINTER(c_int), _P],
+    "gnnhip_s2v_forward_f32": [_I] * 8 + [_P] * 11 + [_P] * 8 + [POINTER(c_int), _P],
     "gnnhip_s2v_forward_batched_f32": [_I] * 8 + [_P] * 11 + [_P] * 7 + [_P, _P],
     "gnnhip_unary_f32": [_I, _P, _Z, _F, _F, _P],
     "gnnhip_relu_f32": [_P, _P, _Z, _P],

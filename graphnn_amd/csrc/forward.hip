@@ -10,12 +10,12 @@ namespace gnnhip {
 // defined in level.hip / spmm.hip / gemm.hip / reduce.hip
 bool fused_hidden_supported(int C);
 int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s);
-int level_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
+int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
                    const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s);
 int readout_dispatch(int B, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                      const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
                      float* logits, float* probs, int* pred, hipStream_t s);
-int spmm_dispatch(int m, int n, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+int spmm_dispatch(int m, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s);
 int gemm_dispatch(int transA, int transB, int m, int n, int k, float alpha, const float* A, int lda,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s);
@@ -62,16 +62,16 @@ int input_any(int N, int K, int C, const float* X, const float* Wn2l, float* msg
     return GNNHIP_OK;
 }
 
-int level_any(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
+int level_any(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
               const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
 {
-    int rc = level_dispatch(N, C, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    int rc = level_dispatch(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
     void* tmp = nullptr;
     const size_t total = (size_t)N * C;
     if ((rc = stream_scratch(s, sizeof(float) * total, &tmp))) return rc;
     float* agg = static_cast<float*>(tmp);
-    if ((rc = spmm_dispatch(N, C, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, agg, C, s))) return rc;
+    if ((rc = spmm_dispatch(N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, agg, C, s))) return rc;
     if ((rc = gemm_dispatch(0, 0, N, C, C, 1.f, agg, C, W, C, 0.f, h_out, C, s))) return rc;
     hipLaunchKernelGGL(bias_add_relu_kernel, dim3(ew_grid(total)), dim3(kBlock), 0, s,
                        h_out, bias, msg, h_out, (float*)nullptr, total, C, 1);
@@ -85,13 +85,13 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const float* __restrict__ 
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) dst[i] = src[i];
 }
 
-int readout_any(int B, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+int readout_any(int B, int N, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                 const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
                 float* logits, float* probs, int* pred, hipStream_t s)
 {
     int rc = readout_dispatch(B, C, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
-    if ((rc = spmm_dispatch(B, C, 1.f, s_row_ptr, s_col_idx, s_val, h, C, 0.f, pool, C, s))) return rc;
+    if ((rc = spmm_dispatch(B, C, (long long)N, 1.f, s_row_ptr, s_col_idx, s_val, h, C, 0.f, pool, C, s))) return rc;
     if ((rc = gemm_dispatch(0, 0, B, H, C, 1.f, pool, C, Wh1, H, 0.f, hidden, H, s))) return rc;
     const size_t bh = (size_t)B * H;
     hipLaunchKernelGGL(bias_add_relu_kernel, dim3(ew_grid(bh)), dim3(kBlock), 0, s,
@@ -124,16 +124,16 @@ int gnnhip_s2v_input_f32(int N, int K, int C, const float* X, const float* W_n2l
     return input_any(N, K, C, X, W_n2l, msg, h0, as_stream(stream));
 }
 
-int gnnhip_s2v_level_f32(int N, int C, const int* row_ptr, const int* col_idx, const float* val,
+int gnnhip_s2v_level_f32(int N, int C, int nnz, const int* row_ptr, const int* col_idx, const float* val,
                          const float* h_in, const float* W, const float* msg, const float* bias,
                          float* h_out, void* stream)
 {
-    GNNHIP_REQUIRE(N >= 0 && C >= 1, "bad shape in s2v_level (N=%d C=%d)", N, C);
+    GNNHIP_REQUIRE(N >= 0 && C >= 1 && nnz >= 0, "bad shape in s2v_level (N=%d C=%d nnz=%d)", N, C, nnz);
     if (N == 0) return GNNHIP_OK;
     GNNHIP_REQUIRE(row_ptr && h_in && W && h_out, "null tensor in s2v_level");
     GNNHIP_REQUIRE(h_in != h_out, "s2v_level cannot run in place");
     if (int rc = require_ready()) return rc;
-    return level_any(N, C, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, as_stream(stream));
+    return level_any(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, as_stream(stream));
 }
 
 int gnnhip_s2v_readout_f32(int B, int N, int C, int H, int Q,
@@ -146,11 +146,11 @@ int gnnhip_s2v_readout_f32(int B, int N, int C, int H, int Q,
     GNNHIP_REQUIRE(s_row_ptr && W_h1 && W_h2 && pool && hidden && logits, "null tensor in s2v_readout");
     GNNHIP_REQUIRE(N == 0 || (s_col_idx && s_val && h), "null tensor in s2v_readout");
     if (int rc = require_ready()) return rc;
-    return readout_any(B, C, H, Q, s_row_ptr, s_col_idx, s_val, h, W_h1, W_h2, pool, hidden, logits, probs, pred,
+    return readout_any(B, N, C, H, Q, s_row_ptr, s_col_idx, s_val, h, W_h1, W_h2, pool, hidden, logits, probs, pred,
                        as_stream(stream));
 }
 
-int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L,
+int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L, int a_nnz,
                            const int* a_row_ptr, const int* a_col_idx, const float* a_val,
                            const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                            const float* X, const float* W_n2l, const float* W_conv,
@@ -159,7 +159,7 @@ int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L,
                            float* pool, float* hidden, float* logits, float* probs, int* pred,
                            int* which_h, void* stream)
 {
-    GNNHIP_REQUIRE(N >= 1 && B >= 1 && K >= 1 && C >= 1 && H >= 1 && Q >= 1 && L >= 0,
+    GNNHIP_REQUIRE(N >= 1 && B >= 1 && K >= 1 && C >= 1 && H >= 1 && Q >= 1 && L >= 0 && a_nnz >= 0,
                    "bad shape in s2v_forward (N=%d B=%d K=%d C=%d H=%d Q=%d L=%d)", N, B, K, C, H, Q, L);
     GNNHIP_REQUIRE(a_row_ptr && s_row_ptr && s_col_idx && s_val && X && W_n2l && W_conv && W_h1 && W_h2,
                    "null input in s2v_forward");
@@ -172,11 +172,11 @@ int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L,
     float* cur = h_a;
     float* nxt = h_b;
     for (int lv = 0; lv < L; ++lv) {
-        if ((rc = level_any(N, C, a_row_ptr, a_col_idx, a_val, cur, W_conv, msg, nullptr, nxt, s))) return rc;
+        if ((rc = level_any(N, C, a_nnz, a_row_ptr, a_col_idx, a_val, cur, W_conv, msg, nullptr, nxt, s))) return rc;
         float* t = cur; cur = nxt; nxt = t;
     }
     if (which_h) *which_h = (cur == h_a) ? 0 : 1;
-    return readout_any(B, C, H, Q, s_row_ptr, s_col_idx, s_val, cur, W_h1, W_h2, pool, hidden, logits, probs, pred, s);
+    return readout_any(B, N, C, H, Q, s_row_ptr, s_col_idx, s_val, cur, W_h1, W_h2, pool, hidden, logits, probs, pred, s);
 }
 
 }  // extern "C"

@@ -145,6 +145,23 @@ int pool_release(void* p);
 // share it.  The pointer stays valid until a later call on the same stream asks
 // for more bytes.
 int stream_scratch(hipStream_t s, size_t bytes, void** p);
+// The same with several independent buffers per stream (slot 0 is stream_scratch's):
+// slot 1 holds the hub pre-pass results, which must outlive a consumer that itself
+// takes slot 0.
+constexpr int kScratchSlots = 2;
+int stream_scratch_slot(hipStream_t s, int slot, size_t bytes, void** p);
+
+// ---- high-degree rows (hub.hip)
+constexpr int kHubThreshold = 256;     // rows with more entries are summed by the pre-pass
+constexpr int kHubChunk = 2048;        // entries per partial sum of the pre-pass
+constexpr int kHubMinRows = 32768;     // smaller matrices skip the pre-pass: its launches would cost more than a long row
+struct HubPlan {
+    const int* row_slot;               // [m], defined for rows longer than kHubThreshold only; -1: not summed
+    const float* agg;                  // [slots][ld]
+    int ld;
+};
+int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
+                const float* B, int ldb, hipStream_t s, HubPlan* plan);
 
 }  // namespace gnnhip
 

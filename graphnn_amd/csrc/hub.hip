@@ -1,0 +1,354 @@
+// Balanced pre-pass for high-degree rows ("hubs") of a CSR matrix.
+//
+// The SpMM and fused-level kernels give a row to a group of lanes, which is right
+// for the short rows of molecule batches and of uniform random graphs but leaves
+// one group, or one workgroup, alone with a row of 10^5 entries on a power-law
+// graph (R-MAT, a = 0.57: the largest of 4M rows holds 160,000 of 64M entries, and
+// the hubs sit next to each other at the low row indices).  Rows with more than
+// kHubThreshold entries are therefore summed here, ahead of the consumer kernel,
+// with the work cut by entries instead of by rows:
+//
+//   count   per 1024 rows: number of hubs and of their chunks (kHubChunk entries each)
+//   scan    exclusive scan of those counts by one workgroup -> slots of hubs and chunks
+//   fill    row_slot[row] (written for hubs only), per hub its first chunk, per chunk its hub
+//   partial one wavefront per chunk: part[chunk][n] = sum of val * B[col, :] over the chunk
+//   combine one lane group per hub: agg[slot][n] = sum of its chunks' partials in chunk order
+//
+// The consumer reads agg[row_slot[row]] for a row whose length exceeds the
+// threshold.  Every sum is taken in an order fixed by the matrix structure, so the
+// result does not depend on scheduling; there are no atomics.
+#include "gnnhip_internal.h"
+
+namespace gnnhip {
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kRowsPerBlock = 1024;          // count / fill: four consecutive rows per lane
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+__device__ __forceinline__ int hub_chunks(int deg) { return (deg + kHubChunk - 1) / kHubChunk; }
+
+// Exclusive prefix over the 256 lanes of the workgroup, in lane order; *total receives the sum.
+__device__ __forceinline__ int block_exclusive_scan(int v, int* sh, int* total)
+{
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    int incl = v;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int o = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += o;
+    }
+    if (lane == kWave - 1) sh[wave] = incl;
+    __syncthreads();
+    int base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) {
+        if (w < wave) base += sh[w];
+        tot += sh[w];
+    }
+    __syncthreads();
+    *total = tot;
+    return base + incl - v;
+}
+
+__global__ __launch_bounds__(kBlock) void hub_count_kernel(int m, const int* __restrict__ row_ptr,
+                                                            int* __restrict__ block_hubs, int* __restrict__ block_chunks)
+{
+    __shared__ int sh[2][kWavesPerBlock];
+    const long long r0 = (long long)blockIdx.x * kRowsPerBlock + threadIdx.x * 4;
+    int hubs = 0, chunks = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const long long r = r0 + i;
+        if (r < m) {
+            const int deg = row_ptr[r + 1] - row_ptr[r];
+            if (deg > kHubThreshold) { ++hubs; chunks += hub_chunks(deg); }
+        }
+    }
+    hubs = wave_sum_i(hubs);
+    chunks = wave_sum_i(chunks);
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (lane == 0) { sh[0][wave] = hubs; sh[1][wave] = chunks; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int h = 0, c = 0;
+        for (int w = 0; w < kWavesPerBlock; ++w) { h += sh[0][w]; c += sh[1][w]; }
+        block_hubs[blockIdx.x] = h;
+        block_chunks[blockIdx.x] = c;
+    }
+}
+
+// In-place exclusive scan of two arrays of nb entries by one workgroup; totals go to counts[0..1].
+constexpr int kScanBlock = 1024;
+__global__ __launch_bounds__(kScanBlock) void hub_scan_kernel(int nb, int* __restrict__ block_hubs,
+                                                               int* __restrict__ block_chunks, int* __restrict__ counts)
+{
+    __shared__ int wave_tot[2][kScanBlock / kWave];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int per = (nb + kScanBlock - 1) / kScanBlock;
+    const int lo = min(tid * per, nb), hi = min(lo + per, nb);
+    int lh = 0, lc = 0;
+    for (int i = lo; i < hi; ++i) { lh += block_hubs[i]; lc += block_chunks[i]; }
+    int ih = lh, ic = lc;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int oh = __shfl_up(ih, d, kWave), oc = __shfl_up(ic, d, kWave);
+        if (lane >= d) { ih += oh; ic += oc; }
+    }
+    if (lane == kWave - 1) { wave_tot[0][wave] = ih; wave_tot[1][wave] = ic; }
+    __syncthreads();
+    int bh = 0, bc = 0;
+    for (int w = 0; w < wave; ++w) { bh += wave_tot[0][w]; bc += wave_tot[1][w]; }
+    int rh = bh + ih - lh, rc = bc + ic - lc;
+    for (int i = lo; i < hi; ++i) {
+        const int h = block_hubs[i], c = block_chunks[i];
+        block_hubs[i] = rh; block_chunks[i] = rc;
+        rh += h; rc += c;
+    }
+    if (tid == kScanBlock - 1) { counts[0] = rh; counts[1] = rc; }
+}
+
+__global__ __launch_bounds__(kBlock) void hub_fill_kernel(int m, const int* __restrict__ row_ptr,
+                                                           const int* __restrict__ block_hubs, const int* __restrict__ block_chunks,
+                                                           int hub_cap, int chunk_cap, int* __restrict__ row_slot,
+                                                           int* __restrict__ hub_row, int* __restrict__ hub_chunk0,
+                                                           int* __restrict__ chunk_hub)
+{
+    __shared__ int sh[kWavesPerBlock];
+    const long long r0 = (long long)blockIdx.x * kRowsPerBlock + threadIdx.x * 4;
+    int deg[4];
+    int hubs = 0, chunks = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const long long r = r0 + i;
+        deg[i] = 0;
+        if (r < m) deg[i] = row_ptr[r + 1] - row_ptr[r];
+        if (deg[i] > kHubThreshold) { ++hubs; chunks += hub_chunks(deg[i]); }
+    }
+    int tot;
+    int slot = block_hubs[blockIdx.x] + block_exclusive_scan(hubs, sh, &tot);
+    int chunk = block_chunks[blockIdx.x] + block_exclusive_scan(chunks, sh, &tot);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (deg[i] > kHubThreshold) {
+            const int nc = hub_chunks(deg[i]);
+            // a hub past the capacity of the buffers keeps slot -1: its consumer sums it in place
+            const bool fits = slot < hub_cap && chunk + nc <= chunk_cap;
+            row_slot[r0 + i] = fits ? slot : -1;
+            if (fits) {
+                hub_row[slot] = (int)(r0 + i);
+                hub_chunk0[slot] = chunk;
+                for (int j = 0; j < nc; ++j) chunk_hub[chunk + j] = slot;
+            }
+            ++slot;
+            chunk += nc;
+        }
+    }
+}
+
+template <int VEC> struct HV;
+template <> struct HV<4> {
+    using T = float4;
+    static __device__ __forceinline__ T zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+    static __device__ __forceinline__ T load(const float* p) { return *reinterpret_cast<const float4*>(p); }
+    static __device__ __forceinline__ void store(float* p, T v) { *reinterpret_cast<float4*>(p) = v; }
+    static __device__ __forceinline__ void fma(T& a, float s, T x) { a.x += s * x.x; a.y += s * x.y; a.z += s * x.z; a.w += s * x.w; }
+    static __device__ __forceinline__ T add(T a, T b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+};
+template <> struct HV<1> {
+    using T = float;
+    static __device__ __forceinline__ T zero() { return 0.f; }
+    static __device__ __forceinline__ T load(const float* p) { return *p; }
+    static __device__ __forceinline__ void store(float* p, T v) { *p = v; }
+    static __device__ __forceinline__ void fma(T& a, float s, T x) { a += s * x; }
+    static __device__ __forceinline__ T add(T a, T b) { return a + b; }
+};
+
+// One wavefront per chunk.  The wavefront is split into 64 / G lane groups; group g takes the
+// chunk's entries g, g + ngroups, ... eight at a time, a lane owns the column slabs
+// (sub + it * G) * VEC.  The groups' sums are added through LDS in group order.
+template <int VEC, int ITERS>
+__global__ __launch_bounds__(kBlock) void hub_partial_kernel(
+    const int* __restrict__ counts, int chunk_cap, int n, const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
+    const float* __restrict__ val, const float* __restrict__ B, int ldb, int logG,
+    const int* __restrict__ hub_row, const int* __restrict__ hub_chunk0, const int* __restrict__ chunk_hub,
+    float* __restrict__ part, int ldp)
+{
+    using V = HV<VEC>;
+    __shared__ float red[kWavesPerBlock][kWave * VEC * ITERS];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int G = 1 << logG, sub = lane & (G - 1), grp = lane >> logG, ngroups = kWave >> logG;
+    const int width = G * VEC * ITERS;
+    const int nchunks = min(counts[1], chunk_cap);
+    for (int c = blockIdx.x * kWavesPerBlock + wave; c < nchunks; c += gridDim.x * kWavesPerBlock) {
+        const int slot = chunk_hub[c];
+        const int row = hub_row[slot];
+        const int rb = row_ptr[row], re = row_ptr[row + 1];
+        const int cb = rb + (c - hub_chunk0[slot]) * kHubChunk;
+        const int ce = min(cb + kHubChunk, re);
+        typename V::T acc[ITERS];
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) acc[it] = V::zero();
+        int t = cb + grp;
+        for (; t + 7 * ngroups < ce; t += 8 * ngroups) {
+            int c8[8];
+            float v8[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) { c8[u] = col_idx[t + u * ngroups]; v8[u] = val[t + u * ngroups]; }
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int col0 = (sub + it * G) * VEC;
+                if (col0 < n) {
+                    typename V::T x[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) x[u] = V::load(B + (size_t)c8[u] * ldb + col0);
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) V::fma(acc[it], v8[u], x[u]);
+                }
+            }
+        }
+        for (; t < ce; t += ngroups) {
+            const int c0 = col_idx[t];
+            const float v0 = val[t];
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int col0 = (sub + it * G) * VEC;
+                if (col0 < n) V::fma(acc[it], v0, V::load(B + (size_t)c0 * ldb + col0));
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) V::store(red[wave] + grp * width + (sub + it * G) * VEC, acc[it]);
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        if (grp == 0) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int col0 = (sub + it * G) * VEC;
+                if (col0 < n) {
+                    typename V::T s = V::zero();
+                    for (int g = 0; g < ngroups; ++g) s = V::add(s, V::load(red[wave] + g * width + col0));
+                    V::store(part + (size_t)c * ldp + col0, s);
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    }
+}
+
+// One lane group per hub: agg[slot] = sum over its chunks, in chunk order.
+template <int VEC, int ITERS>
+__global__ __launch_bounds__(kBlock) void hub_combine_kernel(
+    const int* __restrict__ counts, int hub_cap, int chunk_cap, int n, const int* __restrict__ row_ptr, int logG,
+    const int* __restrict__ hub_row, const int* __restrict__ hub_chunk0,
+    const float* __restrict__ part, int ldp, float* __restrict__ agg)
+{
+    using V = HV<VEC>;
+    const int G = 1 << logG, sub = threadIdx.x & (G - 1), grp = threadIdx.x >> logG, ngroups = kBlock >> logG;
+    const int nhubs = min(counts[0], hub_cap);
+    for (int slot = blockIdx.x * ngroups + grp; slot < nhubs; slot += gridDim.x * ngroups) {
+        const int row = hub_row[slot];
+        const int deg = row_ptr[row + 1] - row_ptr[row];
+        const int c0 = hub_chunk0[slot], nc = hub_chunks(deg);
+        if (c0 + nc > chunk_cap) continue;       // never written by fill (slot -1 for the consumer)
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int col0 = (sub + it * G) * VEC;
+            if (col0 < n) {
+                typename V::T s = V::zero();
+                for (int j = 0; j < nc; ++j) s = V::add(s, V::load(part + (size_t)(c0 + j) * ldp + col0));
+                V::store(agg + (size_t)slot * ldp + col0, s);
+            }
+        }
+    }
+}
+
+inline int ilog2_ceil_(int x)
+{
+    int l = 0;
+    while ((1 << l) < x) ++l;
+    return l;
+}
+
+inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+template <int VEC, int ITERS>
+void launch_partial_combine(hipStream_t s, const int* counts, int hub_cap, int chunk_cap, int n, const int* row_ptr,
+                            const int* col_idx, const float* val, const float* B, int ldb, int logG, const int* hub_row,
+                            const int* hub_chunk0, const int* chunk_hub, float* part, int ldp, float* agg)
+{
+    const unsigned grid = kNumCU * 8;
+    hipLaunchKernelGGL((hub_partial_kernel<VEC, ITERS>), dim3(grid), dim3(kBlock), 0, s, counts, chunk_cap, n, row_ptr,
+                       col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp);
+    hipLaunchKernelGGL((hub_combine_kernel<VEC, ITERS>), dim3(kNumCU * 2), dim3(kBlock), 0, s, counts, hub_cap, chunk_cap, n,
+                       row_ptr, logG, hub_row, hub_chunk0, part, ldp, agg);
+}
+
+}  // namespace
+
+// Sums the hubs of A (rows longer than kHubThreshold) times B[:, 0..n) into plan->agg.
+// n <= 1024.  The buffers live in the stream's plan scratch and stay valid until the next
+// hub_prepass on the same stream.
+int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
+                const float* B, int ldb, hipStream_t s, HubPlan* plan)
+{
+    plan->row_slot = nullptr;
+    plan->agg = nullptr;
+    plan->ld = 0;
+    if (m < kHubMinRows || nnz <= kHubThreshold || n > kWave * 16) return GNNHIP_OK;
+    const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && aligned16(B);
+    const int vec = vec4 ? 4 : 1;
+    const int units = (n + vec - 1) / vec;
+    const int logG = ilog2_ceil_(units < kWave ? units : kWave);
+    const int G = 1 << logG;
+    const int iters = (units + G - 1) / G;                   // 1..4
+    const int ldp = (int)round_up((size_t)n, 4);
+
+    const int nb = (m + kRowsPerBlock - 1) / kRowsPerBlock;
+    const long long hub_cap_ll = nnz / (kHubThreshold + 1) + 1;
+    const long long chunk_cap_ll = nnz / kHubChunk + hub_cap_ll + 1;
+    const int hub_cap = (int)(hub_cap_ll < m ? hub_cap_ll : m);
+    const int chunk_cap = (int)chunk_cap_ll;
+
+    size_t off = 0;
+    auto carve = [&](size_t bytes) { const size_t o = off; off = round_up(off + bytes, 256); return o; };
+    const size_t o_counts = carve(sizeof(int) * 4);
+    const size_t o_bh = carve(sizeof(int) * nb), o_bc = carve(sizeof(int) * nb);
+    const size_t o_slot = carve(sizeof(int) * (size_t)m);
+    const size_t o_hrow = carve(sizeof(int) * (size_t)hub_cap), o_hc0 = carve(sizeof(int) * (size_t)hub_cap);
+    const size_t o_chub = carve(sizeof(int) * (size_t)chunk_cap);
+    const size_t o_part = carve(sizeof(float) * (size_t)chunk_cap * ldp);
+    const size_t o_agg = carve(sizeof(float) * (size_t)hub_cap * ldp);
+    void* base = nullptr;
+    if (int rc = stream_scratch_slot(s, 1, off, &base)) return rc;
+    char* b = static_cast<char*>(base);
+    int* counts = reinterpret_cast<int*>(b + o_counts);
+    int* bh = reinterpret_cast<int*>(b + o_bh);
+    int* bc = reinterpret_cast<int*>(b + o_bc);
+    int* row_slot = reinterpret_cast<int*>(b + o_slot);
+    int* hub_row = reinterpret_cast<int*>(b + o_hrow);
+    int* hub_chunk0 = reinterpret_cast<int*>(b + o_hc0);
+    int* chunk_hub = reinterpret_cast<int*>(b + o_chub);
+    float* part = reinterpret_cast<float*>(b + o_part);
+    float* agg = reinterpret_cast<float*>(b + o_agg);
+
+    hipLaunchKernelGGL(hub_count_kernel, dim3(nb), dim3(kBlock), 0, s, m, row_ptr, bh, bc);
+    hipLaunchKernelGGL(hub_scan_kernel, dim3(1), dim3(kScanBlock), 0, s, nb, bh, bc, counts);
+    hipLaunchKernelGGL(hub_fill_kernel, dim3(nb), dim3(kBlock), 0, s, m, row_ptr, bh, bc, hub_cap, chunk_cap, row_slot,
+                       hub_row, hub_chunk0, chunk_hub);
+    if (vec4) {
+        if (iters <= 1) launch_partial_combine<4, 1>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
+        else if (iters == 2) launch_partial_combine<4, 2>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
+        else launch_partial_combine<4, 4>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
+    } else {
+        if (iters <= 1) launch_partial_combine<1, 1>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
+        else if (iters == 2) launch_partial_combine<1, 2>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
+        else launch_partial_combine<1, 4>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
+    }
+    GNNHIP_LAUNCH_CHECK("hub_prepass");
+    plan->row_slot = row_slot;
+    plan->agg = agg;
+    plan->ld = ldp;
+    return GNNHIP_OK;
+}
+
+}  // namespace gnnhip

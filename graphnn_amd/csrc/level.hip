@@ -167,13 +167,15 @@ __global__ __launch_bounds__(kBlock) void s2v_input_kernel(
 //      columns of block jb are permuted so that the lane ends up owning row t,
 //      columns (C/4) q .. (C/4) q + C/4 - 1: contiguous float4s for the epilogue;
 //   3. epilogue: + bias + msg, ReLU, float4 stores.
-constexpr int kWaveLongRow = 256;   // entries; longer rows are gathered by all groups of the wavefront together
+constexpr int kWaveLongRow = kHubThreshold;   // entries; longer rows come from the hub pre-pass or, without one,
+                                              // are gathered by all groups of the wavefront together
 
 template <int C>
 __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
     int N, const int* __restrict__ row_ptr, const int* __restrict__ col_idx, const float* __restrict__ val,
     const float* __restrict__ h_in, const float* __restrict__ W, const float* __restrict__ msg,
-    const float* __restrict__ bias, float* __restrict__ h_out)
+    const float* __restrict__ bias, float* __restrict__ h_out,
+    const int* __restrict__ hub_slot, const float* __restrict__ hub_agg, int hub_ld)
 {
     constexpr int G = C / 4;             // lanes per gathered row
     constexpr int RPR = kWave / G;       // rows gathered per round
@@ -212,13 +214,19 @@ __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
         int st[ROUNDS], en[ROUNDS], c0[ROUNDS];
         float v0[ROUNDS];
         bool is_long[ROUNDS];
+        int hub[ROUNDS];
 #pragma unroll
         for (int rd = 0; rd < ROUNDS; ++rd) {
             const int lr = rd * RPR + grp;
             st[rd] = __shfl(rp, lr, kWave);
             en[rd] = __shfl(rp, lr + 1, kWave);
             is_long[rd] = (en[rd] - st[rd] > kWaveLongRow);
-            if (is_long[rd]) en[rd] = st[rd];
+            hub[rd] = -1;
+            if (is_long[rd]) {
+                en[rd] = st[rd];
+                if (hub_slot) hub[rd] = hub_slot[row0 + lr];      // the pre-pass has summed this row
+                if (hub[rd] >= 0) is_long[rd] = false;
+            }
             c0[rd] = 0;
             v0[rd] = 0.f;
             if (st[rd] + tx < en[rd]) { c0[rd] = col_idx[st[rd] + tx]; v0[rd] = val[st[rd] + tx]; }
@@ -272,6 +280,7 @@ __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
                         if (j + u < cnt) f4_fma(acc, vj[u], xx[u]);
                 }
             }
+            if (hub[rd] >= 0) acc = *reinterpret_cast<const float4*>(hub_agg + (size_t)hub[rd] * hub_ld + tx * 4);
             *reinterpret_cast<float4*>(tile + lr * LDT + tx * 4) = acc;
         }
 
@@ -464,14 +473,14 @@ int launch_input(int N, int K, const float* X, const float* Wn2l, float* msg, fl
 
 template <int C>
 int launch_level(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-                 const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
+                 const float* W, const float* msg, const float* bias, float* h_out, const HubPlan& hubs, hipStream_t s)
 {
     constexpr int kWavesPerBlock = kBlock / kWave;
     const long long ntiles = ((long long)N + 15) / 16;
     long long blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > kNumCU * 8) blocks = kNumCU * 8;          // persistent beyond this
     hipLaunchKernelGGL((s2v_level_kernel<C>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
-                       N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out);
+                       N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs.row_slot, hubs.agg, hubs.ld);
     GNNHIP_LAUNCH_CHECK("s2v_level");
     return GNNHIP_OK;
 }
@@ -511,15 +520,18 @@ int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float
     return GNNHIP_EUNSUPPORTED;
 }
 
-int level_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
+int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
                    const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
 {
     if (!(aligned16(h_in) && aligned16(W) && aligned16(h_out) && (!msg || aligned16(msg)) && (!bias || aligned16(bias))))
         return GNNHIP_EUNSUPPORTED;
+    HubPlan hubs{nullptr, nullptr, 0};
+    if (C == 16 || C == 32 || C == 64)
+        if (int rc = hub_prepass(N, C, nnz, row_ptr, col_idx, val, h_in, C, s, &hubs)) return rc;
     switch (C) {
-    case 16: return launch_level<16>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
-    case 32: return launch_level<32>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
-    case 64: return launch_level<64>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    case 16: return launch_level<16>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
+    case 32: return launch_level<32>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
+    case 64: return launch_level<64>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
     case 128:
     case 256: return level_wide_dispatch(N, C, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
     }

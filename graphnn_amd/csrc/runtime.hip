@@ -30,7 +30,7 @@ struct Runtime {
     size_t bytes_in_use = 0;
     size_t bytes_parked = 0;
     size_t n_driver_allocs = 0;
-    std::unordered_map<hipStream_t, std::pair<void*, size_t>> scratch;   // per-stream library scratch
+    std::map<std::pair<hipStream_t, int>, std::pair<void*, size_t>> scratch;   // library scratch per (stream, slot)
 };
 
 Runtime& rt()
@@ -111,12 +111,15 @@ int pool_release(void* p)
     return GNNHIP_OK;
 }
 
-int stream_scratch(hipStream_t s, size_t bytes, void** p)
+int stream_scratch(hipStream_t s, size_t bytes, void** p) { return stream_scratch_slot(s, 0, bytes, p); }
+
+int stream_scratch_slot(hipStream_t s, int which, size_t bytes, void** p)
 {
     Runtime& r = rt();
     std::lock_guard<std::mutex> lock(r.mu);
     if (!r.ready) return set_error(GNNHIP_ENOTINIT, "gnnhip_init has not been called");
-    auto& slot = r.scratch[s];
+    if (which < 0 || which >= kScratchSlots) return set_error(GNNHIP_EINVAL, "bad scratch slot %d", which);
+    auto& slot = r.scratch[std::make_pair(s, which)];
     if (slot.second < bytes) {
         size_t want = (bytes + 65535) / 65536 * 65536;
         if (want < slot.second * 2) want = slot.second * 2;

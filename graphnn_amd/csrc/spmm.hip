@@ -11,9 +11,12 @@
 // HBM/L2 requests in flight per lane.  Accumulation is in registers in CSR order
 // (deterministic, no atomics) and each output element is written exactly once.
 //
-// Rows longer than kLongRow entries are set aside inside the workgroup and then
-// processed by all of its 256 lanes together, which split the row's entries and
-// combine the partial sums in LDS in a fixed order (still deterministic).
+// Long rows: on matrices of at least kHubMinRows rows a pre-pass (hub.hip) sums the
+// rows longer than kHubThreshold entries with the work cut by entries, and the row's
+// group here only scales and stores that sum.  Elsewhere rows longer than kLongRow
+// entries are set aside inside the workgroup and then processed by all of its 256
+// lanes together, which split the row's entries and combine the partial sums in LDS
+// in a fixed order (still deterministic).
 //
 // Bound: HBM.  Algorithmic bytes per launch: 4(m+1) + 8 nnz + 4 k n + 4 m n.
 #include "gnnhip_internal.h"
@@ -63,7 +66,7 @@ template <int VEC, int ITERS>
 __global__ __launch_bounds__(kBlock) void spmm_rowgroup_kernel(
     int m, int n, float alpha, const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
     const float* __restrict__ val, const float* __restrict__ B, int ldb, float beta, float* C, int ldc,
-    int logG, int long_row)
+    int logG, int long_row, const int* __restrict__ hub_slot, const float* __restrict__ hub_agg, int hub_ld)
 {
     using V = Vec<VEC>;
     __shared__ int lr_list[kBlock];
@@ -82,6 +85,10 @@ __global__ __launch_bounds__(kBlock) void spmm_rowgroup_kernel(
 
     int start = 0, end = 0;
     if (row < m) { start = row_ptr[row]; end = row_ptr[row + 1]; }
+    // a row summed by the hub pre-pass only scales and stores
+    int hslot = -1;
+    if (hub_slot && end - start > kHubThreshold) hslot = hub_slot[row];
+    if (hslot >= 0) end = start;
     const bool deferred = (end - start > long_row);
     if (deferred) {
         if (sub == 0) lr_list[atomicAdd(&lr_count, 1)] = (int)row;
@@ -127,6 +134,7 @@ __global__ __launch_bounds__(kBlock) void spmm_rowgroup_kernel(
         for (int it = 0; it < ITERS; ++it) {
             const int col0 = (sub + it * G) * VEC;
             if (col0 < n) {
+                if (hslot >= 0) acc[it] = V::axpby(V::zero(), alpha, V::load(hub_agg + (size_t)hslot * hub_ld + col0));
                 float* dst = C + (size_t)row * ldc + col0;
                 if (beta == 0.f) V::store(dst, acc[it]);
                 else V::store(dst, V::axpby(acc[it], beta, V::load(dst)));
@@ -201,12 +209,12 @@ inline int ilog2_ceil(int x)
 
 template <int VEC, int ITERS>
 int launch_slab(int m, int n, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                const float* B, int ldb, float beta, float* C, int ldc, int logG, hipStream_t s)
+                const float* B, int ldb, float beta, float* C, int ldc, int logG, const HubPlan& hubs, hipStream_t s)
 {
     const int groups_per_block = kBlock >> logG;
     const unsigned blocks = ceil_div_u((size_t)m, (size_t)groups_per_block);
     hipLaunchKernelGGL((spmm_rowgroup_kernel<VEC, ITERS>), dim3(blocks), dim3(kBlock), 0, s,
-                       m, n, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, logG, kLongRow);
+                       m, n, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, logG, kLongRow, hubs.row_slot, hubs.agg, hubs.ld);
     GNNHIP_LAUNCH_CHECK("spmm_rowgroup");
     return GNNHIP_OK;
 }
@@ -214,7 +222,7 @@ int launch_slab(int m, int n, float alpha, const int* row_ptr, const int* col_id
 }  // namespace
 
 // Shared with the fused forward: C = alpha*A*B + beta*C on stream s.
-int spmm_dispatch(int m, int n, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+int spmm_dispatch(int m, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s)
 {
     const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && aligned16(B) && aligned16(C);
@@ -230,14 +238,16 @@ int spmm_dispatch(int m, int n, float alpha, const int* row_ptr, const int* col_
         const float* Bs = B + col0;
         float* Cs = C + col0;
         int rc;
+        HubPlan hubs;
+        if ((rc = hub_prepass(m, w, nnz, row_ptr, col_idx, val, Bs, ldb, s, &hubs))) return rc;
         if (vec4) {
-            if (iters <= 1) rc = launch_slab<4, 1>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, s);
-            else if (iters == 2) rc = launch_slab<4, 2>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, s);
-            else rc = launch_slab<4, 4>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, s);
+            if (iters <= 1) rc = launch_slab<4, 1>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
+            else if (iters == 2) rc = launch_slab<4, 2>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
+            else rc = launch_slab<4, 4>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
         } else {
-            if (iters <= 1) rc = launch_slab<1, 1>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, s);
-            else if (iters == 2) rc = launch_slab<1, 2>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, s);
-            else rc = launch_slab<1, 4>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, s);
+            if (iters <= 1) rc = launch_slab<1, 1>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
+            else if (iters == 2) rc = launch_slab<1, 2>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
+            else rc = launch_slab<1, 4>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
         }
         if (rc) return rc;
     }
@@ -248,15 +258,15 @@ int spmm_dispatch(int m, int n, float alpha, const int* row_ptr, const int* col_
 
 using namespace gnnhip;
 
-extern "C" int gnnhip_spmm_csr_f32(int m, int k, int n, float alpha, const int* row_ptr, const int* col_idx,
+extern "C" int gnnhip_spmm_csr_f32(int m, int k, int n, int nnz, float alpha, const int* row_ptr, const int* col_idx,
                                    const float* val, const float* B, int ldb, float beta, float* C, int ldc,
                                    void* stream)
 {
-    GNNHIP_REQUIRE(m >= 0 && k >= 0 && n >= 0, "negative dimension in spmm (m=%d k=%d n=%d)", m, k, n);
+    GNNHIP_REQUIRE(m >= 0 && k >= 0 && n >= 0 && nnz >= 0, "negative dimension in spmm (m=%d k=%d n=%d nnz=%d)", m, k, n, nnz);
     if (m == 0 || n == 0) return GNNHIP_OK;
     GNNHIP_REQUIRE(row_ptr && C, "null row_ptr or output in spmm");
     GNNHIP_REQUIRE(ldb >= n && ldc >= n, "leading dimension smaller than n in spmm (ldb=%d ldc=%d n=%d)", ldb, ldc, n);
     GNNHIP_REQUIRE(k == 0 || B, "null dense operand in spmm");   // col_idx / val may be null when A has no entries
     if (int rc = require_ready()) return rc;
-    return spmm_dispatch(m, n, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, as_stream(stream));
+    return spmm_dispatch(m, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, as_stream(stream));
 }

@@ -158,7 +158,7 @@ inline void FactorGraph::BuildFusedSteps(Plan& plan)
                                    A->value.rows() == H->value.rows(),
                                    "fused level: operand shapes do not chain");
                             O->value.Reshape(H->value.shape.dims);
-                            GNN_HIP(gnnhip_s2v_level_f32((int)H->value.rows(), (int)H->value.cols(), A->value.data->row_ptr,
+                            GNN_HIP(gnnhip_s2v_level_f32((int)H->value.rows(), (int)H->value.cols(), A->value.data->nnz, A->value.data->row_ptr,
                                                          A->value.data->col_idx, A->value.data->val, H->value.data->ptr,
                                                          W->value.data->ptr, M->value.data->ptr, nullptr,
                                                          O->value.data->ptr, GpuHandle::Stream()));

@@ -71,7 +71,7 @@ inline void TensorTemplate<GPU, DENSE, float>::MM(SpTensor<GPU, float>& a, DTens
     GetDims(a.rows(), a.cols(), transA, b.rows(), b.cols(), transB, m, n, k);
     Reshape({m, n});
     if (transA == Trans::N) {
-        GNN_HIP(gnnhip_spmm_csr_f32((int)m, (int)k, (int)n, alpha, a.data->row_ptr, a.data->col_idx, a.data->val,
+        GNN_HIP(gnnhip_spmm_csr_f32((int)m, (int)k, (int)n, a.data->nnz, alpha, a.data->row_ptr, a.data->col_idx, a.data->val,
                                     b.data->ptr, (int)b.cols(), beta, data->ptr, (int)n, GpuHandle::Stream()));
     } else {
         GNN_HIP(gnnhip_spmm_csr_t_f32((int)a.rows(), (int)a.cols(), (int)n, alpha, a.data->row_ptr, a.data->col_idx,

@@ -68,7 +68,7 @@ def spmm(row_ptr, col_idx, val, B, m, alpha=1.0, beta=0.0, out=None):
         out = torch.empty((m, n), dtype=torch.float32, device=B.device)
     elif tuple(out.shape) != (m, n):
         raise ValueError("out has the wrong shape")
-    check(_lib().gnnhip_spmm_csr_f32(m, k, n, alpha, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"),
+    check(_lib().gnnhip_spmm_csr_f32(m, k, n, int(col_idx.numel()), alpha, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"),
                                      _f32(val, "val"), _f32(B, "B"), n, beta, _f32(out, "out"), n, _stream()))
     return out
 
@@ -112,7 +112,7 @@ def s2v_level(row_ptr, col_idx, val, h_in, W, msg=None, bias=None, out=None):
         raise ValueError("bias must have C entries")
     if out is None:
         out = torch.empty_like(h_in)
-    check(_lib().gnnhip_s2v_level_f32(N, C, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"), _f32(val, "val"),
+    check(_lib().gnnhip_s2v_level_f32(N, C, int(col_idx.numel()), _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"), _f32(val, "val"),
                                       _f32(h_in, "h_in"), _f32(W, "W"), _f32(msg, "msg"), _f32(bias, "bias"),
                                       _f32(out, "out"), _stream()))
     return out
@@ -169,7 +169,7 @@ def s2v_forward(a_csr, s_csr, X, W_n2l, W_conv, W_h1, W_h2, L, bufs=None):
     if bufs is None:
         bufs = ForwardBuffers(N, B, C, H, Q, X.device)
     check(_lib().gnnhip_s2v_forward_f32(
-        N, B, K, C, H, Q, L,
+        N, B, K, C, H, Q, L, int(a_csr[1].numel()),
         _i32(a_csr[0], "a_row_ptr"), _i32(a_csr[1], "a_col_idx"), _f32(a_csr[2], "a_val"),
         _i32(s_csr[0], "s_row_ptr"), _i32(s_csr[1], "s_col_idx"), _f32(s_csr[2], "s_val"),
         _f32(X, "X"), _f32(W_n2l, "W_n2l"), _f32(W_conv, "W_conv"), _f32(W_h1, "W_h1"), _f32(W_h2, "W_h2"),

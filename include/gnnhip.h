@@ -72,8 +72,11 @@ int gnnhip_stream_sync(void* stream);
 
 /* ---- C[m,n] = alpha * A * B + beta * C, A CSR [m,k], B dense [k,n].
  *      DTensor<GPU>::MM(SpTensor, DTensor, Trans::N, Trans::N) + CSRMMKernel
- *      (src/tensor/gpu_dense_tensor.cu:227-239,257-270).  beta == 0 overwrites C. */
-int gnnhip_spmm_csr_f32(int m, int k, int n, float alpha, const int* row_ptr, const int* col_idx,
+ *      (src/tensor/gpu_dense_tensor.cu:227-239,257-270).  beta == 0 overwrites C.
+ *      nnz is the host-side entry count of A (SparseData::nnz, include/tensor/t_data.h:123-165);
+ *      it sizes the buffers of the balanced pass over high-degree rows.  A value smaller than
+ *      row_ptr[m] is safe (rows that do not fit are summed in place), a larger one wastes memory. */
+int gnnhip_spmm_csr_f32(int m, int k, int n, int nnz, float alpha, const int* row_ptr, const int* col_idx,
                         const float* val, const float* B, int ldb, float beta, float* C, int ldc,
                         void* stream);
 
@@ -89,8 +92,9 @@ int gnnhip_gemm_f32(int transA, int transB, int m, int n, int k, float alpha, co
  *      (examples/graph_classification/src/kernel_mean_field.cpp:35-42,
  *       src/nn/matmul.cpp:13-33, src/nn/elewise_add.cpp:13-33, src/nn/relu.cu:9-13;
  *       bias as in src/nn/fully_connected.cpp:28-39).  msg and bias may be NULL.
- *      A is [N,N] CSR, h_in/h_out/msg are [N,C], W is [C,C]; h_out must not alias h_in. */
-int gnnhip_s2v_level_f32(int N, int C, const int* row_ptr, const int* col_idx, const float* val,
+ *      A is [N,N] CSR with nnz entries (see gnnhip_spmm_csr_f32), h_in/h_out/msg are [N,C], W is [C,C];
+ *      h_out must not alias h_in. */
+int gnnhip_s2v_level_f32(int N, int C, int nnz, const int* row_ptr, const int* col_idx, const float* val,
                          const float* h_in, const float* W, const float* msg, const float* bias,
                          float* h_out, void* stream);
 
@@ -113,10 +117,10 @@ int gnnhip_s2v_readout_f32(int B, int N, int C, int H, int Q,
 
 /* ---- whole forward = input + L levels + readout, device-resident.
  *      h_a / h_b are [N,C] ping-pong buffers; *which_h (host int, may be NULL)
- *      receives 0 if the final embedding is in h_a, 1 if in h_b.
+ *      receives 0 if the final embedding is in h_a, 1 if in h_b.  a_nnz: entries of A.
  *      Op sequence of examples/graph_classification/src/kernel_mean_field.cpp:31-49 scheduled by
  *      FactorGraph::SequentialForward (src/nn/factor_graph.cpp:75-144). */
-int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L,
+int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L, int a_nnz,
                            const int* a_row_ptr, const int* a_col_idx, const float* a_val,
                            const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                            const float* X, const float* W_n2l, const float* W_conv,

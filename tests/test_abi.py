@@ -46,21 +46,21 @@ def test_argument_validation_needs_no_gpu():
     lib = binding.load_library()
     f = ctypes.c_float
     # negative sizes, bad op codes, null pointers: rejected before any device work
-    assert lib.gnnhip_spmm_csr_f32(-1, 1, 1, f(1), None, None, None, None, 1, f(0), None, 1, None) == -1
+    assert lib.gnnhip_spmm_csr_f32(-1, 1, 1, 0, f(1), None, None, None, None, 1, f(0), None, 1, None) == -1
     assert b"negative" in lib.gnnhip_last_error()
-    assert lib.gnnhip_spmm_csr_f32(4, 4, 8, f(1), None, None, None, None, 8, f(0), None, 8, None) == -1
+    assert lib.gnnhip_spmm_csr_f32(4, 4, 8, 0, f(1), None, None, None, None, 8, f(0), None, 8, None) == -1
     assert lib.gnnhip_gemm_f32(2, 0, 1, 1, 1, f(1), None, 1, None, 1, f(0), None, 1, None) == -1
     assert lib.gnnhip_unary_f32(99, None, 10, f(0), f(0), None) == -1
     assert lib.gnnhip_reduce_f32(9, None, 10, None, None) == -1
     assert lib.gnnhip_row_argmax_f32(None, 3, 0, None, None) == -1
-    assert lib.gnnhip_s2v_forward_f32(0, 1, 1, 1, 1, 1, 1, *([None] * 19), None, None) == -1
+    assert lib.gnnhip_s2v_forward_f32(0, 1, 1, 1, 1, 1, 1, 0, *([None] * 19), None, None) == -1
     x = np.zeros(8, np.float32)
     p = x.ctypes.data_as(ctypes.c_void_p)
-    assert lib.gnnhip_s2v_level_f32(2, 4, p, p, p, p, p, None, None, p, None) == -1      # in place is refused
+    assert lib.gnnhip_s2v_level_f32(2, 4, 0, p, p, p, p, p, None, None, p, None) == -1      # in place is refused
     assert b"in place" in lib.gnnhip_last_error()
     # empty work is a successful no-op
     assert lib.gnnhip_unary_f32(6, None, 0, f(0), f(0), None) == 0
-    assert lib.gnnhip_spmm_csr_f32(0, 0, 0, f(1), None, None, None, None, 0, f(0), None, 0, None) == 0
+    assert lib.gnnhip_spmm_csr_f32(0, 0, 0, 0, f(1), None, None, None, None, 0, f(0), None, 0, None) == 0
     assert lib.gnnhip_memset0(None, 0, None) == 0
 
 
