@@ -777,3 +777,20 @@ def test_rmat_forward_with_jagged_softmax(gpu, oracle):
     got_soft = _n(soft_d).reshape(nsub, 1024)
     assert np.allclose(got_soft.sum(axis=1), 1.0, atol=1e-5)
     assert np.abs(got_soft - soft.reshape(nsub, 1024)).max() < 1e-4
+
+
+def test_level_dense_graph_two_launch_route(gpu, oracle):
+    """a large graph with 14 entries per row takes the SpMM-then-contraction route; same result as the
+    fused kernel's on the same inputs and as the reference path"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(77)
+    N, C, deg = 40000, 32, 14
+    rp, ci, v = synth.erdos_renyi_csr(77, N, N * deg)
+    v = (rng.random(v.size) * 0.2).astype(np.float32)
+    h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
+    W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
+    msg = rng.standard_normal((N, C)).astype(np.float32)
+    bias = rng.standard_normal(C).astype(np.float32)
+    want = oracle.level(rp, ci, v, h_in, W, msg, bias)
+    got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu), _t(bias, gpu)))
+    assert max_rel(got, want) < PARITY_TOL
