@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the structure2vec mean-field forward on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-spmm]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-spmm] [--extra]
 
 A step is one forward (input + L levels + readout) over one synthetic batch of
 configuration 2 (256 graphs, hidden 64, 4 levels) with every input already
@@ -107,6 +107,109 @@ def time_spmm_cfg3(dev, reps=20, warmup=3):
     return float(ms.mean()), float(ms.min()), spmm_algorithmic_bytes(n, n, nnz, d), (n, nnz, d)
 
 
+FP32_MFMA_PEAK_TFLOPS = 157.3   # MI355X dense FP32 matrix, published
+
+
+def _event_ms(fn, reps, warmup=2):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def time_level_cfg4(dev):
+    """One fused level at configuration 4 (10,000 graphs, hidden 256): the FP32 matrix-core kernel."""
+    import torch
+    from graphnn_amd import batching, ops, synth
+    batch, w, cfg = synth.make_config(4)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    t = lambda arr: torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
+    a_d = tuple(map(t, a))
+    msg, h0 = ops.s2v_input(t(batch.one_hot()), t(w.W_n2l))
+    Wc = t(w.W_conv)
+    out = torch.empty_like(h0)
+    ms = _event_ms(lambda: ops.s2v_level(*a_d, h0, Wc, msg, out=out), 20)
+    N, E, C = batch.num_nodes, int(a[1].size), cfg["C"]
+    flops = 2.0 * N * C * C + 2.0 * E * C + 2.0 * N * C
+    return {"workload": "configuration 4: one level, %d nodes, %d entries, hidden %d" % (N, E, C),
+            "kernel": "s2v_level_wide_kernel<256,8>", "avg_ms": ms,
+            "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS},
+            "algorithmic_GBps": level_algorithmic_bytes(N, E, C) / (ms * 1e-3) / 1e9}
+
+
+def time_cfg5(dev, scale=22):
+    """Configuration 5: R-MAT (a=.57, b=c=.19), 16 entries per row, generated on the device with the
+    same recursive-quadrant rule as synth.rmat_csr (torch's generator, so not the parity inputs);
+    level, SpMM, jagged softmax over segments of 1024 node scores, sum-pool."""
+    import torch
+    from graphnn_amd import ops
+    N, E, C, K = 1 << scale, 16 << scale, 64, 16
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    rows = torch.zeros(E, dtype=torch.int64, device=dev)
+    cols = torch.zeros(E, dtype=torch.int64, device=dev)
+    for _ in range(scale):
+        u = torch.rand(E, device=dev, generator=g)
+        rows = (rows << 1) | (u >= 0.76).long()
+        cols = (cols << 1) | (((u >= 0.57) & (u < 0.76)) | (u >= 0.95)).long()
+    key, _ = torch.sort(rows * N + cols)
+    del rows, cols
+    r = key // N
+    ci = (key - r * N).int()
+    cnt = torch.bincount(r, minlength=N)
+    del key, r
+    rp = torch.zeros(N + 1, dtype=torch.int32, device=dev)
+    rp[1:] = torch.cumsum(cnt, 0).int()
+    val = torch.ones(E, dtype=torch.float32, device=dev)
+    lab = torch.randint(0, K, (N,), device=dev, generator=g)
+    X = torch.zeros((N, K), dtype=torch.float32, device=dev)
+    X[torch.arange(N, device=dev), lab] = 1.0
+    Wn = torch.randn((K, C), device=dev, generator=g) * 0.1
+    Wc = torch.randn((C, C), device=dev, generator=g) * 0.1
+    wsc = torch.randn((C, 1), device=dev, generator=g) * 0.1
+    B = N // 1024
+    s_rp = (torch.arange(B + 1, device=dev) * 1024).int()
+    s_ci = torch.arange(N, device=dev).int()
+    s_v = torch.ones(N, device=dev)
+    lens = torch.full((B,), 1024, dtype=torch.int32, device=dev)
+    msg, h0 = ops.s2v_input(X, Wn)
+    h1 = torch.empty_like(h0)
+    agg = torch.empty_like(h0)
+    score = torch.empty((N, 1), dtype=torch.float32, device=dev)
+    pool = torch.empty((B, C), dtype=torch.float32, device=dev)
+    res = {"workload": "configuration 5: R-MAT scale %d, %d rows, %d entries, max row %d, %d rows over 256 entries, hidden %d"
+                       % (scale, N, E, int(cnt.max()), int((cnt > 256).sum()), C)}
+    ms = _event_ms(lambda: ops.s2v_level(rp, ci, val, h0, Wc, msg, out=h1), 5)
+    res["level"] = {"avg_ms": ms, "algorithmic_GBps": level_algorithmic_bytes(N, E, C) / (ms * 1e-3) / 1e9,
+                    "gather_GBps": (4.0 * E * C + 12.0 * N * C + 8.0 * E) / (ms * 1e-3) / 1e9}
+    ms = _event_ms(lambda: ops.spmm(rp, ci, val, h0, N, out=agg), 5)
+    res["spmm"] = {"avg_ms": ms, "algorithmic_GBps": spmm_algorithmic_bytes(N, N, E, C) / (ms * 1e-3) / 1e9,
+                   "gather_GBps": (4.0 * E * C + 4.0 * N * C + 8.0 * E) / (ms * 1e-3) / 1e9}
+    ms = _event_ms(lambda: ops.gemm(h1, wsc, out=score), 5)
+    res["score"] = {"avg_ms": ms}
+    ms = _event_ms(lambda: ops.jagged_softmax(score, lens), 5)
+    res["jagged_softmax"] = {"avg_ms": ms, "GBps": 8.0 * N / (ms * 1e-3) / 1e9}
+    ms = _event_ms(lambda: ops.spmm(s_rp, s_ci, s_v, h1, B, out=pool), 5)
+    res["sum_pool"] = {"avg_ms": ms, "GBps": (4.0 * N * C + 8.0 * N) / (ms * 1e-3) / 1e9}
+    # size-independent checks at full size: A * ones = row lengths exactly; each softmax segment sums to 1
+    ones = torch.ones((N, 4), device=dev, dtype=torch.float32)
+    deg = ops.spmm(rp, ci, val, ones, N)
+    assert bool((deg[:, 0] == cnt.float()).all()), "row-length check failed on the R-MAT matrix"
+    sc = torch.randn((N, 1), device=dev, generator=g)
+    ops.jagged_softmax(sc, lens)
+    seg = sc.view(B, 1024).double().sum(dim=1)
+    assert float((seg - 1.0).abs().max()) < 1e-5, "jagged softmax segments do not sum to 1"
+    return res
+
+
 def cpu_baseline(host, budget_s=12.0):
     """The CPU restatement of the reference path on the same batch, timed on this host."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
@@ -133,6 +236,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-spmm", action="store_true", help="skip the configuration-3 SpMM roofline leg")
+    ap.add_argument("--extra", action="store_true",
+                    help="also time the configuration-4 level (FP32 matrix cores) and the configuration-5 "
+                         "kernels (R-MAT, 4M rows) and report them under \"extra\"")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one element-wise copy kernel of known size (1 GiB read, 1 GiB written) "
                          "so hardware counters collected over this run can be scaled")
@@ -199,6 +305,9 @@ def main():
         ops.relu(src, dst)              # map1_kernel<FReLU>: reads 4n bytes, writes 4n bytes
         torch.cuda.synchronize()
         out["calibration"] = {"kernel": "map1_kernel<FReLU>", "bytes_read": 4 * n, "bytes_written": 4 * n}
+
+    if args.extra:
+        out["extra"] = {"cfg4_level": time_level_cfg4(dev), "cfg5": time_cfg5(dev)}
 
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline(host)
     print(json.dumps(out))
