@@ -210,6 +210,30 @@ def time_cfg5(dev, scale=22):
     return res
 
 
+def end_to_end_host_layer(host, reps=300):
+    """The same batch through the C++ host layer as graphnn's example drives it: host batch build,
+    CSR construction, host-to-device copies, FactorGraph::FeedForward (TEST phase), loss/accuracy read back.
+    Runs the prebuilt driver graphnn_amd/host/build/host_forward_bench as a child process."""
+    import subprocess
+    import tempfile
+    from graphnn_amd import synth
+    exe = os.path.join(ROOT, "graphnn_amd", "host", "build", "host_forward_bench")
+    if not os.path.exists(exe):
+        return {"skipped": "graphnn_amd/host/build/host_forward_bench is not built"}
+    cfg = host["cfg"]
+    with tempfile.TemporaryDirectory() as d:
+        synth.write_graphnn_txt(host["batch"], os.path.join(d, "graphs.txt"))
+        r = subprocess.run([exe, d] + [str(cfg[k]) for k in ("K", "C", "H", "Q", "L")] + [str(reps)],
+                           capture_output=True, text=True, timeout=300)
+    if r.returncode != 0:
+        return {"skipped": "host_forward_bench failed: " + (r.stderr or r.stdout)[-300:]}
+    res = json.loads(r.stdout.strip().splitlines()[-1])
+    res["graphs_per_s"] = res["graphs"] / (res["us_per_batch"] * 1e-6)
+    res["what"] = ("GetBatch-style host batch build + CSR build + H2D + FactorGraph::FeedForward (fused plan) + "
+                   "loss/accuracy read-back, per batch; PCIe-inclusive, never `value`")
+    return res
+
+
 def cpu_baseline(host, budget_s=12.0):
     """The CPU restatement of the reference path on the same batch, timed on this host."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
@@ -305,6 +329,8 @@ def main():
         ops.relu(src, dst)              # map1_kernel<FReLU>: reads 4n bytes, writes 4n bytes
         torch.cuda.synchronize()
         out["calibration"] = {"kernel": "map1_kernel<FReLU>", "bytes_read": 4 * n, "bytes_written": 4 * n}
+
+    out["end_to_end"] = end_to_end_host_layer(host)
 
     if args.extra:
         out["extra"] = {"cfg4_level": time_level_cfg4(dev), "cfg5": time_cfg5(dev)}
