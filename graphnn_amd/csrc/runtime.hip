@@ -11,6 +11,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <map>
+#include <string.h>
 #include <mutex>
 #include <unordered_map>
 
@@ -19,6 +20,19 @@ namespace gnnhip {
 namespace {
 
 thread_local char g_err[512] = "";
+
+// Pinned staging for host-to-device copies: two halves used in turn.  A copy is placed in the current
+// half and sent from there asynchronously, so the caller's buffer is free as soon as the call returns
+// and nothing waits for the device.  A half is reused only after the event recorded behind its last
+// copy has completed.
+constexpr size_t kStagingHalf = 2u << 20;
+struct Staging {
+    char* base = nullptr;              // 2 * kStagingHalf bytes from hipHostMalloc
+    hipEvent_t done[2] = {nullptr, nullptr};
+    bool pending[2] = {false, false};
+    int half = 0;
+    size_t used = 0;
+};
 
 struct Runtime {
     std::mutex mu;
@@ -31,6 +45,7 @@ struct Runtime {
     size_t bytes_parked = 0;
     size_t n_driver_allocs = 0;
     std::map<std::pair<hipStream_t, int>, std::pair<void*, size_t>> scratch;   // library scratch per (stream, slot)
+    std::map<hipStream_t, struct Staging> staging;  // pinned upload buffers per stream
 };
 
 Runtime& rt()
@@ -180,6 +195,11 @@ int gnnhip_shutdown(void)
     for (auto& kv : r.all) (void)hipFree(kv.first);
     for (auto& kv : r.scratch) (void)hipFree(kv.second.first);
     r.scratch.clear();
+    for (auto& kv : r.staging) {
+        if (kv.second.base) (void)hipHostFree(kv.second.base);
+        for (hipEvent_t e : kv.second.done) if (e) (void)hipEventDestroy(e);
+    }
+    r.staging.clear();
     r.all.clear();
     r.live.clear();
     r.parked.clear();
@@ -239,8 +259,43 @@ int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void
     if (int rc = require_ready()) return rc;
     // Ordered after earlier work on the stream; returns once the host buffer has been read, so the
     // caller may overwrite it at once (the reference's blocking cudaMemcpy gives callers the same promise).
-    GNNHIP_HIP(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, as_stream(stream)));
-    GNNHIP_HIP(hipStreamSynchronize(as_stream(stream)));
+    hipStream_t s = as_stream(stream);
+    if (bytes <= kStagingHalf) {
+        Runtime& r = rt();
+        std::lock_guard<std::mutex> lock(r.mu);
+        Staging& st = r.staging[s];
+        if (!st.base) {
+            void* q = nullptr;
+            if (hipHostMalloc(&q, 2 * kStagingHalf, hipHostMallocDefault) == hipSuccess && q) {
+                st.base = static_cast<char*>(q);
+                GNNHIP_HIP(hipEventCreateWithFlags(&st.done[0], hipEventDisableTiming));
+                GNNHIP_HIP(hipEventCreateWithFlags(&st.done[1], hipEventDisableTiming));
+            } else {
+                (void)hipGetLastError();
+            }
+        }
+        if (st.base) {
+            const size_t need = (bytes + 255) & ~(size_t)255;
+            if (st.used + need > kStagingHalf) {
+                // close this half behind its last copy and move to the other one once the device has left it
+                GNNHIP_HIP(hipEventRecord(st.done[st.half], s));
+                st.pending[st.half] = true;
+                st.half ^= 1;
+                st.used = 0;
+                if (st.pending[st.half]) {
+                    GNNHIP_HIP(hipEventSynchronize(st.done[st.half]));
+                    st.pending[st.half] = false;
+                }
+            }
+            char* slot = st.base + (size_t)st.half * kStagingHalf + st.used;
+            memcpy(slot, src_host, bytes);
+            st.used += need;
+            GNNHIP_HIP(hipMemcpyAsync(dst_device, slot, bytes, hipMemcpyHostToDevice, s));
+            return GNNHIP_OK;
+        }
+    }
+    GNNHIP_HIP(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, s));
+    GNNHIP_HIP(hipStreamSynchronize(s));
     return GNNHIP_OK;
 }
 
