@@ -34,6 +34,8 @@ namespace gnnhip {
 // spmm.hip
 int spmm_dispatch(int m, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s);
+// input_wide.hip
+int input_wide_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s);
 // level_wide.hip
 int level_wide_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
                         const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s);
@@ -544,6 +546,8 @@ int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float
     case 16: return small ? launch_input<16, 1>(N, K, X, Wn2l, msg, h0, s) : launch_input<16, 4>(N, K, X, Wn2l, msg, h0, s);
     case 32: return small ? launch_input<32, 1>(N, K, X, Wn2l, msg, h0, s) : launch_input<32, 4>(N, K, X, Wn2l, msg, h0, s);
     case 64: return small ? launch_input<64, 1>(N, K, X, Wn2l, msg, h0, s) : launch_input<64, 4>(N, K, X, Wn2l, msg, h0, s);
+    case 128:
+    case 256: return input_wide_dispatch(N, K, C, X, Wn2l, msg, h0, s);
     }
     return GNNHIP_EUNSUPPORTED;
 }

@@ -319,8 +319,8 @@ def _small_problem(seed, B, K, C, H, Q, lo=3, hi=40):
     return batch, w, a, s
 
 
-@pytest.mark.parametrize("C", [16, 32, 64, 48, 128])
-@pytest.mark.parametrize("K", [7, 38, 64])
+@pytest.mark.parametrize("C", [16, 32, 64, 48, 128, 256])
+@pytest.mark.parametrize("K", [7, 17, 38, 64, 70])
 def test_input_stage(gpu, oracle, C, K):
     from graphnn_amd import ops
     batch, w, a, s = _small_problem(10 + C + K, 9, K, C, 8, 2)
