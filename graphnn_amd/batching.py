@@ -37,3 +37,37 @@ def node2node_csr(num_nodes, edge_x, edge_y, average=False):
 def subgraph_csr(num_subgraph, subg_id, node_idx, average=False):
     """S [B,N]: row g lists the nodes added to subgraph g in AddNode order."""
     return _stable_csr(subg_id, node_idx, num_subgraph, average)
+
+
+def edge2node_csr(num_nodes, edge_y, average=False):
+    """[N,E]: row i lists the indices of the edges that end in node i, in edge order
+    (Edge2NodeMsgPass, src/nn/msg_pass.cpp:72-94)."""
+    edge_y = np.asarray(edge_y)
+    return _stable_csr(edge_y, np.arange(edge_y.size, dtype=np.int32), num_nodes, average)
+
+
+def node2edge_csr(edge_x):
+    """[E,N]: row e holds the tail node of edge e (Node2EdgeMsgPass, src/nn/msg_pass.cpp:98-116)."""
+    edge_x = np.asarray(edge_x, dtype=np.int32)
+    E = edge_x.size
+    return np.arange(E + 1, dtype=np.int32), edge_x.copy(), np.ones(E, dtype=np.float32)
+
+
+def edge2edge_csr(num_nodes, edge_x, edge_y):
+    """[E,E]: row e = (x -> y) lists the edges that end in x and do not start in y, in edge order
+    (Edge2EdgeMsgPass, src/nn/msg_pass.cpp:120-152)."""
+    edge_x = np.asarray(edge_x, dtype=np.int64)
+    edge_y = np.asarray(edge_y, dtype=np.int64)
+    E = edge_x.size
+    in_rp, in_edges, _ = edge2node_csr(num_nodes, edge_y)
+    lens = (in_rp[1:] - in_rp[:-1])[edge_x]                      # candidates per row: in-degree of the tail
+    row_of = np.repeat(np.arange(E, dtype=np.int64), lens)
+    start = np.repeat(in_rp[:-1][edge_x].astype(np.int64), lens)
+    within = np.arange(row_of.size, dtype=np.int64) - np.repeat(np.cumsum(lens) - lens, lens)
+    cand = in_edges[start + within].astype(np.int64)
+    keep = edge_x[cand] != edge_y[row_of]
+    counts = np.bincount(row_of[keep], minlength=E)
+    row_ptr = np.zeros(E + 1, dtype=np.int32)
+    np.cumsum(counts, out=row_ptr[1:])
+    col = cand[keep].astype(np.int32)
+    return row_ptr, col, np.ones(col.size, dtype=np.float32)

@@ -1,8 +1,11 @@
 // Message-passing operands: CSR matrices built from the batch GraphStruct on the host and
 // copied to the device (interface of graphnn's include/nn/msg_pass.h; construction rules of
-// src/nn/msg_pass.cpp:46-67 and :156-177).  Row i of the node-to-node matrix lists the
-// in-neighbours of node i in edge order; row g of the subgraph matrix lists the nodes of
-// graph g in AddNode order; values are 1, or 1/row length when `average` is set.
+// src/nn/msg_pass.cpp:46-177).  Row i of the node-to-node matrix lists the in-neighbours of
+// node i in edge order; row g of the subgraph matrix lists the nodes of graph g in AddNode
+// order; values are 1, or 1/row length when `average` is set.  The edge-based operands of the
+// loopy-BP embedding: edge-to-node [N,E] (edges that end in node i), node-to-edge [E,N] (the
+// tail of edge e) and edge-to-edge [E,E] (edges that end in the tail of edge e, except its own
+// reverse).
 #ifndef MSG_PASS_H
 #define MSG_PASS_H
 
@@ -70,6 +73,99 @@ protected:
         }
         rp[graph->num_nodes] = nnz;
         ASSERT(nnz == (int)graph->num_edges, "edge count does not match the in-edge lists");
+    }
+};
+
+template<typename mode, typename Dtype>
+class Edge2NodeMsgPass : public IMsgPass<mode, Dtype>
+{
+public:
+    static std::string StrType() { return "Edge2NodeMsgPass"; }
+    using OutType = std::shared_ptr< SpTensorVar<mode, Dtype> >;
+    OutType CreateOutVar() { return std::make_shared< SpTensorVar<mode, Dtype> >(fmt::sprintf("%s:out_0", this->name)); }
+    Edge2NodeMsgPass(std::string _name, bool _average = false) : IMsgPass<mode, Dtype>(_name, _average) {}
+
+protected:
+    virtual void InitCPUWeight(GraphStruct* graph) override
+    {
+        auto& w = this->cpu_weight;
+        w.Reshape({graph->num_nodes, graph->num_edges});
+        w.ResizeSp((int)graph->num_edges, (int)graph->num_nodes + 1);
+        int* rp = w.data->row_ptr;
+        int* ci = w.data->col_idx;
+        Dtype* va = w.data->val;
+        int nnz = 0;
+        for (unsigned i = 0; i < graph->num_nodes; ++i) {
+            rp[i] = nnz;
+            const auto& in = graph->in_edges->head[i];
+            const Dtype weight = this->average ? (Dtype)(1.0 / (double)in.size()) : (Dtype)1.0;
+            for (size_t j = 0; j < in.size(); ++j) { ci[nnz] = in[j].first; va[nnz] = weight; ++nnz; }
+        }
+        rp[graph->num_nodes] = nnz;
+        ASSERT(nnz == (int)graph->num_edges, "edge count does not match the in-edge lists");
+    }
+};
+
+template<typename mode, typename Dtype>
+class Node2EdgeMsgPass : public IMsgPass<mode, Dtype>
+{
+public:
+    static std::string StrType() { return "Node2EdgeMsgPass"; }
+    using OutType = std::shared_ptr< SpTensorVar<mode, Dtype> >;
+    OutType CreateOutVar() { return std::make_shared< SpTensorVar<mode, Dtype> >(fmt::sprintf("%s:out_0", this->name)); }
+    Node2EdgeMsgPass(std::string _name, bool _average = false) : IMsgPass<mode, Dtype>(_name, _average) {}
+
+protected:
+    virtual void InitCPUWeight(GraphStruct* graph) override
+    {
+        auto& w = this->cpu_weight;
+        const int E = (int)graph->num_edges;
+        w.Reshape({graph->num_edges, graph->num_nodes});
+        w.ResizeSp(E, E + 1);
+        for (int e = 0; e < E; ++e) {
+            w.data->row_ptr[e] = e;
+            w.data->col_idx[e] = graph->edge_list[e].first;
+            w.data->val[e] = (Dtype)1.0;
+        }
+        w.data->row_ptr[E] = E;
+    }
+};
+
+template<typename mode, typename Dtype>
+class Edge2EdgeMsgPass : public IMsgPass<mode, Dtype>
+{
+public:
+    static std::string StrType() { return "Edge2EdgeMsgPass"; }
+    using OutType = std::shared_ptr< SpTensorVar<mode, Dtype> >;
+    OutType CreateOutVar() { return std::make_shared< SpTensorVar<mode, Dtype> >(fmt::sprintf("%s:out_0", this->name)); }
+    Edge2EdgeMsgPass(std::string _name, bool _average = false) : IMsgPass<mode, Dtype>(_name, _average) {}
+
+protected:
+    virtual void InitCPUWeight(GraphStruct* graph) override
+    {
+        auto& w = this->cpu_weight;
+        const int E = (int)graph->num_edges;
+        // entries: for every edge (x -> y), the edges that end in x and do not start in y
+        size_t cnt = 0;
+        for (int e = 0; e < E; ++e) {
+            const int from = graph->edge_list[e].first, to = graph->edge_list[e].second;
+            for (const auto& in : graph->in_edges->head[from]) cnt += (in.second != to);
+        }
+        w.Reshape({graph->num_edges, graph->num_edges});
+        w.ResizeSp((int)cnt, E + 1);
+        int nnz = 0;
+        for (int e = 0; e < E; ++e) {
+            w.data->row_ptr[e] = nnz;
+            const int from = graph->edge_list[e].first, to = graph->edge_list[e].second;
+            for (const auto& in : graph->in_edges->head[from]) {
+                if (in.second == to) continue;           // the same edge in the other direction
+                w.data->col_idx[nnz] = in.first;
+                w.data->val[nnz] = (Dtype)1.0;
+                ++nnz;
+            }
+        }
+        w.data->row_ptr[E] = nnz;
+        ASSERT(nnz == (int)cnt, "edge-to-edge entry count changed between the two passes");
     }
 };
 

@@ -5,7 +5,9 @@
 //   host_csr_check <in.bin> <out.bin> <average 0|1>
 //   in.bin : int32 B, N, E, then subg_id[N], node_idx[N], edge_x[E], edge_y[E]
 //   out.bin: int32 a_row_ptr[N+1], a_col[E], fp32 a_val[E], int32 s_row_ptr[B+1], s_col[N], fp32 s_val[N],
-//            int32 flags {contiguous_subgraphs, max_subgraph_nodes}
+//            int32 flags {contiguous_subgraphs, max_subgraph_nodes},
+//            then the edge-based operands: e2n row_ptr[N+1], col[E], val[E]; n2e row_ptr[E+1], col[E], val[E];
+//            int32 nnz of e2e, e2e row_ptr[E+1], col[nnz], val[nnz]
 #include <cstdio>
 #include <vector>
 #include "tensor/tensor_all.h"
@@ -58,6 +60,25 @@ int main(int argc, char** argv)
     auto* sf = dynamic_cast<SubgraphMsgPass<CPU, float>*>(fg.factor_list[1].get());
     int flags[2] = {sf->contiguous_subgraphs ? 1 : 0, sf->max_subgraph_nodes};
     fwrite(flags, 4, 2, o);
+
+    // ---- edge-based operands of the loopy-BP embedding
+    FactorGraph fg2;
+    auto gv2 = add_const<GraphVar>(fg2, "graph", true);
+    auto e2n = af< Edge2NodeMsgPass<CPU, float> >(fg2, {gv2}, average);
+    auto n2e = af< Node2EdgeMsgPass<CPU, float> >(fg2, {gv2});
+    auto e2e = af< Edge2EdgeMsgPass<CPU, float> >(fg2, {gv2});
+    fg2.FeedForward({e2n, n2e, e2e}, feed, Phase::TEST);
+    auto& d1 = *e2n->value.data;
+    auto& d2 = *n2e->value.data;
+    auto& d3 = *e2e->value.data;
+    ASSERT(d1.nnz == E && d1.len_ptr == N + 1 && d2.nnz == E && d2.len_ptr == E + 1 && d3.len_ptr == E + 1, "unexpected CSR sizes");
+    ASSERT(e2n->value.rows() == (size_t)N && e2n->value.cols() == (size_t)E && n2e->value.rows() == (size_t)E &&
+           n2e->value.cols() == (size_t)N && e2e->value.rows() == (size_t)E && e2e->value.cols() == (size_t)E, "unexpected shapes");
+    fwrite(d1.row_ptr, 4, N + 1, o); fwrite(d1.col_idx, 4, E, o); fwrite(d1.val, 4, E, o);
+    fwrite(d2.row_ptr, 4, E + 1, o); fwrite(d2.col_idx, 4, E, o); fwrite(d2.val, 4, E, o);
+    int nnz3 = d3.nnz;
+    fwrite(&nnz3, 4, 1, o);
+    fwrite(d3.row_ptr, 4, E + 1, o); fwrite(d3.col_idx, 4, nnz3, o); fwrite(d3.val, 4, nnz3, o);
     fclose(o);
     return 0;
 }

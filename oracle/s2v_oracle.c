@@ -74,6 +74,65 @@ void orc_csr_node2node(int num_nodes, int num_edges, const int* edge_x, const in
     free(fill);
 }
 
+/* Edge2NodeMsgPass::InitCPUWeight (src/nn/msg_pass.cpp:72-94): matrix [N, E]; row i lists the
+ * indices of the edges that end in node i, in insertion order; value 1 or 1/indeg. */
+void orc_csr_edge2node(int num_nodes, int num_edges, const int* edge_y, int average,
+                       int* row_ptr, int* col_idx, float* val)
+{
+    int* fill = (int*)calloc((size_t)num_nodes + 1, sizeof(int));
+    for (int e = 0; e < num_edges; ++e) fill[edge_y[e] + 1]++;
+    row_ptr[0] = 0;
+    for (int i = 0; i < num_nodes; ++i) row_ptr[i + 1] = row_ptr[i] + fill[i + 1];
+    for (int i = 0; i < num_nodes; ++i) fill[i] = row_ptr[i];
+    for (int e = 0; e < num_edges; ++e) {
+        int y = edge_y[e];
+        int deg = row_ptr[y + 1] - row_ptr[y];
+        int pos = fill[y]++;
+        col_idx[pos] = e;
+        val[pos] = average ? (float)(1.0 / (double)deg) : 1.0f;
+    }
+    free(fill);
+}
+
+/* Node2EdgeMsgPass::InitCPUWeight (src/nn/msg_pass.cpp:98-116): matrix [E, N]; row e holds one
+ * entry, the tail node of edge e, value 1. */
+void orc_csr_node2edge(int num_edges, const int* edge_x, int* row_ptr, int* col_idx, float* val)
+{
+    for (int e = 0; e < num_edges; ++e) { row_ptr[e] = e; col_idx[e] = edge_x[e]; val[e] = 1.0f; }
+    row_ptr[num_edges] = num_edges;
+}
+
+/* Edge2EdgeMsgPass::InitCPUWeight (src/nn/msg_pass.cpp:120-152): matrix [E, E]; row e = (x -> y)
+ * lists, in insertion order, the edges (u -> x) that end in x, except those that start in y
+ * (the same edge in the other direction); value 1.  Returns the number of entries; col_idx and
+ * val may be NULL to count only (row_ptr is always written). */
+int orc_csr_edge2edge(int num_nodes, int num_edges, const int* edge_x, const int* edge_y,
+                      int* row_ptr, int* col_idx, float* val)
+{
+    /* in-edge lists of every node in insertion order: a stable grouping of edge indices by head */
+    int* start = (int*)calloc((size_t)num_nodes + 1, sizeof(int));
+    int* fill = (int*)calloc((size_t)num_nodes + 1, sizeof(int));
+    int* in_edge = (int*)malloc(sizeof(int) * (size_t)(num_edges > 0 ? num_edges : 1));
+    for (int e = 0; e < num_edges; ++e) start[edge_y[e] + 1]++;
+    for (int i = 0; i < num_nodes; ++i) start[i + 1] += start[i];
+    for (int i = 0; i < num_nodes; ++i) fill[i] = start[i];
+    for (int e = 0; e < num_edges; ++e) in_edge[fill[edge_y[e]]++] = e;
+    int nnz = 0;
+    for (int e = 0; e < num_edges; ++e) {
+        row_ptr[e] = nnz;
+        const int from = edge_x[e], to = edge_y[e];
+        for (int t = start[from]; t < start[from + 1]; ++t) {
+            const int other = in_edge[t];
+            if (edge_x[other] == to) continue;
+            if (col_idx) { col_idx[nnz] = other; val[nnz] = 1.0f; }
+            ++nnz;
+        }
+    }
+    row_ptr[num_edges] = nnz;
+    free(start); free(fill); free(in_edge);
+    return nnz;
+}
+
 /* GraphStruct::AddNode(subg, n) appends n to subgraph[subg]
  * (src/util/graph_struct.cpp:72-75); SubgraphMsgPass::InitCPUWeight lists each
  * subgraph's nodes in insertion order (src/nn/msg_pass.cpp:156-177). */

@@ -20,6 +20,11 @@ extern "C" {
 /* ---- batch graph -> CSR (integer work, bit-exact contract) ---- */
 void orc_csr_node2node(int num_nodes, int num_edges, const int* edge_x, const int* edge_y,
                        int average, int* row_ptr, int* col_idx, float* val);
+void orc_csr_edge2node(int num_nodes, int num_edges, const int* edge_y, int average,
+                       int* row_ptr, int* col_idx, float* val);
+void orc_csr_node2edge(int num_edges, const int* edge_x, int* row_ptr, int* col_idx, float* val);
+int orc_csr_edge2edge(int num_nodes, int num_edges, const int* edge_x, const int* edge_y,
+                      int* row_ptr, int* col_idx, float* val);
 void orc_csr_subgraph(int num_subgraph, int num_nodes, const int* subg_id, const int* node_idx,
                       int average, int* row_ptr, int* col_idx, float* val);
 

@@ -44,6 +44,30 @@ class Oracle:
         self.lib.orc_csr_node2node(N, E, _ptr(ex), _ptr(ey), int(average), _ptr(rp), _ptr(ci), _ptr(v))
         return rp, ci, v
 
+    def csr_edge2node(self, N, ey, average=False):
+        ey = np.ascontiguousarray(ey, np.int32)
+        E = ey.size
+        rp, ci, v = np.zeros(N + 1, np.int32), np.zeros(E, np.int32), np.zeros(E, np.float32)
+        self.lib.orc_csr_edge2node(N, E, _ptr(ey), int(average), _ptr(rp), _ptr(ci), _ptr(v))
+        return rp, ci, v
+
+    def csr_node2edge(self, ex):
+        ex = np.ascontiguousarray(ex, np.int32)
+        E = ex.size
+        rp, ci, v = np.zeros(E + 1, np.int32), np.zeros(E, np.int32), np.zeros(E, np.float32)
+        self.lib.orc_csr_node2edge(E, _ptr(ex), _ptr(rp), _ptr(ci), _ptr(v))
+        return rp, ci, v
+
+    def csr_edge2edge(self, N, ex, ey):
+        ex, ey = np.ascontiguousarray(ex, np.int32), np.ascontiguousarray(ey, np.int32)
+        E = ex.size
+        rp = np.zeros(E + 1, np.int32)
+        self.lib.orc_csr_edge2edge.restype = ctypes.c_int
+        nnz = self.lib.orc_csr_edge2edge(N, E, _ptr(ex), _ptr(ey), _ptr(rp), None, None)
+        ci, v = np.zeros(max(nnz, 1), np.int32), np.zeros(max(nnz, 1), np.float32)
+        self.lib.orc_csr_edge2edge(N, E, _ptr(ex), _ptr(ey), _ptr(rp), _ptr(ci), _ptr(v))
+        return rp, ci[:nnz], v[:nnz]
+
     def csr_subgraph(self, B, sid, nid, average=False):
         N = len(sid)
         sid = np.ascontiguousarray(sid, dtype=np.int32)

@@ -794,3 +794,33 @@ def test_level_dense_graph_two_launch_route(gpu, oracle):
     want = oracle.level(rp, ci, v, h_in, W, msg, bias)
     got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu), _t(bias, gpu)))
     assert max_rel(got, want) < PARITY_TOL
+
+
+def test_edge_embedding_step_with_edge_based_operands(gpu, oracle):
+    """one loopy-BP style update on edge states, built from the edge-to-edge, node-to-edge and edge-to-node
+    operands (src/nn/msg_pass.cpp:72-152) and the same SpMM / GEMM / element-wise entry points"""
+    from graphnn_amd import ops
+    batch = synth.molecule_batch(321, 40, 6, 2)
+    N, E, K, C = batch.num_nodes, batch.num_edges, 6, 32
+    rng = np.random.default_rng(4)
+    n2e = batching.node2edge_csr(batch.edge_x)
+    e2e = batching.edge2edge_csr(N, batch.edge_x, batch.edge_y)
+    e2n = batching.edge2node_csr(N, batch.edge_y, average=True)
+    X = batch.one_hot()
+    W1 = (rng.standard_normal((K, C)) * 0.3).astype(np.float32)
+    W2 = (rng.standard_normal((C, C)) * 0.3).astype(np.float32)
+    m0 = np.maximum(rng.standard_normal((E, C)), 0).astype(np.float32)
+    # reference path
+    inp = oracle.spmm(*n2e, oracle.gemm(X, W1), E)
+    m1 = np.maximum(oracle.gemm(oracle.spmm(*e2e, m0, E), W2) + inp, 0)
+    node = oracle.spmm(*e2n, m1, N)
+    # device
+    inp_d = ops.spmm(*_csr_t(n2e, gpu), ops.gemm(_t(X, gpu), _t(W1, gpu)), E)
+    lin_d = ops.gemm(ops.spmm(*_csr_t(e2e, gpu), _t(m0, gpu), E), _t(W2, gpu))
+    m1_d = ops.relu(ops.add(lin_d, inp_d))
+    node_d = ops.spmm(*_csr_t(e2n, gpu), m1_d, N)
+    assert max_rel(_n(m1_d), m1) < PARITY_TOL
+    assert max_rel(_n(node_d), node) < PARITY_TOL
+    # the same update through the fused level entry: A = edge-to-edge, h = edge states, msg = inp
+    fused = ops.s2v_level(*_csr_t(e2e, gpu), _t(m0, gpu), _t(W2, gpu), inp_d)
+    assert max_rel(_n(fused), m1) < PARITY_TOL

@@ -31,7 +31,12 @@ def _run(tmp_path, B, N, E, sid, nid, ex, ey, average):
 
     res = (take(N + 1, np.int32), take(E, np.int32), take(E, np.float32),
            take(B + 1, np.int32), take(N, np.int32), take(N, np.float32), take(2, np.int32))
+    e2n = (take(N + 1, np.int32), take(E, np.int32), take(E, np.float32))
+    n2e = (take(E + 1, np.int32), take(E, np.int32), take(E, np.float32))
+    nnz = int(take(1, np.int32)[0])
+    e2e = (take(E + 1, np.int32), take(nnz, np.int32), take(nnz, np.float32))
     assert pos == len(raw)
+    _run.edge_operands = (e2n, n2e, e2e)
     return res
 
 
@@ -48,6 +53,13 @@ def test_cpp_builders_match_oracle_random(oracle, tmp_path, average):
     for got, want in zip((srp, sci, sv), oracle.csr_subgraph(B, sid, nid, average)):
         assert np.array_equal(got, want)
     assert flags[0] == 0 and flags[1] == np.bincount(sid, minlength=B).max()
+    e2n, n2e, e2e = _run.edge_operands
+    for got, want in zip(e2n, oracle.csr_edge2node(N, ey, average)):
+        assert np.array_equal(got, want)
+    for got, want in zip(n2e, oracle.csr_node2edge(ex)):
+        assert np.array_equal(got, want)
+    for got, want in zip(e2e, oracle.csr_edge2edge(N, ex, ey)):
+        assert np.array_equal(got, want)
 
 
 def test_cpp_builders_on_a_getbatch_style_batch(oracle, tmp_path):
@@ -59,3 +71,9 @@ def test_cpp_builders_on_a_getbatch_style_batch(oracle, tmp_path):
         assert np.array_equal(got, want)
     assert np.array_equal(sci, np.arange(b.num_nodes)) and np.all(sv == 1)
     assert flags[0] == 1 and flags[1] == b.graph_sizes.max()       # contiguous layout recognised
+    e2n, n2e, e2e = _run.edge_operands
+    for got, want in zip(e2e, oracle.csr_edge2edge(b.num_nodes, b.edge_x, b.edge_y)):
+        assert np.array_equal(got, want)
+    # undirected graphs stored in both directions: every edge sees the other in-edges of its tail
+    indeg = np.bincount(b.edge_y, minlength=b.num_nodes)
+    assert e2e[1].size == int((indeg * (indeg - 1)).sum())

@@ -403,3 +403,48 @@ def test_forward_against_float64_dense_model(oracle):
     A = _dense_of(*a, batch.num_nodes, batch.num_nodes)
     want_lvl = np.maximum(A @ got["h"][0].astype(np.float64) @ w.W_conv.astype(np.float64) + bias + got["msg"], 0)
     assert max_rel(lvl, want_lvl) < 1e-4
+
+
+def test_edge_based_operands_against_dense_definitions(oracle):
+    """Edge2Node / Node2Edge / Edge2Edge (src/nn/msg_pass.cpp:72-152) against matrices written straight
+    from their definitions, and the numpy builders against the oracle"""
+    from graphnn_amd import batching
+    rng = np.random.default_rng(12)
+    N, E = 23, 90
+    ex = rng.integers(0, N, E); ey = rng.integers(0, N, E)
+    ex[5], ey[5] = ey[4], ex[4]                                   # a reverse pair
+    ex[7], ey[7] = 3, 3                                           # a self-loop
+    def dense(rp, ci, v, rows, cols):
+        M = np.zeros((rows, cols))
+        for r in range(rows):
+            for t in range(rp[r], rp[r + 1]):
+                M[r, ci[t]] += v[t]
+        return M
+    for average in (False, True):
+        rp, ci, v = oracle.csr_edge2node(N, ey, average)
+        want = np.zeros((N, E))
+        for e in range(E):
+            want[ey[e], e] = 1.0
+        if average:
+            want = want / np.maximum(want.sum(axis=1, keepdims=True), 1)
+        assert np.allclose(dense(rp, ci, v, N, E), want, atol=1e-7)
+        assert all(np.all(np.diff(ci[rp[r]:rp[r + 1]]) > 0) for r in range(N))       # insertion order = ascending e
+        for got, w2 in zip(batching.edge2node_csr(N, ey, average), (rp, ci, v)):
+            assert np.array_equal(got, w2)
+    rp, ci, v = oracle.csr_node2edge(ex)
+    assert np.array_equal(rp, np.arange(E + 1)) and np.array_equal(ci, ex) and np.all(v == 1)
+    for got, w2 in zip(batching.node2edge_csr(ex), (rp, ci, v)):
+        assert np.array_equal(got, w2)
+    rp, ci, v = oracle.csr_edge2edge(N, ex, ey)
+    want = np.zeros((E, E))
+    for e in range(E):
+        for o in range(E):
+            if ey[o] == ex[e] and ex[o] != ey[e]:
+                want[e, o] = 1.0
+    assert np.array_equal(dense(rp, ci, v, E, E), want)
+    assert all(np.all(np.diff(ci[rp[r]:rp[r + 1]]) > 0) for r in range(E))
+    for got, w2 in zip(batching.edge2edge_csr(N, ex, ey), (rp, ci, v)):
+        assert np.array_equal(got, w2)
+    # no edges at all
+    rp, ci, v = oracle.csr_edge2edge(4, np.zeros(0, np.int32), np.zeros(0, np.int32))
+    assert np.array_equal(rp, [0]) and ci.size == 0
