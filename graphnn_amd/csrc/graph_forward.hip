@@ -111,10 +111,19 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     const int gi = tid / G, tx = tid % G;
 
     GNNHIP_PHASE_MARK(0);
+    // The position of the first graph (node range, then entry range) is asked for ahead of the weight
+    // loads, so the two dependent trips to memory run under them instead of after them.
+    int next_node0 = 0, next_n = 0;
+    if ((int)blockIdx.x < B) { next_node0 = s_row_ptr[blockIdx.x]; next_n = s_row_ptr[blockIdx.x + 1] - next_node0; }
     // this wavefront's 16 columns of W^T, level contraction: wreg[s] = Wc[KS q + s][16 jb + t]
     float wreg[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) wreg[s] = Wc[(size_t)(KS * q + s) * C + 16 * jb + t];
+    int next_e0 = 0, next_e1 = 0;
+    if ((int)blockIdx.x < B && next_n >= 0 && next_n <= n16max) {
+        next_e0 = a_row_ptr[next_node0];
+        next_e1 = a_row_ptr[next_node0 + next_n];
+    }
 
     if (ro_staged) {
         // coalesced reads; the transposed layout lets a wavefront read one output's weights contiguously
@@ -124,8 +133,9 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     // (the staged copies become visible to all lanes at the first barrier of the graph loop)
     GNNHIP_PHASE_MARK(1);
     for (int g = blockIdx.x; g < B; g += gridDim.x) {
-        const int node0 = s_row_ptr[g];
-        const int n = s_row_ptr[g + 1] - node0;
+        const bool first = (g == (int)blockIdx.x);
+        const int node0 = first ? next_node0 : s_row_ptr[g];
+        const int n = first ? next_n : s_row_ptr[g + 1] - node0;
         if (n > n16max || n < 0) {                      // host promised max_graph_nodes; refuse instead of overrunning LDS
             if (tid == 0 && status) atomicOr(status, 1);
             continue;
@@ -140,8 +150,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
             wx[s] = Wn2l[(size_t)min(k, K - 1) * C + 16 * jb + t];
             if (k >= K) wx[s] = 0.f;
         }
-        const int e0 = a_row_ptr[node0];
-        const int ne = a_row_ptr[node0 + n] - e0;
+        const int e0 = first ? next_e0 : a_row_ptr[node0];
+        const int ne = (first ? next_e1 : a_row_ptr[node0 + n]) - e0;
         const bool staged = (ne <= ecap);
 
         // ---- stage the graph's CSR slice (L uses) and check the block-diagonal promise
