@@ -9,7 +9,8 @@
  *
  * How each function is pinned (tests/test_oracle_*.py):
  *   CSR builders      brute force vs dense adjacency, invariants, and the
- *                     reference's own GraphStruct compiled into oracle/_ref
+ *                     reference's own GraphStruct compiled into oracle/_ref;
+ *                     the edge-based operands against their dense definitions
  *   spmm / gemm       fp64 brute force, identity / known-answer matrices
  *                     (reference test matrix test/gpu_tensor_test.cpp:311-336),
  *                     and Intel MKL mkl_scsrmm / cblas_sgemm called with the
