@@ -36,6 +36,8 @@ SIGNATURES = {
     "gnnhip_memset0": [_P, _Z, _P],
     "gnnhip_stream_sync": [_P],
     "gnnhip_spmm_csr_f32": [_I, _I, _I, _I, _F, _P, _P, _P, _P, _I, _F, _P, _I, _P],
+    "gnnhip_csr_group_i32": [_I, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P],
+    "gnnhip_csr_transpose_f32": [_I, _I, _I, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_gemm_f32": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P],
     "gnnhip_s2v_level_f32": [_I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_s2v_input_f32": [_I, _I, _I, _P, _P, _P, _P, _P],

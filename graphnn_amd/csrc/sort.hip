@@ -1,0 +1,333 @@
+// Device-side grouping of (key, payload) pairs into CSR, and CSR transposition.
+//
+// graphnn builds the CSR operands of a batch on the host by walking per-node lists
+// (src/nn/msg_pass.cpp:46-177); row i of such a matrix lists the payloads of the pairs
+// whose key is i, in insertion order.  That is a stable sort of the pair indices by key.
+// Here: a least-significant-digit radix sort (8-bit digits, as many passes as the key range
+// needs) whose every pass is stable, then the row pointers from the sorted keys.
+//
+// One pass over n pairs, tiles of 2048 pairs per workgroup:
+//   histogram   per tile, 256 LDS counters -> hist[digit][tile]
+//   scan        exclusive scan of hist in digit-major order (three launches, any length)
+//   scatter     a wavefront takes 512 consecutive pairs of the tile, 64 at a time; lanes with
+//               the same digit find each other with eight ballots, their rank is the running
+//               count of that digit in the wavefront's segment plus the number of lower lanes;
+//               segment counts are then prefixed over the four wavefronts.  Destination =
+//               scanned hist[digit][tile] + rank.  Order inside a digit = input order: stable.
+// No atomics on global memory; the result is a pure function of the input.
+#include "gnnhip_internal.h"
+
+namespace gnnhip {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kItems = 8;
+constexpr int kTile = kBlock * kItems;          // 2048 pairs per workgroup
+constexpr int kSeg = kTile / kWavesPerBlock;    // 512 consecutive pairs per wavefront
+constexpr int kDigits = 256;
+
+__global__ __launch_bounds__(kBlock) void radix_hist_kernel(const unsigned* __restrict__ keys, long long n, int shift,
+                                                             int ntiles, int* __restrict__ hist)
+{
+    __shared__ int h[kDigits];
+    h[threadIdx.x] = 0;
+    __syncthreads();
+    const long long base = (long long)blockIdx.x * kTile;
+#pragma unroll
+    for (int i = 0; i < kItems; ++i) {
+        const long long idx = base + i * kBlock + threadIdx.x;
+        if (idx < n) atomicAdd(&h[(keys[idx] >> shift) & (kDigits - 1)], 1);
+    }
+    __syncthreads();
+    hist[(size_t)threadIdx.x * ntiles + blockIdx.x] = h[threadIdx.x];
+}
+
+// ---- exclusive scan of an int array of any length: segment sums, scan of the sums, apply
+constexpr int kScanSeg = 4096;                  // elements per workgroup: 256 lanes x 16
+__device__ __forceinline__ int block_scan_256(int v, int* sh, int* total)
+{
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    int incl = v;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int o = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += o;
+    }
+    if (lane == kWave - 1) sh[wave] = incl;
+    __syncthreads();
+    int base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) {
+        if (w < wave) base += sh[w];
+        tot += sh[w];
+    }
+    __syncthreads();
+    *total = tot;
+    return base + incl - v;
+}
+
+__global__ __launch_bounds__(kBlock) void scan_segment_sums_kernel(const int* __restrict__ x, long long n, int* __restrict__ seg_sum)
+{
+    __shared__ int sh[kWavesPerBlock];
+    const long long base = (long long)blockIdx.x * kScanSeg + threadIdx.x * 16;
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) if (base + i < n) s += x[base + i];
+    int tot;
+    block_scan_256(s, sh, &tot);
+    if (threadIdx.x == 0) seg_sum[blockIdx.x] = tot;
+}
+
+// one workgroup: exclusive scan of nseg values in place; total to *total_out (may be null)
+__global__ __launch_bounds__(1024) void scan_small_kernel(int* __restrict__ x, int nseg, int* __restrict__ total_out)
+{
+    __shared__ int wave_tot[1024 / kWave];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int per = (nseg + 1023) / 1024;
+    const int lo = min(tid * per, nseg), hi = min(lo + per, nseg);
+    int local = 0;
+    for (int i = lo; i < hi; ++i) local += x[i];
+    int incl = local;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int o = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += o;
+    }
+    if (lane == kWave - 1) wave_tot[wave] = incl;
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < wave; ++w) base += wave_tot[w];
+    int run = base + incl - local;
+    for (int i = lo; i < hi; ++i) { const int v = x[i]; x[i] = run; run += v; }
+    if (tid == 1023 && total_out) *total_out = run;
+}
+
+__global__ __launch_bounds__(kBlock) void scan_apply_kernel(int* __restrict__ x, long long n, const int* __restrict__ seg_off)
+{
+    __shared__ int sh[kWavesPerBlock];
+    const long long base = (long long)blockIdx.x * kScanSeg + threadIdx.x * 16;
+    int v[16];
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { v[i] = (base + i < n) ? x[base + i] : 0; s += v[i]; }
+    int tot;
+    int run = seg_off[blockIdx.x] + block_scan_256(s, sh, &tot);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        if (base + i < n) x[base + i] = run;
+        run += v[i];
+    }
+}
+
+// seg_scratch: at least ceil(n / 4096) ints.  n <= 4096 * 2^22 (the small scan handles what one
+// workgroup walks comfortably; far beyond every use here).
+int exclusive_scan_i32(int* x, long long n, int* seg_scratch, hipStream_t s)
+{
+    if (n <= 0) return GNNHIP_OK;
+    const int nseg = (int)((n + kScanSeg - 1) / kScanSeg);
+    hipLaunchKernelGGL(scan_segment_sums_kernel, dim3(nseg), dim3(kBlock), 0, s, x, n, seg_scratch);
+    hipLaunchKernelGGL(scan_small_kernel, dim3(1), dim3(1024), 0, s, seg_scratch, nseg, (int*)nullptr);
+    hipLaunchKernelGGL(scan_apply_kernel, dim3(nseg), dim3(kBlock), 0, s, x, n, seg_scratch);
+    GNNHIP_LAUNCH_CHECK("exclusive_scan_i32");
+    return GNNHIP_OK;
+}
+
+__global__ __launch_bounds__(kBlock) void radix_scatter_kernel(
+    const unsigned* __restrict__ keys, const unsigned* __restrict__ vals, long long n, int shift, int ntiles,
+    const int* __restrict__ hist_scanned, unsigned* __restrict__ keys_out, unsigned* __restrict__ vals_out, int first_pass)
+{
+    __shared__ int cnt[kWavesPerBlock][kDigits];      // running, then total, count of each digit per wavefront segment
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    for (int i = threadIdx.x; i < kWavesPerBlock * kDigits; i += kBlock) (&cnt[0][0])[i] = 0;
+    __syncthreads();
+
+    const long long seg0 = (long long)blockIdx.x * kTile + wave * kSeg;
+    unsigned k[kItems], v[kItems];
+    int rank[kItems];
+    const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (kWave - lane));
+#pragma unroll
+    for (int i = 0; i < kItems; ++i) {
+        const long long idx = seg0 + i * kWave + lane;
+        const bool live = idx < n;
+        k[i] = live ? keys[idx] : 0u;
+        v[i] = live ? (first_pass ? (unsigned)idx : vals[idx]) : 0u;
+        const unsigned d = (k[i] >> shift) & (kDigits - 1);
+        // lanes of this round with the same digit (dead lanes match nobody)
+        unsigned long long same = __ballot(live);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const unsigned long long bal = __ballot((d >> b) & 1u);
+            same &= ((d >> b) & 1u) ? bal : ~bal;
+        }
+        int r = 0;
+        if (live) {
+            const int before = cnt[wave][d];                       // every lane of the group reads before its leader writes
+            r = before + __popcll(same & below);
+            if ((same & below) == 0) cnt[wave][d] = before + __popcll(same);
+        }
+        rank[i] = r;
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    }
+    __syncthreads();
+    // prefix of the segment counts over the wavefronts, per digit (lane t handles digit t)
+    {
+        const int d = threadIdx.x;
+        int run = 0;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) { const int c = cnt[w][d]; cnt[w][d] = run; run += c; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kItems; ++i) {
+        const long long idx = seg0 + i * kWave + lane;
+        if (idx < n) {
+            const unsigned d = (k[i] >> shift) & (kDigits - 1);
+            const long long dst = (long long)hist_scanned[(size_t)d * ntiles + blockIdx.x] + cnt[wave][d] + rank[i];
+            keys_out[dst] = k[i];
+            vals_out[dst] = v[i];
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void gather_strided_kernel(const int* __restrict__ src, int stride, long long n, unsigned* __restrict__ dst)
+{
+    const long long i = (long long)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) dst[i] = (unsigned)src[i * stride];
+}
+
+// row_ptr from the sorted keys: position i opens every row in (key[i-1], key[i]]; the last position closes the rest
+__global__ __launch_bounds__(kBlock) void row_ptr_from_sorted_kernel(const unsigned* __restrict__ keys, long long n, int rows, int* __restrict__ row_ptr)
+{
+    const long long i = (long long)blockIdx.x * kBlock + threadIdx.x;
+    if (n == 0) {
+        for (long long r = i; r <= rows; r += (long long)gridDim.x * kBlock) row_ptr[r] = 0;
+        return;
+    }
+    if (i >= n) return;
+    const long long k = keys[i];
+    const long long kprev = (i == 0) ? -1 : (long long)keys[i - 1];
+    for (long long r = kprev + 1; r <= k; ++r) row_ptr[r] = (int)i;
+    if (i == n - 1)
+        for (long long r = k + 1; r <= rows; ++r) row_ptr[r] = (int)n;
+}
+
+__global__ __launch_bounds__(kBlock) void fill_grouped_kernel(const unsigned* __restrict__ keys_sorted, const unsigned* __restrict__ perm,
+                                                               long long n, const int* __restrict__ payload, int stride,
+                                                               const float* __restrict__ val_in, int average,
+                                                               const int* __restrict__ row_ptr, int* __restrict__ col_idx, float* __restrict__ val)
+{
+    const long long i = (long long)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const unsigned src = perm[i];
+    col_idx[i] = payload[(long long)src * stride];
+    float w = val_in ? val_in[src] : 1.0f;
+    if (average) {
+        const unsigned r = keys_sorted[i];
+        w = (float)(1.0 / (double)(row_ptr[r + 1] - row_ptr[r]));      // as the reference: double divide, then narrowed
+    }
+    val[i] = w;
+}
+
+// row index of every entry of a CSR matrix
+__global__ __launch_bounds__(kBlock) void expand_rows_kernel(int m, const int* __restrict__ row_ptr, int* __restrict__ row_of)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const long long row = ((long long)blockIdx.x * kBlock + threadIdx.x) / kWave;
+    if (row >= m) return;
+    const int a = row_ptr[row], b = row_ptr[row + 1];
+    for (int t = a + lane; t < b; t += kWave) row_of[t] = (int)row;
+}
+
+inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+}  // namespace
+
+// Groups n pairs by key (0 <= key < rows) keeping input order inside a group:
+//   row_ptr[rows + 1], col_idx[i] = payload of the i-th pair in grouped order,
+//   val[i] = val_in of that pair (or 1), or 1 / group size when average is set.
+// key / payload are read with the given strides (in ints).  Uses scratch slot 0 of the stream.
+int csr_group_pairs(int rows, long long n, const int* key, int key_stride, const int* payload, int payload_stride,
+                    const float* val_in, int average, int* row_ptr, int* col_idx, float* val, hipStream_t s)
+{
+    const int ntiles = (int)((n + kTile - 1) / kTile);
+    const long long nhist = (long long)kDigits * (ntiles > 0 ? ntiles : 1);
+    size_t off = 0;
+    auto carve = [&](size_t bytes) { const size_t o = off; off = round_up(off + bytes, 256); return o; };
+    const size_t o_k0 = carve(sizeof(unsigned) * (size_t)(n > 0 ? n : 1)), o_k1 = carve(sizeof(unsigned) * (size_t)(n > 0 ? n : 1));
+    const size_t o_v0 = carve(sizeof(unsigned) * (size_t)(n > 0 ? n : 1)), o_v1 = carve(sizeof(unsigned) * (size_t)(n > 0 ? n : 1));
+    const size_t o_hist = carve(sizeof(int) * (size_t)nhist);
+    const size_t o_seg = carve(sizeof(int) * (size_t)((nhist + kScanSeg - 1) / kScanSeg + 1));
+    void* base = nullptr;
+    if (int rc = stream_scratch(s, off, &base)) return rc;
+    char* b = static_cast<char*>(base);
+    unsigned* k0 = reinterpret_cast<unsigned*>(b + o_k0);
+    unsigned* k1 = reinterpret_cast<unsigned*>(b + o_k1);
+    unsigned* v0 = reinterpret_cast<unsigned*>(b + o_v0);
+    unsigned* v1 = reinterpret_cast<unsigned*>(b + o_v1);
+    int* hist = reinterpret_cast<int*>(b + o_hist);
+    int* seg = reinterpret_cast<int*>(b + o_seg);
+
+    const unsigned egrid = (unsigned)((n + kBlock - 1) / kBlock);
+    if (n > 0) {
+        hipLaunchKernelGGL(gather_strided_kernel, dim3(egrid), dim3(kBlock), 0, s, key, key_stride, n, k0);
+        int bits = 1;
+        while (bits < 31 && (1ll << bits) < (long long)rows) ++bits;
+        bool first = true;
+        for (int shift = 0; shift < bits; shift += 8) {
+            hipLaunchKernelGGL(radix_hist_kernel, dim3(ntiles), dim3(kBlock), 0, s, k0, n, shift, ntiles, hist);
+            if (int rc = exclusive_scan_i32(hist, nhist, seg, s)) return rc;
+            hipLaunchKernelGGL(radix_scatter_kernel, dim3(ntiles), dim3(kBlock), 0, s, k0, v0, n, shift, ntiles, hist, k1, v1, first ? 1 : 0);
+            unsigned* t = k0; k0 = k1; k1 = t;
+            t = v0; v0 = v1; v1 = t;
+            first = false;
+        }
+    }
+    const unsigned rgrid = n > 0 ? egrid : (unsigned)(((long long)rows + kBlock) / kBlock);
+    hipLaunchKernelGGL(row_ptr_from_sorted_kernel, dim3(rgrid), dim3(kBlock), 0, s, k0, n, rows, row_ptr);
+    if (n > 0)
+        hipLaunchKernelGGL(fill_grouped_kernel, dim3(egrid), dim3(kBlock), 0, s, k0, v0, n, payload, payload_stride, val_in, average,
+                           row_ptr, col_idx, val);
+    GNNHIP_LAUNCH_CHECK("csr_group_pairs");
+    return GNNHIP_OK;
+}
+
+}  // namespace gnnhip
+
+using namespace gnnhip;
+
+extern "C" {
+
+int gnnhip_csr_group_i32(int rows, int n, const int* key, int key_stride, const int* payload, int payload_stride,
+                         int average, int* row_ptr, int* col_idx, float* val, void* stream)
+{
+    GNNHIP_REQUIRE(rows >= 0 && n >= 0 && key_stride >= 1 && payload_stride >= 1, "bad shape in csr_group (rows=%d n=%d)", rows, n);
+    GNNHIP_REQUIRE(row_ptr != nullptr, "null row_ptr in csr_group");
+    GNNHIP_REQUIRE(n == 0 || (key && payload && col_idx && val), "null array in csr_group");
+    GNNHIP_REQUIRE(n == 0 || rows >= 1, "pairs but no rows in csr_group");
+    if (int rc = require_ready()) return rc;
+    return csr_group_pairs(rows, n, key, key_stride, payload, payload_stride, nullptr, average, row_ptr, col_idx, val, as_stream(stream));
+}
+
+int gnnhip_csr_transpose_f32(int m, int k, int nnz, const int* row_ptr, const int* col_idx, const float* val,
+                             int* t_row_ptr, int* t_col_idx, float* t_val, void* stream)
+{
+    GNNHIP_REQUIRE(m >= 0 && k >= 0 && nnz >= 0, "bad shape in csr_transpose (m=%d k=%d nnz=%d)", m, k, nnz);
+    GNNHIP_REQUIRE(row_ptr && t_row_ptr, "null row pointers in csr_transpose");
+    GNNHIP_REQUIRE(nnz == 0 || (col_idx && val && t_col_idx && t_val), "null array in csr_transpose");
+    GNNHIP_REQUIRE(nnz == 0 || k >= 1, "entries but no columns in csr_transpose");
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    int* row_of = nullptr;
+    if (nnz > 0) {
+        // the row index of every entry lives in plan scratch (slot 1); the sort itself uses slot 0
+        void* p = nullptr;
+        if (int rc = stream_scratch_slot(s, 1, sizeof(int) * (size_t)nnz, &p)) return rc;
+        row_of = static_cast<int*>(p);
+        const unsigned grid = (unsigned)(((long long)m * kWave + kBlock - 1) / kBlock);
+        if (m > 0) hipLaunchKernelGGL(expand_rows_kernel, dim3(grid), dim3(kBlock), 0, s, m, row_ptr, row_of);
+    }
+    return csr_group_pairs(k, nnz, col_idx, 1, row_of, 1, val, 0, t_row_ptr, t_col_idx, t_val, s);
+}
+
+}  // extern "C"

@@ -31,6 +31,7 @@ public:
         auto* gv = dynamic_cast<GraphVar*>(operands[0].get());
         ASSERT(gv && gv->graph, "message passing needs a bound GraphVar");
         auto& out = detail::sparse_var<mode, Dtype>(outputs[0], "IMsgPass").value;
+        if (BuildOnDevice(gv->graph, out)) return;
         InitCPUWeight(gv->graph);
         out.CopyFrom(cpu_weight);          // host -> device (or host -> host) copy of the three CSR arrays
     }
@@ -42,9 +43,55 @@ public:
 
 protected:
     virtual void InitCPUWeight(GraphStruct* graph) = 0;
+    // Operands that are a grouping of the flat edge list can be built on the device from one copy
+    // of that list; returns false where the host construction is to be used.
+    virtual bool BuildOnDevice(GraphStruct*, SpTensor<mode, Dtype>&) { return false; }
     SpTensor<CPU, Dtype> cpu_weight;
     bool average;
 };
+
+namespace detail
+{
+// CSR [num_rows, num_cols] on the device whose row y lists, in edge order, the tail x (payload_is_edge
+// false) or the index (true) of every edge x -> y: one copy of the (x, y) pairs, then a stable
+// grouping by y (gnnhip_csr_group_i32).
+inline void group_edges_on_device(GraphStruct* graph, bool payload_is_edge, bool average, size_t num_cols,
+                                  SpTensor<GPU, float>& out, DTensor<GPU, int>& staging)
+{
+    static_assert(sizeof(std::pair<int, int>) == 2 * sizeof(int), "edge list is not a flat (x, y) array");
+    const int E = (int)graph->num_edges, N = (int)graph->num_nodes;
+    out.Reshape({(size_t)N, num_cols});
+    out.ResizeSp(E, N + 1);
+    staging.Reshape({(size_t)(payload_is_edge ? 3 : 2) * (size_t)std::max(E, 1)});
+    int* pairs = staging.data->ptr;
+    if (E > 0) GNN_HIP(gnnhip_memcpy_h2d(pairs, graph->edge_list.data(), sizeof(int) * 2 * (size_t)E, GpuHandle::Stream()));
+    const int* payload = pairs;
+    int payload_stride = 2;
+    if (payload_is_edge) {
+        // edge indices 0..E-1 behind the pairs
+        DTensor<CPU, int> idx({(size_t)std::max(E, 1)});
+        for (int e = 0; e < E; ++e) idx.data->ptr[e] = e;
+        if (E > 0) GNN_HIP(gnnhip_memcpy_h2d(pairs + 2 * (size_t)E, idx.data->ptr, sizeof(int) * (size_t)E, GpuHandle::Stream()));
+        payload = pairs + 2 * (size_t)E;
+        payload_stride = 1;
+    }
+    GNN_HIP(gnnhip_csr_group_i32(N, E, pairs + 1, 2, payload, payload_stride, average ? 1 : 0,
+                                 out.data->row_ptr, out.data->col_idx, out.data->val, GpuHandle::Stream()));
+}
+template<typename Dtype, typename SpT>
+inline bool group_edges_if_gpu(GraphStruct*, bool, bool, size_t, SpT&, DTensor<GPU, int>&) { return false; }
+// Below this many edges the host loop plus three small copies is quicker than the dozen launches of
+// the device sort (configuration 2, 16k edges: 0.26 ms per batch against 0.29 ms).
+constexpr unsigned kDeviceGroupingMinEdges = 1u << 16;
+template<>
+inline bool group_edges_if_gpu<float, SpTensor<GPU, float> >(GraphStruct* graph, bool payload_is_edge, bool average, size_t num_cols,
+                                                             SpTensor<GPU, float>& out, DTensor<GPU, int>& staging)
+{
+    if (graph->num_edges < kDeviceGroupingMinEdges) return false;
+    group_edges_on_device(graph, payload_is_edge, average, num_cols, out, staging);
+    return true;
+}
+}  // namespace detail
 
 template<typename mode, typename Dtype>
 class Node2NodeMsgPass : public IMsgPass<mode, Dtype>
@@ -56,6 +103,12 @@ public:
     Node2NodeMsgPass(std::string _name, bool _average = false) : IMsgPass<mode, Dtype>(_name, _average) {}
 
 protected:
+    virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out) override
+    {
+        return detail::group_edges_if_gpu<Dtype>(graph, false, this->average, graph->num_nodes, out, edge_staging);
+    }
+    DTensor<GPU, int> edge_staging;
+
     virtual void InitCPUWeight(GraphStruct* graph) override
     {
         auto& w = this->cpu_weight;
@@ -86,6 +139,12 @@ public:
     Edge2NodeMsgPass(std::string _name, bool _average = false) : IMsgPass<mode, Dtype>(_name, _average) {}
 
 protected:
+    virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out) override
+    {
+        return detail::group_edges_if_gpu<Dtype>(graph, true, this->average, graph->num_edges, out, edge_staging);
+    }
+    DTensor<GPU, int> edge_staging;
+
     virtual void InitCPUWeight(GraphStruct* graph) override
     {
         auto& w = this->cpu_weight;

@@ -358,3 +358,28 @@ def row_scale(scale, y):
         raise ValueError("one factor per row is needed")
     check(_lib().gnnhip_row_scale_f32(rows, cols, _f32(scale, "scale"), _f32(y, "y"), _stream()))
     return y
+
+
+# ---- device-side CSR construction
+def csr_group(rows, key, payload, average=False, key_stride=1, payload_stride=1, n=None):
+    """row i lists payload[e] of the pairs with key[e] == i in input order (device arrays, int32)"""
+    if n is None:
+        n = key.numel() // key_stride
+    dev = key.device
+    row_ptr = torch.empty(rows + 1, dtype=torch.int32, device=dev)
+    col_idx = torch.empty(n, dtype=torch.int32, device=dev)
+    val = torch.empty(n, dtype=torch.float32, device=dev)
+    check(_lib().gnnhip_csr_group_i32(rows, n, _i32(key, "key"), key_stride, _i32(payload, "payload"), payload_stride,
+                                      int(average), _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"), _f32(val, "val"), _stream()))
+    return row_ptr, col_idx, val
+
+
+def csr_transpose(row_ptr, col_idx, val, m, k):
+    nnz = col_idx.numel()
+    dev = row_ptr.device
+    t_rp = torch.empty(k + 1, dtype=torch.int32, device=dev)
+    t_ci = torch.empty(nnz, dtype=torch.int32, device=dev)
+    t_v = torch.empty(nnz, dtype=torch.float32, device=dev)
+    check(_lib().gnnhip_csr_transpose_f32(m, k, nnz, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"), _f32(val, "val"),
+                                          _i32(t_rp, "t_row_ptr"), _i32(t_ci, "t_col_idx"), _f32(t_v, "t_val"), _stream()))
+    return t_rp, t_ci, t_v

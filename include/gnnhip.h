@@ -80,6 +80,23 @@ int gnnhip_spmm_csr_f32(int m, int k, int n, int nnz, float alpha, const int* ro
                         const float* val, const float* B, int ldb, float beta, float* C, int ldc,
                         void* stream);
 
+/* ---- CSR from (key, payload) pairs on the device: row i lists the payloads of the pairs with key i in
+ *      input order, i.e. what the message-pass factors build on the host from the per-node lists:
+ *      Node2NodeMsgPass (key = edge head y, payload = edge tail x), Edge2NodeMsgPass (payload = edge
+ *      index), SubgraphMsgPass (key = subgraph, payload = node) -- src/nn/msg_pass.cpp:46-94,156-177,
+ *      lists filled by GraphStruct::AddEdge / AddNode (src/util/graph_struct.cpp:62-75).
+ *      key[e * key_stride], payload[e * payload_stride] (strides in ints, so an array of (x, y) pairs
+ *      can be passed as it is).  val = 1, or 1 / row length when average != 0.  Stable radix sort,
+ *      no atomics on global memory: the result is bit-identical to the host construction. */
+int gnnhip_csr_group_i32(int rows, int n, const int* key, int key_stride, const int* payload, int payload_stride,
+                         int average, int* row_ptr, int* col_idx, float* val, void* stream);
+
+/* ---- CSR of the transpose: A [m,k] with nnz entries -> A^T [k,m]; entries of a row of A^T keep the
+ *      order of the rows of A they came from.  The reference transposes implicitly inside cuSPARSE
+ *      csrmm for MM(SpTensor, DTensor, Trans::T) (src/tensor/gpu_dense_tensor.cu:271-296). */
+int gnnhip_csr_transpose_f32(int m, int k, int nnz, const int* row_ptr, const int* col_idx, const float* val,
+                             int* t_row_ptr, int* t_col_idx, float* t_val, void* stream);
+
 /* ---- C[m,n] = alpha * op(A) * op(B) + beta * C, all dense row-major.
  *      DTensor<GPU>::MM(DTensor, DTensor) (src/tensor/gpu_dense_tensor.cu:192-224).
  *      transA/transB: 0 = N, 1 = T.  lda/ldb/ldc are row strides of the stored matrices. */

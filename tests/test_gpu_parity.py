@@ -824,3 +824,83 @@ def test_edge_embedding_step_with_edge_based_operands(gpu, oracle):
     # the same update through the fused level entry: A = edge-to-edge, h = edge states, msg = inp
     fused = ops.s2v_level(*_csr_t(e2e, gpu), _t(m0, gpu), _t(W2, gpu), inp_d)
     assert max_rel(_n(fused), m1) < PARITY_TOL
+
+
+# ------------------------------------------------------------------ device-side CSR construction
+@pytest.mark.parametrize("average", [False, True])
+def test_device_csr_group_matches_host_builders(gpu, oracle, average):
+    from graphnn_amd import ops
+    rng = np.random.default_rng(808)
+    # random multigraph with empty rows, a hub, keys needing two radix passes
+    N, E = 3000, 20000
+    ex = rng.integers(0, N, E).astype(np.int32); ey = rng.integers(0, N, E).astype(np.int32)
+    ey[1000:4000] = 77                                            # one row of 3000+ entries
+    ey[ey == 5] = 6                                               # an empty row
+    want = oracle.csr_node2node(N, ex, ey, average)
+    got = ops.csr_group(N, _t(ey, gpu), _t(ex, gpu), average)
+    for g, w in zip(got, want):
+        assert np.array_equal(_n(g), w)
+    # the same from an interleaved (x, y) array, as GraphStruct::edge_list stores it
+    pairs = _t(np.stack([ex, ey], axis=1).reshape(-1), gpu)
+    got = ops.csr_group(N, pairs[1:], pairs, average, key_stride=2, payload_stride=2, n=E)
+    for g, w in zip(got, want):
+        assert np.array_equal(_n(g), w)
+    # edge-to-node: payload = edge index
+    got = ops.csr_group(N, _t(ey, gpu), _t(np.arange(E, dtype=np.int32), gpu), average)
+    for g, w in zip(got, oracle.csr_edge2node(N, ey, average)):
+        assert np.array_equal(_n(g), w)
+    # subgraph operand with shuffled AddNode order
+    B = 37
+    perm = rng.permutation(N)
+    sid = np.sort(rng.integers(0, B, N))[perm].astype(np.int32); nid = np.arange(N, dtype=np.int32)[perm]
+    got = ops.csr_group(B, _t(sid, gpu), _t(nid, gpu), average)
+    for g, w in zip(got, oracle.csr_subgraph(B, sid, nid, average)):
+        assert np.array_equal(_n(g), w)
+
+
+def test_device_csr_group_edge_cases_and_scale(gpu, oracle):
+    import torch
+    from graphnn_amd import ops
+    # no pairs; one row; one pair
+    rp, ci, v = ops.csr_group(5, torch.zeros(0, dtype=torch.int32, device=gpu), torch.zeros(0, dtype=torch.int32, device=gpu))
+    assert np.array_equal(_n(rp), np.zeros(6, np.int32)) and ci.numel() == 0
+    rp, ci, v = ops.csr_group(1, _t(np.zeros(700, np.int32), gpu), _t(np.arange(700, dtype=np.int32)[::-1].copy(), gpu), True)
+    assert np.array_equal(_n(rp), [0, 700]) and np.array_equal(_n(ci), np.arange(700)[::-1]) and np.all(_n(v) == np.float32(1.0 / 700))
+    rp, ci, v = ops.csr_group(9, _t(np.array([8], np.int32), gpu), _t(np.array([3], np.int32), gpu))
+    assert np.array_equal(_n(rp), [0] * 9 + [1]) and _n(ci)[0] == 3
+    # three radix passes (2^17 rows) and several tiles per pass, against the numpy stable sort
+    rng = np.random.default_rng(9)
+    rows, n = (1 << 17) + 3, 700_001
+    key = rng.integers(0, rows, n).astype(np.int32); pay = rng.integers(0, 1 << 30, n).astype(np.int32)
+    rp, ci, v = ops.csr_group(rows, _t(key, gpu), _t(pay, gpu))
+    order = np.argsort(key, kind="stable")
+    assert np.array_equal(_n(ci), pay[order])
+    want_rp = np.zeros(rows + 1, np.int64); np.cumsum(np.bincount(key, minlength=rows), out=want_rp[1:])
+    assert np.array_equal(_n(rp), want_rp)
+    # a configuration-2 batch: identical to what the host builds
+    batch, w, cfg = synth.make_config(2)
+    want = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    got = ops.csr_group(batch.num_nodes, _t(batch.edge_y, gpu), _t(batch.edge_x, gpu))
+    for g, w_ in zip(got, want):
+        assert np.array_equal(_n(g), w_)
+
+
+def test_device_csr_transpose(gpu, oracle):
+    from graphnn_amd import ops
+    rng = np.random.default_rng(10)
+    m, k = 411, 233
+    csr = _random_csr(rng, m, k, 3000)
+    t_rp, t_ci, t_v = ops.csr_transpose(*_csr_t(csr, gpu), m, k)
+    import scipy.sparse as sp
+    A = sp.csr_matrix((csr[2], csr[1], csr[0]), shape=(m, k))
+    # entry order inside a row of A^T: by row of A, then by position in that row (stable)
+    rows_of = np.repeat(np.arange(m), np.diff(csr[0]))
+    order = np.argsort(csr[1], kind="stable")
+    assert np.array_equal(_n(t_ci), rows_of[order]) and np.array_equal(_n(t_v), csr[2][order])
+    want_rp = np.zeros(k + 1, np.int64); np.cumsum(np.bincount(csr[1], minlength=k), out=want_rp[1:])
+    assert np.array_equal(_n(t_rp), want_rp)
+    # A^T B through the forward SpMM equals the transposed product of the reference path
+    B = rng.standard_normal((m, 24)).astype(np.float32)
+    got = _n(ops.spmm(t_rp, t_ci, t_v, _t(B, gpu), k))
+    assert max_rel(got, oracle.spmm_T(*csr, B, m, k)) < PARITY_TOL
+    assert np.allclose(got, (A.T @ B), atol=1e-4)
