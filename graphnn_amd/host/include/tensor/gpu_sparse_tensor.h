@@ -29,6 +29,23 @@ public:
         data->Reserve(newNNZ, newNPtr);
         data->nnz = newNNZ;
         data->len_ptr = newNPtr;
+        t_valid = false;                   // every builder resizes first: the cached transpose is stale
+    }
+    // CSR of the transpose, built on the device at the first use after the matrix was (re)built and kept
+    // for the following ones (the backward pass multiplies by A^T once per level).  The product with it
+    // goes through the forward SpMM: no atomics, the same bits on every run.
+    SparseData<GPU, Dtype>& Transposed()
+    {
+        if (!t_valid) {
+            if (!t_data) t_data = std::make_shared< SparseData<GPU, Dtype> >();
+            t_data->Reserve(data->nnz, (int)shape[1] + 1);
+            t_data->nnz = data->nnz;
+            t_data->len_ptr = (int)shape[1] + 1;
+            GNN_HIP(gnnhip_csr_transpose_f32((int)shape[0], (int)shape[1], data->nnz, data->row_ptr, data->col_idx, data->val,
+                                             t_data->row_ptr, t_data->col_idx, t_data->val, GpuHandle::Stream()));
+            t_valid = true;
+        }
+        return *t_data;
     }
     // three host-to-device copies, ordered on the layer's stream
     void CopyFrom(SpTensor<CPU, Dtype>& src)
@@ -49,7 +66,7 @@ public:
         GNN_HIP(gnnhip_memcpy_d2d(data->col_idx, src.data->col_idx, sizeof(int) * (size_t)data->nnz, s));
         GNN_HIP(gnnhip_memcpy_d2d(data->row_ptr, src.data->row_ptr, sizeof(int) * (size_t)data->len_ptr, s));
     }
-    void ShallowCopy(SpTensor<GPU, Dtype>& src) { shape = src.shape; data = src.data; }
+    void ShallowCopy(SpTensor<GPU, Dtype>& src) { shape = src.shape; data = src.data; t_valid = false; }
 
     void ArgMax(DTensor<GPU, int>& dst, uint axis = 0)
     {
@@ -60,6 +77,10 @@ public:
     }
 
     std::shared_ptr< SparseData<GPU, Dtype> > data;
+
+private:
+    std::shared_ptr< SparseData<GPU, Dtype> > t_data;   // transpose, see Transposed()
+    bool t_valid = false;
 };
 
 // dense <- alpha * op(sparse) * dense + beta * dense
@@ -74,9 +95,9 @@ inline void TensorTemplate<GPU, DENSE, float>::MM(SpTensor<GPU, float>& a, DTens
         GNN_HIP(gnnhip_spmm_csr_f32((int)m, (int)k, (int)n, a.data->nnz, alpha, a.data->row_ptr, a.data->col_idx, a.data->val,
                                     b.data->ptr, (int)b.cols(), beta, data->ptr, (int)n, GpuHandle::Stream()));
     } else {
-        GNN_HIP(gnnhip_spmm_csr_t_f32((int)a.rows(), (int)a.cols(), (int)n, alpha, a.data->row_ptr, a.data->col_idx,
-                                      a.data->val, b.data->ptr, (int)b.cols(), beta, data->ptr, (int)n,
-                                      GpuHandle::Stream()));
+        auto& t = a.Transposed();
+        GNN_HIP(gnnhip_spmm_csr_f32((int)m, (int)k, (int)n, t.nnz, alpha, t.row_ptr, t.col_idx, t.val,
+                                    b.data->ptr, (int)b.cols(), beta, data->ptr, (int)n, GpuHandle::Stream()));
     }
 }
 
