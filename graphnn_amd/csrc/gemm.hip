@@ -93,9 +93,74 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
 
 }  // namespace
 
+namespace {
+
+// ---- tall A times a matrix of at most four columns (node scores h * w, readouts with one or two
+// classes): a group of G lanes walks one row of A in 128-bit pieces and reduces with shuffles.
+// Reads A once at streaming rate; the tile kernel would spend a 64-column tile on it.
+template <int NCOL, bool TB>
+__global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(
+    int m, int k, float alpha, const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb,
+    float beta, float* C, int ldc, int logG)
+{
+    const int G = 1 << logG;
+    const int sub = threadIdx.x & (G - 1);
+    const long long row = ((long long)blockIdx.x * kBlock + threadIdx.x) >> logG;
+    float acc[NCOL];
+#pragma unroll
+    for (int j = 0; j < NCOL; ++j) acc[j] = 0.f;
+    if (row < m) {
+        const float* a = A + (size_t)row * lda;
+        for (int kk = sub * 4; kk < k; kk += G * 4) {
+            const float4 x = *reinterpret_cast<const float4*>(a + kk);
+#pragma unroll
+            for (int j = 0; j < NCOL; ++j) {
+                const float b0 = TB ? B[(size_t)j * ldb + kk] : B[(size_t)kk * ldb + j];
+                const float b1 = TB ? B[(size_t)j * ldb + kk + 1] : B[(size_t)(kk + 1) * ldb + j];
+                const float b2 = TB ? B[(size_t)j * ldb + kk + 2] : B[(size_t)(kk + 2) * ldb + j];
+                const float b3 = TB ? B[(size_t)j * ldb + kk + 3] : B[(size_t)(kk + 3) * ldb + j];
+                acc[j] += x.x * b0 + x.y * b1 + x.z * b2 + x.w * b3;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < NCOL; ++j)
+        for (int d = G >> 1; d >= 1; d >>= 1) acc[j] += __shfl_xor(acc[j], d, kWave);
+    if (row < m && sub == 0) {
+#pragma unroll
+        for (int j = 0; j < NCOL; ++j) {
+            float* c = C + (size_t)row * ldc + j;
+            *c = (beta == 0.f) ? alpha * acc[j] : alpha * acc[j] + beta * *c;
+        }
+    }
+}
+
+template <int NCOL>
+void launch_skinny(bool tb, int m, int k, float alpha, const float* A, int lda, const float* B, int ldb,
+                   float beta, float* C, int ldc, hipStream_t s)
+{
+    int logG = 0;
+    while ((4 << logG) < k && logG < 6) ++logG;              // G * 4 >= k, at most one wavefront per row
+    const unsigned grid = ceil_div_u((size_t)m << logG, kBlock);
+    if (tb) hipLaunchKernelGGL((sgemm_skinny_kernel<NCOL, true>), dim3(grid), dim3(kBlock), 0, s, m, k, alpha, A, lda, B, ldb, beta, C, ldc, logG);
+    else hipLaunchKernelGGL((sgemm_skinny_kernel<NCOL, false>), dim3(grid), dim3(kBlock), 0, s, m, k, alpha, A, lda, B, ldb, beta, C, ldc, logG);
+}
+
+}  // namespace
+
 int gemm_dispatch(int transA, int transB, int m, int n, int k, float alpha, const float* A, int lda,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s)
 {
+    if (!transA && n <= 4 && m >= 4096 && k >= 4 && k % 4 == 0 && lda % 4 == 0 && aligned16(A)) {
+        switch (n) {
+        case 1: launch_skinny<1>(transB, m, k, alpha, A, lda, B, ldb, beta, C, ldc, s); break;
+        case 2: launch_skinny<2>(transB, m, k, alpha, A, lda, B, ldb, beta, C, ldc, s); break;
+        case 3: launch_skinny<3>(transB, m, k, alpha, A, lda, B, ldb, beta, C, ldc, s); break;
+        default: launch_skinny<4>(transB, m, k, alpha, A, lda, B, ldb, beta, C, ldc, s); break;
+        }
+        GNNHIP_LAUNCH_CHECK("sgemm_skinny");
+        return GNNHIP_OK;
+    }
     dim3 grid(ceil_div_u((size_t)m, BM), ceil_div_u((size_t)n, BN));
     dim3 block(kBlock);
     if (!transA && !transB)

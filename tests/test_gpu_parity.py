@@ -128,7 +128,8 @@ def test_spmm_long_rows(gpu, oracle, n):
 
 
 # ------------------------------------------------------------------ GEMM
-@pytest.mark.parametrize("shape", [(1, 1, 1), (7, 5, 3), (64, 64, 16), (65, 63, 17), (300, 2, 32), (1000, 64, 38), (33, 130, 70)])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (7, 5, 3), (64, 64, 16), (65, 63, 17), (300, 2, 32), (1000, 64, 38), (33, 130, 70),
+                                   (5000, 1, 64), (4097, 2, 32), (6000, 3, 8), (5001, 4, 260), (5000, 1, 4)])
 def test_gemm_all_transposes(gpu, oracle, shape):
     from graphnn_amd import ops
     m, n, k = shape
