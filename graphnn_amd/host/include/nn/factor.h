@@ -12,6 +12,14 @@ namespace gnn
 
 typedef std::vector< std::shared_ptr<Variable> > VarPtrList;
 
+// what a message-pass factor learnt about the layout of the last batch while building its operand
+struct BatchLayout
+{
+    bool block_diagonal = false;           // node-to-node operand: no edge joins two subgraphs
+    bool contiguous_subgraphs = false;     // subgraph operand: graph g owns one contiguous, ascending node range
+    int max_subgraph_nodes = 0;
+};
+
 class Factor
 {
 public:
@@ -27,6 +35,8 @@ public:
 
     // tag used by the inference-time fusion pass of FactorGraph; "" = never fused
     virtual const char* FuseKind() const { return ""; }
+    // layout facts of the last batch, for factors that build batch operands (null otherwise)
+    virtual const BatchLayout* Layout() const { return nullptr; }
 
     std::string name;
     PropErr properr;

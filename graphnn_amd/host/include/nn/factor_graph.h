@@ -155,6 +155,7 @@ protected:
     Plan* GetPlan(const std::vector<VarPtr>& targets, const std::map<std::string, void*>& feed_dict, Phase phase);
     void BuildPlan(Plan& plan);
     void BuildFusedSteps(Plan& plan);      // nn/s2v_fusion.h
+    void FoldWholeForward(Plan& plan);     // nn/s2v_fusion.h
 
     std::vector<size_t> always_ready;       // params and non-placeholder constants
     std::vector< std::unique_ptr<Plan> > plans;

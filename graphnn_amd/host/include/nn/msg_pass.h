@@ -37,9 +37,8 @@ public:
     }
 
     // layout facts about the last batch, gathered while the CSR was built (used to choose kernels)
-    bool block_diagonal = false;           // node2node: no edge joins two subgraphs
-    bool contiguous_subgraphs = false;     // subgraph: graph g owns one contiguous, ascending node range
-    int max_subgraph_nodes = 0;
+    virtual const BatchLayout* Layout() const override { return &layout; }
+    BatchLayout layout;
 
 protected:
     virtual void InitCPUWeight(GraphStruct* graph) = 0;
@@ -101,10 +100,12 @@ public:
     using OutType = std::shared_ptr< SpTensorVar<mode, Dtype> >;
     OutType CreateOutVar() { return std::make_shared< SpTensorVar<mode, Dtype> >(fmt::sprintf("%s:out_0", this->name)); }
     Node2NodeMsgPass(std::string _name, bool _average = false) : IMsgPass<mode, Dtype>(_name, _average) {}
+    virtual const char* FuseKind() const override { return "msg_node2node"; }
 
 protected:
     virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out) override
     {
+        this->layout.block_diagonal = false;           // not examined on this route
         return detail::group_edges_if_gpu<Dtype>(graph, false, this->average, graph->num_nodes, out, edge_staging);
     }
     DTensor<GPU, int> edge_staging;
@@ -126,7 +127,16 @@ protected:
         }
         rp[graph->num_nodes] = nnz;
         ASSERT(nnz == (int)graph->num_edges, "edge count does not match the in-edge lists");
+        // does any edge join two subgraphs?  (node -> subgraph from the subgraph lists)
+        node_subgraph.assign(graph->num_nodes, -1);
+        for (unsigned g = 0; g < graph->num_subgraph; ++g)
+            for (int node : graph->subgraph->head[g])
+                if (node >= 0 && node < (int)graph->num_nodes) node_subgraph[node] = (int)g;
+        bool diagonal = true;
+        for (const auto& e : graph->edge_list) diagonal = diagonal && node_subgraph[e.first] == node_subgraph[e.second];
+        this->layout.block_diagonal = diagonal;
     }
+    std::vector<int> node_subgraph;
 };
 
 template<typename mode, typename Dtype>
@@ -236,6 +246,7 @@ public:
     using OutType = std::shared_ptr< SpTensorVar<mode, Dtype> >;
     OutType CreateOutVar() { return std::make_shared< SpTensorVar<mode, Dtype> >(fmt::sprintf("%s:out_0", this->name)); }
     SubgraphMsgPass(std::string _name, bool _average = false) : IMsgPass<mode, Dtype>(_name, _average) {}
+    virtual const char* FuseKind() const override { return "msg_subgraph"; }
 
 protected:
     virtual void InitCPUWeight(GraphStruct* graph) override
@@ -262,8 +273,8 @@ protected:
         }
         rp[graph->num_subgraph] = nnz;
         ASSERT(nnz == (int)graph->num_nodes, "node count does not match the subgraph lists");
-        this->contiguous_subgraphs = contiguous;
-        this->max_subgraph_nodes = biggest;
+        this->layout.contiguous_subgraphs = contiguous;
+        this->layout.max_subgraph_nodes = biggest;
     }
 };
 

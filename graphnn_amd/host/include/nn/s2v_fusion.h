@@ -3,6 +3,8 @@
 //
 //   MatMul(sparse A, h) -> MatMul(., W) -> ElewiseAdd(., msg) -> ReLU      => gnnhip_s2v_level_f32
 //   MatMul(dense X, W)  -> ReLU                                             => gnnhip_s2v_input_f32
+//   input -> levels -> MatMul(S, h) -> MatMul(., W1) -> ReLU -> MatMul(., W2), when the batch is laid
+//   out as GetBatch lays it out (contiguous graphs, no edge between graphs)  => gnnhip_s2v_forward_batched_f32
 //
 // (the chains of examples/graph_classification/src/kernel_mean_field.cpp:31-47).  A chain
 // is folded only at Phase::TEST and only when its intermediate variables have no other
@@ -26,6 +28,8 @@ struct FusedStep
     std::vector<size_t> factors;            // graph factors this step stands for
     std::function<void(Phase)> run;
     bool fused;
+    enum Tag { SINGLE, INPUT, LEVEL, FORWARD } tag = SINGLE;
+    std::vector<size_t> vars;               // INPUT: X, W, msg, h0;  LEVEL: A, h_in, W, msg, h_out
 };
 }  // namespace detail
 
@@ -152,6 +156,8 @@ inline void FactorGraph::BuildFusedSteps(Plan& plan)
                         auto step = std::make_shared<detail::FusedStep>();
                         step->factors = {f1, f2, f3, f4};
                         step->fused = true;
+                        step->tag = detail::FusedStep::LEVEL;
+                        step->vars = {a, b, w, other, factor_nodes[f4].out[0]};
                         step->run = [A, H, W, M, O](Phase) {
                             ASSERT(A->value.cols() == H->value.rows() && H->value.cols() == W->value.rows() &&
                                    W->value.rows() == W->value.cols() && M->value.shape == H->value.shape &&
@@ -180,6 +186,8 @@ inline void FactorGraph::BuildFusedSteps(Plan& plan)
                     auto step = std::make_shared<detail::FusedStep>();
                     step->factors = {f1, fr};
                     step->fused = true;
+                    step->tag = detail::FusedStep::INPUT;
+                    step->vars = {a, b, p1, factor_nodes[fr].out[0]};
                     step->run = [X, W, M, O](Phase) {
                         ASSERT(X->value.rank() == 2 && W->value.rank() == 2 && X->value.cols() == W->value.rows(), "mat dim doesn't match");
                         M->value.Reshape({X->value.rows(), W->value.cols()});
@@ -200,6 +208,153 @@ inline void FactorGraph::BuildFusedSteps(Plan& plan)
             plan.steps.push_back(single_step(f1));
         }
     }
+    if (fold) FoldWholeForward(plan);
+}
+
+// Second pass over the steps: input + a chain of levels with one A and one W + the readout
+// MatMul(S, h) -> MatMul(., W1) -> ReLU -> MatMul(., W2) become one step that, batch by batch, calls the
+// one-launch graph-resident forward when the batch is block diagonal with contiguous graphs (facts the
+// message-pass factors record while they build their operands) and the library covers the shape, and
+// otherwise runs the steps it replaced.  The one-launch kernel keeps the inner levels' embeddings and
+// the pre-activation of the hidden layer in LDS, so those variables must be private to the chain.
+inline void FactorGraph::FoldWholeForward(Plan& plan)
+{
+    typedef DTensorVar<GPU, float> DVar;
+    typedef SpTensorVar<GPU, float> SVar;
+    typedef detail::FusedStep Step;
+    auto& steps = plan.steps;
+    std::vector<bool> is_target(var_list.size(), false);
+    for (size_t v : plan.target_idx) is_target[v] = true;
+    auto dense = [&](size_t v) { return dynamic_cast<DVar*>(var_list[v].get()); };
+    auto sparse = [&](size_t v) { return dynamic_cast<SVar*>(var_list[v].get()); };
+    auto find_step = [&](std::function<bool(const Step&)> pred) -> int {
+        for (size_t i = 0; i < steps.size(); ++i) if (steps[i] && pred(*steps[i])) return (int)i;
+        return -1;
+    };
+    auto single_of_kind = [&](const Step& st, const char* k) {
+        return st.tag == Step::SINGLE && st.factors.size() == 1 && !strcmp(factor_list[st.factors[0]]->FuseKind(), k);
+    };
+
+    for (size_t si = 0; si < steps.size(); ++si) {
+        if (!steps[si] || steps[si]->tag != Step::INPUT) continue;
+        const size_t vX = steps[si]->vars[0], vWn = steps[si]->vars[1], vMsg = steps[si]->vars[2], vH0 = steps[si]->vars[3];
+        std::vector<int> chain = {(int)si};
+        // ---- levels
+        size_t cur = vH0, vA = (size_t)-1, vWc = (size_t)-1;
+        std::vector<size_t> inner;                       // embeddings the one-launch kernel does not write
+        for (;;) {
+            const int li = find_step([&](const Step& st) {
+                return st.tag == Step::LEVEL && st.vars[1] == cur && st.vars[3] == vMsg &&
+                       (vA == (size_t)-1 || (st.vars[0] == vA && st.vars[2] == vWc));
+            });
+            if (li < 0) break;
+            vA = steps[li]->vars[0];
+            vWc = steps[li]->vars[2];
+            inner.push_back(cur);
+            cur = steps[li]->vars[4];
+            chain.push_back(li);
+        }
+        const int L = (int)chain.size() - 1;
+        if (L < 1) continue;
+        // ---- readout
+        const int i5 = find_step([&](const Step& st) {
+            return single_of_kind(st, "matmul_nn") && sparse(factor_nodes[st.factors[0]].in[0]) && factor_nodes[st.factors[0]].in[1] == cur;
+        });
+        if (i5 < 0) continue;
+        const size_t vS = factor_nodes[steps[i5]->factors[0]].in[0], vPool = factor_nodes[steps[i5]->factors[0]].out[0];
+        // the hidden layer: MatMul + ReLU, already folded into one input-style step or still two factors
+        size_t vW1, vLin, vHid;
+        int i6 = find_step([&](const Step& st) { return st.tag == Step::INPUT && st.vars[0] == vPool; });
+        int i7 = -1;
+        if (i6 >= 0) {
+            vW1 = steps[i6]->vars[1]; vLin = steps[i6]->vars[2]; vHid = steps[i6]->vars[3];
+        } else {
+            i6 = find_step([&](const Step& st) {
+                return single_of_kind(st, "matmul_nn") && factor_nodes[st.factors[0]].in[0] == vPool && dense(factor_nodes[st.factors[0]].in[1]);
+            });
+            if (i6 < 0) continue;
+            vW1 = factor_nodes[steps[i6]->factors[0]].in[1];
+            vLin = factor_nodes[steps[i6]->factors[0]].out[0];
+            i7 = find_step([&](const Step& st) { return single_of_kind(st, "relu") && factor_nodes[st.factors[0]].in[0] == vLin; });
+            if (i7 < 0) continue;
+            vHid = factor_nodes[steps[i7]->factors[0]].out[0];
+        }
+        const int i8 = find_step([&](const Step& st) {
+            return single_of_kind(st, "matmul_nn") && factor_nodes[st.factors[0]].in[0] == vHid && dense(factor_nodes[st.factors[0]].in[1]);
+        });
+        if (i8 < 0) continue;
+        const size_t vW2 = factor_nodes[steps[i8]->factors[0]].in[1], vLogits = factor_nodes[steps[i8]->factors[0]].out[0];
+        if (!(dense(vX) && dense(vWn) && dense(vWc) && dense(vW1) && dense(vW2) && dense(vPool) && dense(vHid) && dense(vLogits) &&
+              dense(vMsg) && dense(cur) && sparse(vA) && sparse(vS))) continue;
+        chain.push_back(i5); chain.push_back(i6); if (i7 >= 0) chain.push_back(i7); chain.push_back(i8);
+
+        // ---- everything between X and the logits is read inside the chain only; what the kernel keeps
+        //      in LDS is not a target either
+        std::vector<bool> in_chain(factor_list.size(), false);
+        for (int c : chain) for (size_t f : steps[c]->factors) in_chain[f] = true;
+        auto private_to_chain = [&](size_t v) {
+            for (size_t f : var_nodes[v].consumers) if (plan.executed[f] && !in_chain[f]) return false;
+            return true;
+        };
+        bool ok = private_to_chain(vMsg) && private_to_chain(cur) && private_to_chain(vPool) && private_to_chain(vLin) &&
+                  private_to_chain(vHid) && !is_target[vLin];
+        inner.erase(inner.begin());                     // h0 is tested with the other inner embeddings below
+        ok = ok && private_to_chain(vH0) && !is_target[vH0];
+        for (size_t v : inner) ok = ok && private_to_chain(v) && !is_target[v];
+        // the operands must come from the message-pass factors that know the batch layout
+        auto producer = [&](size_t v) -> Factor* {
+            return var_nodes[v].producers.size() == 1 ? factor_list[var_nodes[v].producers[0]].get() : nullptr;
+        };
+        Factor* fa = producer(vA);
+        Factor* fs = producer(vS);
+        if (!ok || !fa || !fs || strcmp(fa->FuseKind(), "msg_node2node") || strcmp(fs->FuseKind(), "msg_subgraph")) continue;
+        const BatchLayout* n2n = fa->Layout();
+        const BatchLayout* sub = fs->Layout();
+        if (!n2n || !sub) continue;
+
+        std::vector< std::shared_ptr<Step> > parts;
+        std::sort(chain.begin(), chain.end());
+        for (int c : chain) parts.push_back(steps[c]);
+        auto step = std::make_shared<Step>();
+        step->fused = true;
+        step->tag = Step::FORWARD;
+        for (auto& p : parts) step->factors.insert(step->factors.end(), p->factors.begin(), p->factors.end());
+        DVar *X = dense(vX), *Wn = dense(vWn), *Wc = dense(vWc), *W1 = dense(vW1), *W2 = dense(vW2), *Msg = dense(vMsg),
+             *Hl = dense(cur), *Pool = dense(vPool), *Hid = dense(vHid), *Logits = dense(vLogits);
+        SVar *A = sparse(vA), *S = sparse(vS);
+        step->run = [=](Phase ph) {
+            bool done = false;
+            if (n2n->block_diagonal && sub->contiguous_subgraphs && sub->max_subgraph_nodes > 0) {
+                const size_t N = X->value.rows(), K = X->value.cols(), C = Wn->value.cols(), H = W1->value.cols(),
+                             Q = W2->value.cols(), B = S->value.rows();
+                ASSERT(Wn->value.rows() == K && Wc->value.rows() == C && Wc->value.cols() == C && W1->value.rows() == C &&
+                       W2->value.rows() == H && A->value.rows() == N && A->value.cols() == N && S->value.cols() == N,
+                       "fused forward: operand shapes do not chain");
+                Msg->value.Reshape({N, C});
+                Hl->value.Reshape({N, C});
+                Pool->value.Reshape({B, C});
+                Hid->value.Reshape({B, H});
+                Logits->value.Reshape({B, Q});
+                const int rc = gnnhip_s2v_forward_batched_f32(
+                    (int)N, (int)B, (int)K, (int)C, (int)H, (int)Q, L, sub->max_subgraph_nodes,
+                    A->value.data->row_ptr, A->value.data->col_idx, A->value.data->val,
+                    S->value.data->row_ptr, S->value.data->col_idx, S->value.data->val,
+                    X->value.data->ptr, Wn->value.data->ptr, Wc->value.data->ptr, W1->value.data->ptr, W2->value.data->ptr,
+                    Msg->value.data->ptr, Hl->value.data->ptr, Pool->value.data->ptr, Hid->value.data->ptr,
+                    Logits->value.data->ptr, nullptr, nullptr, nullptr, GpuHandle::Stream());
+                if (rc == GNNHIP_OK) done = true;
+                else ASSERT(rc == GNNHIP_EUNSUPPORTED, gnnhip_last_error());
+            }
+            if (!done) for (auto& p : parts) p->run(ph);
+        };
+        // the new step takes the place of the last part; the others leave the schedule
+        const int last = chain.back();
+        size_t folded = 0;
+        for (int c : chain) { folded += steps[c]->fused ? 1 : 0; steps[c].reset(); }
+        steps[last] = step;
+        plan.n_fused = plan.n_fused - folded + 1;
+    }
+    steps.erase(std::remove(steps.begin(), steps.end(), std::shared_ptr<Step>()), steps.end());
 }
 
 inline FactorGraph::VarList FactorGraph::FeedForward(std::vector<VarPtr> targets, std::map<std::string, void*> feed_dict,

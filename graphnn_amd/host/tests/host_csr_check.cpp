@@ -5,7 +5,7 @@
 //   host_csr_check <in.bin> <out.bin> <average 0|1>
 //   in.bin : int32 B, N, E, then subg_id[N], node_idx[N], edge_x[E], edge_y[E]
 //   out.bin: int32 a_row_ptr[N+1], a_col[E], fp32 a_val[E], int32 s_row_ptr[B+1], s_col[N], fp32 s_val[N],
-//            int32 flags {contiguous_subgraphs, max_subgraph_nodes},
+//            int32 flags {contiguous_subgraphs, max_subgraph_nodes, block_diagonal},
 //            then the edge-based operands: e2n row_ptr[N+1], col[E], val[E]; n2e row_ptr[E+1], col[E], val[E];
 //            int32 nnz of e2e, e2e row_ptr[E+1], col[nnz], val[nnz]
 #include <cstdio>
@@ -58,8 +58,9 @@ int main(int argc, char** argv)
     fwrite(ad.row_ptr, 4, N + 1, o); fwrite(ad.col_idx, 4, E, o); fwrite(ad.val, 4, E, o);
     fwrite(sd.row_ptr, 4, B + 1, o); fwrite(sd.col_idx, 4, N, o); fwrite(sd.val, 4, N, o);
     auto* sf = dynamic_cast<SubgraphMsgPass<CPU, float>*>(fg.factor_list[1].get());
-    int flags[2] = {sf->contiguous_subgraphs ? 1 : 0, sf->max_subgraph_nodes};
-    fwrite(flags, 4, 2, o);
+    int flags[3] = {sf->layout.contiguous_subgraphs ? 1 : 0, sf->layout.max_subgraph_nodes,
+                    fg.factor_list[0]->Layout()->block_diagonal ? 1 : 0};
+    fwrite(flags, 4, 3, o);
 
     // ---- edge-based operands of the loopy-BP embedding
     FactorGraph fg2;

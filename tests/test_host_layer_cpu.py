@@ -30,7 +30,7 @@ def _run(tmp_path, B, N, E, sid, nid, ex, ey, average):
         return a
 
     res = (take(N + 1, np.int32), take(E, np.int32), take(E, np.float32),
-           take(B + 1, np.int32), take(N, np.int32), take(N, np.float32), take(2, np.int32))
+           take(B + 1, np.int32), take(N, np.int32), take(N, np.float32), take(3, np.int32))
     e2n = (take(N + 1, np.int32), take(E, np.int32), take(E, np.float32))
     n2e = (take(E + 1, np.int32), take(E, np.int32), take(E, np.float32))
     nnz = int(take(1, np.int32)[0])
@@ -52,7 +52,7 @@ def test_cpp_builders_match_oracle_random(oracle, tmp_path, average):
         assert np.array_equal(got, want)
     for got, want in zip((srp, sci, sv), oracle.csr_subgraph(B, sid, nid, average)):
         assert np.array_equal(got, want)
-    assert flags[0] == 0 and flags[1] == np.bincount(sid, minlength=B).max()
+    assert flags[0] == 0 and flags[1] == np.bincount(sid, minlength=B).max() and flags[2] == 0     # edges cross subgraphs
     e2n, n2e, e2e = _run.edge_operands
     for got, want in zip(e2n, oracle.csr_edge2node(N, ey, average)):
         assert np.array_equal(got, want)
@@ -70,7 +70,7 @@ def test_cpp_builders_on_a_getbatch_style_batch(oracle, tmp_path):
     for got, want in zip((arp, aci, av), oracle.csr_node2node(b.num_nodes, b.edge_x, b.edge_y)):
         assert np.array_equal(got, want)
     assert np.array_equal(sci, np.arange(b.num_nodes)) and np.all(sv == 1)
-    assert flags[0] == 1 and flags[1] == b.graph_sizes.max()       # contiguous layout recognised
+    assert flags[0] == 1 and flags[1] == b.graph_sizes.max() and flags[2] == 1      # GetBatch layout recognised
     e2n, n2e, e2e = _run.edge_operands
     for got, want in zip(e2e, oracle.csr_edge2edge(b.num_nodes, b.edge_x, b.edge_y)):
         assert np.array_equal(got, want)
