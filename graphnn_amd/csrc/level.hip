@@ -216,6 +216,14 @@ __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
     const long long wave_stride = (long long)gridDim.x * kWavesPerBlock;
     for (long long tile_id = (long long)blockIdx.x * kWavesPerBlock + wave; tile_id < ntiles; tile_id += wave_stride) {
         const long long row0 = tile_id * 16;
+        // msg of this tile is asked for first, so its trip to memory runs under the gather and the
+        // contraction instead of after them
+        float4 mpre[NJB];
+#pragma unroll
+        for (int jb = 0; jb < NJB; ++jb) {
+            mpre[jb] = f4_zero();
+            if (msg && row0 + t < N) mpre[jb] = *reinterpret_cast<const float4*>(msg + (size_t)(row0 + t) * C + KS * q + 4 * jb);
+        }
         if (DENSE) {
 #pragma unroll
             for (int rd = 0; rd < ROUNDS; ++rd) {
@@ -373,10 +381,7 @@ __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
                     const float4 b4 = *reinterpret_cast<const float4*>(bias + cbase);
                     v.x += b4.x; v.y += b4.y; v.z += b4.z; v.w += b4.w;
                 }
-                if (msg) {
-                    const float4 mm = *reinterpret_cast<const float4*>(msg + off);
-                    v.x += mm.x; v.y += mm.y; v.z += mm.z; v.w += mm.w;
-                }
+                v.x += mpre[jb].x; v.y += mpre[jb].y; v.z += mpre[jb].z; v.w += mpre[jb].w;
                 *reinterpret_cast<float4*>(h_out + off) =
                     make_float4(relu_ref(v.x), relu_ref(v.y), relu_ref(v.z), relu_ref(v.w));
             }
