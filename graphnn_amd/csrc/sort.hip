@@ -190,10 +190,13 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(
     }
 }
 
-__global__ __launch_bounds__(kBlock) void gather_strided_kernel(const int* __restrict__ src, int stride, long long n, unsigned* __restrict__ dst)
+// keys as unsigned, forced into [0, rows): a key outside that range is a caller error, but it must not
+// send the row-pointer kernels out of bounds
+__global__ __launch_bounds__(kBlock) void gather_strided_kernel(const int* __restrict__ src, int stride, long long n, int rows,
+                                                                 unsigned* __restrict__ dst)
 {
     const long long i = (long long)blockIdx.x * kBlock + threadIdx.x;
-    if (i < n) dst[i] = (unsigned)src[i * stride];
+    if (i < n) dst[i] = (unsigned)min(max(src[i * stride], 0), rows - 1);
 }
 
 // row_ptr from the sorted keys: position i opens every row in (key[i-1], key[i]]; the last position closes the rest
@@ -270,7 +273,7 @@ int csr_group_pairs(int rows, long long n, const int* key, int key_stride, const
 
     const unsigned egrid = (unsigned)((n + kBlock - 1) / kBlock);
     if (n > 0) {
-        hipLaunchKernelGGL(gather_strided_kernel, dim3(egrid), dim3(kBlock), 0, s, key, key_stride, n, k0);
+        hipLaunchKernelGGL(gather_strided_kernel, dim3(egrid), dim3(kBlock), 0, s, key, key_stride, n, rows, k0);
         int bits = 1;
         while (bits < 31 && (1ll << bits) < (long long)rows) ++bits;
         bool first = true;
