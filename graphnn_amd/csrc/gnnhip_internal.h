@@ -152,7 +152,7 @@ constexpr int kScratchSlots = 2;
 int stream_scratch_slot(hipStream_t s, int slot, size_t bytes, void** p);
 
 // ---- high-degree rows (hub.hip)
-constexpr int kHubThreshold = 256;     // rows with more entries are summed by the pre-pass
+constexpr int kHubThreshold = 64;      // rows with more entries are summed by the pre-pass
 constexpr int kHubChunk = 2048;        // entries per partial sum of the pre-pass
 constexpr int kHubMinRows = 32768;     // smaller matrices skip the pre-pass: its launches would cost more than a long row
 struct HubPlan {

@@ -685,12 +685,12 @@ def _hub_matrix(rng, m, k, long_rows):
 
 @pytest.mark.parametrize("n", [64, 128, 7, 36, 300])
 def test_spmm_hub_rows_balanced_pass(gpu, oracle, n):
-    """matrix large enough for the balanced pass over long rows: rows of 257 (one chunk), 2048, 2049 and
-    9000 entries (several chunks), neighbours at the low indices, an empty row between them"""
+    """matrix large enough for the balanced pass over long rows: rows of 65 and 257 (one chunk), 2048, 2049 and
+    9000 entries (several chunks), 64 (just below the threshold), neighbours at the low indices, an empty row between them"""
     from graphnn_amd import ops
     rng = np.random.default_rng(500 + n)
     m = k = 40000
-    csr = _hub_matrix(rng, m, k, [(0, 9000), (1, 2049), (2, 0), (3, 2048), (4, 257), (5, 256), (17000, 5000), (m - 1, 700)])
+    csr = _hub_matrix(rng, m, k, [(0, 9000), (1, 2049), (2, 0), (3, 2048), (4, 257), (5, 256), (6, 65), (7, 64), (17000, 5000), (m - 1, 700)])
     B = rng.standard_normal((k, n)).astype(np.float32)
     C0 = rng.standard_normal((m, n)).astype(np.float32)
     got = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m))
@@ -707,7 +707,7 @@ def test_level_hub_rows_balanced_pass(gpu, oracle, C):
     from graphnn_amd import ops
     rng = np.random.default_rng(600 + C)
     N = 36000
-    csr = _hub_matrix(rng, N, N, [(0, 12000), (1, 4100), (7, 300), (15, 257), (16, 2048), (20000, 3000), (N - 1, 1000)])
+    csr = _hub_matrix(rng, N, N, [(0, 12000), (1, 4100), (7, 300), (15, 257), (16, 2048), (17, 65), (18, 64), (19, 49), (20000, 3000), (N - 1, 1000)])
     h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
     W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
     msg = rng.standard_normal((N, C)).astype(np.float32)
