@@ -565,8 +565,8 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
     if (C == 16 || C == 32 || C == 64) {
         // On power-law graphs the per-row gather of the fused kernel is latency-bound (a lane group walks
         // a row of 50..250 entries a few loads at a time, and such rows sit next to each other), while the
-        // SpMM keeps far more gathers in flight.  Measured on R-MAT (4M rows, 16 entries per row, long-row threshold 256):
-        // fused 8.7 ms, SpMM into h_out + contraction in place 5.9 ms; on a uniform random graph of the same
+        // SpMM keeps far more gathers in flight.  Measured on R-MAT (4M rows, 16 entries per row): fused
+        // 6.2 ms, SpMM into h_out + contraction in place 4.7 ms; on a uniform random graph of the same
         // density the fused kernel wins by 12 % (0.81 vs 0.91 ms per 1M rows).  The host only knows the
         // mean degree, and dense graphs in practice are the skewed ones, so large graphs with at least
         // kTwoStepMeanDegree entries per row take the two launches.
