@@ -11,12 +11,10 @@ namespace gnnhip {
 bool fused_hidden_supported(int C);
 int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s);
 int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-                   const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s);
+                   const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph = false);
 int readout_dispatch(int B, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                      const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
                      float* logits, float* probs, int* pred, hipStream_t s);
-int spmm_dispatch(int m, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                  const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s);
 int gemm_dispatch(int transA, int transB, int m, int n, int k, float alpha, const float* A, int lda,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s);
 int row_softmax_dispatch(float* x, int rows, int cols, hipStream_t s);
@@ -63,15 +61,15 @@ int input_any(int N, int K, int C, const float* X, const float* Wn2l, float* msg
 }
 
 int level_any(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-              const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
+              const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph = false)
 {
-    int rc = level_dispatch(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    int rc = level_dispatch(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s, same_graph);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
     void* tmp = nullptr;
     const size_t total = (size_t)N * C;
     if ((rc = stream_scratch(s, sizeof(float) * total, &tmp))) return rc;
     float* agg = static_cast<float*>(tmp);
-    if ((rc = spmm_dispatch(N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, agg, C, s))) return rc;
+    if ((rc = spmm_dispatch(N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, agg, C, s, same_graph))) return rc;
     if ((rc = gemm_dispatch(0, 0, N, C, C, 1.f, agg, C, W, C, 0.f, h_out, C, s))) return rc;
     hipLaunchKernelGGL(bias_add_relu_kernel, dim3(ew_grid(total)), dim3(kBlock), 0, s,
                        h_out, bias, msg, h_out, (float*)nullptr, total, C, 1);
@@ -172,7 +170,7 @@ int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L, int 
     float* cur = h_a;
     float* nxt = h_b;
     for (int lv = 0; lv < L; ++lv) {
-        if ((rc = level_any(N, C, a_nnz, a_row_ptr, a_col_idx, a_val, cur, W_conv, msg, nullptr, nxt, s))) return rc;
+        if ((rc = level_any(N, C, a_nnz, a_row_ptr, a_col_idx, a_val, cur, W_conv, msg, nullptr, nxt, s, lv > 0))) return rc;
         float* t = cur; cur = nxt; nxt = t;
     }
     if (which_h) *which_h = (cur == h_a) ? 0 : 1;

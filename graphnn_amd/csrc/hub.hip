@@ -288,8 +288,11 @@ void launch_partial_combine(hipStream_t s, const int* counts, int hub_cap, int c
 // Sums the hubs of A (rows longer than kHubThreshold) times B[:, 0..n) into plan->agg.
 // n <= 1024.  The buffers live in the stream's plan scratch and stay valid until the next
 // hub_prepass on the same stream.
+// reuse_plan: the caller guarantees that the structure of A has not changed since the previous call on
+// this stream with the same arguments (the levels of one forward); the three planning launches
+// (count, scan, fill) are then skipped and only the sums are recomputed.
 int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
-                const float* B, int ldb, hipStream_t s, HubPlan* plan)
+                const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan)
 {
     plan->row_slot = nullptr;
     plan->agg = nullptr;
@@ -331,10 +334,17 @@ int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_
     float* part = reinterpret_cast<float*>(b + o_part);
     float* agg = reinterpret_cast<float*>(b + o_agg);
 
-    hipLaunchKernelGGL(hub_count_kernel, dim3(nb), dim3(kBlock), 0, s, m, row_ptr, bh, bc);
-    hipLaunchKernelGGL(hub_scan_kernel, dim3(1), dim3(kScanBlock), 0, s, nb, bh, bc, counts);
-    hipLaunchKernelGGL(hub_fill_kernel, dim3(nb), dim3(kBlock), 0, s, m, row_ptr, bh, bc, hub_cap, chunk_cap, row_slot,
-                       hub_row, hub_chunk0, chunk_hub);
+    struct Memo { hipStream_t s; const int* row_ptr; int m, n; long long nnz; void* base; };
+    static thread_local Memo memo = {nullptr, nullptr, 0, 0, 0, nullptr};
+    const bool planned = reuse_plan && memo.row_ptr == row_ptr && memo.s == s && memo.m == m && memo.n == n &&
+                         memo.nnz == nnz && memo.base == base;
+    if (!planned) {
+        hipLaunchKernelGGL(hub_count_kernel, dim3(nb), dim3(kBlock), 0, s, m, row_ptr, bh, bc);
+        hipLaunchKernelGGL(hub_scan_kernel, dim3(1), dim3(kScanBlock), 0, s, nb, bh, bc, counts);
+        hipLaunchKernelGGL(hub_fill_kernel, dim3(nb), dim3(kBlock), 0, s, m, row_ptr, bh, bc, hub_cap, chunk_cap, row_slot,
+                           hub_row, hub_chunk0, chunk_hub);
+        memo = Memo{s, row_ptr, m, n, nnz, base};
+    }
     if (vec4) {
         if (iters <= 1) launch_partial_combine<4, 1>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
         else if (iters == 2) launch_partial_combine<4, 2>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);

@@ -32,8 +32,6 @@
 namespace gnnhip {
 
 // spmm.hip
-int spmm_dispatch(int m, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                  const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s);
 // input_wide.hip
 int input_wide_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s);
 // level_wide.hip
@@ -558,8 +556,10 @@ int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float
 }
 
 int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-                   const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
+                   const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph)
 {
+    // same_graph: the previous call on this stream had the same A (a later level of one forward), so the
+    // plan of the long-row pass is still in place and only its sums are redone
     if (!(aligned16(h_in) && aligned16(W) && aligned16(h_out) && (!msg || aligned16(msg)) && (!bias || aligned16(bias))))
         return GNNHIP_EUNSUPPORTED;
     if (C == 16 || C == 32 || C == 64) {
@@ -572,7 +572,7 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
         // kTwoStepMeanDegree entries per row take the two launches.
         const bool two_step = N >= kHubMinRows && nnz >= two_step_degree() * (long long)N;
         if (two_step) {
-            if (int rc = spmm_dispatch(N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, h_out, C, s)) return rc;
+            if (int rc = spmm_dispatch(N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, h_out, C, s, same_graph)) return rc;
             const HubPlan none{nullptr, nullptr, 0};
             switch (C) {
             case 16: return launch_level<16, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, none, s);
@@ -581,7 +581,7 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
             }
         }
         HubPlan hubs{nullptr, nullptr, 0};
-        if (int rc = hub_prepass(N, C, nnz, row_ptr, col_idx, val, h_in, C, s, &hubs)) return rc;
+        if (int rc = hub_prepass(N, C, nnz, row_ptr, col_idx, val, h_in, C, s, &hubs, same_graph)) return rc;
         switch (C) {
         case 16: return launch_level<16, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
         case 32: return launch_level<32, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);

@@ -223,7 +223,7 @@ int launch_slab(int m, int n, float alpha, const int* row_ptr, const int* col_id
 
 // Shared with the fused forward: C = alpha*A*B + beta*C on stream s.
 int spmm_dispatch(int m, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                  const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s)
+                  const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
 {
     const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && aligned16(B) && aligned16(C);
     const int vec = vec4 ? 4 : 1;
@@ -239,7 +239,7 @@ int spmm_dispatch(int m, int n, long long nnz, float alpha, const int* row_ptr, 
         float* Cs = C + col0;
         int rc;
         HubPlan hubs;
-        if ((rc = hub_prepass(m, w, nnz, row_ptr, col_idx, val, Bs, ldb, s, &hubs))) return rc;
+        if ((rc = hub_prepass(m, w, nnz, row_ptr, col_idx, val, Bs, ldb, s, &hubs, reuse_plan && n <= slab_max))) return rc;
         if (vec4) {
             if (iters <= 1) rc = launch_slab<4, 1>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
             else if (iters == 2) rc = launch_slab<4, 2>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
