@@ -32,6 +32,10 @@
 namespace gnnhip {
 
 // spmm.hip
+// level_stream.hip
+int level_stream_dispatch(int N, int C, bool dense, const int* row_ptr, const int* col_idx, const float* val,
+                          const float* h_in, const float* W, const float* msg, const float* bias, float* h_out,
+                          const HubPlan& hubs, hipStream_t s);
 // input_wide.hip
 int input_wide_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s);
 // level_wide.hip
@@ -212,7 +216,34 @@ __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
 
     const long long ntiles = ((long long)N + 15) / 16;
     const long long wave_stride = (long long)gridDim.x * kWavesPerBlock;
-    for (long long tile_id = (long long)blockIdx.x * kWavesPerBlock + wave; tile_id < ntiles; tile_id += wave_stride) {
+    const long long tile_first = (long long)blockIdx.x * kWavesPerBlock + wave;
+
+    // The CSR data of a tile is asked for one tile ahead (its first batch of column indices and
+    // weights) and two tiles ahead (its 17 row pointers), so that a tile's chain of dependent
+    // memory trips is the gather alone.  Tiles past the end read row_ptr[N] 17 times: empty rows.
+    auto load_rp = [&](long long tid) -> int {
+        int r = 0;
+        const long long rr = tid * 16 + lane;
+        if (!DENSE && lane <= 16) r = row_ptr[rr < (long long)N ? rr : (long long)N];
+        return r;
+    };
+    int c0n[ROUNDS];
+    float v0n[ROUNDS];
+    auto load_first_batch = [&](int rp) {
+#pragma unroll
+        for (int rd = 0; rd < ROUNDS; ++rd) {
+            const int lr = rd * RPR + grp;
+            const int s0 = __shfl(rp, lr, kWave), e0 = __shfl(rp, lr + 1, kWave);
+            c0n[rd] = 0;
+            v0n[rd] = 0.f;
+            if (!DENSE && e0 - s0 <= kWaveLongRow && s0 + tx < e0) { c0n[rd] = col_idx[s0 + tx]; v0n[rd] = val[s0 + tx]; }
+        }
+    };
+    int rp_cur = load_rp(tile_first);
+    int rp_nxt = load_rp(tile_first + wave_stride);
+    if (!DENSE) load_first_batch(rp_cur);
+
+    for (long long tile_id = tile_first; tile_id < ntiles; tile_id += wave_stride) {
         const long long row0 = tile_id * 16;
         // msg of this tile is asked for first, so its trip to memory runs under the gather and the
         // contraction instead of after them
@@ -231,10 +262,7 @@ __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
                 *reinterpret_cast<float4*>(tile + lr * LDT + tx * 4) = x;
             }
         } else {
-            // one coalesced load of the 17 row pointers of this tile
-            int rp = 0;
-            if (lane <= 16) rp = row_ptr[min(row0 + lane, (long long)N)];
-
+            const int rp = rp_cur;
             int st[ROUNDS], en[ROUNDS], c0[ROUNDS];
             float v0[ROUNDS];
             bool is_long[ROUNDS];
@@ -251,24 +279,25 @@ __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
                     if (hub[rd] >= 0) is_long[rd] = false;
                     en[rd] = st[rd];
                 }
-                c0[rd] = 0;
-                v0[rd] = 0.f;
-                if (st[rd] + tx < en[rd]) { c0[rd] = col_idx[st[rd] + tx]; v0[rd] = val[st[rd] + tx]; }
+                c0[rd] = c0n[rd];
+                v0[rd] = v0n[rd];
             }
 
             // ---- gather-sum; the first four neighbours of every row of the tile are fetched together
             float4 x[ROUNDS][4];
-            float vv[ROUNDS][4];
 #pragma unroll
             for (int rd = 0; rd < ROUNDS; ++rd) {
                 const int cnt = en[rd] - st[rd];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int cj = __shfl(c0[rd], u & (G - 1), G);
-                    vv[rd][u] = __shfl(v0[rd], u & (G - 1), G);
                     x[rd][u] = (u < cnt && u < G) ? *reinterpret_cast<const float4*>(h_in + (size_t)cj * C + tx * 4) : f4_zero();
                 }
             }
+            // the next tile's first batch and the row pointers of the tile after it, behind the gathers
+            rp_cur = rp_nxt;
+            rp_nxt = load_rp(tile_id + 2 * wave_stride);
+            load_first_batch(rp_cur);
 #pragma unroll
             for (int rd = 0; rd < ROUNDS; ++rd) {
                 const int lr = rd * RPR + grp;
@@ -276,7 +305,7 @@ __global__ __launch_bounds__(kBlock) void s2v_level_kernel(
                 float4 acc = f4_zero();
 #pragma unroll
                 for (int u = 0; u < 4; ++u)
-                    if (u < cnt_all && u < G) f4_fma(acc, vv[rd][u], x[rd][u]);
+                    if (u < cnt_all && u < G) f4_fma(acc, __shfl(v0[rd], u & (G - 1), G), x[rd][u]);
                 // the rest of the row: entries 4.. of the first batch, then further batches of G
                 for (int base = st[rd]; base < en[rd]; base += G) {
                     int c = c0[rd];
@@ -574,6 +603,9 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
         if (two_step) {
             if (int rc = spmm_dispatch(N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, h_out, C, s, same_graph)) return rc;
             const HubPlan none{nullptr, nullptr, 0};
+            if (int rc = level_stream_dispatch(N, C, true, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, none, s);
+                rc != GNNHIP_EUNSUPPORTED)
+                return rc;
             switch (C) {
             case 16: return launch_level<16, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, none, s);
             case 32: return launch_level<32, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, none, s);
@@ -582,6 +614,10 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
         }
         HubPlan hubs{nullptr, nullptr, 0};
         if (int rc = hub_prepass(N, C, nnz, row_ptr, col_idx, val, h_in, C, s, &hubs, same_graph)) return rc;
+        // activations of 4 GiB and more keep the kernel with 64-bit addressing below
+        if (int rc = level_stream_dispatch(N, C, false, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
+            rc != GNNHIP_EUNSUPPORTED)
+            return rc;
         switch (C) {
         case 16: return launch_level<16, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
         case 32: return launch_level<32, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
