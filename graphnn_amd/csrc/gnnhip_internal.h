@@ -148,12 +148,8 @@ int stream_scratch(hipStream_t s, size_t bytes, void** p);
 // The same with several independent buffers per stream (slot 0 is stream_scratch's):
 // slot 1 holds the hub pre-pass results, which must outlive a consumer that itself
 // takes slot 0.
-constexpr int kScratchSlots = 3;
+constexpr int kScratchSlots = 2;
 int stream_scratch_slot(hipStream_t s, int slot, size_t bytes, void** p);
-// count counters per stream (slot 2, at most 16384), zero when first handed out.  A kernel that uses them
-// leaves them zero when it ends, so launches ordered on one stream can share them without a memset in
-// between.
-int stream_counters(hipStream_t s, int count, int** p);
 
 // ---- high-degree rows (hub.hip)
 constexpr int kHubThreshold = 64;      // rows with more entries are summed by the pre-pass

@@ -45,7 +45,6 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
-constexpr int kQueues = 32;          // tile counters of a launch
 constexpr int kWaveLongRow = 48;     // entries; longer rows are gathered by all groups of the wavefront together,
                                      // and past kHubThreshold they come from the pre-pass when there is one
 
@@ -89,7 +88,7 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
     int N, const int* __restrict__ row_ptr, const int* __restrict__ col_idx, const float* __restrict__ val,
     const float* __restrict__ h_in, const float* __restrict__ W, const float* __restrict__ msg,
     const float* __restrict__ bias, float* __restrict__ h_out,
-    const int* __restrict__ hub_slot, const float* __restrict__ hub_agg, int hub_ld, int* __restrict__ queue)
+    const int* __restrict__ hub_slot, const float* __restrict__ hub_agg, int hub_ld)
 {
     constexpr int G = C / 4;             // lanes per gathered row
     constexpr int RPR = kWave / G;       // lane groups per wavefront
@@ -155,27 +154,9 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
     // byte offset of columns 4 tx .. 4 tx + 3 of row r of an activation matrix
     auto row_off = [&](int r) -> int { return (int)((unsigned)r * (unsigned)kRowBytes + (unsigned)tx_off); };
 
-    // Tiles: a wavefront's first three are fixed (its index, then steps of the number of wavefronts); with a
-    // queue the later ones are drawn from counters, because the hardware serves the oldest wavefront of a
-    // SIMD first and a fixed split would leave the younger ones with work when the older have finished.
-    // Counter p = block % kQueues (one per 256 bytes: a returning atomic on one address completes every
-    // ~9 ns, so one counter for all tiles would take longer than the kernel) hands out the tiles
-    // 3 nwaves + p, + kQueues, ...; the wavefronts that end up on one SIMD come from blocks 256 apart and
-    // share a counter.  queue[kQueues * 64] counts the wavefronts that have finished.  All counters are
-    // zero at launch and the last wavefront to finish sets them back to zero.
     const int ntiles = (N + 15) / 16;
     const int nwaves = (int)gridDim.x * kWavesPerBlock;
     const int tile_first = (int)blockIdx.x * kWavesPerBlock + wave;
-    const int part = (int)blockIdx.x % kQueues;
-    auto draw = [&]() -> int {                 // lane 0 counts one tile; without a queue nothing happens
-        // d starts with any value: only lane 0's is read, and only with a queue.  The index hidden in z is 0;
-        // an address the compiler cannot prove uniform keeps it from rewriting the atomic into a form that
-        // waits for the result on the spot.
-        int d, z;
-        asm volatile("v_mov_b32 %1, 0" : "=v"(d), "=v"(z));
-        if (queue && lane == 0) d = atomicAdd(queue + part * 64 + z, 1);
-        return d;
-    };
 
     // Row pointers of the rows grp * ROUNDS .. grp * ROUNDS + ROUNDS of a tile.  Past row N they read 0,
     // which makes those rows empty (their entry counts are not positive).  The whole offset sits in the
@@ -214,11 +195,7 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
         // msg is read, and h_out written, one row per lane group: every instruction covers whole rows.
         // Rows past N are out of range.
         const int out_off = row_off(row0 + grp * ROUNDS);
-        float4 mrow[ROUNDS];
-#pragma unroll
-        for (int rd = 0; rd < ROUNDS; ++rd) mrow[rd] = buf_load4(msg_rsrc, out_off + rd * kRowBytes, 0);
 
-        const int drawn = draw();              // the tile three steps ahead
         if constexpr (DENSE) {
 #pragma unroll
             for (int rd = 0; rd < ROUNDS; ++rd) {
@@ -352,6 +329,10 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
         }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
         GNNHIP_PHASE_ACC(3);
+        // msg is asked for once the gathered rows have left their registers; the contraction covers its trip
+        float4 mrow[ROUNDS];
+#pragma unroll
+        for (int rd = 0; rd < ROUNDS; ++rd) mrow[rd] = buf_load4(msg_rsrc, out_off + rd * kRowBytes, 0);
 
         // ---- contraction: lane (q, t) supplies tile[t][KS q + s] at step s
         float areg[KS];
@@ -397,13 +378,8 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");     // the tile is rewritten by the next iteration
         tile_id = tile_n1;
         tile_n1 = tile_n2;
-        tile_n2 = queue ? 3 * nwaves + __builtin_amdgcn_readfirstlane(drawn) * kQueues + part : tile_n2 + nwaves;
+        tile_n2 += nwaves;
         GNNHIP_PHASE_ACC(5);
-    }
-    if (queue && lane == 0) {
-        if (atomicAdd(queue + kQueues * 64, 1) == nwaves - 1) {           // every wavefront has drawn its last tile
-            for (int i = 0; i <= kQueues; ++i) __hip_atomic_store(queue + i * 64, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
     }
     GNNHIP_PHASE_FINI
 }
@@ -416,15 +392,11 @@ int launch_level_stream(int N, const int* row_ptr, const int* col_idx, const flo
     const long long ntiles = ((long long)N + 15) / 16;
     long long blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
     constexpr bool kWLds = (C == 64);
-    constexpr int kMinW = (C == 64) ? (DENSE ? 4 : 3) : 4;
+    constexpr int kMinW = (C == 64 && !DENSE) ? 3 : 4;    // hidden 64 needs 128 registers and spills for four
     const long long resident = (long long)kNumCU * kMinW;  // a workgroup puts one wavefront on each SIMD
     if (blocks > resident) blocks = resident;              // persistent beyond this
-    // with more than three tiles per wavefront the later ones are handed out through a counter
-    int* queue = nullptr;
-    if (ntiles > 3 * blocks * kWavesPerBlock)
-        if (int rc = stream_counters(s, (kQueues + 1) * 64, &queue)) return rc;
     hipLaunchKernelGGL((s2v_level_stream_kernel<C, DENSE, kWLds, kMinW>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
-                       N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs.row_slot, hubs.agg, hubs.ld, queue);
+                       N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs.row_slot, hubs.agg, hubs.ld);
     GNNHIP_LAUNCH_CHECK("s2v_level_stream");
     return GNNHIP_OK;
 }

@@ -149,29 +149,10 @@ int stream_scratch_slot(hipStream_t s, int which, size_t bytes, void** p)
             (void)hipStreamSynchronize(s);
             (void)hipFree(slot.first);
         }
-        if (which == 2) {
-            // counters start at zero; a blocking memset, once per stream
-            e = hipMemset(q, 0, want);
-            if (e != hipSuccess) {
-                (void)hipFree(q);
-                return set_error(GNNHIP_EHIP, "hipMemset of the stream counters failed: %s", hipGetErrorString(e));
-            }
-        }
         slot.first = q;
         slot.second = want;
     }
     *p = slot.first;
-    return GNNHIP_OK;
-}
-
-int stream_counters(hipStream_t s, int count, int** p)
-{
-    // one allocation for the life of the stream: a second one would not inherit the zeros
-    constexpr int kMaxCounters = 16384;
-    if (count < 0 || count > kMaxCounters) return set_error(GNNHIP_EINVAL, "too many stream counters (%d)", count);
-    void* q = nullptr;
-    if (int rc = stream_scratch_slot(s, 2, kMaxCounters * sizeof(int), &q)) return rc;
-    *p = static_cast<int*>(q);
     return GNNHIP_OK;
 }
 

@@ -31,6 +31,7 @@ struct FusedStep
     enum Tag { SINGLE, INPUT, LEVEL, FORWARD } tag = SINGLE;
     std::vector<size_t> vars;               // INPUT: X, W, msg, h0;  LEVEL: A, h_in, W, msg, h_out
 };
+constexpr size_t kOneLaunchMaxNodes = 20000;   // larger batches run the forward as separate kernels
 }  // namespace detail
 
 inline size_t FactorGraph::LastPlanFactorCount() const { return last_plan ? last_plan->steps.size() : 0; }
@@ -324,7 +325,10 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
         SVar *A = sparse(vA), *S = sparse(vS);
         step->run = [=](Phase ph) {
             bool done = false;
-            if (n2n->block_diagonal && sub->contiguous_subgraphs && sub->max_subgraph_nodes > 0) {
+            // Past about 20,000 nodes the chip is full either way and the separate kernels are faster
+            // (1,000 graphs of configuration 2: 62 us against 70 us in one launch; 256 graphs: 40 against 23).
+            if (n2n->block_diagonal && sub->contiguous_subgraphs && sub->max_subgraph_nodes > 0 &&
+                X->value.rows() <= detail::kOneLaunchMaxNodes) {
                 const size_t N = X->value.rows(), K = X->value.cols(), C = Wn->value.cols(), H = W1->value.cols(),
                              Q = W2->value.cols(), B = S->value.rows();
                 ASSERT(Wn->value.rows() == K && Wc->value.rows() == C && Wc->value.cols() == C && W1->value.rows() == C &&
