@@ -135,3 +135,30 @@ def test_skewed_configuration_5_properties(gpu):
     pool = ops.spmm(s_rp, torch.arange(N, device=gpu).int(), torch.ones(N, device=gpu), out, B)
     want_pool = out.view(B, 1024, C).double().sum(dim=1)
     assert float((pool.double() - want_pool).abs().max()) <= 1e-4 * float(want_pool.abs().max())
+
+
+def test_level_past_4_gib_of_activations(gpu):
+    """16.8M nodes at hidden 64: each of h_in, msg and h_out spans 4 GiB, past the reach of the 32-bit buffer
+    offsets of the streaming level kernel, so the kernel with 64-bit addressing runs.  Ring graph with
+    weights (every node sums its two neighbours); sampled rows against float64, the rows at both ends of
+    the address range included."""
+    import torch
+    from graphnn_amd import ops
+    n, c = (1 << 24) + 48, 64
+    assert n * c * 4 >= 0xFFFF0000
+    idx = torch.arange(n, device=gpu, dtype=torch.int64)
+    ci = torch.stack(((idx - 1) % n, (idx + 1) % n), dim=1).to(torch.int32).reshape(-1).contiguous()
+    rp = (2 * torch.arange(n + 1, device=gpu, dtype=torch.int64)).to(torch.int32)
+    g = torch.Generator(device=gpu); g.manual_seed(24)
+    val = torch.rand((2 * n,), generator=g, device=gpu) + 0.5
+    h = torch.rand((n, c), generator=g, device=gpu)
+    msg = torch.randn((n, c), generator=g, device=gpu)
+    W = torch.randn((c, c), generator=g, device=gpu) * 0.1
+    out = ops.s2v_level(rp, ci, val, h, W, msg)
+    rows = torch.cat((torch.arange(0, 40, device=gpu), torch.arange(n - 40, n, device=gpu),
+                      torch.randint(0, n, (2000,), device=gpu, generator=g)))
+    left, right = (rows - 1) % n, (rows + 1) % n
+    agg = val[2 * rows].double()[:, None] * h[left].double() + val[2 * rows + 1].double()[:, None] * h[right].double()
+    want = torch.relu(agg @ W.double() + msg[rows].double())
+    got = out[rows].double()
+    assert float((got - want).abs().max()) <= PARITY_TOL * max(1.0, float(want.abs().max()))
