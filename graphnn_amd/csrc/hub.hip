@@ -10,9 +10,12 @@
 //
 //   count   per 1024 rows: number of hubs and of their chunks (kHubChunk entries each)
 //   scan    exclusive scan of those counts by one workgroup -> slots of hubs and chunks
+//           (only past kFillScanBlocks workgroups; below that every workgroup of fill adds up the
+//           counts before its own)
 //   fill    row_slot[row] (written for hubs only), per hub its first chunk, per chunk its hub
-//   partial one wavefront per chunk: part[chunk][n] = sum of val * B[col, :] over the chunk
-//   combine one lane group per hub: agg[slot][n] = sum of its chunks' partials in chunk order
+//   partial one wavefront per chunk: sum of val * B[col, :] over the chunk; a hub of one chunk is
+//           finished with that, for a longer one the wavefront that delivers the last chunk adds the
+//           chunks' sums in chunk order: agg[slot][n]
 //
 // The consumer reads agg[row_slot[row]] for a row whose length exceeds the
 // threshold.  Every sum is taken in an order fixed by the matrix structure, so the
@@ -26,6 +29,7 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kRowsPerBlock = 1024;          // count / fill: four consecutive rows per lane
 constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kFillScanBlocks = 4096;       // up to this many workgroups (4M rows) fill does the scan itself
 
 __device__ __forceinline__ int hub_chunks(int deg) { return (deg + kHubChunk - 1) / kHubChunk; }
 
@@ -109,13 +113,41 @@ __global__ __launch_bounds__(kScanBlock) void hub_scan_kernel(int nb, int* __res
     if (tid == kScanBlock - 1) { counts[0] = rh; counts[1] = rc; }
 }
 
-__global__ __launch_bounds__(kBlock) void hub_fill_kernel(int m, const int* __restrict__ row_ptr,
+// SCAN: block_hubs / block_chunks hold the raw counts of hub_count_kernel and every workgroup adds up
+// the entries before its own (few workgroups); otherwise they hold the exclusive scan already.
+template <bool SCAN>
+__global__ __launch_bounds__(kBlock) void hub_fill_kernel(int m, int nb, const int* __restrict__ row_ptr,
                                                            const int* __restrict__ block_hubs, const int* __restrict__ block_chunks,
                                                            int hub_cap, int chunk_cap, int* __restrict__ row_slot,
                                                            int* __restrict__ hub_row, int* __restrict__ hub_chunk0,
-                                                           int* __restrict__ chunk_hub)
+                                                           int* __restrict__ chunk_hub, int* __restrict__ hub_done,
+                                                           int* __restrict__ counts)
 {
     __shared__ int sh[kWavesPerBlock];
+    __shared__ int base_sh[2];
+    int slot0, chunk0;
+    if (SCAN) {
+        int h = 0, c = 0;
+        for (int i = threadIdx.x; i < (int)blockIdx.x; i += kBlock) { h += block_hubs[i]; c += block_chunks[i]; }
+        h = wave_sum_i(h);
+        c = wave_sum_i(c);
+        __shared__ int part_sh[2][kWavesPerBlock];
+        if ((threadIdx.x & (kWave - 1)) == 0) { part_sh[0][threadIdx.x / kWave] = h; part_sh[1][threadIdx.x / kWave] = c; }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int hh = 0, cc = 0;
+            for (int w = 0; w < kWavesPerBlock; ++w) { hh += part_sh[0][w]; cc += part_sh[1][w]; }
+            base_sh[0] = hh;
+            base_sh[1] = cc;
+            if ((int)blockIdx.x == nb - 1) { counts[0] = hh + block_hubs[blockIdx.x]; counts[1] = cc + block_chunks[blockIdx.x]; }
+        }
+        __syncthreads();
+        slot0 = base_sh[0];
+        chunk0 = base_sh[1];
+    } else {
+        slot0 = block_hubs[blockIdx.x];
+        chunk0 = block_chunks[blockIdx.x];
+    }
     const long long r0 = (long long)blockIdx.x * kRowsPerBlock + threadIdx.x * 4;
     int deg[4];
     int hubs = 0, chunks = 0;
@@ -127,8 +159,8 @@ __global__ __launch_bounds__(kBlock) void hub_fill_kernel(int m, const int* __re
         if (deg[i] > kHubThreshold) { ++hubs; chunks += hub_chunks(deg[i]); }
     }
     int tot;
-    int slot = block_hubs[blockIdx.x] + block_exclusive_scan(hubs, sh, &tot);
-    int chunk = block_chunks[blockIdx.x] + block_exclusive_scan(chunks, sh, &tot);
+    int slot = slot0 + block_exclusive_scan(hubs, sh, &tot);
+    int chunk = chunk0 + block_exclusive_scan(chunks, sh, &tot);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         if (deg[i] > kHubThreshold) {
@@ -139,8 +171,9 @@ __global__ __launch_bounds__(kBlock) void hub_fill_kernel(int m, const int* __re
             if (fits) {
                 hub_row[slot] = (int)(r0 + i);
                 hub_chunk0[slot] = chunk;
-                for (int j = 0; j < nc; ++j) chunk_hub[chunk + j] = slot;
+                hub_done[slot] = 0;
             }
+            for (int j = 0; j < nc && chunk + j < chunk_cap; ++j) chunk_hub[chunk + j] = fits ? slot : -1;
             ++slot;
             chunk += nc;
         }
@@ -173,7 +206,7 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
     const int* __restrict__ counts, int chunk_cap, int n, const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
     const float* __restrict__ val, const float* __restrict__ B, int ldb, int logG,
     const int* __restrict__ hub_row, const int* __restrict__ hub_chunk0, const int* __restrict__ chunk_hub,
-    float* __restrict__ part, int ldp)
+    float* part, int ldp, float* __restrict__ agg, int* hub_done)
 {
     using V = HV<VEC>;
     __shared__ float red[kWavesPerBlock][kWave * VEC * ITERS];
@@ -183,8 +216,10 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
     const int nchunks = min(counts[1], chunk_cap);
     for (int c = blockIdx.x * kWavesPerBlock + wave; c < nchunks; c += gridDim.x * kWavesPerBlock) {
         const int slot = chunk_hub[c];
+        if (slot < 0) continue;                  // chunk of a hub that did not fit the buffers
         const int row = hub_row[slot];
         const int rb = row_ptr[row], re = row_ptr[row + 1];
+        const int nc = hub_chunks(re - rb);
         const int cb = rb + (c - hub_chunk0[slot]) * kHubChunk;
         const int ce = min(cb + kHubChunk, re);
         typename V::T acc[ITERS];
@@ -220,6 +255,7 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) V::store(red[wave] + grp * width + (sub + it * G) * VEC, acc[it]);
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        float* dst = (nc == 1) ? agg + (size_t)slot * ldp : part + (size_t)c * ldp;
         if (grp == 0) {
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
@@ -227,36 +263,41 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
                 if (col0 < n) {
                     typename V::T s = V::zero();
                     for (int g = 0; g < ngroups; ++g) s = V::add(s, V::load(red[wave] + g * width + col0));
-                    V::store(part + (size_t)c * ldp + col0, s);
+                    V::store(dst + col0, s);
                 }
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-    }
-}
-
-// One lane group per hub: agg[slot] = sum over its chunks, in chunk order.
-template <int VEC, int ITERS>
-__global__ __launch_bounds__(kBlock) void hub_combine_kernel(
-    const int* __restrict__ counts, int hub_cap, int chunk_cap, int n, const int* __restrict__ row_ptr, int logG,
-    const int* __restrict__ hub_row, const int* __restrict__ hub_chunk0,
-    const float* __restrict__ part, int ldp, float* __restrict__ agg)
-{
-    using V = HV<VEC>;
-    const int G = 1 << logG, sub = threadIdx.x & (G - 1), grp = threadIdx.x >> logG, ngroups = kBlock >> logG;
-    const int nhubs = min(counts[0], hub_cap);
-    for (int slot = blockIdx.x * ngroups + grp; slot < nhubs; slot += gridDim.x * ngroups) {
-        const int row = hub_row[slot];
-        const int deg = row_ptr[row + 1] - row_ptr[row];
-        const int c0 = hub_chunk0[slot], nc = hub_chunks(deg);
-        if (c0 + nc > chunk_cap) continue;       // never written by fill (slot -1 for the consumer)
+        if (nc > 1) {
+            // The wavefront that delivers the last chunk of the hub adds the chunks' sums, always in chunk
+            // order.  Release: this chunk's sum is visible before the count; acquire: the other sums are
+            // read from L2 after the count said they are there.
+            __threadfence();
+            int last = 0;
+            if (lane == 0) last = (atomicAdd(hub_done + slot, 1) == nc - 1);
+            last = __shfl(last, 0, kWave);
+            if (last) {
+                __threadfence();
+                const int c0 = hub_chunk0[slot];
+                if (grp == 0) {
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            const int col0 = (sub + it * G) * VEC;
-            if (col0 < n) {
-                typename V::T s = V::zero();
-                for (int j = 0; j < nc; ++j) s = V::add(s, V::load(part + (size_t)(c0 + j) * ldp + col0));
-                V::store(agg + (size_t)slot * ldp + col0, s);
+                    for (int it = 0; it < ITERS; ++it) {
+                        const int col0 = (sub + it * G) * VEC;
+                        if (col0 < n) {
+                            float sum[VEC];
+#pragma unroll
+                            for (int e = 0; e < VEC; ++e) sum[e] = 0.f;
+                            for (int j = 0; j < nc; ++j)
+#pragma unroll
+                                for (int e = 0; e < VEC; ++e)
+                                    sum[e] += __hip_atomic_load(part + (size_t)(c0 + j) * ldp + col0 + e, __ATOMIC_RELAXED,
+                                                                __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                            for (int e = 0; e < VEC; ++e) agg[(size_t)slot * ldp + col0 + e] = sum[e];
+                        }
+                    }
+                }
+                if (lane == 0) __hip_atomic_store(hub_done + slot, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next pass over this plan
             }
         }
     }
@@ -272,15 +313,13 @@ inline int ilog2_ceil_(int x)
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 template <int VEC, int ITERS>
-void launch_partial_combine(hipStream_t s, const int* counts, int hub_cap, int chunk_cap, int n, const int* row_ptr,
-                            const int* col_idx, const float* val, const float* B, int ldb, int logG, const int* hub_row,
-                            const int* hub_chunk0, const int* chunk_hub, float* part, int ldp, float* agg)
+void launch_partial(hipStream_t s, const int* counts, int chunk_cap, int n, const int* row_ptr, const int* col_idx,
+                    const float* val, const float* B, int ldb, int logG, const int* hub_row, const int* hub_chunk0,
+                    const int* chunk_hub, float* part, int ldp, float* agg, int* hub_done)
 {
     const unsigned grid = kNumCU * 8;
     hipLaunchKernelGGL((hub_partial_kernel<VEC, ITERS>), dim3(grid), dim3(kBlock), 0, s, counts, chunk_cap, n, row_ptr,
-                       col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp);
-    hipLaunchKernelGGL((hub_combine_kernel<VEC, ITERS>), dim3(kNumCU * 2), dim3(kBlock), 0, s, counts, hub_cap, chunk_cap, n,
-                       row_ptr, logG, hub_row, hub_chunk0, part, ldp, agg);
+                       col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
 }
 
 }  // namespace
@@ -289,7 +328,7 @@ void launch_partial_combine(hipStream_t s, const int* counts, int hub_cap, int c
 // n <= 1024.  The buffers live in the stream's plan scratch and stay valid until the next
 // hub_prepass on the same stream.
 // reuse_plan: the caller guarantees that the structure of A has not changed since the previous call on
-// this stream with the same arguments (the levels of one forward); the three planning launches
+// this stream with the same arguments (the levels of one forward); the planning launches
 // (count, scan, fill) are then skipped and only the sums are recomputed.
 int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
                 const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan)
@@ -319,6 +358,7 @@ int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_
     const size_t o_slot = carve(sizeof(int) * (size_t)m);
     const size_t o_hrow = carve(sizeof(int) * (size_t)hub_cap), o_hc0 = carve(sizeof(int) * (size_t)hub_cap);
     const size_t o_chub = carve(sizeof(int) * (size_t)chunk_cap);
+    const size_t o_done = carve(sizeof(int) * (size_t)hub_cap);
     const size_t o_part = carve(sizeof(float) * (size_t)chunk_cap * ldp);
     const size_t o_agg = carve(sizeof(float) * (size_t)hub_cap * ldp);
     void* base = nullptr;
@@ -331,6 +371,7 @@ int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_
     int* hub_row = reinterpret_cast<int*>(b + o_hrow);
     int* hub_chunk0 = reinterpret_cast<int*>(b + o_hc0);
     int* chunk_hub = reinterpret_cast<int*>(b + o_chub);
+    int* hub_done = reinterpret_cast<int*>(b + o_done);
     float* part = reinterpret_cast<float*>(b + o_part);
     float* agg = reinterpret_cast<float*>(b + o_agg);
 
@@ -340,19 +381,24 @@ int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_
                          memo.nnz == nnz && memo.base == base;
     if (!planned) {
         hipLaunchKernelGGL(hub_count_kernel, dim3(nb), dim3(kBlock), 0, s, m, row_ptr, bh, bc);
-        hipLaunchKernelGGL(hub_scan_kernel, dim3(1), dim3(kScanBlock), 0, s, nb, bh, bc, counts);
-        hipLaunchKernelGGL(hub_fill_kernel, dim3(nb), dim3(kBlock), 0, s, m, row_ptr, bh, bc, hub_cap, chunk_cap, row_slot,
-                           hub_row, hub_chunk0, chunk_hub);
+        if (nb <= kFillScanBlocks) {
+            hipLaunchKernelGGL(hub_fill_kernel<true>, dim3(nb), dim3(kBlock), 0, s, m, nb, row_ptr, bh, bc, hub_cap, chunk_cap,
+                               row_slot, hub_row, hub_chunk0, chunk_hub, hub_done, counts);
+        } else {
+            hipLaunchKernelGGL(hub_scan_kernel, dim3(1), dim3(kScanBlock), 0, s, nb, bh, bc, counts);
+            hipLaunchKernelGGL(hub_fill_kernel<false>, dim3(nb), dim3(kBlock), 0, s, m, nb, row_ptr, bh, bc, hub_cap, chunk_cap,
+                               row_slot, hub_row, hub_chunk0, chunk_hub, hub_done, counts);
+        }
         memo = Memo{s, row_ptr, m, n, nnz, base};
     }
     if (vec4) {
-        if (iters <= 1) launch_partial_combine<4, 1>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
-        else if (iters == 2) launch_partial_combine<4, 2>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
-        else launch_partial_combine<4, 4>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
+        if (iters <= 1) launch_partial<4, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
+        else if (iters == 2) launch_partial<4, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
+        else launch_partial<4, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
     } else {
-        if (iters <= 1) launch_partial_combine<1, 1>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
-        else if (iters == 2) launch_partial_combine<1, 2>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
-        else launch_partial_combine<1, 4>(s, counts, hub_cap, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg);
+        if (iters <= 1) launch_partial<1, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
+        else if (iters == 2) launch_partial<1, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
+        else launch_partial<1, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
     }
     GNNHIP_LAUNCH_CHECK("hub_prepass");
     plan->row_slot = row_slot;
