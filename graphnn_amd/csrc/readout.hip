@@ -1,0 +1,177 @@
+// Readout of batches of many small graphs, one wavefront per graph:
+//     pool = S * h ; hidden = ReLU(pool * W_h1) ; logits = hidden * W_h2 ;
+//     probs = softmax(logits) ; pred = argmax(logits)
+// (MatMul(S, h) -> MatMul -> ReLU -> MatMul of examples/graph_classification/src/kernel_mean_field.cpp:45-49,
+// row softmax of src/tensor/gpu_dense_tensor.cu:298-370, arg-max with the lowest index winning ties as in
+// src/tensor/cpu_dense_tensor.cpp:176-196.)
+//
+// W_h1 and W_h2 are copied into LDS once per workgroup.  A wavefront then takes graphs g, g + nwaves, ...
+// and never synchronises with the other wavefronts of its workgroup:
+//   1. sum-pool: G = C/4 lanes take one row of h as float4s; the 64/G lane groups walk the graph's rows
+//      four at a time each, their sums are added in group order through LDS;
+//   2. hidden: lane j adds pool[c] * W_h1[c][j] over c in order (pool broadcast from LDS, W_h1 rows read by
+//      consecutive lanes);
+//   3. logits the same way over the hidden units, then softmax and arg-max inside the wavefront.
+// Hidden sizes 16 to 256.  Algorithmic bytes: 4NC (h) + 8N (S) + 4B(C + H + 2Q) + 4(CH + HQ).
+#include "gnnhip_internal.h"
+#include <math.h>
+
+namespace gnnhip {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kMaxLds = 150 * 1024;
+
+template <int C>
+__global__ __launch_bounds__(kBlock) void s2v_readout_wave_kernel(
+    int B, int H, int Q, const int* __restrict__ s_row_ptr, const int* __restrict__ s_col_idx,
+    const float* __restrict__ s_val, const float* __restrict__ h, const float* __restrict__ Wh1,
+    const float* __restrict__ Wh2, float* __restrict__ pool, float* __restrict__ hidden,
+    float* __restrict__ logits, float* __restrict__ probs, int* __restrict__ pred)
+{
+    constexpr int G = C / 4;             // lanes per row of h
+    constexpr int RPR = kWave / G;       // rows in flight per step of the wavefront
+    extern __shared__ float smem[];
+    float* w1 = smem;                    // [C][H]
+    float* w2 = w1 + (size_t)C * H;      // [H][Q]
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int per_wave = RPR * C + C + H + Q;
+    float* part = w2 + (size_t)H * Q + (size_t)wave * per_wave;   // [RPR][C]
+    float* pl = part + RPR * C;          // [C]
+    float* hid = pl + C;                 // [H]
+    float* lg = hid + H;                 // [Q]
+    const int grp = lane / G, tx = lane % G;
+
+    for (int i = threadIdx.x; i < C * H; i += kBlock) w1[i] = Wh1[i];
+    for (int i = threadIdx.x; i < H * Q; i += kBlock) w2[i] = Wh2[i];
+    __syncthreads();
+
+    const int nwaves = (int)gridDim.x * kWavesPerBlock;
+    for (int g = (int)blockIdx.x * kWavesPerBlock + wave; g < B; g += nwaves) {
+        const int start = s_row_ptr[g], end = s_row_ptr[g + 1];
+        // ---- sum-pool
+        float4 acc = f4_zero();
+        int t = start + grp;
+        for (; t + 3 * RPR < end; t += 4 * RPR) {
+            int c[4];
+            float v[4];
+            float4 x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) { c[u] = s_col_idx[t + u * RPR]; v[u] = s_val[t + u * RPR]; }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const float4*>(h + (size_t)c[u] * C + tx * 4);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) f4_fma(acc, v[u], x[u]);
+        }
+        for (; t < end; t += RPR)
+            f4_fma(acc, s_val[t], *reinterpret_cast<const float4*>(h + (size_t)s_col_idx[t] * C + tx * 4));
+        *reinterpret_cast<float4*>(part + grp * C + tx * 4) = acc;
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        for (int cc = lane; cc < C; cc += kWave) {
+            float s = 0.f;
+#pragma unroll
+            for (int p = 0; p < RPR; ++p) s += part[p * C + cc];
+            pl[cc] = s;
+            pool[(size_t)g * C + cc] = s;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        // ---- hidden = ReLU(pool * W_h1)
+        for (int j = lane; j < H; j += kWave) {
+            float s = 0.f;
+#pragma unroll 16
+            for (int cc = 0; cc < C; ++cc) s += pl[cc] * w1[(size_t)cc * H + j];
+            s = relu_ref(s);
+            hid[j] = s;
+            hidden[(size_t)g * H + j] = s;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        // ---- logits = hidden * W_h2
+        for (int q = lane; q < Q; q += kWave) {
+            float s = 0.f;
+#pragma unroll 8
+            for (int j = 0; j < H; ++j) s += hid[j] * w2[(size_t)j * Q + q];
+            lg[q] = s;
+            logits[(size_t)g * Q + q] = s;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        // ---- softmax + argmax over Q
+        if (probs || pred) {
+            const float first = lg[0];
+            float mx = first;                       // the reference scan starts at element 0
+            float bv = -INFINITY;
+            int bi = 0x7fffffff;
+            for (int q = lane; q < Q; q += kWave) {
+                const float v = lg[q];
+                mx = max_keep(mx, v);
+                const float vv = (v != v) ? -INFINITY : v;     // a NaN that is not first never wins
+                argmax_combine(bv, bi, vv, q);
+            }
+            mx = wave_max(mx);
+            wave_argmax(bv, bi);
+            if (first != first) bi = 0;             // a NaN in column 0 is never displaced
+            if (pred && lane == 0) pred[g] = bi;
+            if (probs) {
+                float s = 0.f;
+                for (int q = lane; q < Q; q += kWave) {
+                    const float e = expf(lg[q] - mx);
+                    lg[q] = e;
+                    s += e;
+                }
+                s = wave_sum(s);
+                for (int q = lane; q < Q; q += kWave) probs[(size_t)g * Q + q] = lg[q] / s;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");     // the wavefront's LDS rows are reused by its next graph
+    }
+}
+
+template <int C>
+int launch_readout_wave(int B, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                        const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
+                        float* logits, float* probs, int* pred, hipStream_t s)
+{
+    constexpr int RPR = kWave / (C / 4);
+    const size_t smem = sizeof(float) * ((size_t)C * H + (size_t)H * Q + (size_t)kWavesPerBlock * (RPR * C + C + H + Q));
+    if (smem > (size_t)kMaxLds) return GNNHIP_EUNSUPPORTED;
+    auto kernel = s2v_readout_wave_kernel<C>;
+    if (smem > 64 * 1024) {
+        static bool raised = false;          // per instantiation; the attribute is a property of the function
+        if (!raised) {
+            GNNHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           kMaxLds));
+            raised = true;
+        }
+    }
+    const long long blocks_needed = ((long long)B + kWavesPerBlock - 1) / kWavesPerBlock;
+    const long long per_cu = smem > 0 ? (long long)(160 * 1024) / (long long)smem : 8;
+    long long cap = (long long)kNumCU * (per_cu < 1 ? 1 : (per_cu > 8 ? 8 : per_cu));
+    const unsigned grid = (unsigned)(blocks_needed < cap ? blocks_needed : cap);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBlock), smem, s, B, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2,
+                       pool, hidden, logits, probs, pred);
+    GNNHIP_LAUNCH_CHECK("s2v_readout_wave");
+    return GNNHIP_OK;
+}
+
+}  // namespace
+
+// One wavefront per graph; for batches of many graphs (the caller decides).  Returns GNNHIP_EUNSUPPORTED
+// for hidden sizes it has no kernel for and when W_h1 and W_h2 do not fit LDS.
+int readout_wave_dispatch(int B, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                          const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
+                          float* logits, float* probs, int* pred, hipStream_t s)
+{
+    if (!aligned16(h)) return GNNHIP_EUNSUPPORTED;
+#define GNNHIP_RO_ARGS B, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s
+    switch (C) {
+    case 16: return launch_readout_wave<16>(GNNHIP_RO_ARGS);
+    case 32: return launch_readout_wave<32>(GNNHIP_RO_ARGS);
+    case 64: return launch_readout_wave<64>(GNNHIP_RO_ARGS);
+    case 128: return launch_readout_wave<128>(GNNHIP_RO_ARGS);
+    case 256: return launch_readout_wave<256>(GNNHIP_RO_ARGS);
+    }
+#undef GNNHIP_RO_ARGS
+    return GNNHIP_EUNSUPPORTED;
+}
+
+}  // namespace gnnhip

@@ -406,6 +406,35 @@ def test_readout_stage(gpu, oracle, C, H, Q):
     assert np.array_equal(pred, oracle.row_argmax(logits))      # arg-max of the logits the device produced: exact
 
 
+@pytest.mark.parametrize("C,H,Q,B", [(64, 32, 2, 1500), (16, 8, 3, 1100), (32, 100, 70, 1030), (128, 64, 5, 300), (256, 128, 2, 260)])
+def test_readout_stage_many_graphs(gpu, oracle, C, H, Q, B):
+    """batches of many graphs take the kernel with one wavefront per graph (graphs of 1 to 60 nodes; the
+    subgraph matrix also gets one empty row and weights other than 1)"""
+    from graphnn_amd import ops
+    batch, w, a, s = _small_problem(70 + C, B, 5, C, H, Q, lo=1, hi=60)
+    rp, ci, v = (np.array(x) for x in s)
+    # graph 3 loses its nodes (an empty row of S), and the weights differ from 1
+    lo, hi = int(rp[3]), int(rp[4])
+    keep = np.ones(rp[-1], dtype=bool); keep[lo:hi] = False
+    ci, v = ci[keep], v[keep]
+    rp = rp.copy(); rp[4:] -= (hi - lo)
+    rng = np.random.default_rng(C + H + B)
+    v = (0.5 + rng.random(v.size)).astype(np.float32)
+    s = (rp.astype(np.int32), ci.astype(np.int32), v)
+    h = np.maximum(rng.standard_normal((batch.num_nodes, C)), 0).astype(np.float32)
+    pool, hidden, logits, probs, pred = (_n(t) for t in ops.s2v_readout(*_csr_t(s, gpu), _t(h, gpu), _t(w.W_h1, gpu),
+                                                                        _t(w.W_h2, gpu), batch.num_graphs))
+    w_pool = oracle.spmm(*s, h, batch.num_graphs)
+    w_hidden = np.maximum(oracle.gemm(w_pool, w.W_h1), 0)
+    w_logits = oracle.gemm(w_hidden, w.W_h2)
+    assert np.all(pool[3] == 0) and np.all(logits[3] == 0)
+    assert max_rel(pool, w_pool) < PARITY_TOL
+    assert max_rel(hidden, w_hidden) < PARITY_TOL
+    assert max_rel(logits, w_logits) < PARITY_TOL
+    assert max_rel(probs, oracle.row_softmax(w_logits)) < PARITY_TOL
+    assert np.array_equal(pred, oracle.row_argmax(logits))      # arg-max of the logits the device produced: exact
+
+
 # ------------------------------------------------------------------ whole forward, configurations 1 and 2
 def _forward_case(gpu, oracle, config_id, B=None):
     from graphnn_amd import ops
