@@ -86,8 +86,7 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const float* __restrict__ 
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) dst[i] = src[i];
 }
 
-constexpr int kWaveReadoutMinGraphs = 1024;        // hidden 16..64: below this a workgroup per graph
-constexpr int kWaveReadoutMinGraphsWide = 256;     // hidden 128/256: below this SpMM + GEMM
+constexpr int kWaveReadoutMinGraphs = 1024;        // below this a workgroup per graph
 constexpr int kWaveReadoutMaxMeanNodes = 2048;     // mean nodes per graph
 
 int readout_any(int B, int N, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
@@ -98,8 +97,7 @@ int readout_any(int B, int N, int C, int H, int Q, const int* s_row_ptr, const i
     // a workgroup per graph).  Few graphs: a workgroup per graph reaches more of the chip.  Graphs of
     // thousands of nodes are left to the SpMM, which balances long rows.
     int rc = GNNHIP_EUNSUPPORTED;
-    const bool wide = C > 64;
-    if (B >= (wide ? kWaveReadoutMinGraphsWide : kWaveReadoutMinGraphs) && (long long)N <= (long long)B * kWaveReadoutMaxMeanNodes)
+    if (B >= kWaveReadoutMinGraphs && (long long)N <= (long long)B * kWaveReadoutMaxMeanNodes)
         rc = readout_wave_dispatch(B, C, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
     rc = readout_dispatch(B, C, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);

@@ -408,8 +408,9 @@ def test_readout_stage(gpu, oracle, C, H, Q):
 
 @pytest.mark.parametrize("C,H,Q,B", [(64, 32, 2, 1500), (16, 8, 3, 1100), (32, 100, 70, 1030), (128, 64, 5, 300), (256, 128, 2, 260)])
 def test_readout_stage_many_graphs(gpu, oracle, C, H, Q, B):
-    """batches of many graphs take the kernel with one wavefront per graph (graphs of 1 to 60 nodes; the
-    subgraph matrix also gets one empty row and weights other than 1)"""
+    """batches of many graphs take the kernel with one wavefront per graph (hidden up to 64; wider ones the
+    SpMM and the GEMMs).  Graphs of 1 to 60 nodes; the subgraph matrix also gets one empty row and weights
+    other than 1"""
     from graphnn_amd import ops
     batch, w, a, s = _small_problem(70 + C, B, 5, C, H, Q, lo=1, hi=60)
     rp, ci, v = (np.array(x) for x in s)
