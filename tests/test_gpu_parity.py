@@ -368,6 +368,29 @@ def test_level_stage_hub_rows_and_weights(gpu, oracle):
     assert max_rel(got, want) < PARITY_TOL
 
 
+@pytest.mark.parametrize("C", [16, 32, 64])
+@pytest.mark.parametrize("N", [20_011, 160_007])
+def test_level_every_row_length_up_to_70(gpu, oracle, C, N):
+    """row lengths 0..70 in turn: the boundaries of the streaming level kernel (4 entries fetched at once, 8
+    with the second go, 16 per batch at hidden 64, 48 for one lane group, 64 for the balanced pass, which only
+    the larger matrix gets); the larger matrix also gives every wavefront several tiles, so the look-ahead of
+    row pointers and first batches runs in its steady state; N is not a multiple of the tile"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(C + N)
+    lens = (np.arange(N) * 7) % 71
+    rp = np.zeros(N + 1, np.int32); np.cumsum(lens, out=rp[1:])
+    nnz = int(rp[-1])
+    ci = rng.integers(0, N, nnz).astype(np.int32)
+    v = (rng.random(nnz) * 0.2).astype(np.float32)
+    h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
+    W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
+    msg = rng.standard_normal((N, C)).astype(np.float32)
+    bias = rng.standard_normal(C).astype(np.float32)
+    want = oracle.level(rp, ci, v, h_in, W, msg, bias)
+    got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu), _t(bias, gpu)))
+    assert max_rel(got, want) < PARITY_TOL
+
+
 @pytest.mark.parametrize("C", [128, 256])
 def test_wide_level_ragged_rows_and_weights(gpu, oracle, C):
     """wide-hidden kernel: empty rows, rows longer than one 64-entry index batch, a row count that is
