@@ -7,6 +7,11 @@
 // workgroup, 4 x 4 outputs per lane, K walked in steps of 16 through two LDS
 // tiles.  Edges are handled by bounds-checked tile loads (zeros) and stores.
 // Bound: HBM for the shapes above; algorithmic bytes 4(mk + kn + mn).
+//
+// Weight gradients are the opposite shape: op(A)^T * G with a small output (hidden x hidden) and k = nodes.
+// One output tile would walk all of k on one CU (1.1 ms at k = 7,450), so such products are split along k:
+// every workgroup takes a range of k, writes its partial tile to scratch, and a second kernel adds the
+// partial tiles in range order (deterministic) and applies alpha and beta.
 #include "gnnhip_internal.h"
 
 namespace gnnhip {
@@ -17,8 +22,10 @@ constexpr int BM = 64, BN = 64, BK = 16, kBlock = 256;
 template <bool TA, bool TB>
 __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
     int m, int n, int k, float alpha, const float* __restrict__ A, int lda,
-    const float* __restrict__ B, int ldb, float beta, float* C, int ldc)
+    const float* __restrict__ B, int ldb, float beta, float* C, int ldc, int k_chunk, float* __restrict__ partial)
 {
+    // partial != nullptr: workgroup z handles k in [z k_chunk, (z+1) k_chunk) and stores its raw sums to
+    // partial[z][m][n]; otherwise one workgroup walks all of k and finishes C itself
     __shared__ float As[BK][BM + 4];     // As[p][i] = op(A)[row0 + i][k0 + p]
     __shared__ float Bs[BK][BN + 4];     // Bs[p][j] = op(B)[k0 + p][col0 + j]
 
@@ -34,8 +41,12 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
 
-    for (int k0 = 0; k0 < k; k0 += BK) {
-        // each lane loads 4 elements of each tile
+    const int k_lo = partial ? (int)blockIdx.z * k_chunk : 0;
+    const int k_hi = partial ? min(k, k_lo + k_chunk) : k;
+    // each lane moves 4 elements of each tile; the elements of step k0 + BK are requested before the
+    // products of step k0 are formed, so a step costs the longer of the two instead of their sum
+    float ra[4], rb[4];
+    auto fetch = [&](int k0) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int idx = tid + e * kBlock;        // 0 .. 1023
@@ -47,8 +58,8 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
                 const long long gi = row0 + i;
                 const int gp = k0 + p;
                 float v = 0.f;
-                if (gi < m && gp < k) v = TA ? A[(size_t)gp * lda + gi] : A[(size_t)gi * lda + gp];
-                As[p][i] = v;
+                if (gi < m && gp < k_hi) v = TA ? A[(size_t)gp * lda + gi] : A[(size_t)gi * lda + gp];
+                ra[e] = v;
             }
             {
                 int j, p;
@@ -57,11 +68,21 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
                 const int gj = col0 + j;
                 const int gp = k0 + p;
                 float v = 0.f;
-                if (gj < n && gp < k) v = TB ? B[(size_t)gj * ldb + gp] : B[(size_t)gp * ldb + gj];
-                Bs[p][j] = v;
+                if (gj < n && gp < k_hi) v = TB ? B[(size_t)gj * ldb + gp] : B[(size_t)gp * ldb + gj];
+                rb[e] = v;
             }
         }
+    };
+    if (k_lo < k_hi) fetch(k_lo);
+    for (int k0 = k_lo; k0 < k_hi; k0 += BK) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int idx = tid + e * kBlock;
+            if (TA) As[idx >> 6][idx & (BM - 1)] = ra[e]; else As[idx & (BK - 1)][idx >> 4] = ra[e];
+            if (TB) Bs[idx & (BK - 1)][idx >> 4] = rb[e]; else Bs[idx >> 6][idx & (BN - 1)] = rb[e];
+        }
         __syncthreads();
+        if (k0 + BK < k_hi) fetch(k0 + BK);
 #pragma unroll
         for (int p = 0; p < BK; ++p) {
             const float4 a = *reinterpret_cast<const float4*>(&As[p][ty * 4]);
@@ -84,10 +105,51 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
         for (int j = 0; j < 4; ++j) {
             const int gj = col0 + tx * 4 + j;
             if (gj >= n) continue;
+            if (partial) {
+                partial[((size_t)blockIdx.z * m + gi) * n + gj] = acc[i][j];
+                continue;
+            }
             float* dst = C + (size_t)gi * ldc + gj;
             const float r = alpha * acc[i][j];
             *dst = (beta == 0.f) ? r : r + beta * (*dst);
         }
+    }
+}
+
+// C = alpha * (sum over z of partial[z]) + beta * C.  A workgroup takes 64 consecutive elements; wavefront w
+// adds the ranges z = w, w + 4, ... (four loads in flight per lane) and the four sums are added in
+// wavefront order, so the result is the same on every run.
+__global__ __launch_bounds__(kBlock) void sgemm_splitk_reduce_kernel(int m, int n, int splits, float alpha,
+                                                                     const float* __restrict__ partial, float beta,
+                                                                     float* C, int ldc)
+{
+    __shared__ float part[kBlock / kWave][kWave];
+    const size_t total = (size_t)m * n;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    constexpr int kWaves = kBlock / kWave;
+    for (size_t base = (size_t)blockIdx.x * kWave; base < total; base += (size_t)gridDim.x * kWave) {
+        const size_t idx = base + lane;
+        float sum = 0.f;
+        if (idx < total) {
+            int z = wave;
+            for (; z + 3 * kWaves < splits; z += 4 * kWaves) {
+                const float p0 = partial[(size_t)z * total + idx], p1 = partial[(size_t)(z + kWaves) * total + idx];
+                const float p2 = partial[(size_t)(z + 2 * kWaves) * total + idx], p3 = partial[(size_t)(z + 3 * kWaves) * total + idx];
+                sum += p0; sum += p1; sum += p2; sum += p3;
+            }
+            for (; z < splits; z += kWaves) sum += partial[(size_t)z * total + idx];
+        }
+        part[wave][lane] = sum;
+        __syncthreads();
+        if (wave == 0 && idx < total) {
+            float t = part[0][lane];
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) t += part[w][lane];
+            float* dst = C + (idx / n) * (size_t)ldc + idx % n;
+            const float r = alpha * t;
+            *dst = (beta == 0.f) ? r : r + beta * (*dst);
+        }
+        __syncthreads();
     }
 }
 
@@ -163,14 +225,37 @@ int gemm_dispatch(int transA, int transB, int m, int n, int k, float alpha, cons
     }
     dim3 grid(ceil_div_u((size_t)m, BM), ceil_div_u((size_t)n, BN));
     dim3 block(kBlock);
+    // few output tiles and a long k: split k so that about two workgroups per CU share the work
+    int k_chunk = 0;
+    float* partial = nullptr;
+    const long long tiles = (long long)grid.x * grid.y;
+    if (tiles <= kNumCU / 4 && k >= 1024) {
+        const long long want = (2 * kNumCU) / tiles;                       // ranges per tile
+        long long chunk = ((long long)k + want - 1) / want;
+        if (chunk < 4 * BK) chunk = 4 * BK;
+        chunk = (chunk + BK - 1) / BK * BK;
+        const int splits = (int)(((long long)k + chunk - 1) / chunk);
+        if (splits > 1) {
+            void* q = nullptr;
+            if (int rc = stream_scratch_slot(s, 2, sizeof(float) * (size_t)splits * m * n, &q)) return rc;
+            partial = static_cast<float*>(q);
+            k_chunk = (int)chunk;
+            grid.z = splits;
+        }
+    }
     if (!transA && !transB)
-        hipLaunchKernelGGL((sgemm_tile_kernel<false, false>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+        hipLaunchKernelGGL((sgemm_tile_kernel<false, false>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
     else if (transA && !transB)
-        hipLaunchKernelGGL((sgemm_tile_kernel<true, false>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+        hipLaunchKernelGGL((sgemm_tile_kernel<true, false>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
     else if (!transA && transB)
-        hipLaunchKernelGGL((sgemm_tile_kernel<false, true>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+        hipLaunchKernelGGL((sgemm_tile_kernel<false, true>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
     else
-        hipLaunchKernelGGL((sgemm_tile_kernel<true, true>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+        hipLaunchKernelGGL((sgemm_tile_kernel<true, true>), grid, block, 0, s, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, k_chunk, partial);
+    if (partial) {
+        const size_t total = (size_t)m * n;
+        const unsigned rgrid = ceil_div_u(total, kWave) < 2048u ? ceil_div_u(total, kWave) : 2048u;
+        hipLaunchKernelGGL(sgemm_splitk_reduce_kernel, dim3(rgrid), block, 0, s, m, n, (int)grid.z, alpha, partial, beta, C, ldc);
+    }
     GNNHIP_LAUNCH_CHECK("sgemm_tile");
     return GNNHIP_OK;
 }

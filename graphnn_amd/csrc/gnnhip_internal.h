@@ -147,8 +147,9 @@ int pool_release(void* p);
 int stream_scratch(hipStream_t s, size_t bytes, void** p);
 // The same with several independent buffers per stream (slot 0 is stream_scratch's):
 // slot 1 holds the hub pre-pass results, which must outlive a consumer that itself
-// takes slot 0.
-constexpr int kScratchSlots = 2;
+// takes slot 0; slot 2 holds the partial tiles of a GEMM split along k, whose operands
+// may sit in slot 0.
+constexpr int kScratchSlots = 3;
 int stream_scratch_slot(hipStream_t s, int slot, size_t bytes, void** p);
 
 // ---- high-degree rows (hub.hip)
