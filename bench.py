@@ -145,6 +145,39 @@ def time_level_cfg4(dev):
             "algorithmic_GBps": level_algorithmic_bytes(N, E, C) / (ms * 1e-3) / 1e9}
 
 
+def time_large_batch(dev, B=30000):
+    """The configuration-2 graph distribution at 30,000 graphs per batch: the stages of the general route
+    (input, one level, readout), the whole forward on it, and the one-launch route."""
+    import torch
+    from graphnn_amd import batching, ops, synth
+    batch, w, cfg = synth.make_config(2, B=B)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    t = lambda arr: torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
+    a_d, s_d = tuple(map(t, a)), tuple(map(t, s))
+    X, Wn, Wc, W1, W2 = t(batch.one_hot()), t(w.W_n2l), t(w.W_conv), t(w.W_h1), t(w.W_h2)
+    N, E, K, C, H, Q, L = batch.num_nodes, batch.num_edges, cfg["K"], cfg["C"], cfg["H"], cfg["Q"], cfg["L"]
+    msg, h0 = ops.s2v_input(X, Wn)
+    h1 = torch.empty_like(h0)
+    bufs = ops.ForwardBuffers(N, B, C, H, Q, dev)
+    bb = ops.BatchedBuffers(N, B, C, H, Q, dev)
+    nmax = int(batch.graph_sizes.max())
+    ms_in = _event_ms(lambda: ops.s2v_input(X, Wn), 20)
+    ms_lv = _event_ms(lambda: ops.s2v_level(*a_d, h0, Wc, msg, out=h1), 20)
+    ms_ro = _event_ms(lambda: ops.s2v_readout(*s_d, h1, W1, W2, B), 20)
+    ms_fw = _event_ms(lambda: ops.s2v_forward(a_d, s_d, X, Wn, Wc, W1, W2, L, bufs=bufs), 20)
+    ms_one = _event_ms(lambda: ops.s2v_forward_batched(a_d, s_d, X, Wn, Wc, W1, W2, L, nmax, bufs=bb), 10)
+    gb = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
+    return {"workload": "%d graphs of the configuration-2 distribution: %d nodes, %d entries, hidden %d, %d levels" % (B, N, E, C, L),
+            "input": {"avg_ms": ms_in, "algorithmic_GBps": gb(4.0 * N * (K + 2 * C) + 4.0 * K * C, ms_in)},
+            "level": {"avg_ms": ms_lv, "kernel": "s2v_level_stream_kernel<64,false,true,3>",
+                      "algorithmic_GBps": gb(level_algorithmic_bytes(N, E, C), ms_lv)},
+            "readout": {"avg_ms": ms_ro, "kernel": "s2v_readout_wave_kernel<64>",
+                        "algorithmic_GBps": gb(4.0 * N * C + 8.0 * N + 4.0 * B * (C + H + 2 * Q), ms_ro)},
+            "forward": {"avg_ms": ms_fw, "graphs_per_s": B / (ms_fw * 1e-3)},
+            "forward_one_launch": {"avg_ms": ms_one, "graphs_per_s": B / (ms_one * 1e-3)}}
+
+
 def time_cfg5(dev, scale=22):
     """Configuration 5: R-MAT (a=.57, b=c=.19), 16 entries per row, generated on the device with the
     same recursive-quadrant rule as synth.rmat_csr (torch's generator, so not the parity inputs);
@@ -333,7 +366,7 @@ def main():
     out["end_to_end"] = end_to_end_host_layer(host)
 
     if args.extra:
-        out["extra"] = {"cfg4_level": time_level_cfg4(dev), "cfg5": time_cfg5(dev)}
+        out["extra"] = {"cfg4_level": time_level_cfg4(dev), "large_batch": time_large_batch(dev), "cfg5": time_cfg5(dev)}
 
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline(host)
     print(json.dumps(out))
