@@ -1,26 +1,26 @@
-// Fused structure2vec kernels for gfx950 (hidden size C in {16, 32, 64}; wider
-// hidden sizes take the unfused route in forward.hip):
+// Fused structure2vec kernels for gfx950, hidden size C in {16, 32, 64}, and the dispatchers of the
+// three stages (wider hidden sizes: input_wide.hip, level_wide.hip; other sizes: the unfused route in
+// forward.hip):
 //
 //   s2v_input_kernel    msg = X * W_n2l ; h0 = ReLU(msg)
-//   s2v_level_kernel    h_out = ReLU((A * h_in) * W + bias + msg)
+//   s2v_level_kernel    h_out = ReLU((A * h_in) * W + bias + msg), with 64-bit addressing: the kernel for
+//                       activations of 4 GiB and more (smaller ones take level_stream.hip)
 //   s2v_readout_kernel  pool = S * h ; hidden = ReLU(pool * W_h1) ;
-//                       logits = hidden * W_h2 ; probs = softmax(logits) ; pred = argmax
+//                       logits = hidden * W_h2 ; probs = softmax(logits) ; pred = argmax,
+//                       one workgroup per graph (many graphs: readout.hip)
 //
 // A level reads h_in (gathered), msg and the CSR arrays once and writes h_out
 // once: 4(N+1) + 8E + 12NC + 4C^2 algorithmic bytes, against roughly nine
 // passes over an N x C activation in the operator-by-operator schedule.  At
 // C = 64 the arithmetic intensity is ~6 flop/byte, far below the machine
-// balance, so the dense C x C contraction runs on plain FMA out of LDS and the
-// kernel is HBM-bound.
+// balance: the kernel is HBM-bound.
 //
-// Layout of one workgroup (256 lanes) in input/level kernels:
+// Layout of one workgroup (256 lanes) in the input kernel:
 //   G = C/4 lanes form a row group; the workgroup holds P = 256/G groups and
-//   processes tiles of R = RT * P rows.  Phase 1 fills an LDS tile [R][C+4]
-//   (level: neighbour gather-sum, one float4 per lane per gathered row; input:
-//   a straight copy of X rows).  Phase 2 multiplies the tile by W held in LDS:
-//   lane (ty, tx) produces rows ty + r*P (r < RT), columns 4tx..4tx+3.
-//   Phase 3 adds bias and msg, applies ReLU and stores float4s.
-// Workgroups are persistent over tiles so W is loaded into LDS once per group.
+//   processes tiles of R = RT * P rows.  Phase 1 copies the tile's rows of X into LDS [R][K+pad],
+//   phase 2 multiplies the tile by W_n2l held in LDS: lane (ty, tx) produces rows ty + r*P (r < RT),
+//   columns 4tx..4tx+3, phase 3 stores msg and ReLU(msg) as float4s.
+// Workgroups are persistent over tiles so W_n2l is loaded into LDS once per group.
 #include "gnnhip_internal.h"
 #include <stdlib.h>
 
