@@ -11,7 +11,9 @@ namespace gnnhip {
 bool fused_hidden_supported(int C);
 int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s);
 int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-                   const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph = false);
+                   const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph = false,
+                   bool relu_in = false);
+bool level_accepts_relu_input(int N, int C, long long nnz);
 int readout_dispatch(int B, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                      const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
                      float* logits, float* probs, int* pred, hipStream_t s);
@@ -56,6 +58,7 @@ int input_any(int N, int K, int C, const float* X, const float* Wn2l, float* msg
     int rc = input_dispatch(N, K, C, X, Wn2l, msg, h0, s);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
     if ((rc = gemm_dispatch(0, 0, N, C, K, 1.f, X, K, Wn2l, C, 0.f, msg, C, s))) return rc;
+    if (!h0) return GNNHIP_OK;
     const size_t total = (size_t)N * C;
     hipLaunchKernelGGL(bias_add_relu_kernel, dim3(ew_grid(total)), dim3(kBlock), 0, s,
                        msg, (const float*)nullptr, (const float*)nullptr, msg, h0, total, C, 1);
@@ -64,10 +67,12 @@ int input_any(int N, int K, int C, const float* X, const float* Wn2l, float* msg
 }
 
 int level_any(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-              const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph = false)
+              const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph = false,
+              bool relu_in = false)
 {
-    int rc = level_dispatch(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s, same_graph);
+    int rc = level_dispatch(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s, same_graph, relu_in);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
+    if (relu_in) return set_error(GNNHIP_EUNSUPPORTED, "no level kernel reads its input through ReLU for this shape");
     void* tmp = nullptr;
     const size_t total = (size_t)N * C;
     if ((rc = stream_scratch(s, sizeof(float) * total, &tmp))) return rc;
@@ -130,7 +135,7 @@ int gnnhip_s2v_input_f32(int N, int K, int C, const float* X, const float* W_n2l
 {
     GNNHIP_REQUIRE(N >= 0 && K >= 1 && C >= 1, "bad shape in s2v_input (N=%d K=%d C=%d)", N, K, C);
     if (N == 0) return GNNHIP_OK;
-    GNNHIP_REQUIRE(X && W_n2l && msg && h0, "null tensor in s2v_input");
+    GNNHIP_REQUIRE(X && W_n2l && msg, "null tensor in s2v_input");
     if (int rc = require_ready()) return rc;
     return input_any(N, K, C, X, W_n2l, msg, h0, as_stream(stream));
 }
@@ -178,13 +183,20 @@ int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L, int 
     GNNHIP_REQUIRE(h_a != h_b && msg != h_a && msg != h_b, "msg, h_a and h_b must be distinct buffers");
     if (int rc = require_ready()) return rc;
     hipStream_t s = as_stream(stream);
-    int rc = input_any(N, K, C, X, W_n2l, msg, h_a, s);
+    // With at least one level, and a level kernel that can read its input through ReLU, h0 = ReLU(msg) is
+    // never stored: the first level gathers from msg.
+    const bool lazy_h0 = L >= 1 && level_accepts_relu_input(N, C, a_nnz);
+    int rc = input_any(N, K, C, X, W_n2l, msg, lazy_h0 ? nullptr : h_a, s);
     if (rc) return rc;
-    float* cur = h_a;
-    float* nxt = h_b;
+    float* cur = lazy_h0 ? msg : h_a;
+    float* nxt = lazy_h0 ? h_a : h_b;
     for (int lv = 0; lv < L; ++lv) {
-        if ((rc = level_any(N, C, a_nnz, a_row_ptr, a_col_idx, a_val, cur, W_conv, msg, nullptr, nxt, s, lv > 0))) return rc;
-        float* t = cur; cur = nxt; nxt = t;
+        if ((rc = level_any(N, C, a_nnz, a_row_ptr, a_col_idx, a_val, cur, W_conv, msg, nullptr, nxt, s, lv > 0,
+                            lazy_h0 && lv == 0)))
+            return rc;
+        float* t = (cur == msg) ? h_b : cur;     // msg stays what it is; the other buffer takes the next level
+        cur = nxt;
+        nxt = t;
     }
     if (which_h) *which_h = (cur == h_a) ? 0 : 1;
     return readout_any(B, N, C, H, Q, s_row_ptr, s_col_idx, s_val, cur, W_h1, W_h2, pool, hidden, logits, probs, pred, s);

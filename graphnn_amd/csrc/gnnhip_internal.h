@@ -162,7 +162,7 @@ struct HubPlan {
     int ld;
 };
 int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
-                const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan = false);
+                const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan = false, bool relu_in = false);
 // spmm.hip: C = alpha*A*B + beta*C on stream s; reuse_plan as for hub_prepass
 int spmm_dispatch(int m, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan = false);

@@ -185,6 +185,7 @@ template <> struct HV<4> {
     using T = float4;
     static __device__ __forceinline__ T zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
     static __device__ __forceinline__ T load(const float* p) { return *reinterpret_cast<const float4*>(p); }
+    static __device__ __forceinline__ T load(const float* p, int relu) { const T v = load(p); return relu ? relu_ref4(v) : v; }
     static __device__ __forceinline__ void store(float* p, T v) { *reinterpret_cast<float4*>(p) = v; }
     static __device__ __forceinline__ void fma(T& a, float s, T x) { a.x += s * x.x; a.y += s * x.y; a.z += s * x.z; a.w += s * x.w; }
     static __device__ __forceinline__ T add(T a, T b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
@@ -193,6 +194,7 @@ template <> struct HV<1> {
     using T = float;
     static __device__ __forceinline__ T zero() { return 0.f; }
     static __device__ __forceinline__ T load(const float* p) { return *p; }
+    static __device__ __forceinline__ T load(const float* p, int relu) { const T v = *p; return relu ? relu_ref(v) : v; }
     static __device__ __forceinline__ void store(float* p, T v) { *p = v; }
     static __device__ __forceinline__ void fma(T& a, float s, T x) { a += s * x; }
     static __device__ __forceinline__ T add(T a, T b) { return a + b; }
@@ -206,8 +208,9 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
     const int* __restrict__ counts, int chunk_cap, int n, const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
     const float* __restrict__ val, const float* __restrict__ B, int ldb, int logG,
     const int* __restrict__ hub_row, const int* __restrict__ hub_chunk0, const int* __restrict__ chunk_hub,
-    float* part, int ldp, float* __restrict__ agg, int* hub_done)
+    float* part, int ldp, float* __restrict__ agg, int* hub_done, int relu_in)
 {
+    // relu_in: the rows of B are used as ReLU(B) (a first level that reads msg in place of h0)
     using V = HV<VEC>;
     __shared__ float red[kWavesPerBlock][kWave * VEC * ITERS];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
@@ -237,7 +240,7 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
                 if (col0 < n) {
                     typename V::T x[8];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) x[u] = V::load(B + (size_t)c8[u] * ldb + col0);
+                    for (int u = 0; u < 8; ++u) x[u] = V::load(B + (size_t)c8[u] * ldb + col0, relu_in);
 #pragma unroll
                     for (int u = 0; u < 8; ++u) V::fma(acc[it], v8[u], x[u]);
                 }
@@ -249,7 +252,7 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
                 const int col0 = (sub + it * G) * VEC;
-                if (col0 < n) V::fma(acc[it], v0, V::load(B + (size_t)c0 * ldb + col0));
+                if (col0 < n) V::fma(acc[it], v0, V::load(B + (size_t)c0 * ldb + col0, relu_in));
             }
         }
 #pragma unroll
@@ -315,11 +318,11 @@ inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 template <int VEC, int ITERS>
 void launch_partial(hipStream_t s, const int* counts, int chunk_cap, int n, const int* row_ptr, const int* col_idx,
                     const float* val, const float* B, int ldb, int logG, const int* hub_row, const int* hub_chunk0,
-                    const int* chunk_hub, float* part, int ldp, float* agg, int* hub_done)
+                    const int* chunk_hub, float* part, int ldp, float* agg, int* hub_done, int relu_in)
 {
     const unsigned grid = kNumCU * 8;
     hipLaunchKernelGGL((hub_partial_kernel<VEC, ITERS>), dim3(grid), dim3(kBlock), 0, s, counts, chunk_cap, n, row_ptr,
-                       col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
+                       col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in);
 }
 
 }  // namespace
@@ -331,7 +334,7 @@ void launch_partial(hipStream_t s, const int* counts, int chunk_cap, int n, cons
 // this stream with the same arguments (the levels of one forward); the planning launches
 // (count, scan, fill) are then skipped and only the sums are recomputed.
 int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
-                const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan)
+                const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan, bool relu_in)
 {
     plan->row_slot = nullptr;
     plan->agg = nullptr;
@@ -392,13 +395,13 @@ int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_
         memo = Memo{s, row_ptr, m, n, nnz, base};
     }
     if (vec4) {
-        if (iters <= 1) launch_partial<4, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
-        else if (iters == 2) launch_partial<4, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
-        else launch_partial<4, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
+        if (iters <= 1) launch_partial<4, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
+        else if (iters == 2) launch_partial<4, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
+        else launch_partial<4, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
     } else {
-        if (iters <= 1) launch_partial<1, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
-        else if (iters == 2) launch_partial<1, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
-        else launch_partial<1, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done);
+        if (iters <= 1) launch_partial<1, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
+        else if (iters == 2) launch_partial<1, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
+        else launch_partial<1, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
     }
     GNNHIP_LAUNCH_CHECK("hub_prepass");
     plan->row_slot = row_slot;

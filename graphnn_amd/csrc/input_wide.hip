@@ -85,7 +85,7 @@ __global__ __launch_bounds__(kBlock) void s2v_input_wide_kernel(
 
         const unsigned bytes = (unsigned)rows * (C * 4);
         const rsrc_t msg_rsrc = make_rsrc(msg + (size_t)row0 * C, bytes);
-        const rsrc_t h0_rsrc = make_rsrc(h0 + (size_t)row0 * C, bytes);
+        const rsrc_t h0_rsrc = make_rsrc(h0 ? h0 + (size_t)row0 * C : nullptr, h0 ? bytes : 0u);      // h0 may be null
 #pragma unroll 1
         for (int rt = 0; rt < kTileRows / 16; ++rt) {
             if (rt * 16 >= rows) break;
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(kBlock) void s2v_input_wide_kernel(
             for (int jb = 0; jb < NB; ++jb) {
                 const float4 v = make_float4(acc[jb][0], acc[jb][1], acc[jb][2], acc[jb][3]);
                 buf_store4(msg_rsrc, voff + 64 * jb, v);
-                buf_store4(h0_rsrc, voff + 64 * jb, relu_ref4(v));
+                if (h0) buf_store4(h0_rsrc, voff + 64 * jb, relu_ref4(v));
             }
         }
     }

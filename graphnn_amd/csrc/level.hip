@@ -35,7 +35,8 @@ namespace gnnhip {
 // level_stream.hip
 int level_stream_dispatch(int N, int C, bool dense, const int* row_ptr, const int* col_idx, const float* val,
                           const float* h_in, const float* W, const float* msg, const float* bias, float* h_out,
-                          const HubPlan& hubs, hipStream_t s);
+                          const HubPlan& hubs, bool relu_in, hipStream_t s);
+bool level_stream_covers(int N, int C);
 // input_wide.hip
 int input_wide_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s);
 // level_wide.hip
@@ -157,8 +158,7 @@ __global__ __launch_bounds__(kBlock) void s2v_input_kernel(
                 const size_t off = ((size_t)row0 + lr) * C + tx * 4;
                 const float4 v = acc[r];
                 *reinterpret_cast<float4*>(msg + off) = v;
-                *reinterpret_cast<float4*>(h0 + off) =
-                    make_float4(relu_ref(v.x), relu_ref(v.y), relu_ref(v.z), relu_ref(v.w));
+                if (h0) *reinterpret_cast<float4*>(h0 + off) = relu_ref4(v);      // no h0: the caller applies ReLU on reading msg
             }
         }
     }
@@ -572,7 +572,7 @@ bool fused_hidden_supported(int C) { return C == 16 || C == 32 || C == 64 || C =
 
 int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s)
 {
-    if (!(aligned16(Wn2l) && aligned16(msg) && aligned16(h0))) return GNNHIP_EUNSUPPORTED;
+    if (!(aligned16(Wn2l) && aligned16(msg) && aligned16(h0))) return GNNHIP_EUNSUPPORTED;      // h0 may be null
     const bool small = small_batch(N);
     switch (C) {
     case 16: return small ? launch_input<16, 1>(N, K, X, Wn2l, msg, h0, s) : launch_input<16, 4>(N, K, X, Wn2l, msg, h0, s);
@@ -584,9 +584,20 @@ int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float
     return GNNHIP_EUNSUPPORTED;
 }
 
-int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-                   const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph)
+// Whether level_dispatch can read h_in as ReLU(h_in): then the forward does not store h0 = ReLU(msg) and the
+// first level gathers from msg (one activation less written, and the gathered rows are the ones the level
+// reads anyway).
+bool level_accepts_relu_input(int N, int C, long long nnz)
 {
+    const bool two_step = N >= kHubMinRows && nnz >= two_step_degree() * (long long)N;
+    return level_stream_covers(N, C) && !two_step;
+}
+
+int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
+                   const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph,
+                   bool relu_in)
+{
+    // relu_in: h_in is read as ReLU(h_in); only where level_accepts_relu_input says so
     // same_graph: the previous call on this stream had the same A (a later level of one forward), so the
     // plan of the long-row pass is still in place and only its sums are redone
     if (!(aligned16(h_in) && aligned16(W) && aligned16(h_out) && (!msg || aligned16(msg)) && (!bias || aligned16(bias))))
@@ -600,10 +611,11 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
         // mean degree, and dense graphs in practice are the skewed ones, so large graphs with at least
         // kTwoStepMeanDegree entries per row take the two launches.
         const bool two_step = N >= kHubMinRows && nnz >= two_step_degree() * (long long)N;
+        if (relu_in && (two_step || !level_stream_covers(N, C))) return GNNHIP_EUNSUPPORTED;
         if (two_step) {
             if (int rc = spmm_dispatch(N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, h_out, C, s, same_graph)) return rc;
             const HubPlan none{nullptr, nullptr, 0};
-            if (int rc = level_stream_dispatch(N, C, true, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, none, s);
+            if (int rc = level_stream_dispatch(N, C, true, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, none, false, s);
                 rc != GNNHIP_EUNSUPPORTED)
                 return rc;
             switch (C) {
@@ -613,9 +625,9 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
             }
         }
         HubPlan hubs{nullptr, nullptr, 0};
-        if (int rc = hub_prepass(N, C, nnz, row_ptr, col_idx, val, h_in, C, s, &hubs, same_graph)) return rc;
+        if (int rc = hub_prepass(N, C, nnz, row_ptr, col_idx, val, h_in, C, s, &hubs, same_graph, relu_in)) return rc;
         // activations of 4 GiB and more keep the kernel with 64-bit addressing below
-        if (int rc = level_stream_dispatch(N, C, false, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
+        if (int rc = level_stream_dispatch(N, C, false, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, relu_in, s);
             rc != GNNHIP_EUNSUPPORTED)
             return rc;
         switch (C) {
@@ -624,6 +636,7 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
         default: return launch_level<64, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
         }
     }
+    if (relu_in) return GNNHIP_EUNSUPPORTED;
     switch (C) {
     case 128:
     case 256: return level_wide_dispatch(N, C, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);

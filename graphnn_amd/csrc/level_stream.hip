@@ -73,17 +73,23 @@ __device__ __forceinline__ void gather4(rsrc_t h_rsrc, int offs, int tx_off, flo
     x[2] = buf_load4(h_rsrc, group_lane<G, U0 + 2>(offs) + tx_off, 0);
     x[3] = buf_load4(h_rsrc, group_lane<G, U0 + 3>(offs) + tx_off, 0);
 }
-template <int G, int U0>
+// RELU_IN: the gathered rows count as ReLU(row) (the first level reading msg where h0 was not stored)
+template <bool RELU_IN>
+__device__ __forceinline__ float4 as_input(const float4& x)
+{
+    return RELU_IN ? relu_ref4(x) : x;
+}
+template <int G, int U0, bool RELU_IN>
 __device__ __forceinline__ void sum4(float4& acc, float w, const float4 (&x)[4])
 {
-    f4_fma(acc, group_lane<G, U0 + 0>(w), x[0]);
-    f4_fma(acc, group_lane<G, U0 + 1>(w), x[1]);
-    f4_fma(acc, group_lane<G, U0 + 2>(w), x[2]);
-    f4_fma(acc, group_lane<G, U0 + 3>(w), x[3]);
+    f4_fma(acc, group_lane<G, U0 + 0>(w), as_input<RELU_IN>(x[0]));
+    f4_fma(acc, group_lane<G, U0 + 1>(w), as_input<RELU_IN>(x[1]));
+    f4_fma(acc, group_lane<G, U0 + 2>(w), as_input<RELU_IN>(x[2]));
+    f4_fma(acc, group_lane<G, U0 + 3>(w), as_input<RELU_IN>(x[3]));
 }
 
 // MINW: wavefronts per SIMD the register allocation must leave room for
-template <int C, bool DENSE, bool WLDS, int MINW>
+template <int C, bool DENSE, bool WLDS, int MINW, bool RELU_IN>
 __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
     int N, const int* __restrict__ row_ptr, const int* __restrict__ col_idx, const float* __restrict__ val,
     const float* __restrict__ h_in, const float* __restrict__ W, const float* __restrict__ msg,
@@ -224,7 +230,7 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
 #pragma unroll
             for (int rd = 0; rd < ROUNDS; ++rd) {
                 acc[rd] = f4_zero();
-                sum4<G, 0>(acc[rd], w0[rd], x[rd]);
+                sum4<G, 0, RELU_IN>(acc[rd], w0[rd], x[rd]);
             }
             GNNHIP_PHASE_ACC(2);
             if (__any(longest > 4 || far)) {
@@ -233,7 +239,7 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
 #pragma unroll
                     for (int rd = 0; rd < ROUNDS; ++rd) gather4<G, 4>(h_rsrc, offs[rd], tx_off, x[rd]);
 #pragma unroll
-                    for (int rd = 0; rd < ROUNDS; ++rd) sum4<G, 4>(acc[rd], w0[rd], x[rd]);
+                    for (int rd = 0; rd < ROUNDS; ++rd) sum4<G, 4, RELU_IN>(acc[rd], w0[rd], x[rd]);
                 }
                 if (__any(longest > kDirect || far)) {
                     // the rest of the first batch, then further batches of G
@@ -261,7 +267,7 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
                                     xx[u] = buf_load4(h_rsrc, (j + u < cnt) ? row_off(cj[u]) : kBufPastEnd, 0);
 #pragma unroll
                                 for (int u = 0; u < 4; ++u)
-                                    if (j + u < cnt) f4_fma(acc[rd], vj[u], xx[u]);
+                                    if (j + u < cnt) f4_fma(acc[rd], vj[u], as_input<RELU_IN>(xx[u]));
                             }
                         }
                     }
@@ -304,9 +310,9 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
 #pragma unroll
                             for (int u = 0; u < 4; ++u) xx[u] = buf_load4(h_rsrc, row_off(c4[u]), 0);
 #pragma unroll
-                            for (int u = 0; u < 4; ++u) f4_fma(a, v4[u], xx[u]);
+                            for (int u = 0; u < 4; ++u) f4_fma(a, v4[u], as_input<RELU_IN>(xx[u]));
                         }
-                        for (; e < le; e += RPR) f4_fma(a, val[e], buf_load4(h_rsrc, row_off(col_idx[e]), 0));
+                        for (; e < le; e += RPR) f4_fma(a, val[e], as_input<RELU_IN>(buf_load4(h_rsrc, row_off(col_idx[e]), 0)));
                         *reinterpret_cast<float4*>(red + grp * C + tx * 4) = a;
                         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
                         if (grp == 0) {
@@ -384,7 +390,7 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
     GNNHIP_PHASE_FINI
 }
 
-template <int C, bool DENSE>
+template <int C, bool DENSE, bool RELU_IN>
 int launch_level_stream(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
                         const float* W, const float* msg, const float* bias, float* h_out, const HubPlan& hubs,
                         hipStream_t s)
@@ -395,33 +401,43 @@ int launch_level_stream(int N, const int* row_ptr, const int* col_idx, const flo
     constexpr int kMinW = (C == 64 && !DENSE) ? 3 : 4;    // hidden 64 needs 128 registers and spills for four
     const long long resident = (long long)kNumCU * kMinW;  // a workgroup puts one wavefront on each SIMD
     if (blocks > resident) blocks = resident;              // persistent beyond this
-    hipLaunchKernelGGL((s2v_level_stream_kernel<C, DENSE, kWLds, kMinW>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL((s2v_level_stream_kernel<C, DENSE, kWLds, kMinW, RELU_IN>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
                        N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs.row_slot, hubs.agg, hubs.ld);
     GNNHIP_LAUNCH_CHECK("s2v_level_stream");
     return GNNHIP_OK;
 }
 
-}  // namespace
-
-// h_in, msg and h_out must each span less than 4 GiB (with room for the 15 rows a last tile may
-// address past N); returns GNNHIP_EUNSUPPORTED otherwise.
-int level_stream_dispatch(int N, int C, bool dense, const int* row_ptr, const int* col_idx, const float* val,
+template <int C>
+int launch_level_stream_c(int N, bool dense, bool relu_in, const int* row_ptr, const int* col_idx, const float* val,
                           const float* h_in, const float* W, const float* msg, const float* bias, float* h_out,
                           const HubPlan& hubs, hipStream_t s)
 {
-    if ((unsigned long long)N * (unsigned)C * 4ull >= 0xFFFF0000ull) return GNNHIP_EUNSUPPORTED;
+    if (dense) return launch_level_stream<C, true, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
+    if (relu_in) return launch_level_stream<C, false, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
+    return launch_level_stream<C, false, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
+}
+
+}  // namespace
+
+// Whether N rows of C floats fit the 32-bit offsets of the kernel (with room for the 15 rows a last tile may
+// address past N).
+bool level_stream_covers(int N, int C)
+{
+    return (C == 16 || C == 32 || C == 64) && (unsigned long long)N * (unsigned)C * 4ull < 0xFFFF0000ull;
+}
+
+// h_in, msg and h_out must each span less than 4 GiB; returns GNNHIP_EUNSUPPORTED otherwise.
+// relu_in (not with dense): h_in is read as ReLU(h_in); hub sums in `hubs` must have been formed the same way.
+int level_stream_dispatch(int N, int C, bool dense, const int* row_ptr, const int* col_idx, const float* val,
+                          const float* h_in, const float* W, const float* msg, const float* bias, float* h_out,
+                          const HubPlan& hubs, bool relu_in, hipStream_t s)
+{
+    if (!level_stream_covers(N, C) || (dense && relu_in)) return GNNHIP_EUNSUPPORTED;
     switch (C) {
-    case 16:
-        return dense ? launch_level_stream<16, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s)
-                     : launch_level_stream<16, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
-    case 32:
-        return dense ? launch_level_stream<32, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s)
-                     : launch_level_stream<32, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
-    case 64:
-        return dense ? launch_level_stream<64, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s)
-                     : launch_level_stream<64, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
+    case 16: return launch_level_stream_c<16>(N, dense, relu_in, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
+    case 32: return launch_level_stream_c<32>(N, dense, relu_in, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
+    default: return launch_level_stream_c<64>(N, dense, relu_in, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
     }
-    return GNNHIP_EUNSUPPORTED;
 }
 
 }  // namespace gnnhip

@@ -323,22 +323,23 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
         DVar *X = dense(vX), *Wn = dense(vWn), *Wc = dense(vWc), *W1 = dense(vW1), *W2 = dense(vW2), *Msg = dense(vMsg),
              *Hl = dense(cur), *Pool = dense(vPool), *Hid = dense(vHid), *Logits = dense(vLogits);
         SVar *A = sparse(vA), *S = sparse(vS);
+        DVar* H0 = dense(vH0);                           // h0: the second embedding buffer of the general route
         step->run = [=](Phase ph) {
             bool done = false;
+            const size_t N = X->value.rows(), K = X->value.cols(), C = Wn->value.cols(), H = W1->value.cols(),
+                         Q = W2->value.cols(), B = S->value.rows();
+            ASSERT(Wn->value.rows() == K && Wc->value.rows() == C && Wc->value.cols() == C && W1->value.rows() == C &&
+                   W2->value.rows() == H && A->value.rows() == N && A->value.cols() == N && S->value.cols() == N,
+                   "fused forward: operand shapes do not chain");
+            Msg->value.Reshape({N, C});
+            Hl->value.Reshape({N, C});
+            Pool->value.Reshape({B, C});
+            Hid->value.Reshape({B, H});
+            Logits->value.Reshape({B, Q});
             // Past about 20,000 nodes the chip is full either way and the separate kernels are faster
             // (1,000 graphs of configuration 2: 62 us against 70 us in one launch; 256 graphs: 40 against 23).
             if (n2n->block_diagonal && sub->contiguous_subgraphs && sub->max_subgraph_nodes > 0 &&
-                X->value.rows() <= detail::kOneLaunchMaxNodes) {
-                const size_t N = X->value.rows(), K = X->value.cols(), C = Wn->value.cols(), H = W1->value.cols(),
-                             Q = W2->value.cols(), B = S->value.rows();
-                ASSERT(Wn->value.rows() == K && Wc->value.rows() == C && Wc->value.cols() == C && W1->value.rows() == C &&
-                       W2->value.rows() == H && A->value.rows() == N && A->value.cols() == N && S->value.cols() == N,
-                       "fused forward: operand shapes do not chain");
-                Msg->value.Reshape({N, C});
-                Hl->value.Reshape({N, C});
-                Pool->value.Reshape({B, C});
-                Hid->value.Reshape({B, H});
-                Logits->value.Reshape({B, Q});
+                N <= detail::kOneLaunchMaxNodes) {
                 const int rc = gnnhip_s2v_forward_batched_f32(
                     (int)N, (int)B, (int)K, (int)C, (int)H, (int)Q, L, sub->max_subgraph_nodes,
                     A->value.data->row_ptr, A->value.data->col_idx, A->value.data->val,
@@ -348,6 +349,22 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
                     Logits->value.data->ptr, nullptr, nullptr, nullptr, GpuHandle::Stream());
                 if (rc == GNNHIP_OK) done = true;
                 else ASSERT(rc == GNNHIP_EUNSUPPORTED, gnnhip_last_error());
+            }
+            if (!done && H0) {
+                // any CSR: input, levels and readout in one call; the library picks which of the two embedding
+                // buffers ends up with the last level, and the variables swap their storage if it is h0's
+                H0->value.Reshape({N, C});
+                int which = 0;
+                const int rc = gnnhip_s2v_forward_f32(
+                    (int)N, (int)B, (int)K, (int)C, (int)H, (int)Q, L, (int)A->value.data->nnz,
+                    A->value.data->row_ptr, A->value.data->col_idx, A->value.data->val,
+                    S->value.data->row_ptr, S->value.data->col_idx, S->value.data->val,
+                    X->value.data->ptr, Wn->value.data->ptr, Wc->value.data->ptr, W1->value.data->ptr, W2->value.data->ptr,
+                    Msg->value.data->ptr, Hl->value.data->ptr, H0->value.data->ptr, Pool->value.data->ptr,
+                    Hid->value.data->ptr, Logits->value.data->ptr, nullptr, nullptr, &which, GpuHandle::Stream());
+                ASSERT(rc == GNNHIP_OK, gnnhip_last_error());
+                if (which == 1) std::swap(Hl->value.data, H0->value.data);
+                done = true;
             }
             if (!done) for (auto& p : parts) p->run(ph);
         };

@@ -116,7 +116,8 @@ int gnnhip_s2v_level_f32(int N, int C, int nnz, const int* row_ptr, const int* c
                          float* h_out, void* stream);
 
 /* ---- msg = X * W_n2l and h0 = ReLU(msg) in one pass
- *      (examples/graph_classification/src/kernel_mean_field.cpp:31-32: MatMul + ReLU).  X [N,K], W_n2l [K,C]. */
+ *      (examples/graph_classification/src/kernel_mean_field.cpp:31-32: MatMul + ReLU).  X [N,K], W_n2l [K,C].
+ *      h0 may be NULL: only msg is written. */
 int gnnhip_s2v_input_f32(int N, int K, int C, const float* X, const float* W_n2l,
                          float* msg, float* h0, void* stream);
 
@@ -134,7 +135,9 @@ int gnnhip_s2v_readout_f32(int B, int N, int C, int H, int Q,
 
 /* ---- whole forward = input + L levels + readout, device-resident.
  *      h_a / h_b are [N,C] ping-pong buffers; *which_h (host int, may be NULL)
- *      receives 0 if the final embedding is in h_a, 1 if in h_b.  a_nnz: entries of A.
+ *      receives 0 if the final embedding is in h_a, 1 if in h_b (which of the two holds which level is
+ *      the library's choice: with L >= 1 the first level may read ReLU(msg) straight from msg, and
+ *      h0 is then never stored).  a_nnz: entries of A.
  *      Op sequence of examples/graph_classification/src/kernel_mean_field.cpp:31-49 scheduled by
  *      FactorGraph::SequentialForward (src/nn/factor_graph.cpp:75-144). */
 int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L, int a_nnz,

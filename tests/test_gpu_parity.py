@@ -772,6 +772,33 @@ def test_level_hub_rows_balanced_pass(gpu, oracle, C):
     assert np.array_equal(got, _n(ops.s2v_level(*_csr_t(csr, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu))))
 
 
+@pytest.mark.parametrize("C,L", [(64, 2), (16, 1), (32, 3)])
+def test_forward_first_level_reads_msg_with_long_rows(gpu, oracle, C, L):
+    """sparse graph of 36,000 nodes with a few very long rows: the forward does not store h0, the first level
+    and the balanced pass over the long rows read ReLU(msg) from msg; every level's embedding, the pooled
+    features and the logits against the reference path"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(700 + C)
+    N, K, H, Q, B = 36000, 9, 16, 3, 36
+    a = _hub_matrix(rng, N, N, [(0, 9000), (1, 2100), (7, 300), (16, 2048), (17, 65), (18, 64), (19, 49), (20000, 3000), (N - 1, 1000)])
+    s = synth.contiguous_subgraph_csr(N, B)
+    lab = rng.integers(0, K, N)
+    X = np.zeros((N, K), np.float32); X[np.arange(N), lab] = 1.0
+    X += (rng.standard_normal(X.shape) * 0.05).astype(np.float32)              # msg with both signs everywhere
+    w = synth.make_weights(synth.Stream(700 + C), K, C, H, Q)
+    w.W_conv = (w.W_conv * 0.02).astype(np.float32)                              # rows of thousands of entries: keep the levels bounded
+    want = oracle.forward(a, s, X, w, L)
+    bufs = ops.s2v_forward(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+                           _t(w.W_h1, gpu), _t(w.W_h2, gpu), L)
+    assert max_rel(_n(bufs.msg), want["msg"]) < PARITY_TOL
+    # the reference path adds a row of thousands of entries sequentially in fp32 and is itself about 1e-4 from
+    # the exact sum there, so the embeddings are held to 3e-4
+    got_h = _n(bufs.h_final)
+    assert max_rel(got_h, want["h"][L]) < 3e-4
+    assert max_rel(_n(bufs.pool), want["pool"]) < 3e-4
+    assert max_rel(_n(bufs.logits), want["logits"]) < 3e-4
+
+
 def test_rmat_forward_with_jagged_softmax(gpu, oracle):
     """the skewed-degree workload at reduced scale: R-MAT (a=0.57, b=c=0.19), 16 entries per row on
     average, subgraphs = contiguous ranges of 1024 nodes; three levels, node score = h . w, jagged
