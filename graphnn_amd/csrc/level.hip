@@ -41,7 +41,8 @@ bool level_stream_covers(int N, int C);
 int input_wide_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s);
 // level_wide.hip
 int level_wide_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-                        const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s);
+                        const float* W, const float* msg, const float* bias, float* h_out, bool relu_in, hipStream_t s);
+bool level_wide_covers(int N, int C);
 
 namespace {
 
@@ -589,6 +590,7 @@ int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float
 // reads anyway).
 bool level_accepts_relu_input(int N, int C, long long nnz)
 {
+    if (level_wide_covers(N, C)) return true;
     const bool two_step = N >= kHubMinRows && nnz >= two_step_degree() * (long long)N;
     return level_stream_covers(N, C) && !two_step;
 }
@@ -636,10 +638,9 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
         default: return launch_level<64, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
         }
     }
-    if (relu_in) return GNNHIP_EUNSUPPORTED;
     switch (C) {
     case 128:
-    case 256: return level_wide_dispatch(N, C, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    case 256: return level_wide_dispatch(N, C, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, relu_in, s);
     }
     return GNNHIP_EUNSUPPORTED;
 }

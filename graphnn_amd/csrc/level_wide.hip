@@ -96,12 +96,12 @@ template <int VEC> struct BufLoad;
 template <> struct BufLoad<4> { static __device__ __forceinline__ float4 get(rsrc_t r, int v, int s) { return buf_load4(r, v, s); } };
 template <> struct BufLoad<2> { static __device__ __forceinline__ float2 get(rsrc_t r, int v, int s) { return buf_load2(r, v, s); } };
 
-template <int VEC>
+template <int VEC, bool RELU_IN>
 __device__ __forceinline__ void vec_fma(float (&acc)[VEC], float a, const typename VecT<VEC>::type& x)
 {
     const float* p = reinterpret_cast<const float*>(&x);
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[i] = fmaf(a, p[i], acc[i]);
+    for (int i = 0; i < VEC; ++i) acc[i] = fmaf(a, RELU_IN ? relu_ref(p[i]) : p[i], acc[i]);
 }
 
 // Everything that steers the gather (row pointers, column indices, edge weights) is uniform
@@ -110,7 +110,8 @@ __device__ __forceinline__ void vec_fma(float (&acc)[VEC], float a, const typena
 // waiting for them never waits for a store.  That matters because on this hardware the FP32 matrix
 // instructions and ordinary vector instructions do not overlap: every vector instruction issued by
 // either wavefront of a SIMD takes time away from its matrix pipe.
-template <int C, int WAVES>
+// RELU_IN: the gathered rows count as ReLU(row) (the first level reading msg where h0 was not stored)
+template <int C, int WAVES, bool RELU_IN>
 __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     int N, int tiles_per_block, const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
     const float* __restrict__ val, const float* __restrict__ h_in, const float* __restrict__ W,
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
         for (int u = 0; u < kInFlight; ++u) {
             if (e + u < ee) {
                 while (e + u >= row_end) flush_row();          // rows ending here (possibly empty ones)
-                vec_fma<VEC>(acc, __int_as_float(a[u]), x[u]);
+                vec_fma<VEC, RELU_IN>(acc, __int_as_float(a[u]), x[u]);
             }
         }
         e += kInFlight;
@@ -388,7 +389,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     GNNHIP_PHASE_FINI
 }
 
-template <int C, int WAVES>
+template <int C, int WAVES, bool RELU_IN>
 int launch_level_wide(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
                       const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
 {
@@ -399,11 +400,11 @@ int launch_level_wide(int N, const int* row_ptr, const int* col_idx, const float
     const size_t smem = sizeof(float) * (2 * kTileRows * (C + 4) + C);
     static bool attr_set = false;                                    // more than 64 KB of LDS has to be asked for
     if (!attr_set) {
-        GNNHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&s2v_level_wide_kernel<C, WAVES>),
+        GNNHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&s2v_level_wide_kernel<C, WAVES, RELU_IN>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    hipLaunchKernelGGL((s2v_level_wide_kernel<C, WAVES>), dim3((unsigned)blocks), dim3(WAVES * kWave), smem, s,
+    hipLaunchKernelGGL((s2v_level_wide_kernel<C, WAVES, RELU_IN>), dim3((unsigned)blocks), dim3(WAVES * kWave), smem, s,
                        N, (int)per, row_ptr, col_idx, val, h_in, W, msg, bias, h_out);
     GNNHIP_LAUNCH_CHECK("s2v_level_wide");
     return GNNHIP_OK;
@@ -411,12 +412,22 @@ int launch_level_wide(int N, const int* row_ptr, const int* col_idx, const float
 
 }  // namespace
 
+// Whether N rows of C floats have a wide kernel (32-bit buffer offsets).
+bool level_wide_covers(int N, int C)
+{
+    return (C == 128 || C == 256) && (unsigned long long)N * (unsigned)C * 4ull < (1ull << 32);
+}
+
 int level_wide_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-                        const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
+                        const float* W, const float* msg, const float* bias, float* h_out, bool relu_in, hipStream_t s)
 {
     switch (C) {
-    case 128: return launch_level_wide<128, 8>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
-    case 256: return launch_level_wide<256, 8>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    case 128:
+        return relu_in ? launch_level_wide<128, 8, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s)
+                       : launch_level_wide<128, 8, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    case 256:
+        return relu_in ? launch_level_wide<256, 8, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s)
+                       : launch_level_wide<256, 8, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
     }
     return GNNHIP_EUNSUPPORTED;
 }

@@ -772,7 +772,7 @@ def test_level_hub_rows_balanced_pass(gpu, oracle, C):
     assert np.array_equal(got, _n(ops.s2v_level(*_csr_t(csr, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu))))
 
 
-@pytest.mark.parametrize("C,L", [(64, 2), (16, 1), (32, 3)])
+@pytest.mark.parametrize("C,L", [(64, 2), (16, 1), (32, 3), (128, 2), (256, 1)])
 def test_forward_first_level_reads_msg_with_long_rows(gpu, oracle, C, L):
     """sparse graph of 36,000 nodes with a few very long rows: the forward does not store h0, the first level
     and the balanced pass over the long rows read ReLU(msg) from msg; every level's embedding, the pooled
