@@ -45,6 +45,7 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kPipeMinRows = 65536;   // from here on the kernel variant that asks for a tile's gathers one tile early
 constexpr int kWaveLongRow = 48;     // entries; longer rows are gathered by all groups of the wavefront together,
                                      // and past kHubThreshold they come from the pre-pass when there is one
 
@@ -89,7 +90,7 @@ __device__ __forceinline__ void sum4(float4& acc, float w, const float4 (&x)[4])
 }
 
 // MINW: wavefronts per SIMD the register allocation must leave room for
-template <int C, bool DENSE, bool WLDS, int MINW, bool RELU_IN>
+template <int C, bool DENSE, bool WLDS, int MINW, bool RELU_IN, bool PIPE>
 __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
     int N, const int* __restrict__ row_ptr, const int* __restrict__ col_idx, const float* __restrict__ val,
     const float* __restrict__ h_in, const float* __restrict__ W, const float* __restrict__ msg,
@@ -193,6 +194,17 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
     load_rp(rp, tile_id < ntiles ? tile_id : ntiles);
     load_rp(rpn, tile_n1 < ntiles ? tile_n1 : ntiles);
     load_first_batch(rp, offs, w0);
+    // PIPE: the gathers of a tile are issued one tile earlier, before the contraction of the tile in hand, so
+    // that they travel while the matrix cores work; the look-ahead of the CSR data is one tile deeper for it
+    int rpq[PIPE ? RN : 1], offq[PIPE ? ROUNDS : 1];
+    float wq[PIPE ? ROUNDS : 1];
+    float4 x[ROUNDS][4];                     // gathered rows: four entries of each of the lane group's rows
+    if constexpr (PIPE && !DENSE) {
+        load_rp(rpq, tile_n2 < ntiles ? tile_n2 : ntiles);
+        load_first_batch(rpn, offq, wq);
+#pragma unroll
+        for (int rd = 0; rd < ROUNDS; ++rd) gather4<G, 0>(h_rsrc, offs[rd], tx_off, x[rd]);
+    }
 
     GNNHIP_PHASE_INIT
     while (tile_id < ntiles) {
@@ -201,6 +213,8 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
         // msg is read, and h_out written, one row per lane group: every instruction covers whole rows.
         // Rows past N are out of range.
         const int out_off = row_off(row0 + grp * ROUNDS);
+        int rpnn[RN], offsn[ROUNDS];             // look-ahead requests of this iteration
+        float w0n[ROUNDS];
 
         if constexpr (DENSE) {
 #pragma unroll
@@ -211,14 +225,13 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
             }
         } else {
             // ---- the first four neighbours of every row of the tile, fetched together
-            float4 x[ROUNDS][4];
+            if constexpr (!PIPE) {
 #pragma unroll
-            for (int rd = 0; rd < ROUNDS; ++rd) gather4<G, 0>(h_rsrc, offs[rd], tx_off, x[rd]);
-            // ---- behind the gathers: the next tile's first batch, and the row pointers of the tile after it
-            int rpnn[RN], offsn[ROUNDS];
-            float w0n[ROUNDS];
-            load_rp(rpnn, tile_n2 < ntiles ? tile_n2 : ntiles);       // tile ntiles: every pointer reads 0 or row_ptr[N]
-            load_first_batch(rpn, offsn, w0n);
+                for (int rd = 0; rd < ROUNDS; ++rd) gather4<G, 0>(h_rsrc, offs[rd], tx_off, x[rd]);
+                // ---- behind the gathers: the next tile's first batch, and the row pointers of the tile after it
+                load_rp(rpnn, tile_n2 < ntiles ? tile_n2 : ntiles);   // tile ntiles: every pointer reads 0 or row_ptr[N]
+                load_first_batch(rpn, offsn, w0n);
+            }                                    // PIPE: x was asked for during the previous tile
             // longest row of the lane group, and whether one of its rows is out of the buffer's reach
             int longest = rp[1] - rp[0];
 #pragma unroll
@@ -327,11 +340,21 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
                     }
                 }
             }
-            // rotate the look-ahead
+            if constexpr (!PIPE) {
+                // rotate the look-ahead
 #pragma unroll
-            for (int i = 0; i < RN; ++i) { rp[i] = rpn[i]; rpn[i] = rpnn[i]; }
+                for (int i = 0; i < RN; ++i) { rp[i] = rpn[i]; rpn[i] = rpnn[i]; }
 #pragma unroll
-            for (int rd = 0; rd < ROUNDS; ++rd) { offs[rd] = offsn[rd]; w0[rd] = w0n[rd]; }
+                for (int rd = 0; rd < ROUNDS; ++rd) { offs[rd] = offsn[rd]; w0[rd] = w0n[rd]; }
+            } else {
+                // the next tile's gathers, the first batch of the tile after it, the row pointers of the third
+                __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+#pragma unroll
+                for (int rd = 0; rd < ROUNDS; ++rd) gather4<G, 0>(h_rsrc, offq[rd], tx_off, x[rd]);
+                const int tile_n3 = tile_n2 + nwaves;
+                load_rp(rpnn, tile_n3 < ntiles ? tile_n3 : ntiles);
+                load_first_batch(rpq, offsn, w0n);
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
         GNNHIP_PHASE_ACC(3);
@@ -382,6 +405,13 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
             buf_store4(out_rsrc, out_off + rd * kRowBytes, 0, relu_ref4(v));
         }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");     // the tile is rewritten by the next iteration
+        if constexpr (PIPE && !DENSE) {
+            // by now the look-ahead requests have arrived: shift them by one tile
+#pragma unroll
+            for (int i = 0; i < RN; ++i) { rp[i] = rpn[i]; rpn[i] = rpq[i]; rpq[i] = rpnn[i]; }
+#pragma unroll
+            for (int rd = 0; rd < ROUNDS; ++rd) { offs[rd] = offq[rd]; w0[rd] = wq[rd]; offq[rd] = offsn[rd]; wq[rd] = w0n[rd]; }
+        }
         tile_id = tile_n1;
         tile_n1 = tile_n2;
         tile_n2 += nwaves;
@@ -390,10 +420,10 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
     GNNHIP_PHASE_FINI
 }
 
-template <int C, bool DENSE, bool RELU_IN>
-int launch_level_stream(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-                        const float* W, const float* msg, const float* bias, float* h_out, const HubPlan& hubs,
-                        hipStream_t s)
+template <int C, bool DENSE, bool RELU_IN, bool PIPE>
+int launch_level_stream_p(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
+                          const float* W, const float* msg, const float* bias, float* h_out, const HubPlan& hubs,
+                          hipStream_t s)
 {
     const long long ntiles = ((long long)N + 15) / 16;
     long long blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
@@ -401,10 +431,25 @@ int launch_level_stream(int N, const int* row_ptr, const int* col_idx, const flo
     constexpr int kMinW = (C == 64 && !DENSE) ? 3 : 4;    // hidden 64 needs 128 registers and spills for four
     const long long resident = (long long)kNumCU * kMinW;  // a workgroup puts one wavefront on each SIMD
     if (blocks > resident) blocks = resident;              // persistent beyond this
-    hipLaunchKernelGGL((s2v_level_stream_kernel<C, DENSE, kWLds, kMinW, RELU_IN>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL((s2v_level_stream_kernel<C, DENSE, kWLds, kMinW, RELU_IN, PIPE>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
                        N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs.row_slot, hubs.agg, hubs.ld);
     GNNHIP_LAUNCH_CHECK("s2v_level_stream");
     return GNNHIP_OK;
+}
+
+template <int C, bool DENSE, bool RELU_IN>
+int launch_level_stream(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
+                        const float* W, const float* msg, const float* bias, float* h_out, const HubPlan& hubs,
+                        hipStream_t s)
+{
+    // Gathers issued a tile ahead pay once every wavefront has several tiles (116,000 nodes: 35 -> 32 us,
+    // uniform random graph of 1M rows, 2 entries per row: 223 -> 205 us); with one or two tiles per
+    // wavefront the longer start of that variant costs more than it gains (7,450 nodes: +1 us per level).
+    if constexpr (C == 64 && !DENSE) {
+        if (N >= kPipeMinRows)
+            return launch_level_stream_p<C, DENSE, RELU_IN, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
+    }
+    return launch_level_stream_p<C, DENSE, RELU_IN, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
 }
 
 template <int C>
