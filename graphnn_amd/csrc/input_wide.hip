@@ -12,6 +12,7 @@
 //
 // Algorithmic bytes: 4 N (K + 2 C) + 4 K C; flops 2 N K C.  HBM-bound (the two outputs).
 #include "gnnhip_internal.h"
+#include "buffer_addr.h"
 
 namespace gnnhip {
 namespace {
@@ -19,20 +20,6 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / kWave;       // 4
 constexpr int kTileRows = 64;
-
-using rsrc_t = __amdgpu_buffer_rsrc_t;
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-constexpr int kRsrcWord3 = 0x00020000;       // raw buffer of 32-bit data on gfx9-family hardware
-
-__device__ __forceinline__ rsrc_t make_rsrc(const void* base, unsigned bytes)
-{
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, kRsrcWord3);
-}
-__device__ __forceinline__ void buf_store4(rsrc_t r, int voff, const float4& x)
-{
-    const u32x4 v = {__float_as_uint(x.x), __float_as_uint(x.y), __float_as_uint(x.z), __float_as_uint(x.w)};
-    __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, 0, 0);
-}
 
 // KS = contraction steps of four: K <= 4 KS.
 template <int C, int KS>
@@ -109,8 +96,8 @@ __global__ __launch_bounds__(kBlock) void s2v_input_wide_kernel(
 #pragma unroll
             for (int jb = 0; jb < NB; ++jb) {
                 const float4 v = make_float4(acc[jb][0], acc[jb][1], acc[jb][2], acc[jb][3]);
-                buf_store4(msg_rsrc, voff + 64 * jb, v);
-                if (h0) buf_store4(h0_rsrc, voff + 64 * jb, relu_ref4(v));
+                buf_store4(msg_rsrc, voff + 64 * jb, 0, v);
+                if (h0) buf_store4(h0_rsrc, voff + 64 * jb, 0, relu_ref4(v));
             }
         }
     }

@@ -45,6 +45,7 @@
 //     flight and waits at the top of the next block.  One explicit wait after
 //     the contraction removes that.
 #include "gnnhip_internal.h"
+#include "buffer_addr.h"
 
 // Phase accounting for a timing build of this file; expands to nothing in the library.
 #ifndef GNNHIP_PHASE_ACC
@@ -65,33 +66,9 @@ template <int VEC> struct VecT;
 template <> struct VecT<2> { using type = float2; };
 template <> struct VecT<4> { using type = float4; };
 
-// Buffer addressing: the memory instruction takes a 128-bit descriptor (base, size), a per-lane 32-bit
-// offset and a scalar 32-bit offset, so a gathered row costs one scalar shift and no per-lane address
-// arithmetic, and lanes whose offset lies past the size are dropped by the hardware (no predication).
-using rsrc_t = __amdgpu_buffer_rsrc_t;
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-constexpr int kRsrcWord3 = 0x00020000;           // raw buffer of 32-bit data on gfx9-family hardware
-
-__device__ __forceinline__ rsrc_t make_rsrc(const void* base, unsigned bytes)
-{
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, kRsrcWord3);
-}
-__device__ __forceinline__ float4 buf_load4(rsrc_t r, int voff, int soff)
-{
-    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
-    return make_float4(__uint_as_float(v[0]), __uint_as_float(v[1]), __uint_as_float(v[2]), __uint_as_float(v[3]));
-}
-__device__ __forceinline__ float2 buf_load2(rsrc_t r, int voff, int soff)
-{
-    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
-    return make_float2(__uint_as_float(v[0]), __uint_as_float(v[1]));
-}
-__device__ __forceinline__ void buf_store4(rsrc_t r, int voff, int soff, const float4& x)
-{
-    const u32x4 v = {__float_as_uint(x.x), __float_as_uint(x.y), __float_as_uint(x.z), __float_as_uint(x.w)};
-    __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, soff, 0);
-}
+// Buffer addressing (buffer_addr.h): the memory instruction takes a 128-bit descriptor (base, size), a
+// per-lane 32-bit offset and a scalar 32-bit offset, so a gathered row costs one scalar shift and no
+// per-lane address arithmetic, and lanes whose offset lies past the size are dropped by the hardware.
 template <int VEC> struct BufLoad;
 template <> struct BufLoad<4> { static __device__ __forceinline__ float4 get(rsrc_t r, int v, int s) { return buf_load4(r, v, s); } };
 template <> struct BufLoad<2> { static __device__ __forceinline__ float2 get(rsrc_t r, int v, int s) { return buf_load2(r, v, s); } };
