@@ -93,6 +93,7 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const float* __restrict__ 
 
 constexpr int kWaveReadoutMinGraphs = 1024;        // below this a workgroup per graph
 constexpr int kWaveReadoutMaxMeanNodes = 2048;     // mean nodes per graph
+constexpr int kBlockReadoutMaxGraphsWide = 4096;   // hidden 128/256: above this SpMM + GEMM
 
 int readout_any(int B, int N, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                 const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
@@ -105,7 +106,10 @@ int readout_any(int B, int N, int C, int H, int Q, const int* s_row_ptr, const i
     if (B >= kWaveReadoutMinGraphs && (long long)N <= (long long)B * kWaveReadoutMaxMeanNodes)
         rc = readout_wave_dispatch(B, C, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
-    rc = readout_dispatch(B, C, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
+    // hidden 128/256: a workgroup per graph up to a few thousand graphs (256 graphs, hidden 256: 20 us against
+    // 67 us for the seven launches below); 10,000 graphs: 116 against 106 us
+    if (C <= 64 || B <= kBlockReadoutMaxGraphsWide)
+        rc = readout_dispatch(B, C, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
     if ((rc = spmm_dispatch(B, C, (long long)N, 1.f, s_row_ptr, s_col_idx, s_val, h, C, 0.f, pool, C, s))) return rc;
     if ((rc = gemm_dispatch(0, 0, B, H, C, 1.f, pool, C, Wh1, H, 0.f, hidden, H, s))) return rc;

@@ -654,6 +654,8 @@ int readout_dispatch(int B, int C, int H, int Q, const int* s_row_ptr, const int
     case 16: return launch_readout<16>(B, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
     case 32: return launch_readout<32>(B, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
     case 64: return launch_readout<64>(B, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
+    case 128: return launch_readout<128>(B, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
+    case 256: return launch_readout<256>(B, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
     }
     return GNNHIP_EUNSUPPORTED;
 }
