@@ -126,6 +126,44 @@ def test_host_api_forward_backward_checkpoint(gpu, oracle, tmp_path, C):
     assert np.frombuffer(blob[:24], dtype=np.uint64).tolist() == [2, C, C]       # "w_conv" sorts first
 
 
+def test_host_api_large_batch_takes_the_separate_kernels(gpu, oracle, tmp_path):
+    """a batch of more than 20,000 nodes: the inference plan still folds the forward into one step, which now
+    calls the whole-forward entry of the library (separate kernels, h0 not stored) instead of the one-launch
+    kernel; loss and accuracy of that plan against the reference path, and against the training plan of the
+    same driver, which runs every factor on its own"""
+    exe = os.path.join(BUILD, "host_forward_check")
+    assert os.path.exists(exe), "build the host layer first: make -C graphnn_amd/host"
+    K, C, H, Q, L = 7, 64, 32, 2, 3
+    batch = synth.molecule_batch(777, 900, K, Q, size_mode="uniform", size_lo=4, size_hi=60)
+    assert batch.num_nodes > 20000
+    w = synth.make_weights(synth.Stream(777), K, C, H, Q)
+    d = str(tmp_path)
+    synth.write_graphnn_txt(batch, d + "/graphs.txt")
+    for name, m in (("w_n2l", w.W_n2l), ("w_conv", w.W_conv), ("w_h1", w.W_h1), ("w_h2", w.W_h2)):
+        m.astype(np.float32).tofile(d + "/%s.bin" % name)
+    r = subprocess.run([exe, d, str(K), str(C), str(H), str(Q), str(L)], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    out = np.fromfile(d + "/out.bin", dtype=np.float32)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    want = oracle.forward(a, s, batch.one_hot(), w, L, batch.label_csr())
+    B, N = batch.num_graphs, batch.num_nodes
+    n_steps, n_fused, loss, acc = out[:4]
+    assert n_fused == 1 and n_steps == 9
+    logits = out[4:4 + B * Q].reshape(B, Q)
+    assert max_rel(logits, want["logits"]) < PARITY_TOL
+    assert abs(loss - want["scalars"][0]) <= 1e-4 * abs(want["scalars"][0])
+    assert abs(acc - want["scalars"][1]) <= 1e-6
+    pos = 4 + B * Q
+    n_steps_t, n_fused_t, loss_t, acc_t = out[pos:pos + 4]
+    assert n_fused_t == 0 and n_steps_t == 4 * L + 14
+    logits_t = out[pos + 4:pos + 4 + B * Q].reshape(B, Q)
+    h_final = out[pos + 4 + B * Q:pos + 4 + B * Q + N * C].reshape(N, C)
+    assert max_rel(logits_t, want["logits"]) < PARITY_TOL
+    assert max_rel(h_final, want["h"][L]) < PARITY_TOL
+    assert abs(loss_t - loss) <= 1e-5 * abs(loss) and acc_t == acc
+
+
 def test_reference_example_runs_unchanged(gpu, tmp_path):
     """graphnn's examples/graph_classification/src/kernel_mean_field.cpp, not a line changed, built against
     the host layer (only possible where the graphnn source tree exists; the binary then travels)."""
