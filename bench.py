@@ -178,6 +178,50 @@ def time_large_batch(dev, B=30000):
             "forward_one_launch": {"avg_ms": ms_one, "graphs_per_s": B / (ms_one * 1e-3)}}
 
 
+def time_device_batch_assembly(dev):
+    """CSR of A from the flat edge list of configuration 4 on the device (stable radix sort) and the CSR
+    transposition used by the backward pass, beside the numpy host builder for the same edge list."""
+    import torch
+    from graphnn_amd import batching, ops, synth
+    batch, _, _ = synth.make_config(4)
+    N, E = batch.num_nodes, batch.num_edges
+    t0 = time.perf_counter()
+    a = batching.node2node_csr(N, batch.edge_x, batch.edge_y)
+    host_ms = (time.perf_counter() - t0) * 1e3
+    ex = torch.from_numpy(np.ascontiguousarray(batch.edge_x, dtype=np.int32)).to(dev)
+    ey = torch.from_numpy(np.ascontiguousarray(batch.edge_y, dtype=np.int32)).to(dev)
+    ms_group = _event_ms(lambda: ops.csr_group(N, ey, ex), 20)
+    rp, ci, v = ops.csr_group(N, ey, ex)
+    same = bool(torch.equal(rp.cpu(), torch.from_numpy(a[0])) and torch.equal(ci.cpu(), torch.from_numpy(a[1])))
+    ms_t = _event_ms(lambda: ops.csr_transpose(rp, ci, v, N, N), 20)
+    return {"workload": "configuration 4 edge list: %d nodes, %d directed edges" % (N, E),
+            "csr_group": {"avg_ms": ms_group, "edges_per_s": E / (ms_group * 1e-3), "equals_host_builder": same},
+            "csr_transpose": {"avg_ms": ms_t, "edges_per_s": E / (ms_t * 1e-3)},
+            "numpy_host_builder_ms": host_ms}
+
+
+def training_step_host_layer(host, reps=100):
+    """One training iteration of graphnn's example loop through the C++ host layer (FeedForward in the TRAIN
+    phase, BackPropagate, momentum-SGD update) on the configuration-2 batch; child process as end_to_end."""
+    import subprocess
+    import tempfile
+    from graphnn_amd import synth
+    exe = os.path.join(ROOT, "graphnn_amd", "host", "build", "host_forward_bench")
+    if not os.path.exists(exe):
+        return {"skipped": "graphnn_amd/host/build/host_forward_bench is not built"}
+    cfg = host["cfg"]
+    with tempfile.TemporaryDirectory() as d:
+        synth.write_graphnn_txt(host["batch"], os.path.join(d, "graphs.txt"))
+        r = subprocess.run([exe, d] + [str(cfg[k]) for k in ("K", "C", "H", "Q", "L")] + [str(reps), "train"],
+                           capture_output=True, text=True, timeout=300)
+    if r.returncode != 0:
+        return {"skipped": "host_forward_bench train failed: " + (r.stderr or r.stdout)[-300:]}
+    res = json.loads(r.stdout.strip().splitlines()[-1])
+    res["what"] = ("GetBatch-style host batch build + FactorGraph::FeedForward(TRAIN) + BackPropagate + "
+                   "MomentumSGDOptimizer::Update per batch, operator-by-operator plan")
+    return res
+
+
 def time_cfg5(dev, scale=22):
     """Configuration 5: R-MAT (a=.57, b=c=.19), 16 entries per row, generated on the device with the
     same recursive-quadrant rule as synth.rmat_csr (torch's generator, so not the parity inputs);
@@ -366,7 +410,9 @@ def main():
     out["end_to_end"] = end_to_end_host_layer(host)
 
     if args.extra:
-        out["extra"] = {"cfg4_level": time_level_cfg4(dev), "large_batch": time_large_batch(dev), "cfg5": time_cfg5(dev)}
+        out["extra"] = {"cfg4_level": time_level_cfg4(dev), "large_batch": time_large_batch(dev), "cfg5": time_cfg5(dev),
+                        "device_batch_assembly": time_device_batch_assembly(dev),
+                        "training_step": training_step_host_layer(host)}
 
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline(host)
     print(json.dumps(out))

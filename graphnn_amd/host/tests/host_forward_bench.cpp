@@ -2,9 +2,12 @@
 // 140-160): build the batch on the host (GraphStruct lists, one-hot node features, label CSR), copy it to
 // the device, FactorGraph::FeedForward in the TEST phase, read loss and accuracy back.
 //
-//   host_forward_bench <dir> K C H Q L reps
+//   host_forward_bench <dir> K C H Q L reps [train]
 //   <dir>/graphs.txt  dataset in graphnn's txt layout (all graphs form the batch); weights are random
 // Prints one JSON line with microseconds per batch: whole, host batch build, copies + forward + read-back.
+// With "train" every batch runs what the example's training loop runs (nn_common.h:158-171):
+// FeedForward in the TRAIN phase, BackPropagate from the loss, one momentum-SGD update; the loss is read
+// back once at the end, as the example only reads it on report iterations.
 #include <chrono>
 #include <cstdio>
 #include <fstream>
@@ -26,7 +29,8 @@ static double us_since(Clock::time_point t0)
 
 int main(int argc, char** argv)
 {
-    ASSERT(argc == 8, "usage: host_forward_bench <dir> K C H Q L reps");
+    ASSERT(argc == 8 || argc == 9, "usage: host_forward_bench <dir> K C H Q L reps [train]");
+    const bool train = argc == 9 && std::string(argv[8]) == "train";
     const std::string dir = argv[1];
     const size_t K = atoi(argv[2]), C = atoi(argv[3]), H = atoi(argv[4]), Q = atoi(argv[5]);
     const int L = atoi(argv[6]), reps = atoi(argv[7]);
@@ -92,6 +96,8 @@ int main(int argc, char** argv)
     feed["label"] = &label;
     feed["graph"] = &graph;
     std::vector< std::shared_ptr<Variable> > targets = {loss, acc};
+    std::vector< std::shared_ptr<Variable> > objs = {loss};
+    MomentumSGDOptimizer<mode, Dtype> learner(&model, 0.001f, 0.9f, 0.0001f);
 
     double t_build = 0, t_device = 0;
     float checksum = 0;
@@ -123,15 +129,23 @@ int main(int argc, char** argv)
         const Clock::time_point t1 = Clock::now();
         input.CopyFrom(x_cpu);
         label.CopyFrom(y_cpu);
-        fg.FeedForward(targets, feed, Phase::TEST);      // builds the CSR of A and S on the host, copies, runs
-        checksum += loss->AsScalar() + acc->AsScalar();
+        if (train) {
+            fg.FeedForward(targets, feed, Phase::TRAIN);
+            fg.BackPropagate(objs);
+            learner.Update();
+            if (it + 1 == reps + warm || it + 1 == warm) checksum += loss->AsScalar();     // drains the stream
+        } else {
+            fg.FeedForward(targets, feed, Phase::TEST);  // builds the CSR of A and S on the host, copies, runs
+            checksum += loss->AsScalar() + acc->AsScalar();
+        }
         const double d = us_since(t1);
         if (it >= warm) { t_build += b; t_device += d; }
     }
     GpuHandle::Destroy();
-    printf("{\"graphs\": %d, \"nodes\": %zu, \"reps\": %d, \"us_per_batch\": %.2f, \"us_host_batch_build\": %.2f, "
-           "\"us_csr_copy_forward_readback\": %.2f, \"fused_factors\": %d, \"checksum\": %.6f}\n",
-           num_graph, N, reps, (t_build + t_device) / reps, t_build / reps, t_device / reps,
-           (int)fg.LastPlanFusedCount(), checksum);
+    printf("{\"graphs\": %d, \"nodes\": %zu, \"reps\": %d, \"mode\": \"%s\", \"us_per_batch\": %.2f, \"us_host_batch_build\": %.2f, "
+           "\"%s\": %.2f, \"fused_factors\": %d, \"plan_steps\": %d, \"checksum\": %.6f}\n",
+           num_graph, N, reps, train ? "train" : "test", (t_build + t_device) / reps, t_build / reps,
+           train ? "us_csr_copy_forward_backward_update" : "us_csr_copy_forward_readback", t_device / reps,
+           (int)fg.LastPlanFusedCount(), (int)fg.LastPlanFactorCount(), checksum);
     return 0;
 }
