@@ -34,6 +34,7 @@ SIGNATURES = {
     "gnnhip_memcpy_d2h": [_P, _P, _Z, _P],
     "gnnhip_memcpy_d2d": [_P, _P, _Z, _P],
     "gnnhip_memset0": [_P, _Z, _P],
+    "gnnhip_memset0_batch": [_I, _P, _P, _P],
     "gnnhip_stream_sync": [_P],
     "gnnhip_spmm_csr_f32": [_I, _I, _I, _I, _F, _P, _P, _P, _P, _I, _F, _P, _I, _P],
     "gnnhip_csr_group_i32": [_I, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P],

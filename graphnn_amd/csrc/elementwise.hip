@@ -103,6 +103,29 @@ __global__ __launch_bounds__(kBlock) void zero_kernel(unsigned char* p, size_t h
     if (tail0 + gid < total) p[tail0 + gid] = 0;    // fewer than 16 tail bytes
 }
 
+// The same for up to kZeroBatch buffers in one launch: blockIdx.y picks the buffer.
+constexpr int kZeroBatch = 48;
+struct ZeroBatch {
+    unsigned char* p[kZeroBatch];
+    size_t bytes[kZeroBatch];
+};
+__global__ __launch_bounds__(kBlock) void zero_batch_kernel(ZeroBatch b)
+{
+    unsigned char* p = b.p[blockIdx.y];
+    const size_t total = b.bytes[blockIdx.y];
+    size_t head = (16 - (reinterpret_cast<uintptr_t>(p) & 15u)) & 15u;
+    if (head > total) head = total;
+    const size_t n16 = (total - head) >> 4;
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    const size_t gid = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    uint4* body = reinterpret_cast<uint4*>(p + head);
+    const uint4 z = make_uint4(0u, 0u, 0u, 0u);
+    for (size_t i = gid; i < n16; i += stride) body[i] = z;
+    if (gid < head) p[gid] = 0;
+    const size_t tail0 = head + (n16 << 4);
+    if (tail0 + gid < total) p[tail0 + gid] = 0;
+}
+
 inline unsigned grid_for(size_t work_items)
 {
     size_t b = (work_items + kBlock - 1) / kBlock;
@@ -226,6 +249,33 @@ int gnnhip_memset0(void* device_ptr, size_t bytes, void* stream)
     size_t n16 = (bytes - head) >> 4;
     hipLaunchKernelGGL(zero_kernel, dim3(grid_for(n16 ? n16 : 1)), dim3(kBlock), 0, as_stream(stream), p, head, n16, bytes);
     GNNHIP_LAUNCH_CHECK("zero");
+    return GNNHIP_OK;
+}
+
+int gnnhip_memset0_batch(int n, void* const* device_ptrs, const size_t* bytes, void* stream)
+{
+    GNNHIP_REQUIRE(n >= 0 && (n == 0 || (device_ptrs && bytes)), "bad arguments in memset0_batch");
+    if (int rc = require_ready()) return rc;
+    int i = 0;
+    while (i < n) {
+        ZeroBatch b;
+        int m = 0;
+        size_t largest = 0;
+        for (; i < n && m < kZeroBatch; ++i) {
+            if (bytes[i] == 0) continue;
+            GNNHIP_REQUIRE(device_ptrs[i] != nullptr, "null pointer in memset0_batch");
+            b.p[m] = static_cast<unsigned char*>(device_ptrs[i]);
+            b.bytes[m] = bytes[i];
+            if (bytes[i] > largest) largest = bytes[i];
+            ++m;
+        }
+        if (m == 0) break;
+        const size_t n16 = largest >> 4;
+        unsigned gx = grid_for(n16 ? n16 : 1);
+        if (gx > 1024u) gx = 1024u;
+        hipLaunchKernelGGL(zero_batch_kernel, dim3(gx, (unsigned)m), dim3(kBlock), 0, as_stream(stream), b);
+        GNNHIP_LAUNCH_CHECK("zero_batch");
+    }
     return GNNHIP_OK;
 }
 

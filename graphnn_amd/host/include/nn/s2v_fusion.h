@@ -402,9 +402,20 @@ inline void FactorGraph::BackPropagate(std::vector<VarPtr> targets, uint n_threa
     const size_t nv = var_list.size(), nf = factor_list.size();
 
     var_has_grad.assign(nv, false);
+    // the reference clears the gradients one by one (src/nn/factor_graph.cpp:190-196); device gradients are
+    // collected and cleared in one launch
+    std::vector<void*> zero_ptr;
+    std::vector<size_t> zero_bytes;
     for (size_t v = 0; v < nv; ++v)
         if (!isConst[v])
-            if (auto* d = dynamic_cast<IDifferentiable*>(var_list[v].get())) d->ZeroGrad();
+            if (auto* d = dynamic_cast<IDifferentiable*>(var_list[v].get())) {
+                void* p = nullptr;
+                size_t bytes = 0;
+                if (!d->GradBuffer(&p, &bytes)) d->ZeroGrad();
+                else if (bytes) { zero_ptr.push_back(p); zero_bytes.push_back(bytes); }
+            }
+    if (!zero_ptr.empty())
+        GNN_HIP(gnnhip_memset0_batch((int)zero_ptr.size(), zero_ptr.data(), zero_bytes.data(), GpuHandle::Stream()));
     for (auto& p : targets) {
         const size_t v = VarIdx(p);
         ASSERT(var_nodes[v].consumers.empty(), "only allow backprop from top variables");

@@ -20,7 +20,24 @@ public:
     virtual ~IDifferentiable() {}
     virtual void ZeroGrad() = 0;
     virtual void OnesGrad() = 0;
+    // Shapes the gradient like the value and reports its device buffer WITHOUT clearing it, so that the
+    // caller can clear many gradients in one launch; false: the gradient has no such buffer, use ZeroGrad.
+    virtual bool GradBuffer(void** device_ptr, size_t* bytes) { (void)device_ptr; (void)bytes; return false; }
 };
+
+namespace detail
+{
+template<typename mode, typename Dtype>
+inline bool grad_buffer(DTensor<mode, Dtype>&, RowSpTensor<mode, Dtype>&, void**, size_t*) { return false; }
+inline bool grad_buffer(DTensor<GPU, float>& value, RowSpTensor<GPU, float>& grad, void** device_ptr, size_t* bytes)
+{
+    if (!(grad.shape == value.shape)) grad.Reshape(value.shape.dims);
+    grad.is_full = true;
+    *device_ptr = grad.data->ptr;
+    *bytes = sizeof(float) * grad.shape.Count();
+    return true;
+}
+}  // namespace detail
 
 class Variable
 {
@@ -93,6 +110,7 @@ public:
         grad.Reshape(value.shape.dims);
         grad.Full().Fill(1);
     }
+    virtual bool GradBuffer(void** device_ptr, size_t* bytes) override { return detail::grad_buffer(value, grad, device_ptr, bytes); }
     void Serialize(FILE* fid) { value.Serialize(fid); }
     void Deserialize(FILE* fid) { value.Deserialize(fid); }
 

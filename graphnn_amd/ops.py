@@ -316,6 +316,15 @@ def memset0(t):
     return t
 
 
+def memset0_batch(tensors):
+    """zero-fill several device buffers in one launch"""
+    n = len(tensors)
+    ptrs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in tensors])
+    sizes = (ctypes.c_size_t * n)(*[t.numel() * t.element_size() for t in tensors])
+    check(_lib().gnnhip_memset0_batch(n, ptrs, sizes, _stream()))
+    return tensors
+
+
 # ---- backward-pass entry points
 def spmm_t(row_ptr, col_idx, val, B, m, k, alpha=1.0, beta=0.0, out=None):
     """out[k,n] = alpha * A^T * B + beta * out, A CSR [m,k], B [m,n]"""

@@ -68,6 +68,9 @@ int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void
 int gnnhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
 int gnnhip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream);
 int gnnhip_memset0(void* device_ptr, size_t bytes, void* stream);
+/* n buffers zeroed in one launch (the gradient tensors FactorGraph::BackPropagate clears one by one,
+ * src/nn/factor_graph.cpp:190-196); entries with 0 bytes are skipped. */
+int gnnhip_memset0_batch(int n, void* const* device_ptrs, const size_t* bytes, void* stream);
 int gnnhip_stream_sync(void* stream);
 
 /* ---- C[m,n] = alpha * A * B + beta * C, A CSR [m,k], B dense [k,n].

@@ -224,6 +224,20 @@ def test_memset0(gpu, n, offset):
     assert np.all(got[offset:offset + n] == 0) and np.all(got[:offset] == 7) and np.all(got[offset + n:] == 7)
 
 
+def test_memset0_batch(gpu):
+    """many buffers in one launch: ragged starts and lengths, an empty one, more buffers than one launch takes"""
+    import torch
+    from graphnn_amd import ops
+    rng = np.random.default_rng(3)
+    sizes = [0, 1, 15, 16, 17, 1000, 4097, 1 << 20] + [int(x) for x in rng.integers(1, 5000, 100)]
+    offs = [int(x) for x in rng.integers(0, 16, len(sizes))]
+    bufs = [torch.full((n + o + 9,), 7, dtype=torch.uint8, device=gpu) for n, o in zip(sizes, offs)]
+    ops.memset0_batch([b[o:o + n] for b, n, o in zip(bufs, sizes, offs)])
+    for b, n, o in zip(bufs, sizes, offs):
+        got = _n(b)
+        assert np.all(got[o:o + n] == 0) and np.all(got[:o] == 7) and np.all(got[o + n:] == 7), (n, o)
+
+
 # ------------------------------------------------------------------ softmax family
 @pytest.mark.parametrize("rows,cols", [(20, 200), (256, 2), (7, 1), (3, 64), (5, 65), (2, 5000)])
 def test_row_softmax(gpu, oracle, rows, cols):
