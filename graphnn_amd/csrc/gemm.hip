@@ -3,9 +3,10 @@
 // The mean-field path only has tall-and-skinny products (m = nodes or graphs,
 // n and k = label types / hidden sizes <= 256), which are HBM-bound: every A
 // element is used n times from LDS, every B element lives in L2.  The kernel is
-// a classic LDS-tiled register-blocked SGEMM: a 64 x 64 output tile per 256-lane
-// workgroup, 4 x 4 outputs per lane, K walked in steps of 16 through two LDS
-// tiles.  Edges are handled by bounds-checked tile loads (zeros) and stores.
+// an LDS-tiled SGEMM on the FP32 matrix cores: a 64 x 64 output tile per 256-lane
+// workgroup, 16 rows x 64 columns per wavefront as four v_mfma_f32_16x16x4_f32
+// accumulators, K walked in steps of 16 through two LDS tiles.  Edges are handled
+// by bounds-checked tile loads (zeros) and stores.
 // Bound: HBM for the shapes above; algorithmic bytes 4(mk + kn + mn).
 //
 // Weight gradients are the opposite shape: op(A)^T * G with a small output (hidden x hidden) and k = nodes.
@@ -25,21 +26,25 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
     const float* __restrict__ B, int ldb, float beta, float* C, int ldc, int k_chunk, float* __restrict__ partial)
 {
     // partial != nullptr: workgroup z handles k in [z k_chunk, (z+1) k_chunk) and stores its raw sums to
-    // partial[z][m][n]; otherwise one workgroup walks all of k and finishes C itself
-    __shared__ float As[BK][BM + 4];     // As[p][i] = op(A)[row0 + i][k0 + p]
-    __shared__ float Bs[BK][BN + 4];     // Bs[p][j] = op(B)[k0 + p][col0 + j]
+    // partial[z][m][n]; otherwise one workgroup walks all of k and finishes C itself.
+    //
+    // Both tiles sit in LDS with k contiguous, so that a lane fetches its four k values of a step with one
+    // 128-bit read.  Wavefront w owns the output rows 16 w .. 16 w + 15 of the tile and all 64 columns: four
+    // accumulators of v_mfma_f32_16x16x4_f32 with the operand roles swapped (out^T = B^T * A^T), which leaves
+    // lane (q = lane/16, t = lane%16) with row t and the columns 16 jb + 4 q .. + 3 of block jb.
+    constexpr int LD = BK + 4;
+    __shared__ float As[BM][LD];         // As[i][p] = op(A)[row0 + i][k0 + p]
+    __shared__ float Bs[BN][LD];         // Bs[j][p] = op(B)[k0 + p][col0 + j]
 
     const int tid = threadIdx.x;
-    const int tx = tid & 15;             // output columns tx*4 .. tx*4+3
-    const int ty = tid >> 4;             // output rows    ty*4 .. ty*4+3
+    const int lane = tid & (kWave - 1), wave = tid / kWave;
+    const int q = lane >> 4, t = lane & 15;
     const long long row0 = (long long)blockIdx.x * BM;
     const int col0 = blockIdx.y * BN;
 
-    float acc[4][4];
+    mfma_f4 acc[BN / 16];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int jb = 0; jb < BN / 16; ++jb) acc[jb] = mfma_f4{0.f, 0.f, 0.f, 0.f};
 
     const int k_lo = partial ? (int)blockIdx.z * k_chunk : 0;
     const int k_hi = partial ? min(k, k_lo + k_chunk) : k;
@@ -51,7 +56,7 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
         for (int e = 0; e < 4; ++e) {
             const int idx = tid + e * kBlock;        // 0 .. 1023
             {
-                // A tile: choose the fast index to follow memory
+                // A tile: the fast index follows memory
                 int i, p;
                 if (TA) { i = idx & (BM - 1); p = idx >> 6; }       // stored A is [k][m]: i contiguous
                 else    { p = idx & (BK - 1); i = idx >> 4; }       // stored A is [m][k]: p contiguous
@@ -78,40 +83,41 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int idx = tid + e * kBlock;
-            if (TA) As[idx >> 6][idx & (BM - 1)] = ra[e]; else As[idx & (BK - 1)][idx >> 4] = ra[e];
-            if (TB) Bs[idx & (BK - 1)][idx >> 4] = rb[e]; else Bs[idx >> 6][idx & (BN - 1)] = rb[e];
+            if (TA) As[idx & (BM - 1)][idx >> 6] = ra[e]; else As[idx >> 4][idx & (BK - 1)] = ra[e];
+            if (TB) Bs[idx >> 4][idx & (BK - 1)] = rb[e]; else Bs[idx & (BN - 1)][idx >> 6] = rb[e];
         }
         __syncthreads();
         if (k0 + BK < k_hi) fetch(k0 + BK);
+        // lane (q, t): k = 4 q + s at instruction s of the step
+        const float4 a = *reinterpret_cast<const float4*>(&As[wave * 16 + t][4 * q]);
 #pragma unroll
-        for (int p = 0; p < BK; ++p) {
-            const float4 a = *reinterpret_cast<const float4*>(&As[p][ty * 4]);
-            const float4 b = *reinterpret_cast<const float4*>(&Bs[p][tx * 4]);
-            const float av[4] = {a.x, a.y, a.z, a.w};
-            const float bv[4] = {b.x, b.y, b.z, b.w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * bv[j];
+        for (int jb = 0; jb < BN / 16; ++jb) {
+            const float4 b = *reinterpret_cast<const float4*>(&Bs[jb * 16 + t][4 * q]);
+            acc[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(b.x, a.x, acc[jb], 0, 0, 0);
+            acc[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(b.y, a.y, acc[jb], 0, 0, 0);
+            acc[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(b.z, a.z, acc[jb], 0, 0, 0);
+            acc[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(b.w, a.w, acc[jb], 0, 0, 0);
         }
         __syncthreads();
     }
 
+    // lane (q, t) holds out[row0 + 16 wave + t][col0 + 16 jb + 4 q + i], i = 0..3
+    const long long gi = row0 + wave * 16 + t;
+    if (gi < m) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const long long gi = row0 + ty * 4 + i;
-        if (gi >= m) continue;
+        for (int jb = 0; jb < BN / 16; ++jb) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int gj = col0 + tx * 4 + j;
-            if (gj >= n) continue;
-            if (partial) {
-                partial[((size_t)blockIdx.z * m + gi) * n + gj] = acc[i][j];
-                continue;
+            for (int i = 0; i < 4; ++i) {
+                const int gj = col0 + jb * 16 + 4 * q + i;
+                if (gj >= n) continue;
+                if (partial) {
+                    partial[((size_t)blockIdx.z * m + gi) * n + gj] = acc[jb][i];
+                    continue;
+                }
+                float* dst = C + (size_t)gi * ldc + gj;
+                const float r = alpha * acc[jb][i];
+                *dst = (beta == 0.f) ? r : r + beta * (*dst);
             }
-            float* dst = C + (size_t)gi * ldc + gj;
-            const float r = alpha * acc[i][j];
-            *dst = (beta == 0.f) ? r : r + beta * (*dst);
         }
     }
 }
