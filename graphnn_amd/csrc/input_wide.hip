@@ -1,4 +1,4 @@
-// Input stage for wide hidden sizes (C = 128 or 256) and up to 64 label types:
+// Input stage for hidden sizes 128 and 256 (and 64 when only msg is wanted) and up to 64 label types:
 //     msg = X * W_n2l ,  h0 = ReLU(msg)
 // MatMul + ReLU of examples/graph_classification/src/kernel_mean_field.cpp:31-32 in one pass,
 // with the K x C contraction on the FP32 matrix cores.
@@ -128,6 +128,7 @@ int input_wide_dispatch(int N, int K, int C, const float* X, const float* Wn2l, 
 {
     if (K > 64 || !(aligned16(msg) && aligned16(h0))) return GNNHIP_EUNSUPPORTED;
     switch (C) {
+    case 64: return input_wide_c<64>(N, K, X, Wn2l, msg, h0, s);
     case 128: return input_wide_c<128>(N, K, X, Wn2l, msg, h0, s);
     case 256: return input_wide_c<256>(N, K, X, Wn2l, msg, h0, s);
     }
