@@ -11,10 +11,11 @@
 // One persistent workgroup of 8 wavefronts per compute unit.  W never moves
 // after start-up: wavefront w keeps the W^T operand of its C/8 output columns
 // in registers (C = 256: 128 registers per lane, half of the register file of
-// the compute unit across the 8 wavefronts).  Per pass over 64 rows:
-//   1. gather-sum  wavefront w sums the neighbour rows of 8 rows, the whole
+// the compute unit across the 8 wavefronts).  Per pass over TR rows (64; 32 or 16
+// on matrices too small to give every compute unit two 64-row passes):
+//   1. gather-sum  wavefront w sums the neighbour rows of TR/8 rows, the whole
 //                  wavefront across the C columns of a row, six row loads in
-//                  flight, and parks the sums in an LDS tile [64][C+4];
+//                  flight, and parks the sums in an LDS tile [TR][C+4];
 //   2. contraction v_mfma_f32_16x16x4_f32, out^T = W^T * tile^T: the lane
 //                  (q = lane/16, t = lane%16) feeds k = (C/4) q + s at step s, so
 //                  four steps of its tile operand are one 128-bit LDS read, and it
@@ -24,8 +25,8 @@
 // The tile is double-buffered and the gather of pass p+1 is spread, one batch
 // of six row loads per 16-row block, over the contraction of pass p; the CSR
 // indices are fetched one batch (columns, weights) or one pass (row pointers)
-// further ahead still.  Only a wavefront whose 8 rows hold more than 24 entries
-// gathers in the open.
+// further ahead still.  Only a wavefront whose rows hold more than six entries
+// per 16-row block of the pass (24 at TR = 64) gathers in the open.
 //
 // What shaped the code (measured on MI355X):
 //   * While a wavefront streams FP32 matrix instructions, every other
@@ -58,7 +59,6 @@
 namespace gnnhip {
 namespace {
 
-constexpr int kTileRows = 64;                    // rows per pass
 constexpr int kInFlight = 6;                     // row gathers in flight per wavefront
 constexpr int kWaitVmcnt0 = 0x0F70;              // s_waitcnt operand: vmcnt(0), other counters unconstrained
 
@@ -88,7 +88,8 @@ __device__ __forceinline__ void vec_fma(float (&acc)[VEC], float a, const typena
 // instructions and ordinary vector instructions do not overlap: every vector instruction issued by
 // either wavefront of a SIMD takes time away from its matrix pipe.
 // RELU_IN: the gathered rows count as ReLU(row) (the first level reading msg where h0 was not stored)
-template <int C, int WAVES, bool RELU_IN>
+// TR: rows per pass (16, 32 or 64)
+template <int C, int WAVES, bool RELU_IN, int TR>
 __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     int N, int tiles_per_block, const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
     const float* __restrict__ val, const float* __restrict__ h_in, const float* __restrict__ W,
@@ -100,6 +101,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     constexpr int NB = CW / 16;                  // 16-column blocks per wavefront
     constexpr int VEC = C / kWave;               // gathered floats per lane
     constexpr int LDT = C + 4;                   // LDS row stride: rows 0..7 start in distinct 16-byte bank groups
+    constexpr int kTileRows = TR;
     constexpr int RPW = kTileRows / WAVES;       // rows gathered per wavefront per pass
     using vec_t = typename VecT<VEC>::type;
 
@@ -127,7 +129,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     const int tile_end = (int)min((long long)ntiles, (long long)tile_begin + tiles_per_block);
     if (tile_begin >= tile_end) return;
 
-    // ---- loaders.  The 9 row pointers of a pass sit in lanes 0..8 of one vector register; columns
+    // ---- loaders.  The RPW + 1 row pointers of a pass sit in lanes 0..RPW of one vector register; columns
     //      and weights of a batch are uniform and come through scalar loads (weights as bit patterns
     //      so that selecting them stays on the scalar unit).
     auto load_rowptrs = [&](int tile_id) {
@@ -167,7 +169,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
             x[u] = BufLoad<VEC>::get(h_rsrc, lane * (VEC * 4), c[u] * (C * 4));     // N C 4 < 2^32 (host-checked)
     };
 
-    // ---- state of the gather of one pass: entries [e, ee) of the wavefront's 8 rows, taken in order;
+    // ---- state of the gather of one pass: entries [e, ee) of the wavefront's RPW rows, taken in order;
     //      a row goes to LDS when its last entry has been added
     int e = 0, ee = 0, lr = 0, row_end = 0, rpv = 0;
     float* dstp = nullptr;
@@ -366,25 +368,37 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     GNNHIP_PHASE_FINI
 }
 
-template <int C, int WAVES, bool RELU_IN>
-int launch_level_wide(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
+template <int C, int WAVES, bool RELU_IN, int TR>
+int launch_level_wide_t(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
                       const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
 {
     if ((unsigned long long)N * C * 4ull >= (1ull << 32)) return GNNHIP_EUNSUPPORTED;   // 32-bit buffer offsets
+    constexpr int kTileRows = TR;
     const long long ntiles = ((long long)N + kTileRows - 1) / kTileRows;
     const long long per = (ntiles + kNumCU - 1) / kNumCU;            // contiguous run of tiles per workgroup
     const long long blocks = (ntiles + per - 1) / per;
     const size_t smem = sizeof(float) * (2 * kTileRows * (C + 4) + C);
     static bool attr_set = false;                                    // more than 64 KB of LDS has to be asked for
     if (!attr_set) {
-        GNNHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&s2v_level_wide_kernel<C, WAVES, RELU_IN>),
+        GNNHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&s2v_level_wide_kernel<C, WAVES, RELU_IN, TR>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    hipLaunchKernelGGL((s2v_level_wide_kernel<C, WAVES, RELU_IN>), dim3((unsigned)blocks), dim3(WAVES * kWave), smem, s,
+    hipLaunchKernelGGL((s2v_level_wide_kernel<C, WAVES, RELU_IN, TR>), dim3((unsigned)blocks), dim3(WAVES * kWave), smem, s,
                        N, (int)per, row_ptr, col_idx, val, h_in, W, msg, bias, h_out);
     GNNHIP_LAUNCH_CHECK("s2v_level_wide");
     return GNNHIP_OK;
+}
+
+// Rows per pass.  The contraction of a 64-row pass keeps one compute unit's matrix pipes busy for 14 us at
+// C = 256, so a matrix with fewer passes than twice the compute units is cut into shorter ones.
+template <int C, int WAVES, bool RELU_IN>
+int launch_level_wide(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
+                      const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
+{
+    if (N >= 2 * kNumCU * 64) return launch_level_wide_t<C, WAVES, RELU_IN, 64>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    if (N >= 2 * kNumCU * 32) return launch_level_wide_t<C, WAVES, RELU_IN, 32>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    return launch_level_wide_t<C, WAVES, RELU_IN, 16>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
 }
 
 }  // namespace

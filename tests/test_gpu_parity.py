@@ -408,12 +408,13 @@ def test_level_every_row_length_up_to_70(gpu, oracle, C, N):
 
 
 @pytest.mark.parametrize("C", [128, 256])
-def test_wide_level_ragged_rows_and_weights(gpu, oracle, C):
+@pytest.mark.parametrize("N", [5_003, 64 * 300 + 37, 40_037])
+def test_wide_level_ragged_rows_and_weights(gpu, oracle, C, N):
     """wide-hidden kernel: empty rows, rows longer than one 64-entry index batch, a row count that is
-    not a multiple of the 64-row pass, non-unit weights"""
+    not a multiple of the pass, non-unit weights; the three sizes take passes of 16, 32 and 64 rows, each
+    with more passes than compute units take one each"""
     from graphnn_amd import ops
-    rng = np.random.default_rng(90 + C)
-    N = 64 * 300 + 37                                   # more passes than compute units take one each
+    rng = np.random.default_rng(90 + C + N)
     lens = rng.integers(0, 7, N); lens[5] = 700; lens[6] = 0; lens[7] = 0; lens[N - 1] = 130; lens[64:72] = 0
     rp = np.zeros(N + 1, np.int32); np.cumsum(lens, out=rp[1:])
     nnz = int(rp[-1])
