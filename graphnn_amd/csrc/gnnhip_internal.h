@@ -67,6 +67,12 @@ constexpr int kDppXor2 = 0x4E;
 constexpr int kDppHalfMirror = 0x141;   // lane i <-> 7-i inside each group of 8
 constexpr int kDppMirror = 0x140;       // lane i <-> 15-i inside each row of 16
 
+// The wave-wide operations below must be called by a whole wavefront (all 64 lanes active).  After the four
+// DPP steps every lane of a row of 16 holds its row's result; the four rows are then combined through
+// v_readlane (scalar registers), as (row0 . row1) . (row2 . row3), which costs no trip through LDS.
+__device__ __forceinline__ float row_value_f(float v, int row) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16 * row)); }
+__device__ __forceinline__ int row_value_i(int v, int row) { return __builtin_amdgcn_readlane(v, 16 * row); }
+
 // Every lane of the wavefront receives the sum over all 64 lanes.
 __device__ __forceinline__ float wave_sum(float v)
 {
@@ -74,9 +80,7 @@ __device__ __forceinline__ float wave_sum(float v)
     v += dpp_mov_f<kDppXor2>(v);
     v += dpp_mov_f<kDppHalfMirror>(v);
     v += dpp_mov_f<kDppMirror>(v);
-    v += __shfl_xor(v, 16, kWave);
-    v += __shfl_xor(v, 32, kWave);
-    return v;
+    return (row_value_f(v, 0) + row_value_f(v, 1)) + (row_value_f(v, 2) + row_value_f(v, 3));
 }
 
 __device__ __forceinline__ int wave_sum_i(int v)
@@ -85,9 +89,7 @@ __device__ __forceinline__ int wave_sum_i(int v)
     v += dpp_mov_i<kDppXor2>(v);
     v += dpp_mov_i<kDppHalfMirror>(v);
     v += dpp_mov_i<kDppMirror>(v);
-    v += __shfl_xor(v, 16, kWave);
-    v += __shfl_xor(v, 32, kWave);
-    return v;
+    return (row_value_i(v, 0) + row_value_i(v, 1)) + (row_value_i(v, 2) + row_value_i(v, 3));
 }
 
 // max with "a < b ? b : a" so that a NaN in b never replaces a (the reference's
@@ -100,9 +102,7 @@ __device__ __forceinline__ float wave_max(float v)
     v = max_keep(v, dpp_mov_f<kDppXor2>(v));
     v = max_keep(v, dpp_mov_f<kDppHalfMirror>(v));
     v = max_keep(v, dpp_mov_f<kDppMirror>(v));
-    v = max_keep(v, __shfl_xor(v, 16, kWave));
-    v = max_keep(v, __shfl_xor(v, 32, kWave));
-    return v;
+    return max_keep(max_keep(row_value_f(v, 0), row_value_f(v, 1)), max_keep(row_value_f(v, 2), row_value_f(v, 3)));
 }
 
 // (value, index) arg-max with the lowest index winning ties.
@@ -117,8 +117,13 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i)
     argmax_combine(v, i, dpp_mov_f<kDppXor2>(v), dpp_mov_i<kDppXor2>(i));
     argmax_combine(v, i, dpp_mov_f<kDppHalfMirror>(v), dpp_mov_i<kDppHalfMirror>(i));
     argmax_combine(v, i, dpp_mov_f<kDppMirror>(v), dpp_mov_i<kDppMirror>(i));
-    argmax_combine(v, i, __shfl_xor(v, 16, kWave), __shfl_xor(i, 16, kWave));
-    argmax_combine(v, i, __shfl_xor(v, 32, kWave), __shfl_xor(i, 32, kWave));
+    float v0 = row_value_f(v, 0), v2 = row_value_f(v, 2);
+    int i0 = row_value_i(i, 0), i2 = row_value_i(i, 2);
+    argmax_combine(v0, i0, row_value_f(v, 1), row_value_i(i, 1));
+    argmax_combine(v2, i2, row_value_f(v, 3), row_value_i(i, 3));
+    argmax_combine(v0, i0, v2, i2);
+    v = v0;
+    i = i0;
 }
 
 // ---------------------------------------------------------------- small vector helpers

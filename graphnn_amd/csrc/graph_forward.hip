@@ -22,6 +22,7 @@
 // wavefront w owns column block w % (C/16) and every (WAVES / (C/16))-th tile, so it
 // keeps only its own 16 columns of W^T in registers.  MFMA operand layout as in level.hip.
 #include "gnnhip_internal.h"
+#include "buffer_addr.h"
 
 // Phase markers for a timing build of this file; they expand to nothing in the library.
 #ifndef GNNHIP_PHASE_MARK
@@ -36,7 +37,7 @@ constexpr size_t kLdsLimit = 160 * 1024;
 constexpr int kReadoutCap = 8192;       // floats of W_h1 and W_h2 staged in LDS; larger layers are read from L2
 
 // LDS carve-up, in floats:
-//   h[n16][C+4] | agg[n16][C+4] (shared with the staged X rows and the pooling partials) | rp[n16+4] | pool[C] | hid[H] | lg[Q]
+//   h[n16][C+4] | agg[n16][C+4] (shared with the staged X rows and the pooling partials) | rp[n16+4] | sv[n16] | hid[H] | lg[Q]
 //   | W_h1, W_h2 (when small) | col[ecap] | val[ecap]
 struct GraphLds {
     // the agg buffer also holds the staged X rows (n x K) and the pooling partials (waves x C)
@@ -51,7 +52,7 @@ struct GraphLds {
     static size_t fixed_floats(int n16, int C, int K, int H, int Q, int block)
     {
         const size_t wro = ((size_t)C * H + (size_t)H * Q <= (size_t)kReadoutCap) ? (size_t)C * H + (size_t)H * Q : 0;
-        size_t f = (size_t)n16 * (C + 4) + agg_floats(n16, C, K, block) + (size_t)(n16 + 4) + C + H + Q + wro;
+        size_t f = (size_t)n16 * (C + 4) + agg_floats(n16, C, K, block) + (size_t)(2 * n16 + 4) + H + Q + wro;
         return (f + 3) / 4 * 4;
     }
     // entries of the edge cache that still fit under the LDS limit
@@ -85,7 +86,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     constexpr int NJB = C / 16;          // column blocks
     constexpr int TS = kWavesPerBlock / NJB;   // wavefronts sharing one column block, splitting tiles
     constexpr int LDT = C + 4;
-    constexpr int kMsgTiles = (WAVES >= 16) ? 2 : 4;   // msg tiles a wavefront keeps in registers across the levels
+    constexpr int kMsgTiles = (WAVES >= 16) ? 2 : 4;
+    constexpr int kXSlots = (WAVES >= 16) ? 8 : 4;     // elements of the graph's X block a lane stages in one go   // msg tiles a wavefront keeps in registers across the levels
 
     extern __shared__ float smem[];
     const bool ro_staged = ((size_t)C * H + (size_t)H * Q <= (size_t)kReadoutCap);
@@ -94,8 +96,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     float* agg = hbuf + (size_t)n16max * LDT;            // [n16max][LDT]; doubles as part[P][C] in the readout
     float* part = agg;
     int* l_rp = reinterpret_cast<int*>(agg + agg_fl);    // [n16max + 1] row pointers relative to the graph's first entry
-    float* pl = reinterpret_cast<float*>(l_rp + n16max + 4);   // [C]
-    float* hid = pl + C;                                 // [H]
+    float* l_sv = reinterpret_cast<float*>(l_rp + n16max + 4);  // [n16max] pooling weights of the graph's rows
+    float* hid = l_sv + n16max;                          // [H]
     float* lg = hid + H;                                 // [Q]
     float* w1s = lg + Q;                                 // W_h1 transposed, [H][C], when staged
     float* w2s = w1s + (size_t)C * H;                    // W_h2 transposed, [Q][H], when staged
@@ -104,11 +106,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     int* e_col = reinterpret_cast<int*>(tail);           // [ecap] neighbour index local to the graph
     float* e_val = tail + ecap;                          // [ecap]
 
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1), wave = tid / kWave;
-    const int q = lane >> 4, t = lane & 15;
-    const int jb = wave % NJB, tsplit = wave / NJB;
-    const int gi = tid / G, tx = tid % G;
+    // the lane's coordinates, used by the start-up code; the graph loop derives its own copies (see there)
+    const int tid0 = threadIdx.x;
 
     GNNHIP_PHASE_MARK(0);
     // The position of the first graph (node range, then entry range) is asked for ahead of the weight
@@ -118,7 +117,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     // this wavefront's 16 columns of W^T, level contraction: wreg[s] = Wc[KS q + s][16 jb + t]
     float wreg[KS];
 #pragma unroll
-    for (int s = 0; s < KS; ++s) wreg[s] = Wc[(size_t)(KS * q + s) * C + 16 * jb + t];
+    for (int s = 0; s < KS; ++s)
+        wreg[s] = Wc[(size_t)(KS * ((tid0 & (kWave - 1)) >> 4) + s) * C + 16 * ((tid0 / kWave) % NJB) + (tid0 & 15)];
     int next_e0 = 0, next_e1 = 0;
     if ((int)blockIdx.x < B && next_n >= 0 && next_n <= n16max) {
         next_e0 = a_row_ptr[next_node0];
@@ -127,12 +127,24 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
 
     if (ro_staged) {
         // coalesced reads; the transposed layout lets a wavefront read one output's weights contiguously
-        for (int i = tid; i < C * H; i += kBlock) w1s[(i % H) * C + i / H] = Wh1[i];
-        for (int i = tid; i < H * Q; i += kBlock) w2s[(i % Q) * H + i / Q] = Wh2[i];
+        for (int i = tid0; i < C * H; i += kBlock) w1s[(i % H) * C + i / H] = Wh1[i];
+        for (int i = tid0; i < H * Q; i += kBlock) w2s[(i % Q) * H + i / Q] = Wh2[i];
     }
     // (the staged copies become visible to all lanes at the first barrier of the graph loop)
     GNNHIP_PHASE_MARK(1);
+    const rsrc_t wn_rsrc = make_rsrc(Wn2l, (unsigned)((size_t)K * C * 4));
     for (int g = blockIdx.x; g < B; g += gridDim.x) {
+        // The lane's coordinates are derived again for every graph from a value the compiler cannot see
+        // through.  Otherwise every per-lane address of the loop body (a dozen 64-bit pointers) is computed
+        // once ahead of the loop, does not fit the 128 registers of a 16-wavefront workgroup, and comes back
+        // from scratch memory in the middle of the latency chains below.
+        int tid = tid0;
+        asm volatile("" : "+v"(tid));
+        const int lane = tid & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+        const int q = lane >> 4, t = lane & 15;
+        const int jb = wave % NJB, tsplit = wave / NJB;
+        const int gi = tid / G, tx = tid % G;
+        const int wx_lane_off = ((KSX * q) * C + 16 * jb + t) * 4;
         const bool first = (g == (int)blockIdx.x);
         const int node0 = first ? next_node0 : s_row_ptr[g];
         const int n = first ? next_n : s_row_ptr[g + 1] - node0;
@@ -141,44 +153,61 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
             continue;
         }
         const int ntile = (n + 15) >> 4;
-        // this wavefront's 16 columns of W_n2l^T for the input stage: k = KSX q + s, zero beyond K.
-        // Loaded per graph (from L2) so the registers are free during the levels.
+        // this wavefront's 16 columns of W_n2l^T for the input stage: k = KSX q + s, zero beyond K (rows past the
+        // end of the buffer read as zero).  Loaded per graph (from L2) so the registers are free during the
+        // levels; one lane offset plus constant strides, so no per-element address lives across the graph loop.
         float wx[KSX];
 #pragma unroll
-        for (int s = 0; s < KSX; ++s) {
-            const int k = KSX * q + s;
-            wx[s] = Wn2l[(size_t)min(k, K - 1) * C + 16 * jb + t];
-            if (k >= K) wx[s] = 0.f;
-        }
+        for (int s = 0; s < KSX; ++s) wx[s] = buf_load_f(wn_rsrc, wx_lane_off + s * (C * 4), 0);
         const int e0 = first ? next_e0 : a_row_ptr[node0];
         const int ne = (first ? next_e1 : a_row_ptr[node0 + n]) - e0;
         const bool staged = (ne <= ecap);
 
-        // ---- stage the graph's CSR slice (L uses) and check the block-diagonal promise
-        for (int i = tid; i <= n; i += kBlock) l_rp[i] = a_row_ptr[node0 + i] - e0;
-        if (staged) {
-            for (int i = tid; i < ne; i += kBlock) {
-                const int c = a_col_idx[e0 + i] - node0;
-                if (c < 0 || c >= n) { if (status) atomicOr(status, 2); }
-                e_col[i] = min(max(c, 0), n - 1);
-                e_val[i] = a_val[e0 + i];
-            }
-        }
-        for (int i = tid; i < n; i += kBlock)
-            if (s_col_idx[node0 + i] != node0 + i) { if (status) atomicOr(status, 4); }
-        // the graph's rows of X, contiguous in memory, parked in the (still unused) agg buffer
+        // ---- stage the graph's CSR slice (L uses), its pooling weights and its rows of X (contiguous in memory;
+        //      parked in the still unused agg buffer), and check the block-diagonal promise.  Everything a lane
+        //      needs is asked for before anything is used, so the staging costs one trip to memory.
         float* xs = agg;
         {
             const float* xg = X + (size_t)node0 * K;
             const int nx = n * K;
-            int base = 0;
-            for (; base + 4 * kBlock <= nx; base += 4 * kBlock) {
-                const float x0 = xg[base + tid], x1 = xg[base + tid + kBlock];
-                const float x2 = xg[base + tid + 2 * kBlock], x3 = xg[base + tid + 3 * kBlock];
-                xs[base + tid] = x0; xs[base + tid + kBlock] = x1;
-                xs[base + tid + 2 * kBlock] = x2; xs[base + tid + 3 * kBlock] = x3;
+            int rp_v = 0, sc_v = 0, c_v = 0;
+            float sv_v = 0.f, v_v = 0.f, xv[kXSlots];
+#pragma unroll
+            for (int u = 0; u < kXSlots; ++u) xv[u] = 0.f;
+            if (tid <= n) rp_v = a_row_ptr[node0 + tid];
+            if (tid < n) { sc_v = s_col_idx[node0 + tid]; sv_v = s_val[node0 + tid]; }
+            if (staged && tid < ne) { c_v = a_col_idx[e0 + tid]; v_v = a_val[e0 + tid]; }
+#pragma unroll
+            for (int u = 0; u < kXSlots; ++u) if (tid + u * kBlock < nx) xv[u] = xg[tid + u * kBlock];
+
+            if (tid <= n) l_rp[tid] = rp_v - e0;
+            if (tid < n) {
+                l_sv[tid] = sv_v;
+                if (sc_v != node0 + tid) { if (status) atomicOr(status, 4); }
             }
-            for (int i = base + tid; i < nx; i += kBlock) xs[i] = xg[i];
+            if (staged && tid < ne) {
+                const int c = c_v - node0;
+                if (c < 0 || c >= n) { if (status) atomicOr(status, 2); }
+                e_col[tid] = min(max(c, 0), n - 1);
+                e_val[tid] = v_v;
+            }
+#pragma unroll
+            for (int u = 0; u < kXSlots; ++u) if (tid + u * kBlock < nx) xs[tid + u * kBlock] = xv[u];
+            // what exceeds one element per lane (kXSlots of X)
+            for (int i = tid + kBlock; i <= n; i += kBlock) l_rp[i] = a_row_ptr[node0 + i] - e0;
+            for (int i = tid + kBlock; i < n; i += kBlock) {
+                l_sv[i] = s_val[node0 + i];
+                if (s_col_idx[node0 + i] != node0 + i) { if (status) atomicOr(status, 4); }
+            }
+            if (staged) {
+                for (int i = tid + kBlock; i < ne; i += kBlock) {
+                    const int c = a_col_idx[e0 + i] - node0;
+                    if (c < 0 || c >= n) { if (status) atomicOr(status, 2); }
+                    e_col[i] = min(max(c, 0), n - 1);
+                    e_val[i] = a_val[e0 + i];
+                }
+            }
+            for (int i = tid + kXSlots * kBlock; i < nx; i += kBlock) xs[i] = xg[i];
         }
         __syncthreads();
 
@@ -212,24 +241,53 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
         __syncthreads();
         GNNHIP_PHASE_MARK(3);
 
+        // The first kGatherEntries neighbours of this lane's row in each of the first kGatherRounds rounds of the
+        // gather (LDS offset and weight) stay in registers for all levels: a level's gather is then one round
+        // of independent LDS reads instead of the chain row pointer -> column -> row.
+        constexpr int kGatherRounds = (WAVES >= 16) ? 2 : 4, kGatherEntries = 4;
+        int g_off[kGatherRounds][kGatherEntries], g_st[kGatherRounds], g_en[kGatherRounds];
+        float g_w[kGatherRounds][kGatherEntries];
+#pragma unroll
+        for (int r = 0; r < kGatherRounds; ++r) {
+            const int lr = r * P + gi;
+            g_st[r] = g_en[r] = 0;
+            if (staged && lr < n) { g_st[r] = l_rp[lr]; g_en[r] = l_rp[lr + 1]; }
+#pragma unroll
+            for (int u = 0; u < kGatherEntries; ++u) {
+                const bool ok = g_st[r] + u < g_en[r];
+                g_off[r][u] = (ok ? e_col[g_st[r] + u] * LDT : 0) + tx * 4;
+                g_w[r][u] = ok ? e_val[g_st[r] + u] : 0.f;
+            }
+        }
+
         for (int lv = 0; lv < L; ++lv) {
-            // ---- gather-sum from LDS: agg[i] = sum_e val_e * h[col_e]
-            for (int r0 = 0; r0 < ntile * 16; r0 += P) {
+            // ---- gather-sum from LDS: agg[i] = sum_e val_e * h[col_e], entries in order
+            if (staged) {
+#pragma unroll
+                for (int r = 0; r < kGatherRounds; ++r) {
+                    if (r * P < ntile * 16) {
+                        const int lr = r * P + gi;
+                        const int cnt = g_en[r] - g_st[r];
+                        float4 x[kGatherEntries];
+#pragma unroll
+                        for (int u = 0; u < kGatherEntries; ++u) x[u] = *reinterpret_cast<const float4*>(hbuf + g_off[r][u]);
+                        float4 acc = f4_zero();
+#pragma unroll
+                        for (int u = 0; u < kGatherEntries; ++u) if (u < cnt) f4_fma(acc, g_w[r][u], x[u]);
+                        for (int e = g_st[r] + kGatherEntries; e < g_en[r]; ++e)
+                            f4_fma(acc, e_val[e], *reinterpret_cast<const float4*>(hbuf + (size_t)e_col[e] * LDT + tx * 4));
+                        if (lr < ntile * 16) *reinterpret_cast<float4*>(agg + (size_t)lr * LDT + tx * 4) = acc;
+                    }
+                }
+            }
+            for (int r0 = staged ? kGatherRounds * P : 0; r0 < ntile * 16; r0 += P) {
                 const int lr = r0 + gi;
                 float4 acc = f4_zero();
                 if (lr < n) {
                     const int st = l_rp[lr], en = l_rp[lr + 1];
                     if (staged) {
-                        int e = st;
-                        for (; e + 1 < en; e += 2) {
-                            const int ca = e_col[e], cb = e_col[e + 1];
-                            const float va = e_val[e], vb = e_val[e + 1];
-                            const float4 xa = *reinterpret_cast<const float4*>(hbuf + (size_t)ca * LDT + tx * 4);
-                            const float4 xb = *reinterpret_cast<const float4*>(hbuf + (size_t)cb * LDT + tx * 4);
-                            f4_fma(acc, va, xa);
-                            f4_fma(acc, vb, xb);
-                        }
-                        if (e < en) f4_fma(acc, e_val[e], *reinterpret_cast<const float4*>(hbuf + (size_t)e_col[e] * LDT + tx * 4));
+                        for (int e = st; e < en; ++e)
+                            f4_fma(acc, e_val[e], *reinterpret_cast<const float4*>(hbuf + (size_t)e_col[e] * LDT + tx * 4));
                     } else {
                         for (int e = st; e < en; ++e) {
                             int c = a_col_idx[e0 + e] - node0;
@@ -283,74 +341,121 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
             }
         }
 
-        // ---- readout: weighted sum-pool over the graph's rows, then the two small dense layers,
-        // one wavefront per output element (64 lanes stride the contraction, DPP reduction)
+        // ---- readout: weighted sum-pool over the graph's rows, then the two small dense layers.
+        // Pooling: a lane owns one column and walks rows, so at C = 64 nothing crosses lanes; one partial
+        // per wavefront goes to LDS.
         {
-            float4 acc = f4_zero();
-            for (int lr = gi; lr < n; lr += P)
-                f4_fma(acc, s_val[node0 + lr], *reinterpret_cast<const float4*>(hbuf + (size_t)lr * LDT + tx * 4));
-            // combine the row groups of this wavefront, then one partial per wavefront goes to LDS
+            constexpr int GP = (C < kWave) ? C : kWave;      // lanes per row
+            constexpr int RS = kWave / GP;                   // rows per wavefront per step
+            const int pc = lane % GP, pr = lane / GP;
+            float acc = 0.f;
+            for (int lr = wave * RS + pr; lr < n; lr += kWavesPerBlock * RS)
+                acc = fmaf(l_sv[lr], hbuf[(size_t)lr * LDT + pc], acc);
 #pragma unroll
-            for (int off = G; off < kWave; off <<= 1) {
-                acc.x += __shfl_xor(acc.x, off, kWave); acc.y += __shfl_xor(acc.y, off, kWave);
-                acc.z += __shfl_xor(acc.z, off, kWave); acc.w += __shfl_xor(acc.w, off, kWave);
-            }
-            if (lane < G) *reinterpret_cast<float4*>(part + (size_t)wave * C + tx * 4) = acc;
+            for (int off = GP; off < kWave; off <<= 1) acc += __shfl_xor(acc, off, kWave);
+            if (lane < GP) part[(size_t)wave * C + pc] = acc;
         }
         __syncthreads();
-        if (tid < C) {
-            float s = 0.f;
+        GNNHIP_PHASE_MARK(12);
+        // every wavefront adds up its own copy of the pooled row (lane c holds column c; C <= 64)
+        float plv = 0.f;
+        if (lane < C) {
 #pragma unroll
-            for (int p = 0; p < kWavesPerBlock; ++p) s += part[(size_t)p * C + tid];
-            pl[tid] = s;
-            pool[(size_t)g * C + tid] = s;
+            for (int p = 0; p < kWavesPerBlock; ++p) plv += part[(size_t)p * C + lane];
+        }
+        if (wave == 0 && lane < C) pool[(size_t)g * C + lane] = plv;
+        GNNHIP_PHASE_MARK(13);
+        // hidden layer: one wavefront per output, two outputs per step so that their reductions overlap
+        for (int j = wave; j < H; j += 2 * kWavesPerBlock) {
+            const int j1 = j + kWavesPerBlock;
+            const bool two = j1 < H;
+            float s0 = 0.f, s1 = 0.f;
+            if (lane < C) {
+                if (ro_staged) {
+                    s0 = plv * w1s[j * C + lane];
+                    if (two) s1 = plv * w1s[j1 * C + lane];
+                } else {
+                    s0 = plv * Wh1[(size_t)lane * H + j];
+                    if (two) s1 = plv * Wh1[(size_t)lane * H + j1];
+                }
+            }
+            s0 = relu_ref(wave_sum(s0));
+            s1 = relu_ref(wave_sum(s1));
+            if (lane == 0) {
+                hid[j] = s0; hidden[(size_t)g * H + j] = s0;
+                if (two) { hid[j1] = s1; hidden[(size_t)g * H + j1] = s1; }
+            }
         }
         __syncthreads();
-        for (int j = wave; j < H; j += kWavesPerBlock) {
-            float s = 0.f;
-            if (ro_staged) {
-                for (int c = lane; c < C; c += kWave) s += pl[c] * w1s[j * C + c];
-            } else {
-                for (int c = lane; c < C; c += kWave) s += pl[c] * Wh1[(size_t)c * H + j];
-            }
-            s = relu_ref(wave_sum(s));
-            if (lane == 0) { hid[j] = s; hidden[(size_t)g * H + j] = s; }
-        }
-        __syncthreads();
-        for (int qq = wave; qq < Q; qq += kWavesPerBlock) {
-            float s = 0.f;
-            if (ro_staged) {
-                for (int j = lane; j < H; j += kWave) s += hid[j] * w2s[qq * H + j];
-            } else {
-                for (int j = lane; j < H; j += kWave) s += hid[j] * Wh2[(size_t)j * Q + qq];
-            }
-            s = wave_sum(s);
-            if (lane == 0) { lg[qq] = s; logits[(size_t)g * Q + qq] = s; }
-        }
-        __syncthreads();
-        if (tid < kWave) {
-            const float first = lg[0];
-            float mx = first;
-            float bv = -INFINITY;
-            int bi = 0x7fffffff;
-            for (int qq = tid; qq < Q; qq += kWave) {
-                const float v = lg[qq];
-                mx = max_keep(mx, v);
-                argmax_combine(bv, bi, (v != v) ? -INFINITY : v, qq);
-            }
-            mx = wave_max(mx);
-            wave_argmax(bv, bi);
-            if (first != first) bi = 0;
-            if (pred && tid == 0) pred[g] = bi;
-            if (probs) {
+        GNNHIP_PHASE_MARK(14);
+        if (Q <= 16) {
+            // few classes: lane q of the first wavefront adds up logit q, and softmax and arg-max follow in
+            // registers, with no further barrier or trip through LDS
+            if (wave == 0) {
                 float s = 0.f;
-                for (int qq = tid; qq < Q; qq += kWave) {
-                    const float e = expf(lg[qq] - mx);
-                    lg[qq] = e;
-                    s += e;
+                if (lane < Q) {
+                    if (ro_staged) {
+#pragma unroll 8
+                        for (int j = 0; j < H; ++j) s = fmaf(hid[j], w2s[lane * H + j], s);
+                    } else {
+#pragma unroll 8
+                        for (int j = 0; j < H; ++j) s = fmaf(hid[j], Wh2[(size_t)j * Q + lane], s);
+                    }
+                    logits[(size_t)g * Q + lane] = s;
+                }
+                if (probs || pred) {
+                    const float first = row_value_f(s, 0);
+                    float mx = (lane < Q) ? max_keep(first, s) : first;     // the reference scan starts at element 0
+                    mx = wave_max(mx);
+                    float bv = -INFINITY;
+                    int bi = 0x7fffffff;
+                    if (lane < Q) { bv = (s != s) ? -INFINITY : s; bi = lane; }   // a NaN that is not first never wins
+                    wave_argmax(bv, bi);
+                    if (first != first) bi = 0;                             // a NaN in column 0 is never displaced
+                    if (pred && lane == 0) pred[g] = bi;
+                    if (probs) {
+                        const float e = (lane < Q) ? expf(s - mx) : 0.f;
+                        const float sum = wave_sum(e);
+                        if (lane < Q) probs[(size_t)g * Q + lane] = e / sum;
+                    }
+                }
+            }
+        } else {
+            for (int qq = wave; qq < Q; qq += kWavesPerBlock) {
+                float s = 0.f;
+                if (ro_staged) {
+                    for (int j = lane; j < H; j += kWave) s += hid[j] * w2s[qq * H + j];
+                } else {
+                    for (int j = lane; j < H; j += kWave) s += hid[j] * Wh2[(size_t)j * Q + qq];
                 }
                 s = wave_sum(s);
-                for (int qq = tid; qq < Q; qq += kWave) probs[(size_t)g * Q + qq] = lg[qq] / s;
+                if (lane == 0) { lg[qq] = s; logits[(size_t)g * Q + qq] = s; }
+            }
+            __syncthreads();
+            if (wave == 0) {
+                const float first = lg[0];
+                float mx = first;
+                float bv = -INFINITY;
+                int bi = 0x7fffffff;
+                for (int qq = lane; qq < Q; qq += kWave) {
+                    const float v = lg[qq];
+                    mx = max_keep(mx, v);
+                    argmax_combine(bv, bi, (v != v) ? -INFINITY : v, qq);
+                }
+                mx = wave_max(mx);
+                wave_argmax(bv, bi);
+                if (first != first) bi = 0;
+                if (pred && lane == 0) pred[g] = bi;
+                if (probs) {
+                    float s = 0.f;
+                    for (int qq = lane; qq < Q; qq += kWave) {
+                        const float e = expf(lg[qq] - mx);
+                        lg[qq] = e;
+                        s += e;
+                    }
+                    s = wave_sum(s);
+                    for (int qq = lane; qq < Q; qq += kWave) probs[(size_t)g * Q + qq] = lg[qq] / s;
+                }
             }
         }
         GNNHIP_PHASE_MARK(7);
