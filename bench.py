@@ -139,7 +139,7 @@ def time_level_cfg4(dev):
     N, E, C = batch.num_nodes, int(a[1].size), cfg["C"]
     flops = 2.0 * N * C * C + 2.0 * E * C + 2.0 * N * C
     return {"workload": "configuration 4: one level, %d nodes, %d entries, hidden %d" % (N, E, C),
-            "kernel": "s2v_level_wide_kernel<256,8>", "avg_ms": ms,
+            "kernel": "s2v_level_wide_kernel<256,8,false,64>", "avg_ms": ms,
             "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS},
             "algorithmic_GBps": level_algorithmic_bytes(N, E, C) / (ms * 1e-3) / 1e9}

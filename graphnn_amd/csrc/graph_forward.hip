@@ -21,6 +21,12 @@
 // lanes per row); the contraction splits (16-column block) x (16-row tile):
 // wavefront w owns column block w % (C/16) and every (WAVES / (C/16))-th tile, so it
 // keeps only its own 16 columns of W^T in registers.  MFMA operand layout as in level.hip.
+//
+// The kernel's time is a chain of latencies of the largest graph, so the code keeps that chain short:
+// the graph's position is asked for ahead of the weight loads; every global load of the staging (row
+// pointers, columns, weights, pooling weights, X) is issued before the first of them is used; the
+// first neighbours of a lane's rows stay in registers for all levels; the readout has three steps
+// (pool partials | pooled row + hidden layer | logits + softmax in the registers of one wavefront).
 #include "gnnhip_internal.h"
 #include "buffer_addr.h"
 
