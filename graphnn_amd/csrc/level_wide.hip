@@ -117,12 +117,17 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
         for (int i = threadIdx.x; i < C; i += kWideBlock) bias_lds[i] = bias[i];
 
     // W^T operand: wreg[jb][s] = W[KS q + s][col0 + 16 jb + t]
+    // (buffer loads: one lane offset, the steps as scalar offsets, so no 64-bit address per element is formed)
     float wreg[NB][KS];
+    {
+        const rsrc_t w_rsrc = make_rsrc(W, (unsigned)(C * C * 4));
+        const int w_lane_off = ((KS * q) * C + col0 + t) * 4;
 #pragma unroll
-    for (int jb = 0; jb < NB; ++jb)
+        for (int jb = 0; jb < NB; ++jb)
 #pragma unroll
-        for (int s = 0; s < KS; ++s)
-            wreg[jb][s] = W[(size_t)(KS * q + s) * C + col0 + 16 * jb + t];
+            for (int s = 0; s < KS; ++s)
+                wreg[jb][s] = buf_load_f(w_rsrc, w_lane_off + 64 * jb, s * (C * 4));
+    }
 
     const int ntiles = (int)(((long long)N + kTileRows - 1) / kTileRows);
     const int tile_begin = (int)min((long long)blockIdx.x * tiles_per_block, (long long)ntiles);
