@@ -46,11 +46,13 @@ constexpr int kReadoutCap = 8192;       // floats of W_h1 and W_h2 staged in LDS
 //   h[n16][C+4] | agg[n16][C+4] (shared with the staged X rows and the pooling partials) | rp[n16+4] | sv[n16] | hid[H] | lg[Q]
 //   | W_h1, W_h2 (when small) | col[ecap] | val[ecap]
 struct GraphLds {
-    // the agg buffer also holds the staged X rows (n x K) and the pooling partials (waves x C)
+    // contraction steps of the input stage: the K label columns in groups of four, an even number of them
+    __host__ __device__ static int input_steps(int K) { return ((K + 3) / 4 + 1) & ~1; }
+    // the agg buffer also holds the staged X rows (n x 4 input_steps(K), zero-padded) and the pooling partials (waves x C)
     __host__ __device__ static size_t agg_floats(int n16, int C, int K, int block)
     {
         size_t a = (size_t)n16 * (C + 4);
-        const size_t p = (size_t)(block / 64) * C, x = (size_t)n16 * K;
+        const size_t p = (size_t)(block / 64) * C, x = (size_t)n16 * 4 * input_steps(K);
         if (p > a) a = p;
         if (x > a) a = x;
         return (a + 3) / 4 * 4;
@@ -76,7 +78,7 @@ struct GraphLds {
 // (column block x row tile) tasks spread over the wavefronts.
 template <int C, int KSX, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
-    int B, int K, int H, int Q, int L, int n16max, int ecap,
+    int B, int K, unsigned k_magic, int H, int Q, int L, int n16max, int ecap,
     const int* __restrict__ a_row_ptr, const int* __restrict__ a_col_idx, const float* __restrict__ a_val,
     const int* __restrict__ s_row_ptr, const int* __restrict__ s_col_idx, const float* __restrict__ s_val,
     const float* __restrict__ X, const float* __restrict__ Wn2l, const float* __restrict__ Wc,
@@ -139,6 +141,10 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     // (the staged copies become visible to all lanes at the first barrier of the graph loop)
     GNNHIP_PHASE_MARK(1);
     const rsrc_t wn_rsrc = make_rsrc(Wn2l, (unsigned)((size_t)K * C * 4));
+    // input stage: srt contraction steps (srt <= KSX), lane group q covers label columns [srt q, srt q + srt);
+    // the staged rows of X have stride KP floats and zeros from column K on
+    const int srt = GraphLds::input_steps(K);
+    const int KP = 4 * srt;
     for (int g = blockIdx.x; g < B; g += gridDim.x) {
         // The lane's coordinates are derived again for every graph from a value the compiler cannot see
         // through.  Otherwise every per-lane address of the loop body (a dozen 64-bit pointers) is computed
@@ -150,7 +156,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
         const int q = lane >> 4, t = lane & 15;
         const int jb = wave % NJB, tsplit = wave / NJB;
         const int gi = tid / G, tx = tid % G;
-        const int wx_lane_off = ((KSX * q) * C + 16 * jb + t) * 4;
+        const int wx_lane_off = ((srt * q) * C + 16 * jb + t) * 4;
         const bool first = (g == (int)blockIdx.x);
         const int node0 = first ? next_node0 : s_row_ptr[g];
         const int n = first ? next_n : s_row_ptr[g + 1] - node0;
@@ -159,8 +165,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
             continue;
         }
         const int ntile = (n + 15) >> 4;
-        // this wavefront's 16 columns of W_n2l^T for the input stage: k = KSX q + s, zero beyond K (rows past the
-        // end of the buffer read as zero).  Loaded per graph (from L2) so the registers are free during the
+        // this wavefront's 16 columns of W_n2l^T for the input stage: k = srt q + s, zero beyond K (rows past the
+        // end of the buffer read as zero; steps s >= srt are loaded but not used).  Loaded per graph (from L2) so the registers are free during the
         // levels; one lane offset plus constant strides, so no per-element address lives across the graph loop.
         float wx[KSX];
 #pragma unroll
@@ -176,6 +182,12 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
         {
             const float* xg = X + (size_t)node0 * K;
             const int nx = n * K;
+            // element i of the graph's block of X (row i / K, column i % K) -> its padded slot; the quotient
+            // comes from one multiply-high by ceil(2^32 / K), exact for i K < 2^32
+            auto x_slot = [&](int i) {
+                const int r = K >= 2 ? (int)__umulhi((unsigned)i, k_magic) : i;
+                return r * KP + (i - r * K);
+            };
             int rp_v = 0, sc_v = 0, c_v = 0;
             float sv_v = 0.f, v_v = 0.f, xv[kXSlots];
 #pragma unroll
@@ -198,7 +210,13 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
                 e_val[tid] = v_v;
             }
 #pragma unroll
-            for (int u = 0; u < kXSlots; ++u) if (tid + u * kBlock < nx) xs[tid + u * kBlock] = xv[u];
+            for (int u = 0; u < kXSlots; ++u) {
+                const int i = tid + u * kBlock;
+                if (i < nx) xs[x_slot(i)] = xv[u];
+            }
+            // columns K .. KP-1 of the staged rows (at most 7) are zero
+            for (int r = tid; r < n; r += kBlock)
+                for (int k = K; k < KP; ++k) xs[r * KP + k] = 0.f;
             // what exceeds one element per lane (kXSlots of X)
             for (int i = tid + kBlock; i <= n; i += kBlock) l_rp[i] = a_row_ptr[node0 + i] - e0;
             for (int i = tid + kBlock; i < n; i += kBlock) {
@@ -213,7 +231,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
                     e_val[i] = a_val[e0 + i];
                 }
             }
-            for (int i = tid + kXSlots * kBlock; i < nx; i += kBlock) xs[i] = xg[i];
+            for (int i = tid + kXSlots * kBlock; i < nx; i += kBlock) xs[x_slot(i)] = xg[i];
         }
         __syncthreads();
 
@@ -227,15 +245,20 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
             for (int tl = tsplit; tl < ntile; tl += TS, ++ti) {
                 const int lr = tl * 16 + t;
                 const bool valid = lr < n;
-                // every lane reads a valid LDS slot (row and k clamped); wx is zero beyond K and
-                // rows beyond n are zeroed below, so the clamped values cannot reach a result
-                const float* xrow = xs + min(lr, n - 1) * K;
+                // every lane reads a valid LDS slot (row clamped; rows beyond n are zeroed below); the
+                // lane's srt values are contiguous and 8-byte aligned
+                const float* xrow = xs + min(lr, n - 1) * KP + srt * q;
                 float xreg[KSX];
 #pragma unroll
-                for (int s = 0; s < KSX; ++s) xreg[s] = xrow[min(KSX * q + s, K - 1)];
+                for (int s2 = 0; s2 < KSX / 2; ++s2) {
+                    float2 v2 = make_float2(0.f, 0.f);
+                    if (2 * s2 < srt) v2 = *reinterpret_cast<const float2*>(xrow + 2 * s2);
+                    xreg[2 * s2] = v2.x; xreg[2 * s2 + 1] = v2.y;
+                }
                 mfma_f4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int s = 0; s < KSX; ++s) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wx[s], xreg[s], acc, 0, 0, 0);
+                for (int s = 0; s < KSX; ++s)
+                    if (s < srt) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wx[s], xreg[s], acc, 0, 0, 0);
                 float4 v = make_float4(acc[0], acc[1], acc[2], acc[3]);      // row lr, columns 16 jb + 4 q + {0..3}
                 if (!valid) v = f4_zero();
                 if (valid) *reinterpret_cast<float4*>(msg + (size_t)(node0 + lr) * C + 16 * jb + 4 * q) = v;
@@ -489,8 +512,9 @@ int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
         configured = smem;
     }
     const int grid = B < kNumCU * 4 ? B : kNumCU * 4;
+    const unsigned k_magic = K >= 2 ? (unsigned)((0x100000000ull + (unsigned)K - 1) / (unsigned)K) : 0u;   // ceil(2^32 / K)
     hipLaunchKernelGGL((s2v_graph_forward_kernel<C, KSX, WAVES>), dim3(grid), dim3(kBlock), smem, s,
-                       B, K, H, Q, L, n16max, ecap, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val,
+                       B, K, k_magic, H, Q, L, n16max, ecap, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val,
                        X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status);
     GNNHIP_LAUNCH_CHECK("s2v_graph_forward");
     return GNNHIP_OK;
