@@ -43,7 +43,7 @@ constexpr size_t kLdsLimit = 160 * 1024;
 constexpr int kReadoutCap = 8192;       // floats of W_h1 and W_h2 staged in LDS; larger layers are read from L2
 
 // LDS carve-up, in floats:
-//   h[n16][C+4] | agg[n16][C+4] (shared with the staged X rows and the pooling partials) | rp[n16+4] | sv[n16] | hid[H] | lg[Q]
+//   h[n16+1][C+4] (the last row stays zero) | agg[n16][C+4] (shared with the staged X rows and the pooling partials) | rp[n16+4] | sv[n16] | hid[H] | lg[Q]
 //   | W_h1, W_h2 (when small) | col[ecap] | val[ecap]
 struct GraphLds {
     // contraction steps of the input stage: the K label columns in groups of four, an even number of them
@@ -60,7 +60,7 @@ struct GraphLds {
     static size_t fixed_floats(int n16, int C, int K, int H, int Q, int block)
     {
         const size_t wro = ((size_t)C * H + (size_t)H * Q <= (size_t)kReadoutCap) ? (size_t)C * H + (size_t)H * Q : 0;
-        size_t f = (size_t)n16 * (C + 4) + agg_floats(n16, C, K, block) + (size_t)(2 * n16 + 4) + H + Q + wro;
+        size_t f = (size_t)(n16 + 1) * (C + 4) + agg_floats(n16, C, K, block) + (size_t)(2 * n16 + 4) + H + Q + wro;
         return (f + 3) / 4 * 4;
     }
     // entries of the edge cache that still fit under the LDS limit
@@ -100,8 +100,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     extern __shared__ float smem[];
     const bool ro_staged = ((size_t)C * H + (size_t)H * Q <= (size_t)kReadoutCap);
     const size_t agg_fl = GraphLds::agg_floats(n16max, C, K, kBlock);
-    float* hbuf = smem;                                  // [n16max][LDT]
-    float* agg = hbuf + (size_t)n16max * LDT;            // [n16max][LDT]; doubles as part[P][C] in the readout
+    float* hbuf = smem;                                  // [n16max + 1][LDT]; row n16max is never written after start-up and holds zeros
+    float* agg = hbuf + (size_t)(n16max + 1) * LDT;      // [n16max][LDT]; doubles as part[P][C] in the readout
     float* part = agg;
     int* l_rp = reinterpret_cast<int*>(agg + agg_fl);    // [n16max + 1] row pointers relative to the graph's first entry
     float* l_sv = reinterpret_cast<float*>(l_rp + n16max + 4);  // [n16max] pooling weights of the graph's rows
@@ -133,6 +133,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
         next_e1 = a_row_ptr[next_node0 + next_n];
     }
 
+    if (tid0 < LDT) hbuf[(size_t)n16max * LDT + tid0] = 0.f;
     if (ro_staged) {
         // coalesced reads; the transposed layout lets a wavefront read one output's weights contiguously
         for (int i = tid0; i < C * H; i += kBlock) w1s[(i % H) * C + i / H] = Wh1[i];
@@ -283,8 +284,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
             if (staged && lr < n) { g_st[r] = l_rp[lr]; g_en[r] = l_rp[lr + 1]; }
 #pragma unroll
             for (int u = 0; u < kGatherEntries; ++u) {
-                const bool ok = g_st[r] + u < g_en[r];
-                g_off[r][u] = (ok ? e_col[g_st[r] + u] * LDT : 0) + tx * 4;
+                const bool ok = g_st[r] + u < g_en[r];       // a missing entry is weight 0 times the zero row
+                g_off[r][u] = (ok ? e_col[g_st[r] + u] : n16max) * LDT + tx * 4;
                 g_w[r][u] = ok ? e_val[g_st[r] + u] : 0.f;
             }
         }
@@ -296,13 +297,12 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
                 for (int r = 0; r < kGatherRounds; ++r) {
                     if (r * P < ntile * 16) {
                         const int lr = r * P + gi;
-                        const int cnt = g_en[r] - g_st[r];
                         float4 x[kGatherEntries];
 #pragma unroll
                         for (int u = 0; u < kGatherEntries; ++u) x[u] = *reinterpret_cast<const float4*>(hbuf + g_off[r][u]);
                         float4 acc = f4_zero();
 #pragma unroll
-                        for (int u = 0; u < kGatherEntries; ++u) if (u < cnt) f4_fma(acc, g_w[r][u], x[u]);
+                        for (int u = 0; u < kGatherEntries; ++u) f4_fma(acc, g_w[r][u], x[u]);
                         for (int e = g_st[r] + kGatherEntries; e < g_en[r]; ++e)
                             f4_fma(acc, e_val[e], *reinterpret_cast<const float4*>(hbuf + (size_t)e_col[e] * LDT + tx * 4));
                         if (lr < ntile * 16) *reinterpret_cast<float4*>(agg + (size_t)lr * LDT + tx * 4) = acc;
