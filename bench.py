@@ -395,6 +395,9 @@ def main():
             "kernel": "spmm_rowgroup_kernel<4,1>",
             "workload": "configuration 3: CSR SpMM, %d rows, %d entries, width %d" % (n, nnz, d),
             "algorithmic_bytes": bytes_alg, "avg_ms": mean_ms, "min_ms": min_ms,
+            # the counted traffic over the same launch time: what the memory system actually moves
+            "traffic_GBps": MEASURED_TRAFFIC_BYTES["spmm_cfg3"] / (mean_ms * 1e-3) / 1e9,
+            "traffic_frac": MEASURED_TRAFFIC_BYTES["spmm_cfg3"] / (mean_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         }
     else:
         out["roofline"] = None

@@ -172,14 +172,14 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
         float wx[KSX];
 #pragma unroll
         for (int s = 0; s < KSX; ++s) wx[s] = buf_load_f(wn_rsrc, wx_lane_off + s * (C * 4), 0);
-        const int e0 = first ? next_e0 : a_row_ptr[node0];
-        const int ne = (first ? next_e1 : a_row_ptr[node0 + n]) - e0;
-        const bool staged = (ne <= ecap);
 
         // ---- stage the graph's CSR slice (L uses), its pooling weights and its rows of X (contiguous in memory;
         //      parked in the still unused agg buffer), and check the block-diagonal promise.  Everything a lane
         //      needs is asked for before anything is used, so the staging costs one trip to memory.
         float* xs = agg;
+        const int e0 = first ? next_e0 : a_row_ptr[node0];
+        const int ne = (first ? next_e1 : a_row_ptr[node0 + n]) - e0;
+        const bool staged = (ne <= ecap);
         {
             const float* xg = X + (size_t)node0 * K;
             const int nx = n * K;
@@ -195,9 +195,10 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
             for (int u = 0; u < kXSlots; ++u) xv[u] = 0.f;
             if (tid <= n) rp_v = a_row_ptr[node0 + tid];
             if (tid < n) { sc_v = s_col_idx[node0 + tid]; sv_v = s_val[node0 + tid]; }
-            if (staged && tid < ne) { c_v = a_col_idx[e0 + tid]; v_v = a_val[e0 + tid]; }
 #pragma unroll
             for (int u = 0; u < kXSlots; ++u) if (tid + u * kBlock < nx) xv[u] = xg[tid + u * kBlock];
+            // (the graph's first entry is the last thing to arrive at start-up: everything above is under way by then)
+            if (staged && tid < ne) { c_v = a_col_idx[e0 + tid]; v_v = a_val[e0 + tid]; }
 
             if (tid <= n) l_rp[tid] = rp_v - e0;
             if (tid < n) {
