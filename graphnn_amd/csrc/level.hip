@@ -40,8 +40,9 @@ bool level_stream_covers(int N, int C);
 // input_wide.hip
 int input_wide_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s);
 // level_wide.hip
-int level_wide_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-                        const float* W, const float* msg, const float* bias, float* h_out, bool relu_in, hipStream_t s);
+int level_wide_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
+                        const float* h_in, const float* W, const float* msg, const float* bias, float* h_out, bool relu_in,
+                        hipStream_t s);
 bool level_wide_covers(int N, int C);
 
 namespace {
@@ -645,7 +646,7 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
     }
     switch (C) {
     case 128:
-    case 256: return level_wide_dispatch(N, C, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, relu_in, s);
+    case 256: return level_wide_dispatch(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, relu_in, s);
     }
     return GNNHIP_EUNSUPPORTED;
 }

@@ -73,6 +73,29 @@ template <int VEC> struct BufLoad;
 template <> struct BufLoad<4> { static __device__ __forceinline__ float4 get(rsrc_t r, int v, int s) { return buf_load4(r, v, s); } };
 template <> struct BufLoad<2> { static __device__ __forceinline__ float2 get(rsrc_t r, int v, int s) { return buf_load2(r, v, s); } };
 
+// A batch of kInFlight consecutive entries of a CSR array (column indices, or edge weights as bit
+// patterns) in scalar registers.  The two scalar loads are written as inline assembly with the batch as a
+// read-write operand: the loaded values land in the registers the batch already occupies, so a batch that
+// is (conditionally) refilled inside the loop needs no copy of the loaded values, and with it no wait for
+// the scalar cache right behind the load.  The compiler does not know that these registers are in flight:
+// batch_wait() must run before a batch is read.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+struct Batch { i32x4 lo; i32x2 hi; };
+static_assert(kInFlight == 6, "a batch is one 4-dword and one 2-dword scalar load");
+__device__ __forceinline__ void batch_load(Batch& b, const int* p)
+{
+    asm volatile("s_load_dwordx4 %0, %2, 0x0\n\ts_load_dwordx2 %1, %2, 0x10" : "+s"(b.lo), "+s"(b.hi) : "s"(p));
+}
+__device__ __forceinline__ void batch_wait(Batch& b)
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(b.lo), "+s"(b.hi));
+}
+__device__ __forceinline__ int batch_get(const Batch& b, int u)      // u is a compile-time constant after unrolling
+{
+    return u == 0 ? b.lo.x : u == 1 ? b.lo.y : u == 2 ? b.lo.z : u == 3 ? b.lo.w : u == 4 ? b.hi.x : b.hi.y;
+}
+
 template <int VEC, bool RELU_IN>
 __device__ __forceinline__ void vec_fma(float (&acc)[VEC], float a, const typename VecT<VEC>::type& x)
 {
@@ -145,33 +168,26 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     };
     const int* val_bits = reinterpret_cast<const int*>(val);
     // entries [s, s + kInFlight) of the CSR arrays.  What lies past the end of the wavefront's rows is
-    // loaded but never added, so the batch is read as it lies; only at the very end of the arrays do
-    // the indices have to be clamped.  No selection on the loaded values here: a scalar load followed
-    // at once by a use of its result is a full trip to the scalar cache each.
+    // loaded but never added, so the batch is read as it lies.  Only a batch that would run past the end
+    // of the arrays starts earlier; batch_ready() then shifts it into place.  The arrays hold at least
+    // kInFlight entries (the host pads shorter ones).
     const int nnz = row_ptr[N];
-    auto load_cols = [&](int s, int (&c)[kInFlight]) {
-        if (s + kInFlight <= nnz) {
-#pragma unroll
-            for (int u = 0; u < kInFlight; ++u) c[u] = col_idx[s + u];
-        } else {
-#pragma unroll
-            for (int u = 0; u < kInFlight; ++u) c[u] = col_idx[min(s + u, nnz - 1)];
-        }
+    auto load_batch = [&](const int* arr, int s, Batch& b) {
+        const int base = max(min(s, nnz - kInFlight), 0);
+        batch_load(b, arr + base);
+        return s - base;                         // by how many entries the batch has to be shifted
     };
-    auto load_weights = [&](int s, int (&a)[kInFlight]) {
-        if (s + kInFlight <= nnz) {
-#pragma unroll
-            for (int u = 0; u < kInFlight; ++u) a[u] = val_bits[s + u];
-        } else {
-#pragma unroll
-            for (int u = 0; u < kInFlight; ++u) a[u] = val_bits[min(s + u, nnz - 1)];
+    auto batch_ready = [&](Batch& b, int shift) {
+        batch_wait(b);
+        for (; shift > 0; --shift) {             // only at the very end of the arrays
+            b.lo.x = b.lo.y; b.lo.y = b.lo.z; b.lo.z = b.lo.w; b.lo.w = b.hi.x; b.hi.x = b.hi.y;
         }
     };
     const rsrc_t h_rsrc = make_rsrc(h_in, (unsigned)((size_t)N * C * 4));
-    auto issue = [&](const int (&c)[kInFlight], vec_t (&x)[kInFlight]) {
+    auto issue = [&](const Batch& c, vec_t (&x)[kInFlight]) {
 #pragma unroll
         for (int u = 0; u < kInFlight; ++u)
-            x[u] = BufLoad<VEC>::get(h_rsrc, lane * (VEC * 4), c[u] * (C * 4));     // N C 4 < 2^32 (host-checked)
+            x[u] = BufLoad<VEC>::get(h_rsrc, lane * (VEC * 4), batch_get(c, u) * (C * 4));     // N C 4 < 2^32 (host-checked)
     };
 
     // ---- state of the gather of one pass: entries [e, ee) of the wavefront's RPW rows, taken in order;
@@ -195,12 +211,12 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
         ++lr;
         row_end = __builtin_amdgcn_readlane(rpv, min(lr + 1, RPW));
     };
-    auto consume = [&](const int (&a)[kInFlight], const vec_t (&x)[kInFlight]) {
+    auto consume = [&](const Batch& a, const vec_t (&x)[kInFlight]) {
 #pragma unroll
         for (int u = 0; u < kInFlight; ++u) {
             if (e + u < ee) {
                 while (e + u >= row_end) flush_row();          // rows ending here (possibly empty ones)
-                vec_fma<VEC, RELU_IN>(acc, __int_as_float(a[u]), x[u]);
+                vec_fma<VEC, RELU_IN>(acc, __int_as_float(batch_get(a, u)), x[u]);
             }
         }
         e += kInFlight;
@@ -226,9 +242,10 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     };
 
     GNNHIP_PHASE_INIT
-    int cC[kInFlight], aC[kInFlight];            // columns / weights of the next batch to issue / to sum
-#pragma unroll
-    for (int u = 0; u < kInFlight; ++u) { cC[u] = 0; aC[u] = 0; }
+    Batch cC, aC;                                // columns / weights of the next batch to issue / to sum
+    cC.lo = i32x4{0, 0, 0, 0}; cC.hi = i32x2{0, 0};
+    aC.lo = i32x4{0, 0, 0, 0}; aC.hi = i32x2{0, 0};
+    int cShift = 0, aShift = 0;                  // shifts owed to cC / aC when they are next read
 
     // ---- first pass: its gather has nothing to hide behind
     int rp_next = load_rowptrs(tile_begin);      // row pointers of the next pass to gather
@@ -236,8 +253,10 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     begin(rp_next, ebN, eeN, tiles + gather_off);
     while (e < ee) {
         vec_t x[kInFlight];
-        load_cols(e, cC);
-        load_weights(e, aC);
+        cShift = load_batch(col_idx, e, cC);
+        aShift = load_batch(val_bits, e, aC);
+        batch_ready(cC, cShift);
+        batch_ready(aC, aShift);
         issue(cC, x);
         consume(aC, x);
     }
@@ -247,7 +266,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
         rp_next = load_rowptrs(tile_begin + 1);
         ebN = __builtin_amdgcn_readlane(rp_next, 0);
         eeN = __builtin_amdgcn_readlane(rp_next, RPW);
-        if (ebN < eeN) { load_cols(ebN, cC); load_weights(ebN, aC); }
+        if (ebN < eeN) { cShift = load_batch(col_idx, ebN, cC); aShift = load_batch(val_bits, ebN, aC); }
     }
     __syncthreads();
     GNNHIP_PHASE_ACC(0);
@@ -282,7 +301,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
             }
             vec_t x[kInFlight];
             const bool batch = e < ee;
-            if (batch) issue(cC, x);
+            if (batch) { batch_ready(cC, cShift); issue(cC, x); }
             store_pending();
             // where the follower of this batch starts: inside this pass, or (after the last block) at the
             // first entry of the next pass; its columns travel while the matrix cores work
@@ -292,7 +311,6 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
             } else if (e + kInFlight >= ee) {
                 ns = ebN; nend = eeN;                     // both zero when there is no next pass
             }
-            if (ns < nend) load_cols(ns, cC);
             GNNHIP_PHASE_ACC(1);
 
             const float* src = cur + (rt * 16 + t) * LDT + KS * q;
@@ -319,6 +337,9 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
 #pragma unroll
                     for (int jb = 0; jb < NB; ++jb) acc_m[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(wreg[jb][s0 + 3], b.w, acc_m[jb], 0, 0, 0);
                 }
+                // the follower's columns are asked for here, behind the first wait for LDS of this block: a
+                // scalar load in flight counts with the LDS reads, and the next wait is 16 matrix instructions away
+                if (s8 == 0 && ns < nend) cShift = load_batch(col_idx, ns, cC);
                 __builtin_amdgcn_sched_barrier(0);            // keeps the read-ahead where it is written
                 b_cur[0] = b_nxt[0]; b_cur[1] = b_nxt[1];
             }
@@ -328,8 +349,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
             // path on which they are still in flight and waits at the top of the next block instead,
             // where the wait also covers the stores issued just before it.
             __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
-            if (batch) consume(aC, x);
-            if (ns < nend) load_weights(ns, aC);
+            if (batch) { batch_ready(aC, aShift); consume(aC, x); }
+            if (ns < nend) aShift = load_batch(val_bits, ns, aC);
             if (rt == 0) {                                // the row pointers asked for at the top have arrived
                 ebN = eeN = 0;
                 if (has_next2) {
@@ -357,12 +378,14 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
         if (e < ee) {                                     // more than four batches: finish in the open
             while (e < ee) {
                 vec_t x[kInFlight];
-                load_cols(e, cC);
-                load_weights(e, aC);
+                cShift = load_batch(col_idx, e, cC);
+                aShift = load_batch(val_bits, e, aC);
+                batch_ready(cC, cShift);
+                batch_ready(aC, aShift);
                 issue(cC, x);
                 consume(aC, x);
             }
-            if (ebN < eeN) { load_cols(ebN, cC); load_weights(ebN, aC); }
+            if (ebN < eeN) { cShift = load_batch(col_idx, ebN, cC); aShift = load_batch(val_bits, ebN, aC); }
         }
         if (has_next) finish();
         store_pending();
@@ -414,9 +437,25 @@ bool level_wide_covers(int N, int C)
     return (C == 128 || C == 256) && (unsigned long long)N * (unsigned)C * 4ull < (1ull << 32);
 }
 
-int level_wide_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-                        const float* W, const float* msg, const float* bias, float* h_out, bool relu_in, hipStream_t s)
+int level_wide_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
+                        const float* h_in, const float* W, const float* msg, const float* bias, float* h_out, bool relu_in,
+                        hipStream_t s)
 {
+    if (nnz < kInFlight) {
+        // the kernel reads whole batches of kInFlight entries: arrays shorter than one batch are copied into
+        // zero-padded scratch
+        void* pad = nullptr;
+        if (int rc = stream_scratch(s, 64, &pad)) return rc;
+        if (int rc = gnnhip_memset0(pad, 64, s)) return rc;
+        int* col_pad = static_cast<int*>(pad);
+        float* val_pad = reinterpret_cast<float*>(col_pad + 8);
+        if (nnz > 0) {
+            if (int rc = gnnhip_memcpy_d2d(col_pad, col_idx, sizeof(int) * (size_t)nnz, s)) return rc;
+            if (int rc = gnnhip_memcpy_d2d(val_pad, val, sizeof(float) * (size_t)nnz, s)) return rc;
+        }
+        col_idx = col_pad;
+        val = val_pad;
+    }
     switch (C) {
     case 128:
         return relu_in ? launch_level_wide<128, 8, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s)

@@ -408,6 +408,31 @@ def test_level_every_row_length_up_to_70(gpu, oracle, C, N):
 
 
 @pytest.mark.parametrize("C", [128, 256])
+@pytest.mark.parametrize("nnz", [0, 1, 5, 6, 7])
+def test_wide_level_fewer_entries_than_one_index_batch(gpu, oracle, C, nnz):
+    """the wide kernel reads column indices and weights six at a time: matrices with fewer entries than that,
+    exactly that many, and one more; the entries sit in the last rows, so the last batch ends at the end of
+    the arrays"""
+    import torch
+    from graphnn_amd import ops
+    rng = np.random.default_rng(300 + C + nnz)
+    N = 77
+    lens = np.zeros(N, np.int64)
+    for i in range(nnz): lens[N - 1 - (i % 3)] += 1
+    rp = np.zeros(N + 1, np.int32); np.cumsum(lens, out=rp[1:])
+    ci = rng.integers(0, N, nnz).astype(np.int32)
+    v = (rng.random(nnz) + 0.5).astype(np.float32)
+    h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
+    W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
+    msg = rng.standard_normal((N, C)).astype(np.float32)
+    want = oracle.level(rp, ci, v, h_in, W, msg, None)
+    ci_d = _t(ci, gpu) if nnz else torch.zeros(1, dtype=torch.int32, device=gpu)[:0]
+    v_d = _t(v, gpu) if nnz else torch.zeros(1, dtype=torch.float32, device=gpu)[:0]
+    got = _n(ops.s2v_level(_t(rp, gpu), ci_d, v_d, _t(h_in, gpu), _t(W, gpu), _t(msg, gpu)))
+    assert max_rel(got, want) < PARITY_TOL
+
+
+@pytest.mark.parametrize("C", [128, 256])
 @pytest.mark.parametrize("N", [5_003, 64 * 300 + 37, 40_037])
 def test_wide_level_ragged_rows_and_weights(gpu, oracle, C, N):
     """wide-hidden kernel: empty rows, rows longer than one 64-entry index batch, a row count that is
