@@ -17,9 +17,40 @@ constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 
 // ---- softmax of one contiguous run by one wavefront (all 64 lanes call this)
+// Runs of up to kWave * kSoftmaxRegs elements are read once and kept in registers (one read and one write
+// per element instead of three reads and two writes, all loads of a lane in flight together); the arithmetic
+// and its order are those of the strided loops below.
+constexpr int kSoftmaxRegs = 16;
 __device__ __forceinline__ void wave_softmax_inplace(float* x, long long len, int lane)
 {
     if (len <= 0) return;
+    if (len <= kWave * kSoftmaxRegs) {
+        const int n = (int)len;
+        const float first = x[0];                     // reference scan starts at element 0
+        float v[kSoftmaxRegs];
+#pragma unroll
+        for (int k = 0; k < kSoftmaxRegs; ++k) {
+            const int j = lane + k * kWave;
+            v[k] = j < n ? x[j] : first;              // the filler cannot change the maximum
+        }
+        float mx = first;
+#pragma unroll
+        for (int k = 0; k < kSoftmaxRegs; ++k) mx = max_keep(mx, v[k]);
+        mx = wave_max(mx);
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < kSoftmaxRegs; ++k) {
+            if (lane + k * kWave < n) {
+                v[k] = expf(v[k] - mx);
+                s += v[k];
+            }
+        }
+        s = wave_sum(s);
+#pragma unroll
+        for (int k = 0; k < kSoftmaxRegs; ++k)
+            if (lane + k * kWave < n) x[lane + k * kWave] = v[k] / s;
+        return;
+    }
     float mx = x[0];                                  // reference scan starts at element 0
     for (long long j = lane; j < len; j += kWave) mx = max_keep(mx, x[j]);
     mx = wave_max(mx);
