@@ -203,12 +203,77 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(
     }
 }
 
+// The same product for k <= 256: a lane keeps its four rows of B in registers, the groups stride the rows of A
+// four at a time (four 128-bit loads in flight per lane), and groups of up to 16 lanes reduce with DPP.
+template <int NCOL, bool TB>
+__global__ __launch_bounds__(kBlock) void sgemm_skinny_rows_kernel(
+    int m, int k, float alpha, const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb,
+    float beta, float* C, int ldc, int logG)
+{
+    constexpr int R = 4;
+    const int G = 1 << logG;
+    const int sub = threadIdx.x & (G - 1);
+    const int kk = sub * 4;
+    const bool live = kk < k;                              // k is a multiple of 4
+    float4 b[NCOL];
+#pragma unroll
+    for (int j = 0; j < NCOL; ++j) {
+        b[j] = f4_zero();
+        if (live) {
+            b[j].x = TB ? B[(size_t)j * ldb + kk] : B[(size_t)kk * ldb + j];
+            b[j].y = TB ? B[(size_t)j * ldb + kk + 1] : B[(size_t)(kk + 1) * ldb + j];
+            b[j].z = TB ? B[(size_t)j * ldb + kk + 2] : B[(size_t)(kk + 2) * ldb + j];
+            b[j].w = TB ? B[(size_t)j * ldb + kk + 3] : B[(size_t)(kk + 3) * ldb + j];
+        }
+    }
+    const long long groups = ((long long)gridDim.x * kBlock) >> logG;
+    const long long group = ((long long)blockIdx.x * kBlock + threadIdx.x) >> logG;
+    // all lanes of a wavefront run the same number of iterations (the reductions are wavefront-wide operations)
+    const long long first = ((long long)blockIdx.x * kBlock + (threadIdx.x & ~(kWave - 1))) >> logG;
+    for (long long base = 0; first + base < m; base += R * groups) {
+        float4 x[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const long long row = group + base + r * groups;
+            x[r] = (live && row < m) ? *reinterpret_cast<const float4*>(A + (size_t)row * lda + kk) : f4_zero();
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const long long row = group + base + r * groups;
+#pragma unroll
+            for (int j = 0; j < NCOL; ++j) {
+                float acc = x[r].x * b[j].x + x[r].y * b[j].y + x[r].z * b[j].z + x[r].w * b[j].w;
+                if (G >= 2) acc += dpp_mov_f<kDppXor1>(acc);
+                if (G >= 4) acc += dpp_mov_f<kDppXor2>(acc);
+                if (G >= 8) acc += dpp_mov_f<kDppHalfMirror>(acc);
+                if (G >= 16) acc += dpp_mov_f<kDppMirror>(acc);
+                if (G >= 32) acc += __shfl_xor(acc, 16, kWave);
+                if (G >= 64) acc += __shfl_xor(acc, 32, kWave);
+                if (row < m && sub == 0) {
+                    float* c = C + (size_t)row * ldc + j;
+                    *c = (beta == 0.f) ? alpha * acc : alpha * acc + beta * *c;
+                }
+            }
+        }
+    }
+}
+
 template <int NCOL>
 void launch_skinny(bool tb, int m, int k, float alpha, const float* A, int lda, const float* B, int ldb,
                    float beta, float* C, int ldc, hipStream_t s)
 {
     int logG = 0;
     while ((4 << logG) < k && logG < 6) ++logG;              // G * 4 >= k, at most one wavefront per row
+    if (k <= 4 * kWave) {
+        const size_t lanes = (size_t)m << logG;
+        size_t blocks = ceil_div_u(ceil_div_u(lanes, 4), kBlock);          // four rows per group
+        if (blocks > (size_t)kNumCU * 32) blocks = (size_t)kNumCU * 32;
+        if (blocks < 1) blocks = 1;
+        const unsigned grid = (unsigned)blocks;
+        if (tb) hipLaunchKernelGGL((sgemm_skinny_rows_kernel<NCOL, true>), dim3(grid), dim3(kBlock), 0, s, m, k, alpha, A, lda, B, ldb, beta, C, ldc, logG);
+        else hipLaunchKernelGGL((sgemm_skinny_rows_kernel<NCOL, false>), dim3(grid), dim3(kBlock), 0, s, m, k, alpha, A, lda, B, ldb, beta, C, ldc, logG);
+        return;
+    }
     const unsigned grid = ceil_div_u((size_t)m << logG, kBlock);
     if (tb) hipLaunchKernelGGL((sgemm_skinny_kernel<NCOL, true>), dim3(grid), dim3(kBlock), 0, s, m, k, alpha, A, lda, B, ldb, beta, C, ldc, logG);
     else hipLaunchKernelGGL((sgemm_skinny_kernel<NCOL, false>), dim3(grid), dim3(kBlock), 0, s, m, k, alpha, A, lda, B, ldb, beta, C, ldc, logG);

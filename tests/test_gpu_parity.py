@@ -129,7 +129,9 @@ def test_spmm_long_rows(gpu, oracle, n):
 
 # ------------------------------------------------------------------ GEMM
 @pytest.mark.parametrize("shape", [(1, 1, 1), (7, 5, 3), (64, 64, 16), (65, 63, 17), (300, 2, 32), (1000, 64, 38), (33, 130, 70),
-                                   (5000, 1, 64), (4097, 2, 32), (6000, 3, 8), (5001, 4, 260), (5000, 1, 4),
+                                   (5000, 1, 64), (4097, 2, 32), (6000, 3, 8), (5001, 4, 260), (5000, 1, 4), (5003, 3, 256),
+                                   (600_001, 2, 64),           # more rows than the row-strided kernel has lane groups
+                                  
                                    # few output tiles, long k (weight gradients): the product is split along k
                                    (64, 64, 7450), (38, 64, 7450), (70, 130, 3000), (64, 32, 1024), (2, 64, 4099)])
 def test_gemm_all_transposes(gpu, oracle, shape):
