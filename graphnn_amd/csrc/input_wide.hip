@@ -24,7 +24,7 @@ constexpr int kTileRows = 64;
 // KS = contraction steps of four: K <= 4 KS.
 template <int C, int KS>
 __global__ __launch_bounds__(kBlock) void s2v_input_wide_kernel(
-    int N, int K, const float* __restrict__ X, const float* __restrict__ Wn2l,
+    int N, int K, unsigned k_magic, int x_vec, const float* __restrict__ X, const float* __restrict__ Wn2l,
     float* __restrict__ msg, float* __restrict__ h0)
 {
     constexpr int CW = C / kWaves;           // output columns per wavefront
@@ -49,24 +49,60 @@ __global__ __launch_bounds__(kBlock) void s2v_input_wide_kernel(
 
     const int lane_off = (t * C + col0 + 4 * q) * 4;      // byte offset of this lane inside a 16-row block
     const int ntiles = (int)(((long long)N + kTileRows - 1) / kTileRows);
-    // X rows of a tile: wavefront w copies rows 16 w .. 16 w + 15, one row per load; the loads of the
-    // next tile are issued before the contraction of the current one
+    // X rows of a tile, asked for before the contraction of the previous tile.  A full tile is 64 K
+    // contiguous floats: with x_vec set (X 16-byte aligned) the workgroup reads them as KS/4 128-bit words per
+    // lane and scatters them into the padded LDS rows (row = element / K by one multiply-high with
+    // ceil(2^32 / K)); the last, partial tile and unaligned X go row by row: wavefront w copies rows
+    // 16 w .. 16 w + 15, one row per load.
+    constexpr int XQ = KS / 4;
     float xv[16];
+    float4 xq[XQ];
+    for (int i = threadIdx.x; i < kTileRows * LDT; i += kBlock) xt[i] = 0.f;      // the padding columns stay zero
+    auto full_tile = [&](int tile) { return x_vec && (long long)(tile + 1) * kTileRows <= (long long)N; };
     auto load_x = [&](int tile) {
-        const long long r0 = (long long)tile * kTileRows + wave * 16;
+        if (full_tile(tile)) {
+            const float4* xg = reinterpret_cast<const float4*>(X + (size_t)tile * kTileRows * K);
 #pragma unroll
-        for (int rr = 0; rr < 16; ++rr)
-            xv[rr] = (lane < K && r0 + rr < N) ? X[(size_t)(r0 + rr) * K + lane] : 0.f;
+            for (int p = 0; p < XQ; ++p) {
+                const int f = threadIdx.x + p * kBlock;
+                xq[p] = (f * 4 < kTileRows * K) ? xg[f] : f4_zero();
+            }
+        } else {
+            const long long r0 = (long long)tile * kTileRows + wave * 16;
+#pragma unroll
+            for (int rr = 0; rr < 16; ++rr)
+                xv[rr] = (lane < K && r0 + rr < N) ? X[(size_t)(r0 + rr) * K + lane] : 0.f;
+        }
+    };
+    auto park_x = [&](int tile) {
+        if (full_tile(tile)) {
+#pragma unroll
+            for (int p = 0; p < XQ; ++p) {
+                const int e = (threadIdx.x + p * kBlock) * 4;
+                if (e < kTileRows * K) {
+                    int r = K >= 2 ? (int)__umulhi((unsigned)e, k_magic) : e;
+                    int c = e - r * K;
+                    const float v[4] = {xq[p].x, xq[p].y, xq[p].z, xq[p].w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        xt[r * LDT + c] = v[i];           // 64 K is a multiple of 4: the four elements exist
+                        if (++c == K) { c = 0; ++r; }
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int rr = 0; rr < 16; ++rr)
+                if (lane < 4 * KS) xt[(wave * 16 + rr) * LDT + lane] = xv[rr];
+        }
     };
     if ((int)blockIdx.x < ntiles) load_x(blockIdx.x);
     for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const long long row0 = (long long)tile * kTileRows;
         const long long left = (long long)N - row0;
         const int rows = (int)(left < kTileRows ? left : kTileRows);
-        __syncthreads();                     // the previous tile has been consumed
-#pragma unroll
-        for (int rr = 0; rr < 16; ++rr)
-            if (lane < 4 * KS) xt[(wave * 16 + rr) * LDT + lane] = xv[rr];
+        __syncthreads();                     // the previous tile has been consumed (first pass: the zero fill is done)
+        park_x(tile);
         __syncthreads();
         if (tile + (int)gridDim.x < ntiles) load_x(tile + gridDim.x);
 
@@ -109,7 +145,9 @@ int launch_input_wide(int N, int K, const float* X, const float* Wn2l, float* ms
     const long long ntiles = ((long long)N + kTileRows - 1) / kTileRows;
     const long long cap = (long long)kNumCU * 4;
     const unsigned grid = (unsigned)(ntiles < cap ? ntiles : cap);
-    hipLaunchKernelGGL((s2v_input_wide_kernel<C, KS>), dim3(grid), dim3(kBlock), 0, s, N, K, X, Wn2l, msg, h0);
+    const unsigned k_magic = K >= 2 ? (unsigned)((0x100000000ull + (unsigned)K - 1) / (unsigned)K) : 0u;   // ceil(2^32 / K)
+    const int x_vec = aligned16(X) ? 1 : 0;
+    hipLaunchKernelGGL((s2v_input_wide_kernel<C, KS>), dim3(grid), dim3(kBlock), 0, s, N, K, k_magic, x_vec, X, Wn2l, msg, h0);
     GNNHIP_LAUNCH_CHECK("s2v_input_wide");
     return GNNHIP_OK;
 }
@@ -119,6 +157,7 @@ int input_wide_c(int N, int K, const float* X, const float* Wn2l, float* msg, fl
 {
     if (K <= 16) return launch_input_wide<C, 4>(N, K, X, Wn2l, msg, h0, s);
     if (K <= 32) return launch_input_wide<C, 8>(N, K, X, Wn2l, msg, h0, s);
+    if (K <= 48) return launch_input_wide<C, 12>(N, K, X, Wn2l, msg, h0, s);
     return launch_input_wide<C, 16>(N, K, X, Wn2l, msg, h0, s);
 }
 

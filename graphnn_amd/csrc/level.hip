@@ -581,7 +581,7 @@ int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float
     case 32: return small ? launch_input<32, 1>(N, K, X, Wn2l, msg, h0, s) : launch_input<32, 4>(N, K, X, Wn2l, msg, h0, s);
     case 64:
         // msg alone (the forward that does not store h0): the matrix-core kernel of the wide sizes is faster
-        // (880,690 nodes, 38 label types: 88 against 109 us); with h0 its 64-byte pieces per row and
+        // (880,690 nodes, 38 label types: 77 against 109 us); with h0 its 64-byte pieces per row and
         // wavefront cost more than they gain (158 against 144 us)
         if (!h0 && K <= 64) return input_wide_dispatch(N, K, C, X, Wn2l, msg, h0, s);
         return small ? launch_input<64, 1>(N, K, X, Wn2l, msg, h0, s) : launch_input<64, 4>(N, K, X, Wn2l, msg, h0, s);
