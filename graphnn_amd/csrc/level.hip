@@ -596,9 +596,9 @@ int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float
 // reads anyway).
 bool level_accepts_relu_input(int N, int C, long long nnz)
 {
-    if (level_wide_covers(N, C)) return true;
     const bool two_step = N >= kHubMinRows && nnz >= two_step_degree() * (long long)N;
-    return level_stream_covers(N, C) && !two_step;
+    if (two_step) return false;
+    return level_wide_covers(N, C) || level_stream_covers(N, C);
 }
 
 int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
@@ -644,6 +644,10 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
         default: return launch_level<64, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
         }
     }
+    // The wide kernel sums a row of any length inside one wavefront.  Large graphs with many entries per row
+    // (in practice the skewed ones, see above) are left to the caller's unfused route, whose SpMM balances
+    // long rows.
+    if (N >= kHubMinRows && nnz >= two_step_degree() * (long long)N) return GNNHIP_EUNSUPPORTED;
     switch (C) {
     case 128:
     case 256: return level_wide_dispatch(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, relu_in, s);

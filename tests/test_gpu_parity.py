@@ -409,6 +409,27 @@ def test_level_every_row_length_up_to_70(gpu, oracle, C, N):
     assert max_rel(got, want) < PARITY_TOL
 
 
+def test_wide_level_on_a_large_dense_skewed_graph(gpu, oracle):
+    """hidden 128 on a graph of 40,000 rows with 14 entries per row on average and two rows of 5,000 and
+    3,000 entries: the level leaves the wide fused kernel (one wavefront per row, whatever its length) for
+    SpMM with the balanced pass + GEMM + epilogue; the forward entry must not hand it ReLU-through-msg"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(77)
+    N, C = 40_000, 128
+    lens = rng.integers(10, 17, N); lens[123] = 5_000; lens[39_999] = 3_000
+    rp = np.zeros(N + 1, np.int32); np.cumsum(lens, out=rp[1:])
+    nnz = int(rp[-1])
+    assert nnz >= 12 * N
+    ci = rng.integers(0, N, nnz).astype(np.int32)
+    v = (rng.random(nnz) * 0.05).astype(np.float32)
+    h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
+    W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
+    msg = rng.standard_normal((N, C)).astype(np.float32)
+    want = oracle.level(rp, ci, v, h_in, W, msg, None)
+    got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu)))
+    assert max_rel(got, want) < PARITY_TOL
+
+
 @pytest.mark.parametrize("C", [128, 256])
 @pytest.mark.parametrize("nnz", [0, 1, 5, 6, 7])
 def test_wide_level_fewer_entries_than_one_index_batch(gpu, oracle, C, nnz):
