@@ -668,7 +668,9 @@ def test_batched_forward_matches_reference_path(gpu, oracle, config_id):
 
 
 @pytest.mark.parametrize("C,K,H,Q,L", [(16, 7, 8, 3, 2), (32, 20, 16, 2, 3), (64, 64, 32, 5, 1), (64, 3, 100, 70, 0),
-                                       (32, 48, 8, 2, 5), (16, 33, 4, 2, 1)])
+                                       (32, 48, 8, 2, 5), (16, 33, 4, 2, 1),
+                                       # label counts around the steps of the input stage (two columns per 64-bit read)
+                                       (64, 1, 8, 2, 2), (32, 2, 8, 2, 1), (64, 17, 16, 3, 2), (16, 49, 8, 2, 1)])
 def test_batched_forward_shapes(gpu, oracle, C, K, H, Q, L):
     seed = 1000 + C + K + L
     batch = synth.molecule_batch(seed, 37, K, Q, size_mode="uniform", size_lo=1, size_hi=70)
@@ -710,6 +712,23 @@ def test_batched_forward_large_and_dense_graphs(gpu, oracle):
     gen = ops.s2v_forward(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
                           _t(w.W_h1, gpu), _t(w.W_h2, gpu), L)
     assert max_rel(_n(gen.logits), _n(bufs.logits)) < PARITY_TOL
+
+
+def test_batched_forward_dense_features_past_the_staging_registers(gpu, oracle):
+    """64 real-valued feature columns on graphs of up to 190 nodes: a graph's block of X (12,160 floats) is longer
+    than what the lanes stage in one go, and its rows outnumber the gather rounds kept in registers"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(123)
+    K, C, H, Q, L = 64, 64, 32, 2, 2
+    batch = synth.molecule_batch(321, 9, K, Q, size_mode="uniform", size_lo=150, size_hi=190)
+    w = synth.make_weights(synth.Stream(321), K, C, H, Q)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = rng.standard_normal((batch.num_nodes, K)).astype(np.float32)
+    want = oracle.forward(a, s, X, w, L, None)
+    bufs = ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+                                   _t(w.W_h1, gpu), _t(w.W_h2, gpu), L, int(batch.graph_sizes.max()))
+    _assert_batched_matches(want, bufs, L)
 
 
 def test_batched_forward_reports_broken_promises(gpu, oracle):
