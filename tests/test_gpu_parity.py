@@ -1050,11 +1050,12 @@ def test_device_csr_group_edge_cases_and_scale(gpu, oracle):
         assert np.array_equal(_n(g), w_)
 
 
-def test_device_csr_transpose(gpu, oracle):
+@pytest.mark.parametrize("m,k,nnz", [(411, 233, 3000), (5000, 7000, 120_000), (3, 70_000, 32_768), (1, 1, 1)])
+def test_device_csr_transpose(gpu, oracle, m, k, nnz):
+    """one tile, many tiles, few long rows of A, a single entry"""
     from graphnn_amd import ops
-    rng = np.random.default_rng(10)
-    m, k = 411, 233
-    csr = _random_csr(rng, m, k, 3000)
+    rng = np.random.default_rng(10 + m)
+    csr = _random_csr(rng, m, k, nnz)
     t_rp, t_ci, t_v = ops.csr_transpose(*_csr_t(csr, gpu), m, k)
     import scipy.sparse as sp
     A = sp.csr_matrix((csr[2], csr[1], csr[0]), shape=(m, k))
