@@ -308,9 +308,11 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
             int ns = 0, nend = 0;
             if (rt < kTileRows / 16 - 1) {
                 if (e + kInFlight < ee) { ns = e + kInFlight; nend = ee; }
-            } else if (e + kInFlight >= ee) {
+            } else if (kTileRows > 16 && e + kInFlight >= ee) {
                 ns = ebN; nend = eeN;                     // both zero when there is no next pass
             }
+            // (a 16-row pass has one block: ebN/eeN still describe the pass being gathered, the row pointers of
+            // the one after it arrive during this block, so its first batch is asked for after the block)
             GNNHIP_PHASE_ACC(1);
 
             const float* src = cur + (rt * 16 + t) * LDT + KS * q;
@@ -375,7 +377,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
             out_rt = rt;
             GNNHIP_PHASE_ACC(4);
         }
-        if (e < ee) {                                     // more than four batches: finish in the open
+        if (kTileRows == 16 || e < ee) {                  // more batches than blocks: finish in the open
             while (e < ee) {
                 vec_t x[kInFlight];
                 cShift = load_batch(col_idx, e, cC);
@@ -403,7 +405,10 @@ int launch_level_wide_t(int N, const int* row_ptr, const int* col_idx, const flo
     if ((unsigned long long)N * C * 4ull >= (1ull << 32)) return GNNHIP_EUNSUPPORTED;   // 32-bit buffer offsets
     constexpr int kTileRows = TR;
     const long long ntiles = ((long long)N + kTileRows - 1) / kTileRows;
-    const long long per = (ntiles + kNumCU - 1) / kNumCU;            // contiguous run of tiles per workgroup
+    // workgroups that fit one compute unit together: two at C = 128 (82 registers per lane, 68 KB of LDS each)
+    constexpr int kPerCU = (C == 128) ? 2 : 1;
+    const long long slots = (long long)kNumCU * kPerCU;
+    const long long per = (ntiles + slots - 1) / slots;              // contiguous run of tiles per workgroup
     const long long blocks = (ntiles + per - 1) / per;
     const size_t smem = sizeof(float) * (2 * kTileRows * (C + 4) + C);
     static bool attr_set = false;                                    // more than 64 KB of LDS has to be asked for
@@ -424,8 +429,9 @@ template <int C, int WAVES, bool RELU_IN>
 int launch_level_wide(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
                       const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
 {
-    if (N >= 2 * kNumCU * 64) return launch_level_wide_t<C, WAVES, RELU_IN, 64>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
-    if (N >= 2 * kNumCU * 32) return launch_level_wide_t<C, WAVES, RELU_IN, 32>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    constexpr int kSlots = kNumCU * ((C == 128) ? 2 : 1);
+    if (N >= 2 * kSlots * 64) return launch_level_wide_t<C, WAVES, RELU_IN, 64>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    if (N >= 2 * kSlots * 32) return launch_level_wide_t<C, WAVES, RELU_IN, 32>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
     return launch_level_wide_t<C, WAVES, RELU_IN, 16>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
 }
 

@@ -456,11 +456,11 @@ def test_wide_level_fewer_entries_than_one_index_batch(gpu, oracle, C, nnz):
 
 
 @pytest.mark.parametrize("C", [128, 256])
-@pytest.mark.parametrize("N", [5_003, 64 * 300 + 37, 40_037])
+@pytest.mark.parametrize("N", [5_003, 10_007, 15_991, 64 * 300 + 37, 40_037, 70_001])
 def test_wide_level_ragged_rows_and_weights(gpu, oracle, C, N):
     """wide-hidden kernel: empty rows, rows longer than one 64-entry index batch, a row count that is
-    not a multiple of the pass, non-unit weights; the three sizes take passes of 16, 32 and 64 rows, each
-    with more passes than compute units take one each"""
+    not a multiple of the pass, non-unit weights; the sizes take passes of 16, 32 and 64 rows, with two to
+    four passes per workgroup (three and more exercise the look-ahead across passes)"""
     from graphnn_amd import ops
     rng = np.random.default_rng(90 + C + N)
     lens = rng.integers(0, 7, N); lens[5] = 700; lens[6] = 0; lens[7] = 0; lens[N - 1] = 130; lens[64:72] = 0
