@@ -162,3 +162,30 @@ def test_level_past_4_gib_of_activations(gpu):
     want = torch.relu(agg @ W.double() + msg[rows].double())
     got = out[rows].double()
     assert float((got - want).abs().max()) <= PARITY_TOL * max(1.0, float(want.abs().max()))
+
+
+def test_spmm_long_rows_past_4m_rows(gpu):
+    """4.3M rows: the planning of the balanced pass over long rows takes its three-launch form (count, scan,
+    fill) past 4,096 row blocks.  One entry per row plus long rows in the first, a middle and the last block;
+    the long rows and sampled short ones against float64."""
+    import torch
+    from graphnn_amd import ops
+    m, k, n = 4_300_007, 50_000, 16
+    g = torch.Generator(device=gpu); g.manual_seed(43)
+    lens = torch.ones(m, dtype=torch.int64, device=gpu)
+    hubs = {5: 70, 2_222_222: 5_000, m - 1: 3_001, m - 2050: 65}
+    for r, l in hubs.items():
+        lens[r] = l
+    rp = torch.zeros(m + 1, dtype=torch.int64, device=gpu)
+    rp[1:] = torch.cumsum(lens, 0)
+    nnz = int(rp[-1].item())
+    ci = torch.randint(0, k, (nnz,), device=gpu, generator=g, dtype=torch.int64).to(torch.int32)
+    val = torch.rand((nnz,), generator=g, device=gpu) - 0.5
+    X = torch.randn((k, n), generator=g, device=gpu)
+    Y = ops.spmm(rp.to(torch.int32), ci, val, X, m)
+    rows = torch.cat((torch.tensor(sorted(hubs), device=gpu), torch.randint(0, m, (3000,), device=gpu, generator=g)))
+    for r in rows.tolist():
+        a, b = int(rp[r].item()), int(rp[r + 1].item())
+        want = (val[a:b].double()[:, None] * X[ci[a:b].long()].double()).sum(0)
+        got = Y[r].double()
+        assert float((got - want).abs().max()) <= PARITY_TOL * max(1.0, float(want.abs().max())), r
