@@ -351,6 +351,21 @@ def test_input_stage(gpu, oracle, C, K):
     assert np.array_equal(_n(h0), np.maximum(_n(msg), 0))       # ReLU of what was stored, exactly
 
 
+@pytest.mark.parametrize("C", [16, 32, 64, 128])
+@pytest.mark.parametrize("K", [5, 38])
+def test_input_stage_many_rows(gpu, oracle, C, K):
+    """40,003 rows: past 32,768 rows the narrow hidden sizes take four row tiles per workgroup, and every
+    kernel gives a workgroup more than one tile; msg and h0 both stored, real-valued X"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(7 * C + K)
+    N = 40_003
+    X = rng.standard_normal((N, K)).astype(np.float32)
+    Wn = (rng.standard_normal((K, C)) * 0.3).astype(np.float32)
+    msg, h0 = ops.s2v_input(_t(X, gpu), _t(Wn, gpu))
+    assert max_rel(_n(msg), oracle.gemm(X, Wn)) < PARITY_TOL
+    assert np.array_equal(_n(h0), np.maximum(_n(msg), 0))
+
+
 @pytest.mark.parametrize("C", [16, 32, 64, 48, 128, 256])
 @pytest.mark.parametrize("with_msg,with_bias", [(True, False), (True, True), (False, False)])
 def test_level_stage(gpu, oracle, C, with_msg, with_bias):
