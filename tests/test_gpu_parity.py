@@ -383,6 +383,33 @@ def test_level_stage(gpu, oracle, C, with_msg, with_bias):
     assert np.all(got >= 0)
 
 
+@pytest.mark.parametrize("C", [16, 32, 64, 128, 256])
+def test_level_stage_row_counts_around_every_threshold(gpu, oracle, C):
+    """row counts on both sides of the tile sizes (16, 64), of the sizes at which the kernels change their
+    rows per pass or start asking for gathers a tile early (16,384, 32,768, 65,536) and of one, two and more
+    tiles per wavefront; ragged rows of 0..5 entries, weights, msg and bias"""
+    from graphnn_amd import ops
+    for N in (1, 15, 16, 17, 63, 64, 65, 1023, 1025, 4097, 12289, 16383, 16385, 32767, 32769, 49153, 65535, 65537):
+        rng = np.random.default_rng(1000 * C + N)
+        lens = rng.integers(0, 6, N)
+        rp = np.zeros(N + 1, np.int32); np.cumsum(lens, out=rp[1:])
+        nnz = int(rp[-1])
+        ci = rng.integers(0, N, nnz).astype(np.int32)
+        v = (rng.random(nnz) * 0.5).astype(np.float32)
+        h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
+        W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
+        msg = rng.standard_normal((N, C)).astype(np.float32)
+        bias = rng.standard_normal(C).astype(np.float32)
+        want = oracle.level(rp, ci, v, h_in, W, msg, bias)
+        if nnz:
+            ci_d, v_d = _t(ci, gpu), _t(v, gpu)
+        else:
+            import torch
+            ci_d = torch.zeros(1, dtype=torch.int32, device=gpu)[:0]; v_d = torch.zeros(1, dtype=torch.float32, device=gpu)[:0]
+        got = _n(ops.s2v_level(_t(rp, gpu), ci_d, v_d, _t(h_in, gpu), _t(W, gpu), _t(msg, gpu), _t(bias, gpu)))
+        assert max_rel(got, want) < PARITY_TOL, N
+
+
 def test_level_stage_hub_rows_and_weights(gpu, oracle):
     """one vertex with thousands of in-neighbours (whole-workgroup gather) and non-unit edge weights"""
     from graphnn_amd import ops
@@ -579,6 +606,28 @@ def test_forward_matches_reference_path(gpu, oracle, config_id):
     assert abs(acc - want["scalars"][1]) <= 1e-6
 
 
+@pytest.mark.parametrize("C,H,Q", [(64, 32, 2), (32, 8, 3), (128, 16, 2), (256, 8, 2)])
+def test_forward_graph_counts_around_the_readout_thresholds(gpu, oracle, C, H, Q):
+    """whole forward (general route) on batches of 1 .. 4,100 small graphs: the readout changes kernel at 1,024
+    graphs (one wavefront per graph, hidden <= 64) and at 4,096 graphs (hidden 128/256: workgroup per graph, then
+    SpMM + GEMM)"""
+    from graphnn_amd import ops
+    K, L = 6, 2
+    for B in (1, 2, 255, 1023, 1024, 1025, 4096, 4100):
+        seed = 31 * C + B
+        batch = synth.molecule_batch(seed, B, K, Q, size_mode="uniform", size_lo=1, size_hi=7)
+        w = synth.make_weights(synth.Stream(seed), K, C, H, Q)
+        a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+        s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+        X = batch.one_hot()
+        want = oracle.forward(a, s, X, w, L, None)
+        bufs = ops.s2v_forward(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+                               _t(w.W_h1, gpu), _t(w.W_h2, gpu), L)
+        for key in ("pool", "hidden", "logits", "probs"):
+            assert max_rel(_n(getattr(bufs, key)), want[key]) < PARITY_TOL, (B, key)
+        assert np.array_equal(_n(bufs.pred), want["pred"]), B
+
+
 def test_forward_every_level_matches(gpu, oracle):
     """level by level through the per-level entry point, against each of the oracle's stored h_l"""
     from graphnn_amd import ops
@@ -692,6 +741,19 @@ def test_batched_forward_shapes(gpu, oracle, C, K, H, Q, L):
     w = synth.make_weights(synth.Stream(seed), K, C, H, Q)
     want, bufs = _batched_case(gpu, oracle, batch, w, L)
     _assert_batched_matches(want, bufs, L)
+
+
+@pytest.mark.parametrize("C", [16, 64])
+def test_batched_forward_graph_counts(gpu, oracle, C):
+    """one graph, more graphs than compute units, exactly and more than the 1,024 workgroups of a launch (each
+    workgroup then walks several graphs); graphs of 1..20 nodes, one of them empty of edges"""
+    K, H, Q, L = 11, 8, 2, 3
+    for B in (1, 257, 1024, 1025, 2500):
+        seed = 17 * C + B
+        batch = synth.molecule_batch(seed, B, K, Q, size_mode="uniform", size_lo=1, size_hi=20)
+        w = synth.make_weights(synth.Stream(seed), K, C, H, Q)
+        want, bufs = _batched_case(gpu, oracle, batch, w, L)
+        _assert_batched_matches(want, bufs, L)
 
 
 def test_batched_forward_large_and_dense_graphs(gpu, oracle):
