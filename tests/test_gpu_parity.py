@@ -897,6 +897,21 @@ def _hub_matrix(rng, m, k, long_rows):
     return rp, ci, v
 
 
+@pytest.mark.parametrize("n", [4, 64, 100])
+def test_spmm_long_rows_around_the_row_count_threshold(gpu, oracle, n):
+    """the balanced pass over long rows starts at 32,768 rows; below it a long row is split inside one workgroup.
+    The same long rows (65, 2,048, 2,049, 5,000 entries, first and last row) one row below, at and above it."""
+    from graphnn_amd import ops
+    for m in (32_767, 32_768, 32_769):
+        rng = np.random.default_rng(m + n)
+        k = 5000
+        csr = _hub_matrix(rng, m, k, [(0, 5000), (9, 65), (10, 2048), (11, 2049), (m // 2, 64), (m - 1, 3000)])
+        B = rng.standard_normal((k, n)).astype(np.float32)
+        got = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m))
+        want = oracle.spmm(*csr, B, m)
+        assert max_rel(got, want) < PARITY_TOL, m
+
+
 @pytest.mark.parametrize("n", [64, 128, 7, 36, 300])
 def test_spmm_hub_rows_balanced_pass(gpu, oracle, n):
     """matrix large enough for the balanced pass over long rows: rows of 65 and 257 (one chunk), 2048, 2049 and
