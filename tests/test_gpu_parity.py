@@ -241,7 +241,7 @@ def test_memset0_batch(gpu):
 
 
 # ------------------------------------------------------------------ softmax family
-@pytest.mark.parametrize("rows,cols", [(20, 200), (256, 2), (7, 1), (3, 64), (5, 65), (2, 5000)])
+@pytest.mark.parametrize("rows,cols", [(20, 200), (256, 2), (7, 1), (3, 64), (5, 65), (2, 5000), (3, 1023), (3, 1024), (3, 1025)])
 def test_row_softmax(gpu, oracle, rows, cols):
     from graphnn_amd import ops
     rng = np.random.default_rng(rows * cols)
