@@ -136,8 +136,18 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     if (tid0 < LDT) hbuf[(size_t)n16max * LDT + tid0] = 0.f;
     if (ro_staged) {
         // coalesced reads; the transposed layout lets a wavefront read one output's weights contiguously
-        for (int i = tid0; i < C * H; i += kBlock) w1s[(i % H) * C + i / H] = Wh1[i];
-        for (int i = tid0; i < H * Q; i += kBlock) w2s[(i % Q) * H + i / Q] = Wh2[i];
+        // (four elements of W_h1 and one of W_h2 per lane are asked for together: one trip to memory for the
+        // usual sizes instead of one per element)
+        const int n1 = C * H, n2 = H * Q;
+        float v1[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { const int i = tid0 + u * kBlock; v1[u] = i < n1 ? Wh1[i] : 0.f; }
+        const float v2 = tid0 < n2 ? Wh2[tid0] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { const int i = tid0 + u * kBlock; if (i < n1) w1s[(i % H) * C + i / H] = v1[u]; }
+        if (tid0 < n2) w2s[(tid0 % Q) * H + tid0 / Q] = v2;
+        for (int i = tid0 + 4 * kBlock; i < n1; i += kBlock) w1s[(i % H) * C + i / H] = Wh1[i];
+        for (int i = tid0 + kBlock; i < n2; i += kBlock) w2s[(i % Q) * H + i / Q] = Wh2[i];
     }
     // (the staged copies become visible to all lanes at the first barrier of the graph loop)
     GNNHIP_PHASE_MARK(1);
