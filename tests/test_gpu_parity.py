@@ -628,6 +628,34 @@ def test_forward_graph_counts_around_the_readout_thresholds(gpu, oracle, C, H, Q
         assert np.array_equal(_n(bufs.pred), want["pred"]), B
 
 
+def test_forward_on_two_streams_interleaved(gpu, oracle):
+    """two forwards queued alternately on two streams (scratch buffers and the plan of the long-row pass are
+    kept per stream): each gives what it gives alone"""
+    import torch
+    from graphnn_amd import ops
+    cases = []
+    for seed, B, C in ((1, 300, 64), (2, 40, 128)):
+        batch = synth.molecule_batch(seed, B, 9, 2, size_mode="uniform", size_lo=5, size_hi=200)
+        w = synth.make_weights(synth.Stream(seed), 9, C, 16, 2)
+        a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+        s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+        args = (_csr_t(a, gpu), _csr_t(s, gpu), _t(batch.one_hot(), gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+                _t(w.W_h1, gpu), _t(w.W_h2, gpu), 3)
+        alone = _n(ops.s2v_forward(*args).logits)
+        cases.append((args, alone))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[], []]
+    for _ in range(6):
+        for k in (0, 1):
+            with torch.cuda.stream(streams[k]):
+                outs[k].append(ops.s2v_forward(*cases[k][0]).logits)
+    torch.cuda.synchronize()
+    for k in (0, 1):
+        for o in outs[k]:
+            assert np.array_equal(_n(o), cases[k][1])
+
+
 def test_forward_every_level_matches(gpu, oracle):
     """level by level through the per-level entry point, against each of the oracle's stored h_l"""
     from graphnn_amd import ops
