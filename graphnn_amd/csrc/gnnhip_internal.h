@@ -157,6 +157,10 @@ int stream_scratch(hipStream_t s, size_t bytes, void** p);
 constexpr int kScratchSlots = 3;
 int stream_scratch_slot(hipStream_t s, int slot, size_t bytes, void** p);
 
+// reduce.hip: device address of the statically allocated segment offsets on the current device
+// (hipGetSymbolAddress once per device; allocates nothing).
+int static_offsets_ptr(int** out);
+
 // ---- high-degree rows (hub.hip)
 constexpr int kHubThreshold = 64;      // rows with more entries are summed by the pre-pass
 constexpr int kHubChunk = 2048;        // entries per partial sum of the pre-pass

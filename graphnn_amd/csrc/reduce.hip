@@ -10,8 +10,21 @@
 // 4 bytes per element for the reductions.
 #include "gnnhip_internal.h"
 
+#include <mutex>
+
 namespace gnnhip {
 namespace {
+
+// Segment offsets of the jagged softmax entry point that allocates nothing: one copy of this array per
+// GPU, held from the moment the library is loaded until the process ends (256 KiB + 4 B).  In host code
+// the array's name is only a handle for hipGetSymbolAddress; kernels receive the address that call
+// returns on the current device.
+constexpr int kStaticMaxSegments = 65536;
+static __device__ __align__(256) int scratch[kStaticMaxSegments + 1];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mu;
+int* g_static_offsets[kMaxDevices] = {};          // device address of `scratch` on each GPU, filled on first use
 
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
@@ -232,6 +245,23 @@ inline unsigned lane_rows_grid(long long rows)
 
 }  // namespace
 
+// Address of the current device's copy of `scratch` (resolved once per device, no allocation).
+int static_offsets_ptr(int** out)
+{
+    int dev = -1;
+    GNNHIP_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return set_error(GNNHIP_EINVAL, "device ordinal %d outside [0,%d)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_static_mu);
+    if (!g_static_offsets[dev]) {
+        void* p = nullptr;
+        GNNHIP_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return set_error(GNNHIP_EHIP, "hipGetSymbolAddress returned a null address for the static offsets");
+        g_static_offsets[dev] = static_cast<int*>(p);
+    }
+    *out = g_static_offsets[dev];
+    return GNNHIP_OK;
+}
+
 int row_softmax_dispatch(float* x, int rows, int cols, hipStream_t s)
 {
     hipLaunchKernelGGL(row_softmax_kernel, dim3(wave_rows_grid(rows)), dim3(kBlock), 0, s, x, rows, cols);
@@ -271,6 +301,25 @@ int gnnhip_jagged_softmax_f32(float* x, const int* lens, int nseg, void* stream)
     void* off = nullptr;
     if (int rc = stream_scratch(s, sizeof(int) * ((size_t)nseg + 1), &off)) return rc;
     hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(kScanBlock), 0, s, lens, nseg, static_cast<int*>(off));
+    GNNHIP_LAUNCH_CHECK("exclusive_scan");
+    hipLaunchKernelGGL(jagged_softmax_kernel, dim3(wave_rows_grid(nseg)), dim3(kBlock), 0, s, x, static_cast<const int*>(off), nseg);
+    GNNHIP_LAUNCH_CHECK("jagged_softmax");
+    return GNNHIP_OK;
+}
+
+int gnnhip_jagged_softmax_static_f32(float* x, const int* lens, int nseg, void* stream)
+{
+    GNNHIP_REQUIRE(nseg >= 0, "negative segment count");
+    GNNHIP_REQUIRE(nseg <= kStaticMaxSegments, "jagged_softmax_static takes at most %d segments, got %d (use gnnhip_jagged_softmax_f32)",
+                   kStaticMaxSegments, nseg);
+    if (nseg == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(x && lens, "null tensor in jagged_softmax_static");
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    int* off = nullptr;
+    if (int rc = static_offsets_ptr(&off)) return rc;
+    // the scan writes off[0..nseg] in full, so what an earlier call left in the array is never read
+    hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(kScanBlock), 0, s, lens, nseg, off);
     GNNHIP_LAUNCH_CHECK("exclusive_scan");
     hipLaunchKernelGGL(jagged_softmax_kernel, dim3(wave_rows_grid(nseg)), dim3(kBlock), 0, s, x, static_cast<const int*>(off), nseg);
     GNNHIP_LAUNCH_CHECK("jagged_softmax");

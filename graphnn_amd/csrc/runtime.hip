@@ -183,6 +183,10 @@ int gnnhip_init(int device_id)
     GNNHIP_HIP(hipSetDevice(device_id));
     r.device = device_id;
     r.ready = true;
+    // resolve this device's copy of the static offsets array now, so the entry point that may not
+    // allocate finds it ready (it resolves it itself if the caller moved to another device)
+    int* unused = nullptr;
+    if (int rc = static_offsets_ptr(&unused)) return rc;
     return GNNHIP_OK;
 }
 

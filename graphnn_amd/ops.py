@@ -264,6 +264,12 @@ def jagged_softmax(x, lens):
     return x
 
 
+def jagged_softmax_static(x, lens):
+    """gnnhip_jagged_softmax_static_f32: the same result, segment offsets in the library's static array."""
+    check(_lib().gnnhip_jagged_softmax_static_f32(_f32(x, "x"), _i32(lens, "lens"), lens.numel(), _stream()))
+    return x
+
+
 def reduce(op, x):
     out = torch.empty((1,), dtype=torch.float32, device=x.device)
     check(_lib().gnnhip_reduce_f32(REDUCE[op], _f32(x, "x"), x.numel(), _f32(out, "out"), _stream()))

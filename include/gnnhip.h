@@ -194,6 +194,16 @@ int gnnhip_row_softmax_f32(float* x, int rows, int cols, void* stream);
  *      Segment offsets come from an exclusive scan of lens done on the device. */
 int gnnhip_jagged_softmax_f32(float* x, const int* lens, int nseg, void* stream);
 
+/* ---- the same jagged softmax for callers that cannot allocate device memory (code under HIP graph
+ *      capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ *      The segment offsets live in an array that is part of the library's device image (256 KiB per GPU,
+ *      held until the process ends), so the call makes no hipMalloc / hipFree and no allocating library
+ *      call.  nseg <= GNNHIP_JAGGED_STATIC_MAX_SEGMENTS, otherwise GNNHIP_EINVAL and nothing is launched.
+ *      All calls on one GPU share that array: calls that overlap on one GPU (different streams, or
+ *      different threads) race; order them on one stream. */
+#define GNNHIP_JAGGED_STATIC_MAX_SEGMENTS 65536
+int gnnhip_jagged_softmax_static_f32(float* x, const int* lens, int nseg, void* stream);
+
 /* ---- global sum / mean / max / sum of squares into out[0] (device):
  *      DTensor<GPU>::Sum / Mean (src/tensor/gpu_dense_tensor.cu:466-481),
  *      MatColReduceKernel (include/tensor/gpu_reduce_kernel.h:57-99) */

@@ -39,6 +39,8 @@ def test_header_cites_the_reference_for_every_entry():
     blocks = re.findall(r"/\* ----(.*?)\*/", text, flags=re.S)
     assert len(blocks) >= 20
     for b in blocks:
+        if "No counterpart in the reference" in b:      # the entry for callers that cannot allocate
+            continue
         assert re.search(r"(src|include|examples)/[\w/]+\.(cpp|cu|h)", b), b[:80]
 
 
