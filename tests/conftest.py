@@ -213,24 +213,110 @@ def ref_graph():
     return ctypes.CDLL(_REF_PATH)
 
 
-def max_rel(a, b, floor=None):
+PARITY_TOL = 1e-4     # the north-star tolerance for fp32 activations and logits
+
+# Floors of the parity metric, measured (see the sweep recorded in DESIGN.md): the smallest floor at which
+# the oracle itself stays within 1e-4 of a float64 model of the same network on configurations 1 and 2
+# (12 to 3,000 graphs) is 1.3e-3 of the tensor's largest magnitude for the embeddings and the hidden layer,
+# 4e-5 for the pooled features and zero for the probabilities.  Two correct fp32 summation orders differ
+# by the sum of two such errors, hence the values below.
+FLOOR_DEFAULT = 2e-3          # fraction of max|ref|: embeddings, hidden layer, general sums
+FLOOR_POOL = 1e-4             # fraction of max|ref|: pooled features (sums of non-negative terms)
+FLOOR_PROBS_ABS = 1e-6        # absolute: probabilities
+
+
+def max_rel(a, b, floor=None, floor_frac=FLOOR_DEFAULT):
     """Parity metric for fp32 tensors: max_i |a_i - b_i| / max(|a_i|, |b_i|, floor).
 
-    The floor defaults to 1% of the reference tensor's largest magnitude.  A fixed
-    tiny floor is not usable: post-ReLU activations are sums with cancellation, so an
-    element that is 1e-5 of the tensor's scale legitimately differs by parts in 1e-2
-    between two correct fp32 summation orders.  With this floor the 1e-4 bound reads
-    "relative 1e-4 on every element that matters, absolute 1e-6 x scale on the rest".
+    floor (absolute) defaults to floor_frac times the reference tensor's largest magnitude.  A fixed tiny
+    floor is not usable on post-ReLU activations and logits: they are sums with cancellation, so an element
+    at 1e-4 of the tensor's scale legitimately differs by parts in 1e-3 between two correct fp32 summation
+    orders (the oracle itself fails a 1e-6 floor against a float64 model, see worst_element).
     """
     a = np.asarray(a, np.float64); b = np.asarray(b, np.float64)
     if a.size == 0:
         return 0.0
     if floor is None:
-        floor = max(1e-2 * float(np.max(np.abs(b))), 1e-30)
+        floor = max(floor_frac * float(np.max(np.abs(b))), 1e-30)
     return float(np.max(np.abs(a - b) / np.maximum(np.maximum(np.abs(a), np.abs(b)), floor)))
 
 
-PARITY_TOL = 1e-4     # the north-star tolerance for fp32 activations and logits
+def worst_element(a, b, floor=1e-6):
+    """(relative error, flat index, a_i, b_i) of the worst element under a fixed absolute floor."""
+    a = np.asarray(a, np.float64).ravel(); b = np.asarray(b, np.float64).ravel()
+    if a.size == 0:
+        return 0.0, -1, 0.0, 0.0
+    rel = np.abs(a - b) / np.maximum(np.maximum(np.abs(a), np.abs(b)), floor)
+    i = int(np.argmax(rel))
+    return float(rel[i]), i, float(a[i]), float(b[i])
+
+
+class Lazy:
+    """A value computed on first use (float64 models are only needed when a comparison misses);
+    lazy[key] is the lazily indexed value."""
+
+    def __init__(self, fn):
+        self._fn, self._done, self._val = fn, False, None
+
+    def __call__(self):
+        if not self._done:
+            self._val, self._done = self._fn(), True
+        return self._val
+
+    def __getitem__(self, key):
+        return Lazy(lambda: self()[key])
+
+
+# Two correct fp32 evaluations of one sum are each a few 1e-5 to 1e-4 from float64 on the worst element of a
+# large tensor, and which of the two is further is a coin toss (observed device/oracle ratios on the tests of
+# this suite: 0.3 to 2.6; the matrix cores do not round partial sums the way a serial fp32 loop does).  The
+# float64 arbiter therefore accepts a device result up to this factor further from float64 than the oracle;
+# a wrong index, a dropped term or reduced precision is off by orders of magnitude.
+ARBITER_SLACK = 4.0
+
+
+def assert_parity(name, got, want, want64=None, tol=PARITY_TOL, floor=None, floor_frac=FLOOR_DEFAULT):
+    """got (device) against want (oracle) under max_rel; prints the worst element under the fixed 1e-6 floor.
+
+    With want64 (a float64 model of the same computation, or a callable giving it) a miss is still a pass
+    when the device is about as close to float64 as the oracle is (ARBITER_SLACK): both are then correct
+    fp32 evaluations that differ in summation order on an element the floor does not cover."""
+    err = max_rel(got, want, floor, floor_frac)
+    rel, i, gi, wi = worst_element(got, want)
+    print("parity %-10s max_rel %.2e (floor %s); worst element under the fixed 1e-6 floor: [%d] device %.9g oracle %.9g rel %.2e"
+          % (name, err, ("%.1e" % floor) if floor is not None else ("%.0e x max|ref|" % floor_frac), i, gi, wi, rel))
+    if err < tol:
+        return err
+    if want64 is not None:
+        if callable(want64):
+            want64 = want64()
+        e_dev = max_rel(got, want64, floor, floor_frac)
+        e_ref = max_rel(want, want64, floor, floor_frac)
+        print("       %-10s vs float64: device %.2e, oracle %.2e" % (name, e_dev, e_ref))
+        assert e_dev <= max(ARBITER_SLACK * e_ref, tol), "%s: device %.3e from float64, oracle %.3e (device vs oracle %.3e)" % (name, e_dev, e_ref, err)
+        return err
+    raise AssertionError("%s differs from the oracle: max_rel %.3e >= %.1e" % (name, err, tol))
+
+
+def forward_float64(a_csr, s_csr, X, w, L):
+    """The network of kernel_mean_field.cpp:31-56 in float64 (scipy CSR products): the arbiter between two
+    fp32 evaluations."""
+    import scipy.sparse as sp
+    N = X.shape[0]; B = len(s_csr[0]) - 1
+    f8 = np.float64
+    A = sp.csr_matrix((a_csr[2].astype(f8), a_csr[1], a_csr[0]), shape=(N, N))
+    S = sp.csr_matrix((s_csr[2].astype(f8), s_csr[1], s_csr[0]), shape=(B, N))
+    msg = X.astype(f8) @ w.W_n2l.astype(f8)
+    h = np.maximum(msg, 0)
+    hs = [h]
+    for _ in range(L):
+        h = np.maximum((A @ h) @ w.W_conv.astype(f8) + msg, 0)
+        hs.append(h)
+    pool = S @ h
+    hidden = np.maximum(pool @ w.W_h1.astype(f8), 0)
+    logits = hidden @ w.W_h2.astype(f8)
+    e = np.exp(logits - logits.max(axis=1, keepdims=True))
+    return dict(msg=msg, h=np.stack(hs), pool=pool, hidden=hidden, logits=logits, probs=e / e.sum(axis=1, keepdims=True))
 
 
 @pytest.fixture(scope="session")

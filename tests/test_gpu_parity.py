@@ -1,7 +1,9 @@
 """Parity of the HIP path (through the C ABI) with the CPU oracle on identical seeded inputs.
 
 Bit-exact for integer / index outputs and for single-rounding element-wise ops;
-PARITY_TOL = 1e-4 (see conftest.max_rel for the floor) for fp32 sums.
+PARITY_TOL = 1e-4 under conftest.max_rel (floors measured per tensor kind) for fp32 sums; where two
+fp32 summation orders legitimately differ by more, a float64 model of the same computation decides
+(conftest.assert_parity).
 """
 import json
 import os
@@ -9,7 +11,7 @@ import os
 import numpy as np
 import pytest
 
-from conftest import PARITY_TOL, max_rel
+from conftest import FLOOR_POOL, FLOOR_PROBS_ABS, PARITY_TOL, Lazy, assert_parity, forward_float64, max_rel
 from graphnn_amd import batching, synth
 
 pytestmark = pytest.mark.gpu
@@ -42,6 +44,65 @@ def _random_csr(rng, m, k, nnz, unit=False, sort_cols=False):
     return rp, ci, v
 
 
+# float64 models of the kernels: assert_parity consults them only when a device result misses the oracle
+# (both are then fp32 evaluations in different summation orders, and float64 tells which one is off)
+def _csr64(rp, ci, v, m, k):
+    import scipy.sparse as sp
+    return sp.csr_matrix((np.asarray(v, np.float64), ci, rp), shape=(m, k))
+
+
+def _spmm_want(oracle, rp, ci, v, B, m, alpha=1.0, beta=0.0, C=None):
+    want = oracle.spmm(rp, ci, v, B, m, alpha=alpha, beta=beta, C=C)
+    def model():
+        y = alpha * (_csr64(rp, ci, v, m, B.shape[0]) @ B.astype(np.float64))
+        return y if C is None else y + beta * C.astype(np.float64)
+    return want, Lazy(model)
+
+
+def _gemm_want(oracle, A, B, ta=False, tb=False, alpha=1.0, beta=0.0, C=None):
+    want = oracle.gemm(A, B, ta, tb, alpha=alpha, beta=beta, C=C)
+    def model():
+        a64, b64 = A.astype(np.float64), B.astype(np.float64)
+        y = alpha * ((a64.T if ta else a64) @ (b64.T if tb else b64))
+        return y if C is None else y + beta * C.astype(np.float64)
+    return want, Lazy(model)
+
+
+def _level_want(oracle, rp, ci, v, h_in, W, msg=None, bias=None):
+    want = oracle.level(rp, ci, v, h_in, W, msg, bias)
+    def model():
+        N = h_in.shape[0]
+        z = (_csr64(rp, ci, v, N, N) @ h_in.astype(np.float64)) @ W.astype(np.float64)
+        if bias is not None:
+            z = z + bias.astype(np.float64)
+        if msg is not None:
+            z = z + msg.astype(np.float64)
+        return np.maximum(z, 0)
+    return want, Lazy(model)
+
+
+def _forward_want(oracle, a, s, X, w, L, lab=None):
+    """the oracle's forward; want["_f64"] is the lazily computed float64 model of the same network"""
+    want = oracle.forward(a, s, X, w, L, lab)
+    want["_f64"] = Lazy(lambda: forward_float64(a, s, X, w, L))
+    return want
+
+
+def _assert_forward_parity(got, want, L, tag="", keys=("msg", "h_final", "pool", "hidden", "logits", "probs")):
+    """got: name -> device array.  Floors as measured for each tensor (conftest): pooled features at 1e-4 of
+    their scale, probabilities at the fixed 1e-6, the rest at the default; a miss is settled by float64."""
+    f64 = want.get("_f64")
+    for key in keys:
+        ref = want["h"][L] if key == "h_final" else want[key]
+        ref64 = None if f64 is None else (f64["h"][L] if key == "h_final" else f64[key])
+        kw = {}
+        if key == "pool":
+            kw["floor_frac"] = FLOOR_POOL
+        elif key == "probs":
+            kw["floor"] = FLOOR_PROBS_ABS
+        assert_parity("%s%s" % (key, tag), got[key], ref, ref64, **kw)
+
+
 # ------------------------------------------------------------------ SpMM
 def test_spmm_known_answer(gpu, oracle):
     from graphnn_amd import ops
@@ -60,12 +121,12 @@ def test_spmm_widths_random_values(gpu, oracle, n):
     csr = _random_csr(rng, m, k, 4000)
     B = rng.standard_normal((k, n)).astype(np.float32)
     C0 = rng.standard_normal((m, n)).astype(np.float32)
-    want = oracle.spmm(*csr, B, m)
+    want, w64 = _spmm_want(oracle, *csr, B, m)
     got = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m))
-    assert max_rel(got, want) < PARITY_TOL
-    want2 = oracle.spmm(*csr, B, m, alpha=0.5, beta=-2.0, C=C0)
+    assert_parity("spmm", got, want, w64)
+    want2, w64b = _spmm_want(oracle, *csr, B, m, alpha=0.5, beta=-2.0, C=C0)
     got2 = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m, alpha=0.5, beta=-2.0, out=_t(C0, gpu)))
-    assert max_rel(got2, want2) < PARITY_TOL
+    assert_parity("spmm", got2, want2, w64b)
 
 
 @pytest.mark.parametrize("n", [2, 64, 128, 256])
@@ -119,9 +180,9 @@ def test_spmm_long_rows(gpu, oracle, n):
     ci = rng.integers(0, k, nnz).astype(np.int32)
     v = rng.standard_normal(nnz).astype(np.float32)
     B = rng.standard_normal((k, n)).astype(np.float32)
-    want = oracle.spmm(rp, ci, v, B, m)
+    want, w64 = _spmm_want(oracle, rp, ci, v, B, m)
     got = _n(ops.spmm(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(B, gpu), m))
-    assert max_rel(got, want) < PARITY_TOL
+    assert_parity("spmm", got, want, w64)
     # twice the same input: identical bits (no atomics, fixed combination order)
     got_again = _n(ops.spmm(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(B, gpu), m))
     assert np.array_equal(got, got_again)
@@ -144,9 +205,9 @@ def test_gemm_all_transposes(gpu, oracle, shape):
             B = rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32)
             C0 = rng.standard_normal((m, n)).astype(np.float32)
             got = _n(ops.gemm(_t(A, gpu), _t(B, gpu), ta, tb))
-            assert max_rel(got, oracle.gemm(A, B, ta, tb)) < PARITY_TOL, (ta, tb)
+            assert_parity("gemm %d%d" % (ta, tb), got, *_gemm_want(oracle, A, B, ta, tb))
             got2 = _n(ops.gemm(_t(A, gpu), _t(B, gpu), ta, tb, alpha=1.5, beta=-0.5, out=_t(C0, gpu)))
-            assert max_rel(got2, oracle.gemm(A, B, ta, tb, alpha=1.5, beta=-0.5, C=C0)) < PARITY_TOL, (ta, tb)
+            assert_parity("gemm %d%d" % (ta, tb), got2, *_gemm_want(oracle, A, B, ta, tb, alpha=1.5, beta=-0.5, C=C0))
 
 
 def test_gemm_reference_test_shape(gpu, oracle):
@@ -376,10 +437,10 @@ def test_level_stage(gpu, oracle, C, with_msg, with_bias):
     h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
     msg = rng.standard_normal((N, C)).astype(np.float32) if with_msg else None
     bias = rng.standard_normal(C).astype(np.float32) if with_bias else None
-    want = oracle.level(*a, h_in, w.W_conv, msg, bias)
+    want, w64 = _level_want(oracle, *a, h_in, w.W_conv, msg, bias)
     got = _n(ops.s2v_level(*_csr_t(a, gpu), _t(h_in, gpu), _t(w.W_conv, gpu),
                            _t(msg, gpu) if with_msg else None, _t(bias, gpu) if with_bias else None))
-    assert max_rel(got, want) < PARITY_TOL
+    assert_parity("level", got, want, w64)
     assert np.all(got >= 0)
 
 
@@ -400,14 +461,14 @@ def test_level_stage_row_counts_around_every_threshold(gpu, oracle, C):
         W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
         msg = rng.standard_normal((N, C)).astype(np.float32)
         bias = rng.standard_normal(C).astype(np.float32)
-        want = oracle.level(rp, ci, v, h_in, W, msg, bias)
+        want, w64 = _level_want(oracle, rp, ci, v, h_in, W, msg, bias)
         if nnz:
             ci_d, v_d = _t(ci, gpu), _t(v, gpu)
         else:
             import torch
             ci_d = torch.zeros(1, dtype=torch.int32, device=gpu)[:0]; v_d = torch.zeros(1, dtype=torch.float32, device=gpu)[:0]
         got = _n(ops.s2v_level(_t(rp, gpu), ci_d, v_d, _t(h_in, gpu), _t(W, gpu), _t(msg, gpu), _t(bias, gpu)))
-        assert max_rel(got, want) < PARITY_TOL, N
+        assert_parity("level", got, want, w64)
 
 
 def test_level_stage_hub_rows_and_weights(gpu, oracle):
@@ -423,9 +484,9 @@ def test_level_stage_hub_rows_and_weights(gpu, oracle):
     h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
     W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
     msg = rng.standard_normal((N, C)).astype(np.float32)
-    want = oracle.level(rp, ci, v, h_in, W, msg, None)
+    want, w64 = _level_want(oracle, rp, ci, v, h_in, W, msg, None)
     got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu)))
-    assert max_rel(got, want) < PARITY_TOL
+    assert_parity("level", got, want, w64)
 
 
 @pytest.mark.parametrize("C", [16, 32, 64])
@@ -446,9 +507,9 @@ def test_level_every_row_length_up_to_70(gpu, oracle, C, N):
     W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
     msg = rng.standard_normal((N, C)).astype(np.float32)
     bias = rng.standard_normal(C).astype(np.float32)
-    want = oracle.level(rp, ci, v, h_in, W, msg, bias)
+    want, w64 = _level_want(oracle, rp, ci, v, h_in, W, msg, bias)
     got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu), _t(bias, gpu)))
-    assert max_rel(got, want) < PARITY_TOL
+    assert_parity("level", got, want, w64)
 
 
 def test_wide_level_on_a_large_dense_skewed_graph(gpu, oracle):
@@ -467,9 +528,9 @@ def test_wide_level_on_a_large_dense_skewed_graph(gpu, oracle):
     h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
     W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
     msg = rng.standard_normal((N, C)).astype(np.float32)
-    want = oracle.level(rp, ci, v, h_in, W, msg, None)
+    want, w64 = _level_want(oracle, rp, ci, v, h_in, W, msg, None)
     got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu)))
-    assert max_rel(got, want) < PARITY_TOL
+    assert_parity("level", got, want, w64)
 
 
 @pytest.mark.parametrize("C", [128, 256])
@@ -490,11 +551,11 @@ def test_wide_level_fewer_entries_than_one_index_batch(gpu, oracle, C, nnz):
     h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
     W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
     msg = rng.standard_normal((N, C)).astype(np.float32)
-    want = oracle.level(rp, ci, v, h_in, W, msg, None)
+    want, w64 = _level_want(oracle, rp, ci, v, h_in, W, msg, None)
     ci_d = _t(ci, gpu) if nnz else torch.zeros(1, dtype=torch.int32, device=gpu)[:0]
     v_d = _t(v, gpu) if nnz else torch.zeros(1, dtype=torch.float32, device=gpu)[:0]
     got = _n(ops.s2v_level(_t(rp, gpu), ci_d, v_d, _t(h_in, gpu), _t(W, gpu), _t(msg, gpu)))
-    assert max_rel(got, want) < PARITY_TOL
+    assert_parity("level", got, want, w64)
 
 
 @pytest.mark.parametrize("C", [128, 256])
@@ -513,9 +574,9 @@ def test_wide_level_ragged_rows_and_weights(gpu, oracle, C, N):
     h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
     W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
     msg = rng.standard_normal((N, C)).astype(np.float32)
-    want = oracle.level(rp, ci, v, h_in, W, msg, None)
+    want, w64 = _level_want(oracle, rp, ci, v, h_in, W, msg, None)
     got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu)))
-    assert max_rel(got, want) < PARITY_TOL
+    assert_parity("level", got, want, w64)
 
 
 @pytest.mark.parametrize("C,H,Q", [(64, 32, 2), (16, 8, 3), (32, 100, 70), (48, 16, 2), (128, 64, 5)])
@@ -574,7 +635,7 @@ def _forward_case(gpu, oracle, config_id, B=None):
     s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
     X = batch.one_hot()
     lab = batch.label_csr()
-    want = oracle.forward(a, s, X, w, cfg["L"], lab)
+    want = _forward_want(oracle, a, s, X, w, cfg["L"], lab)
     bufs = ops.s2v_forward(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
                            _t(w.W_h1, gpu), _t(w.W_h2, gpu), cfg["L"])
     got = dict(msg=_n(bufs.msg), h_final=_n(bufs.h_final), pool=_n(bufs.pool), hidden=_n(bufs.hidden),
@@ -586,10 +647,7 @@ def _forward_case(gpu, oracle, config_id, B=None):
 def test_forward_matches_reference_path(gpu, oracle, config_id):
     from graphnn_amd import ops
     batch, cfg, a, s, X, w, lab, want, got, bufs = _forward_case(gpu, oracle, config_id)
-    assert max_rel(got["msg"], want["msg"]) < PARITY_TOL
-    assert max_rel(got["h_final"], want["h"][cfg["L"]]) < PARITY_TOL
-    for key in ("pool", "hidden", "logits", "probs"):
-        assert max_rel(got[key], want[key]) < PARITY_TOL, key
+    _assert_forward_parity(got, want, cfg["L"])
     # argmax predictions bit-exact with the reference path
     assert np.array_equal(got["pred"], want["pred"])
     # loss / accuracy tail of the graph, operator by operator on the device
@@ -620,11 +678,11 @@ def test_forward_graph_counts_around_the_readout_thresholds(gpu, oracle, C, H, Q
         a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
         s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
         X = batch.one_hot()
-        want = oracle.forward(a, s, X, w, L, None)
+        want = _forward_want(oracle, a, s, X, w, L)
         bufs = ops.s2v_forward(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
                                _t(w.W_h1, gpu), _t(w.W_h2, gpu), L)
-        for key in ("pool", "hidden", "logits", "probs"):
-            assert max_rel(_n(getattr(bufs, key)), want[key]) < PARITY_TOL, (B, key)
+        _assert_forward_parity({k: _n(getattr(bufs, k)) for k in ("pool", "hidden", "logits", "probs")}, want, L,
+                               tag=" B=%d" % B, keys=("pool", "hidden", "logits", "probs"))
         assert np.array_equal(_n(bufs.pred), want["pred"]), B
 
 
@@ -737,7 +795,7 @@ def _batched_case(gpu, oracle, batch, w, L):
     a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
     s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
     X = batch.one_hot()
-    want = oracle.forward(a, s, X, w, L, batch.label_csr())
+    want = _forward_want(oracle, a, s, X, w, L, batch.label_csr())
     bufs = ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
                                    _t(w.W_h1, gpu), _t(w.W_h2, gpu), L, int(batch.graph_sizes.max()))
     return want, bufs
@@ -745,10 +803,7 @@ def _batched_case(gpu, oracle, batch, w, L):
 
 def _assert_batched_matches(want, bufs, L):
     assert int(_n(bufs.status)[0]) == 0
-    assert max_rel(_n(bufs.msg), want["msg"]) < PARITY_TOL
-    assert max_rel(_n(bufs.h_final), want["h"][L]) < PARITY_TOL
-    for key in ("pool", "hidden", "logits", "probs"):
-        assert max_rel(_n(getattr(bufs, key)), want[key]) < PARITY_TOL, key
+    _assert_forward_parity({k: _n(getattr(bufs, k)) for k in ("msg", "h_final", "pool", "hidden", "logits", "probs")}, want, L)
     assert np.array_equal(_n(bufs.pred), want["pred"])
 
 
@@ -809,7 +864,7 @@ def test_batched_forward_large_and_dense_graphs(gpu, oracle):
     s = (s[0], s[1], (rng.random(N) * 0.5).astype(np.float32))                    # weighted pooling
     X = rng.standard_normal((N, K)).astype(np.float32)
     w = synth.make_weights(synth.Stream(5), K, C, H, Q)
-    want = oracle.forward(a, s, X, w, L, None)
+    want = _forward_want(oracle, a, s, X, w, L)
     bufs = ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
                                    _t(w.W_h1, gpu), _t(w.W_h2, gpu), L, 200)
     _assert_batched_matches(want, bufs, L)
@@ -830,7 +885,7 @@ def test_batched_forward_dense_features_past_the_staging_registers(gpu, oracle):
     a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
     s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
     X = rng.standard_normal((batch.num_nodes, K)).astype(np.float32)
-    want = oracle.forward(a, s, X, w, L, None)
+    want = _forward_want(oracle, a, s, X, w, L)
     bufs = ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
                                    _t(w.W_h1, gpu), _t(w.W_h2, gpu), L, int(batch.graph_sizes.max()))
     _assert_batched_matches(want, bufs, L)
@@ -936,8 +991,8 @@ def test_spmm_long_rows_around_the_row_count_threshold(gpu, oracle, n):
         csr = _hub_matrix(rng, m, k, [(0, 5000), (9, 65), (10, 2048), (11, 2049), (m // 2, 64), (m - 1, 3000)])
         B = rng.standard_normal((k, n)).astype(np.float32)
         got = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m))
-        want = oracle.spmm(*csr, B, m)
-        assert max_rel(got, want) < PARITY_TOL, m
+        want, w64 = _spmm_want(oracle, *csr, B, m)
+        assert_parity("spmm m=%d" % m, got, want, w64)
 
 
 @pytest.mark.parametrize("n", [64, 128, 7, 36, 300])
@@ -951,10 +1006,10 @@ def test_spmm_hub_rows_balanced_pass(gpu, oracle, n):
     B = rng.standard_normal((k, n)).astype(np.float32)
     C0 = rng.standard_normal((m, n)).astype(np.float32)
     got = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m))
-    want = oracle.spmm(*csr, B, m)
-    assert max_rel(got, want) < PARITY_TOL
+    want, w64 = _spmm_want(oracle, *csr, B, m)
+    assert_parity("spmm", got, want, w64)
     got2 = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m, alpha=-0.5, beta=1.5, out=_t(C0, gpu)))
-    assert max_rel(got2, oracle.spmm(*csr, B, m, alpha=-0.5, beta=1.5, C=C0)) < PARITY_TOL
+    assert_parity("spmm", got2, *_spmm_want(oracle, *csr, B, m, alpha=-0.5, beta=1.5, C=C0))
     # deterministic: the same bits on a second run
     assert np.array_equal(got, _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m)))
 
@@ -968,9 +1023,9 @@ def test_level_hub_rows_balanced_pass(gpu, oracle, C):
     h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
     W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
     msg = rng.standard_normal((N, C)).astype(np.float32)
-    want = oracle.level(*csr, h_in, W, msg, None)
+    want, w64 = _level_want(oracle, *csr, h_in, W, msg, None)
     got = _n(ops.s2v_level(*_csr_t(csr, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu)))
-    assert max_rel(got, want) < PARITY_TOL
+    assert_parity("level", got, want, w64)
     assert np.array_equal(got, _n(ops.s2v_level(*_csr_t(csr, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu))))
 
 
@@ -989,16 +1044,13 @@ def test_forward_first_level_reads_msg_with_long_rows(gpu, oracle, C, L):
     X += (rng.standard_normal(X.shape) * 0.05).astype(np.float32)              # msg with both signs everywhere
     w = synth.make_weights(synth.Stream(700 + C), K, C, H, Q)
     w.W_conv = (w.W_conv * 0.02).astype(np.float32)                              # rows of thousands of entries: keep the levels bounded
-    want = oracle.forward(a, s, X, w, L)
+    want = _forward_want(oracle, a, s, X, w, L)
     bufs = ops.s2v_forward(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
                            _t(w.W_h1, gpu), _t(w.W_h2, gpu), L)
-    assert max_rel(_n(bufs.msg), want["msg"]) < PARITY_TOL
     # the reference path adds a row of thousands of entries sequentially in fp32 and is itself about 1e-4 from
-    # the exact sum there, so the embeddings are held to 3e-4
-    got_h = _n(bufs.h_final)
-    assert max_rel(got_h, want["h"][L]) < 3e-4
-    assert max_rel(_n(bufs.pool), want["pool"]) < 3e-4
-    assert max_rel(_n(bufs.logits), want["logits"]) < 3e-4
+    # the exact sum there: where the device misses the oracle by more than 1e-4, the float64 model decides
+    # (the device must be no further from it than the oracle is)
+    _assert_forward_parity({k: _n(getattr(bufs, k)) for k in ("msg", "h_final", "pool", "hidden", "logits", "probs")}, want, L)
 
 
 def test_rmat_forward_with_jagged_softmax(gpu, oracle):
@@ -1041,7 +1093,7 @@ def test_rmat_forward_with_jagged_softmax(gpu, oracle):
         exact = np.maximum((A64 @ h.astype(np.float64)) @ W64 + msg64, 0).astype(np.float32)
         got = _n(ops.s2v_level(*a_d, _t(h, gpu), Wc_d, msg_d))
         assert max_rel(got, exact) < PARITY_TOL
-        assert max_rel(got[short], h_next[short]) < PARITY_TOL
+        assert_parity("level, short rows", got[short], h_next[short], exact[short])
         h_d = ops.s2v_level(*a_d, h_d, Wc_d, msg_d)                                                # chained
         h = h_next
         h64 = np.maximum((A64 @ h64) @ W64 + msg64, 0)
@@ -1077,9 +1129,9 @@ def test_level_dense_graph_two_launch_route(gpu, oracle, C):
     W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
     msg = rng.standard_normal((N, C)).astype(np.float32)
     bias = rng.standard_normal(C).astype(np.float32)
-    want = oracle.level(rp, ci, v, h_in, W, msg, bias)
+    want, w64 = _level_want(oracle, rp, ci, v, h_in, W, msg, bias)
     got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu), _t(bias, gpu)))
-    assert max_rel(got, want) < PARITY_TOL
+    assert_parity("level", got, want, w64)
 
 
 def test_edge_embedding_step_with_edge_based_operands(gpu, oracle):

@@ -405,6 +405,41 @@ def test_forward_against_float64_dense_model(oracle):
     assert max_rel(lvl, want_lvl) < 1e-4
 
 
+def _min_floor(got, ref64, tol=1e-4):
+    """smallest floor (as a fraction of max|ref|) under which max_rel(got, ref64) stays below tol"""
+    g = np.asarray(got, np.float64)
+    d = np.abs(g - ref64)
+    den = np.maximum(np.abs(g), np.abs(ref64))
+    bad = d > tol * den
+    return 0.0 if not bad.any() else float((d[bad] / tol).max() / np.abs(ref64).max())
+
+
+@pytest.mark.parametrize("config_id,B", [(1, 50), (1, 200), (2, 256), (2, 1000)])
+def test_parity_floors_are_the_smallest_the_oracle_itself_survives(oracle, config_id, B):
+    """The floors of conftest.max_rel are measured, not picked: against a float64 model of the same network
+    the oracle (a correct fp32 evaluation) needs a floor of about 1e-3 of the tensor's scale on embeddings,
+    hidden layer and logits to stay within 1e-4, 3e-5 on the pooled features and none on the probabilities.
+    The floors in use must cover that with at most a factor of four to spare."""
+    from conftest import FLOOR_DEFAULT, FLOOR_POOL, FLOOR_PROBS_ABS, forward_float64
+    batch, w, cfg = synth.make_config(config_id, B=B)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    got = oracle.forward(a, s, X, w, cfg["L"], batch.label_csr())
+    want = forward_float64(a, s, X, w, cfg["L"])
+    need = {k: _min_floor(got[k][1:] if k == "h" else got[k], want[k][1:] if k == "h" else want[k])
+            for k in ("h", "pool", "hidden", "logits", "probs")}
+    print("configuration %d, %d graphs: smallest floor / max|ref| " % (config_id, B)
+          + "  ".join("%s %.2e" % kv for kv in need.items()))
+    assert max(need["h"], need["hidden"], need["logits"]) <= FLOOR_DEFAULT
+    assert need["pool"] <= FLOOR_POOL
+    assert max_rel(got["probs"], want["probs"], floor=FLOOR_PROBS_ABS) < 1e-4
+    if config_id == 2:
+        # ... and are not generous: a floor four times smaller already fails the oracle itself
+        assert max(need["h"], need["hidden"], need["logits"]) > FLOOR_DEFAULT / 4
+        assert need["pool"] > FLOOR_POOL / 10
+
+
 def test_edge_based_operands_against_dense_definitions(oracle):
     """Edge2Node / Node2Edge / Edge2Edge (src/nn/msg_pass.cpp:72-152) against matrices written straight
     from their definitions, and the numpy builders against the oracle"""
