@@ -8,6 +8,8 @@
 #include <stdint.h>
 #include <stddef.h>
 
+#include <mutex>
+
 #include "gnnhip.h"
 
 namespace gnnhip {
@@ -42,6 +44,23 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
             return ::gnnhip::set_error(GNNHIP_EHIP, "launch of %s failed: %s", name, \
                                        hipGetErrorString(e__));                     \
     } while (0)
+
+// Kernels that use more than 64 KB of dynamic LDS have to be allowed to, once per kernel instantiation.
+// A function-local `static LdsLimit limit;` per instantiation keeps the largest size granted so far;
+// raise() is safe to call from several host threads (the runtime serves one device per process).
+struct LdsLimit {
+    std::mutex mu;
+    size_t granted = 0;
+    hipError_t raise(const void* kernel, size_t bytes)
+    {
+        if (bytes <= 64 * 1024) return hipSuccess;
+        std::lock_guard<std::mutex> lock(mu);
+        if (bytes <= granted) return hipSuccess;
+        hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e == hipSuccess) granted = bytes;
+        return e;
+    }
+};
 
 inline unsigned ceil_div_u(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
 

@@ -515,12 +515,10 @@ int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
     const int ecap = GraphLds::edge_cap(n16max, C, K, H, Q, kBlock);
     if (ecap < 0) return GNNHIP_EUNSUPPORTED;
     const size_t smem = sizeof(float) * (GraphLds::fixed_floats(n16max, C, K, H, Q, kBlock) + 2 * (size_t)ecap);
-    static size_t configured = 0;           // largest dynamic LDS size this kernel has been allowed so far
-    if (smem > 64 * 1024 && smem > configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) { (void)hipGetLastError(); return GNNHIP_EUNSUPPORTED; }
-        configured = smem;
+    static LdsLimit lds_limit;              // largest dynamic LDS size this kernel instantiation has been allowed so far
+    if (lds_limit.raise(reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES>), smem) != hipSuccess) {
+        (void)hipGetLastError();
+        return GNNHIP_EUNSUPPORTED;
     }
     const int grid = B < kNumCU * 4 ? B : kNumCU * 4;
     const unsigned k_magic = K >= 2 ? (unsigned)((0x100000000ull + (unsigned)K - 1) / (unsigned)K) : 0u;   // ceil(2^32 / K)

@@ -19,7 +19,8 @@
 //
 // The consumer reads agg[row_slot[row]] for a row whose length exceeds the
 // threshold.  Every sum is taken in an order fixed by the matrix structure, so the
-// result does not depend on scheduling; there are no atomics.
+// result does not depend on scheduling: no value is accumulated with atomics.  The one
+// atomic counter per hub (hub_done) only elects the wavefront that adds the chunks' sums.
 #include "gnnhip_internal.h"
 
 namespace gnnhip {

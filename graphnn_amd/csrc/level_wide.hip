@@ -87,6 +87,20 @@ __device__ __forceinline__ void batch_load(Batch& b, const int* p)
 {
     asm volatile("s_load_dwordx4 %0, %2, 0x0\n\ts_load_dwordx2 %1, %2, 0x10" : "+s"(b.lo), "+s"(b.hi) : "s"(p));
 }
+// The first n < kInFlight entries of an array that holds no more than n, zeros behind them: one scalar load
+// per entry, each under its own (uniform) condition, and the wait right here.
+__device__ __forceinline__ void batch_load_short(Batch& b, const int* p, int n)
+{
+    int t0 = 0, t1 = 0, t2 = 0, t3 = 0, t4 = 0;
+    if (n > 0) asm volatile("s_load_dword %0, %1, 0x0" : "+s"(t0) : "s"(p));
+    if (n > 1) asm volatile("s_load_dword %0, %1, 0x4" : "+s"(t1) : "s"(p));
+    if (n > 2) asm volatile("s_load_dword %0, %1, 0x8" : "+s"(t2) : "s"(p));
+    if (n > 3) asm volatile("s_load_dword %0, %1, 0xc" : "+s"(t3) : "s"(p));
+    if (n > 4) asm volatile("s_load_dword %0, %1, 0x10" : "+s"(t4) : "s"(p));
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(t0), "+s"(t1), "+s"(t2), "+s"(t3), "+s"(t4));
+    b.lo.x = t0; b.lo.y = t1; b.lo.z = t2; b.lo.w = t3;
+    b.hi.x = t4; b.hi.y = 0;
+}
 __device__ __forceinline__ void batch_wait(Batch& b)
 {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(b.lo), "+s"(b.hi));
@@ -169,10 +183,15 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     const int* val_bits = reinterpret_cast<const int*>(val);
     // entries [s, s + kInFlight) of the CSR arrays.  What lies past the end of the wavefront's rows is
     // loaded but never added, so the batch is read as it lies.  Only a batch that would run past the end
-    // of the arrays starts earlier; batch_ready() then shifts it into place.  The arrays hold at least
-    // kInFlight entries (the host pads shorter ones).
+    // of the arrays starts earlier; batch_ready() then shifts it into place.  The entry count that bounds
+    // these reads is the matrix's own (row_ptr[N], read here), never a count passed by the host.  A matrix
+    // with fewer entries than one batch is read entry by entry, with zeros behind the last one.
     const int nnz = row_ptr[N];
     auto load_batch = [&](const int* arr, int s, Batch& b) {
+        if (nnz < kInFlight) {
+            batch_load_short(b, arr, nnz);
+            return s;
+        }
         const int base = max(min(s, nnz - kInFlight), 0);
         batch_load(b, arr + base);
         return s - base;                         // by how many entries the batch has to be shifted
@@ -411,12 +430,8 @@ int launch_level_wide_t(int N, const int* row_ptr, const int* col_idx, const flo
     const long long per = (ntiles + slots - 1) / slots;              // contiguous run of tiles per workgroup
     const long long blocks = (ntiles + per - 1) / per;
     const size_t smem = sizeof(float) * (2 * kTileRows * (C + 4) + C);
-    static bool attr_set = false;                                    // more than 64 KB of LDS has to be asked for
-    if (!attr_set) {
-        GNNHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&s2v_level_wide_kernel<C, WAVES, RELU_IN, TR>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_set = true;
-    }
+    static LdsLimit lds_limit;                                       // one per kernel instantiation
+    GNNHIP_HIP(lds_limit.raise(reinterpret_cast<const void*>(&s2v_level_wide_kernel<C, WAVES, RELU_IN, TR>), smem));
     hipLaunchKernelGGL((s2v_level_wide_kernel<C, WAVES, RELU_IN, TR>), dim3((unsigned)blocks), dim3(WAVES * kWave), smem, s,
                        N, (int)per, row_ptr, col_idx, val, h_in, W, msg, bias, h_out);
     GNNHIP_LAUNCH_CHECK("s2v_level_wide");
@@ -447,21 +462,7 @@ int level_wide_dispatch(int N, int C, long long nnz, const int* row_ptr, const i
                         const float* h_in, const float* W, const float* msg, const float* bias, float* h_out, bool relu_in,
                         hipStream_t s)
 {
-    if (nnz < kInFlight) {
-        // the kernel reads whole batches of kInFlight entries: arrays shorter than one batch are copied into
-        // zero-padded scratch
-        void* pad = nullptr;
-        if (int rc = stream_scratch(s, 64, &pad)) return rc;
-        if (int rc = gnnhip_memset0(pad, 64, s)) return rc;
-        int* col_pad = static_cast<int*>(pad);
-        float* val_pad = reinterpret_cast<float*>(col_pad + 8);
-        if (nnz > 0) {
-            if (int rc = gnnhip_memcpy_d2d(col_pad, col_idx, sizeof(int) * (size_t)nnz, s)) return rc;
-            if (int rc = gnnhip_memcpy_d2d(val_pad, val, sizeof(float) * (size_t)nnz, s)) return rc;
-        }
-        col_idx = col_pad;
-        val = val_pad;
-    }
+    (void)nnz;                                   // the kernel bounds its index reads with row_ptr[N]
     switch (C) {
     case 128:
         return relu_in ? launch_level_wide<128, 8, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s)

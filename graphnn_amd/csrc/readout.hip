@@ -136,14 +136,8 @@ int launch_readout_wave(int B, int H, int Q, const int* s_row_ptr, const int* s_
     const size_t smem = sizeof(float) * ((size_t)C * H + (size_t)H * Q + (size_t)kWavesPerBlock * (RPR * C + C + H + Q));
     if (smem > (size_t)kMaxLds) return GNNHIP_EUNSUPPORTED;
     auto kernel = s2v_readout_wave_kernel<C>;
-    if (smem > 64 * 1024) {
-        static bool raised = false;          // per instantiation; the attribute is a property of the function
-        if (!raised) {
-            GNNHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           kMaxLds));
-            raised = true;
-        }
-    }
+    static LdsLimit lds_limit;               // one per kernel instantiation
+    GNNHIP_HIP(lds_limit.raise(reinterpret_cast<const void*>(kernel), smem > 64 * 1024 ? (size_t)kMaxLds : smem));
     const long long blocks_needed = ((long long)B + kWavesPerBlock - 1) / kWavesPerBlock;
     const long long per_cu = smem > 0 ? (long long)(160 * 1024) / (long long)smem : 8;
     long long cap = (long long)kNumCU * (per_cu < 1 ? 1 : (per_cu > 8 ? 8 : per_cu));

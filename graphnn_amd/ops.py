@@ -101,7 +101,9 @@ def s2v_input(X, W_n2l):
     return msg, h0
 
 
-def s2v_level(row_ptr, col_idx, val, h_in, W, msg=None, bias=None, out=None):
+def s2v_level(row_ptr, col_idx, val, h_in, W, msg=None, bias=None, out=None, nnz_hint=None):
+    """nnz_hint: the host-side entry count handed to the library (default: the arrays' length); it only
+    sizes scratch, so any value from 0 up must give the same result."""
     N, C = h_in.shape
     _check_csr(row_ptr, col_idx, val, N, "A")
     if tuple(W.shape) != (C, C):
@@ -112,7 +114,8 @@ def s2v_level(row_ptr, col_idx, val, h_in, W, msg=None, bias=None, out=None):
         raise ValueError("bias must have C entries")
     if out is None:
         out = torch.empty_like(h_in)
-    check(_lib().gnnhip_s2v_level_f32(N, C, int(col_idx.numel()), _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"), _f32(val, "val"),
+    nnz = int(col_idx.numel()) if nnz_hint is None else int(nnz_hint)
+    check(_lib().gnnhip_s2v_level_f32(N, C, nnz, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"), _f32(val, "val"),
                                       _f32(h_in, "h_in"), _f32(W, "W"), _f32(msg, "msg"), _f32(bias, "bias"),
                                       _f32(out, "out"), _stream()))
     return out

@@ -53,7 +53,10 @@ int gnnhip_shutdown(void);
 /* ---- pooled device memory: MemHolder<GPU>::MallocArr / Recycle / ForceDel
  *      (include/util/mem_holder.h:20-51, src/util/mem_holder.cpp:15-97).
  *      malloc takes the smallest parked block >= bytes or allocates; recycle
- *      parks the block for reuse; free returns it to the driver. */
+ *      parks the block for reuse; free returns it to the driver.
+ *      recycle knows nothing of streams (neither does MemHolder): the block may be handed out again at
+ *      once, so the caller must not recycle a block while work queued on a stream still uses it unless the
+ *      next user is ordered behind that work (same stream, or an event). */
 int gnnhip_malloc(void** device_ptr, size_t bytes);
 int gnnhip_recycle(void* device_ptr);
 int gnnhip_free(void* device_ptr);
@@ -77,7 +80,8 @@ int gnnhip_stream_sync(void* stream);
  *      DTensor<GPU>::MM(SpTensor, DTensor, Trans::N, Trans::N) + CSRMMKernel
  *      (src/tensor/gpu_dense_tensor.cu:227-239,257-270).  beta == 0 overwrites C.
  *      nnz is the host-side entry count of A (SparseData::nnz, include/tensor/t_data.h:123-165);
- *      it sizes the buffers of the balanced pass over high-degree rows.  A value smaller than
+ *      it sizes the buffers of the balanced pass over high-degree rows and nothing else: every read of
+ *      col_idx / val is bounded by the matrix's own row_ptr[m] on the device.  A value smaller than
  *      row_ptr[m] is safe (rows that do not fit are summed in place), a larger one wastes memory. */
 int gnnhip_spmm_csr_f32(int m, int k, int n, int nnz, float alpha, const int* row_ptr, const int* col_idx,
                         const float* val, const float* B, int ldb, float beta, float* C, int ldc,

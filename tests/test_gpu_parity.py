@@ -558,6 +558,31 @@ def test_wide_level_fewer_entries_than_one_index_batch(gpu, oracle, C, nnz):
     assert_parity("level", got, want, w64)
 
 
+@pytest.mark.parametrize("C", [64, 128, 256])
+@pytest.mark.parametrize("hint", [0, 5, 6, 1000])
+def test_level_entry_count_hint_does_not_bound_the_reads(gpu, oracle, C, hint):
+    """the nnz argument only sizes scratch: a 77-row matrix with 10 entries gives the same bits whether the
+    host states 0, 5, 6 or 1,000 entries (the kernels bound their index reads with row_ptr[N] on the device;
+    the hidden-128/256 kernel reads indices six at a time and once took the host's count for it)"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(900 + C)
+    N, nnz = 77, 10
+    lens = np.zeros(N, np.int64)
+    for i in range(nnz): lens[[3, 40, 76][i % 3]] += 1
+    rp = np.zeros(N + 1, np.int32); np.cumsum(lens, out=rp[1:])
+    ci = rng.integers(0, N, nnz).astype(np.int32)
+    v = (rng.random(nnz) + 0.5).astype(np.float32)
+    h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
+    W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
+    msg = rng.standard_normal((N, C)).astype(np.float32)
+    want, w64 = _level_want(oracle, rp, ci, v, h_in, W, msg, None)
+    args = (_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu))
+    exact = _n(ops.s2v_level(*args))
+    got = _n(ops.s2v_level(*args, nnz_hint=hint))
+    assert np.array_equal(got, exact)
+    assert_parity("level", got, want, w64)
+
+
 @pytest.mark.parametrize("C", [128, 256])
 @pytest.mark.parametrize("N", [5_003, 10_007, 15_991, 64 * 300 + 37, 40_037, 70_001])
 def test_wide_level_ragged_rows_and_weights(gpu, oracle, C, N):
