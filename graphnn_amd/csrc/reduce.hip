@@ -122,6 +122,22 @@ __global__ __launch_bounds__(kBlock) void jagged_softmax_kernel(float* x, const 
     }
 }
 
+// ---- gradient of the jagged softmax: per segment z = <grad, out>, dst += (grad - z) * out
+//      (the CPU rule, src/nn/jagged_softmax.cpp:8-31; graphnn's GPU overload is an empty body)
+__global__ __launch_bounds__(kBlock) void jagged_softmax_deriv_kernel(float* __restrict__ dst, const float* __restrict__ out,
+                                                                      const float* __restrict__ grad, const int* __restrict__ off, int nseg)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    for (long long s = (long long)blockIdx.x * kWavesPerBlock + wave; s < nseg; s += (long long)gridDim.x * kWavesPerBlock) {
+        const int a = off[s], b = off[s + 1];
+        float z = 0.f;
+        for (int j = a + lane; j < b; j += kWave) z += grad[j] * out[j];
+        z = wave_sum(z);
+        for (int j = a + lane; j < b; j += kWave) dst[j] += (grad[j] - z) * out[j];
+    }
+}
+
 // ---- global reductions: stage 1 writes one partial per workgroup, stage 2 combines
 // them in index order, so the result does not depend on scheduling.
 template <bool IS_MAX>
@@ -304,6 +320,23 @@ int gnnhip_jagged_softmax_f32(float* x, const int* lens, int nseg, void* stream)
     GNNHIP_LAUNCH_CHECK("exclusive_scan");
     hipLaunchKernelGGL(jagged_softmax_kernel, dim3(wave_rows_grid(nseg)), dim3(kBlock), 0, s, x, static_cast<const int*>(off), nseg);
     GNNHIP_LAUNCH_CHECK("jagged_softmax");
+    return GNNHIP_OK;
+}
+
+int gnnhip_jagged_softmax_deriv_f32(float* dst, const float* out, const float* grad, const int* lens, int nseg, void* stream)
+{
+    GNNHIP_REQUIRE(nseg >= 0, "negative segment count");
+    if (nseg == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(dst && out && grad && lens, "null tensor in jagged_softmax_deriv");
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    void* off = nullptr;
+    if (int rc = stream_scratch(s, sizeof(int) * ((size_t)nseg + 1), &off)) return rc;
+    hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(kScanBlock), 0, s, lens, nseg, static_cast<int*>(off));
+    GNNHIP_LAUNCH_CHECK("exclusive_scan");
+    hipLaunchKernelGGL(jagged_softmax_deriv_kernel, dim3(wave_rows_grid(nseg)), dim3(kBlock), 0, s, dst, out, grad,
+                       static_cast<const int*>(off), nseg);
+    GNNHIP_LAUNCH_CHECK("jagged_softmax_deriv");
     return GNNHIP_OK;
 }
 

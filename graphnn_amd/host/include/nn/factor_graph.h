@@ -112,6 +112,7 @@ public:
     // switch the inference-time kernel fusion off (every factor then runs as written)
     void EnableFusion(bool on) { fusion_enabled = on; ++version; }
     // how the last FeedForward was executed: number of factor launches and of fused steps
+    std::vector< std::vector<std::string> > PlanSteps(std::vector<VarPtr> targets, std::map<std::string, void*> feed_dict, Phase phase);
     size_t LastPlanFactorCount() const;
     size_t LastPlanFusedCount() const;
 

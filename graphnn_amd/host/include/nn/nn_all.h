@@ -17,6 +17,9 @@
 #include "nn/in_top_k.h"
 #include "nn/type_cast.h"
 #include "nn/softmax.h"
+#include "nn/jagged_softmax.h"
+#include "nn/reduce.h"
+#include "nn/fully_connected.h"
 #include "nn/param_set.h"
 #include "nn/optimizer.h"
 

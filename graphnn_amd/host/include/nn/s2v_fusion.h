@@ -30,9 +30,24 @@ struct FusedStep
     bool fused;
     enum Tag { SINGLE, INPUT, LEVEL, FORWARD } tag = SINGLE;
     std::vector<size_t> vars;               // INPUT: X, W, msg, h0;  LEVEL: A, h_in, W, msg, h_out
+    bool bias_row = false;                  // LEVEL through FullyConnected: W may carry a bias row
 };
 constexpr size_t kOneLaunchMaxNodes = 20000;   // larger batches run the forward as separate kernels
 }  // namespace detail
+
+// The factor names of every step of the plan a FeedForward with these arguments would run, in
+// execution order (a folded step lists the factors it stands for).  Runs nothing.
+inline std::vector< std::vector<std::string> > FactorGraph::PlanSteps(std::vector<VarPtr> targets,
+                                                                      std::map<std::string, void*> feed_dict, Phase phase)
+{
+    Plan* plan = GetPlan(targets, feed_dict, phase);
+    std::vector< std::vector<std::string> > out;
+    for (auto& step : plan->steps) {
+        out.emplace_back();
+        for (size_t f : step->factors) out.back().push_back(factor_list[f]->name);
+    }
+    return out;
+}
 
 inline size_t FactorGraph::LastPlanFactorCount() const { return last_plan ? last_plan->steps.size() : 0; }
 inline size_t FactorGraph::LastPlanFusedCount() const { return last_plan ? last_plan->n_fused : 0; }
@@ -136,16 +151,26 @@ inline void FactorGraph::BuildFusedSteps(Plan& plan)
         return step;
     };
 
+    // A folded chain runs where its LAST factor stood in the order: only there are the operands of all
+    // of its factors ready (msg and W enter the level at its second and third factor, and their
+    // producers may sit anywhere before those, e.g. behind the sparse product when msg comes out of a
+    // deeper chain than h_in does).
+    std::vector< std::shared_ptr<detail::FusedStep> > emit_at(factor_list.size());
     const bool fold = fusion_enabled && plan.phase == Phase::TEST;
     for (size_t f1 : plan.order) {
-        if (taken[f1]) continue;
+        if (taken[f1]) {
+            if (emit_at[f1]) plan.steps.push_back(emit_at[f1]);
+            continue;
+        }
         bool done = false;
         if (fold && !strcmp(kind(f1), "matmul_nn") && factor_nodes[f1].in.size() == 2 && factor_nodes[f1].out.size() == 1) {
             const size_t a = factor_nodes[f1].in[0], b = factor_nodes[f1].in[1], p1 = factor_nodes[f1].out[0];
             size_t f2 = 0, f3 = 0, f4 = 0;
             // ---- level: sparse x dense, then dense x dense, then + msg, then ReLU
             if (gpu_sparse(a) && gpu_dense(b) && gpu_dense(p1) && sole_reader(p1, f2) && !taken[f2] &&
-                !strcmp(kind(f2), "matmul_nn") && factor_nodes[f2].in[0] == p1 && gpu_dense(factor_nodes[f2].in[1])) {
+                (!strcmp(kind(f2), "matmul_nn") || !strcmp(kind(f2), "fully_connected")) && factor_nodes[f2].in.size() == 2 &&
+                factor_nodes[f2].in[0] == p1 && gpu_dense(factor_nodes[f2].in[1])) {
+                const bool through_fc = !strcmp(kind(f2), "fully_connected");
                 const size_t w = factor_nodes[f2].in[1], p2 = factor_nodes[f2].out[0];
                 if (sole_reader(p2, f3) && !taken[f3] && !strcmp(kind(f3), "elewise_add2") && factor_nodes[f3].in.size() == 2) {
                     const size_t other = factor_nodes[f3].in[0] == p2 ? factor_nodes[f3].in[1] : factor_nodes[f3].in[0];
@@ -159,19 +184,24 @@ inline void FactorGraph::BuildFusedSteps(Plan& plan)
                         step->fused = true;
                         step->tag = detail::FusedStep::LEVEL;
                         step->vars = {a, b, w, other, factor_nodes[f4].out[0]};
-                        step->run = [A, H, W, M, O](Phase) {
-                            ASSERT(A->value.cols() == H->value.rows() && H->value.cols() == W->value.rows() &&
-                                   W->value.rows() == W->value.cols() && M->value.shape == H->value.shape &&
+                        step->bias_row = through_fc;
+                        step->run = [A, H, W, M, O, through_fc](Phase) {
+                            const size_t C = H->value.cols();
+                            // FullyConnected: rows [0, C) of the parameter are the weights, row C (if there) the bias
+                            const bool bias = through_fc && W->value.rows() == C + 1;
+                            ASSERT(A->value.cols() == H->value.rows() && W->value.cols() == C &&
+                                   (W->value.rows() == C || bias) && M->value.shape == H->value.shape &&
                                    A->value.rows() == H->value.rows(),
                                    "fused level: operand shapes do not chain");
                             O->value.Reshape(H->value.shape.dims);
-                            GNN_HIP(gnnhip_s2v_level_f32((int)H->value.rows(), (int)H->value.cols(), A->value.data->nnz, A->value.data->row_ptr,
+                            GNN_HIP(gnnhip_s2v_level_f32((int)H->value.rows(), (int)C, A->value.data->nnz, A->value.data->row_ptr,
                                                          A->value.data->col_idx, A->value.data->val, H->value.data->ptr,
-                                                         W->value.data->ptr, M->value.data->ptr, nullptr,
+                                                         W->value.data->ptr, M->value.data->ptr,
+                                                         bias ? W->value.data->ptr + C * C : nullptr,
                                                          O->value.data->ptr, GpuHandle::Stream()));
                         };
                         for (size_t f : step->factors) taken[f] = true;
-                        plan.steps.push_back(step);
+                        emit_at[f4] = step;                 // f4 reads f3 reads f2 reads f1: it is the last of the four
                         plan.n_fused++;
                         done = true;
                     }
@@ -198,7 +228,7 @@ inline void FactorGraph::BuildFusedSteps(Plan& plan)
                                                      O->value.data->ptr, GpuHandle::Stream()));
                     };
                     for (size_t f : step->factors) taken[f] = true;
-                    plan.steps.push_back(step);
+                    plan.steps.push_back(step);             // both operands are f1's; other readers of the product may precede the ReLU
                     plan.n_fused++;
                     done = true;
                 }
@@ -245,7 +275,7 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
         std::vector<size_t> inner;                       // embeddings the one-launch kernel does not write
         for (;;) {
             const int li = find_step([&](const Step& st) {
-                return st.tag == Step::LEVEL && st.vars[1] == cur && st.vars[3] == vMsg &&
+                return st.tag == Step::LEVEL && !st.bias_row && st.vars[1] == cur && st.vars[3] == vMsg &&
                        (vA == (size_t)-1 || (st.vars[0] == vA && st.vars[2] == vWc));
             });
             if (li < 0) break;

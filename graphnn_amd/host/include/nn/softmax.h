@@ -27,25 +27,5 @@ public:
     }
 };
 
-// operands: a column vector and an int tensor of segment lengths
-template<typename mode, typename Dtype>
-class JaggedSoftmax : public Factor
-{
-public:
-    static std::string StrType() { return "JaggedSoftmax"; }
-    using OutType = std::shared_ptr< DTensorVar<mode, Dtype> >;
-    OutType CreateOutVar() { return std::make_shared< DTensorVar<mode, Dtype> >(fmt::sprintf("%s:out_0", this->name)); }
-    JaggedSoftmax(std::string _name, PropErr _properr = PropErr::T) : Factor(_name, _properr) {}
-
-    virtual void Forward(std::vector< std::shared_ptr<Variable> >& operands,
-                         std::vector< std::shared_ptr<Variable> >& outputs, Phase) override
-    {
-        ASSERT(operands.size() == 2 && outputs.size() == 1, "unexpected operand count for " << StrType());
-        auto& out = detail::dense_var<mode, Dtype>(outputs[0], "JaggedSoftmax").value;
-        out.CopyFrom(detail::dense_var<mode, Dtype>(operands[0], "JaggedSoftmax").value);
-        out.JaggedSoftmax(detail::dense_var<mode, int>(operands[1], "JaggedSoftmax").value);
-    }
-};
-
 }  // namespace gnn
 #endif

@@ -267,6 +267,13 @@ def jagged_softmax(x, lens):
     return x
 
 
+def jagged_softmax_deriv(dst, out, grad, lens):
+    """dst += (grad - <grad, out> per segment) * out"""
+    check(_lib().gnnhip_jagged_softmax_deriv_f32(_f32(dst, "dst"), _f32(out, "out"), _f32(grad, "grad"), _i32(lens, "lens"),
+                                                 lens.numel(), _stream()))
+    return dst
+
+
 def jagged_softmax_static(x, lens):
     """gnnhip_jagged_softmax_static_f32: the same result, segment offsets in the library's static array."""
     check(_lib().gnnhip_jagged_softmax_static_f32(_f32(x, "x"), _i32(lens, "lens"), lens.numel(), _stream()))

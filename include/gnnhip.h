@@ -255,6 +255,12 @@ int gnnhip_csr_axpy_f32(int rows, int cols, float a, const int* row_ptr, const i
 /* ---- dst[i] += grad[i] where out[i] > 0 : ReLUDeriv(GPU) + ReLUDerivKernel (src/nn/relu.cu:18-37) */
 int gnnhip_relu_deriv_f32(size_t n, const float* out, const float* grad, float* dst, void* stream);
 
+/* ---- dst += (grad - <grad, out>_segment) * out over the segments of a jagged softmax output:
+ *      JaggedSoftmaxDeriv (CPU rule src/nn/jagged_softmax.cpp:8-31, called by JaggedSoftmax::Backward :57-74;
+ *      graphnn's own GPU overload, src/nn/jagged_softmax.cu:9-12, is an empty body). */
+int gnnhip_jagged_softmax_deriv_f32(float* dst, const float* out, const float* grad, const int* lens, int nseg,
+                                    void* stream);
+
 /* ---- y[i] *= x[i] : DTensor<GPU>::ElewiseMul(DTensor) with equal shapes
  *      (src/tensor/gpu_dense_tensor.cu:611-628, include/tensor/gpu_binary_functor.h:40-95) */
 int gnnhip_mul_f32(size_t n, const float* x, float* y, void* stream);

@@ -323,6 +323,24 @@ void orc_jagged_softmax(float* x, const int* lens, int nseg)
     free(off);
 }
 
+/* Gradient of the jagged softmax (CPU JaggedSoftmaxDeriv, src/nn/jagged_softmax.cpp:8-31):
+ * per segment z = dot(grad, out) (MKL_Dot), buf = (grad - z) * out, dst += buf. */
+void orc_jagged_softmax_deriv(float* dst, const float* out, const float* grad, const int* lens, int nseg)
+{
+    size_t off = 0;
+    for (int s = 0; s < nseg; ++s) {
+        const int n = lens[s];
+        float z = 0.0f;
+        for (int j = 0; j < n; ++j) z += grad[off + j] * out[off + j];
+        for (int j = 0; j < n; ++j) {
+            float b = grad[off + j] - z;
+            b = b * out[off + j];
+            dst[off + j] = 1.0f * b + dst[off + j];
+        }
+        off += (size_t)n;
+    }
+}
+
 /* Global sum / mean: sequential fp32 accumulation, mean = s / cnt
  * (src/tensor/cpu_dense_tensor.cpp:269-295). */
 float orc_sum(const float* x, size_t n)

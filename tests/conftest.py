@@ -128,6 +128,13 @@ class Oracle:
         self.lib.orc_jagged_softmax(_ptr(x), _ptr(lens), len(lens))
         return x
 
+    def jagged_softmax_deriv(self, dst, out, grad, lens):
+        dst = np.array(dst, np.float32, copy=True)
+        out = np.ascontiguousarray(out, np.float32); grad = np.ascontiguousarray(grad, np.float32)
+        lens = np.ascontiguousarray(lens, np.int32)
+        self.lib.orc_jagged_softmax_deriv(_ptr(dst), _ptr(out), _ptr(grad), _ptr(lens), len(lens))
+        return dst
+
     def sum(self, x):
         x = np.ascontiguousarray(x, np.float32)
         return float(self.lib.orc_sum(_ptr(x), ctypes.c_size_t(x.size)))

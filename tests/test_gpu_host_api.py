@@ -126,6 +126,85 @@ def test_host_api_forward_backward_checkpoint(gpu, oracle, tmp_path, C):
     assert np.frombuffer(blob[:24], dtype=np.uint64).tolist() == [2, C, C]       # "w_conv" sorts first
 
 
+def test_host_api_bias_level_jagged_softmax_reduce(gpu, oracle, tmp_path):
+    """FullyConnected (weights + bias row), JaggedSoftmax and Reduce through FactorGraph: the inference plan folds
+    MatMul(A, h) -> FullyConnected -> ElewiseAdd -> ReLU into the level kernel with its bias argument, the
+    training plan runs every factor on its own; attention weights, pooled features and the two reductions against
+    the oracle, the gradients of all three parameters against float64 autograd of the same network"""
+    import torch
+    exe = os.path.join(BUILD, "host_ops_check")
+    assert os.path.exists(exe), "build the host layer first: make -C graphnn_amd/host"
+    K, C, L = 9, 64, 2
+    batch = synth.molecule_batch(555, 37, K, 2, size_mode="uniform", size_lo=1, size_hi=90)
+    st = synth.Stream(555)
+    w = synth.make_weights(st, K, C, 8, 2)
+    rng = np.random.default_rng(555)
+    fc = np.concatenate([w.W_conv, (rng.standard_normal((1, C)) * 0.3).astype(np.float32)])
+    w_score = (rng.standard_normal((C, 1)) * 0.5).astype(np.float32)
+    d = str(tmp_path)
+    synth.write_graphnn_txt(batch, d + "/graphs.txt")
+    w.W_n2l.astype(np.float32).tofile(d + "/w_n2l.bin"); fc.tofile(d + "/fc.bin"); w_score.tofile(d + "/w_score.bin")
+    r = subprocess.run([exe, d, str(K), str(C), str(L)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    out = np.fromfile(d + "/out.bin", dtype=np.float32)
+
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    B, N = batch.num_graphs, batch.num_nodes
+    lens = batch.graph_sizes.astype(np.int32)
+    # the reference path, operator by operator
+    msg = oracle.gemm(X, w.W_n2l)
+    h = np.maximum(msg, 0)
+    for _ in range(L):
+        h = oracle.level(*a, h, fc[:C], msg, fc[C])
+    att = oracle.jagged_softmax(oracle.gemm(h, w_score), lens)
+    pool = oracle.spmm(*s, h, B)
+    obj = oracle.sum(oracle.gemm(att, h, transA=True))
+    pm = oracle.mean(pool)
+    pos = 0
+
+    def take(n):
+        nonlocal pos
+        v = out[pos:pos + n]; pos += n
+        return v
+
+    for phase in ("test", "train"):
+        n_steps, n_fused, got_obj, got_pm = take(4)
+        if phase == "test":
+            # input stage and L levels folded: 2 operands + 1 + L + score, softmax, pool, z, two reductions
+            assert n_fused == L + 1 and n_steps == 2 + 1 + L + 6
+        else:
+            assert n_fused == 0 and n_steps == 2 + 2 + 4 * L + 6
+        got_att = take(N).reshape(N, 1)
+        got_pool = take(B * C).reshape(B, C)
+        assert max_rel(got_att, att) < PARITY_TOL, phase
+        assert np.allclose(np.add.reduceat(got_att[:, 0].astype(np.float64), np.concatenate([[0], np.cumsum(lens)[:-1]])), 1.0, atol=1e-5)
+        assert max_rel(got_pool, pool) < PARITY_TOL, phase
+        assert abs(got_obj - obj) <= 1e-4 * abs(obj) and abs(got_pm - pm) <= 1e-4 * abs(pm), phase
+    # gradients of obj: float64 autograd of the same network
+    t64 = lambda m: torch.tensor(np.asarray(m, np.float64), requires_grad=True)
+    Wn, Fc, Ws = t64(w.W_n2l), t64(fc), t64(w_score)
+    A = torch.tensor(_dense(a, N, N)); X64 = torch.tensor(X.astype(np.float64))
+    m64 = X64 @ Wn
+    h64 = torch.relu(m64)
+    for _ in range(L):
+        h64 = torch.relu((A @ h64) @ Fc[:C] + Fc[C] + m64)
+    sc = (h64 @ Ws)[:, 0]
+    seg = torch.tensor(np.repeat(np.arange(B), lens))
+    mx = torch.zeros(B, dtype=torch.float64).scatter_reduce(0, seg, sc.detach(), "amax", include_self=False)
+    e = torch.exp(sc - mx[seg])
+    att64 = e / torch.zeros(B, dtype=torch.float64).index_add(0, seg, e)[seg]
+    obj64 = (att64[:, None] * h64).sum()
+    obj64.backward()
+    assert abs(float(obj64) - obj) <= 1e-4 * abs(obj)
+    for name, p64 in (("w_n2l", Wn), ("fc", Fc), ("w_score", Ws)):
+        g64 = p64.grad.numpy()
+        got = take(g64.size).reshape(g64.shape)
+        assert max_rel(got, g64) < PARITY_TOL, name
+    assert pos == out.size
+
+
 def test_host_api_large_batch_takes_the_separate_kernels(gpu, oracle, tmp_path):
     """a batch of more than 20,000 nodes: the inference plan still folds the forward into one step, which now
     calls the whole-forward entry of the library (separate kernels, h0 not stored) instead of the one-launch

@@ -335,6 +335,25 @@ def test_jagged_softmax(gpu, oracle):
     assert np.allclose(sums, 1.0, atol=1e-4)
 
 
+def test_jagged_softmax_gradient(gpu, oracle):
+    """dst += (grad - <grad, out>) * out per segment (src/nn/jagged_softmax.cpp:8-31), ragged segments"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(61)
+    lens = rng.integers(0, 50, 2500).astype(np.int32)
+    lens[[0, 9]] = 0; lens[4] = 1; lens[700] = 9000
+    n = int(lens.sum())
+    p = oracle.jagged_softmax((rng.standard_normal(n) * 2).astype(np.float32), lens)
+    g = rng.standard_normal(n).astype(np.float32)
+    d0 = rng.standard_normal(n).astype(np.float32)
+    want = oracle.jagged_softmax_deriv(d0, p, g, lens)
+    got = _n(ops.jagged_softmax_deriv(_t(d0, gpu), _t(p, gpu), _t(g, gpu), _t(lens, gpu)))
+    off = np.concatenate([[0], np.cumsum(lens)])
+    seg = np.repeat(np.arange(lens.size), lens)
+    z = np.bincount(seg, weights=g.astype(np.float64) * p, minlength=lens.size)
+    want64 = d0 + (g - z[seg]) * p.astype(np.float64)
+    assert_parity("jagged softmax gradient", got, want, want64)
+
+
 # ------------------------------------------------------------------ reductions and index ops
 @pytest.mark.parametrize("n", [1, 63, 256, 4000, 16385, 3_000_001])
 def test_reduce(gpu, oracle, n):

@@ -77,3 +77,14 @@ def test_cpp_builders_on_a_getbatch_style_batch(oracle, tmp_path):
     # undirected graphs stored in both directions: every edge sees the other in-edges of its tail
     indeg = np.bincount(b.edge_y, minlength=b.num_nodes)
     assert e2e[1].size == int((indeg * (indeg - 1)).sum())
+
+
+def test_folded_level_runs_after_the_producers_of_all_its_operands():
+    """inference plan of a graph whose msg comes out of a deeper chain than the fed embedding: the folded level
+    must be scheduled where its last factor stood, behind the step that produces msg (no GPU: nothing runs)"""
+    exe = os.path.join(ROOT, "graphnn_amd", "host", "build", "host_plan_check")
+    if not os.path.exists(exe):
+        subprocess.check_call(["make", "-C", os.path.join(ROOT, "graphnn_amd", "host"), "build/host_plan_check"])
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "host_plan_check ok" in r.stdout

@@ -324,6 +324,38 @@ def test_jagged_softmax_equals_per_segment(oracle):
 
 
 # ------------------------------------------------------------------ reductions, arg-max, CE, top-k
+def test_jagged_softmax_gradient_is_the_softmax_jacobian(oracle):
+    """dst += J^T g with J the Jacobian of softmax, segment by segment: checked against the Jacobian
+    written out in float64 (d p_i / d x_j = p_i (delta_ij - p_j)) and against a central difference"""
+    rng = _rng(23)
+    lens = np.array([1, 4, 0, 7, 2], np.int32)
+    x = rng.standard_normal(int(lens.sum())).astype(np.float32)
+    g = rng.standard_normal(x.size).astype(np.float32)
+    d0 = rng.standard_normal(x.size).astype(np.float32)
+    p = oracle.jagged_softmax(x, lens)
+    got = oracle.jagged_softmax_deriv(d0, p, g, lens)
+    want = d0.astype(np.float64).copy()
+    off = 0
+    for n in lens:
+        pp = p[off:off + n].astype(np.float64)
+        J = np.diag(pp) - np.outer(pp, pp)
+        want[off:off + n] += J.T @ g[off:off + n].astype(np.float64)
+        off += n
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+    # central difference of <g, softmax(x)> in float64
+    def f(xv):
+        tot, o = 0.0, 0
+        for n in lens:
+            if n:
+                e = np.exp(xv[o:o + n] - xv[o:o + n].max())
+                tot += float(g[o:o + n].astype(np.float64) @ (e / e.sum()))
+            o += n
+        return tot
+    x64 = x.astype(np.float64)
+    num = np.array([(f(x64 + 1e-6 * np.eye(x.size)[i]) - f(x64 - 1e-6 * np.eye(x.size)[i])) / 2e-6 for i in range(x.size)])
+    assert np.allclose(got - d0, num, atol=1e-4)
+
+
 def test_reductions(oracle):
     ints = np.arange(1, 1001, dtype=np.float32)
     assert oracle.sum(ints) == 500500.0 and oracle.mean(ints) == 500.5 and oracle.max(ints) == 1000.0
