@@ -139,7 +139,7 @@ def time_level_cfg4(dev):
     N, E, C = batch.num_nodes, int(a[1].size), cfg["C"]
     flops = 2.0 * N * C * C + 2.0 * E * C + 2.0 * N * C
     return {"workload": "configuration 4: one level, %d nodes, %d entries, hidden %d" % (N, E, C),
-            "kernel": "s2v_level_wide_kernel<256,8,false,64>", "avg_ms": ms,
+            "kernel": "s2v_level_wide_kernel<256,8,false,64>", "avg_ms": ms, "flops": flops,
             "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS},
             "algorithmic_GBps": level_algorithmic_bytes(N, E, C) / (ms * 1e-3) / 1e9}
@@ -263,7 +263,7 @@ def time_cfg5(dev, scale=22):
     score = torch.empty((N, 1), dtype=torch.float32, device=dev)
     pool = torch.empty((B, C), dtype=torch.float32, device=dev)
     res = {"workload": "configuration 5: R-MAT scale %d, %d rows, %d entries, max row %d, %d rows over 256 entries, hidden %d"
-                       % (scale, N, E, int(cnt.max()), int((cnt > 256).sum()), C)}
+                       % (scale, N, E, int(cnt.max()), int((cnt > 256).sum()), C), "shape": (N, E, C, B)}
     ms = _event_ms(lambda: ops.s2v_level(rp, ci, val, h0, Wc, msg, out=h1), 5)
     res["level"] = {"avg_ms": ms, "algorithmic_GBps": level_algorithmic_bytes(N, E, C) / (ms * 1e-3) / 1e9,
                     "gather_GBps": (4.0 * E * C + 12.0 * N * C + 8.0 * E) / (ms * 1e-3) / 1e9}
@@ -285,6 +285,35 @@ def time_cfg5(dev, scale=22):
     seg = sc.view(B, 1024).double().sum(dim=1)
     assert float((seg - 1.0).abs().max()) < 1e-5, "jagged softmax segments do not sum to 1"
     return res
+
+
+def kernel_rooflines(dev):
+    """The other kernels of the path at the sizes they are built for, each against the roofline that bounds
+    it: the hidden-256 level of configuration 4 against the FP32 matrix peak, the configuration-5 kernels
+    (R-MAT, 4.2M rows) against HBM.  achieved = algorithmic bytes (or flops) per launch / HIP-event time."""
+    def hbm(kernel, workload, nbytes, ms, **more):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        d = {"kernel": kernel, "workload": workload, "bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+             "frac": gbs / HBM_PEAK_GBS, "algorithmic_bytes": nbytes, "avg_ms": ms, "traffic": None}
+        d.update(more)
+        return d
+    c4 = time_level_cfg4(dev)
+    r4 = dict(c4["roofline"], kernel=c4["kernel"], workload=c4["workload"], avg_ms=c4["avg_ms"], flops=c4["flops"],
+              algorithmic_GBps=c4["algorithmic_GBps"], traffic=None)
+    c5 = time_cfg5(dev)
+    N, E, C, B = c5["shape"]
+    w5 = c5["workload"]
+    return [
+        r4,
+        hbm("s2v_level_stream_kernel<64,true,...> + hub_partial_kernel + spmm_rowgroup_kernel (two-launch level)", w5 + ": one level",
+            level_algorithmic_bytes(N, E, C), c5["level"]["avg_ms"], gather_GBps=c5["level"]["gather_GBps"]),
+        hbm("spmm_rowgroup_kernel<4,1> + hub_partial_kernel<4,1>", w5 + ": SpMM A*h",
+            spmm_algorithmic_bytes(N, N, E, C), c5["spmm"]["avg_ms"], gather_GBps=c5["spmm"]["gather_GBps"]),
+        hbm("sgemm_skinny_rows_kernel<1>", w5 + ": node scores h*w", 4 * N * (C + 1), c5["score"]["avg_ms"]),
+        hbm("exclusive_scan_kernel + jagged_softmax_kernel", w5 + ": jagged softmax over %d segments of 1024" % B,
+            8 * N + 4 * B, c5["jagged_softmax"]["avg_ms"]),
+        hbm("spmm_rowgroup_kernel<4,1>", w5 + ": sum-pool S*h", 4 * N * C + 8 * N + 4 * (B + 1) + 4 * B * C, c5["sum_pool"]["avg_ms"]),
+    ]
 
 
 def end_to_end_host_layer(host, reps=300):
@@ -311,12 +340,7 @@ def end_to_end_host_layer(host, reps=300):
     return res
 
 
-def cpu_baseline(host, budget_s=12.0):
-    """The CPU restatement of the reference path on the same batch, timed on this host."""
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    from conftest import Oracle
-    orc = Oracle()
-    threads = int(orc.lib.orc_num_threads())
+def _time_oracle_forward(orc, host, budget_s):
     batch, cfg = host["batch"], host["cfg"]
     orc.forward(host["a"], host["s"], host["X"], host["w"], cfg["L"], None)      # warm-up
     reps, t0 = 0, time.perf_counter()
@@ -326,8 +350,125 @@ def cpu_baseline(host, budget_s=12.0):
         el = time.perf_counter() - t0
         if el >= budget_s or reps >= 100000:
             break
-    return dict(value=batch.num_graphs * reps / el, unit="graphs/s", cores=threads, kind="port",
-                sample="%d forwards of the same configuration-2 batch in %.1f s (gcc -O3 -mavx2, OpenMP over rows)" % (reps, el))
+    return batch.num_graphs * reps / el, reps, el
+
+
+def _load_mkl():
+    """libmkl_rt of the image's conda tree (oneMKL), or None.  Loaded only by the child process of mkl_baseline."""
+    import ctypes
+    for name in ("libmkl_rt.so.2", "libmkl_rt.so.1", "libmkl_rt.so", "/opt/conda/lib/libmkl_rt.so.2",
+                 "/opt/conda/lib/libmkl_rt.so.1", "/opt/conda/lib/libmkl_rt.so", "/opt/intel/mkl/lib/intel64/libmkl_rt.so",
+                 "/opt/intel/oneapi/mkl/latest/lib/intel64/libmkl_rt.so"):
+        try:
+            return ctypes.CDLL(name)
+        except OSError:
+            continue
+    return None
+
+
+def mkl_child(budget_s=8.0):
+    """Child-process body: the reference CPU path with its own arithmetic library on the configuration-2
+    batch: mkl_scsrmm("GLNC") for A*h and S*h, cblas_sgemm for the dense products, as DTensor<CPU>::MM calls
+    them (src/tensor/cpu_dense_tensor.cpp:198-225); the element-wise steps in numpy.  Prints one JSON line."""
+    import ctypes
+    mkl = _load_mkl()
+    if mkl is None:
+        print(json.dumps({"available": False, "note": "MKL not available on this host"}))
+        return
+    from graphnn_amd import batching, synth
+    batch, w, cfg = synth.make_config(2)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    sg = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    P = lambda arr: arr.ctypes.data_as(ctypes.c_void_p)
+    ci_t, cf = ctypes.c_int, ctypes.c_float
+
+    def csrmm(csr, Bm, out):
+        rp, ci, v = csr
+        m, k, n = ci_t(out.shape[0]), ci_t(Bm.shape[0]), ci_t(Bm.shape[1])
+        al, be = cf(1.0), cf(0.0)
+        pe = rp[1:]
+        mkl.mkl_scsrmm(ctypes.c_char_p(b"N"), ctypes.byref(m), ctypes.byref(n), ctypes.byref(k), ctypes.byref(al),
+                       ctypes.c_char_p(b"GLNC"), P(v), P(ci), P(rp), P(pe), P(Bm), ctypes.byref(n), ctypes.byref(be),
+                       P(out), ctypes.byref(n))
+
+    def sgemm(A, Bm, out):
+        mkl.cblas_sgemm(101, 111, 111, A.shape[0], Bm.shape[1], A.shape[1], cf(1.0), P(A), A.shape[1], P(Bm), Bm.shape[1],
+                        cf(0.0), P(out), Bm.shape[1])
+
+    N, B, C, H, Q, L = batch.num_nodes, batch.num_graphs, cfg["C"], cfg["H"], cfg["Q"], cfg["L"]
+    f = np.float32
+    msg, h, agg, lin = (np.empty((N, C), f) for _ in range(4))
+    pool, hid, logits = np.empty((B, C), f), np.empty((B, H), f), np.empty((B, Q), f)
+
+    def forward():
+        sgemm(X, w.W_n2l, msg)
+        np.maximum(msg, 0, out=h)
+        for _ in range(L):
+            csrmm(a, h, agg)
+            sgemm(agg, w.W_conv, lin)
+            np.add(lin, msg, out=lin)
+            np.maximum(lin, 0, out=h)
+        csrmm(sg, h, pool)
+        sgemm(pool, w.W_h1, hid)
+        np.maximum(hid, 0, out=hid)
+        sgemm(hid, w.W_h2, logits)
+        e = np.exp(logits - logits.max(axis=1, keepdims=True))
+        return e / e.sum(axis=1, keepdims=True)
+
+    forward()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        forward()
+        reps += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s:
+            break
+    mkl.mkl_get_max_threads.restype = ctypes.c_int
+    buf = ctypes.create_string_buffer(256)
+    mkl.mkl_get_version_string(buf, 256)
+    print(json.dumps({"available": True, "value": B * reps / el, "unit": "graphs/s", "cores": int(mkl.mkl_get_max_threads()),
+                      "version": buf.value.decode(errors="replace").strip(),
+                      "logits_checksum": float(np.abs(logits).sum()),
+                      "sample": "%d forwards of the configuration-2 batch in %.1f s: mkl_scsrmm \"GLNC\" + cblas_sgemm, "
+                                "element-wise steps in numpy" % (reps, el)}))
+
+
+def mkl_baseline():
+    """Runs mkl_child in a process of its own (MKL brings its own OpenMP runtime; it stays out of this one)."""
+    import subprocess
+    env = dict(os.environ, MKL_THREADING_LAYER="GNU")
+    try:
+        r = subprocess.run([sys.executable, os.path.abspath(__file__), "--mkl-child"], capture_output=True, text=True,
+                           timeout=120, env=env)
+        if r.returncode == 0 and r.stdout.strip():
+            return json.loads(r.stdout.strip().splitlines()[-1])
+        return {"available": False, "note": "MKL not available on this host", "detail": (r.stderr or r.stdout)[-200:]}
+    except Exception as exc:          # a broken MKL install must not cost the bench line
+        return {"available": False, "note": "MKL not available on this host", "detail": str(exc)[:200]}
+
+
+def cpu_baseline(host, budget_s=8.0):
+    """The CPU restatement of the reference path on the same batch, timed on this host: all OpenMP threads,
+    one thread, and the same path on the reference's own arithmetic library (MKL) where the host has it."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from conftest import Oracle
+    orc = Oracle()
+    threads = int(orc.lib.orc_num_threads())
+    value, reps, el = _time_oracle_forward(orc, host, budget_s)
+    orc.lib.orc_set_num_threads(1)
+    value1, reps1, el1 = _time_oracle_forward(orc, host, budget_s)
+    orc.lib.orc_set_num_threads(threads)
+    mkl = mkl_baseline()
+    if mkl.get("available"):
+        want = orc.forward(host["a"], host["s"], host["X"], host["w"], host["cfg"]["L"], None)
+        ref = float(np.abs(want["logits"]).sum())
+        mkl["agrees_with_port"] = bool(abs(mkl["logits_checksum"] - ref) <= 1e-4 * ref)
+    return dict(value=value, unit="graphs/s", cores=threads, kind="port",
+                sample="%d forwards of the same configuration-2 batch in %.1f s (gcc -O3 -mavx2, OpenMP over rows)" % (reps, el),
+                value_1_thread=value1,
+                sample_1_thread="%d forwards in %.1f s with one thread" % (reps1, el1),
+                mkl=mkl)
 
 
 def main():
@@ -340,10 +481,18 @@ def main():
     ap.add_argument("--extra", action="store_true",
                     help="also time the configuration-4 level (FP32 matrix cores) and the configuration-5 "
                          "kernels (R-MAT, 4M rows) and report them under \"extra\"")
+    ap.add_argument("--no-rooflines", action="store_true",
+                    help="skip the configuration-4 / configuration-5 kernel rooflines")
+    ap.add_argument("--only", default="", help="comma-separated legs to run alone (for profiling): "
+                                                "forward, spmm, cfg4, cfg5")
+    ap.add_argument("--mkl-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one element-wise copy kernel of known size (1 GiB read, 1 GiB written) "
                          "so hardware counters collected over this run can be scaled")
     args = ap.parse_args()
+    if args.mkl_child:
+        mkl_child()
+        return
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
 
@@ -353,6 +502,30 @@ def main():
     from graphnn_amd import ops
     ops.init(0)
     dev = torch.device("cuda:0")
+
+    if args.only:
+        # single legs for profiler runs (counters are collected over one kernel's launches at a time)
+        legs = set(args.only.split(","))
+        res = {}
+        if "forward" in legs:
+            dev_args, host = build_forward_workload(dev)
+            sec, _ = time_forward(dev_args, host["cfg"], host["batch"], args.steps, args.warmup, "graph_resident")
+            res["forward_ms"] = sec * 1e3
+        if "spmm" in legs:
+            res["spmm_cfg3_ms"] = time_spmm_cfg3(dev)[0]
+        if "cfg4" in legs:
+            res["cfg4_level"] = time_level_cfg4(dev)
+        if "cfg5" in legs:
+            res["cfg5"] = time_cfg5(dev)
+        if args.calibrate:
+            n = 1 << 28
+            src = torch.ones(n, device=dev, dtype=torch.float32)
+            dst = torch.empty_like(src)
+            ops.relu(src, dst)
+            torch.cuda.synchronize()
+            res["calibration"] = {"kernel": "map1_kernel<FReLU>", "bytes_read": 4 * n, "bytes_written": 4 * n}
+        print(json.dumps(res))
+        return
 
     dev_args, host = build_forward_workload(dev)
     batch, cfg = host["batch"], host["cfg"]
@@ -392,6 +565,8 @@ def main():
         out["roofline"] = {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES["spmm_cfg3"],
+            "traffic_source": "constant: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 of spmm_rowgroup_kernel<4,1> from the rocprofv3 "
+                              "--pmc runs summarised in profiles/bench_forward_cfg2_spmm_cfg3.md (not re-measured in this run)",
             "kernel": "spmm_rowgroup_kernel<4,1>",
             "workload": "configuration 3: CSR SpMM, %d rows, %d entries, width %d" % (n, nnz, d),
             "algorithmic_bytes": bytes_alg, "avg_ms": mean_ms, "min_ms": min_ms,
@@ -412,8 +587,11 @@ def main():
 
     out["end_to_end"] = end_to_end_host_layer(host)
 
+    if not args.no_rooflines:
+        out["rooflines"] = kernel_rooflines(dev)
+
     if args.extra:
-        out["extra"] = {"cfg4_level": time_level_cfg4(dev), "large_batch": time_large_batch(dev), "cfg5": time_cfg5(dev),
+        out["extra"] = {"large_batch": time_large_batch(dev),
                         "device_batch_assembly": time_device_batch_assembly(dev),
                         "training_step": training_step_host_layer(host)}
 
