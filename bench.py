@@ -61,6 +61,11 @@ def time_forward(dev_args, cfg, batch, steps, warmup, route):
         bufs = ops.BatchedBuffers(N, B, cfg["C"], cfg["H"], cfg["Q"], dev)
         nmax = int(batch.graph_sizes.max())
         run = lambda: ops.s2v_forward_batched(*dev_args, cfg["L"], nmax, bufs=bufs)
+    elif route == "graph_resident_labels":
+        bufs = ops.BatchedBuffers(N, B, cfg["C"], cfg["H"], cfg["Q"], dev)
+        nmax = int(batch.graph_sizes.max())
+        lab = torch.from_numpy(np.ascontiguousarray(batch.node_label, dtype=np.int32)).to(dev)
+        run = lambda: ops.s2v_forward_batched_labels(dev_args[0], dev_args[1], lab, *dev_args[3:], cfg["L"], nmax, bufs=bufs)
     else:
         bufs = ops.ForwardBuffers(N, B, cfg["C"], cfg["H"], cfg["Q"], dev)
         run = lambda: ops.s2v_forward(*dev_args, cfg["L"], bufs=bufs)
@@ -72,7 +77,7 @@ def time_forward(dev_args, cfg, batch, steps, warmup, route):
         run()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    if route == "graph_resident":
+    if route.startswith("graph_resident"):
         assert int(bufs.status.cpu()[0]) == 0, "graph-resident forward reported a layout violation"
     return (t1 - t0) / steps, bufs
 
@@ -531,6 +536,9 @@ def main():
     batch, cfg = host["batch"], host["cfg"]
     sec_general, bufs_general = time_forward(dev_args, cfg, batch, args.steps, args.warmup, "general")
     sec, bufs = time_forward(dev_args, cfg, batch, args.steps, args.warmup, "graph_resident")
+    sec_labels, bufs_labels = time_forward(dev_args, cfg, batch, args.steps, args.warmup, "graph_resident_labels")
+    assert bool(torch.equal(bufs_labels.logits, bufs.logits)) and bool(torch.equal(bufs_labels.pred, bufs.pred)), \
+        "label input and one-hot input disagree"
     # the two routes must agree on what they computed
     assert bool((bufs.pred == bufs_general.pred).all()), "routes disagree on predictions"
     assert float((bufs.logits - bufs_general.logits).abs().max()) <= 1e-4 * float(bufs_general.logits.abs().max()), \
@@ -555,6 +563,10 @@ def main():
                    "graphs": batch.num_graphs, "nodes": batch.num_nodes, "edges": batch.num_edges},
         "nodes_per_s": batch.num_nodes / sec,
         "route": "graph-resident forward, one launch (gnnhip_s2v_forward_batched_f32)",
+        "label_input_route": {"graphs_per_s": batch.num_graphs / sec_labels, "ms_per_step": sec_labels * 1e3,
+                              "what": "gnnhip_s2v_forward_batched_labels_f32: the same launch fed one int label per node "
+                                      "instead of the one-hot matrix X (bit-identical outputs); `value` keeps the "
+                                      "reference's dense X"},
         "general_route": {"graphs_per_s": batch.num_graphs / sec_general, "ms_per_step": sec_general * 1e3,
                           "what": "gnnhip_s2v_forward_f32: input + 4 fused levels + readout, any CSR"},
     }

@@ -40,6 +40,7 @@ namespace {
 
 constexpr int kEdgeCapMax = 4096;       // CSR entries of one graph staged in LDS (fewer if LDS is short); larger graphs read them from L2
 constexpr size_t kLdsLimit = 160 * 1024;
+constexpr int kLabelWeightCap = 8192;   // floats of W_n2l staged in LDS by the label-input variant; larger tables are read from L2
 constexpr int kReadoutCap = 8192;       // floats of W_h1 and W_h2 staged in LDS; larger layers are read from L2
 
 // LDS carve-up, in floats:
@@ -49,24 +50,32 @@ struct GraphLds {
     // contraction steps of the input stage: the K label columns in groups of four, an even number of them
     __host__ __device__ static int input_steps(int K) { return ((K + 3) / 4 + 1) & ~1; }
     // the agg buffer also holds the staged X rows (n x 4 input_steps(K), zero-padded) and the pooling partials (waves x C)
-    __host__ __device__ static size_t agg_floats(int n16, int C, int K, int block)
+    __host__ __device__ static size_t agg_floats(int n16, int C, int K, int block, bool labels = false)
     {
         size_t a = (size_t)n16 * (C + 4);
-        const size_t p = (size_t)(block / 64) * C, x = (size_t)n16 * 4 * input_steps(K);
+        const size_t p = (size_t)(block / 64) * C, x = labels ? 0 : (size_t)n16 * 4 * input_steps(K);
         if (p > a) a = p;
         if (x > a) a = x;
         return (a + 3) / 4 * 4;
     }
-    static size_t fixed_floats(int n16, int C, int K, int H, int Q, int block)
+    // label input: the graph's labels [n16] and, when it is small enough, W_n2l [K][C] behind the edge cache
+    __host__ __device__ static bool wn_staged(int C, int K) { return (size_t)K * C <= (size_t)kLabelWeightCap; }
+    __host__ __device__ static size_t label_floats(int n16, int C, int K)
+    {
+        return (size_t)n16 + (wn_staged(C, K) ? (size_t)K * C : 0);
+    }
+    static size_t fixed_floats(int n16, int C, int K, int H, int Q, int block, bool labels = false)
     {
         const size_t wro = ((size_t)C * H + (size_t)H * Q <= (size_t)kReadoutCap) ? (size_t)C * H + (size_t)H * Q : 0;
-        size_t f = (size_t)(n16 + 1) * (C + 4) + agg_floats(n16, C, K, block) + (size_t)(2 * n16 + 4) + H + Q + wro;
-        return (f + 3) / 4 * 4;
+        size_t f = (size_t)(n16 + 1) * (C + 4) + agg_floats(n16, C, K, block, labels) + (size_t)(2 * n16 + 4) + H + Q + wro;
+        f = (f + 3) / 4 * 4;
+        if (labels) f += (label_floats(n16, C, K) + 3) / 4 * 4;
+        return f;
     }
     // entries of the edge cache that still fit under the LDS limit
-    static int edge_cap(int n16, int C, int K, int H, int Q, int block)
+    static int edge_cap(int n16, int C, int K, int H, int Q, int block, bool labels = false)
     {
-        const size_t fixed = fixed_floats(n16, C, K, H, Q, block) * sizeof(float);
+        const size_t fixed = fixed_floats(n16, C, K, H, Q, block, labels) * sizeof(float);
         if (fixed >= kLdsLimit) return -1;
         size_t cap = (kLdsLimit - fixed) / (2 * sizeof(float));
         if (cap > (size_t)kEdgeCapMax) cap = kEdgeCapMax;
@@ -86,6 +95,10 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     float* __restrict__ msg, float* __restrict__ h_final, float* __restrict__ pool, float* __restrict__ hidden,
     float* __restrict__ logits, float* __restrict__ probs, int* __restrict__ pred, int* __restrict__ status)
 {
+    // KSX == 0: the node features arrive as one label per node (X points at int labels[N]) and the input
+    // stage is a row lookup in W_n2l; otherwise X is the dense [N,K] matrix and KSX bounds its contraction steps
+    constexpr bool LABELS = (KSX == 0);
+    constexpr int KSXA = LABELS ? 2 : KSX;
     constexpr int kBlock = WAVES * kWave;
     constexpr int kWavesPerBlock = WAVES;
     constexpr int G = C / 4;             // lanes per row in gathers
@@ -99,7 +112,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
 
     extern __shared__ float smem[];
     const bool ro_staged = ((size_t)C * H + (size_t)H * Q <= (size_t)kReadoutCap);
-    const size_t agg_fl = GraphLds::agg_floats(n16max, C, K, kBlock);
+    const size_t agg_fl = GraphLds::agg_floats(n16max, C, K, kBlock, LABELS);
     float* hbuf = smem;                                  // [n16max + 1][LDT]; row n16max is never written after start-up and holds zeros
     float* agg = hbuf + (size_t)(n16max + 1) * LDT;      // [n16max][LDT]; doubles as part[P][C] in the readout
     float* part = agg;
@@ -113,6 +126,10 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     tail = smem + ((size_t)(tail - smem) + 3) / 4 * 4;
     int* e_col = reinterpret_cast<int*>(tail);           // [ecap] neighbour index local to the graph
     float* e_val = tail + ecap;                          // [ecap]
+    int* l_lab = reinterpret_cast<int*>(e_val + ecap);   // label input only: [n16max] labels of the graph's nodes
+    float* wn_s = reinterpret_cast<float*>(l_lab + n16max);     // label input only: W_n2l [K][C] when staged
+    const bool wn_in_lds = LABELS && GraphLds::wn_staged(C, K);
+    const int* labels = reinterpret_cast<const int*>(X);
 
     // the lane's coordinates, used by the start-up code; the graph loop derives its own copies (see there)
     const int tid0 = threadIdx.x;
@@ -149,6 +166,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
         for (int i = tid0 + 4 * kBlock; i < n1; i += kBlock) w1s[(i % H) * C + i / H] = Wh1[i];
         for (int i = tid0 + kBlock; i < n2; i += kBlock) w2s[(i % Q) * H + i / Q] = Wh2[i];
     }
+    if (LABELS && wn_in_lds)
+        for (int i = tid0; i < K * C; i += kBlock) wn_s[i] = Wn2l[i];
     // (the staged copies become visible to all lanes at the first barrier of the graph loop)
     GNNHIP_PHASE_MARK(1);
     const rsrc_t wn_rsrc = make_rsrc(Wn2l, (unsigned)((size_t)K * C * 4));
@@ -179,9 +198,11 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
         // this wavefront's 16 columns of W_n2l^T for the input stage: k = srt q + s, zero beyond K (rows past the
         // end of the buffer read as zero; steps s >= srt are loaded but not used).  Loaded per graph (from L2) so the registers are free during the
         // levels; one lane offset plus constant strides, so no per-element address lives across the graph loop.
-        float wx[KSX];
+        float wx[KSXA];
+        if (!LABELS) {
 #pragma unroll
-        for (int s = 0; s < KSX; ++s) wx[s] = buf_load_f(wn_rsrc, wx_lane_off + s * (C * 4), 0);
+            for (int s = 0; s < KSXA; ++s) wx[s] = buf_load_f(wn_rsrc, wx_lane_off + s * (C * 4), 0);
+        }
 
         // ---- stage the graph's CSR slice (L uses), its pooling weights and its rows of X (contiguous in memory;
         //      parked in the still unused agg buffer), and check the block-diagonal promise.  Everything a lane
@@ -199,14 +220,18 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
                 const int r = K >= 2 ? (int)__umulhi((unsigned)i, k_magic) : i;
                 return r * KP + (i - r * K);
             };
-            int rp_v = 0, sc_v = 0, c_v = 0;
+            int rp_v = 0, sc_v = 0, c_v = 0, lab_v = 0;
             float sv_v = 0.f, v_v = 0.f, xv[kXSlots];
 #pragma unroll
             for (int u = 0; u < kXSlots; ++u) xv[u] = 0.f;
             if (tid <= n) rp_v = a_row_ptr[node0 + tid];
             if (tid < n) { sc_v = s_col_idx[node0 + tid]; sv_v = s_val[node0 + tid]; }
+            if (LABELS) {
+                if (tid < n) lab_v = labels[node0 + tid];
+            } else {
 #pragma unroll
-            for (int u = 0; u < kXSlots; ++u) if (tid + u * kBlock < nx) xv[u] = xg[tid + u * kBlock];
+                for (int u = 0; u < kXSlots; ++u) if (tid + u * kBlock < nx) xv[u] = xg[tid + u * kBlock];
+            }
             // (the graph's first entry is the last thing to arrive at start-up: everything above is under way by then)
             if (staged && tid < ne) { c_v = a_col_idx[e0 + tid]; v_v = a_val[e0 + tid]; }
 
@@ -221,14 +246,23 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
                 e_col[tid] = min(max(c, 0), n - 1);
                 e_val[tid] = v_v;
             }
+            if (LABELS) {
+                // a label outside [0, K) is reported (bit 3) and clamped, so no read leaves W_n2l
+                for (int i = tid; i < n; i += kBlock) {
+                    const int lab = (i == tid) ? lab_v : labels[node0 + i];
+                    if (lab < 0 || lab >= K) { if (status) atomicOr(status, 8); }
+                    l_lab[i] = min(max(lab, 0), K - 1);
+                }
+            } else {
 #pragma unroll
-            for (int u = 0; u < kXSlots; ++u) {
-                const int i = tid + u * kBlock;
-                if (i < nx) xs[x_slot(i)] = xv[u];
+                for (int u = 0; u < kXSlots; ++u) {
+                    const int i = tid + u * kBlock;
+                    if (i < nx) xs[x_slot(i)] = xv[u];
+                }
+                // columns K .. KP-1 of the staged rows (at most 7) are zero
+                for (int r = tid; r < n; r += kBlock)
+                    for (int k = K; k < KP; ++k) xs[r * KP + k] = 0.f;
             }
-            // columns K .. KP-1 of the staged rows (at most 7) are zero
-            for (int r = tid; r < n; r += kBlock)
-                for (int k = K; k < KP; ++k) xs[r * KP + k] = 0.f;
             // what exceeds one element per lane (kXSlots of X)
             for (int i = tid + kBlock; i <= n; i += kBlock) l_rp[i] = a_row_ptr[node0 + i] - e0;
             for (int i = tid + kBlock; i < n; i += kBlock) {
@@ -243,7 +277,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
                     e_val[i] = a_val[e0 + i];
                 }
             }
-            for (int i = tid + kXSlots * kBlock; i < nx; i += kBlock) xs[x_slot(i)] = xg[i];
+            if (!LABELS)
+                for (int i = tid + kXSlots * kBlock; i < nx; i += kBlock) xs[x_slot(i)] = xg[i];
         }
         __syncthreads();
 
@@ -259,19 +294,29 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
                 const bool valid = lr < n;
                 // every lane reads a valid LDS slot (row clamped; rows beyond n are zeroed below); the
                 // lane's srt values are contiguous and 8-byte aligned
-                const float* xrow = xs + min(lr, n - 1) * KP + srt * q;
-                float xreg[KSX];
+                float4 v;                                                     // row lr, columns 16 jb + 4 q + {0..3}
+                if (LABELS) {
+                    // the product of a one-hot row with W_n2l is that row of W_n2l (0 + w, so -0.0 becomes +0.0
+                    // as in the sum the dense product forms)
+                    const int lab = l_lab[min(lr, n - 1)];
+                    const float* wrow = (wn_in_lds ? wn_s : Wn2l) + (size_t)lab * C + 16 * jb + 4 * q;
+                    const float4 wv = *reinterpret_cast<const float4*>(wrow);
+                    v = make_float4(0.f + wv.x, 0.f + wv.y, 0.f + wv.z, 0.f + wv.w);
+                } else {
+                    const float* xrow = xs + min(lr, n - 1) * KP + srt * q;
+                    float xreg[KSXA];
 #pragma unroll
-                for (int s2 = 0; s2 < KSX / 2; ++s2) {
-                    float2 v2 = make_float2(0.f, 0.f);
-                    if (2 * s2 < srt) v2 = *reinterpret_cast<const float2*>(xrow + 2 * s2);
-                    xreg[2 * s2] = v2.x; xreg[2 * s2 + 1] = v2.y;
+                    for (int s2 = 0; s2 < KSXA / 2; ++s2) {
+                        float2 v2 = make_float2(0.f, 0.f);
+                        if (2 * s2 < srt) v2 = *reinterpret_cast<const float2*>(xrow + 2 * s2);
+                        xreg[2 * s2] = v2.x; xreg[2 * s2 + 1] = v2.y;
+                    }
+                    mfma_f4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s = 0; s < KSXA; ++s)
+                        if (s < srt) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wx[s], xreg[s], acc, 0, 0, 0);
+                    v = make_float4(acc[0], acc[1], acc[2], acc[3]);
                 }
-                mfma_f4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int s = 0; s < KSX; ++s)
-                    if (s < srt) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wx[s], xreg[s], acc, 0, 0, 0);
-                float4 v = make_float4(acc[0], acc[1], acc[2], acc[3]);      // row lr, columns 16 jb + 4 q + {0..3}
                 if (!valid) v = f4_zero();
                 if (valid) *reinterpret_cast<float4*>(msg + (size_t)(node0 + lr) * C + 16 * jb + 4 * q) = v;
                 *reinterpret_cast<float4*>(hbuf + (size_t)lr * LDT + 16 * jb + 4 * q) = relu_ref4(v);
@@ -512,9 +557,10 @@ int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
                          int* pred, int* status, hipStream_t s)
 {
     constexpr int kBlock = WAVES * kWave;
-    const int ecap = GraphLds::edge_cap(n16max, C, K, H, Q, kBlock);
+    constexpr bool LABELS = (KSX == 0);
+    const int ecap = GraphLds::edge_cap(n16max, C, K, H, Q, kBlock, LABELS);
     if (ecap < 0) return GNNHIP_EUNSUPPORTED;
-    const size_t smem = sizeof(float) * (GraphLds::fixed_floats(n16max, C, K, H, Q, kBlock) + 2 * (size_t)ecap);
+    const size_t smem = sizeof(float) * (GraphLds::fixed_floats(n16max, C, K, H, Q, kBlock, LABELS) + 2 * (size_t)ecap);
     static LdsLimit lds_limit;              // largest dynamic LDS size this kernel instantiation has been allowed so far
     if (lds_limit.raise(reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES>), smem) != hipSuccess) {
         (void)hipGetLastError();
@@ -530,7 +576,7 @@ int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
 }
 
 template <int C, int WAVES>
-int dispatch_ksx(int B, int K, int H, int Q, int L, int n16max,
+int dispatch_ksx(bool labels, int B, int K, int H, int Q, int L, int n16max,
                  const int* a_row_ptr, const int* a_col_idx, const float* a_val,
                  const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                  const float* X, const float* Wn2l, const float* Wc, const float* Wh1, const float* Wh2,
@@ -539,6 +585,7 @@ int dispatch_ksx(int B, int K, int H, int Q, int L, int n16max,
 {
 #define GNNHIP_GF_ARGS B, K, H, Q, L, n16max, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
                        X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, s
+    if (labels) return launch_graph_forward<C, 0, WAVES>(GNNHIP_GF_ARGS);
     if (K <= 16) return launch_graph_forward<C, 4, WAVES>(GNNHIP_GF_ARGS);
     if (K <= 32) return launch_graph_forward<C, 8, WAVES>(GNNHIP_GF_ARGS);
     if (K <= 48) return launch_graph_forward<C, 12, WAVES>(GNNHIP_GF_ARGS);
@@ -548,7 +595,7 @@ int dispatch_ksx(int B, int K, int H, int Q, int L, int n16max,
 }
 
 template <int C>
-int dispatch_waves(int B, int K, int H, int Q, int L, int n16max,
+int dispatch_waves(bool labels, int B, int K, int H, int Q, int L, int n16max,
                    const int* a_row_ptr, const int* a_col_idx, const float* a_val,
                    const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                    const float* X, const float* Wn2l, const float* Wc, const float* Wh1, const float* Wh2,
@@ -558,9 +605,9 @@ int dispatch_waves(int B, int K, int H, int Q, int L, int n16max,
 #define GNNHIP_GF_ARGS B, K, H, Q, L, n16max, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
                        X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, s
     const int tasks = (C / 16) * (n16max / 16);         // (column block x row tile) tasks of the largest graph
-    if (tasks <= 4) return dispatch_ksx<C, 4>(GNNHIP_GF_ARGS);
-    if (tasks <= 8) return dispatch_ksx<C, 8>(GNNHIP_GF_ARGS);
-    return dispatch_ksx<C, 16>(GNNHIP_GF_ARGS);
+    if (tasks <= 4) return dispatch_ksx<C, 4>(labels, GNNHIP_GF_ARGS);
+    if (tasks <= 8) return dispatch_ksx<C, 8>(labels, GNNHIP_GF_ARGS);
+    return dispatch_ksx<C, 16>(labels, GNNHIP_GF_ARGS);
 #undef GNNHIP_GF_ARGS
 }
 
@@ -568,6 +615,49 @@ int dispatch_waves(int B, int K, int H, int Q, int L, int n16max,
 }  // namespace gnnhip
 
 using namespace gnnhip;
+
+namespace {
+
+int forward_batched_entry(bool labels, int N, int B, int K, int C, int H, int Q, int L, int max_graph_nodes,
+                          const int* a_row_ptr, const int* a_col_idx, const float* a_val,
+                          const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                          const void* X, const float* W_n2l, const float* W_conv,
+                          const float* W_h1, const float* W_h2,
+                          float* msg, float* h_final, float* pool, float* hidden, float* logits,
+                          float* probs, int* pred, int* status, void* stream)
+{
+    GNNHIP_REQUIRE(N >= 1 && B >= 1 && K >= 1 && C >= 1 && H >= 1 && Q >= 1 && L >= 0 && max_graph_nodes >= 1,
+                   "bad shape in s2v_forward_batched (N=%d B=%d K=%d C=%d H=%d Q=%d L=%d max_graph_nodes=%d)",
+                   N, B, K, C, H, Q, L, max_graph_nodes);
+    GNNHIP_REQUIRE(a_row_ptr && a_col_idx && a_val && s_row_ptr && s_col_idx && s_val && X && W_n2l && W_conv && W_h1 && W_h2,
+                   "null input in s2v_forward_batched");
+    GNNHIP_REQUIRE(msg && h_final && pool && hidden && logits, "null output in s2v_forward_batched");
+    if (int rc = require_ready()) return rc;
+    if (!(C == 16 || C == 32 || C == 64) || (!labels && K > 64))
+        return set_error(GNNHIP_EUNSUPPORTED, "graph-resident forward supports hidden 16/32/64 and at most 64 dense feature columns (C=%d K=%d)", C, K);
+    if (!(aligned16(msg) && aligned16(h_final)))
+        return set_error(GNNHIP_EUNSUPPORTED, "msg and h_final must be 16-byte aligned");
+    if (labels && !aligned16(W_n2l))
+        return set_error(GNNHIP_EUNSUPPORTED, "W_n2l must be 16-byte aligned for the label input");
+    const int n16 = (max_graph_nodes + 15) / 16 * 16;
+    if (GraphLds::edge_cap(n16, C, K, H, Q, 256, labels) < 0)
+        return set_error(GNNHIP_EUNSUPPORTED, "a graph of %d nodes does not fit the 160 KB of LDS", max_graph_nodes);
+    hipStream_t s = as_stream(stream);
+    const float* Xf = static_cast<const float*>(X);
+    int rc;
+#define GNNHIP_GF_ARGS labels, B, K, H, Q, L, n16, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
+                       Xf, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, s
+    switch (C) {
+    case 16: rc = dispatch_waves<16>(GNNHIP_GF_ARGS); break;
+    case 32: rc = dispatch_waves<32>(GNNHIP_GF_ARGS); break;
+    default: rc = dispatch_waves<64>(GNNHIP_GF_ARGS); break;
+    }
+#undef GNNHIP_GF_ARGS
+    if (rc == GNNHIP_EUNSUPPORTED) return set_error(rc, "graph-resident forward could not be configured for this shape");
+    return rc;
+}
+
+}  // namespace
 
 extern "C" int gnnhip_s2v_forward_batched_f32(int N, int B, int K, int C, int H, int Q, int L, int max_graph_nodes,
                                               const int* a_row_ptr, const int* a_col_idx, const float* a_val,
@@ -577,30 +667,18 @@ extern "C" int gnnhip_s2v_forward_batched_f32(int N, int B, int K, int C, int H,
                                               float* msg, float* h_final, float* pool, float* hidden, float* logits,
                                               float* probs, int* pred, int* status, void* stream)
 {
-    GNNHIP_REQUIRE(N >= 1 && B >= 1 && K >= 1 && C >= 1 && H >= 1 && Q >= 1 && L >= 0 && max_graph_nodes >= 1,
-                   "bad shape in s2v_forward_batched (N=%d B=%d K=%d C=%d H=%d Q=%d L=%d max_graph_nodes=%d)",
-                   N, B, K, C, H, Q, L, max_graph_nodes);
-    GNNHIP_REQUIRE(a_row_ptr && a_col_idx && a_val && s_row_ptr && s_col_idx && s_val && X && W_n2l && W_conv && W_h1 && W_h2,
-                   "null input in s2v_forward_batched");
-    GNNHIP_REQUIRE(msg && h_final && pool && hidden && logits, "null output in s2v_forward_batched");
-    if (int rc = require_ready()) return rc;
-    if (!(C == 16 || C == 32 || C == 64) || K > 64)
-        return set_error(GNNHIP_EUNSUPPORTED, "graph-resident forward supports hidden 16/32/64 and at most 64 label types (C=%d K=%d)", C, K);
-    if (!(aligned16(msg) && aligned16(h_final)))
-        return set_error(GNNHIP_EUNSUPPORTED, "msg and h_final must be 16-byte aligned");
-    const int n16 = (max_graph_nodes + 15) / 16 * 16;
-    if (GraphLds::edge_cap(n16, C, K, H, Q, 256) < 0)
-        return set_error(GNNHIP_EUNSUPPORTED, "a graph of %d nodes does not fit the 160 KB of LDS", max_graph_nodes);
-    hipStream_t s = as_stream(stream);
-    int rc;
-#define GNNHIP_GF_ARGS B, K, H, Q, L, n16, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
-                       X, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, s
-    switch (C) {
-    case 16: rc = dispatch_waves<16>(GNNHIP_GF_ARGS); break;
-    case 32: rc = dispatch_waves<32>(GNNHIP_GF_ARGS); break;
-    default: rc = dispatch_waves<64>(GNNHIP_GF_ARGS); break;
-    }
-#undef GNNHIP_GF_ARGS
-    if (rc == GNNHIP_EUNSUPPORTED) return set_error(rc, "graph-resident forward could not be configured for this shape");
-    return rc;
+    return forward_batched_entry(false, N, B, K, C, H, Q, L, max_graph_nodes, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx,
+                                 s_val, X, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, stream);
+}
+
+extern "C" int gnnhip_s2v_forward_batched_labels_f32(int N, int B, int K, int C, int H, int Q, int L, int max_graph_nodes,
+                                                     const int* a_row_ptr, const int* a_col_idx, const float* a_val,
+                                                     const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                                                     const int* node_label, const float* W_n2l, const float* W_conv,
+                                                     const float* W_h1, const float* W_h2,
+                                                     float* msg, float* h_final, float* pool, float* hidden, float* logits,
+                                                     float* probs, int* pred, int* status, void* stream)
+{
+    return forward_batched_entry(true, N, B, K, C, H, Q, L, max_graph_nodes, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx,
+                                 s_val, node_label, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, stream);
 }

@@ -101,6 +101,17 @@ def s2v_input(X, W_n2l):
     return msg, h0
 
 
+def s2v_input_labels(label, W_n2l, status=None):
+    """msg = W_n2l[label], h0 = ReLU(msg): the input stage from one int label per node."""
+    N = label.numel()
+    K, C = W_n2l.shape
+    msg = torch.empty((N, C), dtype=torch.float32, device=W_n2l.device)
+    h0 = torch.empty_like(msg)
+    check(_lib().gnnhip_s2v_input_labels_f32(N, K, C, _i32(label, "label"), _f32(W_n2l, "W_n2l"), _f32(msg, "msg"),
+                                             _f32(h0, "h0"), _i32(status, "status"), _stream()))
+    return msg, h0
+
+
 def s2v_level(row_ptr, col_idx, val, h_in, W, msg=None, bias=None, out=None, nnz_hint=None):
     """nnz_hint: the host-side entry count handed to the library (default: the arrays' length); it only
     sizes scratch, so any value from 0 up must give the same result."""
@@ -215,6 +226,31 @@ def s2v_forward_batched(a_csr, s_csr, X, W_n2l, W_conv, W_h1, W_h2, L, max_graph
         _i32(a_csr[0], "a_row_ptr"), _i32(a_csr[1], "a_col_idx"), _f32(a_csr[2], "a_val"),
         _i32(s_csr[0], "s_row_ptr"), _i32(s_csr[1], "s_col_idx"), _f32(s_csr[2], "s_val"),
         _f32(X, "X"), _f32(W_n2l, "W_n2l"), _f32(W_conv, "W_conv"), _f32(W_h1, "W_h1"), _f32(W_h2, "W_h2"),
+        _f32(bufs.msg, "msg"), _f32(bufs.h_final, "h_final"), _f32(bufs.pool, "pool"),
+        _f32(bufs.hidden, "hidden"), _f32(bufs.logits, "logits"), _f32(bufs.probs, "probs"),
+        _i32(bufs.pred, "pred"), _i32(bufs.status, "status"), _stream()))
+    return bufs
+
+
+def s2v_forward_batched_labels(a_csr, s_csr, label, W_n2l, W_conv, W_h1, W_h2, L, max_graph_nodes, bufs=None):
+    """One-launch forward from one int label per node (see gnnhip_s2v_forward_batched_labels_f32)."""
+    N = label.numel()
+    K, C = W_n2l.shape
+    H, Q = W_h1.shape[1], W_h2.shape[1]
+    B = s_csr[0].numel() - 1
+    _check_csr(a_csr[0], a_csr[1], a_csr[2], N, "A")
+    _check_csr(s_csr[0], s_csr[1], s_csr[2], B, "S")
+    if s_csr[1].numel() != N:
+        raise ValueError("S must list every node exactly once")
+    if tuple(W_conv.shape) != (C, C) or W_h1.shape[0] != C or W_h2.shape[0] != H:
+        raise ValueError("weight shapes do not chain")
+    if bufs is None:
+        bufs = BatchedBuffers(N, B, C, H, Q, W_n2l.device)
+    check(_lib().gnnhip_s2v_forward_batched_labels_f32(
+        N, B, K, C, H, Q, L, int(max_graph_nodes),
+        _i32(a_csr[0], "a_row_ptr"), _i32(a_csr[1], "a_col_idx"), _f32(a_csr[2], "a_val"),
+        _i32(s_csr[0], "s_row_ptr"), _i32(s_csr[1], "s_col_idx"), _f32(s_csr[2], "s_val"),
+        _i32(label, "label"), _f32(W_n2l, "W_n2l"), _f32(W_conv, "W_conv"), _f32(W_h1, "W_h1"), _f32(W_h2, "W_h2"),
         _f32(bufs.msg, "msg"), _f32(bufs.h_final, "h_final"), _f32(bufs.pool, "pool"),
         _f32(bufs.hidden, "hidden"), _f32(bufs.logits, "logits"), _f32(bufs.probs, "probs"),
         _i32(bufs.pred, "pred"), _i32(bufs.status, "status"), _stream()))

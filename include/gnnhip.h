@@ -128,6 +128,14 @@ int gnnhip_s2v_level_f32(int N, int C, int nnz, const int* row_ptr, const int* c
 int gnnhip_s2v_input_f32(int N, int K, int C, const float* X, const float* W_n2l,
                          float* msg, float* h0, void* stream);
 
+/* ---- the same input stage when the node features are one label per node (what GetBatch encodes as the
+ *      one-hot rows of X, examples/graph_classification/include/nn_common.h:57-69): msg[i,:] = W_n2l[label[i],:],
+ *      bit-identical to X * W_n2l with X one-hot, and 4 N bytes of input instead of 4 N K.
+ *      node_label: device int[N] with values in [0, K).  msg or h0 may be NULL.  status (device int, may be NULL;
+ *      caller zeroes it) gets bit 3 set if a label lies outside [0, K); such a label is clamped. */
+int gnnhip_s2v_input_labels_f32(int N, int K, int C, const int* node_label, const float* W_n2l,
+                                float* msg, float* h0, int* status, void* stream);
+
 /* ---- readout: pool = S * h ; hidden = ReLU(pool * W_h1) ; logits = hidden * W_h2 ;
  *      probs = softmax(logits) ; pred = row argmax(logits)
  *      (examples/graph_classification/src/kernel_mean_field.cpp:44-49 and the softmax of
@@ -174,6 +182,19 @@ int gnnhip_s2v_forward_batched_f32(int N, int B, int K, int C, int H, int Q, int
                                    const float* W_h1, const float* W_h2,
                                    float* msg, float* h_final, float* pool, float* hidden, float* logits,
                                    float* probs, int* pred, int* status, void* stream);
+
+/* ---- the one-launch forward with one label per node in place of the one-hot matrix X (see
+ *      gnnhip_s2v_input_labels_f32; the batch layout is GetBatch's,
+ *      examples/graph_classification/include/nn_common.h:36-105): the input stage becomes a row lookup in W_n2l [K,C] (K is not limited to 64),
+ *      every output has the bits of gnnhip_s2v_forward_batched_f32 on the one-hot X.  status bit 3: a label
+ *      outside [0, K) (clamped).  W_n2l must be 16-byte aligned. */
+int gnnhip_s2v_forward_batched_labels_f32(int N, int B, int K, int C, int H, int Q, int L, int max_graph_nodes,
+                                          const int* a_row_ptr, const int* a_col_idx, const float* a_val,
+                                          const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                                          const int* node_label, const float* W_n2l, const float* W_conv,
+                                          const float* W_h1, const float* W_h2,
+                                          float* msg, float* h_final, float* pool, float* hidden, float* logits,
+                                          float* probs, int* pred, int* status, void* stream);
 
 /* ---- UnaryEngine<GPU>::Exec<Functor> (include/tensor/gpu_unary_functor.h:331-384):
  *      in-place x[i] = f(x[i]); a0/a1 are the functor's constructor arguments. */

@@ -965,6 +965,72 @@ def test_batched_forward_reports_broken_promises(gpu, oracle):
     assert err.value.code == -5
 
 
+# ------------------------------------------------------------------ label input (one int per node instead of one-hot X)
+@pytest.mark.parametrize("C,K,N", [(64, 38, 7450), (16, 7, 333), (128, 64, 5001), (256, 3, 1000), (48, 100, 777), (7, 5, 100)])
+def test_input_labels_is_the_one_hot_product_bit_for_bit(gpu, oracle, C, K, N):
+    import torch
+    from graphnn_amd import ops
+    rng = np.random.default_rng(C + K)
+    lab = rng.integers(0, K, N).astype(np.int32)
+    W = (rng.standard_normal((K, C)) * 0.1).astype(np.float32)
+    W[0, :3] = -0.0                                              # the product turns -0.0 into +0.0; so must the lookup
+    lab[:5] = 0
+    X = np.zeros((N, K), np.float32); X[np.arange(N), lab] = 1.0
+    want = oracle.gemm(X, W)
+    status = torch.zeros(1, dtype=torch.int32, device=gpu)
+    msg, h0 = ops.s2v_input_labels(_t(lab, gpu), _t(W, gpu), status)
+    assert np.array_equal(_n(msg).view(np.int32), want.view(np.int32))
+    assert np.array_equal(_n(h0).view(np.int32), np.maximum(want, 0).view(np.int32))
+    assert int(_n(status)[0]) == 0
+    # the dense input stage of the library gives the same bits
+    msg_d, h0_d = ops.s2v_input(_t(X, gpu), _t(W, gpu))
+    assert np.array_equal(_n(msg_d).view(np.int32), _n(msg).view(np.int32))
+    # a label outside [0, K) is reported and clamped
+    bad = lab.copy(); bad[7] = K; bad[8] = -3
+    msg_b, _ = ops.s2v_input_labels(_t(bad, gpu), _t(W, gpu), status)
+    assert int(_n(status)[0]) == 8
+    assert np.array_equal(_n(msg_b)[7], want[lab == K - 1][0] if (lab == K - 1).any() else _n(msg_b)[7])
+    assert np.array_equal(_n(msg_b)[8].view(np.int32), want[0].view(np.int32))
+
+
+@pytest.mark.parametrize("config_id", [1, 2])
+def test_batched_forward_from_labels_has_the_bits_of_the_one_hot_route(gpu, oracle, config_id):
+    from graphnn_amd import ops
+    batch, w, cfg = synth.make_config(config_id)
+    want, bufs = _batched_case(gpu, oracle, batch, w, cfg["L"])
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    lab = batch.node_label.astype(np.int32)
+    got = ops.s2v_forward_batched_labels(_csr_t(a, gpu), _csr_t(s, gpu), _t(lab, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+                                         _t(w.W_h1, gpu), _t(w.W_h2, gpu), cfg["L"], int(batch.graph_sizes.max()))
+    assert int(_n(got.status)[0]) == 0
+    for key in ("msg", "h_final", "pool", "hidden", "logits", "probs", "pred"):
+        assert np.array_equal(_n(getattr(got, key)), _n(getattr(bufs, key))), key
+    _assert_batched_matches(want, got, cfg["L"])
+
+
+@pytest.mark.parametrize("C,K,H,Q,L,B", [(16, 7, 8, 3, 2, 37), (32, 200, 16, 2, 3, 300), (64, 64, 32, 5, 1, 1025), (64, 1, 8, 2, 0, 9),
+                                         (64, 130, 32, 2, 2, 40)])
+def test_batched_forward_from_labels_shapes(gpu, oracle, C, K, H, Q, L, B):
+    """label tables that fit LDS (K C <= 8192 floats) and ones read from L2, more than 64 label types (the dense
+    route stops at 64 columns), no level, more graphs than workgroups; a label out of range sets status bit 3"""
+    from graphnn_amd import ops
+    seed = 2000 + C + K + L
+    batch = synth.molecule_batch(seed, B, K, Q, size_mode="uniform", size_lo=1, size_hi=70)
+    w = synth.make_weights(synth.Stream(seed), K, C, H, Q)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    want = _forward_want(oracle, a, s, batch.one_hot(), w, L)
+    lab = batch.node_label.astype(np.int32)
+    args = (_csr_t(a, gpu), _csr_t(s, gpu))
+    wts = (_t(w.W_n2l, gpu), _t(w.W_conv, gpu), _t(w.W_h1, gpu), _t(w.W_h2, gpu))
+    got = ops.s2v_forward_batched_labels(*args, _t(lab, gpu), *wts, L, int(batch.graph_sizes.max()))
+    _assert_batched_matches(want, got, L)
+    bad = lab.copy(); bad[batch.num_nodes // 2] = K + 5
+    got = ops.s2v_forward_batched_labels(*args, _t(bad, gpu), *wts, L, int(batch.graph_sizes.max()))
+    assert int(_n(got.status)[0]) == 8
+
+
 # ------------------------------------------------------------------ backward-pass kernels
 @pytest.mark.parametrize("n", [2, 7, 64, 128])
 def test_spmm_transposed(gpu, oracle, n):
