@@ -26,6 +26,7 @@ thread_local char g_err[512] = "";
 // and nothing waits for the device.  A half is reused only after the event recorded behind its last
 // copy has completed.
 constexpr size_t kStagingHalf = 2u << 20;
+constexpr size_t kReadbackBytes = 4096;
 struct Staging {
     char* base = nullptr;              // 2 * kStagingHalf bytes from hipHostMalloc
     hipEvent_t done[2] = {nullptr, nullptr};
@@ -46,6 +47,7 @@ struct Runtime {
     size_t n_driver_allocs = 0;
     std::map<std::pair<hipStream_t, int>, std::pair<void*, size_t>> scratch;   // library scratch per (stream, slot)
     std::map<hipStream_t, struct Staging> staging;  // pinned upload buffers per stream
+    std::map<hipStream_t, void*> readback;          // pinned landing buffer for small device-to-host reads, per stream
 };
 
 Runtime& rt()
@@ -204,6 +206,8 @@ int gnnhip_shutdown(void)
         for (hipEvent_t e : kv.second.done) if (e) (void)hipEventDestroy(e);
     }
     r.staging.clear();
+    for (auto& kv : r.readback) if (kv.second) (void)hipHostFree(kv.second);
+    r.readback.clear();
     r.all.clear();
     r.live.clear();
     r.parked.clear();
@@ -308,8 +312,31 @@ int gnnhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void
     if (bytes == 0) return GNNHIP_OK;
     GNNHIP_REQUIRE(dst_host && src_device, "null pointer in memcpy_d2h");
     if (int rc = require_ready()) return rc;
-    GNNHIP_HIP(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
-    GNNHIP_HIP(hipStreamSynchronize(as_stream(stream)));
+    hipStream_t s = as_stream(stream);
+    if (bytes <= kReadbackBytes) {
+        // small reads (scalars such as the loss) land in pinned memory: the copy is then a plain DMA that
+        // the stream wait covers, instead of the runtime's staged path for pageable destinations
+        Runtime& r = rt();
+        void* pin = nullptr;
+        {
+            std::lock_guard<std::mutex> lock(r.mu);
+            void*& slot = r.readback[s];
+            if (!slot && (hipHostMalloc(&slot, kReadbackBytes, hipHostMallocDefault) != hipSuccess || !slot)) {
+                (void)hipGetLastError();
+                slot = nullptr;
+            }
+            pin = slot;
+        }
+        if (pin) {
+            // one reader per stream at a time (the caller's thread owns the stream while it waits)
+            GNNHIP_HIP(hipMemcpyAsync(pin, src_device, bytes, hipMemcpyDeviceToHost, s));
+            GNNHIP_HIP(hipStreamSynchronize(s));
+            memcpy(dst_host, pin, bytes);
+            return GNNHIP_OK;
+        }
+    }
+    GNNHIP_HIP(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, s));
+    GNNHIP_HIP(hipStreamSynchronize(s));
     return GNNHIP_OK;
 }
 

@@ -51,6 +51,21 @@ protected:
 
 namespace detail
 {
+// val = 1, or 1 / row length when average is set (computed as the reference does: 1.0 / (double)size)
+template<typename Dtype>
+inline void fill_row_weights(const int* row_ptr, int rows, bool average, Dtype* val)
+{
+    if (!average) {
+        std::fill(val, val + row_ptr[rows], (Dtype)1.0);
+        return;
+    }
+    for (int i = 0; i < rows; ++i) {
+        const int len = row_ptr[i + 1] - row_ptr[i];
+        const Dtype weight = len ? (Dtype)(1.0 / (double)len) : (Dtype)1.0;
+        std::fill(val + row_ptr[i], val + row_ptr[i + 1], weight);
+    }
+}
+
 // CSR [num_rows, num_cols] on the device whose row y lists, in edge order, the tail x (payload_is_edge
 // false) or the index (true) of every edge x -> y: one copy of the (x, y) pairs, then a stable
 // grouping by y (gnnhip_csr_group_i32).
@@ -116,22 +131,13 @@ protected:
         w.Reshape({graph->num_nodes, graph->num_nodes});
         w.ResizeSp((int)graph->num_edges, (int)graph->num_nodes + 1);
         int* rp = w.data->row_ptr;
-        int* ci = w.data->col_idx;
-        Dtype* va = w.data->val;
-        int nnz = 0;
-        for (unsigned i = 0; i < graph->num_nodes; ++i) {
-            rp[i] = nnz;
-            const auto& in = graph->in_edges->head[i];
-            const Dtype weight = this->average ? (Dtype)(1.0 / (double)in.size()) : (Dtype)1.0;
-            for (size_t j = 0; j < in.size(); ++j) { ci[nnz] = in[j].second; va[nnz] = weight; ++nnz; }
-        }
-        rp[graph->num_nodes] = nnz;
-        ASSERT(nnz == (int)graph->num_edges, "edge count does not match the in-edge lists");
-        // does any edge join two subgraphs?  (node -> subgraph from the subgraph lists)
+        // rows from the flat edge list (stable by head node): the entries of in_edges->head[i], row after row
+        graph->GroupEdgesByHead(false, rp, w.data->col_idx);
+        detail::fill_row_weights(rp, (int)graph->num_nodes, this->average, w.data->val);
+        // does any edge join two subgraphs?  (node -> subgraph from the AddNode records)
         node_subgraph.assign(graph->num_nodes, -1);
-        for (unsigned g = 0; g < graph->num_subgraph; ++g)
-            for (int node : graph->subgraph->head[g])
-                if (node >= 0 && node < (int)graph->num_nodes) node_subgraph[node] = (int)g;
+        for (const auto& sn : graph->node_list)
+            if (sn.second >= 0 && sn.second < (int)graph->num_nodes) node_subgraph[sn.second] = sn.first;
         bool diagonal = true;
         for (const auto& e : graph->edge_list) diagonal = diagonal && node_subgraph[e.first] == node_subgraph[e.second];
         this->layout.block_diagonal = diagonal;
@@ -160,18 +166,8 @@ protected:
         auto& w = this->cpu_weight;
         w.Reshape({graph->num_nodes, graph->num_edges});
         w.ResizeSp((int)graph->num_edges, (int)graph->num_nodes + 1);
-        int* rp = w.data->row_ptr;
-        int* ci = w.data->col_idx;
-        Dtype* va = w.data->val;
-        int nnz = 0;
-        for (unsigned i = 0; i < graph->num_nodes; ++i) {
-            rp[i] = nnz;
-            const auto& in = graph->in_edges->head[i];
-            const Dtype weight = this->average ? (Dtype)(1.0 / (double)in.size()) : (Dtype)1.0;
-            for (size_t j = 0; j < in.size(); ++j) { ci[nnz] = in[j].first; va[nnz] = weight; ++nnz; }
-        }
-        rp[graph->num_nodes] = nnz;
-        ASSERT(nnz == (int)graph->num_edges, "edge count does not match the in-edge lists");
+        graph->GroupEdgesByHead(true, w.data->row_ptr, w.data->col_idx);
+        detail::fill_row_weights(w.data->row_ptr, (int)graph->num_nodes, this->average, w.data->val);
     }
 };
 
@@ -254,25 +250,15 @@ protected:
         auto& w = this->cpu_weight;
         w.Reshape({graph->num_subgraph, graph->num_nodes});
         w.ResizeSp((int)graph->num_nodes, (int)graph->num_subgraph + 1);
+        ASSERT(graph->node_list.size() == graph->num_nodes, "node count does not match the subgraph lists");
         int* rp = w.data->row_ptr;
         int* ci = w.data->col_idx;
-        Dtype* va = w.data->val;
-        int nnz = 0, biggest = 0;
+        graph->GroupNodesBySubgraph(rp, ci);
+        detail::fill_row_weights(rp, (int)graph->num_subgraph, this->average, w.data->val);
+        int biggest = 0;
         bool contiguous = true;
-        for (unsigned g = 0; g < graph->num_subgraph; ++g) {
-            rp[g] = nnz;
-            const auto& nodes = graph->subgraph->head[g];
-            const Dtype weight = this->average ? (Dtype)(1.0 / (double)nodes.size()) : (Dtype)1.0;
-            for (size_t j = 0; j < nodes.size(); ++j) {
-                contiguous = contiguous && nodes[j] == nnz;
-                ci[nnz] = nodes[j];
-                va[nnz] = weight;
-                ++nnz;
-            }
-            biggest = std::max(biggest, (int)nodes.size());
-        }
-        rp[graph->num_subgraph] = nnz;
-        ASSERT(nnz == (int)graph->num_nodes, "node count does not match the subgraph lists");
+        for (unsigned g = 0; g < graph->num_subgraph; ++g) biggest = std::max(biggest, rp[g + 1] - rp[g]);
+        for (int i = 0; i < (int)graph->num_nodes; ++i) contiguous = contiguous && ci[i] == i;
         this->layout.contiguous_subgraphs = contiguous;
         this->layout.max_subgraph_nodes = biggest;
     }

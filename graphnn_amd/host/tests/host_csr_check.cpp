@@ -38,6 +38,27 @@ int main(int argc, char** argv)
     for (int i = 0; i < N; ++i) g.AddNode(sid[i], nid[i]);
     for (int e = 0; e < E; ++e) g.AddEdge(e, ex[e], ey[e]);
 
+    // the per-node and per-subgraph lists, made on demand, hold what graphnn's AddEdge / AddNode would have
+    // appended (src/util/graph_struct.cpp:62-75): (edge, other end) per edge in edge order, nodes in AddNode order
+    {
+        std::vector<size_t> seen_out(N, 0), seen_in(N, 0), seen_sub(B, 0);
+        ASSERT(g.out_edges->n == N && g.in_edges->n == N && g.subgraph->n == B, "list counts");
+        for (int e = 0; e < E; ++e) {
+            auto& o = g.out_edges->head[ex[e]];
+            auto& in = g.in_edges->head[ey[e]];
+            ASSERT(seen_out[ex[e]] < o.size() && o[seen_out[ex[e]]] == std::make_pair(e, ey[e]), "out_edges differ at edge " << e);
+            ASSERT(seen_in[ey[e]] < in.size() && in[seen_in[ey[e]]] == std::make_pair(e, ex[e]), "in_edges differ at edge " << e);
+            seen_out[ex[e]]++; seen_in[ey[e]]++;
+        }
+        for (int i = 0; i < N; ++i) {
+            ASSERT(seen_out[i] == g.out_edges->head[i].size() && seen_in[i] == g.in_edges->head[i].size(), "stale list entries at node " << i);
+            auto& sg = g.subgraph->head[sid[i]];
+            ASSERT(seen_sub[sid[i]] < sg.size() && sg[seen_sub[sid[i]]] == nid[i], "subgraph list differs at node " << i);
+            seen_sub[sid[i]]++;
+        }
+        for (int b = 0; b < B; ++b) ASSERT(seen_sub[b] == g.subgraph->head[b].size(), "stale subgraph entries");
+    }
+
     FactorGraph fg;
     auto gv = add_const<GraphVar>(fg, "graph", true);
     auto a = af< Node2NodeMsgPass<CPU, float> >(fg, {gv}, average);
