@@ -444,3 +444,51 @@ def csr_transpose(row_ptr, col_idx, val, m, k):
     check(_lib().gnnhip_csr_transpose_f32(m, k, nnz, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"), _f32(val, "val"),
                                           _i32(t_rp, "t_row_ptr"), _i32(t_ci, "t_col_idx"), _f32(t_v, "t_val"), _stream()))
     return t_rp, t_ci, t_v
+
+
+# ---------------------------------------------------------------- training iteration
+def loss_acc(logits, lrow_ptr, lcol, lval, want_rows=False):
+    """mean cross-entropy (softmax inside) and mean top-1 accuracy of a batch in one pass over the logits"""
+    B, Q = logits.shape
+    dev = logits.device
+    probs = torch.empty_like(logits)
+    loss = torch.empty((1,), dtype=torch.float32, device=dev)
+    acc = torch.empty((1,), dtype=torch.float32, device=dev)
+    loss_rows = torch.empty((B,), dtype=torch.float32, device=dev) if want_rows else None
+    hit = torch.empty((B,), dtype=torch.int32, device=dev) if want_rows else None
+    check(_lib().gnnhip_s2v_loss_acc_f32(B, Q, _f32(logits, "logits"), _i32(lrow_ptr, "lrow_ptr"), _i32(lcol, "lcol"),
+                                         _f32(lval, "lval"), _f32(probs, "probs"), _f32(loss_rows, "loss_rows"),
+                                         _i32(hit, "hit"), _f32(loss, "loss"), _f32(acc, "acc"), _stream()))
+    return loss, acc, probs, loss_rows, hit
+
+
+def readout_backward(s_csr, probs, label_csr, scale, hidden, W_h1, W_h2, N):
+    B, Q = probs.shape
+    C, H = W_h1.shape
+    dev = probs.device
+    dlogits = torch.empty((B, Q), dtype=torch.float32, device=dev)
+    du = torch.empty((B, H), dtype=torch.float32, device=dev)
+    g_h = torch.empty((N, C), dtype=torch.float32, device=dev)
+    check(_lib().gnnhip_s2v_readout_backward_f32(
+        B, N, C, H, Q, _i32(s_csr[0], "s_row_ptr"), _i32(s_csr[1], "s_col_idx"), _f32(s_csr[2], "s_val"),
+        _f32(probs, "probs"), _i32(label_csr[0], "lrow_ptr"), _i32(label_csr[1], "lcol"), _f32(label_csr[2], "lval"),
+        float(scale), _f32(hidden, "hidden"), _f32(W_h1, "W_h1"), _f32(W_h2, "W_h2"),
+        _f32(dlogits, "dlogits"), _f32(du, "du"), _f32(g_h, "g_h"), _stream()))
+    return dlogits, du, g_h
+
+
+def grad_gate(h, g, dz=None, acc=None, accumulate=False):
+    check(_lib().gnnhip_s2v_grad_gate_f32(h.numel(), _f32(h, "h"), _f32(g, "g"), _f32(dz, "dz"), _f32(acc, "acc"),
+                                          1 if accumulate else 0, _stream()))
+
+
+def momentum_sgd_batch(ws, gs, vs, lr, momentum, l2):
+    n = len(ws)
+    P = ctypes.c_void_p * n
+    Z = ctypes.c_size_t * n
+    wp, gp = P(*[t.data_ptr() for t in ws]), P(*[t.data_ptr() for t in gs])
+    vp = P(*[t.data_ptr() for t in vs]) if vs is not None else None
+    for t in list(ws) + list(gs) + (list(vs) if vs is not None else []):
+        _f32(t, "tensor")
+    cnt = Z(*[t.numel() for t in ws])
+    check(_lib().gnnhip_momentum_sgd_batch_f32(n, wp, gp, vp, cnt, float(lr), float(momentum), float(l2), _stream()))

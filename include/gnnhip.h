@@ -290,6 +290,44 @@ int gnnhip_mul_f32(size_t n, const float* x, float* y, void* stream);
  *      (BCastEleWiseMulKernel, src/tensor/gpu_dense_tensor.cu:654-713) */
 int gnnhip_row_scale_f32(int rows, int cols, const float* scale, float* y, void* stream);
 
+/* ================= one training iteration in few launches ================= */
+
+/* ---- loss and accuracy of a batch from its logits in one pass: the rows of
+ *      CrossEntropy::Forward with softmax inside (src/nn/cross_entropy.cpp:33-50: DTensor::Softmax, then
+ *      CalcCrossEntropy with the clamp of :18-19), their mean (ReduceMean, src/nn/reduce_mean.cpp:14-42),
+ *      truth = SpTensor::ArgMax of the label rows (src/tensor/cpu_sparse_tensor.cpp:86-103), hit = IsInTopK with
+ *      k = 1 (src/nn/in_top_k.cpp:6-23), its mean after TypeCast: what
+ *      examples/graph_classification/src/kernel_mean_field.cpp:51-56 appends to the forward.
+ *      logits [B,Q]; labels CSR [B,Q]; probs [B,Q], loss_rows [B], hit_rows int[B] may be NULL;
+ *      loss_mean / acc_mean are device floats (one of them may be NULL). */
+int gnnhip_s2v_loss_acc_f32(int B, int Q, const float* logits, const int* lrow_ptr, const int* lcol, const float* lval,
+                            float* probs, float* loss_rows, int* hit_rows, float* loss_mean, float* acc_mean, void* stream);
+
+/* ---- backward of the readout for a batch whose pooling matrix S lists every node exactly once:
+ *      dlogits = scale * (probs - y)                       CrossEntropy::Backward (src/nn/cross_entropy.cpp:52-78),
+ *                                                          scale = 1/B from ReduceMean::Backward (src/nn/reduce_mean.cpp:44-65)
+ *      du = (dlogits * W_h2^T) . [hidden > 0]              MatMul::Backward + ReLUDeriv (src/nn/matmul.cpp:35-76, src/nn/relu.cu:18-37)
+ *      g_h[node,:] = s_val * (du * W_h1^T)[graph of node]  MatMul::Backward of pool = S * h
+ *      dlogits [B,Q], du [B,H] and g_h [N,C] are overwritten; the weight gradients are hidden^T * dlogits and
+ *      pool^T * du (gnnhip_gemm_f32). */
+int gnnhip_s2v_readout_backward_f32(int B, int N, int C, int H, int Q,
+                                    const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                                    const float* probs, const int* lrow_ptr, const int* lcol, const float* lval, float scale,
+                                    const float* hidden, const float* W_h1, const float* W_h2,
+                                    float* dlogits, float* du, float* g_h, void* stream);
+
+/* ---- dz = g where h > 0, else 0 (ReLUDeriv, src/nn/relu.cu:18-37), and acc = dz or acc += dz (the gradient that
+ *      ElewiseAdd::Backward passes on to msg, src/nn/elewise_add.cpp:35-52, summed over the levels).
+ *      dz may alias g; dz or acc may be NULL. */
+int gnnhip_s2v_grad_gate_f32(size_t n, const float* h, const float* g, float* dz, float* acc, int accumulate, void* stream);
+
+/* ---- MomentumSGDOptimizer::Update over n tensors in one launch (src/nn/optimizer.cpp:69-92):
+ *      momentum > 0:  g += l2 w ; v = lr g + momentum v ; w -= v ; g = 0      (v: the optimizer's acc_grad_dict)
+ *      momentum == 0: w = -lr g + (1 - lr l2) w ; g = 0                        (v may be NULL)
+ *      w, g, v: host arrays of n device pointers; count: host array of element counts. */
+int gnnhip_momentum_sgd_batch_f32(int n, float* const* w, float* const* g, float* const* v, const size_t* count,
+                                  float lr, float momentum, float l2, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

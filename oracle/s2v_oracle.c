@@ -341,6 +341,22 @@ void orc_jagged_softmax_deriv(float* dst, const float* out, const float* grad, c
     }
 }
 
+/* One MomentumSGDOptimizer::Update on one tensor (src/nn/optimizer.cpp:69-92), as the calls it makes:
+ * grad.RowSparseAxpy(l2, value); acc.RowSparseAxpby(lr, grad, momentum); value.Axpy(-1, acc); grad.RowSpZeros()
+ * (full gradients: the row-sparse forms are the dense axpy / axpby); momentum == 0 takes the plain SGD branch
+ * value.RowSparseAxpby(-lr, grad, 1 - lr * l2). */
+void orc_momentum_sgd(size_t n, float* w, float* g, float* v, float lr, float momentum, float l2)
+{
+    if (momentum > 0.0f) {
+        orc_axpy(n, l2, w, g);
+        orc_axpby(n, lr, g, momentum, v);
+        orc_axpy(n, -1.0f, v, w);
+    } else {
+        orc_axpby(n, -lr, g, 1 - lr * l2, w);
+    }
+    for (size_t i = 0; i < n; ++i) g[i] = 0.0f;
+}
+
 /* Global sum / mean: sequential fp32 accumulation, mean = s / cnt
  * (src/tensor/cpu_dense_tensor.cpp:269-295). */
 float orc_sum(const float* x, size_t n)

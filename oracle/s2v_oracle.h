@@ -40,6 +40,7 @@ void orc_axpby(size_t n, float a, const float* x, float b, float* y);
 void orc_unary(int op, float* x, size_t n, float a0, float a1);
 void orc_row_softmax(float* x, int rows, int cols);
 void orc_jagged_softmax(float* x, const int* lens, int nseg);
+void orc_momentum_sgd(size_t n, float* w, float* g, float* v, float lr, float momentum, float l2);
 void orc_jagged_softmax_deriv(float* dst, const float* out, const float* grad, const int* lens, int nseg);
 float orc_sum(const float* x, size_t n);
 float orc_mean(const float* x, size_t n);

@@ -135,6 +135,13 @@ class Oracle:
         self.lib.orc_jagged_softmax_deriv(_ptr(dst), _ptr(out), _ptr(grad), _ptr(lens), len(lens))
         return dst
 
+    def momentum_sgd(self, w, g, v, lr, momentum, l2):
+        """one update; returns the new (w, g, v)"""
+        w, g, v = (np.array(a, np.float32, copy=True) for a in (w, g, v))
+        self.lib.orc_momentum_sgd(ctypes.c_size_t(w.size), _ptr(w), _ptr(g), _ptr(v), ctypes.c_float(lr),
+                                  ctypes.c_float(momentum), ctypes.c_float(l2))
+        return w, g, v
+
     def sum(self, x):
         x = np.ascontiguousarray(x, np.float32)
         return float(self.lib.orc_sum(_ptr(x), ctypes.c_size_t(x.size)))

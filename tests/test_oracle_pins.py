@@ -356,6 +356,31 @@ def test_jagged_softmax_gradient_is_the_softmax_jacobian(oracle):
     assert np.allclose(got - d0, num, atol=1e-4)
 
 
+def test_momentum_sgd_two_steps_closed_form(oracle):
+    """two consecutive updates with l2 != 0 and momentum 0.9 against the recurrence written out in float64
+    (g' = g + l2 w; v' = lr g' + m v; w' = w - v'; src/nn/optimizer.cpp:69-92), the velocity starting at
+    zero, and the plain-SGD branch for momentum 0.  (ClipGradients is not part of this optimizer: only
+    AdamOptimizer::Update calls it, src/nn/optimizer.cpp:108.)"""
+    rng = _rng(31)
+    lr, m, l2 = 0.05, 0.9, 0.01
+    w0 = rng.standard_normal(1000).astype(np.float32)
+    g1 = rng.standard_normal(1000).astype(np.float32)
+    g2 = rng.standard_normal(1000).astype(np.float32)
+    w, g, v = oracle.momentum_sgd(w0, g1, np.zeros_like(w0), lr, m, l2)
+    assert not g.any()
+    w, g, v = oracle.momentum_sgd(w, g2, v, lr, m, l2)
+    W0, G1, G2 = (a.astype(np.float64) for a in (w0, g1, g2))
+    V1 = lr * (G1 + l2 * W0)
+    W1 = W0 - V1
+    V2 = lr * (G2 + l2 * W1) + m * V1
+    W2 = W1 - V2
+    assert np.allclose(v, V2, rtol=1e-5, atol=1e-7) and np.allclose(w, W2, rtol=1e-5, atol=1e-6)
+    # the step is not a plain SGD step: the second update moves further along g1 than lr alone would
+    assert not np.allclose(w, W1 - lr * (G2 + l2 * W1), atol=1e-3)
+    w_sgd, g_sgd, _ = oracle.momentum_sgd(w0, g1, np.zeros_like(w0), lr, 0.0, l2)
+    assert np.allclose(w_sgd, (1 - lr * l2) * W0 - lr * G1, rtol=1e-5, atol=1e-6) and not g_sgd.any()
+
+
 def test_reductions(oracle):
     ints = np.arange(1, 1001, dtype=np.float32)
     assert oracle.sum(ints) == 500500.0 and oracle.mean(ints) == 500.5 and oracle.max(ints) == 1000.0
