@@ -27,6 +27,7 @@ public:
             in->template Derived<matType>().value.ArgMax(out, axis);
         });
     }
+    virtual const char* FuseKind() const override { return axis == 0 ? "arg_max" : ""; }
     uint axis;
 };
 

@@ -62,6 +62,11 @@ public:
         g_lhs.Axpy(1.0, probs);
     }
 
+    // the inference and training plans fold CrossEntropy(softmax inside) -> ReduceMean into one launch
+    virtual const char* FuseKind() const override { return need_softmax ? "cross_entropy_softmax" : ""; }
+    // the probabilities of the last forward (Backward reads them); the fused loss tail writes them here
+    virtual void* FusePayload() override { return &probs; }
+
     bool need_softmax;
 protected:
     DTensor<mode, Dtype> probs;

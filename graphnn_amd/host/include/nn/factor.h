@@ -35,6 +35,8 @@ public:
 
     // tag used by the inference-time fusion pass of FactorGraph; "" = never fused
     virtual const char* FuseKind() const { return ""; }
+    // a tensor the fused plans fill on the factor's behalf (CrossEntropy: its probabilities), or null
+    virtual void* FusePayload() { return nullptr; }
     // layout facts of the last batch, for factors that build batch operands (null otherwise)
     virtual const BatchLayout* Layout() const { return nullptr; }
 

@@ -156,7 +156,10 @@ protected:
     Plan* GetPlan(const std::vector<VarPtr>& targets, const std::map<std::string, void*>& feed_dict, Phase phase);
     void BuildPlan(Plan& plan);
     void BuildFusedSteps(Plan& plan);      // nn/s2v_fusion.h
+    void BuildSteps(Plan& plan, bool fold);
     void FoldWholeForward(Plan& plan);     // nn/s2v_fusion.h
+    void FoldLossTail(Plan& plan);         // nn/s2v_fusion.h
+    std::shared_ptr<detail::FusedStep> MakeSingleStep(size_t f);
 
     std::vector<size_t> always_ready;       // params and non-placeholder constants
     std::vector< std::unique_ptr<Plan> > plans;

@@ -32,6 +32,7 @@ public:
         IsInTopK(detail::dense_var<mode, Dtype>(operands[0], "InTopK").value, detail::dense_var<mode, int>(operands[1], "InTopK").value,
                  detail::dense_var<mode, int>(outputs[0], "InTopK").value, topK);
     }
+    virtual const char* FuseKind() const override { return topK == 1 ? "in_top_1" : ""; }
     int topK;
 };
 

@@ -4,6 +4,7 @@
 #define OPTIMIZER_H
 
 #include <cmath>
+#include <vector>
 #include "nn/param_set.h"
 
 namespace gnn
@@ -58,6 +59,45 @@ public:
     }
 };
 
+namespace detail
+{
+// Every tensor of the parameter set updated by one launch (device, full gradients); false where that route
+// does not apply and the caller updates tensor by tensor.
+template<typename mode, typename Dtype>
+struct BatchedMomentumUpdate
+{
+    static bool Run(ParamSet<mode, Dtype>*, std::map<std::string, std::shared_ptr< DTensor<mode, Dtype> > >&, Dtype, Dtype, Dtype) { return false; }
+};
+template<>
+struct BatchedMomentumUpdate<GPU, float>
+{
+    static bool Run(ParamSet<GPU, float>* set, std::map<std::string, std::shared_ptr< DTensor<GPU, float> > >& velocity,
+                    float lr, float momentum, float l2)
+    {
+        std::vector<float*> w, g, v;
+        std::vector<size_t> count;
+        for (auto& kv : set->params) {
+            auto& p = kv.second;
+            if (!p->grad.is_full || !(p->grad.shape == p->value.shape)) return false;
+            if (momentum > 0) {
+                auto& vel = velocity[kv.first];
+                if (!vel) {
+                    vel = std::make_shared< DTensor<GPU, float> >(p->grad.shape);
+                    vel->Zeros();
+                }
+                v.push_back(vel->data->ptr);
+            }
+            w.push_back(p->value.data->ptr);
+            g.push_back(p->grad.data->ptr);
+            count.push_back(p->value.shape.Count());
+        }
+        GNN_HIP(gnnhip_momentum_sgd_batch_f32((int)w.size(), w.data(), g.data(), momentum > 0 ? v.data() : nullptr, count.data(),
+                                              lr, momentum, l2, GpuHandle::Stream()));
+        return true;
+    }
+};
+}  // namespace detail
+
 template<typename mode, typename Dtype>
 class MomentumSGDOptimizer : public IOptimizer<mode, Dtype>
 {
@@ -68,6 +108,7 @@ public:
     // g <- g + l2 * w ;  v <- momentum * v + lr * g ;  w <- w - v     (plain SGD when momentum == 0)
     virtual void Update() override
     {
+        if (detail::BatchedMomentumUpdate<mode, Dtype>::Run(this->param_set, acc_grad_dict, this->cur_lr, momentum, this->l2_penalty)) return;
         for (auto& kv : this->param_set->params) {
             auto& p = kv.second;
             auto g = p->grad.Full();

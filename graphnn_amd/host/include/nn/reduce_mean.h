@@ -32,6 +32,7 @@ public:
         auto g_in = detail::dense_var<mode, Dtype>(operands[0], "ReduceMean").grad.Full();
         g_in.Add(g_out.AsScalar() / (Dtype)g_in.shape.Count());
     }
+    virtual const char* FuseKind() const override { return (axis == -1 && !keep_dim) ? "reduce_mean" : ""; }
     int axis;
     bool keep_dim;
 };

@@ -23,14 +23,29 @@ namespace gnn
 
 namespace detail
 {
+// What the folded forward of a training plan keeps for its backward pass.
+struct TrainState
+{
+    DTensor<GPU, float> hstack;             // [(L + 1) N, C]: the embeddings of every level, h0 first
+    DTensor<GPU, float> ustack;             // [L N, C]: A^T dz of every level
+    DTensor<GPU, float> g, dmsg, dl, du;    // [N, C], [N, C], [B, Q], [B, H]
+    DTensor<GPU, float>* probs = nullptr;   // the CrossEntropy factor's probabilities (filled by the loss tail)
+    SpTensorVar<GPU, float>* label = nullptr;
+    size_t loss_var = (size_t)-1;           // the variable BackPropagate must start from
+    bool loss_attached = false;             // a folded loss tail reads this forward's logits
+    bool fused_ran = false;                 // the last forward took the folded route (else the factors ran one by one)
+};
+
 struct FusedStep
 {
     std::vector<size_t> factors;            // graph factors this step stands for
     std::function<void(Phase)> run;
     bool fused;
-    enum Tag { SINGLE, INPUT, LEVEL, FORWARD } tag = SINGLE;
-    std::vector<size_t> vars;               // INPUT: X, W, msg, h0;  LEVEL: A, h_in, W, msg, h_out
+    enum Tag { SINGLE, INPUT, LEVEL, FORWARD, LOSS } tag = SINGLE;
+    std::vector<size_t> vars;               // INPUT: X, W, msg, h0;  LEVEL: A, h_in, W, msg, h_out;  FORWARD: logits
     bool bias_row = false;                  // LEVEL through FullyConnected: W may carry a bias row
+    std::shared_ptr<TrainState> train;      // FORWARD of a training plan
+    std::function<void()> backward;         // FORWARD of a training plan: gradients of the four weight matrices
 };
 constexpr size_t kOneLaunchMaxNodes = 20000;   // larger batches run the forward as separate kernels
 }  // namespace detail
@@ -117,7 +132,45 @@ inline void FactorGraph::BuildPlan(Plan& plan)
     BuildFusedSteps(plan);
 }
 
+inline std::shared_ptr<detail::FusedStep> FactorGraph::MakeSingleStep(size_t f)
+{
+    auto step = std::make_shared<detail::FusedStep>();
+    step->factors.push_back(f);
+    step->fused = false;
+    auto fac = factor_list[f];
+    auto ins = std::make_shared<VarList>();
+    auto outs = std::make_shared<VarList>();
+    for (size_t v : factor_nodes[f].in) ins->push_back(var_list[v]);
+    for (size_t v : factor_nodes[f].out) outs->push_back(var_list[v]);
+    step->run = [fac, ins, outs](Phase ph) { fac->Forward(*ins, *outs, ph); };
+    return step;
+}
+
+// Inference plans fold whatever chain they recognise.  A training plan folds only what still lets
+// BackPropagate work: the loss tail (it leaves behind what the factors' Backward read), and the whole forward
+// when the loss tail hangs off its logits (the folded forward then brings its own backward pass).
 inline void FactorGraph::BuildFusedSteps(Plan& plan)
+{
+    if (plan.phase == Phase::TEST) {
+        BuildSteps(plan, fusion_enabled);
+        if (fusion_enabled) { FoldWholeForward(plan); FoldLossTail(plan); }
+        return;
+    }
+    if (fusion_enabled) {
+        BuildSteps(plan, true);
+        FoldWholeForward(plan);
+        FoldLossTail(plan);
+        bool ok = true;
+        for (auto& st : plan.steps)
+            if (st->fused && st->tag != detail::FusedStep::LOSS &&
+                !(st->tag == detail::FusedStep::FORWARD && st->train && st->train->loss_attached)) ok = false;
+        if (ok) return;
+    }
+    BuildSteps(plan, false);
+    if (fusion_enabled) FoldLossTail(plan);
+}
+
+inline void FactorGraph::BuildSteps(Plan& plan, bool fold)
 {
     typedef DTensorVar<GPU, float> DVar;
     typedef SpTensorVar<GPU, float> SVar;
@@ -138,25 +191,13 @@ inline void FactorGraph::BuildFusedSteps(Plan& plan)
     };
     auto gpu_dense = [&](size_t v) { return dynamic_cast<DVar*>(var_list[v].get()); };
     auto gpu_sparse = [&](size_t v) { return dynamic_cast<SVar*>(var_list[v].get()); };
-    auto single_step = [&](size_t f) {
-        auto step = std::make_shared<detail::FusedStep>();
-        step->factors.push_back(f);
-        step->fused = false;
-        auto fac = factor_list[f];
-        auto ins = std::make_shared<VarList>();
-        auto outs = std::make_shared<VarList>();
-        for (size_t v : factor_nodes[f].in) ins->push_back(var_list[v]);
-        for (size_t v : factor_nodes[f].out) outs->push_back(var_list[v]);
-        step->run = [fac, ins, outs](Phase ph) { fac->Forward(*ins, *outs, ph); };
-        return step;
-    };
+    auto single_step = [&](size_t f) { return MakeSingleStep(f); };
 
     // A folded chain runs where its LAST factor stood in the order: only there are the operands of all
     // of its factors ready (msg and W enter the level at its second and third factor, and their
     // producers may sit anywhere before those, e.g. behind the sparse product when msg comes out of a
     // deeper chain than h_in does).
     std::vector< std::shared_ptr<detail::FusedStep> > emit_at(factor_list.size());
-    const bool fold = fusion_enabled && plan.phase == Phase::TEST;
     for (size_t f1 : plan.order) {
         if (taken[f1]) {
             if (emit_at[f1]) plan.steps.push_back(emit_at[f1]);
@@ -239,7 +280,6 @@ inline void FactorGraph::BuildFusedSteps(Plan& plan)
             plan.steps.push_back(single_step(f1));
         }
     }
-    if (fold) FoldWholeForward(plan);
 }
 
 // Second pass over the steps: input + a chain of levels with one A and one W + the readout
@@ -354,6 +394,104 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
              *Hl = dense(cur), *Pool = dense(vPool), *Hid = dense(vHid), *Logits = dense(vLogits);
         SVar *A = sparse(vA), *S = sparse(vS);
         DVar* H0 = dense(vH0);                           // h0: the second embedding buffer of the general route
+        step->vars = {vLogits};
+        if (plan.phase == Phase::TRAIN) {
+            // ---- training: every level's embedding is kept (stacked), and the step carries its backward pass.
+            // The factors it stands for, one by one and in plan order, are the fallback for batches the folded
+            // route does not take; BackPropagate then walks them as usual.
+            std::vector<size_t> pos(factor_list.size(), 0);
+            for (size_t i = 0; i < plan.order.size(); ++i) pos[plan.order[i]] = i;
+            std::vector<size_t> fs_sorted = step->factors;
+            std::sort(fs_sorted.begin(), fs_sorted.end(), [&](size_t x, size_t y) { return pos[x] < pos[y]; });
+            std::vector< std::shared_ptr<Step> > singles;
+            for (size_t f : fs_sorted) singles.push_back(MakeSingleStep(f));
+            auto st = std::make_shared<detail::TrainState>();
+            step->train = st;
+            const bool cWn = isConst[vWn], cWc = isConst[vWc], cW1 = isConst[vW1], cW2 = isConst[vW2];
+            step->run = [=](Phase ph) {
+                const size_t N = X->value.rows(), K = X->value.cols(), C = Wn->value.cols(), H = W1->value.cols(),
+                             Q = W2->value.cols(), B = S->value.rows();
+                ASSERT(Wn->value.rows() == K && Wc->value.rows() == C && Wc->value.cols() == C && W1->value.rows() == C &&
+                       W2->value.rows() == H && A->value.rows() == N && A->value.cols() == N && S->value.cols() == N,
+                       "fused forward: operand shapes do not chain");
+                // the folded backward needs S to list every node once and the per-graph LDS of its readout kernel
+                st->fused_ran = st->loss_attached && sub->contiguous_subgraphs && (Q + H + C) * 16 <= 64 * 1024;
+                if (!st->fused_ran) {
+                    for (auto& p : singles) p->run(ph);
+                    return;
+                }
+                void* s = GpuHandle::Stream();
+                const size_t NC = N * C;
+                st->hstack.Reshape({(size_t)(L + 1) * N, C});
+                Msg->value.Reshape({N, C});
+                Pool->value.Reshape({B, C});
+                Hid->value.Reshape({B, H});
+                Logits->value.Reshape({B, Q});
+                float* hs = st->hstack.data->ptr;
+                GNN_HIP(gnnhip_s2v_input_f32((int)N, (int)K, (int)C, X->value.data->ptr, Wn->value.data->ptr, Msg->value.data->ptr, hs, s));
+                for (int l = 0; l < L; ++l)
+                    GNN_HIP(gnnhip_s2v_level_f32((int)N, (int)C, A->value.data->nnz, A->value.data->row_ptr, A->value.data->col_idx,
+                                                 A->value.data->val, hs + (size_t)l * NC, Wc->value.data->ptr, Msg->value.data->ptr,
+                                                 nullptr, hs + (size_t)(l + 1) * NC, s));
+                GNN_HIP(gnnhip_s2v_readout_f32((int)B, (int)N, (int)C, (int)H, (int)Q, S->value.data->row_ptr, S->value.data->col_idx,
+                                               S->value.data->val, hs + (size_t)L * NC, W1->value.data->ptr, W2->value.data->ptr,
+                                               Pool->value.data->ptr, Hid->value.data->ptr, Logits->value.data->ptr, nullptr, nullptr, s));
+            };
+            // Backward of the folded forward (the gradient rules of src/nn/matmul.cpp:35-76, src/nn/relu.cu:18-37,
+            // src/nn/elewise_add.cpp:35-52, src/nn/cross_entropy.cpp:52-78 and src/nn/reduce_mean.cpp:44-65 composed):
+            //   g_L = S^T ((dlogits W2^T . [hidden > 0]) W1^T),  dlogits = (probs - y) / B
+            //   level l = L..1:  dz = g_l . [h_l > 0];  dmsg += dz;  u_l = A^T dz;  g_{l-1} = u_l W^T
+            //   dmsg += g_0 . [h_0 > 0]
+            //   dW_conv += [h_0; ..; h_{L-1}]^T [u_1; ..; u_L],  dW_n2l += X^T dmsg,  dW_h1 += pool^T du,  dW_h2 += hidden^T dlogits
+            // (A^T dz_l serves both the gradient of W, h_{l-1}^T (A^T dz_l) = (A h_{l-1})^T dz_l, and g_{l-1}.)
+            step->backward = [=]() {
+                ASSERT(st->fused_ran && st->probs && st->label, "folded backward without a folded forward");
+                const size_t N = X->value.rows(), K = X->value.cols(), C = Wn->value.cols(), H = W1->value.cols(),
+                             Q = W2->value.cols(), B = S->value.rows();
+                const size_t NC = N * C;
+                void* s = GpuHandle::Stream();
+                st->g.Reshape({N, C});
+                st->dmsg.Reshape({N, C});
+                st->dl.Reshape({B, Q});
+                st->du.Reshape({B, H});
+                if (L > 0) st->ustack.Reshape({(size_t)L * N, C});
+                auto& lab = st->label->value;
+                GNN_HIP(gnnhip_s2v_readout_backward_f32((int)B, (int)N, (int)C, (int)H, (int)Q, S->value.data->row_ptr,
+                                                        S->value.data->col_idx, S->value.data->val, st->probs->data->ptr,
+                                                        lab.data->row_ptr, lab.data->col_idx, lab.data->val, 1.0f / (float)B,
+                                                        Hid->value.data->ptr, W1->value.data->ptr, W2->value.data->ptr,
+                                                        st->dl.data->ptr, st->du.data->ptr, st->g.data->ptr, s));
+                float* hs = st->hstack.data->ptr;
+                float* g = st->g.data->ptr;
+                float* dmsg = st->dmsg.data->ptr;
+                if (L > 0) {
+                    auto& at = A->value.Transposed();
+                    float* us = st->ustack.data->ptr;
+                    for (int l = L; l >= 1; --l) {
+                        GNN_HIP(gnnhip_s2v_grad_gate_f32(NC, hs + (size_t)l * NC, g, g, dmsg, l < L ? 1 : 0, s));
+                        float* u = us + (size_t)(l - 1) * NC;
+                        GNN_HIP(gnnhip_spmm_csr_f32((int)N, (int)N, (int)C, at.nnz, 1.0f, at.row_ptr, at.col_idx, at.val, g, (int)C,
+                                                    0.0f, u, (int)C, s));
+                        GNN_HIP(gnnhip_gemm_f32(0, 1, (int)N, (int)C, (int)C, 1.0f, u, (int)C, Wc->value.data->ptr, (int)C, 0.0f, g, (int)C, s));
+                    }
+                    GNN_HIP(gnnhip_s2v_grad_gate_f32(NC, hs, g, nullptr, dmsg, 1, s));
+                    if (!cWc)
+                        GNN_HIP(gnnhip_gemm_f32(1, 0, (int)C, (int)C, (int)((size_t)L * N), 1.0f, hs, (int)C, us, (int)C, 1.0f,
+                                                Wc->grad.Full().data->ptr, (int)C, s));
+                } else {
+                    GNN_HIP(gnnhip_s2v_grad_gate_f32(NC, hs, g, nullptr, dmsg, 0, s));
+                }
+                if (!cWn)
+                    GNN_HIP(gnnhip_gemm_f32(1, 0, (int)K, (int)C, (int)N, 1.0f, X->value.data->ptr, (int)K, dmsg, (int)C, 1.0f,
+                                            Wn->grad.Full().data->ptr, (int)C, s));
+                if (!cW1)
+                    GNN_HIP(gnnhip_gemm_f32(1, 0, (int)C, (int)H, (int)B, 1.0f, Pool->value.data->ptr, (int)C, st->du.data->ptr, (int)H, 1.0f,
+                                            W1->grad.Full().data->ptr, (int)H, s));
+                if (!cW2)
+                    GNN_HIP(gnnhip_gemm_f32(1, 0, (int)H, (int)Q, (int)B, 1.0f, Hid->value.data->ptr, (int)H, st->dl.data->ptr, (int)Q, 1.0f,
+                                            W2->grad.Full().data->ptr, (int)Q, s));
+            };
+        } else
         step->run = [=](Phase ph) {
             bool done = false;
             const size_t N = X->value.rows(), K = X->value.cols(), C = Wn->value.cols(), H = W1->value.cols(),
@@ -408,6 +546,95 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
     steps.erase(std::remove(steps.begin(), steps.end(), std::shared_ptr<Step>()), steps.end());
 }
 
+// The tail that turns logits into the two numbers a training loop looks at,
+//   CrossEntropy(logits, y, softmax inside) -> ReduceMean                       (the loss)
+//   ArgMax(y) -> InTopK(logits, ., 1) -> TypeCast -> ReduceMean                 (the accuracy; optional)
+// (examples/graph_classification/src/kernel_mean_field.cpp:51-56), becomes one call of gnnhip_s2v_loss_acc_f32.
+// It leaves behind what the factors' Backward read (the CrossEntropy factor's probabilities, the loss rows), so
+// a training plan may fold it as well.
+inline void FactorGraph::FoldLossTail(Plan& plan)
+{
+    typedef DTensorVar<GPU, float> DVar;
+    typedef SpTensorVar<GPU, float> SVar;
+    typedef detail::FusedStep Step;
+    auto& steps = plan.steps;
+    std::vector<bool> is_target(var_list.size(), false);
+    for (size_t v : plan.target_idx) is_target[v] = true;
+    auto dense = [&](size_t v) { return dynamic_cast<DVar*>(var_list[v].get()); };
+    auto kind_is = [&](size_t f, const char* k) { return !strcmp(factor_list[f]->FuseKind(), k); };
+    // the step that is exactly factor f on its own, or -1
+    auto single_step_of = [&](size_t f) -> int {
+        for (size_t i = 0; i < steps.size(); ++i)
+            if (steps[i] && steps[i]->tag == Step::SINGLE && steps[i]->factors.size() == 1 && steps[i]->factors[0] == f) return (int)i;
+        return -1;
+    };
+    // the one executed reader of v, of the given kind, when v is private to it
+    auto sole_reader = [&](size_t v, const char* k, size_t& reader) {
+        if (is_target[v]) return false;
+        size_t n = 0;
+        for (size_t f : var_nodes[v].consumers) if (plan.executed[f]) { reader = f; ++n; }
+        return n == 1 && kind_is(reader, k) && single_step_of(reader) >= 0;
+    };
+    for (size_t f_ce = 0; f_ce < factor_list.size(); ++f_ce) {
+        if (!plan.executed[f_ce] || !kind_is(f_ce, "cross_entropy_softmax") || single_step_of(f_ce) < 0) continue;
+        if (factor_nodes[f_ce].in.size() != 2) continue;
+        const size_t vLogits = factor_nodes[f_ce].in[0], vY = factor_nodes[f_ce].in[1], vCe = factor_nodes[f_ce].out[0];
+        DVar *Logits = dense(vLogits), *Ce = dense(vCe);
+        SVar* Y = dynamic_cast<SVar*>(var_list[vY].get());
+        auto* probs = static_cast<DTensor<GPU, float>*>(factor_list[f_ce]->FusePayload());
+        size_t f_m1 = 0;
+        if (!Logits || !Ce || !Y || !probs || !sole_reader(vCe, "reduce_mean", f_m1)) continue;
+        DVar* Loss = dense(factor_nodes[f_m1].out[0]);
+        if (!Loss) continue;
+        std::vector<size_t> fs = {f_ce, f_m1};
+        // the accuracy chain on the same logits and labels, if there is one
+        DVar* Acc = nullptr;
+        for (size_t f_am : var_nodes[vY].consumers) {
+            if (!plan.executed[f_am] || !kind_is(f_am, "arg_max") || single_step_of(f_am) < 0) continue;
+            size_t f_tk = 0, f_tc = 0, f_m2 = 0;
+            const size_t vTruth = factor_nodes[f_am].out[0];
+            if (!sole_reader(vTruth, "in_top_1", f_tk) || factor_nodes[f_tk].in.size() != 2 || factor_nodes[f_tk].in[0] != vLogits ||
+                factor_nodes[f_tk].in[1] != vTruth) continue;
+            if (!sole_reader(factor_nodes[f_tk].out[0], "type_cast", f_tc)) continue;
+            if (!sole_reader(factor_nodes[f_tc].out[0], "reduce_mean", f_m2)) continue;
+            Acc = dense(factor_nodes[f_m2].out[0]);
+            if (!Acc) continue;
+            fs.insert(fs.end(), {f_am, f_tk, f_tc, f_m2});
+            break;
+        }
+        auto step = std::make_shared<Step>();
+        step->fused = true;
+        step->tag = Step::LOSS;
+        step->factors = fs;
+        step->run = [=](Phase) {
+            ASSERT(Logits->value.rank() == 2 && Logits->value.rows() == Y->value.rows() && Logits->value.cols() == Y->value.cols(),
+                   "loss tail: logits and labels disagree in shape");
+            const size_t B = Logits->value.rows(), Q = Logits->value.cols();
+            probs->Reshape({B, Q});
+            Ce->value.Reshape({B, 1});
+            Loss->value.Reshape({1});
+            if (Acc) Acc->value.Reshape({1});
+            GNN_HIP(gnnhip_s2v_loss_acc_f32((int)B, (int)Q, Logits->value.data->ptr, Y->value.data->row_ptr, Y->value.data->col_idx,
+                                            Y->value.data->val, probs->data->ptr, Ce->value.data->ptr, nullptr,
+                                            Loss->value.data->ptr, Acc ? Acc->value.data->ptr : nullptr, GpuHandle::Stream()));
+        };
+        int last = -1;
+        for (size_t f : fs) { const int i = single_step_of(f); last = std::max(last, i); }
+        for (size_t f : fs) steps[single_step_of(f)].reset();
+        steps[last] = step;
+        plan.n_fused++;
+        // a folded training forward that ends in these logits starts its backward pass from this loss
+        for (auto& st : steps)
+            if (st && st->tag == Step::FORWARD && st->train && !st->vars.empty() && st->vars[0] == vLogits) {
+                st->train->probs = probs;
+                st->train->label = Y;
+                st->train->loss_var = factor_nodes[f_m1].out[0];
+                st->train->loss_attached = true;
+            }
+    }
+    steps.erase(std::remove(steps.begin(), steps.end(), std::shared_ptr<Step>()), steps.end());
+}
+
 inline FactorGraph::VarList FactorGraph::FeedForward(std::vector<VarPtr> targets, std::map<std::string, void*> feed_dict,
                                                      Phase phase, uint n_thread)
 {
@@ -428,7 +655,15 @@ inline void FactorGraph::BackPropagate(std::vector<VarPtr> targets, uint n_threa
     if (n_thread != 1) throw std::runtime_error("not implemented");
     ASSERT(last_plan && last_plan->version == version, "unexpected change of computation graph in backward stage");
     Plan& plan = *last_plan;
-    ASSERT(plan.n_fused == 0, "BackPropagate needs a FeedForward run with Phase::TRAIN (inference plans fuse factors)");
+    // A folded step is fine when it left behind what Backward reads (the loss tail), or when it brings its own
+    // backward pass (the folded forward of a training plan, if its last run took the folded route).
+    detail::FusedStep* folded_forward = nullptr;
+    for (auto& st : plan.steps) {
+        if (!st->fused || st->tag == detail::FusedStep::LOSS) continue;
+        ASSERT(plan.phase == Phase::TRAIN && st->tag == detail::FusedStep::FORWARD && st->train,
+               "BackPropagate needs a FeedForward run with Phase::TRAIN (inference plans fuse factors)");
+        if (st->train->fused_ran) folded_forward = st.get();
+    }
     const size_t nv = var_list.size(), nf = factor_list.size();
 
     var_has_grad.assign(nv, false);
@@ -446,6 +681,15 @@ inline void FactorGraph::BackPropagate(std::vector<VarPtr> targets, uint n_threa
             }
     if (!zero_ptr.empty())
         GNN_HIP(gnnhip_memset0_batch((int)zero_ptr.size(), zero_ptr.data(), zero_bytes.data(), GpuHandle::Stream()));
+    if (folded_forward) {
+        // gradients of the weight matrices straight from the folded forward's own backward pass; the variables
+        // between them were never materialised, so only the loss the fold was built around can be the start
+        ASSERT(targets.size() == 1 && VarIdx(targets[0]) == folded_forward->train->loss_var,
+               "after a folded training forward BackPropagate starts from the mean cross-entropy it was built around; "
+               "call EnableFusion(false) for other targets");
+        folded_forward->backward();
+        return;
+    }
     for (auto& p : targets) {
         const size_t v = VarIdx(p);
         ASSERT(var_nodes[v].consumers.empty(), "only allow backprop from top variables");

@@ -25,6 +25,7 @@ public:
         if (auto* src_i = dynamic_cast<DTensorVar<mode, int>*>(operands[0].get())) out.CopyFrom(src_i->value);
         else out.CopyFrom(detail::dense_var<mode, Dtype>(operands[0], "TypeCast").value);
     }
+    virtual const char* FuseKind() const override { return "type_cast"; }
     // nothing flows back through a cast from integers
     virtual void Backward(std::vector< std::shared_ptr<Variable> >&, std::vector<bool>&,
                           std::vector< std::shared_ptr<Variable> >&) override {}

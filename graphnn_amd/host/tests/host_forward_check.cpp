@@ -1,7 +1,8 @@
 // Test driver for the host API layer: builds the structure2vec mean-field graph through
 // FactorGraph / af<> / add_diff<> exactly as a graphnn user would, runs it on one batch with
 // weights read from files, and writes what it computed so the Python test can compare with
-// the CPU oracle:  inference pass (fused plan), training pass (factor by factor), gradients.
+// the CPU oracle:  inference pass (fused plan), training pass (folded forward + backward, then factor by
+// factor), gradients, two optimizer steps, checkpoint.
 //
 //   host_forward_check <dir> K C H Q L
 //   <dir>/graphs.txt            dataset in graphnn's txt layout (all graphs form the batch)
@@ -152,23 +153,45 @@ int main(int argc, char** argv)
     out.push_back(loss->AsScalar());
     out.push_back(acc->AsScalar());
     append(out, logits->value);
-    // 2. training pass: every factor runs on its own
+    // 2. training pass: the plan folds the forward (keeping every level for its backward pass) and the loss tail
     fg.FeedForward(targets, feed, Phase::TRAIN);
     out.push_back((float)fg.LastPlanFactorCount());
     out.push_back((float)fg.LastPlanFusedCount());
     out.push_back(loss->AsScalar());
     out.push_back(acc->AsScalar());
     append(out, logits->value);
-    append(out, h->value);
-    // 3. gradients of the loss
+    // 3. gradients of the loss from the folded backward pass
     fg.BackPropagate({loss});
     for (auto& p : {w_n2l, w_conv, w_h1, w_h2}) {
         auto g = p->grad.Full();
         append(out, g);
     }
-    // 4. one momentum-SGD step, then the loss again (must not go up for a small step)
-    MomentumSGDOptimizer<mode, Dtype> opt(&model, 0.01f, 0.9f, 0.0f);
+    // 3b. the same with every factor on its own (forward and backward as graphnn schedules them)
+    fg.EnableFusion(false);
+    fg.FeedForward(targets, feed, Phase::TRAIN);
+    out.push_back((float)fg.LastPlanFactorCount());
+    out.push_back((float)fg.LastPlanFusedCount());
+    out.push_back(loss->AsScalar());
+    append(out, h->value);
+    fg.BackPropagate({loss});
+    for (auto& p : {w_n2l, w_conv, w_h1, w_h2}) {
+        auto g = p->grad.Full();
+        append(out, g);
+    }
+    fg.EnableFusion(true);
+    // 4. two momentum-SGD steps with weight decay (all four tensors in one launch each): weights after the first,
+    //    gradients of the second iteration, weights after the second; then the loss
+    MomentumSGDOptimizer<mode, Dtype> opt(&model, 0.01f, 0.9f, 0.001f);
     opt.Update();
+    for (auto& p : {w_n2l, w_conv, w_h1, w_h2}) append(out, p->value);
+    fg.FeedForward(targets, feed, Phase::TRAIN);
+    fg.BackPropagate({loss});
+    for (auto& p : {w_n2l, w_conv, w_h1, w_h2}) {
+        auto g = p->grad.Full();
+        append(out, g);
+    }
+    opt.Update();
+    for (auto& p : {w_n2l, w_conv, w_h1, w_h2}) append(out, p->value);
     fg.FeedForward(targets, feed, Phase::TEST);
     out.push_back(loss->AsScalar());
     // 5. checkpoint round trip in graphnn's wire format

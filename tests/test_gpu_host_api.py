@@ -90,33 +90,60 @@ def test_host_api_forward_backward_checkpoint(gpu, oracle, tmp_path, C):
         v = out[pos:pos + n]; pos += n
         return v
 
-    # 1. inference plan: input, levels and readout (4 L + 6 factors) folded into the one-launch forward,
-    #    the other 8 factors (two message-pass operands, loss and accuracy) on their own
+    # 1. inference plan: input, levels and readout (4 L + 6 factors) folded into the one-launch forward, the six
+    #    factors of the loss / accuracy tail into one step, the two message-pass operands on their own
     n_steps, n_fused, loss, acc = take(4)
-    assert n_fused == 1
-    assert n_steps == 9
+    assert n_fused == 2
+    assert n_steps == 4
     logits = take(B * Q).reshape(B, Q)
     assert max_rel(logits, want["logits"]) < PARITY_TOL
     assert abs(loss - want["scalars"][0]) <= 1e-4 * abs(want["scalars"][0])
     assert abs(acc - want["scalars"][1]) <= 1e-6
-    # 2. training plan: every factor on its own, same numbers
+    # 2. training plan: the two message-pass operands, the folded forward (every level kept) and the loss tail
     n_steps_t, n_fused_t, loss_t, acc_t = take(4)
-    assert n_fused_t == 0 and n_steps_t == 4 * L + 14
+    assert n_fused_t == 2 and n_steps_t == 4
     logits_t = take(B * Q).reshape(B, Q)
-    h_final = take(N * C).reshape(N, C)
     assert max_rel(logits_t, want["logits"]) < PARITY_TOL
-    assert max_rel(h_final, want["h"][L]) < PARITY_TOL
     assert abs(loss_t - loss) <= 1e-5 * abs(loss) and acc_t == acc
-    # 3. gradients against the float64 model
+    # 3. gradients of the folded backward pass against the float64 model, at the parity tolerance
     A = _dense(a, N, N); S = _dense(s, B, N)
     loss64, logits64, h64, grads64 = _model_and_grads(A, S, X.astype(np.float64), w, L, batch.graph_label)
     assert abs(loss_t - loss64) <= 1e-5 * abs(loss64)
-    for name, g64 in zip(("w_n2l", "w_conv", "w_h1", "w_h2"), grads64):
+    names = ("w_n2l", "w_conv", "w_h1", "w_h2")
+    grads_dev = []
+    for name, g64 in zip(names, grads64):
         got = take(g64.size).reshape(g64.shape)
-        assert max_rel(got, g64) < 1e-3, name
-    # 4. one small momentum-SGD step does not raise the loss; 5. the checkpoint restores the weights
+        grads_dev.append(got)
+        assert max_rel(got, g64) < PARITY_TOL, name
+    # 3b. factor by factor (4 L + 14 factors, nothing folded): the same loss, embeddings and gradients
+    n_steps_u, n_fused_u, loss_u = take(3)
+    assert n_fused_u == 0 and n_steps_u == 4 * L + 14
+    assert abs(loss_u - loss_t) <= 1e-6 * abs(loss_t)
+    assert max_rel(take(N * C).reshape(N, C), want["h"][L]) < PARITY_TOL
+    for name, g64, gf in zip(names, grads64, grads_dev):
+        got = take(g64.size).reshape(g64.shape)
+        assert max_rel(got, g64) < PARITY_TOL, name
+        assert max_rel(got, gf) < PARITY_TOL, name
+    # 4. two momentum-SGD steps (lr 0.01, momentum 0.9, weight decay 0.001) against the oracle's update rule
+    #    (src/nn/optimizer.cpp:69-92) applied to the gradients the device produced
+    w_host = [m.astype(np.float32) for m in (w.W_n2l, w.W_conv, w.W_h1, w.W_h2)]
+    vel = [np.zeros_like(m) for m in w_host]
+    w1_dev = []
+    for i, name in enumerate(names):
+        w_host[i], _, vel[i] = oracle.momentum_sgd(w_host[i], grads_dev[i], vel[i], 0.01, 0.9, 0.001)
+        got = take(w_host[i].size).reshape(w_host[i].shape)
+        w1_dev.append(got)
+        assert np.allclose(got, w_host[i], rtol=1e-6, atol=1e-8), name
+    grads2 = [take(m.size).reshape(m.shape) for m in w_host]
+    for i, name in enumerate(names):
+        assert not np.allclose(grads2[i], grads_dev[i], rtol=1e-3), name          # the weights moved: a new gradient
+        want_w, _, _ = oracle.momentum_sgd(w1_dev[i], grads2[i], vel[i], 0.01, 0.9, 0.001)
+        got = take(want_w.size).reshape(want_w.shape)
+        assert np.allclose(got, want_w, rtol=1e-6, atol=1e-8), name
+        # momentum is at work: the second step is not lr * gradient alone
+        assert not np.allclose(got, w1_dev[i] - 0.01 * (grads2[i] + 0.001 * w1_dev[i]), rtol=1e-4, atol=1e-7), name
     loss_after_step, loss_after_reload = take(2)
-    assert loss_after_step <= loss_t + 1e-6
+    assert loss_after_step < loss_t
     assert loss_after_reload == loss_after_step
     assert pos == out.size
     # checkpoint layout: per parameter (name order) rank, dims, count as size_t, then fp32 data
@@ -228,18 +255,16 @@ def test_host_api_large_batch_takes_the_separate_kernels(gpu, oracle, tmp_path):
     want = oracle.forward(a, s, batch.one_hot(), w, L, batch.label_csr())
     B, N = batch.num_graphs, batch.num_nodes
     n_steps, n_fused, loss, acc = out[:4]
-    assert n_fused == 1 and n_steps == 9
+    assert n_fused == 2 and n_steps == 4
     logits = out[4:4 + B * Q].reshape(B, Q)
     assert max_rel(logits, want["logits"]) < PARITY_TOL
     assert abs(loss - want["scalars"][0]) <= 1e-4 * abs(want["scalars"][0])
     assert abs(acc - want["scalars"][1]) <= 1e-6
     pos = 4 + B * Q
     n_steps_t, n_fused_t, loss_t, acc_t = out[pos:pos + 4]
-    assert n_fused_t == 0 and n_steps_t == 4 * L + 14
+    assert n_fused_t == 2 and n_steps_t == 4
     logits_t = out[pos + 4:pos + 4 + B * Q].reshape(B, Q)
-    h_final = out[pos + 4 + B * Q:pos + 4 + B * Q + N * C].reshape(N, C)
     assert max_rel(logits_t, want["logits"]) < PARITY_TOL
-    assert max_rel(h_final, want["h"][L]) < PARITY_TOL
     assert abs(loss_t - loss) <= 1e-5 * abs(loss) and acc_t == acc
 
 
