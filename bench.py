@@ -223,7 +223,8 @@ def training_step_host_layer(host, reps=100):
         return {"skipped": "host_forward_bench train failed: " + (r.stderr or r.stdout)[-300:]}
     res = json.loads(r.stdout.strip().splitlines()[-1])
     res["what"] = ("GetBatch-style host batch build + FactorGraph::FeedForward(TRAIN) + BackPropagate + "
-                   "MomentumSGDOptimizer::Update per batch, operator-by-operator plan")
+                   "MomentumSGDOptimizer::Update per batch; the training plan folds the forward (levels kept), the loss "
+                   "tail, the backward pass and the update of all tensors")
     return res
 
 

@@ -69,6 +69,7 @@ SIGNATURES = {
     "gnnhip_row_scale_f32": [_I, _I, _P, _P, _P],
     "gnnhip_s2v_loss_acc_f32": [_I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_s2v_readout_backward_f32": [_I] * 5 + [_P] * 7 + [_F] + [_P] * 6 + [_P],
+    "gnnhip_s2v_level_backward_f32": [_I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_s2v_grad_gate_f32": [_Z, _P, _P, _P, _P, _I, _P],
     "gnnhip_momentum_sgd_batch_f32": [_I, _P, _P, _P, _P, _F, _F, _F, _P],
     "gnnhip_last_error": [],

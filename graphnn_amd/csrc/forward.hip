@@ -14,6 +14,8 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
                    const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph = false,
                    bool relu_in = false);
 bool level_accepts_relu_input(int N, int C, long long nnz);
+int level_backward_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* dz,
+                            const float* W, float* u, float* g_prev, hipStream_t s);
 int readout_dispatch(int B, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                      const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
                      float* logits, float* probs, int* pred, hipStream_t s);
@@ -154,6 +156,21 @@ int gnnhip_s2v_level_f32(int N, int C, int nnz, const int* row_ptr, const int* c
     GNNHIP_REQUIRE(h_in != h_out, "s2v_level cannot run in place");
     if (int rc = require_ready()) return rc;
     return level_any(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, as_stream(stream));
+}
+
+int gnnhip_s2v_level_backward_f32(int N, int C, int nnz, const int* t_row_ptr, const int* t_col_idx, const float* t_val,
+                                  const float* dz, const float* W, float* u, float* g_prev, void* stream)
+{
+    GNNHIP_REQUIRE(N >= 0 && C >= 1 && nnz >= 0, "bad shape in s2v_level_backward (N=%d C=%d nnz=%d)", N, C, nnz);
+    if (N == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(t_row_ptr && dz && W && u && g_prev, "null tensor in s2v_level_backward");
+    GNNHIP_REQUIRE(dz != u && dz != g_prev && u != g_prev, "s2v_level_backward needs three distinct buffers");
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    int rc = level_backward_dispatch(N, C, nnz, t_row_ptr, t_col_idx, t_val, dz, W, u, g_prev, s);
+    if (rc != GNNHIP_EUNSUPPORTED) return rc;
+    if ((rc = spmm_dispatch(N, C, nnz, 1.f, t_row_ptr, t_col_idx, t_val, dz, C, 0.f, u, C, s))) return rc;
+    return gemm_dispatch(0, 1, N, C, C, 1.f, u, C, W, C, 0.f, g_prev, C, s);
 }
 
 int gnnhip_s2v_readout_f32(int B, int N, int C, int H, int Q,

@@ -90,12 +90,15 @@ __device__ __forceinline__ void sum4(float4& acc, float w, const float4 (&x)[4])
 }
 
 // MINW: wavefronts per SIMD the register allocation must leave room for
-template <int C, bool DENSE, bool WLDS, int MINW, bool RELU_IN, bool PIPE>
+// BWD: the backward pass of a level through the same machinery, out = (A' x) W^T with A' = A^T handed in as a
+// CSR matrix: W is read transposed, the aggregated rows A' x are also stored (agg_out: they are the other
+// factor of the weight gradient) and the result is stored as it is (no ReLU; msg and bias are null).
+template <int C, bool DENSE, bool WLDS, int MINW, bool RELU_IN, bool PIPE, bool BWD = false>
 __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
     int N, const int* __restrict__ row_ptr, const int* __restrict__ col_idx, const float* __restrict__ val,
     const float* __restrict__ h_in, const float* __restrict__ W, const float* __restrict__ msg,
     const float* __restrict__ bias, float* __restrict__ h_out,
-    const int* __restrict__ hub_slot, const float* __restrict__ hub_agg, int hub_ld)
+    const int* __restrict__ hub_slot, const float* __restrict__ hub_agg, int hub_ld, float* __restrict__ agg_out = nullptr)
 {
     constexpr int G = C / 4;             // lanes per gathered row
     constexpr int RPR = kWave / G;       // lane groups per wavefront
@@ -129,10 +132,12 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
             for (int s4 = 0; s4 < KS / 4; ++s4) {
                 float4 w4;
                 const int col = KS * (t >> 2) + 4 * jb + (t & 3);
-                w4.x = W[(size_t)(KS * q + 4 * s4 + 0) * C + col];
-                w4.y = W[(size_t)(KS * q + 4 * s4 + 1) * C + col];
-                w4.z = W[(size_t)(KS * q + 4 * s4 + 2) * C + col];
-                w4.w = W[(size_t)(KS * q + 4 * s4 + 3) * C + col];
+                const int k0 = KS * q + 4 * s4;
+                // element (k, col) of the operand: W[k][col], or W[col][k] when the level runs backward
+                w4.x = BWD ? W[(size_t)col * C + k0 + 0] : W[(size_t)(k0 + 0) * C + col];
+                w4.y = BWD ? W[(size_t)col * C + k0 + 1] : W[(size_t)(k0 + 1) * C + col];
+                w4.z = BWD ? W[(size_t)col * C + k0 + 2] : W[(size_t)(k0 + 2) * C + col];
+                w4.w = BWD ? W[(size_t)col * C + k0 + 3] : W[(size_t)(k0 + 3) * C + col];
                 wl[(jb * (KS / 4) + s4) * kWave + lane] = w4;
             }
         __syncthreads();
@@ -141,7 +146,8 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
         for (int jb = 0; jb < NJB; ++jb)
 #pragma unroll
             for (int s = 0; s < KS; ++s)
-                wreg[jb][s] = W[(size_t)(KS * q + s) * C + KS * (t >> 2) + 4 * jb + (t & 3)];
+                wreg[jb][s] = BWD ? W[(size_t)(KS * (t >> 2) + 4 * jb + (t & 3)) * C + KS * q + s]
+                                  : W[(size_t)(KS * q + s) * C + KS * (t >> 2) + 4 * jb + (t & 3)];
     }
 
     int E = 0;
@@ -358,6 +364,13 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
         }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
         GNNHIP_PHASE_ACC(3);
+        if constexpr (BWD) {
+            // the aggregated rows, as the lane groups hold them: whole 4 C-byte rows
+            const rsrc_t agg_rsrc = make_rsrc(agg_out, act_bytes);
+#pragma unroll
+            for (int rd = 0; rd < ROUNDS; ++rd)
+                buf_store4(agg_rsrc, out_off + rd * kRowBytes, 0, *reinterpret_cast<const float4*>(tile + (grp * ROUNDS + rd) * LDT + tx * 4));
+        }
         // msg is asked for once the gathered rows have left their registers; the contraction covers its trip
         float4 mrow[ROUNDS];
 #pragma unroll
@@ -402,7 +415,7 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
             float4 v = *reinterpret_cast<const float4*>(tile + (grp * ROUNDS + rd) * LDT + tx * 4);
             if (bias) { v.x += bias4.x; v.y += bias4.y; v.z += bias4.z; v.w += bias4.w; }
             v.x += mrow[rd].x; v.y += mrow[rd].y; v.z += mrow[rd].z; v.w += mrow[rd].w;
-            buf_store4(out_rsrc, out_off + rd * kRowBytes, 0, relu_ref4(v));
+            buf_store4(out_rsrc, out_off + rd * kRowBytes, 0, BWD ? v : relu_ref4(v));
         }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");     // the tile is rewritten by the next iteration
         if constexpr (PIPE && !DENSE) {
@@ -462,6 +475,23 @@ int launch_level_stream_c(int N, bool dense, bool relu_in, const int* row_ptr, c
     return launch_level_stream<C, false, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
 }
 
+template <int C>
+int launch_level_stream_backward(int N, const int* row_ptr, const int* col_idx, const float* val, const float* x,
+                                 const float* W, float* agg_out, float* out, const HubPlan& hubs, hipStream_t s)
+{
+    const long long ntiles = ((long long)N + 15) / 16;
+    long long blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
+    constexpr bool kWLds = (C == 64);
+    constexpr int kMinW = (C == 64) ? 3 : 4;
+    const long long resident = (long long)kNumCU * kMinW;
+    if (blocks > resident) blocks = resident;
+    hipLaunchKernelGGL((s2v_level_stream_kernel<C, false, kWLds, kMinW, false, false, true>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                       N, row_ptr, col_idx, val, x, W, (const float*)nullptr, (const float*)nullptr, out, hubs.row_slot, hubs.agg,
+                       hubs.ld, agg_out);
+    GNNHIP_LAUNCH_CHECK("s2v_level_stream (backward)");
+    return GNNHIP_OK;
+}
+
 }  // namespace
 
 // Whether N rows of C floats fit the 32-bit offsets of the kernel (with room for the 15 rows a last tile may
@@ -469,6 +499,18 @@ int launch_level_stream_c(int N, bool dense, bool relu_in, const int* row_ptr, c
 bool level_stream_covers(int N, int C)
 {
     return (C == 16 || C == 32 || C == 64) && (unsigned long long)N * (unsigned)C * 4ull < 0xFFFF0000ull;
+}
+
+// agg_out = A' x and out = agg_out W^T in one pass (A' in CSR form); same limits as level_stream_dispatch.
+int level_stream_backward_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* x,
+                                   const float* W, float* agg_out, float* out, const HubPlan& hubs, hipStream_t s)
+{
+    if (!level_stream_covers(N, C)) return GNNHIP_EUNSUPPORTED;
+    switch (C) {
+    case 16: return launch_level_stream_backward<16>(N, row_ptr, col_idx, val, x, W, agg_out, out, hubs, s);
+    case 32: return launch_level_stream_backward<32>(N, row_ptr, col_idx, val, x, W, agg_out, out, hubs, s);
+    default: return launch_level_stream_backward<64>(N, row_ptr, col_idx, val, x, W, agg_out, out, hubs, s);
+    }
 }
 
 // h_in, msg and h_out must each span less than 4 GiB; returns GNNHIP_EUNSUPPORTED otherwise.

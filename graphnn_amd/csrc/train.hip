@@ -85,8 +85,9 @@ __global__ __launch_bounds__(kWave) void loss_acc_final_kernel(int nb, int B, co
     }
 }
 
-// ------------------------------------------------------------------ readout backward, one wavefront per graph
-// LDS per wavefront: dlogits[Q] | du[H] | dpool[C]
+// ------------------------------------------------------------------ readout backward, one workgroup per graph
+// LDS: dlogits[Q] | du[H] | dpool[C].  The three small products run on the lanes that own their outputs; the
+// graph's gradient rows (its nodes x C) are then written by all lanes, row-contiguous.
 __global__ __launch_bounds__(kBlock) void readout_backward_kernel(
     int B, int C, int H, int Q, const int* __restrict__ s_row_ptr, const int* __restrict__ s_col_idx, const float* __restrict__ s_val,
     const float* __restrict__ probs, const int* __restrict__ lrow_ptr, const int* __restrict__ lcol, const float* __restrict__ lval,
@@ -94,45 +95,45 @@ __global__ __launch_bounds__(kBlock) void readout_backward_kernel(
     float* __restrict__ dlogits, float* __restrict__ du, float* __restrict__ g_h)
 {
     extern __shared__ float smem[];
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    float* dl = smem + (size_t)wave * (Q + H + C);
+    float* dl = smem;
     float* duw = dl + Q;
     float* dp = duw + H;
-    for (int g = blockIdx.x * kWavesPerBlock + wave; g < B; g += gridDim.x * kWavesPerBlock) {
+    const int tid = threadIdx.x;
+    for (int g = blockIdx.x; g < B; g += gridDim.x) {
         // dlogits = scale * (probs - y): CrossEntropy::Backward with softmax inside (src/nn/cross_entropy.cpp:52-78),
         // scale = the gradient ReduceMean hands to every row (src/nn/reduce_mean.cpp:44-65)
-        for (int q = lane; q < Q; q += kWave) {
+        for (int q = tid; q < Q; q += kBlock) {
             float y = 0.f;
             for (int k = lrow_ptr[g]; k < lrow_ptr[g + 1]; ++k) if (lcol[k] == q) y += lval[k];
             const float v = (probs[(size_t)g * Q + q] - y) * scale;
             dl[q] = v;
             dlogits[(size_t)g * Q + q] = v;
         }
-        __builtin_amdgcn_wave_barrier();
+        __syncthreads();
         // du = (dlogits W_h2^T) . [hidden > 0]
-        for (int j = lane; j < H; j += kWave) {
+        for (int j = tid; j < H; j += kBlock) {
             float s = 0.f;
             for (int q = 0; q < Q; ++q) s = fmaf(dl[q], Wh2[(size_t)j * Q + q], s);
             const float v = hidden[(size_t)g * H + j] > 0.f ? s : 0.f;
             duw[j] = v;
             du[(size_t)g * H + j] = v;
         }
-        __builtin_amdgcn_wave_barrier();
+        __syncthreads();
         // dpool = du W_h1^T
-        for (int c = lane; c < C; c += kWave) {
+        for (int c = tid; c < C; c += kBlock) {
             float s = 0.f;
             for (int j = 0; j < H; ++j) s = fmaf(duw[j], Wh1[(size_t)c * H + j], s);
             dp[c] = s;
         }
-        __builtin_amdgcn_wave_barrier();
+        __syncthreads();
         // gradient rows of the graph's nodes: S^T dpool restricted to this graph (every node is listed once)
-        const int a = s_row_ptr[g], b = s_row_ptr[g + 1];
-        for (int t = a; t < b; ++t) {
-            const float sv = s_val[t];
-            float* dst = g_h + (size_t)s_col_idx[t] * C;
-            for (int c = lane; c < C; c += kWave) dst[c] = sv * dp[c];
+        const int a = s_row_ptr[g];
+        const int total = (s_row_ptr[g + 1] - a) * C;
+        for (int i = tid; i < total; i += kBlock) {
+            const int r = i / C, c = i - r * C;
+            g_h[(size_t)s_col_idx[a + r] * C + c] = s_val[a + r] * dp[c];
         }
-        __builtin_amdgcn_wave_barrier();
+        __syncthreads();
     }
 }
 
@@ -223,11 +224,11 @@ int gnnhip_s2v_readout_backward_f32(int B, int N, int C, int H, int Q,
     GNNHIP_REQUIRE(s_row_ptr && s_col_idx && s_val && probs && lrow_ptr && lcol && lval && hidden && W_h1 && W_h2 && dlogits && du && g_h,
                    "null tensor in s2v_readout_backward");
     if (int rc = require_ready()) return rc;
-    const size_t smem = sizeof(float) * (size_t)kWavesPerBlock * ((size_t)Q + H + C);
+    const size_t smem = sizeof(float) * ((size_t)Q + H + C);
     if (smem > 64 * 1024)
         return set_error(GNNHIP_EUNSUPPORTED, "readout backward keeps Q + H + C = %d floats per graph in LDS; too many", Q + H + C);
-    long long blocks = ((long long)B + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (blocks > (long long)kNumCU * 8) blocks = (long long)kNumCU * 8;
+    long long blocks = B;
+    if (blocks > (long long)kNumCU * 16) blocks = (long long)kNumCU * 16;
     hipLaunchKernelGGL(readout_backward_kernel, dim3((unsigned)blocks), dim3(kBlock), smem, as_stream(stream), B, C, H, Q,
                        s_row_ptr, s_col_idx, s_val, probs, lrow_ptr, lcol, lval, scale, hidden, W_h1, W_h2, dlogits, du, g_h);
     GNNHIP_LAUNCH_CHECK("readout_backward");

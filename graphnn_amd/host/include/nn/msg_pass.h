@@ -15,6 +15,35 @@
 namespace gnn
 {
 
+namespace detail
+{
+// stable CSR transpose on the host (row c of the result lists, in ascending row order, the rows of `a` with an
+// entry in column c), handed to the device tensor as its cached transpose; host tensors keep none
+template<typename Dtype>
+inline void send_transpose(SpTensor<CPU, Dtype>&, SpTensor<CPU, Dtype>&, std::vector<int>&, SpTensor<CPU, Dtype>&) {}
+template<typename Dtype>
+inline void send_transpose(SpTensor<CPU, Dtype>& a, SpTensor<CPU, Dtype>& t, std::vector<int>& cursor, SpTensor<GPU, Dtype>& out)
+{
+    const int m = (int)a.rows(), k = (int)a.cols(), nnz = a.data->nnz;
+    t.Reshape({(size_t)k, (size_t)m});
+    t.ResizeSp(nnz, k + 1);
+    cursor.assign((size_t)k + 1, 0);
+    const int* rp = a.data->row_ptr;
+    const int* ci = a.data->col_idx;
+    for (int e = 0; e < nnz; ++e) cursor[(size_t)ci[e] + 1]++;
+    int* trp = t.data->row_ptr;
+    trp[0] = 0;
+    for (int c = 0; c < k; ++c) { trp[c + 1] = trp[c] + cursor[(size_t)c + 1]; cursor[c] = trp[c]; }
+    for (int r = 0; r < m; ++r)
+        for (int e = rp[r]; e < rp[r + 1]; ++e) {
+            const int dst = cursor[ci[e]]++;
+            t.data->col_idx[dst] = r;
+            t.data->val[dst] = a.data->val[e];
+        }
+    out.SetTransposed(t);
+}
+}  // namespace detail
+
 template<typename mode, typename Dtype>
 class IMsgPass : public Factor
 {
@@ -24,7 +53,7 @@ public:
     IMsgPass(std::string _name, bool _average) : Factor(_name, PropErr::N), average(_average) {}
 
     virtual void Forward(std::vector< std::shared_ptr<Variable> >& operands,
-                         std::vector< std::shared_ptr<Variable> >& outputs, Phase) override
+                         std::vector< std::shared_ptr<Variable> >& outputs, Phase phase) override
     {
         ASSERT(operands.size() == 1, "unexpected input size for " << StrType());
         ASSERT(outputs.size() == 1, "unexpected output size for " << StrType());
@@ -34,6 +63,9 @@ public:
         if (BuildOnDevice(gv->graph, out)) return;
         InitCPUWeight(gv->graph);
         out.CopyFrom(cpu_weight);          // host -> device (or host -> host) copy of the three CSR arrays
+        // training multiplies by the transpose in the backward pass: the matrix is on the host right now,
+        // so its transpose goes along instead of being sorted out on the device later
+        if (phase == Phase::TRAIN && TransposeForBackward()) detail::send_transpose(cpu_weight, cpu_transpose, cursor, out);
     }
 
     // layout facts about the last batch, gathered while the CSR was built (used to choose kernels)
@@ -45,7 +77,9 @@ protected:
     // Operands that are a grouping of the flat edge list can be built on the device from one copy
     // of that list; returns false where the host construction is to be used.
     virtual bool BuildOnDevice(GraphStruct*, SpTensor<mode, Dtype>&) { return false; }
-    SpTensor<CPU, Dtype> cpu_weight;
+    virtual bool TransposeForBackward() const { return false; }
+    SpTensor<CPU, Dtype> cpu_weight, cpu_transpose;
+    std::vector<int> cursor;
     bool average;
 };
 
@@ -118,6 +152,7 @@ public:
     virtual const char* FuseKind() const override { return "msg_node2node"; }
 
 protected:
+    virtual bool TransposeForBackward() const override { return true; }
     virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out) override
     {
         this->layout.block_diagonal = false;           // not examined on this route

@@ -28,7 +28,7 @@ struct TrainState
 {
     DTensor<GPU, float> hstack;             // [(L + 1) N, C]: the embeddings of every level, h0 first
     DTensor<GPU, float> ustack;             // [L N, C]: A^T dz of every level
-    DTensor<GPU, float> g, dmsg, dl, du;    // [N, C], [N, C], [B, Q], [B, H]
+    DTensor<GPU, float> g, g2, dmsg, dl, du;   // [N, C] x 3, [B, Q], [B, H]
     DTensor<GPU, float>* probs = nullptr;   // the CrossEntropy factor's probabilities (filled by the loss tail)
     SpTensorVar<GPU, float>* label = nullptr;
     size_t loss_var = (size_t)-1;           // the variable BackPropagate must start from
@@ -415,7 +415,7 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
                        W2->value.rows() == H && A->value.rows() == N && A->value.cols() == N && S->value.cols() == N,
                        "fused forward: operand shapes do not chain");
                 // the folded backward needs S to list every node once and the per-graph LDS of its readout kernel
-                st->fused_ran = st->loss_attached && sub->contiguous_subgraphs && (Q + H + C) * 16 <= 64 * 1024;
+                st->fused_ran = st->loss_attached && sub->contiguous_subgraphs && (Q + H + C) * 4 <= 64 * 1024;
                 if (!st->fused_ran) {
                     for (auto& p : singles) p->run(ph);
                     return;
@@ -451,6 +451,7 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
                 const size_t NC = N * C;
                 void* s = GpuHandle::Stream();
                 st->g.Reshape({N, C});
+                st->g2.Reshape({N, C});
                 st->dmsg.Reshape({N, C});
                 st->dl.Reshape({B, Q});
                 st->du.Reshape({B, H});
@@ -467,12 +468,12 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
                 if (L > 0) {
                     auto& at = A->value.Transposed();
                     float* us = st->ustack.data->ptr;
+                    float* g2 = st->g2.data->ptr;
                     for (int l = L; l >= 1; --l) {
                         GNN_HIP(gnnhip_s2v_grad_gate_f32(NC, hs + (size_t)l * NC, g, g, dmsg, l < L ? 1 : 0, s));
-                        float* u = us + (size_t)(l - 1) * NC;
-                        GNN_HIP(gnnhip_spmm_csr_f32((int)N, (int)N, (int)C, at.nnz, 1.0f, at.row_ptr, at.col_idx, at.val, g, (int)C,
-                                                    0.0f, u, (int)C, s));
-                        GNN_HIP(gnnhip_gemm_f32(0, 1, (int)N, (int)C, (int)C, 1.0f, u, (int)C, Wc->value.data->ptr, (int)C, 0.0f, g, (int)C, s));
+                        GNN_HIP(gnnhip_s2v_level_backward_f32((int)N, (int)C, at.nnz, at.row_ptr, at.col_idx, at.val, g,
+                                                              Wc->value.data->ptr, us + (size_t)(l - 1) * NC, g2, s));
+                        std::swap(g, g2);
                     }
                     GNN_HIP(gnnhip_s2v_grad_gate_f32(NC, hs, g, nullptr, dmsg, 1, s));
                     if (!cWc)

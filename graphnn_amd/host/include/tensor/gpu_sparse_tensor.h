@@ -47,6 +47,22 @@ public:
         }
         return *t_data;
     }
+    // The transpose handed over by a builder that had the matrix on the host anyway (three small copies instead
+    // of the dozen launches of the device transposition); t must be the stable transpose of what this tensor
+    // holds: row c of t lists the rows of the matrix that have an entry in column c, in ascending row order.
+    void SetTransposed(SpTensor<CPU, Dtype>& t)
+    {
+        ASSERT(t.rows() == shape[1] && t.cols() == shape[0] && t.data->nnz == data->nnz, "not the transpose of this matrix");
+        if (!t_data) t_data = std::make_shared< SparseData<GPU, Dtype> >();
+        t_data->Reserve(t.data->nnz, t.data->len_ptr);
+        t_data->nnz = t.data->nnz;
+        t_data->len_ptr = t.data->len_ptr;
+        void* s = GpuHandle::Stream();
+        GNN_HIP(gnnhip_memcpy_h2d(t_data->val, t.data->val, sizeof(Dtype) * (size_t)t.data->nnz, s));
+        GNN_HIP(gnnhip_memcpy_h2d(t_data->col_idx, t.data->col_idx, sizeof(int) * (size_t)t.data->nnz, s));
+        GNN_HIP(gnnhip_memcpy_h2d(t_data->row_ptr, t.data->row_ptr, sizeof(int) * (size_t)t.data->len_ptr, s));
+        t_valid = true;
+    }
     // three host-to-device copies, ordered on the layer's stream
     void CopyFrom(SpTensor<CPU, Dtype>& src)
     {

@@ -477,6 +477,20 @@ def readout_backward(s_csr, probs, label_csr, scale, hidden, W_h1, W_h2, N):
     return dlogits, du, g_h
 
 
+def s2v_level_backward(t_row_ptr, t_col_idx, t_val, dz, W, u=None, g_prev=None):
+    """u = A^T dz, g_prev = u W^T; the CSR arrays are those of A^T"""
+    N, C = dz.shape
+    _check_csr(t_row_ptr, t_col_idx, t_val, N, "A^T")
+    if u is None:
+        u = torch.empty_like(dz)
+    if g_prev is None:
+        g_prev = torch.empty_like(dz)
+    check(_lib().gnnhip_s2v_level_backward_f32(N, C, int(t_col_idx.numel()), _i32(t_row_ptr, "t_row_ptr"), _i32(t_col_idx, "t_col_idx"),
+                                               _f32(t_val, "t_val"), _f32(dz, "dz"), _f32(W, "W"), _f32(u, "u"), _f32(g_prev, "g_prev"),
+                                               _stream()))
+    return u, g_prev
+
+
 def grad_gate(h, g, dz=None, acc=None, accumulate=False):
     check(_lib().gnnhip_s2v_grad_gate_f32(h.numel(), _f32(h, "h"), _f32(g, "g"), _f32(dz, "dz"), _f32(acc, "acc"),
                                           1 if accumulate else 0, _stream()))

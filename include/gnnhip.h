@@ -321,6 +321,16 @@ int gnnhip_s2v_readout_backward_f32(int B, int N, int C, int H, int Q,
  *      dz may alias g; dz or acc may be NULL. */
 int gnnhip_s2v_grad_gate_f32(size_t n, const float* h, const float* g, float* dz, float* acc, int accumulate, void* stream);
 
+/* ---- backward of one mean-field level past its ReLU gate, in one pass:
+ *      u = A^T * dz ;  g_prev = u * W^T
+ *      (MatMul::Backward twice, src/nn/matmul.cpp:35-76: through lin = agg * W and through agg = A * h_prev, taken
+ *      in the other order, which is the same product; the reference runs cuSPARSE csrmm(T) + cuBLAS,
+ *      src/tensor/gpu_dense_tensor.cu:271-294).  A^T is handed in as a CSR matrix [N,N] with nnz entries
+ *      (gnnhip_csr_transpose_f32).  u [N,C] is also the other factor of the weight gradient:
+ *      dW += h_prev^T * u  (= (A h_prev)^T dz).  dz, u and g_prev are three distinct buffers. */
+int gnnhip_s2v_level_backward_f32(int N, int C, int nnz, const int* t_row_ptr, const int* t_col_idx, const float* t_val,
+                                  const float* dz, const float* W, float* u, float* g_prev, void* stream);
+
 /* ---- MomentumSGDOptimizer::Update over n tensors in one launch (src/nn/optimizer.cpp:69-92):
  *      momentum > 0:  g += l2 w ; v = lr g + momentum v ; w -= v ; g = 0      (v: the optimizer's acc_grad_dict)
  *      momentum == 0: w = -lr g + (1 - lr l2) w ; g = 0                        (v may be NULL)

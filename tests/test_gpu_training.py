@@ -87,6 +87,29 @@ def test_readout_backward(gpu, oracle, C, H, Q, B):
     assert_parity("g_h", _n(gh), w_gh, gh64)
 
 
+@pytest.mark.parametrize("C", [16, 32, 64, 128])
+@pytest.mark.parametrize("N", [77, 7450, 40_000])
+def test_level_backward(gpu, oracle, C, N):
+    """u = A^T dz and g_prev = u W^T in one pass (hidden 16/32/64; hidden 128 takes SpMM + GEMM inside the entry):
+    ragged rows, two long rows (the larger matrix sends them through the balanced pass), signed dz"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(C + N)
+    lens = rng.integers(0, 7, N); lens[N // 3] = min(N, 3000); lens[N - 1] = 70
+    rp = np.zeros(N + 1, np.int32); np.cumsum(lens, out=rp[1:])
+    nnz = int(rp[-1])
+    ci = rng.integers(0, N, nnz).astype(np.int32)
+    v = (rng.random(nnz) * 0.5).astype(np.float32)
+    dz = (rng.standard_normal((N, C)) * (rng.random((N, C)) < 0.5)).astype(np.float32)      # about half the gates closed
+    W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
+    u, g = ops.s2v_level_backward(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(dz, gpu), _t(W, gpu))
+    w_u = oracle.spmm(rp, ci, v, dz, N)
+    w_g = oracle.gemm(w_u, W, transB=True)
+    import scipy.sparse as sp
+    u64 = sp.csr_matrix((v.astype(np.float64), ci, rp), shape=(N, N)) @ dz.astype(np.float64)
+    assert_parity("u", _n(u), w_u, u64)
+    assert_parity("g_prev", _n(g), w_g, u64 @ W.astype(np.float64).T)
+
+
 def test_grad_gate_is_exact(gpu):
     import torch
     from graphnn_amd import ops
@@ -162,10 +185,11 @@ def test_training_iteration_composed_from_the_c_abi(gpu, oracle, config_id, C):
     at = ops.csr_transpose(*a_d, N, N)
     us = torch.empty((L, N, C), device=gpu)
     dmsg = torch.empty((N, C), device=gpu)
+    g2 = torch.empty_like(g)
     for l in range(L, 0, -1):
         ops.grad_gate(hs[l], g, g, dmsg, accumulate=(l < L))
-        ops.spmm(*at, g, N, out=us[l - 1])
-        g = ops.gemm(us[l - 1], Wc, transB=True)
+        ops.s2v_level_backward(*at, g, Wc, u=us[l - 1], g_prev=g2)
+        g, g2 = g2, g
     ops.grad_gate(hs[0], g, None, dmsg, accumulate=True)
     gWc = ops.gemm(hs[:L].reshape(L * N, C), us.reshape(L * N, C), transA=True)
     gWn = ops.gemm(X_d, dmsg, transA=True)
