@@ -278,6 +278,14 @@ def time_cfg5(dev, scale=22):
                    "gather_GBps": (4.0 * E * C + 4.0 * N * C + 8.0 * E) / (ms * 1e-3) / 1e9}
     ms = _event_ms(lambda: ops.gemm(h1, wsc, out=score), 5)
     res["score"] = {"avg_ms": ms}
+    # the whole forward (input, 3 levels, readout): levels two and three reuse the plan that level one made for A
+    H, Q, L = 64, 2, 3
+    Wh1 = torch.randn((C, H), device=dev, generator=g) * 0.1
+    Wh2 = torch.randn((H, Q), device=dev, generator=g) * 0.1
+    bufs = ops.ForwardBuffers(N, B, C, H, Q, dev)
+    ms = _event_ms(lambda: ops.s2v_forward((rp, ci, val), (s_rp, s_ci, s_v), X, Wn, Wc, Wh1, Wh2, L, bufs=bufs), 5)
+    res["forward"] = {"avg_ms": ms, "levels": L, "graphs": B}
+    del bufs
     ms = _event_ms(lambda: ops.jagged_softmax(score, lens), 5)
     res["jagged_softmax"] = {"avg_ms": ms, "GBps": 8.0 * N / (ms * 1e-3) / 1e9}
     ms = _event_ms(lambda: ops.spmm(s_rp, s_ci, s_v, h1, B, out=pool), 5)

@@ -79,7 +79,7 @@ int level_any(int N, int C, long long nnz, const int* row_ptr, const int* col_id
     const size_t total = (size_t)N * C;
     if ((rc = stream_scratch(s, sizeof(float) * total, &tmp))) return rc;
     float* agg = static_cast<float*>(tmp);
-    if ((rc = spmm_dispatch(N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, agg, C, s, same_graph))) return rc;
+    if ((rc = spmm_dispatch(N, N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, agg, C, s, same_graph))) return rc;
     if ((rc = gemm_dispatch(0, 0, N, C, C, 1.f, agg, C, W, C, 0.f, h_out, C, s))) return rc;
     hipLaunchKernelGGL(bias_add_relu_kernel, dim3(ew_grid(total)), dim3(kBlock), 0, s,
                        h_out, bias, msg, h_out, (float*)nullptr, total, C, 1);
@@ -113,7 +113,7 @@ int readout_any(int B, int N, int C, int H, int Q, const int* s_row_ptr, const i
     if (C <= 64 || B <= kBlockReadoutMaxGraphsWide)
         rc = readout_dispatch(B, C, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
-    if ((rc = spmm_dispatch(B, C, (long long)N, 1.f, s_row_ptr, s_col_idx, s_val, h, C, 0.f, pool, C, s))) return rc;
+    if ((rc = spmm_dispatch(B, N, C, (long long)N, 1.f, s_row_ptr, s_col_idx, s_val, h, C, 0.f, pool, C, s))) return rc;
     if ((rc = gemm_dispatch(0, 0, B, H, C, 1.f, pool, C, Wh1, H, 0.f, hidden, H, s))) return rc;
     const size_t bh = (size_t)B * H;
     hipLaunchKernelGGL(bias_add_relu_kernel, dim3(ew_grid(bh)), dim3(kBlock), 0, s,
@@ -169,7 +169,7 @@ int gnnhip_s2v_level_backward_f32(int N, int C, int nnz, const int* t_row_ptr, c
     hipStream_t s = as_stream(stream);
     int rc = level_backward_dispatch(N, C, nnz, t_row_ptr, t_col_idx, t_val, dz, W, u, g_prev, s);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
-    if ((rc = spmm_dispatch(N, C, nnz, 1.f, t_row_ptr, t_col_idx, t_val, dz, C, 0.f, u, C, s))) return rc;
+    if ((rc = spmm_dispatch(N, N, C, nnz, 1.f, t_row_ptr, t_col_idx, t_val, dz, C, 0.f, u, C, s))) return rc;
     return gemm_dispatch(0, 1, N, C, C, 1.f, u, C, W, C, 0.f, g_prev, C, s);
 }
 

@@ -173,7 +173,7 @@ int stream_scratch(hipStream_t s, size_t bytes, void** p);
 // slot 1 holds the hub pre-pass results, which must outlive a consumer that itself
 // takes slot 0; slot 2 holds the partial tiles of a GEMM split along k, whose operands
 // may sit in slot 0.
-constexpr int kScratchSlots = 3;
+constexpr int kScratchSlots = 5;     // 3: plan of the column-ordered SpMM, 4: its partial sums
 int stream_scratch_slot(hipStream_t s, int slot, size_t bytes, void** p);
 
 // reduce.hip: device address of the statically allocated segment offsets on the current device
@@ -191,9 +191,22 @@ struct HubPlan {
 };
 int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
                 const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan = false, bool relu_in = false);
-// spmm.hip: C = alpha*A*B + beta*C on stream s; reuse_plan as for hub_prepass
-int spmm_dispatch(int m, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+// spmm.hip: C = alpha*A*B + beta*C on stream s (A is [m,k]); reuse_plan as for hub_prepass
+int spmm_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan = false);
+
+// sort.hip
+int exclusive_scan_i32(int* x, long long n, int* seg_scratch, hipStream_t s);
+size_t radix_hist_ints(long long n);
+size_t radix_seg_ints(long long n);
+int radix_order_by_digit(const unsigned* keys, long long n, int shift, unsigned* keys_out, unsigned* perm_out, int* hist, int* seg,
+                         hipStream_t s);
+int spmm_plain_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+                        const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan = false);
+// pieces.hip: C = alpha*A*B + beta*C for large matrices with many entries per row, the rows cut into pieces that
+// are summed in the order of their first column; GNNHIP_EUNSUPPORTED where the caller keeps its own route
+int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+                         const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan);
 
 }  // namespace gnnhip
 

@@ -623,7 +623,7 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
         const bool two_step = N >= kHubMinRows && nnz >= two_step_degree() * (long long)N;
         if (relu_in && (two_step || !level_stream_covers(N, C))) return GNNHIP_EUNSUPPORTED;
         if (two_step) {
-            if (int rc = spmm_dispatch(N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, h_out, C, s, same_graph)) return rc;
+            if (int rc = spmm_dispatch(N, N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, h_out, C, s, same_graph)) return rc;
             const HubPlan none{nullptr, nullptr, 0};
             if (int rc = level_stream_dispatch(N, C, true, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, none, false, s);
                 rc != GNNHIP_EUNSUPPORTED)

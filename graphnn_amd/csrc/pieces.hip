@@ -1,0 +1,320 @@
+// CSR SpMM for large matrices with many entries per row (power-law graphs): column-ordered pieces.
+//
+// On an R-MAT matrix the gathers of C = A * B miss the 4 MB L2 of their die most of the time: the rows a
+// workgroup walks touch unrelated rows of B, and a popular row of B is fetched again and again (counted: ten
+// times the size of B).  CSR columns are sorted inside a row, so a run of consecutive entries of a long row
+// covers a narrow range of columns.  This pass cuts every row into pieces of at most kPiece consecutive
+// entries, orders the pieces by the column they start at (two stable radix passes on the top sixteen bits of
+// that column), copies the entries into that order, and sums the pieces in that order, each die taking one
+// contiguous eighth of it.  What runs together then starts in the same narrow band of B; measured on R-MAT
+// with 4M rows and 16 entries per row this brings the fetched bytes from 14 GB (pieces in row order) to 8 GB.
+//
+//   plan     pieces per row -> offsets (scan) -> piece records + keys -> order by first column ->
+//            entries copied in piece order (a CSR matrix whose rows are the pieces)
+//   sums     one lane group per piece, entries read front to back; the sums are stored in the order they are formed
+//   combine  C = P * sums + beta * C, P the 0/1 matrix that picks the pieces of a row in piece order
+//            (the plain row-group SpMM: rows without entries get beta * C, very long rows its hub pass)
+//
+// Every sum is taken in an order fixed by the matrix (no atomics): the result does not depend on scheduling.
+// The plan depends on A only (structure and values) and is reused by the later levels of one forward.
+// Bound: HBM / L2.  Algorithmic bytes as for the plain SpMM, plus 8 bytes of partial sums per column and piece.
+#include "gnnhip_internal.h"
+
+#include <cstdlib>
+
+namespace gnnhip {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kPiece = 32;              // entries per piece
+
+struct PieceRec { int start, end, id; };    // entries [start, end); id = first[row] + index of the piece in its row
+
+__device__ __forceinline__ int pieces_of(int deg) { return (deg + kPiece - 1) / kPiece; }
+
+// counts[r] = pieces of row r (counts[m] = 0, so that the scan leaves the total there)
+__global__ __launch_bounds__(kBlock) void piece_count_kernel(int m, const int* __restrict__ row_ptr, int* __restrict__ counts)
+{
+    for (long long r = (long long)blockIdx.x * kBlock + threadIdx.x; r <= m; r += (long long)gridDim.x * kBlock)
+        counts[r] = r < m ? pieces_of(row_ptr[r + 1] - row_ptr[r]) : 0;
+}
+
+// One lane per piece slot: the row that owns piece id is found by bisection in the scanned counts.
+// Slots at or past the number of pieces get an empty record and the largest key (they sort to the end).
+__global__ __launch_bounds__(kBlock) void piece_fill_kernel(int m, long long slots, const int* __restrict__ row_ptr,
+                                                            const int* __restrict__ col_idx, const int* __restrict__ first,
+                                                            int shift, PieceRec* __restrict__ rec, unsigned* __restrict__ keys)
+{
+    const int total = first[m];
+    for (long long id = (long long)blockIdx.x * kBlock + threadIdx.x; id < slots; id += (long long)gridDim.x * kBlock) {
+        if (id >= total) {
+            rec[id] = PieceRec{0, 0, (int)id};
+            keys[id] = 0xFFFFu;
+            continue;
+        }
+        int lo = 0, hi = m;                          // largest row with first[row] <= id
+        while (hi - lo > 1) {
+            const int mid = (int)(((long long)lo + hi) >> 1);
+            if (first[mid] <= (int)id) lo = mid; else hi = mid;
+        }
+        const int row = lo;
+        const int k = (int)id - first[row];
+        const int rb = row_ptr[row], re = row_ptr[row + 1];
+        const int start = rb + k * kPiece;
+        const int end = min(start + kPiece, re);
+        rec[id] = PieceRec{start, end, (int)id};
+        keys[id] = ((unsigned)col_idx[start] >> shift) & 0xFFFFu;
+    }
+}
+
+// ordered[i] = rec[perm[i]]
+__global__ __launch_bounds__(kBlock) void piece_permute_kernel(long long slots, const unsigned* __restrict__ perm,
+                                                               const PieceRec* __restrict__ rec, PieceRec* __restrict__ ordered)
+{
+    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < slots; i += (long long)gridDim.x * kBlock)
+        ordered[i] = rec[perm[i]];
+}
+
+// lens[i] = entries of the i-th piece in order (lens[slots] = 0, so that the scan leaves the total there);
+// where[id] = i, the place of piece id in the order; ones[i] = 1 (the values of the matrix that picks pieces)
+__global__ __launch_bounds__(kBlock) void piece_place_kernel(long long slots, const PieceRec* __restrict__ ordered, int* __restrict__ lens,
+                                                             int* __restrict__ where, float* __restrict__ ones)
+{
+    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i <= slots; i += (long long)gridDim.x * kBlock) {
+        if (i == slots) { lens[i] = 0; continue; }
+        const PieceRec r = ordered[i];
+        lens[i] = r.end - r.start;
+        where[r.id] = (int)i;
+        ones[i] = 1.f;
+    }
+}
+
+// Entries copied into piece order: half a wavefront per piece (kPiece = 32 entries, one per lane), four pieces
+// per turn so that their dependent loads (record, place, entry) overlap.  The empty pieces at the end are skipped.
+__global__ __launch_bounds__(kBlock) void piece_gather_kernel(const int* __restrict__ count, const PieceRec* __restrict__ ordered,
+                                                              const int* __restrict__ at, const int* __restrict__ col_idx,
+                                                              const float* __restrict__ val, int* __restrict__ col_out,
+                                                              float* __restrict__ val_out)
+{
+    static_assert(kPiece == 32, "one lane per entry of a piece");
+    constexpr int kTurn = 4;
+    const int sub = threadIdx.x & (kPiece - 1);
+    const long long per = kBlock / kPiece;
+    const long long total = *count;
+    for (long long i0 = ((long long)blockIdx.x * per + threadIdx.x / kPiece) * kTurn; i0 < total; i0 += (long long)gridDim.x * per * kTurn) {
+        PieceRec r[kTurn];
+        int dst[kTurn], c[kTurn];
+        float v[kTurn];
+#pragma unroll
+        for (int u = 0; u < kTurn; ++u) {
+            const bool live = i0 + u < total;
+            r[u] = live ? ordered[i0 + u] : PieceRec{0, 0, 0};
+            dst[u] = live ? at[i0 + u] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < kTurn; ++u) {
+            const bool live = r[u].start + sub < r[u].end;
+            c[u] = live ? col_idx[r[u].start + sub] : 0;
+            v[u] = live ? val[r[u].start + sub] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < kTurn; ++u)
+            if (r[u].start + sub < r[u].end) { col_out[dst[u] + sub] = c[u]; val_out[dst[u] + sub] = v[u]; }
+    }
+}
+
+template <int VEC> struct PV;
+template <> struct PV<4> {
+    using T = float4;
+    static __device__ __forceinline__ T zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+    static __device__ __forceinline__ T load(const float* p) { return *reinterpret_cast<const float4*>(p); }
+    static __device__ __forceinline__ void store(float* p, T v) { *reinterpret_cast<float4*>(p) = v; }
+    static __device__ __forceinline__ void fma(T& a, float s, T x) { a.x += s * x.x; a.y += s * x.y; a.z += s * x.z; a.w += s * x.w; }
+};
+template <> struct PV<1> {
+    using T = float;
+    static __device__ __forceinline__ T zero() { return 0.f; }
+    static __device__ __forceinline__ T load(const float* p) { return *p; }
+    static __device__ __forceinline__ void store(float* p, T v) { *p = v; }
+    static __device__ __forceinline__ void fma(T& a, float s, T x) { a += s * x; }
+};
+
+// One lane group (G lanes) per piece, pieces taken in order; die x (workgroups x, x + 8, ...) walks the
+// x-th eighth of that order front to back, a workgroup taking the next ngroups pieces of its die when the
+// hardware starts it (so the pieces in flight on a die stay close together in the order; a fixed stride per
+// workgroup lets them drift apart and costs a quarter more fetched bytes).  The launch covers the host's bound
+// on the number of pieces; workgroups past the real count leave at once.  Inner loop as in the row-group SpMM:
+// the group reads G column indices and values at once and hands them round by shuffle, four gathers in flight.
+template <int VEC, int ITERS>
+__global__ __launch_bounds__(kBlock) void piece_sum_kernel(
+    const int* __restrict__ count, int n, float alpha, const int* __restrict__ at, const int* __restrict__ col_idx, const float* __restrict__ val,
+    const float* __restrict__ B, int ldb, float* __restrict__ part, int ldp, int logG)
+{
+    using V = PV<VEC>;
+    const int G = 1 << logG;
+    const int sub = threadIdx.x & (G - 1);
+    const int grp = threadIdx.x >> logG;
+    const int ngroups = kBlock >> logG;
+    const int xcd = blockIdx.x % kNumXCD, bx = blockIdx.x / kNumXCD;
+    const long long total = *count;                               // the real pieces (the empty ones behind them are skipped)
+    const long long lo = total * xcd / kNumXCD, hi = total * (xcd + 1) / kNumXCD;
+    {
+        const long long i = lo + (long long)bx * ngroups + grp;
+        if (i >= hi) return;
+        const int start = at[i], end = at[i + 1];
+        typename V::T acc[ITERS];
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) acc[it] = V::zero();
+        for (int base = start; base < end; base += G) {
+            const int t = base + sub;
+            int c = 0;
+            float v = 0.f;
+            if (t < end) { c = col_idx[t]; v = alpha * val[t]; }
+            const int cnt = min(G, end - base);
+            for (int j = 0; j < cnt; j += 4) {
+                int cj[4];
+                float vj[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    cj[u] = __shfl(c, (j + u) & (G - 1), G);
+                    vj[u] = __shfl(v, (j + u) & (G - 1), G);
+                }
+#pragma unroll
+                for (int it = 0; it < ITERS; ++it) {
+                    const int col0 = (sub + it * G) * VEC;
+                    if (col0 < n) {
+                        typename V::T x[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+                            x[u] = (j + u < cnt) ? V::load(B + (size_t)cj[u] * ldb + col0) : V::zero();
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+                            if (j + u < cnt) V::fma(acc[it], vj[u], x[u]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int col0 = (sub + it * G) * VEC;
+            if (col0 < n) V::store(part + (size_t)i * ldp + col0, acc[it]);
+        }
+    }
+}
+
+inline int ilog2_ceil_p(int x)
+{
+    int l = 0;
+    while ((1 << l) < x) ++l;
+    return l;
+}
+inline size_t round_up_p(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// Mean entries per row from which a matrix of at least kHubMinRows rows takes this route;
+// GNNHIP_PIECES_DEGREE overrides it (read once; 0 switches the route off), which is how the crossover was measured.
+inline long long pieces_degree()
+{
+    static const long long d = [] {
+        const char* e = getenv("GNNHIP_PIECES_DEGREE");
+        return (e && *e) ? atoll(e) : 12ll;
+    }();
+    return d;
+}
+
+}  // namespace
+
+int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+                         const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
+{
+    const long long deg = pieces_degree();
+    if (deg <= 0 || m < kHubMinRows || nnz < deg * (long long)m || n > kWave * 16 || nnz >= (1ll << 31) - 64) return GNNHIP_EUNSUPPORTED;
+    const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && aligned16(B);
+    const int vec = vec4 ? 4 : 1;
+    const int units = (n + vec - 1) / vec;
+    const int logG = ilog2_ceil_p(units < kWave ? units : kWave);
+    const int G = 1 << logG;
+    const int iters = (units + G - 1) / G;                        // 1..4 (3 runs as 4)
+    const int ldp = (int)round_up_p((size_t)n, 4);
+
+    // Every row has at most one piece that is not full.  The host does not know how many pieces there are, so
+    // the arrays and the launches are sized for this bound; the slots past the real pieces hold empty pieces,
+    // ordered last, that no row picks.
+    const long long slots = nnz / kPiece + m;
+    if (slots >= (1ll << 31) - 64) return GNNHIP_EUNSUPPORTED;
+    size_t off = 0;
+    auto carve = [&](size_t bytes) { const size_t o = off; off = round_up_p(off + bytes, 256); return o; };
+    const size_t o_first = carve(sizeof(int) * ((size_t)m + 1)), o_where = carve(sizeof(int) * (size_t)slots);
+    const size_t o_at = carve(sizeof(int) * ((size_t)slots + 1)), o_ones = carve(sizeof(float) * (size_t)slots);
+    const size_t o_col = carve(sizeof(int) * (size_t)nnz), o_val = carve(sizeof(float) * (size_t)nnz);
+    const size_t longest = (size_t)(slots + 1 > (long long)m + 1 ? slots + 1 : (long long)m + 1);
+    const size_t o_seg = carve(sizeof(int) * (longest / 4096 + 2 + radix_seg_ints(slots)));
+    const size_t o_rec = carve(sizeof(PieceRec) * (size_t)slots), o_ord = carve(sizeof(PieceRec) * (size_t)slots);
+    const size_t o_keys = carve(sizeof(unsigned) * (size_t)slots), o_keys2 = carve(sizeof(unsigned) * (size_t)slots);
+    const size_t o_perm = carve(sizeof(unsigned) * (size_t)slots);
+    const size_t o_hist = carve(sizeof(int) * radix_hist_ints(slots));
+    void* base = nullptr;
+    if (int rc = stream_scratch_slot(s, 3, off, &base)) return rc;
+    void* pbase = nullptr;
+    if (int rc = stream_scratch_slot(s, 4, sizeof(float) * (size_t)slots * ldp, &pbase)) return rc;
+    char* b = static_cast<char*>(base);
+    int* first = reinterpret_cast<int*>(b + o_first);
+    int* where = reinterpret_cast<int*>(b + o_where);
+    int* at = reinterpret_cast<int*>(b + o_at);
+    float* ones = reinterpret_cast<float*>(b + o_ones);
+    int* col_ord = reinterpret_cast<int*>(b + o_col);
+    float* val_ord = reinterpret_cast<float*>(b + o_val);
+    int* seg = reinterpret_cast<int*>(b + o_seg);
+    PieceRec* rec = reinterpret_cast<PieceRec*>(b + o_rec);
+    PieceRec* ordered = reinterpret_cast<PieceRec*>(b + o_ord);
+    unsigned* keys = reinterpret_cast<unsigned*>(b + o_keys);
+    unsigned* keys2 = reinterpret_cast<unsigned*>(b + o_keys2);
+    unsigned* perm = reinterpret_cast<unsigned*>(b + o_perm);
+    int* hist = reinterpret_cast<int*>(b + o_hist);
+    float* part = static_cast<float*>(pbase);
+
+    struct Memo { hipStream_t s; const int* row_ptr; const int* col_idx; const float* val; int m; long long nnz; void* base; };
+    static thread_local Memo memo = {nullptr, nullptr, nullptr, nullptr, 0, 0, nullptr};
+    const bool planned = reuse_plan && memo.row_ptr == row_ptr && memo.col_idx == col_idx && memo.val == val && memo.s == s &&
+                         memo.m == m && memo.nnz == nnz && memo.base == base;
+    const unsigned egrid = kNumCU * 16;
+    if (!planned) {
+        hipLaunchKernelGGL(piece_count_kernel, dim3(egrid), dim3(kBlock), 0, s, m, row_ptr, first);
+        if (int rc = exclusive_scan_i32(first, (long long)m + 1, seg, s)) return rc;
+        int bits = 1;
+        while (bits < 31 && (1ll << bits) < (long long)k) ++bits;
+        const int shift = bits > 16 ? bits - 16 : 0;
+        hipLaunchKernelGGL(piece_fill_kernel, dim3(egrid), dim3(kBlock), 0, s, m, slots, row_ptr, col_idx, first, shift, rec, keys);
+        // two stable passes, low digit first: the pieces end up ordered by the top 16 bits of their first column
+        if (int rc = radix_order_by_digit(keys, slots, 0, keys2, perm, hist, seg, s)) return rc;
+        hipLaunchKernelGGL(piece_permute_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, perm, rec, ordered);
+        if (int rc = radix_order_by_digit(keys2, slots, 8, keys, perm, hist, seg, s)) return rc;
+        hipLaunchKernelGGL(piece_permute_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, perm, ordered, rec);
+        hipLaunchKernelGGL(piece_place_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, rec, at, where, ones);
+        if (int rc = exclusive_scan_i32(at, slots + 1, seg, s)) return rc;
+        hipLaunchKernelGGL(piece_gather_kernel, dim3(egrid), dim3(kBlock), 0, s, first + m, rec, at, col_idx, val, col_ord, val_ord);
+        GNNHIP_LAUNCH_CHECK("spmm_pieces plan");
+        memo = Memo{s, row_ptr, col_idx, val, m, nnz, base};
+    }
+    // workgroups for the bound on the pieces of one die, times the number of dies
+    const int sum_groups = kBlock >> logG;
+    const unsigned sgrid = (unsigned)(((slots + kNumXCD - 1) / kNumXCD + 1 + sum_groups - 1) / sum_groups) * kNumXCD;
+#define GNNHIP_PIECES_LAUNCH(V, I)                                                                                               \
+    hipLaunchKernelGGL((piece_sum_kernel<V, I>), dim3(sgrid), dim3(kBlock), 0, s, first + m, n, alpha, at, col_ord, val_ord, B, ldb, \
+                       part, ldp, logG)
+    if (vec4) {
+        if (iters <= 1) GNNHIP_PIECES_LAUNCH(4, 1);
+        else if (iters == 2) GNNHIP_PIECES_LAUNCH(4, 2);
+        else GNNHIP_PIECES_LAUNCH(4, 4);
+    } else {
+        if (iters <= 1) GNNHIP_PIECES_LAUNCH(1, 1);
+        else if (iters == 2) GNNHIP_PIECES_LAUNCH(1, 2);
+        else GNNHIP_PIECES_LAUNCH(1, 4);
+    }
+#undef GNNHIP_PIECES_LAUNCH
+    GNNHIP_LAUNCH_CHECK("spmm_pieces sums");
+    // C = P * part + beta * C: row r of P has a one at where[first[r] + j] for each of its pieces j, in piece order.
+    // `slots` stands in for the number of entries of P (an upper bound is all the row-group route needs).
+    return spmm_plain_dispatch(m, (int)slots, n, slots, 1.f, first, where, ones, part, ldp, beta, C, ldc, s, false);
+}
+
+}  // namespace gnnhip

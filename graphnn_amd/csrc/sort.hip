@@ -120,6 +120,8 @@ __global__ __launch_bounds__(kBlock) void scan_apply_kernel(int* __restrict__ x,
     }
 }
 
+}  // namespace
+
 // seg_scratch: at least ceil(n / 4096) ints.  n <= 4096 * 2^22 (the small scan handles what one
 // workgroup walks comfortably; far beyond every use here).
 int exclusive_scan_i32(int* x, long long n, int* seg_scratch, hipStream_t s)
@@ -132,6 +134,8 @@ int exclusive_scan_i32(int* x, long long n, int* seg_scratch, hipStream_t s)
     GNNHIP_LAUNCH_CHECK("exclusive_scan_i32");
     return GNNHIP_OK;
 }
+
+namespace {
 
 __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(
     const unsigned* __restrict__ keys, const unsigned* __restrict__ vals, long long n, int shift, int ntiles,
@@ -245,6 +249,24 @@ __global__ __launch_bounds__(kBlock) void expand_rows_kernel(int m, const int* _
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 }  // namespace
+
+// One stable pass of the radix sort: perm_out[i] = index of the key that comes i-th when the n keys are ordered by
+// the 8-bit digit (key >> shift) & 255 (equal digits keep their input order); keys_out receives the keys in that
+// order.  hist needs radix_hist_ints(n) ints, seg radix_seg_ints(n).
+size_t radix_hist_ints(long long n) { return (size_t)kDigits * (size_t)((n + kTile - 1) / kTile > 0 ? (n + kTile - 1) / kTile : 1); }
+size_t radix_seg_ints(long long n) { return (radix_hist_ints(n) + kScanSeg - 1) / kScanSeg + 1; }
+int radix_order_by_digit(const unsigned* keys, long long n, int shift, unsigned* keys_out, unsigned* perm_out, int* hist, int* seg,
+                         hipStream_t s)
+{
+    if (n <= 0) return GNNHIP_OK;
+    const int ntiles = (int)((n + kTile - 1) / kTile);
+    hipLaunchKernelGGL(radix_hist_kernel, dim3(ntiles), dim3(kBlock), 0, s, keys, n, shift, ntiles, hist);
+    if (int rc = exclusive_scan_i32(hist, (long long)kDigits * ntiles, seg, s)) return rc;
+    hipLaunchKernelGGL(radix_scatter_kernel, dim3(ntiles), dim3(kBlock), 0, s, keys, (const unsigned*)nullptr, n, shift, ntiles, hist,
+                       keys_out, perm_out, 1);
+    GNNHIP_LAUNCH_CHECK("radix_order_by_digit");
+    return GNNHIP_OK;
+}
 
 // Groups n pairs by key (0 <= key < rows) keeping input order inside a group:
 //   row_ptr[rows + 1], col_idx[i] = payload of the i-th pair in grouped order,

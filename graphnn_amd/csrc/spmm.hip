@@ -222,9 +222,21 @@ int launch_slab(int m, int n, float alpha, const int* row_ptr, const int* col_id
 }  // namespace
 
 // Shared with the fused forward: C = alpha*A*B + beta*C on stream s.
-int spmm_dispatch(int m, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+int spmm_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
 {
+    // large matrices with many entries per row (power-law graphs): rows cut into pieces, summed in column order
+    if (int rc = spmm_pieces_dispatch(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, s, reuse_plan);
+        rc != GNNHIP_EUNSUPPORTED)
+        return rc;
+    return spmm_plain_dispatch(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, s, reuse_plan);
+}
+
+// The row-group route alone (with its pass over very long rows); nnz may be an upper bound.
+int spmm_plain_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+                        const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
+{
+    (void)k;
     const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && aligned16(B) && aligned16(C);
     const int vec = vec4 ? 4 : 1;
     // columns are processed in slabs of at most 64 lanes * vec * 4
@@ -268,5 +280,5 @@ extern "C" int gnnhip_spmm_csr_f32(int m, int k, int n, int nnz, float alpha, co
     GNNHIP_REQUIRE(ldb >= n && ldc >= n, "leading dimension smaller than n in spmm (ldb=%d ldc=%d n=%d)", ldb, ldc, n);
     GNNHIP_REQUIRE(k == 0 || B, "null dense operand in spmm");   // col_idx / val may be null when A has no entries
     if (int rc = require_ready()) return rc;
-    return spmm_dispatch(m, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, as_stream(stream));
+    return spmm_dispatch(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, as_stream(stream));
 }

@@ -1124,6 +1124,33 @@ def test_spmm_hub_rows_balanced_pass(gpu, oracle, n):
     assert np.array_equal(got, _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m)))
 
 
+@pytest.mark.parametrize("n", [64, 128, 7, 36, 300])
+def test_spmm_column_ordered_pieces_on_a_power_law_matrix(gpu, oracle, n):
+    """R-MAT, 65,536 rows, 16 entries per row on average (rows of up to 13,000 entries, a third of the rows
+    empty): large and dense enough for the route that cuts rows into pieces of 32 entries and sums them in the
+    order of their first column; random weights, alpha and beta, the same bits on a second run"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(600 + n)
+    a = synth.rmat_csr(0x5EED0005, 16, 16 << 16)
+    N = 1 << 16
+    assert (np.diff(a[0]) == 0).sum() > 1000 and np.diff(a[0]).max() > 5000
+    v = (rng.random(a[1].size) * 0.2 - 0.05).astype(np.float32)
+    csr = (a[0], a[1], v)
+    B = rng.standard_normal((N, n)).astype(np.float32)
+    C0 = rng.standard_normal((N, n)).astype(np.float32)
+    got = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), N))
+    want, w64 = _spmm_want(oracle, *csr, B, N)
+    assert_parity("spmm", got, want, w64)
+    got2 = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), N, alpha=-0.5, beta=1.5, out=_t(C0, gpu)))
+    assert_parity("spmm", got2, *_spmm_want(oracle, *csr, B, N, alpha=-0.5, beta=1.5, C=C0))
+    assert np.array_equal(got, _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), N)))
+    # rows of at most 32 entries are one piece each: their sums are the row-order sums of the reference path
+    short = np.diff(a[0]) <= 32
+    unit = (a[0], a[1], np.ones_like(v))
+    got_u = _n(ops.spmm(*_csr_t(unit, gpu), _t(B, gpu), N))
+    assert np.array_equal(got_u[short], oracle.spmm(*unit, B, N)[short])
+
+
 @pytest.mark.parametrize("C", [16, 64])
 def test_level_hub_rows_balanced_pass(gpu, oracle, C):
     from graphnn_amd import ops
