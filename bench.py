@@ -143,8 +143,19 @@ def time_level_cfg4(dev):
     ms = _event_ms(lambda: ops.s2v_level(*a_d, h0, Wc, msg, out=out), 20)
     N, E, C = batch.num_nodes, int(a[1].size), cfg["C"]
     flops = 2.0 * N * C * C + 2.0 * E * C + 2.0 * N * C
+    # the readout (sum-pool + MLP + softmax, one workgroup per 16 graphs) and the whole forward of the configuration
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    s_d = tuple(map(t, s))
+    B, H, Q, L = batch.num_graphs, cfg["H"], cfg["Q"], cfg["L"]
+    X, Wn, W1, W2 = t(batch.one_hot()), t(w.W_n2l), t(w.W_h1), t(w.W_h2)
+    bufs = ops.ForwardBuffers(N, B, C, H, Q, dev)
+    ms_ro = _event_ms(lambda: ops.s2v_readout(*s_d, out, W1, W2, B), 20)
+    ms_fw = _event_ms(lambda: ops.s2v_forward(a_d, s_d, X, Wn, Wc, W1, W2, L, bufs=bufs), 20)
     return {"workload": "configuration 4: one level, %d nodes, %d entries, hidden %d" % (N, E, C),
             "kernel": "s2v_level_wide_kernel<256,8,false,64>", "avg_ms": ms, "flops": flops,
+            "readout": {"avg_ms": ms_ro, "kernel": "s2v_readout_tile_kernel<256>", "graphs": B,
+                        "algorithmic_GBps": (4.0 * N * C + 8.0 * N + 4.0 * B * (C + H + 2 * Q) + 4.0 * (C * H + H * Q)) / (ms_ro * 1e-3) / 1e9},
+            "forward": {"avg_ms": ms_fw, "levels": L, "graphs_per_s": B / (ms_fw * 1e-3)},
             "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS},
             "algorithmic_GBps": level_algorithmic_bytes(N, E, C) / (ms * 1e-3) / 1e9}

@@ -22,6 +22,9 @@ int readout_dispatch(int B, int C, int H, int Q, const int* s_row_ptr, const int
 int readout_wave_dispatch(int B, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                           const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
                           float* logits, float* probs, int* pred, hipStream_t s);
+int readout_tile_dispatch(int B, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                          const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
+                          float* logits, float* probs, int* pred, hipStream_t s);
 int gemm_dispatch(int transA, int transB, int m, int n, int k, float alpha, const float* A, int lda,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s);
 int row_softmax_dispatch(float* x, int rows, int cols, hipStream_t s);
@@ -95,7 +98,8 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const float* __restrict__ 
 
 constexpr int kWaveReadoutMinGraphs = 1024;        // below this a workgroup per graph
 constexpr int kWaveReadoutMaxMeanNodes = 2048;     // mean nodes per graph
-constexpr int kBlockReadoutMaxGraphsWide = 4096;   // hidden 128/256: above this SpMM + GEMM
+constexpr int kBlockReadoutMaxGraphsWide = 4096;   // hidden 128/256: above this a workgroup per tile of graphs (or SpMM + GEMM)
+constexpr int kTileReadoutMinGraphs = 4096;
 
 int readout_any(int B, int N, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                 const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
@@ -110,6 +114,9 @@ int readout_any(int B, int N, int C, int H, int Q, const int* s_row_ptr, const i
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
     // hidden 128/256: a workgroup per graph up to a few thousand graphs (256 graphs, hidden 256: 20 us against
     // 67 us for the seven launches below); 10,000 graphs: 116 against 106 us
+    if (C > 64 && B > kTileReadoutMinGraphs && (long long)N <= (long long)B * kWaveReadoutMaxMeanNodes)
+        rc = readout_tile_dispatch(B, C, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
+    if (rc != GNNHIP_EUNSUPPORTED) return rc;
     if (C <= 64 || B <= kBlockReadoutMaxGraphsWide)
         rc = readout_dispatch(B, C, H, Q, s_row_ptr, s_col_idx, s_val, h, Wh1, Wh2, pool, hidden, logits, probs, pred, s);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;

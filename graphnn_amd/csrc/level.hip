@@ -603,6 +603,15 @@ bool level_accepts_relu_input(int N, int C, long long nnz)
     return level_wide_covers(N, C) || level_stream_covers(N, C);
 }
 
+// row_ptr[i] = i (i <= n), col_idx[i] = i, val[i] = 1: the n x n identity in CSR form
+__global__ __launch_bounds__(kBlock) void identity_csr_kernel(int n, int* __restrict__ row_ptr, int* __restrict__ col_idx,
+                                                              float* __restrict__ val)
+{
+    const long long i = (long long)blockIdx.x * kBlock + threadIdx.x;
+    if (i <= n) row_ptr[i] = (int)i;
+    if (i < n) { col_idx[i] = (int)i; val[i] = 1.f; }
+}
+
 int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
                    const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph,
                    bool relu_in)
@@ -646,15 +655,28 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
         default: return launch_level<64, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, s);
         }
     }
+    if (!level_wide_covers(N, C)) return GNNHIP_EUNSUPPORTED;
     // The wide kernel sums a row of any length inside one wavefront.  Large graphs with many entries per row
-    // (in practice the skewed ones, see above) are left to the caller's unfused route, whose SpMM balances
-    // long rows.
-    if (N >= kHubMinRows && nnz >= two_step_degree() * (long long)N) return GNNHIP_EUNSUPPORTED;
-    switch (C) {
-    case 128:
-    case 256: return level_wide_dispatch(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, relu_in, s);
+    // (in practice the skewed ones, see above) take two steps: the SpMM, which balances long rows, leaves A * h_in
+    // in scratch, and the wide kernel reads those rows through the identity matrix (one entry per row: its
+    // gather becomes a plain read of the row, 12 bytes of indices against C * 4 of data) for the contraction
+    // and the epilogue.
+    if (N >= kHubMinRows && nnz >= two_step_degree() * (long long)N) {
+        if (relu_in) return GNNHIP_EUNSUPPORTED;
+        void *tmp = nullptr, *idp = nullptr;
+        if (int rc = stream_scratch(s, sizeof(float) * (size_t)N * C, &tmp)) return rc;
+        if (int rc = stream_scratch_slot(s, 5, sizeof(int) * (3 * (size_t)N + 1), &idp)) return rc;
+        float* agg = static_cast<float*>(tmp);
+        int* id_row_ptr = static_cast<int*>(idp);
+        int* id_col = id_row_ptr + N + 1;
+        float* id_val = reinterpret_cast<float*>(id_col + N);
+        if (int rc = spmm_dispatch(N, N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, agg, C, s, same_graph)) return rc;
+        hipLaunchKernelGGL(identity_csr_kernel, dim3((unsigned)(((long long)N + kBlock) / kBlock)), dim3(kBlock), 0, s, N, id_row_ptr,
+                           id_col, id_val);
+        GNNHIP_LAUNCH_CHECK("identity_csr");
+        return level_wide_dispatch(N, C, N, id_row_ptr, id_col, id_val, agg, W, msg, bias, h_out, false, s);
     }
-    return GNNHIP_EUNSUPPORTED;
+    return level_wide_dispatch(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, relu_in, s);
 }
 
 // u = A' dz and g_prev = u W^T in one pass (A' = the transposed adjacency in CSR form); GNNHIP_EUNSUPPORTED where

@@ -531,13 +531,16 @@ def test_level_every_row_length_up_to_70(gpu, oracle, C, N):
     assert_parity("level", got, want, w64)
 
 
-def test_wide_level_on_a_large_dense_skewed_graph(gpu, oracle):
-    """hidden 128 on a graph of 40,000 rows with 14 entries per row on average and two rows of 5,000 and
-    3,000 entries: the level leaves the wide fused kernel (one wavefront per row, whatever its length) for
-    SpMM with the balanced pass + GEMM + epilogue; the forward entry must not hand it ReLU-through-msg"""
+@pytest.mark.parametrize("C", [128, 256])
+def test_wide_level_on_a_large_dense_skewed_graph(gpu, oracle, C):
+    """hidden 128 / 256 on a graph of 40,000 rows with 14 entries per row on average and two rows of 5,000 and
+    3,000 entries: the level leaves the one-launch wide kernel (one wavefront per row, whatever its length) for
+    SpMM with the balanced pass, then the wide kernel's contraction and epilogue over the summed rows (read
+    through the identity matrix).  The result carries the bits of those two steps made by hand, which is how
+    the route shows; the forward entry must not hand it ReLU-through-msg"""
     from graphnn_amd import ops
     rng = np.random.default_rng(77)
-    N, C = 40_000, 128
+    N = 40_000
     lens = rng.integers(10, 17, N); lens[123] = 5_000; lens[39_999] = 3_000
     rp = np.zeros(N + 1, np.int32); np.cumsum(lens, out=rp[1:])
     nnz = int(rp[-1])
@@ -550,6 +553,19 @@ def test_wide_level_on_a_large_dense_skewed_graph(gpu, oracle):
     want, w64 = _level_want(oracle, rp, ci, v, h_in, W, msg, None)
     got = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu)))
     assert_parity("level", got, want, w64)
+    import torch
+    agg = ops.spmm(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), N)
+    eye = (torch.arange(N + 1, dtype=torch.int32, device=gpu), torch.arange(N, dtype=torch.int32, device=gpu),
+           torch.ones(N, dtype=torch.float32, device=gpu))
+    by_hand = _n(ops.s2v_level(*eye, agg, _t(W, gpu), _t(msg, gpu)))
+    assert np.array_equal(got, by_hand)
+    # with a bias row, and the same bits on a second run
+    bias = rng.standard_normal(C).astype(np.float32)
+    want_b, w64_b = _level_want(oracle, rp, ci, v, h_in, W, msg, bias)
+    got_b = _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu), bias=_t(bias, gpu)))
+    assert_parity("level", got_b, want_b, w64_b)
+    assert np.array_equal(got_b, _n(ops.s2v_level(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(h_in, gpu), _t(W, gpu), _t(msg, gpu),
+                                                 bias=_t(bias, gpu))))
 
 
 @pytest.mark.parametrize("C", [128, 256])
