@@ -194,6 +194,27 @@ def time_large_batch(dev, B=30000):
             "forward_one_launch": {"avg_ms": ms_one, "graphs_per_s": B / (ms_one * 1e-3)}}
 
 
+def time_one_launch_by_graphs(dev, sizes=(256, 400, 600, 1024, 2000)):
+    """The one-launch forward (label input) on the configuration-2 graph distribution at several batch sizes:
+    past 256 graphs (one per compute unit) a small launch ahead of it orders the graphs largest first."""
+    import torch
+    from graphnn_amd import batching, ops, synth
+    t = lambda arr: torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
+    res = {}
+    for B in sizes:
+        batch, w, cfg = synth.make_config(2, B=B)
+        a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+        s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+        a_d, s_d = tuple(map(t, a)), tuple(map(t, s))
+        lab = t(np.asarray(batch.node_label).astype(np.int32))
+        W = [t(x) for x in (w.W_n2l, w.W_conv, w.W_h1, w.W_h2)]
+        bb = ops.BatchedBuffers(batch.num_nodes, B, cfg["C"], cfg["H"], cfg["Q"], dev)
+        nmax = int(batch.graph_sizes.max())
+        ms = _event_ms(lambda: ops.s2v_forward_batched_labels(a_d, s_d, lab, *W, cfg["L"], nmax, bufs=bb), 30)
+        res[str(B)] = {"us": ms * 1e3, "graphs_per_s": B / (ms * 1e-3)}
+    return res
+
+
 def time_device_batch_assembly(dev):
     """CSR of A from the flat edge list of configuration 4 on the device (stable radix sort) and the CSR
     transposition used by the backward pass, beside the numpy host builder for the same edge list."""
@@ -312,7 +333,7 @@ def time_cfg5(dev, scale=22):
     return res
 
 
-def kernel_rooflines(dev):
+def kernel_rooflines(dev, forwards=None):
     """The other kernels of the path at the sizes they are built for, each against the roofline that bounds
     it: the hidden-256 level of configuration 4 against the FP32 matrix peak, the configuration-5 kernels
     (R-MAT, 4.2M rows) against HBM.  achieved = algorithmic bytes (or flops) per launch / HIP-event time."""
@@ -328,11 +349,16 @@ def kernel_rooflines(dev):
     c5 = time_cfg5(dev)
     N, E, C, B = c5["shape"]
     w5 = c5["workload"]
+    if forwards is not None:
+        forwards["configuration 4"] = {"forward": c4["forward"], "readout": c4["readout"]}
+        forwards["configuration 5"] = {"forward": c5["forward"]}
+        forwards["one_launch_by_graphs"] = time_one_launch_by_graphs(dev)
     return [
         r4,
-        hbm("s2v_level_stream_kernel<64,true,...> + hub_partial_kernel + spmm_rowgroup_kernel (two-launch level)", w5 + ": one level",
+        hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + spmm_rowgroup_kernel<4,1> (sums of a row's pieces) + "
+            "s2v_level_stream_kernel<64,true,...> (contraction over the summed rows)", w5 + ": one level, plan included",
             level_algorithmic_bytes(N, E, C), c5["level"]["avg_ms"], gather_GBps=c5["level"]["gather_GBps"]),
-        hbm("spmm_rowgroup_kernel<4,1> + hub_partial_kernel<4,1>", w5 + ": SpMM A*h",
+        hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + spmm_rowgroup_kernel<4,1>", w5 + ": SpMM A*h, plan included",
             spmm_algorithmic_bytes(N, N, E, C), c5["spmm"]["avg_ms"], gather_GBps=c5["spmm"]["gather_GBps"]),
         hbm("sgemm_skinny_rows_kernel<1>", w5 + ": node scores h*w", 4 * N * (C + 1), c5["score"]["avg_ms"]),
         hbm("exclusive_scan_kernel + jagged_softmax_kernel", w5 + ": jagged softmax over %d segments of 1024" % B,
@@ -620,12 +646,15 @@ def main():
     out["end_to_end"] = end_to_end_host_layer(host)
 
     if not args.no_rooflines:
-        out["rooflines"] = kernel_rooflines(dev)
+        out["forwards"] = {}
+        out["rooflines"] = kernel_rooflines(dev, out["forwards"])
+        out["training_step"] = training_step_host_layer(host)
 
     if args.extra:
         out["extra"] = {"large_batch": time_large_batch(dev),
-                        "device_batch_assembly": time_device_batch_assembly(dev),
-                        "training_step": training_step_host_layer(host)}
+                        "device_batch_assembly": time_device_batch_assembly(dev)}
+        if "training_step" not in out:
+            out["extra"]["training_step"] = training_step_host_layer(host)
 
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline(host)
     print(json.dumps(out))

@@ -83,8 +83,97 @@ struct GraphLds {
     }
 };
 
+// Batches of more graphs than compute units are taken largest graph first: the graph of rank r in that order
+// goes to workgroup r % gridDim.x as its (r / gridDim.x)-th graph.  Big graphs then start at once and small
+// ones fill the slots that free up (400 graphs of the 10..110-node distribution: 34 -> 28 us).  The order is by
+// the number of 16-row tiles, descending, equal counts in batch order.  It is worked out once per launch by the
+// one-workgroup kernel below, which leaves a record per rank (graph, first node, node count, first entry, end
+// of entries): the forward kernel then finds its graph with one read instead of two dependent ones.  Working
+// the order out inside every workgroup of the forward kernel was tried first and costs 2.4 .. 7 us per
+// workgroup, more than it saves.  What a graph's results are does not depend on the order.
+constexpr int kOrderMinGraphs = kNumCU;          // up to here every graph has a compute unit of its own
+constexpr int kOrderBlock = 1024;
+constexpr int kOrderSlots = 4;                   // graphs a lane looks at
+constexpr int kOrderMaxGraphs = kOrderSlots * kOrderBlock;
+constexpr int kOrderRec = 8;                     // ints per record (five used; 32-byte records)
+inline bool graphs_ordered(int B) { return B > kOrderMinGraphs && B <= kOrderMaxGraphs; }
+
+__global__ __launch_bounds__(kOrderBlock) void graph_order_kernel(int B, int n16max, const int* __restrict__ a_row_ptr,
+                                                                  const int* __restrict__ s_row_ptr, int* __restrict__ order)
+{
+    constexpr int kWaves = kOrderBlock / kWave;
+    // counts[(ncls - 1 - cls) * nchunks + chunk] = graphs of tile count cls among graphs 64 chunk .. 64 chunk + 63;
+    // an exclusive scan over that array in index order gives, for every (class, chunk), the rank of its first
+    // graph (classes descending, batch order inside a class).  Graphs the host's size bound does not cover
+    // form the top class: they come first and are refused by the forward kernel.
+    __shared__ int counts[(kOrderMaxGraphs / kWave) * 64];       // up to 64 chunks x 64 classes
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int ncls = n16max / 16 + 2;                            // <= 64 (host-checked)
+    const int nchunks = (B + kWave - 1) / kWave;
+    const int total = ncls * nchunks;
+    int first[kOrderSlots], count[kOrderSlots], e0[kOrderSlots], e1[kOrderSlots], cls[kOrderSlots];
+#pragma unroll
+    for (int j = 0; j < kOrderSlots; ++j) {
+        const int g = (wave + j * kWaves) * kWave + lane;
+        first[j] = 0; count[j] = -1; e0[j] = 0; e1[j] = 0;
+        if (g < B) { first[j] = s_row_ptr[g]; count[j] = s_row_ptr[g + 1] - first[j]; }
+    }
+#pragma unroll
+    for (int j = 0; j < kOrderSlots; ++j) {
+        const int g = (wave + j * kWaves) * kWave + lane;
+        const bool fits = count[j] >= 0 && count[j] <= n16max;
+        if (fits) { e0[j] = a_row_ptr[first[j]]; e1[j] = a_row_ptr[first[j] + count[j]]; }
+        cls[j] = g >= B ? -1 : fits ? (count[j] + 15) >> 4 : ncls - 1;
+    }
+#pragma unroll
+    for (int j = 0; j < kOrderSlots; ++j) {
+        const int ch = wave + j * kWaves;
+        if (ch < nchunks) {
+            for (int c = 0; c < ncls; ++c) {
+                const unsigned long long m = __ballot(cls[j] == c);
+                if (lane == 0) counts[(ncls - 1 - c) * nchunks + ch] = __popcll(m);
+            }
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        int carry = 0;
+        for (int base = 0; base < total; base += kWave) {
+            const int i = base + lane;
+            const int v = i < total ? counts[i] : 0;
+            int incl = v;
+#pragma unroll
+            for (int d = 1; d < kWave; d <<= 1) {
+                const int o = __shfl_up(incl, d, kWave);
+                if (lane >= d) incl += o;
+            }
+            if (i < total) counts[i] = carry + incl - v;
+            carry += __shfl(incl, kWave - 1, kWave);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kOrderSlots; ++j) {
+        const int ch = wave + j * kWaves;
+        if (ch < nchunks) {
+            unsigned long long mine = 0;
+            for (int c = 0; c < ncls; ++c) {
+                const unsigned long long m = __ballot(cls[j] == c);
+                if (cls[j] == c) mine = m;
+            }
+            if (cls[j] >= 0) {
+                const int rank = counts[(ncls - 1 - cls[j]) * nchunks + ch] + __popcll(mine & ((1ull << lane) - 1ull));
+                int4* rec = reinterpret_cast<int4*>(order + (size_t)rank * kOrderRec);
+                rec[0] = make_int4(ch * kWave + lane, first[j], count[j], e0[j]);
+                rec[1] = make_int4(e1[j], 0, 0, 0);
+            }
+        }
+    }
+}
+
 // WAVES wavefronts per workgroup (4, 8 or 16): chosen by the host so that the largest graph's
 // (column block x row tile) tasks spread over the wavefronts.
+// order: null (graphs in batch order), or the records graph_order_kernel left.
 template <int C, int KSX, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     int B, int K, unsigned k_magic, int H, int Q, int L, int n16max, int ecap,
@@ -93,7 +182,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     const float* __restrict__ X, const float* __restrict__ Wn2l, const float* __restrict__ Wc,
     const float* __restrict__ Wh1, const float* __restrict__ Wh2,
     float* __restrict__ msg, float* __restrict__ h_final, float* __restrict__ pool, float* __restrict__ hidden,
-    float* __restrict__ logits, float* __restrict__ probs, int* __restrict__ pred, int* __restrict__ status)
+    float* __restrict__ logits, float* __restrict__ probs, int* __restrict__ pred, int* __restrict__ status,
+    const int* __restrict__ order)
 {
     // KSX == 0: the node features arrive as one label per node (X points at int labels[N]) and the input
     // stage is a row lookup in W_n2l; otherwise X is the dense [N,K] matrix and KSX bounds its contraction steps
@@ -137,15 +227,23 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     GNNHIP_PHASE_MARK(0);
     // The position of the first graph (node range, then entry range) is asked for ahead of the weight
     // loads, so the two dependent trips to memory run under them instead of after them.
-    int next_node0 = 0, next_n = 0;
-    if ((int)blockIdx.x < B) { next_node0 = s_row_ptr[blockIdx.x]; next_n = s_row_ptr[blockIdx.x + 1] - next_node0; }
+    int next_g = blockIdx.x, next_node0 = 0, next_n = 0, next_e0 = 0, next_e1 = 0;
+    if ((int)blockIdx.x < B) {
+        if (order) {
+            const int4 r0 = *reinterpret_cast<const int4*>(order + (size_t)blockIdx.x * kOrderRec);
+            next_g = r0.x; next_node0 = r0.y; next_n = r0.z; next_e0 = r0.w;
+            next_e1 = order[(size_t)blockIdx.x * kOrderRec + 4];
+        } else {
+            next_node0 = s_row_ptr[blockIdx.x];
+            next_n = s_row_ptr[blockIdx.x + 1] - next_node0;
+        }
+    }
     // this wavefront's 16 columns of W^T, level contraction: wreg[s] = Wc[KS q + s][16 jb + t]
     float wreg[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s)
         wreg[s] = Wc[(size_t)(KS * ((tid0 & (kWave - 1)) >> 4) + s) * C + 16 * ((tid0 / kWave) % NJB) + (tid0 & 15)];
-    int next_e0 = 0, next_e1 = 0;
-    if ((int)blockIdx.x < B && next_n >= 0 && next_n <= n16max) {
+    if (!order && (int)blockIdx.x < B && next_n >= 0 && next_n <= n16max) {
         next_e0 = a_row_ptr[next_node0];
         next_e1 = a_row_ptr[next_node0 + next_n];
     }
@@ -175,7 +273,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     // the staged rows of X have stride KP floats and zeros from column K on
     const int srt = GraphLds::input_steps(K);
     const int KP = 4 * srt;
-    for (int g = blockIdx.x; g < B; g += gridDim.x) {
+    for (int slot = blockIdx.x; slot < B; slot += gridDim.x) {
         // The lane's coordinates are derived again for every graph from a value the compiler cannot see
         // through.  Otherwise every per-lane address of the loop body (a dozen 64-bit pointers) is computed
         // once ahead of the loop, does not fit the 128 registers of a 16-wavefront workgroup, and comes back
@@ -187,9 +285,18 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
         const int jb = wave % NJB, tsplit = wave / NJB;
         const int gi = tid / G, tx = tid % G;
         const int wx_lane_off = ((srt * q) * C + 16 * jb + t) * 4;
-        const bool first = (g == (int)blockIdx.x);
-        const int node0 = first ? next_node0 : s_row_ptr[g];
-        const int n = first ? next_n : s_row_ptr[g + 1] - node0;
+        const bool first = (slot == (int)blockIdx.x);   // the position of this graph was asked for at start-up
+        int g = slot, node0, n, rec_e0 = 0, rec_e1 = 0;
+        if (first) {
+            g = next_g; node0 = next_node0; n = next_n;
+        } else if (order) {
+            const int4 r0 = *reinterpret_cast<const int4*>(order + (size_t)slot * kOrderRec);
+            g = r0.x; node0 = r0.y; n = r0.z; rec_e0 = r0.w;
+            rec_e1 = order[(size_t)slot * kOrderRec + 4];
+        } else {
+            node0 = s_row_ptr[g];
+            n = s_row_ptr[g + 1] - node0;
+        }
         if (n > n16max || n < 0) {                      // host promised max_graph_nodes; refuse instead of overrunning LDS
             if (tid == 0 && status) atomicOr(status, 1);
             continue;
@@ -208,8 +315,8 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
         //      parked in the still unused agg buffer), and check the block-diagonal promise.  Everything a lane
         //      needs is asked for before anything is used, so the staging costs one trip to memory.
         float* xs = agg;
-        const int e0 = first ? next_e0 : a_row_ptr[node0];
-        const int ne = (first ? next_e1 : a_row_ptr[node0 + n]) - e0;
+        const int e0 = first ? next_e0 : order ? rec_e0 : a_row_ptr[node0];
+        const int ne = (first ? next_e1 : order ? rec_e1 : a_row_ptr[node0 + n]) - e0;
         const bool staged = (ne <= ecap);
         {
             const float* xg = X + (size_t)node0 * K;
@@ -567,10 +674,18 @@ int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
         return GNNHIP_EUNSUPPORTED;
     }
     const int grid = B < kNumCU * 4 ? B : kNumCU * 4;
+    int* order = nullptr;
+    if (graphs_ordered(B) && n16max / 16 + 2 <= 64) {
+        void* p = nullptr;
+        if (int rc = stream_scratch(s, sizeof(int) * kOrderRec * (size_t)B, &p)) return rc;
+        order = static_cast<int*>(p);
+        hipLaunchKernelGGL(graph_order_kernel, dim3(1), dim3(kOrderBlock), 0, s, B, n16max, a_row_ptr, s_row_ptr, order);
+        GNNHIP_LAUNCH_CHECK("graph_order");
+    }
     const unsigned k_magic = K >= 2 ? (unsigned)((0x100000000ull + (unsigned)K - 1) / (unsigned)K) : 0u;   // ceil(2^32 / K)
     hipLaunchKernelGGL((s2v_graph_forward_kernel<C, KSX, WAVES>), dim3(grid), dim3(kBlock), smem, s,
                        B, K, k_magic, H, Q, L, n16max, ecap, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val,
-                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status);
+                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, order);
     GNNHIP_LAUNCH_CHECK("s2v_graph_forward");
     return GNNHIP_OK;
 }

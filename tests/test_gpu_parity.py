@@ -934,6 +934,61 @@ def test_batched_forward_large_and_dense_graphs(gpu, oracle):
     assert max_rel(_n(gen.logits), _n(bufs.logits)) < PARITY_TOL
 
 
+@pytest.mark.parametrize("B,C,hi", [(257, 64, 110), (300, 16, 40), (1023, 64, 70), (1500, 32, 33), (1024, 16, 20), (1025, 16, 20),
+                                    (4096, 64, 40), (4097, 64, 40)])
+def test_batched_forward_takes_graphs_largest_first(gpu, oracle, B, C, hi):
+    """between 257 and 4,096 graphs the one-launch forward hands the graphs to its workgroups largest first (an
+    order a small launch ahead of it derives from the sizes), beyond that in batch order: every graph must come
+    out exactly once, with the bits
+    it has in a batch of at most 256 graphs (which is taken in batch order).  Sizes 1..hi, so several size
+    classes with many members each; one graph breaks the size promise and is refused (status bit 0) while
+    the others are unaffected"""
+    from graphnn_amd import ops
+    K, H, Q, L = 11, 16, 3, 2
+    seed = 7000 + B
+    batch = synth.molecule_batch(seed, B, K, Q, size_mode="uniform", size_lo=1, size_hi=hi)
+    w = synth.make_weights(synth.Stream(seed), K, C, H, Q)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    sizes = np.asarray(batch.graph_sizes).astype(np.int64)
+    off = np.concatenate([[0], np.cumsum(sizes)])
+    nmax = int(sizes.max())
+    wts = (_t(w.W_n2l, gpu), _t(w.W_conv, gpu), _t(w.W_h1, gpu), _t(w.W_h2, gpu))
+    keys = ("msg", "h_final", "pool", "hidden", "logits", "probs", "pred")
+    big = ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), *wts, L, nmax)
+    assert int(_n(big.status)[0]) == 0
+    got = {k: _n(getattr(big, k)) for k in keys}
+    for b0 in range(0, B, 256):
+        b1 = min(B, b0 + 256)
+        n0, n1 = int(off[b0]), int(off[b1])
+        e0, e1 = int(a[0][n0]), int(a[0][n1])
+        a_part = (a[0][n0:n1 + 1] - e0, a[1][e0:e1] - n0, a[2][e0:e1])
+        s_part = ((off[b0:b1 + 1] - n0).astype(np.int32), np.arange(n1 - n0, dtype=np.int32), np.ones(n1 - n0, np.float32))
+        part = ops.s2v_forward_batched(_csr_t(a_part, gpu), _csr_t(s_part, gpu), _t(X[n0:n1], gpu), *wts, L, nmax)
+        assert int(_n(part.status)[0]) == 0
+        for k in keys:
+            rows = slice(n0, n1) if k in ("msg", "h_final") else slice(b0, b1)
+            assert np.array_equal(got[k][rows], _n(getattr(part, k))), (k, b0)
+    if B <= 300:
+        want = _forward_want(oracle, a, s, X, w, L)
+        _assert_batched_matches(want, big, L)
+    # a promise one tile short of the largest graphs: they are refused, every other graph keeps its values
+    short = (nmax - 1) // 16 * 16
+    if short >= 16:
+        fresh = ops.BatchedBuffers(batch.num_nodes, B, C, H, Q, gpu)
+        for k in ("pool", "logits"):
+            getattr(fresh, k).fill_(-7.0)
+        ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), *wts, L, short, bufs=fresh)
+        assert int(_n(fresh.status)[0]) & 1
+        fits = sizes <= short
+        assert 0 < fits.sum() < B
+        # (a smaller promise may pick a workgroup shape that adds in another order: the same values, not the same bits)
+        assert max_rel(_n(fresh.logits)[fits], got["logits"][fits]) < PARITY_TOL
+        assert max_rel(_n(fresh.pool)[fits], got["pool"][fits]) < PARITY_TOL
+        assert np.all(_n(fresh.logits)[~fits] == -7.0)
+
+
 def test_batched_forward_dense_features_past_the_staging_registers(gpu, oracle):
     """64 real-valued feature columns on graphs of up to 190 nodes: a graph's block of X (12,160 floats) is longer
     than what the lanes stage in one go, and its rows outnumber the gather rounds kept in registers"""
