@@ -32,11 +32,19 @@ struct PieceRec { int start, end, id; };    // entries [start, end); id = first[
 
 __device__ __forceinline__ int pieces_of(int deg) { return (deg + kPiece - 1) / kPiece; }
 
-// counts[r] = pieces of row r (counts[m] = 0, so that the scan leaves the total there)
-__global__ __launch_bounds__(kBlock) void piece_count_kernel(int m, const int* __restrict__ row_ptr, int* __restrict__ counts)
+// counts[r] = pieces of row r (counts[m] = 0, so that the scan leaves the total there).  The host's entry count
+// `cap` sizes every array of the plan; should the matrix hold more entries than that, the rows that reach past
+// entry `cap` (the last rows) get no pieces and are summed from the CSR arrays by piece_tail_kernel.
+__global__ __launch_bounds__(kBlock) void piece_count_kernel(int m, const int* __restrict__ row_ptr, int cap, int* __restrict__ counts)
 {
-    for (long long r = (long long)blockIdx.x * kBlock + threadIdx.x; r <= m; r += (long long)gridDim.x * kBlock)
-        counts[r] = r < m ? pieces_of(row_ptr[r + 1] - row_ptr[r]) : 0;
+    for (long long r = (long long)blockIdx.x * kBlock + threadIdx.x; r <= m; r += (long long)gridDim.x * kBlock) {
+        int c = 0;
+        if (r < m) {
+            const int e1 = row_ptr[r + 1];
+            if (e1 <= cap) c = pieces_of(e1 - row_ptr[r]);
+        }
+        counts[r] = c;
+    }
 }
 
 // One lane per piece slot: the row that owns piece id is found by bisection in the scanned counts.
@@ -138,6 +146,9 @@ template <> struct PV<1> {
     static __device__ __forceinline__ void store(float* p, T v) { *p = v; }
     static __device__ __forceinline__ void fma(T& a, float s, T x) { a += s * x; }
 };
+template <int VEC> __device__ __forceinline__ typename PV<VEC>::T pv_add(typename PV<VEC>::T a, typename PV<VEC>::T b);
+template <> __device__ __forceinline__ float4 pv_add<4>(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+template <> __device__ __forceinline__ float pv_add<1>(float a, float b) { return a + b; }
 
 // One lane group (G lanes) per piece, pieces taken in order; die x (workgroups x, x + 8, ...) walks the
 // x-th eighth of that order front to back, a workgroup taking the next ngroups pieces of its die when the
@@ -202,6 +213,46 @@ __global__ __launch_bounds__(kBlock) void piece_sum_kernel(
     }
 }
 
+// The rows that reach past entry `cap` (none when the host's entry count is the matrix's own): C[row] += alpha * A[row] * B,
+// after the combine pass has left beta * C[row] there.  Rows are taken from the last one down, a lane group each;
+// the first row that ends inside the plan ends the walk.
+template <int VEC, int ITERS>
+__global__ __launch_bounds__(kBlock) void piece_tail_kernel(int m, int n, float alpha, const int* __restrict__ row_ptr, int cap,
+                                                            const int* __restrict__ col_idx, const float* __restrict__ val,
+                                                            const float* __restrict__ B, int ldb, float* C, int ldc, int logG)
+{
+    using V = PV<VEC>;
+    const int G = 1 << logG;
+    const int sub = threadIdx.x & (G - 1);
+    const int grp = threadIdx.x >> logG;
+    const int ngroups = kBlock >> logG;
+    for (long long back = (long long)blockIdx.x * ngroups + grp; back < m; back += (long long)gridDim.x * ngroups) {
+        const int row = m - 1 - (int)back;
+        const int start = row_ptr[row], end = row_ptr[row + 1];
+        if (end <= cap) break;
+        typename V::T acc[ITERS];
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) acc[it] = V::zero();
+        for (int t = start; t < end; ++t) {
+            const int c = col_idx[t];
+            const float v = alpha * val[t];
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int col0 = (sub + it * G) * VEC;
+                if (col0 < n) V::fma(acc[it], v, V::load(B + (size_t)c * ldb + col0));
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int col0 = (sub + it * G) * VEC;
+            if (col0 < n) {
+                float* dst = C + (size_t)row * ldc + col0;
+                V::store(dst, pv_add<VEC>(acc[it], V::load(dst)));
+            }
+        }
+    }
+}
+
 inline int ilog2_ceil_p(int x)
 {
     int l = 0;
@@ -227,10 +278,13 @@ int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const 
                          const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
 {
     const long long deg = pieces_degree();
-    if (deg <= 0 || m < kHubMinRows || nnz < deg * (long long)m || n > kWave * 16 || nnz >= (1ll << 31) - 64) return GNNHIP_EUNSUPPORTED;
+    if (deg <= 0 || m < kHubMinRows || nnz < deg * (long long)m || nnz >= (1ll << 31) - 64) return GNNHIP_EUNSUPPORTED;
     const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && aligned16(B);
+    const bool cvec4 = vec4 && (ldc % 4 == 0) && aligned16(C);     // the pass that reads and writes C
     const int vec = vec4 ? 4 : 1;
     const int units = (n + vec - 1) / vec;
+    // a lane group covers at most 64 x 4 column units (wider operands stay with the caller's route, which cuts them into slabs)
+    if (units > kWave * 4 || (n + (cvec4 ? 4 : 1) - 1) / (cvec4 ? 4 : 1) > kWave * 4) return GNNHIP_EUNSUPPORTED;
     const int logG = ilog2_ceil_p(units < kWave ? units : kWave);
     const int G = 1 << logG;
     const int iters = (units + G - 1) / G;                        // 1..4 (3 runs as 4)
@@ -278,7 +332,7 @@ int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const 
                          memo.m == m && memo.nnz == nnz && memo.base == base;
     const unsigned egrid = kNumCU * 16;
     if (!planned) {
-        hipLaunchKernelGGL(piece_count_kernel, dim3(egrid), dim3(kBlock), 0, s, m, row_ptr, first);
+        hipLaunchKernelGGL(piece_count_kernel, dim3(egrid), dim3(kBlock), 0, s, m, row_ptr, (int)nnz, first);
         if (int rc = exclusive_scan_i32(first, (long long)m + 1, seg, s)) return rc;
         int bits = 1;
         while (bits < 31 && (1ll << bits) < (long long)k) ++bits;
@@ -314,7 +368,30 @@ int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const 
     GNNHIP_LAUNCH_CHECK("spmm_pieces sums");
     // C = P * part + beta * C: row r of P has a one at where[first[r] + j] for each of its pieces j, in piece order.
     // `slots` stands in for the number of entries of P (an upper bound is all the row-group route needs).
-    return spmm_plain_dispatch(m, (int)slots, n, slots, 1.f, first, where, ones, part, ldp, beta, C, ldc, s, false);
+    if (int rc = spmm_plain_dispatch(m, (int)slots, n, slots, 1.f, first, where, ones, part, ldp, beta, C, ldc, s, false)) return rc;
+    // rows past the host's entry count, if any (C is read and written here: its own vector width)
+    const unsigned tgrid = kNumCU * 4;
+#define GNNHIP_PIECES_TAIL(V, I)                                                                                                  \
+    hipLaunchKernelGGL((piece_tail_kernel<V, I>), dim3(tgrid), dim3(kBlock), 0, s, m, n, alpha, row_ptr, (int)nnz, col_idx, val, \
+                       B, ldb, C, ldc, tlogG)
+    {
+        const int tvec = cvec4 ? 4 : 1;
+        const int tunits = (n + tvec - 1) / tvec;
+        const int tlogG = ilog2_ceil_p(tunits < kWave ? tunits : kWave);
+        const int titers = (tunits + (1 << tlogG) - 1) >> tlogG;
+        if (cvec4) {
+            if (titers <= 1) GNNHIP_PIECES_TAIL(4, 1);
+            else if (titers == 2) GNNHIP_PIECES_TAIL(4, 2);
+            else GNNHIP_PIECES_TAIL(4, 4);
+        } else {
+            if (titers <= 1) GNNHIP_PIECES_TAIL(1, 1);
+            else if (titers == 2) GNNHIP_PIECES_TAIL(1, 2);
+            else GNNHIP_PIECES_TAIL(1, 4);
+        }
+    }
+#undef GNNHIP_PIECES_TAIL
+    GNNHIP_LAUNCH_CHECK("spmm_pieces tail");
+    return GNNHIP_OK;
 }
 
 }  // namespace gnnhip

@@ -60,15 +60,18 @@ def _check_csr(row_ptr, col_idx, val, rows, name):
         raise ValueError("%s: col_idx and val differ in length" % name)
 
 
-def spmm(row_ptr, col_idx, val, B, m, alpha=1.0, beta=0.0, out=None):
-    """out[m,n] = alpha * A * B + beta * out, A CSR with m rows and B.shape[0] columns."""
+def spmm(row_ptr, col_idx, val, B, m, alpha=1.0, beta=0.0, out=None, nnz_hint=None):
+    """out[m,n] = alpha * A * B + beta * out, A CSR with m rows and B.shape[0] columns.
+    nnz_hint: the host-side entry count handed to the library (default: the arrays' length); it only sizes
+    scratch, so any value from 0 up must give the same values."""
     k, n = B.shape
     _check_csr(row_ptr, col_idx, val, m, "A")
     if out is None:
         out = torch.empty((m, n), dtype=torch.float32, device=B.device)
     elif tuple(out.shape) != (m, n):
         raise ValueError("out has the wrong shape")
-    check(_lib().gnnhip_spmm_csr_f32(m, k, n, int(col_idx.numel()), alpha, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"),
+    nnz = int(col_idx.numel()) if nnz_hint is None else int(nnz_hint)
+    check(_lib().gnnhip_spmm_csr_f32(m, k, n, nnz, alpha, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"),
                                      _f32(val, "val"), _f32(B, "B"), n, beta, _f32(out, "out"), n, _stream()))
     return out
 

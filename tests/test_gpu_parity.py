@@ -1220,6 +1220,14 @@ def test_spmm_column_ordered_pieces_on_a_power_law_matrix(gpu, oracle, n):
     unit = (a[0], a[1], np.ones_like(v))
     got_u = _n(ops.spmm(*_csr_t(unit, gpu), _t(B, gpu), N))
     assert np.array_equal(got_u[short], oracle.spmm(*unit, B, N)[short])
+    # a host-side entry count below the matrix's own (but still dense enough for this route): the plan covers the
+    # rows that end inside it, the last rows are summed from the CSR arrays
+    for hint in (a[1].size - 1, 13 * N):
+        got_h = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), N, alpha=-0.5, beta=1.5, out=_t(C0, gpu), nnz_hint=hint))
+        inside = a[0][1:] <= hint
+        assert 0 < inside.sum() < N
+        assert np.array_equal(got_h[inside], got2[inside]), hint
+        assert_parity("spmm", got_h, *_spmm_want(oracle, *csr, B, N, alpha=-0.5, beta=1.5, C=C0))
 
 
 @pytest.mark.parametrize("C", [16, 64])
