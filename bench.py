@@ -535,7 +535,7 @@ def main():
     ap.add_argument("--no-rooflines", action="store_true",
                     help="skip the configuration-4 / configuration-5 kernel rooflines")
     ap.add_argument("--only", default="", help="comma-separated legs to run alone (for profiling): "
-                                                "forward, spmm, cfg4, cfg5")
+                                                "forward, spmm, cfg4, cfg5, train, sizes")
     ap.add_argument("--mkl-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one element-wise copy kernel of known size (1 GiB read, 1 GiB written) "
@@ -568,6 +568,11 @@ def main():
             res["cfg4_level"] = time_level_cfg4(dev)
         if "cfg5" in legs:
             res["cfg5"] = time_cfg5(dev)
+        if "train" in legs:
+            _, host = build_forward_workload(dev)
+            res["training_step"] = training_step_host_layer(host)
+        if "sizes" in legs:
+            res["one_launch_by_graphs"] = time_one_launch_by_graphs(dev)
         if args.calibrate:
             n = 1 << 28
             src = torch.ones(n, device=dev, dtype=torch.float32)

@@ -285,6 +285,10 @@ int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const 
     const int units = (n + vec - 1) / vec;
     // a lane group covers at most 64 x 4 column units (wider operands stay with the caller's route, which cuts them into slabs)
     if (units > kWave * 4 || (n + (cvec4 ? 4 : 1) - 1) / (cvec4 ? 4 : 1) > kWave * 4) return GNNHIP_EUNSUPPORTED;
+    // Narrow operands stay with the row-group route: with fewer than eight lanes per piece a wavefront reads the
+    // entries of more than eight pieces at once, 128 bytes apart, and fetches whole lines for a few bytes each
+    // (width 4 on the 4M-row R-MAT matrix: 16.6 GB fetched, 2.7 ms against 0.26 ms).
+    if (units < 8) return GNNHIP_EUNSUPPORTED;
     const int logG = ilog2_ceil_p(units < kWave ? units : kWave);
     const int G = 1 << logG;
     const int iters = (units + G - 1) / G;                        // 1..4 (3 runs as 4)

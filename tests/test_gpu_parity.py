@@ -1195,11 +1195,12 @@ def test_spmm_hub_rows_balanced_pass(gpu, oracle, n):
     assert np.array_equal(got, _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m)))
 
 
-@pytest.mark.parametrize("n", [64, 128, 7, 36, 300])
+@pytest.mark.parametrize("n", [64, 128, 9, 36, 300, 32, 4])
 def test_spmm_column_ordered_pieces_on_a_power_law_matrix(gpu, oracle, n):
     """R-MAT, 65,536 rows, 16 entries per row on average (rows of up to 13,000 entries, a third of the rows
     empty): large and dense enough for the route that cuts rows into pieces of 32 entries and sums them in the
-    order of their first column; random weights, alpha and beta, the same bits on a second run"""
+    order of their first column (operands of at least eight column units; width 4 stays with the row-group
+    route); random weights, alpha and beta, the same bits on a second run"""
     from graphnn_amd import ops
     rng = np.random.default_rng(600 + n)
     a = synth.rmat_csr(0x5EED0005, 16, 16 << 16)
