@@ -205,6 +205,17 @@ int spmm_plain_dispatch(int m, int k, int n, long long nnz, float alpha, const i
                         const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan = false);
 // pieces.hip: C = alpha*A*B + beta*C for large matrices with many entries per row, the rows cut into pieces that
 // are summed in the order of their first column; GNNHIP_EUNSUPPORTED where the caller keeps its own route
+struct PiecesOperand {
+    const int* first;      // row pointers of P [m + 1]
+    const int* where;      // column indices of P: the place of each piece among the partial sums
+    const float* ones;     // values of P
+    const float* part;     // the partial sums [slots, ld]
+    int ld;
+    long long slots;       // columns of P (an upper bound of its entries)
+    bool plan_reused;
+};
+int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+                     const float* B, int ldb, hipStream_t s, bool reuse_plan, PiecesOperand* out);
 int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
                          const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan);
 

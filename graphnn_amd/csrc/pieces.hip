@@ -33,15 +33,16 @@ struct PieceRec { int start, end, id; };    // entries [start, end); id = first[
 __device__ __forceinline__ int pieces_of(int deg) { return (deg + kPiece - 1) / kPiece; }
 
 // counts[r] = pieces of row r (counts[m] = 0, so that the scan leaves the total there).  The host's entry count
-// `cap` sizes every array of the plan; should the matrix hold more entries than that, the rows that reach past
-// entry `cap` (the last rows) get no pieces and are summed from the CSR arrays by piece_tail_kernel.
+// `cap` sizes every array of the plan; should the matrix hold more entries than that, a row that reaches past
+// entry `cap` (the last rows) is one piece whatever its length: no entries are copied for it, and
+// piece_tail_kernel forms its sum from the CSR arrays.
 __global__ __launch_bounds__(kBlock) void piece_count_kernel(int m, const int* __restrict__ row_ptr, int cap, int* __restrict__ counts)
 {
     for (long long r = (long long)blockIdx.x * kBlock + threadIdx.x; r <= m; r += (long long)gridDim.x * kBlock) {
         int c = 0;
         if (r < m) {
-            const int e1 = row_ptr[r + 1];
-            if (e1 <= cap) c = pieces_of(e1 - row_ptr[r]);
+            const int e0 = row_ptr[r], e1 = row_ptr[r + 1];
+            c = e1 <= cap ? pieces_of(e1 - e0) : (e1 > e0 ? 1 : 0);
         }
         counts[r] = c;
     }
@@ -49,7 +50,7 @@ __global__ __launch_bounds__(kBlock) void piece_count_kernel(int m, const int* _
 
 // One lane per piece slot: the row that owns piece id is found by bisection in the scanned counts.
 // Slots at or past the number of pieces get an empty record and the largest key (they sort to the end).
-__global__ __launch_bounds__(kBlock) void piece_fill_kernel(int m, long long slots, const int* __restrict__ row_ptr,
+__global__ __launch_bounds__(kBlock) void piece_fill_kernel(int m, long long slots, const int* __restrict__ row_ptr, int cap,
                                                             const int* __restrict__ col_idx, const int* __restrict__ first,
                                                             int shift, PieceRec* __restrict__ rec, unsigned* __restrict__ keys)
 {
@@ -69,7 +70,7 @@ __global__ __launch_bounds__(kBlock) void piece_fill_kernel(int m, long long slo
         const int k = (int)id - first[row];
         const int rb = row_ptr[row], re = row_ptr[row + 1];
         const int start = rb + k * kPiece;
-        const int end = min(start + kPiece, re);
+        const int end = re <= cap ? min(start + kPiece, re) : start;     // a row past the host's count: an empty stand-in
         rec[id] = PieceRec{start, end, (int)id};
         keys[id] = ((unsigned)col_idx[start] >> shift) & 0xFFFFu;
     }
@@ -146,9 +147,6 @@ template <> struct PV<1> {
     static __device__ __forceinline__ void store(float* p, T v) { *p = v; }
     static __device__ __forceinline__ void fma(T& a, float s, T x) { a += s * x; }
 };
-template <int VEC> __device__ __forceinline__ typename PV<VEC>::T pv_add(typename PV<VEC>::T a, typename PV<VEC>::T b);
-template <> __device__ __forceinline__ float4 pv_add<4>(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
-template <> __device__ __forceinline__ float pv_add<1>(float a, float b) { return a + b; }
 
 // One lane group (G lanes) per piece, pieces taken in order; die x (workgroups x, x + 8, ...) walks the
 // x-th eighth of that order front to back, a workgroup taking the next ngroups pieces of its die when the
@@ -213,13 +211,14 @@ __global__ __launch_bounds__(kBlock) void piece_sum_kernel(
     }
 }
 
-// The rows that reach past entry `cap` (none when the host's entry count is the matrix's own): C[row] += alpha * A[row] * B,
-// after the combine pass has left beta * C[row] there.  Rows are taken from the last one down, a lane group each;
-// the first row that ends inside the plan ends the walk.
+// The rows that reach past entry `cap` (none when the host's entry count is the matrix's own): the sum of the row,
+// alpha * A[row] * B, goes where the row's one stand-in piece has its place among the partial sums.  Rows are
+// taken from the last one down, a lane group each; the first row that ends inside the plan ends the walk.
 template <int VEC, int ITERS>
 __global__ __launch_bounds__(kBlock) void piece_tail_kernel(int m, int n, float alpha, const int* __restrict__ row_ptr, int cap,
                                                             const int* __restrict__ col_idx, const float* __restrict__ val,
-                                                            const float* __restrict__ B, int ldb, float* C, int ldc, int logG)
+                                                            const float* __restrict__ B, int ldb, const int* __restrict__ first,
+                                                            const int* __restrict__ where, float* __restrict__ part, int ldp, int logG)
 {
     using V = PV<VEC>;
     const int G = 1 << logG;
@@ -230,6 +229,7 @@ __global__ __launch_bounds__(kBlock) void piece_tail_kernel(int m, int n, float 
         const int row = m - 1 - (int)back;
         const int start = row_ptr[row], end = row_ptr[row + 1];
         if (end <= cap) break;
+        if (start == end) continue;
         typename V::T acc[ITERS];
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) acc[it] = V::zero();
@@ -242,13 +242,11 @@ __global__ __launch_bounds__(kBlock) void piece_tail_kernel(int m, int n, float 
                 if (col0 < n) V::fma(acc[it], v, V::load(B + (size_t)c * ldb + col0));
             }
         }
+        float* dst = part + (size_t)where[first[row]] * ldp;
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
             const int col0 = (sub + it * G) * VEC;
-            if (col0 < n) {
-                float* dst = C + (size_t)row * ldc + col0;
-                V::store(dst, pv_add<VEC>(acc[it], V::load(dst)));
-            }
+            if (col0 < n) V::store(dst + col0, acc[it]);
         }
     }
 }
@@ -274,17 +272,19 @@ inline long long pieces_degree()
 
 }  // namespace
 
-int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                         const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
+// The partial sums alpha * (piece of A) * B of every piece, in column order, and the matrix P that picks the pieces of
+// each row (out->first / where / ones: CSR arrays of P [m, out->slots], out->part: the sums, row stride out->ld);
+// A * B is P * part.  GNNHIP_EUNSUPPORTED (nothing launched) where the caller keeps its own route.
+int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+                     const float* B, int ldb, hipStream_t s, bool reuse_plan, PiecesOperand* out)
 {
     const long long deg = pieces_degree();
     if (deg <= 0 || m < kHubMinRows || nnz < deg * (long long)m || nnz >= (1ll << 31) - 64) return GNNHIP_EUNSUPPORTED;
     const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && aligned16(B);
-    const bool cvec4 = vec4 && (ldc % 4 == 0) && aligned16(C);     // the pass that reads and writes C
     const int vec = vec4 ? 4 : 1;
     const int units = (n + vec - 1) / vec;
     // a lane group covers at most 64 x 4 column units (wider operands stay with the caller's route, which cuts them into slabs)
-    if (units > kWave * 4 || (n + (cvec4 ? 4 : 1) - 1) / (cvec4 ? 4 : 1) > kWave * 4) return GNNHIP_EUNSUPPORTED;
+    if (units > kWave * 4) return GNNHIP_EUNSUPPORTED;
     // Narrow operands stay with the row-group route: with fewer than eight lanes per piece a wavefront reads the
     // entries of more than eight pieces at once, 128 bytes apart, and fetches whole lines for a few bytes each
     // (width 4 on the 4M-row R-MAT matrix: 16.6 GB fetched, 2.7 ms against 0.26 ms).
@@ -341,7 +341,7 @@ int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const 
         int bits = 1;
         while (bits < 31 && (1ll << bits) < (long long)k) ++bits;
         const int shift = bits > 16 ? bits - 16 : 0;
-        hipLaunchKernelGGL(piece_fill_kernel, dim3(egrid), dim3(kBlock), 0, s, m, slots, row_ptr, col_idx, first, shift, rec, keys);
+        hipLaunchKernelGGL(piece_fill_kernel, dim3(egrid), dim3(kBlock), 0, s, m, slots, row_ptr, (int)nnz, col_idx, first, shift, rec, keys);
         // two stable passes, low digit first: the pieces end up ordered by the top 16 bits of their first column
         if (int rc = radix_order_by_digit(keys, slots, 0, keys2, perm, hist, seg, s)) return rc;
         hipLaunchKernelGGL(piece_permute_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, perm, rec, ordered);
@@ -370,32 +370,40 @@ int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const 
     }
 #undef GNNHIP_PIECES_LAUNCH
     GNNHIP_LAUNCH_CHECK("spmm_pieces sums");
-    // C = P * part + beta * C: row r of P has a one at where[first[r] + j] for each of its pieces j, in piece order.
-    // `slots` stands in for the number of entries of P (an upper bound is all the row-group route needs).
-    if (int rc = spmm_plain_dispatch(m, (int)slots, n, slots, 1.f, first, where, ones, part, ldp, beta, C, ldc, s, false)) return rc;
-    // rows past the host's entry count, if any (C is read and written here: its own vector width)
+    // rows past the host's entry count, if any: their sums go to the place of their stand-in piece
     const unsigned tgrid = kNumCU * 4;
 #define GNNHIP_PIECES_TAIL(V, I)                                                                                                  \
     hipLaunchKernelGGL((piece_tail_kernel<V, I>), dim3(tgrid), dim3(kBlock), 0, s, m, n, alpha, row_ptr, (int)nnz, col_idx, val, \
-                       B, ldb, C, ldc, tlogG)
-    {
-        const int tvec = cvec4 ? 4 : 1;
-        const int tunits = (n + tvec - 1) / tvec;
-        const int tlogG = ilog2_ceil_p(tunits < kWave ? tunits : kWave);
-        const int titers = (tunits + (1 << tlogG) - 1) >> tlogG;
-        if (cvec4) {
-            if (titers <= 1) GNNHIP_PIECES_TAIL(4, 1);
-            else if (titers == 2) GNNHIP_PIECES_TAIL(4, 2);
-            else GNNHIP_PIECES_TAIL(4, 4);
-        } else {
-            if (titers <= 1) GNNHIP_PIECES_TAIL(1, 1);
-            else if (titers == 2) GNNHIP_PIECES_TAIL(1, 2);
-            else GNNHIP_PIECES_TAIL(1, 4);
-        }
+                       B, ldb, first, where, part, ldp, logG)
+    if (vec4) {
+        if (iters <= 1) GNNHIP_PIECES_TAIL(4, 1);
+        else if (iters == 2) GNNHIP_PIECES_TAIL(4, 2);
+        else GNNHIP_PIECES_TAIL(4, 4);
+    } else {
+        if (iters <= 1) GNNHIP_PIECES_TAIL(1, 1);
+        else if (iters == 2) GNNHIP_PIECES_TAIL(1, 2);
+        else GNNHIP_PIECES_TAIL(1, 4);
     }
 #undef GNNHIP_PIECES_TAIL
     GNNHIP_LAUNCH_CHECK("spmm_pieces tail");
+    out->first = first;
+    out->where = where;
+    out->ones = ones;
+    out->part = part;
+    out->ld = ldp;
+    out->slots = slots;
+    out->plan_reused = planned;
     return GNNHIP_OK;
+}
+
+int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+                         const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
+{
+    PiecesOperand po;
+    if (int rc = spmm_pieces_sums(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, s, reuse_plan, &po)) return rc;
+    // C = P * part + beta * C: row r of P has a one at where[first[r] + j] for each of its pieces j, in piece order.
+    // `slots` stands in for the number of entries of P (an upper bound is all the row-group route needs).
+    return spmm_plain_dispatch(m, (int)po.slots, n, po.slots, 1.f, po.first, po.where, po.ones, po.part, po.ld, beta, C, ldc, s, false);
 }
 
 }  // namespace gnnhip
