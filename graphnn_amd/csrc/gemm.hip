@@ -204,13 +204,13 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(
 }
 
 // The same product for k <= 256: a lane keeps its four rows of B in registers, the groups stride the rows of A
-// four at a time (four 128-bit loads in flight per lane), and groups of up to 16 lanes reduce with DPP.
+// eight at a time (eight 128-bit loads in flight per lane), and groups of up to 16 lanes reduce with DPP.
 template <int NCOL, bool TB>
 __global__ __launch_bounds__(kBlock) void sgemm_skinny_rows_kernel(
     int m, int k, float alpha, const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb,
     float beta, float* C, int ldc, int logG)
 {
-    constexpr int R = 4;
+    constexpr int R = 8;
     const int G = 1 << logG;
     const int sub = threadIdx.x & (G - 1);
     const int kk = sub * 4;
@@ -266,7 +266,7 @@ void launch_skinny(bool tb, int m, int k, float alpha, const float* A, int lda, 
     while ((4 << logG) < k && logG < 6) ++logG;              // G * 4 >= k, at most one wavefront per row
     if (k <= 4 * kWave) {
         const size_t lanes = (size_t)m << logG;
-        size_t blocks = ceil_div_u(ceil_div_u(lanes, 4), kBlock);          // four rows per group
+        size_t blocks = ceil_div_u(ceil_div_u(lanes, 8), kBlock);          // eight rows per group
         if (blocks > (size_t)kNumCU * 32) blocks = (size_t)kNumCU * 32;
         if (blocks < 1) blocks = 1;
         const unsigned grid = (unsigned)blocks;

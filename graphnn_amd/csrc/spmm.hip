@@ -26,6 +26,7 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kLongRow = 2048;      // entries; longer rows are processed by the whole workgroup
+constexpr long long kOneRowMeanEntries = 256;   // mean entries per row from which every row gets a workgroup (matrices below kHubMinRows rows)
 
 // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one contiguous
 // slice of the row space so rows that share neighbours share an L2.
@@ -62,6 +63,8 @@ template <> struct Vec<1> {
 // Rows longer than long_row entries are parked in an LDS list and processed
 // afterwards by the whole workgroup: group g takes entries g, g + ngroups, ...
 // and the partial sums are added through LDS in group order.
+// long_row < 0: one row per workgroup, summed that way whatever its length (few, long rows: pooling 1,024 nodes
+// into each of 4,096 subgraphs ran one workgroup per compute unit with a lane group per row: 0.265 ms).
 template <int VEC, int ITERS>
 __global__ __launch_bounds__(kBlock) void spmm_rowgroup_kernel(
     int m, int n, float alpha, const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
@@ -78,18 +81,20 @@ __global__ __launch_bounds__(kBlock) void spmm_rowgroup_kernel(
     const int grp = threadIdx.x >> logG;
     const int ngroups = kBlock >> logG;
     const unsigned bid = xcd_remap(blockIdx.x, gridDim.x);
-    const long long row = (long long)bid * ngroups + grp;
+    const bool one_row = long_row < 0;
+    const bool owner = !one_row || grp == 0;          // the lane group that answers for `row`
+    const long long row = one_row ? (long long)bid : (long long)bid * ngroups + grp;
 
     if (threadIdx.x == 0) lr_count = 0;
     __syncthreads();
 
     int start = 0, end = 0;
-    if (row < m) { start = row_ptr[row]; end = row_ptr[row + 1]; }
+    if (row < m && owner) { start = row_ptr[row]; end = row_ptr[row + 1]; }
     // a row summed by the hub pre-pass only scales and stores
     int hslot = -1;
     if (hub_slot && end - start > kHubThreshold) hslot = hub_slot[row];
     if (hslot >= 0) end = start;
-    const bool deferred = (end - start > long_row);
+    const bool deferred = one_row ? (end > start) : (end - start > long_row);
     if (deferred) {
         if (sub == 0) lr_list[atomicAdd(&lr_count, 1)] = (int)row;
         end = start;      // the group idles through the main phase
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(kBlock) void spmm_rowgroup_kernel(
         }
     }
 
-    if (row < m && !deferred) {
+    if (row < m && !deferred && owner) {
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
             const int col0 = (sub + it * G) * VEC;
@@ -209,12 +214,13 @@ inline int ilog2_ceil(int x)
 
 template <int VEC, int ITERS>
 int launch_slab(int m, int n, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                const float* B, int ldb, float beta, float* C, int ldc, int logG, const HubPlan& hubs, hipStream_t s)
+                const float* B, int ldb, float beta, float* C, int ldc, int logG, const HubPlan& hubs, bool one_row, hipStream_t s)
 {
-    const int groups_per_block = kBlock >> logG;
+    const int groups_per_block = one_row ? 1 : kBlock >> logG;
     const unsigned blocks = ceil_div_u((size_t)m, (size_t)groups_per_block);
     hipLaunchKernelGGL((spmm_rowgroup_kernel<VEC, ITERS>), dim3(blocks), dim3(kBlock), 0, s,
-                       m, n, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, logG, kLongRow, hubs.row_slot, hubs.agg, hubs.ld);
+                       m, n, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, logG, one_row ? -1 : kLongRow, hubs.row_slot, hubs.agg,
+                       hubs.ld);
     GNNHIP_LAUNCH_CHECK("spmm_rowgroup");
     return GNNHIP_OK;
 }
@@ -237,6 +243,8 @@ int spmm_plain_dispatch(int m, int k, int n, long long nnz, float alpha, const i
                         const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
 {
     (void)k;
+    // few rows of hundreds of entries each (sum-pooling into subgraphs): a workgroup per row instead of a lane group
+    const bool one_row = m < kHubMinRows && nnz >= kOneRowMeanEntries * (long long)m;
     const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && aligned16(B) && aligned16(C);
     const int vec = vec4 ? 4 : 1;
     // columns are processed in slabs of at most 64 lanes * vec * 4
@@ -253,13 +261,13 @@ int spmm_plain_dispatch(int m, int k, int n, long long nnz, float alpha, const i
         HubPlan hubs;
         if ((rc = hub_prepass(m, w, nnz, row_ptr, col_idx, val, Bs, ldb, s, &hubs, reuse_plan && n <= slab_max))) return rc;
         if (vec4) {
-            if (iters <= 1) rc = launch_slab<4, 1>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
-            else if (iters == 2) rc = launch_slab<4, 2>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
-            else rc = launch_slab<4, 4>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
+            if (iters <= 1) rc = launch_slab<4, 1>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, one_row, s);
+            else if (iters == 2) rc = launch_slab<4, 2>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, one_row, s);
+            else rc = launch_slab<4, 4>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, one_row, s);
         } else {
-            if (iters <= 1) rc = launch_slab<1, 1>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
-            else if (iters == 2) rc = launch_slab<1, 2>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
-            else rc = launch_slab<1, 4>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, s);
+            if (iters <= 1) rc = launch_slab<1, 1>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, one_row, s);
+            else if (iters == 2) rc = launch_slab<1, 2>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, one_row, s);
+            else rc = launch_slab<1, 4>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, one_row, s);
         }
         if (rc) return rc;
     }

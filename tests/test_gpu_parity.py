@@ -1195,6 +1195,34 @@ def test_spmm_hub_rows_balanced_pass(gpu, oracle, n):
     assert np.array_equal(got, _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m)))
 
 
+@pytest.mark.parametrize("m,n", [(37, 64), (300, 7), (1, 128), (2000, 300), (4096, 4)])
+def test_spmm_few_long_rows_take_a_workgroup_each(gpu, oracle, m, n):
+    """rows of several hundred entries on average and fewer than 32,768 of them (sum-pooling into subgraphs): every
+    row is summed by a whole workgroup; empty rows, a row of one entry and a row of 5,000 among them; alpha, beta"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(900 + m + n)
+    k = 20_000
+    lens = rng.integers(200, 700, m)
+    lens[0] = 5_000
+    if m > 3:
+        lens[1] = 0; lens[2] = 1; lens[m - 1] = 0
+    rp = np.zeros(m + 1, np.int32); np.cumsum(lens, out=rp[1:])
+    nnz = int(rp[-1])
+    assert nnz >= 256 * m
+    ci = rng.integers(0, k, nnz).astype(np.int32)
+    v = (rng.random(nnz) * 0.2 - 0.05).astype(np.float32)
+    csr = (rp, ci, v)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    C0 = rng.standard_normal((m, n)).astype(np.float32)
+    got = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m))
+    assert_parity("spmm", got, *_spmm_want(oracle, *csr, B, m))
+    got2 = _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m, alpha=-0.5, beta=1.5, out=_t(C0, gpu)))
+    assert_parity("spmm", got2, *_spmm_want(oracle, *csr, B, m, alpha=-0.5, beta=1.5, C=C0))
+    assert np.array_equal(got, _n(ops.spmm(*_csr_t(csr, gpu), _t(B, gpu), m)))
+    if m > 3:
+        assert np.all(got[1] == 0) and np.array_equal(got2[1], (1.5 * C0[1]).astype(np.float32))
+
+
 @pytest.mark.parametrize("n", [64, 128, 9, 36, 300, 32, 4])
 def test_spmm_column_ordered_pieces_on_a_power_law_matrix(gpu, oracle, n):
     """R-MAT, 65,536 rows, 16 entries per row on average (rows of up to 13,000 entries, a third of the rows
