@@ -31,6 +31,7 @@ SIGNATURES = {
     "gnnhip_free": [_P],
     "gnnhip_pool_stats": [POINTER(c_size_t), POINTER(c_size_t), POINTER(c_size_t)],
     "gnnhip_memcpy_h2d": [_P, _P, _Z, _P],
+    "gnnhip_memcpy_h2d_sparse32": [_P, _P, _Z, _P],
     "gnnhip_memcpy_d2h": [_P, _P, _Z, _P],
     "gnnhip_memcpy_d2d": [_P, _P, _Z, _P],
     "gnnhip_memset0": [_P, _Z, _P],
@@ -69,7 +70,7 @@ SIGNATURES = {
     "gnnhip_row_scale_f32": [_I, _I, _P, _P, _P],
     "gnnhip_s2v_loss_acc_f32": [_I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_s2v_readout_backward_f32": [_I] * 5 + [_P] * 7 + [_F] + [_P] * 6 + [_P],
-    "gnnhip_s2v_level_backward_f32": [_I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P],
+    "gnnhip_s2v_level_backward_f32": [_I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_s2v_grad_gate_f32": [_Z, _P, _P, _P, _P, _I, _P],
     "gnnhip_momentum_sgd_batch_f32": [_I, _P, _P, _P, _P, _F, _F, _F, _P],
     "gnnhip_last_error": [],

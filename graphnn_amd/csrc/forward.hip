@@ -15,7 +15,7 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
                    bool relu_in = false);
 bool level_accepts_relu_input(int N, int C, long long nnz);
 int level_backward_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* dz,
-                            const float* W, float* u, float* g_prev, hipStream_t s);
+                            const float* W, float* u, float* g_prev, const float* gate, float* acc, hipStream_t s);
 int readout_dispatch(int B, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                      const float* h, const float* Wh1, const float* Wh2, float* pool, float* hidden,
                      float* logits, float* probs, int* pred, hipStream_t s);
@@ -166,18 +166,24 @@ int gnnhip_s2v_level_f32(int N, int C, int nnz, const int* row_ptr, const int* c
 }
 
 int gnnhip_s2v_level_backward_f32(int N, int C, int nnz, const int* t_row_ptr, const int* t_col_idx, const float* t_val,
-                                  const float* dz, const float* W, float* u, float* g_prev, void* stream)
+                                  const float* dz, const float* W, float* u, float* g_prev, const float* gate_h, float* acc,
+                                  void* stream)
 {
     GNNHIP_REQUIRE(N >= 0 && C >= 1 && nnz >= 0, "bad shape in s2v_level_backward (N=%d C=%d nnz=%d)", N, C, nnz);
     if (N == 0) return GNNHIP_OK;
     GNNHIP_REQUIRE(t_row_ptr && dz && W && u && g_prev, "null tensor in s2v_level_backward");
     GNNHIP_REQUIRE(dz != u && dz != g_prev && u != g_prev, "s2v_level_backward needs three distinct buffers");
+    GNNHIP_REQUIRE(acc != dz && acc != u && acc != g_prev && gate_h != g_prev && gate_h != u,
+                   "s2v_level_backward: acc and gate_h must not alias the other buffers");
     if (int rc = require_ready()) return rc;
     hipStream_t s = as_stream(stream);
-    int rc = level_backward_dispatch(N, C, nnz, t_row_ptr, t_col_idx, t_val, dz, W, u, g_prev, s);
+    int rc = level_backward_dispatch(N, C, nnz, t_row_ptr, t_col_idx, t_val, dz, W, u, g_prev, gate_h, acc, s);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
     if ((rc = spmm_dispatch(N, N, C, nnz, 1.f, t_row_ptr, t_col_idx, t_val, dz, C, 0.f, u, C, s))) return rc;
-    return gemm_dispatch(0, 1, N, C, C, 1.f, u, C, W, C, 0.f, g_prev, C, s);
+    if ((rc = gemm_dispatch(0, 1, N, C, C, 1.f, u, C, W, C, 0.f, g_prev, C, s))) return rc;
+    if (gate_h) return gnnhip_s2v_grad_gate_f32((size_t)N * C, gate_h, g_prev, g_prev, acc, 1, stream);
+    if (acc) return gnnhip_axpy_f32((size_t)N * C, 1.f, g_prev, acc, stream);
+    return GNNHIP_OK;
 }
 
 int gnnhip_s2v_readout_f32(int B, int N, int C, int H, int Q,

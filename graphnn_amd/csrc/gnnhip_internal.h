@@ -173,7 +173,7 @@ int stream_scratch(hipStream_t s, size_t bytes, void** p);
 // slot 1 holds the hub pre-pass results, which must outlive a consumer that itself
 // takes slot 0; slot 2 holds the partial tiles of a GEMM split along k, whose operands
 // may sit in slot 0.
-constexpr int kScratchSlots = 6;     // 3: plan of the column-ordered SpMM, 4: its partial sums, 5: identity matrix of the wide level
+constexpr int kScratchSlots = 7;     // 3: plan of the column-ordered SpMM, 4: its partial sums, 5: identity matrix of the wide level, 6: (index, value) pairs of a sparse upload
 int stream_scratch_slot(hipStream_t s, int slot, size_t bytes, void** p);
 
 // reduce.hip: device address of the statically allocated segment offsets on the current device

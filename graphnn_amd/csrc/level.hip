@@ -38,7 +38,8 @@ int level_stream_dispatch(int N, int C, bool dense, const int* row_ptr, const in
                           const HubPlan& hubs, bool relu_in, hipStream_t s);
 bool level_stream_covers(int N, int C);
 int level_stream_backward_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* x,
-                                   const float* W, float* agg_out, float* out, const HubPlan& hubs, hipStream_t s);
+                                   const float* W, float* agg_out, float* out, const float* gate, float* acc, const HubPlan& hubs,
+                                   hipStream_t s);
 // input_wide.hip
 int input_wide_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s);
 // level_wide.hip
@@ -682,14 +683,15 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
 // u = A' dz and g_prev = u W^T in one pass (A' = the transposed adjacency in CSR form); GNNHIP_EUNSUPPORTED where
 // the caller has to take the SpMM and the GEMM.
 int level_backward_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* dz,
-                            const float* W, float* u, float* g_prev, hipStream_t s)
+                            const float* W, float* u, float* g_prev, const float* gate, float* acc, hipStream_t s)
 {
     if (!(C == 16 || C == 32 || C == 64) || !level_stream_covers(N, C)) return GNNHIP_EUNSUPPORTED;
-    if (!(aligned16(dz) && aligned16(W) && aligned16(u) && aligned16(g_prev))) return GNNHIP_EUNSUPPORTED;
+    if (!(aligned16(dz) && aligned16(W) && aligned16(u) && aligned16(g_prev) && (!gate || aligned16(gate)) && (!acc || aligned16(acc))))
+        return GNNHIP_EUNSUPPORTED;
     if (N >= kHubMinRows && nnz >= two_step_degree() * (long long)N) return GNNHIP_EUNSUPPORTED;     // dense and skewed: balanced SpMM
     HubPlan hubs{nullptr, nullptr, 0};
     if (int rc = hub_prepass(N, C, nnz, row_ptr, col_idx, val, dz, C, s, &hubs, false, false)) return rc;
-    return level_stream_backward_dispatch(N, C, row_ptr, col_idx, val, dz, W, u, g_prev, hubs, s);
+    return level_stream_backward_dispatch(N, C, row_ptr, col_idx, val, dz, W, u, g_prev, gate, acc, hubs, s);
 }
 
 int readout_dispatch(int B, int C, int H, int Q, const int* s_row_ptr, const int* s_col_idx, const float* s_val,

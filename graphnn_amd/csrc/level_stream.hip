@@ -92,13 +92,15 @@ __device__ __forceinline__ void sum4(float4& acc, float w, const float4 (&x)[4])
 // MINW: wavefronts per SIMD the register allocation must leave room for
 // BWD: the backward pass of a level through the same machinery, out = (A' x) W^T with A' = A^T handed in as a
 // CSR matrix: W is read transposed, the aggregated rows A' x are also stored (agg_out: they are the other
-// factor of the weight gradient) and the result is stored as it is (no ReLU; msg and bias are null).
+// factor of the weight gradient).  No ReLU and no bias; `msg`, when given, is the embedding whose ReLU the
+// gradient passes next: out = out where msg > 0, else 0, and acc_io (when given) += out.
 template <int C, bool DENSE, bool WLDS, int MINW, bool RELU_IN, bool PIPE, bool BWD = false>
 __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
     int N, const int* __restrict__ row_ptr, const int* __restrict__ col_idx, const float* __restrict__ val,
     const float* __restrict__ h_in, const float* __restrict__ W, const float* __restrict__ msg,
     const float* __restrict__ bias, float* __restrict__ h_out,
-    const int* __restrict__ hub_slot, const float* __restrict__ hub_agg, int hub_ld, float* __restrict__ agg_out = nullptr)
+    const int* __restrict__ hub_slot, const float* __restrict__ hub_agg, int hub_ld, float* __restrict__ agg_out = nullptr,
+    float* __restrict__ acc_io = nullptr)
 {
     constexpr int G = C / 4;             // lanes per gathered row
     constexpr int RPR = kWave / G;       // lane groups per wavefront
@@ -413,9 +415,24 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
 #pragma unroll
         for (int rd = 0; rd < ROUNDS; ++rd) {
             float4 v = *reinterpret_cast<const float4*>(tile + (grp * ROUNDS + rd) * LDT + tx * 4);
-            if (bias) { v.x += bias4.x; v.y += bias4.y; v.z += bias4.z; v.w += bias4.w; }
-            v.x += mrow[rd].x; v.y += mrow[rd].y; v.z += mrow[rd].z; v.w += mrow[rd].w;
-            buf_store4(out_rsrc, out_off + rd * kRowBytes, 0, BWD ? v : relu_ref4(v));
+            if constexpr (BWD) {
+                if (msg) {
+                    v.x = mrow[rd].x > 0.f ? v.x : 0.f; v.y = mrow[rd].y > 0.f ? v.y : 0.f;
+                    v.z = mrow[rd].z > 0.f ? v.z : 0.f; v.w = mrow[rd].w > 0.f ? v.w : 0.f;
+                }
+                if (acc_io) {
+                    // every row belongs to one tile: nobody else touches it during the launch
+                    const rsrc_t acc_rsrc = make_rsrc(acc_io, act_bytes);
+                    float4 a = buf_load4(acc_rsrc, out_off + rd * kRowBytes, 0);
+                    a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+                    buf_store4(acc_rsrc, out_off + rd * kRowBytes, 0, a);
+                }
+                buf_store4(out_rsrc, out_off + rd * kRowBytes, 0, v);
+            } else {
+                if (bias) { v.x += bias4.x; v.y += bias4.y; v.z += bias4.z; v.w += bias4.w; }
+                v.x += mrow[rd].x; v.y += mrow[rd].y; v.z += mrow[rd].z; v.w += mrow[rd].w;
+                buf_store4(out_rsrc, out_off + rd * kRowBytes, 0, relu_ref4(v));
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");     // the tile is rewritten by the next iteration
         if constexpr (PIPE && !DENSE) {
@@ -477,7 +494,8 @@ int launch_level_stream_c(int N, bool dense, bool relu_in, const int* row_ptr, c
 
 template <int C>
 int launch_level_stream_backward(int N, const int* row_ptr, const int* col_idx, const float* val, const float* x,
-                                 const float* W, float* agg_out, float* out, const HubPlan& hubs, hipStream_t s)
+                                 const float* W, float* agg_out, float* out, const float* gate, float* acc, const HubPlan& hubs,
+                                 hipStream_t s)
 {
     const long long ntiles = ((long long)N + 15) / 16;
     long long blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
@@ -486,8 +504,8 @@ int launch_level_stream_backward(int N, const int* row_ptr, const int* col_idx, 
     const long long resident = (long long)kNumCU * kMinW;
     if (blocks > resident) blocks = resident;
     hipLaunchKernelGGL((s2v_level_stream_kernel<C, false, kWLds, kMinW, false, false, true>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
-                       N, row_ptr, col_idx, val, x, W, (const float*)nullptr, (const float*)nullptr, out, hubs.row_slot, hubs.agg,
-                       hubs.ld, agg_out);
+                       N, row_ptr, col_idx, val, x, W, gate, (const float*)nullptr, out, hubs.row_slot, hubs.agg,
+                       hubs.ld, agg_out, acc);
     GNNHIP_LAUNCH_CHECK("s2v_level_stream (backward)");
     return GNNHIP_OK;
 }
@@ -502,14 +520,16 @@ bool level_stream_covers(int N, int C)
 }
 
 // agg_out = A' x and out = agg_out W^T in one pass (A' in CSR form); same limits as level_stream_dispatch.
+// gate / acc (both may be null): out is zeroed where gate <= 0, then acc += out.
 int level_stream_backward_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* x,
-                                   const float* W, float* agg_out, float* out, const HubPlan& hubs, hipStream_t s)
+                                   const float* W, float* agg_out, float* out, const float* gate, float* acc, const HubPlan& hubs,
+                                   hipStream_t s)
 {
     if (!level_stream_covers(N, C)) return GNNHIP_EUNSUPPORTED;
     switch (C) {
-    case 16: return launch_level_stream_backward<16>(N, row_ptr, col_idx, val, x, W, agg_out, out, hubs, s);
-    case 32: return launch_level_stream_backward<32>(N, row_ptr, col_idx, val, x, W, agg_out, out, hubs, s);
-    default: return launch_level_stream_backward<64>(N, row_ptr, col_idx, val, x, W, agg_out, out, hubs, s);
+    case 16: return launch_level_stream_backward<16>(N, row_ptr, col_idx, val, x, W, agg_out, out, gate, acc, hubs, s);
+    case 32: return launch_level_stream_backward<32>(N, row_ptr, col_idx, val, x, W, agg_out, out, gate, acc, hubs, s);
+    default: return launch_level_stream_backward<64>(N, row_ptr, col_idx, val, x, W, agg_out, out, gate, acc, hubs, s);
     }
 }
 

@@ -440,8 +440,8 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
             // Backward of the folded forward (the gradient rules of src/nn/matmul.cpp:35-76, src/nn/relu.cu:18-37,
             // src/nn/elewise_add.cpp:35-52, src/nn/cross_entropy.cpp:52-78 and src/nn/reduce_mean.cpp:44-65 composed):
             //   g_L = S^T ((dlogits W2^T . [hidden > 0]) W1^T),  dlogits = (probs - y) / B
-            //   level l = L..1:  dz = g_l . [h_l > 0];  dmsg += dz;  u_l = A^T dz;  g_{l-1} = u_l W^T
-            //   dmsg += g_0 . [h_0 > 0]
+            //   dz_L = g_L . [h_L > 0];  dmsg = dz_L
+            //   level l = L..1:  u_l = A^T dz_l;  dz_{l-1} = (u_l W^T) . [h_{l-1} > 0];  dmsg += dz_{l-1}
             //   dW_conv += [h_0; ..; h_{L-1}]^T [u_1; ..; u_L],  dW_n2l += X^T dmsg,  dW_h1 += pool^T du,  dW_h2 += hidden^T dlogits
             // (A^T dz_l serves both the gradient of W, h_{l-1}^T (A^T dz_l) = (A h_{l-1})^T dz_l, and g_{l-1}.)
             step->backward = [=]() {
@@ -469,13 +469,14 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
                     auto& at = A->value.Transposed();
                     float* us = st->ustack.data->ptr;
                     float* g2 = st->g2.data->ptr;
+                    GNN_HIP(gnnhip_s2v_grad_gate_f32(NC, hs + (size_t)L * NC, g, g, dmsg, 0, s));
                     for (int l = L; l >= 1; --l) {
-                        GNN_HIP(gnnhip_s2v_grad_gate_f32(NC, hs + (size_t)l * NC, g, g, dmsg, l < L ? 1 : 0, s));
+                        // g_{l-1} comes out past the gate of h_{l-1} and is added to dmsg in the same pass
                         GNN_HIP(gnnhip_s2v_level_backward_f32((int)N, (int)C, at.nnz, at.row_ptr, at.col_idx, at.val, g,
-                                                              Wc->value.data->ptr, us + (size_t)(l - 1) * NC, g2, s));
+                                                              Wc->value.data->ptr, us + (size_t)(l - 1) * NC, g2,
+                                                              hs + (size_t)(l - 1) * NC, dmsg, s));
                         std::swap(g, g2);
                     }
-                    GNN_HIP(gnnhip_s2v_grad_gate_f32(NC, hs, g, nullptr, dmsg, 1, s));
                     if (!cWc)
                         GNN_HIP(gnnhip_gemm_f32(1, 0, (int)C, (int)C, (int)((size_t)L * N), 1.0f, hs, (int)C, us, (int)C, 1.0f,
                                                 Wc->grad.Full().data->ptr, (int)C, s));

@@ -35,7 +35,9 @@ public:
     void CopyFrom(DTensor<CPU, Dtype>& src)
     {
         Reshape(src.shape.dims);
-        GNN_HIP(gnnhip_memcpy_h2d(data->ptr, src.data->ptr, sizeof(Dtype) * shape.Count(), GpuHandle::Stream()));
+        // 32-bit elements: only the non-zero words travel when they are few (one-hot feature matrices)
+        static_assert(sizeof(Dtype) == 4, "dense GPU tensors hold 32-bit elements");
+        GNN_HIP(gnnhip_memcpy_h2d_sparse32(data->ptr, src.data->ptr, shape.Count(), GpuHandle::Stream()));
     }
     void CopyFrom(DTensor<GPU, Dtype>& src)
     {

@@ -480,8 +480,9 @@ def readout_backward(s_csr, probs, label_csr, scale, hidden, W_h1, W_h2, N):
     return dlogits, du, g_h
 
 
-def s2v_level_backward(t_row_ptr, t_col_idx, t_val, dz, W, u=None, g_prev=None):
-    """u = A^T dz, g_prev = u W^T; the CSR arrays are those of A^T"""
+def s2v_level_backward(t_row_ptr, t_col_idx, t_val, dz, W, u=None, g_prev=None, gate_h=None, acc=None):
+    """u = A^T dz, g_prev = u W^T (zeroed where gate_h <= 0 when gate_h is given), acc += g_prev when acc is given;
+    the CSR arrays are those of A^T"""
     N, C = dz.shape
     _check_csr(t_row_ptr, t_col_idx, t_val, N, "A^T")
     if u is None:
@@ -490,7 +491,7 @@ def s2v_level_backward(t_row_ptr, t_col_idx, t_val, dz, W, u=None, g_prev=None):
         g_prev = torch.empty_like(dz)
     check(_lib().gnnhip_s2v_level_backward_f32(N, C, int(t_col_idx.numel()), _i32(t_row_ptr, "t_row_ptr"), _i32(t_col_idx, "t_col_idx"),
                                                _f32(t_val, "t_val"), _f32(dz, "dz"), _f32(W, "W"), _f32(u, "u"), _f32(g_prev, "g_prev"),
-                                               _stream()))
+                                               _f32(gate_h, "gate_h"), _f32(acc, "acc"), _stream()))
     return u, g_prev
 
 
@@ -509,3 +510,17 @@ def momentum_sgd_batch(ws, gs, vs, lr, momentum, l2):
         _f32(t, "tensor")
     cnt = Z(*[t.numel() for t in ws])
     check(_lib().gnnhip_momentum_sgd_batch_f32(n, wp, gp, vp, cnt, float(lr), float(momentum), float(l2), _stream()))
+
+
+def upload_sparse32(host_array, out=None):
+    """Host numpy array of 32-bit elements -> device tensor through gnnhip_memcpy_h2d_sparse32 (non-zero words only
+    when they are few); the device tensor has the bits of the host array."""
+    import numpy as np
+    a = np.ascontiguousarray(host_array)
+    if a.dtype.itemsize != 4:
+        raise ValueError("upload_sparse32 takes 32-bit elements")
+    tdt = {"float32": torch.float32, "int32": torch.int32}[a.dtype.name]
+    if out is None:
+        out = torch.empty(a.shape, dtype=tdt, device="cuda")
+    check(_lib().gnnhip_memcpy_h2d_sparse32(ctypes.c_void_p(out.data_ptr()), a.ctypes.data_as(ctypes.c_void_p), a.size, _stream()))
+    return out

@@ -66,8 +66,12 @@ int gnnhip_pool_stats(size_t* bytes_in_use, size_t* bytes_parked, size_t* n_driv
  *      (src/tensor/gpu_dense_tensor.cu:97-150), SpTensor<GPU>::CopyFrom
  *      (src/tensor/gpu_sparse_tensor.cu:55-73).  h2d returns once the host buffer
  *      has been read (it may be overwritten at once); d2h blocks until the data is in
- *      host memory; d2d and memset0 are asynchronous on the stream. */
+ *      host memory; d2d and memset0 are asynchronous on the stream.
+ *      h2d_sparse32 is h2d for `words` 32-bit words that are mostly zero (the one-hot feature matrix GetBatch
+ *      fills, examples/graph_classification/include/nn_common.h:60-75): it sends the non-zero words with their
+ *      positions and rebuilds the buffer on the device (same bits, same promise); dense data takes the plain copy. */
 int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream);
+int gnnhip_memcpy_h2d_sparse32(void* dst_device, const void* src_host, size_t words, void* stream);
 int gnnhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
 int gnnhip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream);
 int gnnhip_memset0(void* device_ptr, size_t bytes, void* stream);
@@ -327,9 +331,14 @@ int gnnhip_s2v_grad_gate_f32(size_t n, const float* h, const float* g, float* dz
  *      in the other order, which is the same product; the reference runs cuSPARSE csrmm(T) + cuBLAS,
  *      src/tensor/gpu_dense_tensor.cu:271-294).  A^T is handed in as a CSR matrix [N,N] with nnz entries
  *      (gnnhip_csr_transpose_f32).  u [N,C] is also the other factor of the weight gradient:
- *      dW += h_prev^T * u  (= (A h_prev)^T dz).  dz, u and g_prev are three distinct buffers. */
+ *      dW += h_prev^T * u  (= (A h_prev)^T dz).  dz, u and g_prev are three distinct buffers.
+ *      gate_h (may be NULL): the embedding h_prev [N,C] whose ReLU the gradient passes next; g_prev is then stored
+ *      past that gate (g_prev where h_prev > 0, else 0: ReLUDeriv, src/nn/relu.cu:18-37), ready to be the dz of the
+ *      level below.  acc (may be NULL): acc += g_prev as stored (the gradient ElewiseAdd::Backward hands to msg,
+ *      src/nn/elewise_add.cpp:35-52, summed over the levels). */
 int gnnhip_s2v_level_backward_f32(int N, int C, int nnz, const int* t_row_ptr, const int* t_col_idx, const float* t_val,
-                                  const float* dz, const float* W, float* u, float* g_prev, void* stream);
+                                  const float* dz, const float* W, float* u, float* g_prev, const float* gate_h, float* acc,
+                                  void* stream);
 
 /* ---- MomentumSGDOptimizer::Update over n tensors in one launch (src/nn/optimizer.cpp:69-92):
  *      momentum > 0:  g += l2 w ; v = lr g + momentum v ; w -= v ; g = 0      (v: the optimizer's acc_grad_dict)

@@ -1488,3 +1488,34 @@ def test_device_csr_transpose(gpu, oracle, m, k, nnz):
     got = _n(ops.spmm(t_rp, t_ci, t_v, _t(B, gpu), k))
     assert max_rel(got, oracle.spmm_T(*csr, B, m, k)) < PARITY_TOL
     assert np.allclose(got, (A.T @ B), atol=1e-4)
+
+
+@pytest.mark.parametrize("shape,density", [((7450, 38), "one_hot"), ((7450, 38), 0.5), ((100, 7), "one_hot"), ((300_000, 64), "one_hot"),
+                                           ((16384,), 0.0), ((16385,), 1.0 / 17), ((40_000, 3), 1.0 / 15), ((5_000_000,), 0.001)])
+def test_sparse_upload_rebuilds_the_same_bits(gpu, shape, density):
+    """host-to-device copy that sends only the non-zero 32-bit words when they are at most one in sixteen (and the
+    plain copy otherwise, or below 16,384 words): the device buffer has the host's bits either way: negative zero
+    and denormals are non-zero words, the last word and the words around tile boundaries are hit, the destination
+    held other data before, and the host array may be overwritten at once"""
+    import torch
+    from graphnn_amd import ops
+    rng = np.random.default_rng(abs(hash((shape, str(density)))) % (2 ** 32))
+    n = int(np.prod(shape))
+    if density == "one_hot":
+        a = np.zeros(shape, np.float32)
+        a[np.arange(shape[0]), rng.integers(0, shape[1], shape[0])] = 1.0
+    else:
+        a = np.where(rng.random(n) < density, rng.standard_normal(n), 0.0).astype(np.float32).reshape(shape)
+    flat = a.reshape(-1)
+    if n > 20_000 and density != 0.5:
+        flat[-1] = -0.0                                       # a non-zero word, at the very end
+        flat[4095] = np.float32(1e-42); flat[4096] = 3.0       # a denormal and the first word of the second tile
+    want = flat.view(np.uint32).copy()
+    out = torch.full(shape, 7.0, dtype=torch.float32, device=gpu)
+    ops.upload_sparse32(a, out=out)
+    flat[:] = 5.0                                             # the host buffer has been read by now
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().reshape(-1).view(np.uint32), want)
+    # int32 data takes the same route
+    b = np.where(rng.random(50_000) < 0.02, rng.integers(-9, 9, 50_000), 0).astype(np.int32)
+    assert np.array_equal(ops.upload_sparse32(b).cpu().numpy(), b)

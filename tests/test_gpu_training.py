@@ -108,6 +108,21 @@ def test_level_backward(gpu, oracle, C, N):
     u64 = sp.csr_matrix((v.astype(np.float64), ci, rp), shape=(N, N)) @ dz.astype(np.float64)
     assert_parity("u", _n(u), w_u, u64)
     assert_parity("g_prev", _n(g), w_g, u64 @ W.astype(np.float64).T)
+    # with the ReLU gate of the level below and the running sum of the msg gradient: the stored g_prev is the
+    # ungated one with the closed gates zeroed (same bits), and acc grows by exactly what was stored
+    h_prev = rng.standard_normal((N, C)).astype(np.float32)
+    h_prev[rng.random((N, C)) < 0.1] = 0.0                       # zeros close the gate, like negative values
+    acc0 = rng.standard_normal((N, C)).astype(np.float32)
+    acc = _t(acc0, gpu)
+    u2, g2 = ops.s2v_level_backward(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(dz, gpu), _t(W, gpu), gate_h=_t(h_prev, gpu), acc=acc)
+    gated = np.where(h_prev > 0, _n(g), np.float32(0))
+    assert np.array_equal(_n(u2), _n(u))
+    assert np.array_equal(_n(g2), gated)
+    assert np.array_equal(_n(acc), acc0 + gated)
+    # the sum alone, without a gate
+    acc = _t(acc0, gpu)
+    _, g3 = ops.s2v_level_backward(_t(rp, gpu), _t(ci, gpu), _t(v, gpu), _t(dz, gpu), _t(W, gpu), acc=acc)
+    assert np.array_equal(_n(g3), _n(g)) and np.array_equal(_n(acc), acc0 + _n(g))
 
 
 def test_grad_gate_is_exact(gpu):
@@ -186,11 +201,11 @@ def test_training_iteration_composed_from_the_c_abi(gpu, oracle, config_id, C):
     us = torch.empty((L, N, C), device=gpu)
     dmsg = torch.empty((N, C), device=gpu)
     g2 = torch.empty_like(g)
+    ops.grad_gate(hs[L], g, g, dmsg, accumulate=False)
     for l in range(L, 0, -1):
-        ops.grad_gate(hs[l], g, g, dmsg, accumulate=(l < L))
-        ops.s2v_level_backward(*at, g, Wc, u=us[l - 1], g_prev=g2)
+        # the gradient comes out past the gate of the level below and is added to the msg gradient on the way
+        ops.s2v_level_backward(*at, g, Wc, u=us[l - 1], g_prev=g2, gate_h=hs[l - 1], acc=dmsg)
         g, g2 = g2, g
-    ops.grad_gate(hs[0], g, None, dmsg, accumulate=True)
     gWc = ops.gemm(hs[:L].reshape(L * N, C), us.reshape(L * N, C), transA=True)
     gWn = ops.gemm(X_d, dmsg, transA=True)
     gW1 = ops.gemm(pool, du, transA=True)
