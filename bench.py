@@ -5,7 +5,8 @@
 
 A step is one forward (input + L levels + readout) over one synthetic batch of
 configuration 2 (256 graphs, hidden 64, 4 levels) with every input already
-resident in HBM.  Prints ONE JSON line: graphs/s as `value`, plus
+resident in HBM, one batch at a time on one stream.  Prints ONE JSON line: graphs/s as `value`, plus
+  four_batches_in_flight  the same launch queued round-robin on four streams
   roofline      the CSR SpMM kernel on configuration 3 (1M rows, 10M entries,
                 width 128): algorithmic bytes / HIP-event time vs 8 TB/s
   cpu_baseline  the CPU restatement (oracle/) timed on this host's cores
@@ -79,6 +80,33 @@ def time_forward(dev_args, cfg, batch, steps, warmup, route):
     t1 = time.perf_counter()
     if route.startswith("graph_resident"):
         assert int(bufs.status.cpu()[0]) == 0, "graph-resident forward reported a layout violation"
+    return (t1 - t0) / steps, bufs
+
+
+def time_forward_pipelined(dev_args, cfg, batch, steps, warmup, nstreams=4):
+    """Wall-clock seconds per forward with `nstreams` batches in flight: the same one-launch forward queued
+    round-robin on several HIP streams (default priority), each stream with its own output buffers.  One
+    workgroup holds one graph and the launch lasts as long as its largest graph, so compute units that finish
+    early start on the next batch.  Returns (seconds per forward, list of the streams' buffers)."""
+    import torch
+    from graphnn_amd import ops
+    N, B = batch.num_nodes, batch.num_graphs
+    dev = dev_args[2].device
+    nmax = int(batch.graph_sizes.max())
+    streams = [torch.cuda.Stream() for _ in range(nstreams)]
+    bufs = [ops.BatchedBuffers(N, B, cfg["C"], cfg["H"], cfg["Q"], dev) for _ in range(nstreams)]
+    calls = [ops.bind_s2v_forward_batched(*dev_args, cfg["L"], nmax, bufs[i], streams[i]) for i in range(nstreams)]
+    torch.cuda.synchronize()
+    for i in range(warmup):
+        calls[i % nstreams]()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        calls[i % nstreams]()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for b in bufs:
+        assert int(b.status.cpu()[0]) == 0, "graph-resident forward reported a layout violation"
     return (t1 - t0) / steps, bufs
 
 
@@ -595,6 +623,10 @@ def main():
     assert float((bufs.logits - bufs_general.logits).abs().max()) <= 1e-4 * float(bufs_general.logits.abs().max()), \
         "routes disagree on logits"
 
+    sec_pipe, bufs_pipe = time_forward_pipelined(dev_args, cfg, batch, 4 * args.steps, args.warmup, 4)
+    for b in bufs_pipe:
+        assert bool(torch.equal(b.logits, bufs.logits)) and bool(torch.equal(b.pred, bufs.pred)), "pipelined forwards disagree"
+
     out = {
         "metric": "s2v forward graphs/sec (B=256,h=64,L=4); SpMM achieved HBM GB/s vs peak",
         "value": batch.num_graphs / sec,
@@ -618,6 +650,10 @@ def main():
                               "what": "gnnhip_s2v_forward_batched_labels_f32: the same launch fed one int label per node "
                                       "instead of the one-hot matrix X (bit-identical outputs); `value` keeps the "
                                       "reference's dense X"},
+        "four_batches_in_flight": {"graphs_per_s": batch.num_graphs / sec_pipe, "ms_per_step": sec_pipe * 1e3, "streams": 4,
+                                   "what": "the same launch queued round-robin on four HIP streams (own output buffers each, "
+                                           "bit-identical outputs): compute units that finish their graph early start on the next "
+                                           "batch; `value` keeps one batch at a time"},
         "general_route": {"graphs_per_s": batch.num_graphs / sec_general, "ms_per_step": sec_general * 1e3,
                           "what": "gnnhip_s2v_forward_f32: input + 4 fused levels + readout, any CSR"},
     }

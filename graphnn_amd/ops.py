@@ -235,6 +235,36 @@ def s2v_forward_batched(a_csr, s_csr, X, W_n2l, W_conv, W_h1, W_h2, L, max_graph
     return bufs
 
 
+def bind_s2v_forward_batched(a_csr, s_csr, X, W_n2l, W_conv, W_h1, W_h2, L, max_graph_nodes, bufs, stream):
+    """The call of s2v_forward_batched with every argument converted once: returns a function that queues one
+    forward on `stream` (a torch.cuda.Stream) and raises on a non-zero status code.  For callers that keep several
+    batches in flight on several streams, where the per-call argument checks of the helper above would be the
+    bottleneck."""
+    N, K = X.shape
+    C, H, Q = W_n2l.shape[1], W_h1.shape[1], W_h2.shape[1]
+    B = s_csr[0].numel() - 1
+    _check_csr(a_csr[0], a_csr[1], a_csr[2], N, "A")
+    _check_csr(s_csr[0], s_csr[1], s_csr[2], B, "S")
+    if s_csr[1].numel() != N:
+        raise ValueError("S must list every node exactly once")
+    if W_n2l.shape[0] != K or tuple(W_conv.shape) != (C, C) or W_h1.shape[0] != C or W_h2.shape[0] != H:
+        raise ValueError("weight shapes do not chain")
+    fn = _lib().gnnhip_s2v_forward_batched_f32
+    args = (N, B, K, C, H, Q, L, int(max_graph_nodes),
+            _i32(a_csr[0], "a_row_ptr"), _i32(a_csr[1], "a_col_idx"), _f32(a_csr[2], "a_val"),
+            _i32(s_csr[0], "s_row_ptr"), _i32(s_csr[1], "s_col_idx"), _f32(s_csr[2], "s_val"),
+            _f32(X, "X"), _f32(W_n2l, "W_n2l"), _f32(W_conv, "W_conv"), _f32(W_h1, "W_h1"), _f32(W_h2, "W_h2"),
+            _f32(bufs.msg, "msg"), _f32(bufs.h_final, "h_final"), _f32(bufs.pool, "pool"),
+            _f32(bufs.hidden, "hidden"), _f32(bufs.logits, "logits"), _f32(bufs.probs, "probs"),
+            _i32(bufs.pred, "pred"), _i32(bufs.status, "status"), ctypes.c_void_p(stream.cuda_stream))
+
+    def queue():
+        rc = fn(*args)
+        if rc:
+            check(rc)
+    return queue
+
+
 def s2v_forward_batched_labels(a_csr, s_csr, label, W_n2l, W_conv, W_h1, W_h2, L, max_graph_nodes, bufs=None):
     """One-launch forward from one int label per node (see gnnhip_s2v_forward_batched_labels_f32)."""
     N = label.numel()

@@ -774,6 +774,41 @@ def test_forward_on_two_streams_interleaved(gpu, oracle):
             assert np.array_equal(_n(o), cases[k][1])
 
 
+def test_one_launch_forward_with_batches_in_flight_on_several_streams(gpu, oracle):
+    """the one-launch forward queued round-robin on three streams through calls bound once (three batches of
+    different sizes, 300 graphs and more so that the graph order is made on each stream's own scratch, and small
+    ones): every round gives each batch the bits it has alone"""
+    import torch
+    from graphnn_amd import ops
+    cases = []
+    for seed, B in ((11, 300), (12, 77), (13, 700)):
+        batch = synth.molecule_batch(seed, B, 9, 2, size_mode="uniform", size_lo=3, size_hi=90)
+        w = synth.make_weights(synth.Stream(seed), 9, 64, 16, 2)
+        a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+        s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+        args = (_csr_t(a, gpu), _csr_t(s, gpu), _t(batch.one_hot(), gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+                _t(w.W_h1, gpu), _t(w.W_h2, gpu), 3, int(batch.graph_sizes.max()))
+        alone = ops.s2v_forward_batched(*args)
+        assert int(_n(alone.status)[0]) == 0
+        cases.append((args, {k: _n(getattr(alone, k)) for k in ("h_final", "logits", "probs", "pred")}, batch))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in cases]
+    bufs = [ops.BatchedBuffers(c[2].num_nodes, c[2].num_graphs, 64, 16, 2, gpu) for c in cases]
+    calls = [ops.bind_s2v_forward_batched(*cases[k][0], bufs[k], streams[k]) for k in range(len(cases))]
+    for rnd in range(5):
+        for b in bufs:
+            b.logits.fill_(-1.0)
+        torch.cuda.synchronize()
+        for _ in range(4):
+            for call in calls:
+                call()
+        torch.cuda.synchronize()
+        for k, b in enumerate(bufs):
+            assert int(_n(b.status)[0]) == 0
+            for key, want in cases[k][1].items():
+                assert np.array_equal(_n(getattr(b, key)), want), (rnd, k, key)
+
+
 def test_forward_every_level_matches(gpu, oracle):
     """level by level through the per-level entry point, against each of the oracle's stored h_l"""
     from graphnn_amd import ops
