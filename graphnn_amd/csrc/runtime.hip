@@ -340,7 +340,7 @@ __attribute__((target("avx2"))) bool collect_nonzero_avx2(const unsigned* w, siz
 }
 
 constexpr int kExpandBlock = 256;
-constexpr int kExpandTile = 4096;        // 32-bit words of the destination per workgroup
+constexpr int kExpandTile = 1024;        // 32-bit words of the destination per workgroup
 
 // dst[0..n) = 0 except dst[idx[i]] = val[i], idx ascending: a workgroup builds its tile of the destination in
 // LDS (zeros, then the entries that fall into it, found by bisection) and writes it out whole.
