@@ -174,7 +174,9 @@ __global__ __launch_bounds__(kOrderBlock) void graph_order_kernel(int B, int n16
 // WAVES wavefronts per workgroup (4, 8 or 16): chosen by the host so that the largest graph's
 // (column block x row tile) tasks spread over the wavefronts.
 // order: null (graphs in batch order), or the records graph_order_kernel left.
-template <int C, int KSX, int WAVES>
+// KEEP: the embeddings of all levels are also stored for a backward pass, h_l at h_levels + l * level_stride
+// (a variant of its own: the extra stores cost the inference kernel 2 % when they are a run-time choice).
+template <int C, int KSX, int WAVES, bool KEEP = false>
 __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     int B, int K, unsigned k_magic, int H, int Q, int L, int n16max, int ecap,
     const int* __restrict__ a_row_ptr, const int* __restrict__ a_col_idx, const float* __restrict__ a_val,
@@ -183,7 +185,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     const float* __restrict__ Wh1, const float* __restrict__ Wh2,
     float* __restrict__ msg, float* __restrict__ h_final, float* __restrict__ pool, float* __restrict__ hidden,
     float* __restrict__ logits, float* __restrict__ probs, int* __restrict__ pred, int* __restrict__ status,
-    const int* __restrict__ order)
+    const int* __restrict__ order, float* __restrict__ h_levels, long long level_stride)
 {
     // KSX == 0: the node features arrive as one label per node (X points at int labels[N]) and the input
     // stage is a row lookup in W_n2l; otherwise X is the dense [N,K] matrix and KSX bounds its contraction steps
@@ -427,6 +429,9 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
                 if (!valid) v = f4_zero();
                 if (valid) *reinterpret_cast<float4*>(msg + (size_t)(node0 + lr) * C + 16 * jb + 4 * q) = v;
                 *reinterpret_cast<float4*>(hbuf + (size_t)lr * LDT + 16 * jb + 4 * q) = relu_ref4(v);
+                if constexpr (KEEP) {
+                    if (valid) *reinterpret_cast<float4*>(h_levels + (size_t)(node0 + lr) * C + 16 * jb + 4 * q) = relu_ref4(v);
+                }
 #pragma unroll
                 for (int i = 0; i < kMsgTiles; ++i) if (i == ti) mreg[i] = v;
             }
@@ -519,6 +524,10 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
                 *reinterpret_cast<float4*>(hbuf + (size_t)lr * LDT + 16 * jb + 4 * q) = v;
                 if (lv == L - 1 && valid)
                     *reinterpret_cast<float4*>(h_final + (size_t)(node0 + lr) * C + 16 * jb + 4 * q) = v;
+                if constexpr (KEEP) {
+                    if (valid)
+                        *reinterpret_cast<float4*>(h_levels + (size_t)(lv + 1) * level_stride + (size_t)(node0 + lr) * C + 16 * jb + 4 * q) = v;
+                }
             }
             __syncthreads();
             if (lv == 0) { GNNHIP_PHASE_MARK(5); }
@@ -661,15 +670,20 @@ int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
                          const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                          const float* X, const float* Wn2l, const float* Wc, const float* Wh1, const float* Wh2,
                          float* msg, float* h_final, float* pool, float* hidden, float* logits, float* probs,
-                         int* pred, int* status, hipStream_t s)
+                         int* pred, int* status, float* h_levels, long long level_stride, hipStream_t s)
 {
     constexpr int kBlock = WAVES * kWave;
     constexpr bool LABELS = (KSX == 0);
     const int ecap = GraphLds::edge_cap(n16max, C, K, H, Q, kBlock, LABELS);
     if (ecap < 0) return GNNHIP_EUNSUPPORTED;
     const size_t smem = sizeof(float) * (GraphLds::fixed_floats(n16max, C, K, H, Q, kBlock, LABELS) + 2 * (size_t)ecap);
-    static LdsLimit lds_limit;              // largest dynamic LDS size this kernel instantiation has been allowed so far
-    if (lds_limit.raise(reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES>), smem) != hipSuccess) {
+    constexpr bool kKeepBuilt = !LABELS;    // the variant that keeps all levels exists for the dense input only
+    const bool keep = h_levels != nullptr;
+    if (keep && !kKeepBuilt) return GNNHIP_EUNSUPPORTED;
+    static LdsLimit lds_limit, lds_limit_keep;      // largest dynamic LDS size each kernel instantiation has been allowed so far
+    const void* fn = keep ? reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES, kKeepBuilt>)
+                          : reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES, false>);
+    if ((keep ? lds_limit_keep : lds_limit).raise(fn, smem) != hipSuccess) {
         (void)hipGetLastError();
         return GNNHIP_EUNSUPPORTED;
     }
@@ -683,9 +697,14 @@ int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
         GNNHIP_LAUNCH_CHECK("graph_order");
     }
     const unsigned k_magic = K >= 2 ? (unsigned)((0x100000000ull + (unsigned)K - 1) / (unsigned)K) : 0u;   // ceil(2^32 / K)
-    hipLaunchKernelGGL((s2v_graph_forward_kernel<C, KSX, WAVES>), dim3(grid), dim3(kBlock), smem, s,
-                       B, K, k_magic, H, Q, L, n16max, ecap, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val,
-                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, order);
+    if (keep)
+        hipLaunchKernelGGL((s2v_graph_forward_kernel<C, KSX, WAVES, kKeepBuilt>), dim3(grid), dim3(kBlock), smem, s,
+                           B, K, k_magic, H, Q, L, n16max, ecap, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val,
+                           X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, order, h_levels, level_stride);
+    else
+        hipLaunchKernelGGL((s2v_graph_forward_kernel<C, KSX, WAVES, false>), dim3(grid), dim3(kBlock), smem, s,
+                           B, K, k_magic, H, Q, L, n16max, ecap, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val,
+                           X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, order, h_levels, level_stride);
     GNNHIP_LAUNCH_CHECK("s2v_graph_forward");
     return GNNHIP_OK;
 }
@@ -696,10 +715,10 @@ int dispatch_ksx(bool labels, int B, int K, int H, int Q, int L, int n16max,
                  const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                  const float* X, const float* Wn2l, const float* Wc, const float* Wh1, const float* Wh2,
                  float* msg, float* h_final, float* pool, float* hidden, float* logits, float* probs,
-                 int* pred, int* status, hipStream_t s)
+                 int* pred, int* status, float* h_levels, long long level_stride, hipStream_t s)
 {
 #define GNNHIP_GF_ARGS B, K, H, Q, L, n16max, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
-                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, s
+                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, h_levels, level_stride, s
     if (labels) return launch_graph_forward<C, 0, WAVES>(GNNHIP_GF_ARGS);
     if (K <= 16) return launch_graph_forward<C, 4, WAVES>(GNNHIP_GF_ARGS);
     if (K <= 32) return launch_graph_forward<C, 8, WAVES>(GNNHIP_GF_ARGS);
@@ -715,10 +734,10 @@ int dispatch_waves(bool labels, int B, int K, int H, int Q, int L, int n16max,
                    const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                    const float* X, const float* Wn2l, const float* Wc, const float* Wh1, const float* Wh2,
                    float* msg, float* h_final, float* pool, float* hidden, float* logits, float* probs,
-                   int* pred, int* status, hipStream_t s)
+                   int* pred, int* status, float* h_levels, long long level_stride, hipStream_t s)
 {
 #define GNNHIP_GF_ARGS B, K, H, Q, L, n16max, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
-                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, s
+                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, h_levels, level_stride, s
     const int tasks = (C / 16) * (n16max / 16);         // (column block x row tile) tasks of the largest graph
     if (tasks <= 4) return dispatch_ksx<C, 4>(labels, GNNHIP_GF_ARGS);
     if (tasks <= 8) return dispatch_ksx<C, 8>(labels, GNNHIP_GF_ARGS);
@@ -739,7 +758,7 @@ int forward_batched_entry(bool labels, int N, int B, int K, int C, int H, int Q,
                           const void* X, const float* W_n2l, const float* W_conv,
                           const float* W_h1, const float* W_h2,
                           float* msg, float* h_final, float* pool, float* hidden, float* logits,
-                          float* probs, int* pred, int* status, void* stream)
+                          float* probs, int* pred, int* status, float* h_levels, void* stream)
 {
     GNNHIP_REQUIRE(N >= 1 && B >= 1 && K >= 1 && C >= 1 && H >= 1 && Q >= 1 && L >= 0 && max_graph_nodes >= 1,
                    "bad shape in s2v_forward_batched (N=%d B=%d K=%d C=%d H=%d Q=%d L=%d max_graph_nodes=%d)",
@@ -760,8 +779,10 @@ int forward_batched_entry(bool labels, int N, int B, int K, int C, int H, int Q,
     hipStream_t s = as_stream(stream);
     const float* Xf = static_cast<const float*>(X);
     int rc;
+    if (h_levels && !aligned16(h_levels)) return set_error(GNNHIP_EUNSUPPORTED, "h_levels must be 16-byte aligned");
+    const long long level_stride = (long long)N * C;
 #define GNNHIP_GF_ARGS labels, B, K, H, Q, L, n16, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
-                       Xf, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, s
+                       Xf, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, h_levels, level_stride, s
     switch (C) {
     case 16: rc = dispatch_waves<16>(GNNHIP_GF_ARGS); break;
     case 32: rc = dispatch_waves<32>(GNNHIP_GF_ARGS); break;
@@ -783,7 +804,7 @@ extern "C" int gnnhip_s2v_forward_batched_f32(int N, int B, int K, int C, int H,
                                               float* probs, int* pred, int* status, void* stream)
 {
     return forward_batched_entry(false, N, B, K, C, H, Q, L, max_graph_nodes, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx,
-                                 s_val, X, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, stream);
+                                 s_val, X, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, nullptr, stream);
 }
 
 extern "C" int gnnhip_s2v_forward_batched_labels_f32(int N, int B, int K, int C, int H, int Q, int L, int max_graph_nodes,
@@ -795,5 +816,21 @@ extern "C" int gnnhip_s2v_forward_batched_labels_f32(int N, int B, int K, int C,
                                                      float* probs, int* pred, int* status, void* stream)
 {
     return forward_batched_entry(true, N, B, K, C, H, Q, L, max_graph_nodes, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx,
-                                 s_val, node_label, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, stream);
+                                 s_val, node_label, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, nullptr, stream);
+}
+
+extern "C" int gnnhip_s2v_forward_batched_train_f32(int N, int B, int K, int C, int H, int Q, int L, int max_graph_nodes,
+                                                    const int* a_row_ptr, const int* a_col_idx, const float* a_val,
+                                                    const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                                                    const float* X, const float* W_n2l, const float* W_conv,
+                                                    const float* W_h1, const float* W_h2,
+                                                    float* msg, float* h_levels, float* pool, float* hidden, float* logits,
+                                                    float* probs, int* pred, int* status, void* stream)
+{
+    GNNHIP_REQUIRE(h_levels, "null h_levels in s2v_forward_batched_train");
+    // the last level doubles as the embedding output of the inference entry
+    float* h_last = h_levels + (size_t)(L > 0 ? L : 0) * (size_t)(N > 0 ? N : 0) * (size_t)(C > 0 ? C : 0);
+    return forward_batched_entry(false, N, B, K, C, H, Q, L, max_graph_nodes, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx,
+                                 s_val, X, W_n2l, W_conv, W_h1, W_h2, msg, h_last, pool, hidden, logits, probs, pred, status, h_levels,
+                                 stream);
 }

@@ -428,6 +428,18 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
                 Hid->value.Reshape({B, H});
                 Logits->value.Reshape({B, Q});
                 float* hs = st->hstack.data->ptr;
+                // small block-diagonal batches: everything in one launch, the levels stored on the way
+                if (n2n->block_diagonal && sub->max_subgraph_nodes > 0 && N <= detail::kOneLaunchMaxNodes) {
+                    const int rc = gnnhip_s2v_forward_batched_train_f32(
+                        (int)N, (int)B, (int)K, (int)C, (int)H, (int)Q, L, sub->max_subgraph_nodes,
+                        A->value.data->row_ptr, A->value.data->col_idx, A->value.data->val,
+                        S->value.data->row_ptr, S->value.data->col_idx, S->value.data->val,
+                        X->value.data->ptr, Wn->value.data->ptr, Wc->value.data->ptr, W1->value.data->ptr, W2->value.data->ptr,
+                        Msg->value.data->ptr, hs, Pool->value.data->ptr, Hid->value.data->ptr, Logits->value.data->ptr,
+                        nullptr, nullptr, nullptr, s);
+                    if (rc == GNNHIP_OK) return;
+                    ASSERT(rc == GNNHIP_EUNSUPPORTED, gnnhip_last_error());
+                }
                 GNN_HIP(gnnhip_s2v_input_f32((int)N, (int)K, (int)C, X->value.data->ptr, Wn->value.data->ptr, Msg->value.data->ptr, hs, s));
                 for (int l = 0; l < L; ++l)
                     GNN_HIP(gnnhip_s2v_level_f32((int)N, (int)C, A->value.data->nnz, A->value.data->row_ptr, A->value.data->col_idx,

@@ -235,6 +235,32 @@ def s2v_forward_batched(a_csr, s_csr, X, W_n2l, W_conv, W_h1, W_h2, L, max_graph
     return bufs
 
 
+def s2v_forward_batched_train(a_csr, s_csr, X, W_n2l, W_conv, W_h1, W_h2, L, max_graph_nodes, bufs=None):
+    """The one-launch forward that keeps every level: returns (bufs, h_levels [(L + 1), N, C]); bufs.h_final is
+    not written (h_levels[L] is that embedding)."""
+    N, K = X.shape
+    C, H, Q = W_n2l.shape[1], W_h1.shape[1], W_h2.shape[1]
+    B = s_csr[0].numel() - 1
+    _check_csr(a_csr[0], a_csr[1], a_csr[2], N, "A")
+    _check_csr(s_csr[0], s_csr[1], s_csr[2], B, "S")
+    if s_csr[1].numel() != N:
+        raise ValueError("S must list every node exactly once")
+    if W_n2l.shape[0] != K or tuple(W_conv.shape) != (C, C) or W_h1.shape[0] != C or W_h2.shape[0] != H:
+        raise ValueError("weight shapes do not chain")
+    if bufs is None:
+        bufs = BatchedBuffers(N, B, C, H, Q, X.device)
+    h_levels = torch.empty((L + 1, N, C), dtype=torch.float32, device=X.device)
+    check(_lib().gnnhip_s2v_forward_batched_train_f32(
+        N, B, K, C, H, Q, L, int(max_graph_nodes),
+        _i32(a_csr[0], "a_row_ptr"), _i32(a_csr[1], "a_col_idx"), _f32(a_csr[2], "a_val"),
+        _i32(s_csr[0], "s_row_ptr"), _i32(s_csr[1], "s_col_idx"), _f32(s_csr[2], "s_val"),
+        _f32(X, "X"), _f32(W_n2l, "W_n2l"), _f32(W_conv, "W_conv"), _f32(W_h1, "W_h1"), _f32(W_h2, "W_h2"),
+        _f32(bufs.msg, "msg"), _f32(h_levels, "h_levels"), _f32(bufs.pool, "pool"),
+        _f32(bufs.hidden, "hidden"), _f32(bufs.logits, "logits"), _f32(bufs.probs, "probs"),
+        _i32(bufs.pred, "pred"), _i32(bufs.status, "status"), _stream()))
+    return bufs, h_levels
+
+
 def bind_s2v_forward_batched(a_csr, s_csr, X, W_n2l, W_conv, W_h1, W_h2, L, max_graph_nodes, bufs, stream):
     """The call of s2v_forward_batched with every argument converted once: returns a function that queues one
     forward on `stream` (a torch.cuda.Stream) and raises on a non-zero status code.  For callers that keep several

@@ -187,6 +187,18 @@ int gnnhip_s2v_forward_batched_f32(int N, int B, int K, int C, int H, int Q, int
                                    float* msg, float* h_final, float* pool, float* hidden, float* logits,
                                    float* probs, int* pred, int* status, void* stream);
 
+/* ---- the one-launch forward of a training iteration: as gnnhip_s2v_forward_batched_f32, and the embeddings of
+ *      all levels are kept for the backward pass (FactorGraph::FeedForward with Phase::TRAIN keeps every factor's
+ *      output, src/nn/factor_graph.cpp:146-180): h_levels [(L + 1), N, C] receives h_0 = ReLU(msg) and h_1 .. h_L
+ *      (h_L is what the inference entry returns as h_final).  Same limits, status bits and return codes. */
+int gnnhip_s2v_forward_batched_train_f32(int N, int B, int K, int C, int H, int Q, int L, int max_graph_nodes,
+                                         const int* a_row_ptr, const int* a_col_idx, const float* a_val,
+                                         const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                                         const float* X, const float* W_n2l, const float* W_conv,
+                                         const float* W_h1, const float* W_h2,
+                                         float* msg, float* h_levels, float* pool, float* hidden, float* logits,
+                                         float* probs, int* pred, int* status, void* stream);
+
 /* ---- the one-launch forward with one label per node in place of the one-hot matrix X (see
  *      gnnhip_s2v_input_labels_f32; the batch layout is GetBatch's,
  *      examples/graph_classification/include/nn_common.h:36-105): the input stage becomes a row lookup in W_n2l [K,C] (K is not limited to 64),

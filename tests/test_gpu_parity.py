@@ -1024,6 +1024,30 @@ def test_batched_forward_takes_graphs_largest_first(gpu, oracle, B, C, hi):
         assert np.all(_n(fresh.logits)[~fits] == -7.0)
 
 
+@pytest.mark.parametrize("C,L,B", [(64, 4, 256), (16, 1, 37), (32, 3, 300), (64, 0, 9)])
+def test_batched_forward_keeps_every_level_for_training(gpu, oracle, C, L, B):
+    """the one-launch forward of a training iteration: h_0 .. h_L as the per-level entry points give them (which
+    have their own parity tests), every other output with the bits of the inference entry"""
+    from graphnn_amd import ops
+    K, H, Q = 9, 16, 2
+    batch = synth.molecule_batch(4000 + C + B, B, K, Q, size_mode="uniform", size_lo=2, size_hi=90)
+    w = synth.make_weights(synth.Stream(4000 + C), K, C, H, Q)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    args = (_csr_t(a, gpu), _csr_t(s, gpu), _t(batch.one_hot(), gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+            _t(w.W_h1, gpu), _t(w.W_h2, gpu), L, int(batch.graph_sizes.max()))
+    plain = ops.s2v_forward_batched(*args)
+    bufs, hl = ops.s2v_forward_batched_train(*args)
+    assert int(_n(bufs.status)[0]) == 0 and tuple(hl.shape) == (L + 1, batch.num_nodes, C)
+    for k in ("msg", "pool", "hidden", "logits", "probs", "pred"):
+        assert np.array_equal(_n(getattr(bufs, k)), _n(getattr(plain, k))), k
+    assert np.array_equal(_n(hl[L]), _n(plain.h_final))
+    want = oracle.forward(a, s, batch.one_hot(), w, L, None)
+    for l in range(L + 1):
+        assert max_rel(_n(hl[l]), want["h"][l]) < PARITY_TOL, l
+    assert np.array_equal(_n(hl[0]), np.maximum(_n(bufs.msg), 0))
+
+
 def test_batched_forward_dense_features_past_the_staging_registers(gpu, oracle):
     """64 real-valued feature columns on graphs of up to 190 nodes: a graph's block of X (12,160 floats) is longer
     than what the lanes stage in one go, and its rows outnumber the gather rounds kept in registers"""
