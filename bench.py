@@ -110,6 +110,17 @@ def time_forward_pipelined(dev_args, cfg, batch, steps, warmup, nstreams=4):
     return (t1 - t0) / steps, bufs
 
 
+def time_stream_copy(dev, n=1 << 28):
+    """What this GPU's memory delivers to the simplest streaming kernel: the element-wise engine reading 1 GiB and
+    writing 1 GiB (map1_kernel<FReLU>), GB/s of the 2 GiB moved; printed beside the nominal 8 TB/s."""
+    import torch
+    from graphnn_amd import ops
+    src = torch.ones(n, device=dev, dtype=torch.float32)
+    dst = torch.empty_like(src)
+    ms = _event_ms(lambda: ops.relu(src, dst), 10)
+    return {"kernel": "map1_kernel<FReLU>", "bytes": 8 * n, "avg_ms": ms, "GBps": 8.0 * n / (ms * 1e-3) / 1e9}
+
+
 def time_spmm_cfg3(dev, reps=20, warmup=3):
     """HIP-event time of the SpMM kernel alone on configuration 3."""
     import torch
@@ -672,6 +683,8 @@ def main():
             # the counted traffic over the same launch time: what the memory system actually moves
             "traffic_GBps": MEASURED_TRAFFIC_BYTES["spmm_cfg3"] / (mean_ms * 1e-3) / 1e9,
             "traffic_frac": MEASURED_TRAFFIC_BYTES["spmm_cfg3"] / (mean_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            # what a plain streaming kernel reaches on this GPU, measured in this run
+            "stream_copy": time_stream_copy(dev),
         }
     else:
         out["roofline"] = None

@@ -232,8 +232,10 @@ int spmm_dispatch(int m, int k, int n, long long nnz, float alpha, const int* ro
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
 {
     // large matrices with many entries per row (power-law graphs): rows cut into pieces, summed in column order
+    // (its scratch, about 40 bytes per entry of A + 4 n bytes per piece, is taken before anything is launched: when
+    // the device cannot give it, the row-group route below, which needs far less, does the product)
     if (int rc = spmm_pieces_dispatch(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, s, reuse_plan);
-        rc != GNNHIP_EUNSUPPORTED)
+        rc != GNNHIP_EUNSUPPORTED && rc != GNNHIP_ENOMEM)
         return rc;
     return spmm_plain_dispatch(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, s, reuse_plan);
 }
