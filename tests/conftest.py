@@ -229,7 +229,7 @@ def ref_graph():
 
 PARITY_TOL = 1e-4     # the north-star tolerance for fp32 activations and logits
 
-# Floors of the parity metric, measured (see the sweep recorded in DESIGN.md): the smallest floor at which
+# Floors of the parity metric, measured (test_oracle_pins.py repeats the sweep on every run): the smallest floor at which
 # the oracle itself stays within 1e-4 of a float64 model of the same network on configurations 1 and 2
 # (12 to 3,000 graphs) is 1.3e-3 of the tensor's largest magnitude for the embeddings and the hidden layer,
 # 4e-5 for the pooled features and zero for the probabilities.  Two correct fp32 summation orders differ
