@@ -400,7 +400,7 @@ def kernel_rooflines(dev, forwards=None):
         hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + spmm_rowgroup_kernel<4,1>", w5 + ": SpMM A*h, plan included",
             spmm_algorithmic_bytes(N, N, E, C), c5["spmm"]["avg_ms"], gather_GBps=c5["spmm"]["gather_GBps"]),
         hbm("sgemm_skinny_rows_kernel<1>", w5 + ": node scores h*w", 4 * N * (C + 1), c5["score"]["avg_ms"]),
-        hbm("exclusive_scan_kernel + jagged_softmax_kernel", w5 + ": jagged softmax over %d segments of 1024" % B,
+        hbm("jagged_softmax_fused_kernel", w5 + ": jagged softmax over %d segments of 1024" % B,
             8 * N + 4 * B, c5["jagged_softmax"]["avg_ms"]),
         hbm("spmm_rowgroup_kernel<4,1>", w5 + ": sum-pool S*h", 4 * N * C + 8 * N + 4 * (B + 1) + 4 * B * C, c5["sum_pool"]["avg_ms"]),
     ]

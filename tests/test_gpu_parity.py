@@ -333,6 +333,14 @@ def test_jagged_softmax(gpu, oracle):
     assert max_rel(got2, want2) < PARITY_TOL
     sums = np.add.reduceat(got2.astype(np.float64), np.concatenate([[0], np.cumsum(lens2)[:-1]])[lens2 > 0])
     assert np.allclose(sums, 1.0, atol=1e-4)
+    # segment counts on both sides of the limit up to which one launch does it all (each workgroup adds up the
+    # lengths ahead of its segments) and beyond which a scan launch comes first; the last workgroup is not full
+    for nseg in (8191, 8192, 8193, 20001):
+        lens3 = rng.integers(0, 9, nseg).astype(np.int32)
+        lens3[nseg // 2] = 3000
+        x3 = (rng.standard_normal(int(lens3.sum())) * 2).astype(np.float32)
+        got3 = _n(ops.jagged_softmax(_t(x3, gpu), _t(lens3, gpu)))
+        assert max_rel(got3, oracle.jagged_softmax(x3, lens3)) < PARITY_TOL, nseg
 
 
 def test_jagged_softmax_gradient(gpu, oracle):
