@@ -226,20 +226,24 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_rows_kernel(
             b[j].w = TB ? B[(size_t)j * ldb + kk + 3] : B[(size_t)(kk + 3) * ldb + j];
         }
     }
-    const long long groups = ((long long)gridDim.x * kBlock) >> logG;
-    const long long group = ((long long)blockIdx.x * kBlock + threadIdx.x) >> logG;
-    // all lanes of a wavefront run the same number of iterations (the reductions are wavefront-wide operations)
-    const long long first = ((long long)blockIdx.x * kBlock + (threadIdx.x & ~(kWave - 1))) >> logG;
-    for (long long base = 0; first + base < m; base += R * groups) {
+    // A workgroup walks one contiguous run of rows (its groups side by side, R turns ahead), so that what is in flight
+    // from one workgroup is one stretch of memory.  All lanes of a wavefront run the same number of iterations (the
+    // reductions are wavefront-wide operations).
+    const int groups = kBlock >> logG;
+    const int group = threadIdx.x >> logG;
+    const long long per_block = ((long long)m + gridDim.x - 1) / gridDim.x;
+    const long long row0 = (long long)blockIdx.x * per_block;
+    const long long row1 = row0 + per_block < m ? row0 + per_block : m;
+    for (long long base = row0; base < row1; base += R * groups) {
         float4 x[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const long long row = group + base + r * groups;
-            x[r] = (live && row < m) ? *reinterpret_cast<const float4*>(A + (size_t)row * lda + kk) : f4_zero();
+            const long long row = base + r * groups + group;
+            x[r] = (live && row < row1) ? *reinterpret_cast<const float4*>(A + (size_t)row * lda + kk) : f4_zero();
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const long long row = group + base + r * groups;
+            const long long row = base + r * groups + group;
 #pragma unroll
             for (int j = 0; j < NCOL; ++j) {
                 float acc = x[r].x * b[j].x + x[r].y * b[j].y + x[r].z * b[j].z + x[r].w * b[j].w;
@@ -249,7 +253,7 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_rows_kernel(
                 if (G >= 16) acc += dpp_mov_f<kDppMirror>(acc);
                 if (G >= 32) acc += __shfl_xor(acc, 16, kWave);
                 if (G >= 64) acc += __shfl_xor(acc, 32, kWave);
-                if (row < m && sub == 0) {
+                if (row < row1 && sub == 0) {
                     float* c = C + (size_t)row * ldc + j;
                     *c = (beta == 0.f) ? alpha * acc : alpha * acc + beta * *c;
                 }
