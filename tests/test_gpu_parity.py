@@ -817,6 +817,50 @@ def test_one_launch_forward_with_batches_in_flight_on_several_streams(gpu, oracl
                 assert np.array_equal(_n(getattr(b, key)), want), (rnd, k, key)
 
 
+def test_forwards_replay_from_a_captured_graph(gpu, oracle):
+    """once a stream has its scratch (a first eager call), the forwards queue kernels only (no allocation, no
+    memset nodes): captured into a HIP graph through torch and replayed five times, with eager forwards and
+    synchronisations between the replays, every replay gives the eager bits; both routes, and a batch of 300
+    graphs whose one-launch forward has the graph-order launch ahead of it"""
+    import torch
+    from graphnn_amd import ops
+    for B in (64, 300):
+        batch, w, cfg = synth.make_config(2, B=B)
+        a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+        s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+        args = (_csr_t(a, gpu), _csr_t(s, gpu), _t(batch.one_hot(), gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
+                _t(w.W_h1, gpu), _t(w.W_h2, gpu), cfg["L"])
+        nmax = int(batch.graph_sizes.max())
+        stream = torch.cuda.Stream()
+        gen = ops.ForwardBuffers(batch.num_nodes, B, cfg["C"], cfg["H"], cfg["Q"], gpu)
+        one = ops.BatchedBuffers(batch.num_nodes, B, cfg["C"], cfg["H"], cfg["Q"], gpu)
+        def both():
+            ops.s2v_forward(*args, bufs=gen)
+            ops.s2v_forward_batched(*args, nmax, bufs=one)
+        with torch.cuda.stream(stream):
+            both()
+        torch.cuda.synchronize()
+        want = (_n(gen.logits), _n(gen.pred), _n(one.logits), _n(one.h_final))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            both()
+        torch.cuda.synchronize()
+        for rep in range(5):
+            for t in (gen.logits, one.logits, one.h_final):
+                t.fill_(-3.0)
+            gen.pred.fill_(-1)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = (_n(gen.logits), _n(gen.pred), _n(one.logits), _n(one.h_final))
+            for g_, w_ in zip(got, want):
+                assert np.array_equal(g_, w_), (B, rep)
+            with torch.cuda.stream(stream):
+                both()                                       # the program's own eager work between replays
+            torch.cuda.synchronize()
+        assert int(_n(one.status)[0]) == 0
+
+
 def test_forward_every_level_matches(gpu, oracle):
     """level by level through the per-level entry point, against each of the oracle's stored h_l"""
     from graphnn_amd import ops
