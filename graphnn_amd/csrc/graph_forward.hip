@@ -171,12 +171,123 @@ __global__ __launch_bounds__(kOrderBlock) void graph_order_kernel(int B, int n16
     }
 }
 
+// Batches of more graphs than compute units can also be packed: a run of consecutive graphs of at most `cap`
+// nodes together is a block-diagonal graph like any other, so one workgroup carries it through the input stage
+// and the levels at the cost of one graph (the kernel's time is per workgroup: start-up, staging, a barrier
+// per stage, and matrix tiles that a 30-node graph leaves three quarters empty), and only the readout runs per
+// graph (a wavefront each).  1,024 graphs of the 10..110-node distribution: 59 -> 45 us.
+// The kernel below cuts the batch into such runs ("bins").  Every 64 consecutive graphs are packed on their
+// own by one wavefront (first fit in batch order; a bin never crosses such a boundary, which costs about one
+// partly filled bin per 64 graphs), so all of it is a few ballots per bin.  A graph of more than cap nodes is a
+// bin of its own (the forward kernel refuses it).  Output: bins[0] = number of bins, then one record of
+// kOrderRec ints per bin from bins + kOrderRec on: first graph, first node, nodes, first entry, end of entries,
+// graphs.
+constexpr int kPackNodes = 128;                  // eight tiles: with four column blocks, two tasks for each of 16 wavefronts
+constexpr int kPackMaxNodes = 208;
+constexpr int kPackMinGraphs = 2 * kNumCU;       // below this the graphs taken one by one, largest first, are as fast
+constexpr int kBinBlock = 1024;
+constexpr int kBinMaxGraphs = 1 << 19;           // segment counts live in LDS (32 KB)
+__global__ __launch_bounds__(kBinBlock) void graph_bins_kernel(int B, int cap, const int* __restrict__ a_row_ptr,
+                                                               const int* __restrict__ s_row_ptr, int* __restrict__ bins)
+{
+    constexpr int kWaves = kBinBlock / kWave;
+    __shared__ int seg_bins[kBinMaxGraphs / kWave + 1];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int nseg = (B + kWave - 1) / kWave;
+    // packs segment `seg` (start / end: first node and end of the lane's graph); with `base` >= 0 the records
+    // are written from bin index `base` on.  Returns the bin count.
+    auto pack = [&](int seg, int start, int end, int base) {
+        const bool live = seg * kWave + lane < B;
+        const int nlive = min(kWave, B - seg * kWave);
+        int first = 0, count = 0;
+        while (first < nlive) {
+            const int node0 = __builtin_amdgcn_readlane(start, first);
+            // lanes from `first` on whose graph still fits behind node0; the bin ends before the first that does not
+            const unsigned long long stop = __ballot(lane >= first && (!live || end - node0 > cap));
+            int next = stop ? (int)__builtin_ctzll(stop) : kWave;
+            if (next == first) next = first + 1;                     // larger than cap: alone
+            next = __builtin_amdgcn_readfirstlane(next);
+            if (base >= 0 && lane < 2)                               // first graph and graph count; the rest follows below
+                bins[(size_t)(1 + base + count) * kOrderRec + (lane ? 5 : 0)] = lane ? next - first : seg * kWave + first;
+            ++count;
+            first = next;
+        }
+        return count;
+    };
+    // the node ranges of this wavefront's first kBinKeep segments stay in registers between the two passes
+    constexpr int kBinKeep = 4;
+    int st[kBinKeep], en[kBinKeep];
+#pragma unroll
+    for (int j = 0; j < kBinKeep; ++j) {
+        const int g = (wave + j * kWaves) * kWave + lane;
+        st[j] = en[j] = 0;
+        if (g < B) { st[j] = s_row_ptr[g]; en[j] = s_row_ptr[g + 1]; }
+    }
+    auto ranges = [&](int seg, int j, int& start, int& end) {
+        if (j < kBinKeep) {
+#pragma unroll
+            for (int u = 0; u < kBinKeep; ++u) if (u == j) { start = st[u]; end = en[u]; }
+        } else {
+            const int g = seg * kWave + lane;
+            start = end = 0;
+            if (g < B) { start = s_row_ptr[g]; end = s_row_ptr[g + 1]; }
+        }
+    };
+    for (int seg = wave, j = 0; seg < nseg; seg += kWaves, ++j) {
+        int start, end;
+        ranges(seg, j, start, end);
+        const int c = pack(seg, start, end, -1);
+        if (lane == 0) seg_bins[seg] = c;
+    }
+    __syncthreads();
+    if (wave == 0) {                                                 // exclusive scan of the segment counts
+        int carry = 0;
+        for (int b0 = 0; b0 < nseg; b0 += kWave) {
+            const int i = b0 + lane;
+            const int v = i < nseg ? seg_bins[i] : 0;
+            int incl = v;
+#pragma unroll
+            for (int d = 1; d < kWave; d <<= 1) {
+                const int o = __shfl_up(incl, d, kWave);
+                if (lane >= d) incl += o;
+            }
+            if (i < nseg) seg_bins[i] = carry + incl - v;
+            carry += __shfl(incl, kWave - 1, kWave);
+        }
+        if (lane == 0) bins[0] = carry;
+    }
+    __syncthreads();
+    for (int seg = wave, j = 0; seg < nseg; seg += kWaves, ++j) {
+        int start, end;
+        ranges(seg, j, start, end);
+        pack(seg, start, end, seg_bins[seg]);
+    }
+    __threadfence_block();
+    __syncthreads();
+    // node and entry ranges, one lane per bin (a bin the forward kernel will refuse gets no entry range)
+    const int nbins = bins[0];
+    for (int b = threadIdx.x; b < nbins; b += kBinBlock) {
+        int* rec = bins + (size_t)(1 + b) * kOrderRec;
+        const int g0 = rec[0], ng = rec[5];
+        const int node0 = s_row_ptr[g0], n = s_row_ptr[g0 + ng] - node0;
+        int e0 = 0, e1 = 0;
+        if (n >= 0 && n <= cap) { e0 = a_row_ptr[node0]; e1 = a_row_ptr[node0 + n]; }
+        rec[1] = node0;
+        rec[2] = n;
+        rec[3] = e0;
+        rec[4] = e1;
+    }
+}
+
 // WAVES wavefronts per workgroup (4, 8 or 16): chosen by the host so that the largest graph's
 // (column block x row tile) tasks spread over the wavefronts.
 // order: null (graphs in batch order), or the records graph_order_kernel left.
 // KEEP: the embeddings of all levels are also stored for a backward pass, h_l at h_levels + l * level_stride
 // (a variant of its own: the extra stores cost the inference kernel 2 % when they are a run-time choice).
-template <int C, int KSX, int WAVES, bool KEEP = false>
+// PACK: `order` holds the bins graph_bins_kernel made (order[0] bins, records from order + kOrderRec on); a workgroup
+// carries a bin through the input stage and the levels as one block-diagonal graph, and its wavefronts run the
+// readout of the bin's graphs, one graph each (H <= 64 and Q <= 64: a lane per hidden unit and per class).
+template <int C, int KSX, int WAVES, bool KEEP = false, bool PACK = false>
 __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     int B, int K, unsigned k_magic, int H, int Q, int L, int n16max, int ecap,
     const int* __restrict__ a_row_ptr, const int* __restrict__ a_col_idx, const float* __restrict__ a_val,
@@ -229,12 +340,17 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     GNNHIP_PHASE_MARK(0);
     // The position of the first graph (node range, then entry range) is asked for ahead of the weight
     // loads, so the two dependent trips to memory run under them instead of after them.
-    int next_g = blockIdx.x, next_node0 = 0, next_n = 0, next_e0 = 0, next_e1 = 0;
-    if ((int)blockIdx.x < B) {
+    int next_g = blockIdx.x, next_node0 = 0, next_n = 0, next_e0 = 0, next_e1 = 0, next_ng = 1;
+    // PACK: the slots are the bins (their number is the first word of `order`, the records follow its first kOrderRec words)
+    const int* recs = PACK ? order + kOrderRec : order;
+    const int nslots = PACK ? order[0] : B;
+    if ((int)blockIdx.x < nslots) {
         if (order) {
-            const int4 r0 = *reinterpret_cast<const int4*>(order + (size_t)blockIdx.x * kOrderRec);
+            const int4 r0 = *reinterpret_cast<const int4*>(recs + (size_t)blockIdx.x * kOrderRec);
             next_g = r0.x; next_node0 = r0.y; next_n = r0.z; next_e0 = r0.w;
-            next_e1 = order[(size_t)blockIdx.x * kOrderRec + 4];
+            const int2 r1 = *reinterpret_cast<const int2*>(recs + (size_t)blockIdx.x * kOrderRec + 4);
+            next_e1 = r1.x;
+            next_ng = r1.y;
         } else {
             next_node0 = s_row_ptr[blockIdx.x];
             next_n = s_row_ptr[blockIdx.x + 1] - next_node0;
@@ -245,13 +361,17 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
 #pragma unroll
     for (int s = 0; s < KS; ++s)
         wreg[s] = Wc[(size_t)(KS * ((tid0 & (kWave - 1)) >> 4) + s) * C + 16 * ((tid0 / kWave) % NJB) + (tid0 & 15)];
-    if (!order && (int)blockIdx.x < B && next_n >= 0 && next_n <= n16max) {
+    if (!order && (int)blockIdx.x < nslots && next_n >= 0 && next_n <= n16max) {
         next_e0 = a_row_ptr[next_node0];
         next_e1 = a_row_ptr[next_node0 + next_n];
     }
 
     if (tid0 < LDT) hbuf[(size_t)n16max * LDT + tid0] = 0.f;
-    if (ro_staged) {
+    if (PACK && ro_staged) {
+        // a lane per output in the readout: the layouts of memory, W_h1 [C][H] and W_h2 [H][Q]
+        for (int i = tid0; i < C * H; i += kBlock) w1s[i] = Wh1[i];
+        for (int i = tid0; i < H * Q; i += kBlock) w2s[i] = Wh2[i];
+    } else if (ro_staged) {
         // coalesced reads; the transposed layout lets a wavefront read one output's weights contiguously
         // (four elements of W_h1 and one of W_h2 per lane are asked for together: one trip to memory for the
         // usual sizes instead of one per element)
@@ -275,7 +395,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
     // the staged rows of X have stride KP floats and zeros from column K on
     const int srt = GraphLds::input_steps(K);
     const int KP = 4 * srt;
-    for (int slot = blockIdx.x; slot < B; slot += gridDim.x) {
+    for (int slot = blockIdx.x; slot < nslots; slot += gridDim.x) {
         // The lane's coordinates are derived again for every graph from a value the compiler cannot see
         // through.  Otherwise every per-lane address of the loop body (a dozen 64-bit pointers) is computed
         // once ahead of the loop, does not fit the 128 registers of a 16-wavefront workgroup, and comes back
@@ -288,13 +408,15 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
         const int gi = tid / G, tx = tid % G;
         const int wx_lane_off = ((srt * q) * C + 16 * jb + t) * 4;
         const bool first = (slot == (int)blockIdx.x);   // the position of this graph was asked for at start-up
-        int g = slot, node0, n, rec_e0 = 0, rec_e1 = 0;
+        int g = slot, node0, n, rec_e0 = 0, rec_e1 = 0, ng = 1;
         if (first) {
-            g = next_g; node0 = next_node0; n = next_n;
+            g = next_g; node0 = next_node0; n = next_n; ng = next_ng;
         } else if (order) {
-            const int4 r0 = *reinterpret_cast<const int4*>(order + (size_t)slot * kOrderRec);
+            const int4 r0 = *reinterpret_cast<const int4*>(recs + (size_t)slot * kOrderRec);
             g = r0.x; node0 = r0.y; n = r0.z; rec_e0 = r0.w;
-            rec_e1 = order[(size_t)slot * kOrderRec + 4];
+            const int2 r1 = *reinterpret_cast<const int2*>(recs + (size_t)slot * kOrderRec + 4);
+            rec_e1 = r1.x;
+            ng = r1.y;
         } else {
             node0 = s_row_ptr[g];
             n = s_row_ptr[g + 1] - node0;
@@ -542,6 +664,59 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
             }
         }
 
+        if constexpr (PACK) {
+            // ---- readout of a bin: graph k of the bin is rows [l_gs[k], l_gs[k + 1]) and belongs to one wavefront,
+            // which pools it (lane c walks column c, rows in order), forms the hidden units (lane j adds
+            // pool[c] * W_h1[c][j] over c, the pooled values handed round by v_readlane), the logits (lane q)
+            // and softmax / arg-max, without a barrier
+            int* l_gs = reinterpret_cast<int*>(agg);         // [ng + 1]; the buffer is free after the last level
+            if (tid <= ng) l_gs[tid] = s_row_ptr[g + tid] - node0;
+            __syncthreads();
+            for (int k = wave; k < ng; k += kWavesPerBlock) {
+                const int r0 = l_gs[k], r1 = l_gs[k + 1];
+                const int gk = g + k;
+                float p = 0.f;
+                if (lane < C)
+                    for (int lr = r0; lr < r1; ++lr) p = fmaf(l_sv[lr], hbuf[(size_t)lr * LDT + lane], p);
+                if (lane < C) pool[(size_t)gk * C + lane] = p;
+                const float* w1 = ro_staged ? w1s : Wh1;      // [C][H] either way
+                const float* w2 = ro_staged ? w2s : Wh2;      // [H][Q]
+                float hv = 0.f;
+#pragma unroll 8
+                for (int c = 0; c < C; ++c) {
+                    const float pc = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), c));
+                    if (lane < H) hv = fmaf(pc, w1[(size_t)c * H + lane], hv);
+                }
+                hv = relu_ref(hv);
+                if (lane < H) hidden[(size_t)gk * H + lane] = hv;
+                float sq = 0.f;
+#pragma unroll 8
+                for (int j = 0; j < H; ++j) {
+                    const float hj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(hv), j));
+                    if (lane < Q) sq = fmaf(hj, w2[(size_t)j * Q + lane], sq);
+                }
+                if (lane < Q) logits[(size_t)gk * Q + lane] = sq;
+                if (probs || pred) {
+                    const float first = row_value_f(sq, 0);
+                    float mx = (lane < Q) ? max_keep(first, sq) : first;     // the reference scan starts at element 0
+                    mx = wave_max(mx);
+                    float bv = -INFINITY;
+                    int bi = 0x7fffffff;
+                    if (lane < Q) { bv = (sq != sq) ? -INFINITY : sq; bi = lane; }   // a NaN that is not first never wins
+                    wave_argmax(bv, bi);
+                    if (first != first) bi = 0;                              // a NaN in column 0 is never displaced
+                    if (pred && lane == 0) pred[gk] = bi;
+                    if (probs) {
+                        const float e = (lane < Q) ? expf(sq - mx) : 0.f;
+                        const float sum = wave_sum(e);
+                        if (lane < Q) probs[(size_t)gk * Q + lane] = e / sum;
+                    }
+                }
+            }
+            GNNHIP_PHASE_MARK(7);
+            __syncthreads();          // LDS is reused by the next bin of this workgroup
+            continue;
+        }
         // ---- readout: weighted sum-pool over the graph's rows, then the two small dense layers.
         // Pooling: a lane owns one column and walks rows, so at C = 64 nothing crosses lanes; one partial
         // per wavefront goes to LDS.
@@ -670,7 +845,7 @@ int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
                          const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                          const float* X, const float* Wn2l, const float* Wc, const float* Wh1, const float* Wh2,
                          float* msg, float* h_final, float* pool, float* hidden, float* logits, float* probs,
-                         int* pred, int* status, float* h_levels, long long level_stride, hipStream_t s)
+                         int* pred, int* status, float* h_levels, long long level_stride, bool pack, hipStream_t s)
 {
     constexpr int kBlock = WAVES * kWave;
     constexpr bool LABELS = (KSX == 0);
@@ -678,18 +853,34 @@ int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
     if (ecap < 0) return GNNHIP_EUNSUPPORTED;
     const size_t smem = sizeof(float) * (GraphLds::fixed_floats(n16max, C, K, H, Q, kBlock, LABELS) + 2 * (size_t)ecap);
     constexpr bool kKeepBuilt = !LABELS;    // the variant that keeps all levels exists for the dense input only
+    // the variant that packs graphs into bins exists for the workgroup shapes bins of 128 nodes and more select
+    constexpr bool kPackBuilt = (WAVES == 16) || (C == 16 && WAVES == 8);
     const bool keep = h_levels != nullptr;
     if (keep && !kKeepBuilt) return GNNHIP_EUNSUPPORTED;
-    static LdsLimit lds_limit, lds_limit_keep;      // largest dynamic LDS size each kernel instantiation has been allowed so far
-    const void* fn = keep ? reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES, kKeepBuilt>)
-                          : reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES, false>);
-    if ((keep ? lds_limit_keep : lds_limit).raise(fn, smem) != hipSuccess) {
+    if (pack && (!kPackBuilt || keep)) return GNNHIP_EUNSUPPORTED;
+    static LdsLimit lds_limit, lds_limit_keep, lds_limit_pack;      // largest dynamic LDS size each kernel instantiation has been allowed so far
+    const void* fn = keep ? reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES, kKeepBuilt, false>)
+                   : pack ? reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES, false, kPackBuilt>)
+                          : reinterpret_cast<const void*>(&s2v_graph_forward_kernel<C, KSX, WAVES, false, false>);
+    if ((keep ? lds_limit_keep : pack ? lds_limit_pack : lds_limit).raise(fn, smem) != hipSuccess) {
         (void)hipGetLastError();
         return GNNHIP_EUNSUPPORTED;
     }
-    const int grid = B < kNumCU * 4 ? B : kNumCU * 4;
+    int grid = B < kNumCU * 4 ? B : kNumCU * 4;
     int* order = nullptr;
-    if (graphs_ordered(B) && n16max / 16 + 2 <= 64) {
+    if (pack) {
+        // bins: at most one per graph; two neighbouring bins hold more than n16max nodes together, and every 64
+        // graphs may leave one bin short
+        const long long N = level_stride / C;
+        long long most = 2 * N / n16max + (B + kWave - 1) / kWave + 1;
+        if (most > B) most = B;
+        if (most < grid) grid = (int)most;
+        void* p = nullptr;
+        if (int rc = stream_scratch(s, sizeof(int) * kOrderRec * ((size_t)B + 1), &p)) return rc;
+        order = static_cast<int*>(p);
+        hipLaunchKernelGGL(graph_bins_kernel, dim3(1), dim3(kBinBlock), 0, s, B, n16max, a_row_ptr, s_row_ptr, order);
+        GNNHIP_LAUNCH_CHECK("graph_bins");
+    } else if (graphs_ordered(B) && n16max / 16 + 2 <= 64) {
         void* p = nullptr;
         if (int rc = stream_scratch(s, sizeof(int) * kOrderRec * (size_t)B, &p)) return rc;
         order = static_cast<int*>(p);
@@ -697,14 +888,14 @@ int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
         GNNHIP_LAUNCH_CHECK("graph_order");
     }
     const unsigned k_magic = K >= 2 ? (unsigned)((0x100000000ull + (unsigned)K - 1) / (unsigned)K) : 0u;   // ceil(2^32 / K)
-    if (keep)
-        hipLaunchKernelGGL((s2v_graph_forward_kernel<C, KSX, WAVES, kKeepBuilt>), dim3(grid), dim3(kBlock), smem, s,
-                           B, K, k_magic, H, Q, L, n16max, ecap, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val,
-                           X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, order, h_levels, level_stride);
-    else
-        hipLaunchKernelGGL((s2v_graph_forward_kernel<C, KSX, WAVES, false>), dim3(grid), dim3(kBlock), smem, s,
-                           B, K, k_magic, H, Q, L, n16max, ecap, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val,
-                           X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, order, h_levels, level_stride);
+#define GNNHIP_GF_LAUNCH(KEEPV, PACKV)                                                                                              \
+    hipLaunchKernelGGL((s2v_graph_forward_kernel<C, KSX, WAVES, KEEPV, PACKV>), dim3(grid), dim3(kBlock), smem, s,                   \
+                       B, K, k_magic, H, Q, L, n16max, ecap, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val,              \
+                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, order, h_levels, level_stride)
+    if (keep) GNNHIP_GF_LAUNCH(kKeepBuilt, false);
+    else if (pack) GNNHIP_GF_LAUNCH(false, kPackBuilt);
+    else GNNHIP_GF_LAUNCH(false, false);
+#undef GNNHIP_GF_LAUNCH
     GNNHIP_LAUNCH_CHECK("s2v_graph_forward");
     return GNNHIP_OK;
 }
@@ -715,10 +906,10 @@ int dispatch_ksx(bool labels, int B, int K, int H, int Q, int L, int n16max,
                  const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                  const float* X, const float* Wn2l, const float* Wc, const float* Wh1, const float* Wh2,
                  float* msg, float* h_final, float* pool, float* hidden, float* logits, float* probs,
-                 int* pred, int* status, float* h_levels, long long level_stride, hipStream_t s)
+                 int* pred, int* status, float* h_levels, long long level_stride, bool pack, hipStream_t s)
 {
 #define GNNHIP_GF_ARGS B, K, H, Q, L, n16max, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
-                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, h_levels, level_stride, s
+                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, h_levels, level_stride, pack, s
     if (labels) return launch_graph_forward<C, 0, WAVES>(GNNHIP_GF_ARGS);
     if (K <= 16) return launch_graph_forward<C, 4, WAVES>(GNNHIP_GF_ARGS);
     if (K <= 32) return launch_graph_forward<C, 8, WAVES>(GNNHIP_GF_ARGS);
@@ -734,10 +925,10 @@ int dispatch_waves(bool labels, int B, int K, int H, int Q, int L, int n16max,
                    const int* s_row_ptr, const int* s_col_idx, const float* s_val,
                    const float* X, const float* Wn2l, const float* Wc, const float* Wh1, const float* Wh2,
                    float* msg, float* h_final, float* pool, float* hidden, float* logits, float* probs,
-                   int* pred, int* status, float* h_levels, long long level_stride, hipStream_t s)
+                   int* pred, int* status, float* h_levels, long long level_stride, bool pack, hipStream_t s)
 {
 #define GNNHIP_GF_ARGS B, K, H, Q, L, n16max, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
-                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, h_levels, level_stride, s
+                       X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, h_levels, level_stride, pack, s
     const int tasks = (C / 16) * (n16max / 16);         // (column block x row tile) tasks of the largest graph
     if (tasks <= 4) return dispatch_ksx<C, 4>(labels, GNNHIP_GF_ARGS);
     if (tasks <= 8) return dispatch_ksx<C, 8>(labels, GNNHIP_GF_ARGS);
@@ -778,17 +969,37 @@ int forward_batched_entry(bool labels, int N, int B, int K, int C, int H, int Q,
         return set_error(GNNHIP_EUNSUPPORTED, "a graph of %d nodes does not fit the 160 KB of LDS", max_graph_nodes);
     hipStream_t s = as_stream(stream);
     const float* Xf = static_cast<const float*>(X);
-    int rc;
     if (h_levels && !aligned16(h_levels)) return set_error(GNNHIP_EUNSUPPORTED, "h_levels must be 16-byte aligned");
     const long long level_stride = (long long)N * C;
-#define GNNHIP_GF_ARGS labels, B, K, H, Q, L, n16, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
-                       Xf, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, h_levels, level_stride, s
-    switch (C) {
-    case 16: rc = dispatch_waves<16>(GNNHIP_GF_ARGS); break;
-    case 32: rc = dispatch_waves<32>(GNNHIP_GF_ARGS); break;
-    default: rc = dispatch_waves<64>(GNNHIP_GF_ARGS); break;
-    }
+    auto run = [&](int n16v, bool pack) {
+#define GNNHIP_GF_ARGS labels, B, K, H, Q, L, n16v, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
+                       Xf, W_n2l, W_conv, W_h1, W_h2, msg, h_final, pool, hidden, logits, probs, pred, status, h_levels, level_stride, pack, s
+        switch (C) {
+        case 16: return dispatch_waves<16>(GNNHIP_GF_ARGS);
+        case 32: return dispatch_waves<32>(GNNHIP_GF_ARGS);
+        default: return dispatch_waves<64>(GNNHIP_GF_ARGS);
+        }
 #undef GNNHIP_GF_ARGS
+    };
+    int rc = GNNHIP_EUNSUPPORTED;
+    // more graphs than compute units: runs of consecutive graphs share a workgroup (bins of at least kPackNodes nodes)
+    if (B >= kPackMinGraphs && B <= kBinMaxGraphs && H <= kWave && Q <= kWave && !h_levels) {
+        // Bin size: a workgroup's time grows with its bin (about 6 us + 20 us per 128 nodes), and the bins run in
+        // rounds of one per compute unit, so the size that just avoids another round wins.  The host knows the
+        // totals only: a bin wastes about half a mean graph, and every 64 graphs about half a bin.
+        int best = 0;
+        double best_cost = 0.0;
+        for (int cand = n16 > kPackNodes ? n16 : kPackNodes; cand <= kPackMaxNodes; cand += 16) {
+            if (GraphLds::edge_cap(cand, C, K, H, Q, 1024, labels) < 256) break;
+            const double fill = (double)cand - 0.5 * (double)N / (double)B;
+            const double nbins = (double)N / (fill > 16.0 ? fill : 16.0) + (double)B / 128.0;
+            const double rounds = (double)(long long)((nbins + kNumCU - 1) / kNumCU);
+            const double cost = rounds * (6.0 + 20.0 * cand / 128.0);
+            if (!best || cost < best_cost) { best = cand; best_cost = cost; }
+        }
+        if (best) rc = run(best, true);
+    }
+    if (rc == GNNHIP_EUNSUPPORTED) rc = run(n16, false);
     if (rc == GNNHIP_EUNSUPPORTED) return set_error(rc, "graph-resident forward could not be configured for this shape");
     return rc;
 }

@@ -47,7 +47,12 @@ struct FusedStep
     std::shared_ptr<TrainState> train;      // FORWARD of a training plan
     std::function<void()> backward;         // FORWARD of a training plan: gradients of the four weight matrices
 };
-constexpr size_t kOneLaunchMaxNodes = 20000;   // larger batches run the forward as separate kernels
+// Larger batches run the forward as separate kernels.  Inference: the one-launch forward packs the graphs of
+// batches past 512 graphs into bins and stays ahead up to about 4,000 graphs of 29 nodes (98 against 124 us at
+// 3,000 graphs, 130 against 139 us at 4,000, 165 against 155 us at 5,000).  Training keeps every level and takes
+// the graphs one by one: there the separate kernels win from about 20,000 nodes.
+constexpr size_t kOneLaunchMaxNodes = 120000;
+constexpr size_t kOneLaunchTrainMaxNodes = 20000;
 }  // namespace detail
 
 // The factor names of every step of the plan a FeedForward with these arguments would run, in
@@ -429,7 +434,7 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
                 Logits->value.Reshape({B, Q});
                 float* hs = st->hstack.data->ptr;
                 // small block-diagonal batches: everything in one launch, the levels stored on the way
-                if (n2n->block_diagonal && sub->max_subgraph_nodes > 0 && N <= detail::kOneLaunchMaxNodes) {
+                if (n2n->block_diagonal && sub->max_subgraph_nodes > 0 && N <= detail::kOneLaunchTrainMaxNodes) {
                     const int rc = gnnhip_s2v_forward_batched_train_f32(
                         (int)N, (int)B, (int)K, (int)C, (int)H, (int)Q, L, sub->max_subgraph_nodes,
                         A->value.data->row_ptr, A->value.data->col_idx, A->value.data->val,
@@ -518,8 +523,7 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
             Pool->value.Reshape({B, C});
             Hid->value.Reshape({B, H});
             Logits->value.Reshape({B, Q});
-            // Past about 20,000 nodes the chip is full either way and the separate kernels are faster
-            // (1,000 graphs of configuration 2: 62 us against 70 us in one launch; 256 graphs: 40 against 23).
+            // small and medium block-diagonal batches in one launch (256 graphs of configuration 2: 23 us against 40)
             if (n2n->block_diagonal && sub->contiguous_subgraphs && sub->max_subgraph_nodes > 0 &&
                 N <= detail::kOneLaunchMaxNodes) {
                 const int rc = gnnhip_s2v_forward_batched_f32(

@@ -177,6 +177,10 @@ int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L, int 
  *      embedding.  status (device int, may be NULL; caller zeroes it) gets bit 0 set if a graph
  *      exceeds max_graph_nodes, bit 1 if an edge leaves its graph, bit 2 if S is not the identity
  *      layout; results are then unspecified but no access goes out of bounds.
+ *      From 512 graphs on (H and Q up to 64) runs of consecutive graphs are packed into bins of 128
+ *      to 208 nodes that one workgroup carries as a single block-diagonal graph; the bound on a graph
+ *      is then the bin size where that is larger than max_graph_nodes.  Node outputs keep their
+ *      bits, graph outputs agree with the unpacked ones to rounding.
  *      Returns GNNHIP_EUNSUPPORTED (nothing launched) for shapes it does not cover
  *      (hidden not in {16,32,64}, more than 64 label types, graph too large for LDS). */
 int gnnhip_s2v_forward_batched_f32(int N, int B, int K, int C, int H, int Q, int L, int max_graph_nodes,
