@@ -574,7 +574,7 @@ def main():
     ap.add_argument("--no-rooflines", action="store_true",
                     help="skip the configuration-4 / configuration-5 kernel rooflines")
     ap.add_argument("--only", default="", help="comma-separated legs to run alone (for profiling): "
-                                                "forward, spmm, cfg4, cfg5, train, sizes")
+                                                "forward, spmm, cfg4, cfg5, train, e2e, sizes")
     ap.add_argument("--mkl-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one element-wise copy kernel of known size (1 GiB read, 1 GiB written) "
@@ -610,6 +610,9 @@ def main():
         if "train" in legs:
             _, host = build_forward_workload(dev)
             res["training_step"] = training_step_host_layer(host)
+        if "e2e" in legs:
+            _, host = build_forward_workload(dev)
+            res["end_to_end"] = end_to_end_host_layer(host)
         if "sizes" in legs:
             res["one_launch_by_graphs"] = time_one_launch_by_graphs(dev)
         if args.calibrate:

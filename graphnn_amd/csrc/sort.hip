@@ -246,6 +246,287 @@ __global__ __launch_bounds__(kBlock) void expand_rows_kernel(int m, const int* _
     for (int t = a + lane; t < b; t += kWave) row_of[t] = (int)row;
 }
 
+// ---- small inputs: the whole grouping in one launch of one workgroup ----
+// A batch of a few hundred small graphs is latency, not bandwidth: the dozen launches of the radix passes
+// cost more than the host loop they replace.  One workgroup of 16 wavefronts instead, everything between
+// the first read of the keys and the last write of the result in LDS:
+//   lengths    LDS counters (atomics), and a check whether the keys already ascend
+//   scan       row_ptr; the counters become cursors
+//   place      every pair takes the next slot of its row in whatever order the hardware serves the
+//              atomics; the slot (16 bits, in LDS) keeps the pair's INDEX, so that the next step can put
+//              every row into input order again.  Ascending keys: pair e is slot e, nothing to order.
+//   order      rows of up to 8 entries: a thread sorts them in registers (a fixed network);
+//              longer rows: a wavefront marks the row's pair indices in a bitmap of its own and reads
+//              the set bits back in ascending order, 64 words at a time (a prefix sum of the
+//              population counts gives every word its first slot)
+//   write      slot after slot, coalesced: payload (and value) of the pair the slot names
+// Global loads are issued sixteen to a thread before the first is used.  The order of the entries is a
+// pure function of the input, as on the radix route.  Sizes: 4 bytes per row, 2 per pair, one bitmap
+// of n bits (as many as fit, up to one per wavefront) in 160 KB of LDS; at most 65,536 pairs.
+constexpr int kSmallPairs = 1 << 16;
+constexpr int kSmallBlock = 1024;
+constexpr int kSmallWaves = kSmallBlock / kWave;
+constexpr int kSmallShort = 8;
+constexpr int kSmallBatch = 16;
+constexpr int kSmallLdsInts = 160 * 1024 / 4;
+constexpr int kSmallMisc = 32;
+
+struct SmallLayout {
+    int slots, longs, misc, bitmaps;      // offsets in ints (the counters start at 0)
+    int words, nbitmaps;                  // words per bitmap, number of bitmaps
+};
+// false: the input does not fit one workgroup's LDS
+inline bool small_layout(long long rows, long long n, SmallLayout* out)
+{
+    if (n < 1 || n > kSmallPairs || rows > kSmallLdsInts) return false;
+    SmallLayout l;
+    l.slots = (int)rows;
+    l.longs = l.slots + (int)((n + 1) / 2);
+    l.misc = l.longs + (int)((n / (kSmallShort + 1) + 2) / 2);
+    l.bitmaps = l.misc + kSmallMisc;
+    l.words = (int)((n + 31) / 32);
+    const int room = kSmallLdsInts - l.bitmaps;
+    if (room < l.words) return false;
+    l.nbitmaps = room / l.words < kSmallWaves ? room / l.words : kSmallWaves;
+    *out = l;
+    return true;
+}
+
+// inclusive prefix sum over the wavefront: shifts inside the rows of 16 lanes (lanes without a source add 0),
+// then the totals of the rows below
+__device__ __forceinline__ int wave_inclusive_scan_i(int v)
+{
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, true);      // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, true);      // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, true);      // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, true);      // row_shr:8
+    const int t0 = __builtin_amdgcn_readlane(v, 15), t1 = __builtin_amdgcn_readlane(v, 31), t2 = __builtin_amdgcn_readlane(v, 47);
+    const int row = (threadIdx.x & (kWave - 1)) >> 4;
+    return v + (row >= 1 ? t0 : 0) + (row >= 2 ? t1 : 0) + (row >= 3 ? t2 : 0);
+}
+
+__device__ __forceinline__ void order_pair(int& a, int& b)
+{
+    const int lo = min(a, b), hi = max(a, b);
+    a = lo;
+    b = hi;
+}
+
+__global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(
+    int rows, int n, SmallLayout lay, const int* __restrict__ key, int key_stride, const int* __restrict__ payload, int payload_stride,
+    const float* __restrict__ val_in, int average, int* __restrict__ row_ptr, int* __restrict__ col_idx, float* __restrict__ val)
+{
+    extern __shared__ int small_lds[];
+    int* cnt = small_lds;
+    unsigned short* slots = reinterpret_cast<unsigned short*>(small_lds + lay.slots);
+    unsigned short* longs = reinterpret_cast<unsigned short*>(small_lds + lay.longs);       // rows of more than kSmallShort entries
+    int* misc = small_lds + lay.misc;              // [0] long rows, [1] keys out of order, [2..17] wavefront totals
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int top = rows - 1;
+
+    for (int r = tid; r < rows; r += kSmallBlock) cnt[r] = 0;
+    if (tid < kSmallMisc) misc[tid] = 0;
+    __syncthreads();
+
+    // lengths.  Lanes hold consecutive pairs; a run of equal keys (a batch that arrives grouped is nothing
+    // else) is counted by its first lane alone.  The keys of the first batch stay in registers for `place`.
+    bool disorder = false;
+    int first_keys[kSmallBatch];
+    for (int base0 = 0; base0 < n; base0 += kSmallBlock * kSmallBatch) {       // every lane walks every batch: the ballots need them
+        const int base = base0 + tid;
+        int k[kSmallBatch], before[kSmallBatch];
+#pragma unroll
+        for (int u = 0; u < kSmallBatch; ++u) {
+            const int e = base + u * kSmallBlock;
+            k[u] = e < n ? key[(long long)e * key_stride] : 0;
+            before[u] = (e < n && e > 0 && lane == 0) ? key[(long long)(e - 1) * key_stride] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < kSmallBatch; ++u) {
+            const int e = base + u * kSmallBlock;
+            const int kk = e < n ? min(max(k[u], 0), top) : -1;
+            if (base0 == 0) first_keys[u] = kk;
+            const int left = __shfl_up(kk, 1, kWave);
+            const int prev = lane == 0 ? (e > 0 && e < n ? min(max(before[u], 0), top) : -1) : left;
+            const bool head = lane == 0 || left != kk;
+            const unsigned long long heads = __ballot(head);
+            if (kk >= 0) {
+                disorder |= prev > kk;
+                if (head) {
+                    const unsigned long long later = lane == kWave - 1 ? 0ull : heads >> (lane + 1);
+                    atomicAdd(&cnt[kk], later ? __ffsll((long long)later) : kWave - lane);
+                }
+            }
+        }
+    }
+    if (disorder) misc[1] = 1;
+    __syncthreads();
+
+    // exclusive scan: a wavefront owns a run of rows and walks it 64 at a time
+    const int uwave = __builtin_amdgcn_readfirstlane(wave);
+    const int seg = ((rows + kSmallWaves - 1) / kSmallWaves + kWave - 1) & ~(kWave - 1);
+    const int s0 = min(uwave * seg, rows), s1 = min(s0 + seg, rows);
+    int part = 0;
+    for (int r = s0 + lane; r < s1; r += kWave) part += cnt[r];
+    part = wave_sum_i(part);
+    if (lane == 0) misc[2 + uwave] = part;
+    __syncthreads();
+    const int upto = wave_inclusive_scan_i(lane < kSmallWaves ? misc[2 + lane] : 0);
+    int carry = uwave ? __builtin_amdgcn_readlane(upto, uwave - 1) : 0;
+    for (int r = s0 + lane; r - lane < s1; r += kWave) {
+        const int c = r < s1 ? cnt[r] : 0;
+        const int through = wave_inclusive_scan_i(c);
+        if (r < s1) cnt[r] = carry + through - c;
+        carry += __builtin_amdgcn_readlane(through, kWave - 1);
+    }
+    const bool ascending = misc[1] == 0;
+    __syncthreads();
+    for (int r = tid; r < rows; r += kSmallBlock) row_ptr[r] = cnt[r];
+    if (tid == 0) row_ptr[rows] = n;
+
+    if (!ascending) {
+        __syncthreads();                  // the starts are on their way out; the counters turn into cursors
+#pragma unroll
+        for (int u = 0; u < kSmallBatch; ++u) {
+            const int e = tid + u * kSmallBlock;
+            if (e < n) slots[atomicAdd(&cnt[first_keys[u]], 1)] = (unsigned short)e;
+        }
+        for (int base = tid + kSmallBlock * kSmallBatch; base < n; base += kSmallBlock * kSmallBatch) {
+            int k[kSmallBatch];
+#pragma unroll
+            for (int u = 0; u < kSmallBatch; ++u) {
+                const int e = base + u * kSmallBlock;
+                k[u] = e < n ? key[(long long)e * key_stride] : 0;
+            }
+#pragma unroll
+            for (int u = 0; u < kSmallBatch; ++u) {
+                const int e = base + u * kSmallBlock;
+                if (e < n) slots[atomicAdd(&cnt[min(max(k[u], 0), top)], 1)] = (unsigned short)e;
+            }
+        }
+        __syncthreads();                  // cnt[r] is now the end of row r
+
+        for (int r0 = 0; r0 < rows; r0 += kSmallBlock) {
+            const int r = r0 + tid;
+            int a = 0, len = 0;
+            if (r < rows) {
+                a = r ? cnt[r - 1] : 0;
+                len = cnt[r] - a;
+            }
+            if (len > kSmallShort) {
+                longs[atomicAdd(&misc[0], 1)] = (unsigned short)r;      // r < 65,536: more rows than that leave no room for their pairs
+                len = 0;
+            }
+            if (__ballot(len >= 2) == 0ull) continue;
+            if (__ballot(len > 4) == 0ull) {
+                // nobody in this wavefront has more than 4: 5 exchanges order 4 values
+                int v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = j < len ? (int)slots[a + j] : 0x7fffffff;
+                order_pair(v[0], v[1]); order_pair(v[2], v[3]); order_pair(v[0], v[2]); order_pair(v[1], v[3]); order_pair(v[1], v[2]);
+                if (len >= 2) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (j < len) slots[a + j] = (unsigned short)v[j];
+                }
+                continue;
+            }
+            int v[kSmallShort];
+#pragma unroll
+            for (int j = 0; j < kSmallShort; ++j) v[j] = j < len ? (int)slots[a + j] : 0x7fffffff;
+            // 19 exchanges order 8 values
+            order_pair(v[0], v[1]); order_pair(v[2], v[3]); order_pair(v[4], v[5]); order_pair(v[6], v[7]);
+            order_pair(v[0], v[2]); order_pair(v[1], v[3]); order_pair(v[4], v[6]); order_pair(v[5], v[7]);
+            order_pair(v[1], v[2]); order_pair(v[5], v[6]); order_pair(v[0], v[4]); order_pair(v[3], v[7]);
+            order_pair(v[1], v[5]); order_pair(v[2], v[6]);
+            order_pair(v[1], v[4]); order_pair(v[3], v[6]);
+            order_pair(v[2], v[4]); order_pair(v[3], v[5]);
+            order_pair(v[3], v[4]);
+            if (len >= 2) {
+#pragma unroll
+                for (int j = 0; j < kSmallShort; ++j)
+                    if (j < len) slots[a + j] = (unsigned short)v[j];
+            }
+        }
+        __syncthreads();
+
+        const int nlong = misc[0];
+        if (nlong > 0 && wave < lay.nbitmaps) {
+            unsigned* bits = reinterpret_cast<unsigned*>(small_lds + lay.bitmaps) + wave * lay.words;
+            for (int i = lane; i < lay.words; i += kWave) bits[i] = 0u;
+            for (int q = wave; q < nlong; q += lay.nbitmaps) {
+                const int r = longs[q];
+                const int a = r ? cnt[r - 1] : 0, b = cnt[r];
+                int lo = 0x7fffffff, hi = -1;
+                for (int i = a + lane; i < b; i += kWave) {
+                    const int e = slots[i];
+                    atomicOr(&bits[e >> 5], 1u << (e & 31));
+                    lo = min(lo, e);
+                    hi = max(hi, e);
+                }
+#pragma unroll
+                for (int d = 1; d < kWave; d <<= 1) {
+                    lo = min(lo, __shfl_xor(lo, d, kWave));
+                    hi = max(hi, __shfl_xor(hi, d, kWave));
+                }
+                __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                const int last_word = hi >> 5;
+                int slot = a;
+                for (int word0 = lo >> 5; word0 <= last_word; word0 += kWave) {
+                    const int word = word0 + lane;
+                    unsigned m = 0u;
+                    if (word <= last_word) {
+                        m = bits[word];
+                        bits[word] = 0u;
+                    }
+                    const int c = __popc(m);
+                    const int through = wave_inclusive_scan_i(c);
+                    int at = slot + through - c;
+                    while (m) {
+                        slots[at++] = (unsigned short)(word * 32 + (__ffs((int)m) - 1));
+                        m &= m - 1u;
+                    }
+                    slot += __shfl(through, kWave - 1, kWave);
+                }
+                __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+        __syncthreads();
+    }
+
+    // slot i holds pair e: out it goes
+    for (int base = tid; base < n; base += kSmallBlock * kSmallBatch) {
+        int e[kSmallBatch], pay[kSmallBatch], k[kSmallBatch];
+        float w[kSmallBatch];
+#pragma unroll
+        for (int u = 0; u < kSmallBatch; ++u) {
+            const int i = base + u * kSmallBlock;
+            e[u] = i < n ? (ascending ? i : (int)slots[i]) : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < kSmallBatch; ++u) {
+            const bool live = base + u * kSmallBlock < n;
+            pay[u] = live ? payload[(long long)e[u] * payload_stride] : 0;
+            w[u] = (live && val_in) ? val_in[e[u]] : 1.0f;
+            k[u] = (live && average) ? key[(long long)e[u] * key_stride] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < kSmallBatch; ++u) {
+            const int i = base + u * kSmallBlock;
+            if (i >= n) continue;
+            if (average) {
+                const int kk = min(max(k[u], 0), top);
+                const int len = ascending ? (kk < top ? cnt[kk + 1] : n) - cnt[kk] : cnt[kk] - (kk ? cnt[kk - 1] : 0);
+                w[u] = (float)(1.0 / (double)len);       // as the reference: double divide, then narrowed
+            }
+            col_idx[i] = pay[u];
+            val[i] = w[u];
+        }
+    }
+}
+
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 }  // namespace
@@ -275,6 +556,16 @@ int radix_order_by_digit(const unsigned* keys, long long n, int shift, unsigned*
 int csr_group_pairs(int rows, long long n, const int* key, int key_stride, const int* payload, int payload_stride,
                     const float* val_in, int average, int* row_ptr, int* col_idx, float* val, hipStream_t s)
 {
+    SmallLayout lay;
+    if (small_layout(rows, n, &lay)) {
+        static LdsLimit limit;
+        if (limit.raise(reinterpret_cast<const void*>(csr_group_small_kernel), sizeof(int) * kSmallLdsInts) != hipSuccess)
+            return set_error(GNNHIP_EHIP, "csr_group: %zu bytes of LDS refused", sizeof(int) * kSmallLdsInts);
+        hipLaunchKernelGGL(csr_group_small_kernel, dim3(1), dim3(kSmallBlock), sizeof(int) * (size_t)(lay.bitmaps + lay.words * lay.nbitmaps), s,
+                           rows, (int)n, lay, key, key_stride, payload, payload_stride, val_in, average, row_ptr, col_idx, val);
+        GNNHIP_LAUNCH_CHECK("csr_group_small");
+        return GNNHIP_OK;
+    }
     const int ntiles = (int)((n + kTile - 1) / kTile);
     const long long nhist = (long long)kDigits * (ntiles > 0 ? ntiles : 1);
     size_t off = 0;

@@ -126,19 +126,51 @@ inline void group_edges_on_device(GraphStruct* graph, bool payload_is_edge, bool
     GNN_HIP(gnnhip_csr_group_i32(N, E, pairs + 1, 2, payload, payload_stride, average ? 1 : 0,
                                  out.data->row_ptr, out.data->col_idx, out.data->val, GpuHandle::Stream()));
 }
+// CSR [num_subgraph, num_nodes] on the device from one copy of the (subgraph, node) records
+inline void group_nodes_on_device(GraphStruct* graph, bool average, SpTensor<GPU, float>& out, DTensor<GPU, int>& staging)
+{
+    static_assert(sizeof(std::pair<int, int>) == 2 * sizeof(int), "node list is not a flat (subgraph, node) array");
+    const int M = (int)graph->node_list.size(), B = (int)graph->num_subgraph;
+    out.Reshape({(size_t)B, (size_t)graph->num_nodes});
+    out.ResizeSp(M, B + 1);
+    staging.Reshape({2 * (size_t)std::max(M, 1)});
+    int* pairs = staging.data->ptr;
+    if (M > 0) GNN_HIP(gnnhip_memcpy_h2d(pairs, graph->node_list.data(), sizeof(int) * 2 * (size_t)M, GpuHandle::Stream()));
+    GNN_HIP(gnnhip_csr_group_i32(B, M, pairs, 2, pairs + 1, 2, average ? 1 : 0, out.data->row_ptr, out.data->col_idx, out.data->val,
+                                 GpuHandle::Stream()));
+}
+// The device groups a batch in one launch of one workgroup when its counters (4 bytes per row) and slots
+// (2.4 bytes per pair, with the lists and one bitmap) fit 160 KB of LDS, and with a radix sort from 65,536
+// pairs.  What is left to the host loop is the range between the two, where the dozen launches of the sort
+// cost more than the loop.
+constexpr size_t kRadixGroupingPairs = 1u << 16;
+inline bool device_grouping_pays(size_t pairs, size_t rows)
+{
+    return pairs >= kRadixGroupingPairs || 4 * rows + 12 * pairs / 5 + 1024 <= 160 * 1024;
+}
 template<typename Dtype, typename SpT>
 inline bool group_edges_if_gpu(GraphStruct*, bool, bool, size_t, SpT&, DTensor<GPU, int>&) { return false; }
-// Below this many edges the host loop plus three small copies is quicker than the dozen launches of
-// the device sort (configuration 2, 16k edges: 0.26 ms per batch against 0.29 ms).
-constexpr unsigned kDeviceGroupingMinEdges = 1u << 16;
 template<>
 inline bool group_edges_if_gpu<float, SpTensor<GPU, float> >(GraphStruct* graph, bool payload_is_edge, bool average, size_t num_cols,
                                                              SpTensor<GPU, float>& out, DTensor<GPU, int>& staging)
 {
-    if (graph->num_edges < kDeviceGroupingMinEdges) return false;
+    if (!device_grouping_pays(graph->num_edges, graph->num_nodes)) return false;
     group_edges_on_device(graph, payload_is_edge, average, num_cols, out, staging);
     return true;
 }
+template<typename Dtype, typename SpT>
+inline bool group_nodes_if_gpu(GraphStruct*, bool, SpT&, DTensor<GPU, int>&) { return false; }
+template<>
+inline bool group_nodes_if_gpu<float, SpTensor<GPU, float> >(GraphStruct* graph, bool average, SpTensor<GPU, float>& out,
+                                                             DTensor<GPU, int>& staging)
+{
+    if (!device_grouping_pays(graph->node_list.size(), graph->num_subgraph)) return false;
+    group_nodes_on_device(graph, average, out, staging);
+    return true;
+}
+// Batches of up to this many nodes are examined on the host for edges between subgraphs (the one-launch
+// forward needs to know before it is chosen); larger ones take the general kernels either way.
+constexpr unsigned kExamineBlocksMaxNodes = 1u << 17;
 }  // namespace detail
 
 template<typename mode, typename Dtype>
@@ -155,10 +187,23 @@ protected:
     virtual bool TransposeForBackward() const override { return true; }
     virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out) override
     {
-        this->layout.block_diagonal = false;           // not examined on this route
-        return detail::group_edges_if_gpu<Dtype>(graph, false, this->average, graph->num_nodes, out, edge_staging);
+        if (!detail::group_edges_if_gpu<Dtype>(graph, false, this->average, graph->num_nodes, out, edge_staging)) return false;
+        this->layout.block_diagonal = graph->num_nodes <= detail::kExamineBlocksMaxNodes && NoEdgeBetweenSubgraphs(graph);
+        return true;
     }
     DTensor<GPU, int> edge_staging;
+
+    // does every edge stay inside one subgraph?  (node -> subgraph from the AddNode records)
+    bool NoEdgeBetweenSubgraphs(GraphStruct* graph)
+    {
+        node_subgraph.assign(graph->num_nodes, -1);
+        for (const auto& sn : graph->node_list)
+            if (sn.second >= 0 && sn.second < (int)graph->num_nodes) node_subgraph[sn.second] = sn.first;
+        const int* where = node_subgraph.data();
+        int differ = 0;
+        for (const auto& e : graph->edge_list) differ |= where[e.first] ^ where[e.second];
+        return differ == 0;
+    }
 
     virtual void InitCPUWeight(GraphStruct* graph) override
     {
@@ -169,13 +214,7 @@ protected:
         // rows from the flat edge list (stable by head node): the entries of in_edges->head[i], row after row
         graph->GroupEdgesByHead(false, rp, w.data->col_idx);
         detail::fill_row_weights(rp, (int)graph->num_nodes, this->average, w.data->val);
-        // does any edge join two subgraphs?  (node -> subgraph from the AddNode records)
-        node_subgraph.assign(graph->num_nodes, -1);
-        for (const auto& sn : graph->node_list)
-            if (sn.second >= 0 && sn.second < (int)graph->num_nodes) node_subgraph[sn.second] = sn.first;
-        bool diagonal = true;
-        for (const auto& e : graph->edge_list) diagonal = diagonal && node_subgraph[e.first] == node_subgraph[e.second];
-        this->layout.block_diagonal = diagonal;
+        this->layout.block_diagonal = NoEdgeBetweenSubgraphs(graph);
     }
     std::vector<int> node_subgraph;
 };
@@ -280,6 +319,28 @@ public:
     virtual const char* FuseKind() const override { return "msg_subgraph"; }
 
 protected:
+    // Nodes added subgraph after subgraph, each with the next index (GetBatch does): the matrix is then the
+    // identity layout, its facts are known from one pass over the records, and the device groups it.
+    virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out) override
+    {
+        const int M = (int)graph->node_list.size();
+        if (M != (int)graph->num_nodes) return false;
+        int biggest = 0, run = 0, prev = 0;
+        bool ordered = true;
+        for (int i = 0; i < M && ordered; ++i) {
+            const int g = graph->node_list[i].first;
+            ordered = graph->node_list[i].second == i && g >= prev && g < (int)graph->num_subgraph;
+            run = g == prev ? run + 1 : 1;
+            biggest = std::max(biggest, run);
+            prev = g;
+        }
+        if (!ordered || !detail::group_nodes_if_gpu<Dtype>(graph, this->average, out, node_staging)) return false;
+        this->layout.contiguous_subgraphs = true;
+        this->layout.max_subgraph_nodes = biggest;
+        return true;
+    }
+    DTensor<GPU, int> node_staging;
+
     virtual void InitCPUWeight(GraphStruct* graph) override
     {
         auto& w = this->cpu_weight;

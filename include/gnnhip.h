@@ -97,8 +97,11 @@ int gnnhip_spmm_csr_f32(int m, int k, int n, int nnz, float alpha, const int* ro
  *      index), SubgraphMsgPass (key = subgraph, payload = node) -- src/nn/msg_pass.cpp:46-94,156-177,
  *      lists filled by GraphStruct::AddEdge / AddNode (src/util/graph_struct.cpp:62-75).
  *      key[e * key_stride], payload[e * payload_stride] (strides in ints, so an array of (x, y) pairs
- *      can be passed as it is).  val = 1, or 1 / row length when average != 0.  Stable radix sort,
- *      no atomics on global memory: the result is bit-identical to the host construction. */
+ *      can be passed as it is).  val = 1, or 1 / row length when average != 0.  Stable radix sort without
+ *      atomics on global memory, or, for up to 65,536 pairs whose rows (4 bytes each) and pairs (2.4 bytes
+ *      each) fit 160 KB of LDS, one launch of one workgroup that puts every row back into input order:
+ *      either way the result is a pure function of the input, bit-identical to the host construction.
+ *      The outputs must not overlap key or payload. */
 int gnnhip_csr_group_i32(int rows, int n, const int* key, int key_stride, const int* payload, int payload_stride,
                          int average, int* row_ptr, int* col_idx, float* val, void* stream);
 

@@ -1631,9 +1631,65 @@ def test_device_csr_group_edge_cases_and_scale(gpu, oracle):
         assert np.array_equal(_n(g), w_)
 
 
-@pytest.mark.parametrize("m,k,nnz", [(411, 233, 3000), (5000, 7000, 120_000), (3, 70_000, 32_768), (1, 1, 1)])
+def _stable_group(rows, key, pay, average=False):
+    order = np.argsort(key, kind="stable")
+    rp = np.zeros(rows + 1, np.int64); np.cumsum(np.bincount(key, minlength=rows), out=rp[1:])
+    lens = np.diff(rp)
+    val = (1.0 / np.repeat(lens, lens).astype(np.float64)).astype(np.float32) if average else np.ones(len(key), np.float32)
+    return rp, pay[order], val
+
+
+@pytest.mark.parametrize("case", ["lengths_around_eight", "hub_in_a_window", "one_row_of_all", "past_one_workgroup", "many_rows", "ascending",
+                                  "ascending_but_one", "long_rows_only", "two_pairs"])
+def test_device_csr_group_of_a_small_batch_in_one_launch(gpu, case):
+    """pairs and rows that fit 160 KB of LDS (4 bytes per row, 2.4 per pair, at most 65,536 pairs) are grouped by one
+    workgroup: rows of up to 8 entries ordered by a thread, longer rows by a wavefront with a bitmap (one bitmap only in
+    the largest cases), keys that already ascend copied through; bit-identical to the stable sort"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(sum(map(ord, case)))
+    if case == "lengths_around_eight":
+        lens = rng.integers(0, 19, 3000); lens[:40] = [0, 7, 8, 9, 10, 1, 64, 65] * 5
+        rows = len(lens); key = rng.permutation(np.repeat(np.arange(rows), lens)).astype(np.int32)
+    elif case == "hub_in_a_window":
+        # a batch as GetBatch lays it out: a row's pairs lie close together; one graph has a hub of 900 pairs
+        rows = 9000; key = np.sort(rng.integers(0, rows, 30000)).astype(np.int32)
+        for i in range(0, 30000, 50):
+            key[i:i + 50] = rng.permutation(key[i:i + 50])
+        key[12000:12900] = key[12000]
+    elif case == "one_row_of_all":
+        rows = 5; key = np.full(65536, 3, np.int32)
+        key[::1000] = 1                                           # not ascending, so that the row is really ordered
+    elif case == "past_one_workgroup":
+        rows = 32768; key = rng.integers(0, rows, 65536).astype(np.int32)
+    elif case == "many_rows":
+        rows = 21000; key = rng.integers(0, rows, 30000).astype(np.int32); key[5000:5400] = 20999
+    elif case == "ascending":
+        rows = 700; key = np.sort(rng.integers(0, rows, 40000)).astype(np.int32)
+    elif case == "ascending_but_one":
+        rows = 700; key = np.sort(rng.integers(0, rows, 40000)).astype(np.int32); key[-1] = 0
+    elif case == "long_rows_only":
+        rows = 256; key = rng.integers(0, rows, 7450).astype(np.int32)
+    else:
+        rows = 3; key = np.array([2, 0], np.int32)
+    n = len(key)
+    pay = rng.integers(0, 1 << 30, n).astype(np.int32)
+    for average in (False, True):
+        rp, ci, v = ops.csr_group(rows, _t(key, gpu), _t(pay, gpu), average)
+        want = _stable_group(rows, key, pay, average)
+        assert np.array_equal(_n(rp), want[0]), case
+        assert np.array_equal(_n(ci), want[1]), case
+        assert np.array_equal(_n(v), want[2]), case
+    # strided pairs, and a second call on the same stream (the counters and bitmaps start clean every time)
+    pairs = _t(np.stack([pay, key], axis=1).reshape(-1), gpu)
+    rp, ci, v = ops.csr_group(rows, pairs[1:], pairs, False, key_stride=2, payload_stride=2, n=n)
+    want = _stable_group(rows, key, pay)
+    assert np.array_equal(_n(rp), want[0]) and np.array_equal(_n(ci), want[1])
+
+
+@pytest.mark.parametrize("m,k,nnz", [(411, 233, 3000), (5000, 7000, 120_000), (3, 70_000, 32_768), (1, 1, 1), (900, 20_000, 65_536),
+                                     (32_768, 32_768, 65_537)])
 def test_device_csr_transpose(gpu, oracle, m, k, nnz):
-    """one tile, many tiles, few long rows of A, a single entry"""
+    """one tile, many tiles, few long rows of A, a single entry, the largest one-launch case, one entry past it"""
     from graphnn_amd import ops
     rng = np.random.default_rng(10 + m)
     csr = _random_csr(rng, m, k, nnz)
