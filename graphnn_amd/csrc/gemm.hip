@@ -10,7 +10,8 @@
 // Bound: HBM for the shapes above; algorithmic bytes 4(mk + kn + mn).
 //
 // Weight gradients are the opposite shape: op(A)^T * G with a small output (hidden x hidden) and k = nodes.
-// One output tile would walk all of k on one CU (1.1 ms at k = 7,450), so such products are split along k:
+// One output tile would walk all of k on one CU (1.1 ms at k = 7,450; 15 us at k = 256, a microsecond per step of 16),
+// so such products are split along k from k = 256:
 // every workgroup takes a range of k, writes its partial tile to scratch, and a second kernel adds the
 // partial tiles in range order (deterministic) and applies alpha and beta.
 #include "gnnhip_internal.h"
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
 }
 
 // C = alpha * (sum over z of partial[z]) + beta * C.  A workgroup takes 64 consecutive elements; wavefront w
-// adds the ranges z = w, w + 4, ... (four loads in flight per lane) and the four sums are added in
+// adds the ranges z = w, w + 4, ... (up to sixteen loads in flight per lane) and the four sums are added in
 // wavefront order, so the result is the same on every run.
 __global__ __launch_bounds__(kBlock) void sgemm_splitk_reduce_kernel(int m, int n, int splits, float alpha,
                                                                      const float* __restrict__ partial, float beta,
@@ -136,8 +137,17 @@ __global__ __launch_bounds__(kBlock) void sgemm_splitk_reduce_kernel(int m, int 
     for (size_t base = (size_t)blockIdx.x * kWave; base < total; base += (size_t)gridDim.x * kWave) {
         const size_t idx = base + lane;
         float sum = 0.f;
+        float* dst = C + (idx / n) * (size_t)ldc + idx % n;
+        const float c_old = (wave == 0 && idx < total && beta != 0.f) ? *dst : 0.f;      // asked for before the sums, not after
         if (idx < total) {
             int z = wave;
+            for (; z + 15 * kWaves < splits; z += 16 * kWaves) {
+                float p[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) p[u] = partial[(size_t)(z + u * kWaves) * total + idx];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) sum += p[u];
+            }
             for (; z + 3 * kWaves < splits; z += 4 * kWaves) {
                 const float p0 = partial[(size_t)z * total + idx], p1 = partial[(size_t)(z + kWaves) * total + idx];
                 const float p2 = partial[(size_t)(z + 2 * kWaves) * total + idx], p3 = partial[(size_t)(z + 3 * kWaves) * total + idx];
@@ -151,9 +161,8 @@ __global__ __launch_bounds__(kBlock) void sgemm_splitk_reduce_kernel(int m, int 
             float t = part[0][lane];
 #pragma unroll
             for (int w = 1; w < kWaves; ++w) t += part[w][lane];
-            float* dst = C + (idx / n) * (size_t)ldc + idx % n;
             const float r = alpha * t;
-            *dst = (beta == 0.f) ? r : r + beta * (*dst);
+            *dst = (beta == 0.f) ? r : r + beta * c_old;
         }
         __syncthreads();
     }
@@ -304,7 +313,7 @@ int gemm_dispatch(int transA, int transB, int m, int n, int k, float alpha, cons
     int k_chunk = 0;
     float* partial = nullptr;
     const long long tiles = (long long)grid.x * grid.y;
-    if (tiles <= kNumCU / 4 && k >= 1024) {
+    if (tiles <= kNumCU / 4 && k >= 256) {
         const long long want = (2 * kNumCU) / tiles;                       // ranges per tile
         long long chunk = ((long long)k + want - 1) / want;
         if (chunk < 4 * BK) chunk = 4 * BK;

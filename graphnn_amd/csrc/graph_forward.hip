@@ -690,7 +690,6 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
                 hv = relu_ref(hv);
                 if (lane < H) hidden[(size_t)gk * H + lane] = hv;
                 float sq = 0.f;
-#pragma unroll 8
                 for (int j = 0; j < H; ++j) {
                     const float hj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(hv), j));
                     if (lane < Q) sq = fmaf(hj, w2[(size_t)j * Q + lane], sq);

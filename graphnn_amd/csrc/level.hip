@@ -51,8 +51,6 @@ bool level_wide_covers(int N, int C);
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kLongRow = 1024;      // level kernel: longer rows are gathered by the whole workgroup
-
 
 // Copy N4 float4s (a compile-time count) from global to LDS.  All of a lane's loads are
 // issued before the first LDS store, so the copy costs one memory round trip.

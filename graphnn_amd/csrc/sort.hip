@@ -246,41 +246,54 @@ __global__ __launch_bounds__(kBlock) void expand_rows_kernel(int m, const int* _
     for (int t = a + lane; t < b; t += kWave) row_of[t] = (int)row;
 }
 
-// ---- small inputs: the whole grouping in one launch of one workgroup ----
+// ---- small inputs: the whole grouping in one launch ----
 // A batch of a few hundred small graphs is latency, not bandwidth: the dozen launches of the radix passes
-// cost more than the host loop they replace.  One workgroup of 16 wavefronts instead, everything between
-// the first read of the keys and the last write of the result in LDS:
-//   lengths    LDS counters (atomics), and a check whether the keys already ascend
+// cost more than the host loop they replace.  One launch of up to 16 workgroups instead.  The rows are cut
+// into as many runs; every workgroup reads ALL keys (they are a few L2 lines per lane) and keeps the pairs
+// of its own run of rows, so no workgroup ever waits for another: the number of keys below its first row,
+// which it counts on the way, is where its part of the result starts.  Between the first read of the keys
+// and the last write of the result everything is in LDS:
+//   lengths    LDS counters (atomics), the pairs below the run, and a check whether the keys already ascend
 //   scan       row_ptr; the counters become cursors
 //   place      every pair takes the next slot of its row in whatever order the hardware serves the
 //              atomics; the slot (16 bits, in LDS) keeps the pair's INDEX, so that the next step can put
-//              every row into input order again.  Ascending keys: pair e is slot e, nothing to order.
+//              every row into input order again.  Ascending keys: the pairs of the run are consecutive
+//              and in order already, nothing to place or to order.
 //   order      rows of up to 8 entries: a thread sorts them in registers (a fixed network);
 //              longer rows: a wavefront marks the row's pair indices in a bitmap of its own and reads
 //              the set bits back in ascending order, 64 words at a time (a prefix sum of the
 //              population counts gives every word its first slot)
 //   write      slot after slot, coalesced: payload (and value) of the pair the slot names
 // Global loads are issued sixteen to a thread before the first is used.  The order of the entries is a
-// pure function of the input, as on the radix route.  Sizes: 4 bytes per row, 2 per pair, one bitmap
-// of n bits (as many as fit, up to one per wavefront) in 160 KB of LDS; at most 65,536 pairs.
+// pure function of the input, as on the radix route.  Sizes: 4 bytes per row of a run, 2 per pair, one
+// bitmap of n bits (as many as fit, up to one per wavefront) in 160 KB of LDS; at most 65,536 pairs.
 constexpr int kSmallPairs = 1 << 16;
 constexpr int kSmallBlock = 1024;
 constexpr int kSmallWaves = kSmallBlock / kWave;
 constexpr int kSmallShort = 8;
 constexpr int kSmallBatch = 16;
 constexpr int kSmallLdsInts = 160 * 1024 / 4;
-constexpr int kSmallMisc = 32;
+constexpr int kSmallMisc = 48;
+constexpr int kSmallGroups = 16;           // workgroups at most
+constexpr int kSmallRunRows = 256;         // rows per workgroup at least
 
 struct SmallLayout {
+    int groups, run;                      // workgroups, rows per workgroup (a multiple of 64)
     int slots, longs, misc, bitmaps;      // offsets in ints (the counters start at 0)
     int words, nbitmaps;                  // words per bitmap, number of bitmaps
 };
-// false: the input does not fit one workgroup's LDS
+// false: the input does not fit the workgroups' LDS
 inline bool small_layout(long long rows, long long n, SmallLayout* out)
 {
-    if (n < 1 || n > kSmallPairs || rows > kSmallLdsInts) return false;
+    if (n < 1 || n > kSmallPairs || rows < 1) return false;
     SmallLayout l;
-    l.slots = (int)rows;
+    long long groups = (rows + kSmallRunRows - 1) / kSmallRunRows;
+    if (groups > kSmallGroups) groups = kSmallGroups;
+    const long long run = ((rows + groups - 1) / groups + kWave - 1) / kWave * kWave;
+    if (run > kSmallLdsInts) return false;
+    l.run = (int)run;
+    l.groups = (int)((rows + run - 1) / run);
+    l.slots = l.run;
     l.longs = l.slots + (int)((n + 1) / 2);
     l.misc = l.longs + (int)((n / (kSmallShort + 1) + 2) / 2);
     l.bitmaps = l.misc + kSmallMisc;
@@ -317,20 +330,23 @@ __global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(
     const float* __restrict__ val_in, int average, int* __restrict__ row_ptr, int* __restrict__ col_idx, float* __restrict__ val)
 {
     extern __shared__ int small_lds[];
-    int* cnt = small_lds;
+    int* cnt = small_lds;                          // one per row of this workgroup's run
     unsigned short* slots = reinterpret_cast<unsigned short*>(small_lds + lay.slots);
     unsigned short* longs = reinterpret_cast<unsigned short*>(small_lds + lay.longs);       // rows of more than kSmallShort entries
-    int* misc = small_lds + lay.misc;              // [0] long rows, [1] keys out of order, [2..17] wavefront totals
+    int* misc = small_lds + lay.misc;              // [0] long rows, [1] keys out of order, [2..17] wavefront totals, [18..33] pairs below
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int uwave = __builtin_amdgcn_readfirstlane(wave);
     const int top = rows - 1;
+    const int lo = (int)blockIdx.x * lay.run, mine = min(lay.run, rows - lo);      // this run: rows lo .. lo + mine - 1
 
-    for (int r = tid; r < rows; r += kSmallBlock) cnt[r] = 0;
+    for (int r = tid; r < mine; r += kSmallBlock) cnt[r] = 0;
     if (tid < kSmallMisc) misc[tid] = 0;
     __syncthreads();
 
     // lengths.  Lanes hold consecutive pairs; a run of equal keys (a batch that arrives grouped is nothing
     // else) is counted by its first lane alone.  The keys of the first batch stay in registers for `place`.
     bool disorder = false;
+    int below = 0;
     int first_keys[kSmallBatch];
     for (int base0 = 0; base0 < n; base0 += kSmallBlock * kSmallBatch) {       // every lane walks every batch: the ballots need them
         const int base = base0 + tid;
@@ -352,26 +368,30 @@ __global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(
             const unsigned long long heads = __ballot(head);
             if (kk >= 0) {
                 disorder |= prev > kk;
-                if (head) {
+                below += kk < lo;
+                if (head && kk >= lo && kk - lo < mine) {
                     const unsigned long long later = lane == kWave - 1 ? 0ull : heads >> (lane + 1);
-                    atomicAdd(&cnt[kk], later ? __ffsll((long long)later) : kWave - lane);
+                    atomicAdd(&cnt[kk - lo], later ? __ffsll((long long)later) : kWave - lane);
                 }
             }
         }
     }
     if (disorder) misc[1] = 1;
+    below = wave_sum_i(below);
+    if (lane == 0) misc[18 + uwave] = below;
     __syncthreads();
 
-    // exclusive scan: a wavefront owns a run of rows and walks it 64 at a time
-    const int uwave = __builtin_amdgcn_readfirstlane(wave);
-    const int seg = ((rows + kSmallWaves - 1) / kSmallWaves + kWave - 1) & ~(kWave - 1);
-    const int s0 = min(uwave * seg, rows), s1 = min(s0 + seg, rows);
+    // exclusive scan: a wavefront owns a stretch of the run and walks it 64 rows at a time
+    const int seg = ((mine + kSmallWaves - 1) / kSmallWaves + kWave - 1) & ~(kWave - 1);
+    const int s0 = min(uwave * seg, mine), s1 = min(s0 + seg, mine);
     int part = 0;
     for (int r = s0 + lane; r < s1; r += kWave) part += cnt[r];
     part = wave_sum_i(part);
     if (lane == 0) misc[2 + uwave] = part;
     __syncthreads();
     const int upto = wave_inclusive_scan_i(lane < kSmallWaves ? misc[2 + lane] : 0);
+    const int first_slot = wave_sum_i(lane < kSmallWaves ? misc[18 + lane] : 0);      // pairs of the runs before this one
+    const int held = __builtin_amdgcn_readlane(upto, kSmallWaves - 1);                 // pairs of this run
     int carry = uwave ? __builtin_amdgcn_readlane(upto, uwave - 1) : 0;
     for (int r = s0 + lane; r - lane < s1; r += kWave) {
         const int c = r < s1 ? cnt[r] : 0;
@@ -381,15 +401,15 @@ __global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(
     }
     const bool ascending = misc[1] == 0;
     __syncthreads();
-    for (int r = tid; r < rows; r += kSmallBlock) row_ptr[r] = cnt[r];
-    if (tid == 0) row_ptr[rows] = n;
+    for (int r = tid; r < mine; r += kSmallBlock) row_ptr[lo + r] = first_slot + cnt[r];
+    if (lo + mine == rows && tid == 0) row_ptr[rows] = n;
 
     if (!ascending) {
         __syncthreads();                  // the starts are on their way out; the counters turn into cursors
 #pragma unroll
         for (int u = 0; u < kSmallBatch; ++u) {
-            const int e = tid + u * kSmallBlock;
-            if (e < n) slots[atomicAdd(&cnt[first_keys[u]], 1)] = (unsigned short)e;
+            const int e = tid + u * kSmallBlock, r = first_keys[u] - lo;
+            if (e < n && r >= 0 && r < mine) slots[atomicAdd(&cnt[r], 1)] = (unsigned short)e;
         }
         for (int base = tid + kSmallBlock * kSmallBatch; base < n; base += kSmallBlock * kSmallBatch) {
             int k[kSmallBatch];
@@ -400,21 +420,21 @@ __global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(
             }
 #pragma unroll
             for (int u = 0; u < kSmallBatch; ++u) {
-                const int e = base + u * kSmallBlock;
-                if (e < n) slots[atomicAdd(&cnt[min(max(k[u], 0), top)], 1)] = (unsigned short)e;
+                const int e = base + u * kSmallBlock, r = min(max(k[u], 0), top) - lo;
+                if (e < n && r >= 0 && r < mine) slots[atomicAdd(&cnt[r], 1)] = (unsigned short)e;
             }
         }
         __syncthreads();                  // cnt[r] is now the end of row r
 
-        for (int r0 = 0; r0 < rows; r0 += kSmallBlock) {
+        for (int r0 = 0; r0 < mine; r0 += kSmallBlock) {
             const int r = r0 + tid;
             int a = 0, len = 0;
-            if (r < rows) {
+            if (r < mine) {
                 a = r ? cnt[r - 1] : 0;
                 len = cnt[r] - a;
             }
             if (len > kSmallShort) {
-                longs[atomicAdd(&misc[0], 1)] = (unsigned short)r;      // r < 65,536: more rows than that leave no room for their pairs
+                longs[atomicAdd(&misc[0], 1)] = (unsigned short)r;
                 len = 0;
             }
             if (__ballot(len >= 2) == 0ull) continue;
@@ -457,23 +477,23 @@ __global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(
             for (int q = wave; q < nlong; q += lay.nbitmaps) {
                 const int r = longs[q];
                 const int a = r ? cnt[r - 1] : 0, b = cnt[r];
-                int lo = 0x7fffffff, hi = -1;
+                int first = 0x7fffffff, last = -1;
                 for (int i = a + lane; i < b; i += kWave) {
                     const int e = slots[i];
                     atomicOr(&bits[e >> 5], 1u << (e & 31));
-                    lo = min(lo, e);
-                    hi = max(hi, e);
+                    first = min(first, e);
+                    last = max(last, e);
                 }
 #pragma unroll
                 for (int d = 1; d < kWave; d <<= 1) {
-                    lo = min(lo, __shfl_xor(lo, d, kWave));
-                    hi = max(hi, __shfl_xor(hi, d, kWave));
+                    first = min(first, __shfl_xor(first, d, kWave));
+                    last = max(last, __shfl_xor(last, d, kWave));
                 }
                 __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
                 __builtin_amdgcn_wave_barrier();
-                const int last_word = hi >> 5;
+                const int last_word = last >> 5;
                 int slot = a;
-                for (int word0 = lo >> 5; word0 <= last_word; word0 += kWave) {
+                for (int word0 = first >> 5; word0 <= last_word; word0 += kWave) {
                     const int word = word0 + lane;
                     unsigned m = 0u;
                     if (word <= last_word) {
@@ -496,18 +516,18 @@ __global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(
         __syncthreads();
     }
 
-    // slot i holds pair e: out it goes
-    for (int base = tid; base < n; base += kSmallBlock * kSmallBatch) {
+    // slot i of this run holds pair e and is entry first_slot + i of the result: out it goes
+    for (int base = tid; base < held; base += kSmallBlock * kSmallBatch) {
         int e[kSmallBatch], pay[kSmallBatch], k[kSmallBatch];
         float w[kSmallBatch];
 #pragma unroll
         for (int u = 0; u < kSmallBatch; ++u) {
             const int i = base + u * kSmallBlock;
-            e[u] = i < n ? (ascending ? i : (int)slots[i]) : 0;
+            e[u] = i < held ? (ascending ? first_slot + i : (int)slots[i]) : 0;
         }
 #pragma unroll
         for (int u = 0; u < kSmallBatch; ++u) {
-            const bool live = base + u * kSmallBlock < n;
+            const bool live = base + u * kSmallBlock < held;
             pay[u] = live ? payload[(long long)e[u] * payload_stride] : 0;
             w[u] = (live && val_in) ? val_in[e[u]] : 1.0f;
             k[u] = (live && average) ? key[(long long)e[u] * key_stride] : 0;
@@ -515,14 +535,14 @@ __global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(
 #pragma unroll
         for (int u = 0; u < kSmallBatch; ++u) {
             const int i = base + u * kSmallBlock;
-            if (i >= n) continue;
+            if (i >= held) continue;
             if (average) {
-                const int kk = min(max(k[u], 0), top);
-                const int len = ascending ? (kk < top ? cnt[kk + 1] : n) - cnt[kk] : cnt[kk] - (kk ? cnt[kk - 1] : 0);
+                const int r = min(max(k[u], 0), top) - lo;
+                const int len = ascending ? (r + 1 < mine ? cnt[r + 1] : held) - cnt[r] : cnt[r] - (r ? cnt[r - 1] : 0);
                 w[u] = (float)(1.0 / (double)len);       // as the reference: double divide, then narrowed
             }
-            col_idx[i] = pay[u];
-            val[i] = w[u];
+            col_idx[first_slot + i] = pay[u];
+            val[first_slot + i] = w[u];
         }
     }
 }
@@ -561,7 +581,7 @@ int csr_group_pairs(int rows, long long n, const int* key, int key_stride, const
         static LdsLimit limit;
         if (limit.raise(reinterpret_cast<const void*>(csr_group_small_kernel), sizeof(int) * kSmallLdsInts) != hipSuccess)
             return set_error(GNNHIP_EHIP, "csr_group: %zu bytes of LDS refused", sizeof(int) * kSmallLdsInts);
-        hipLaunchKernelGGL(csr_group_small_kernel, dim3(1), dim3(kSmallBlock), sizeof(int) * (size_t)(lay.bitmaps + lay.words * lay.nbitmaps), s,
+        hipLaunchKernelGGL(csr_group_small_kernel, dim3(lay.groups), dim3(kSmallBlock), sizeof(int) * (size_t)(lay.bitmaps + lay.words * lay.nbitmaps), s,
                            rows, (int)n, lay, key, key_stride, payload, payload_stride, val_in, average, row_ptr, col_idx, val);
         GNNHIP_LAUNCH_CHECK("csr_group_small");
         return GNNHIP_OK;

@@ -139,14 +139,14 @@ inline void group_nodes_on_device(GraphStruct* graph, bool average, SpTensor<GPU
     GNN_HIP(gnnhip_csr_group_i32(B, M, pairs, 2, pairs + 1, 2, average ? 1 : 0, out.data->row_ptr, out.data->col_idx, out.data->val,
                                  GpuHandle::Stream()));
 }
-// The device groups a batch in one launch of one workgroup when its counters (4 bytes per row) and slots
-// (2.4 bytes per pair, with the lists and one bitmap) fit 160 KB of LDS, and with a radix sort from 65,536
-// pairs.  What is left to the host loop is the range between the two, where the dozen launches of the sort
-// cost more than the loop.
+// The device groups a batch in one launch (up to 16 workgroups, each a run of the rows) when a run's counters
+// (4 bytes per row) and the slots of all pairs (2.35 bytes each, with the lists and one bitmap) fit 160 KB of
+// LDS, and with a radix sort from 65,536 pairs.  What is left to the host loop is what neither covers (fewer
+// pairs than that over more than about 40,000 rows), where the dozen launches of the sort cost more than the loop.
 constexpr size_t kRadixGroupingPairs = 1u << 16;
 inline bool device_grouping_pays(size_t pairs, size_t rows)
 {
-    return pairs >= kRadixGroupingPairs || 4 * rows + 12 * pairs / 5 + 1024 <= 160 * 1024;
+    return pairs >= kRadixGroupingPairs || rows / 4 + 47 * pairs / 20 + 1024 <= 160 * 1024;
 }
 template<typename Dtype, typename SpT>
 inline bool group_edges_if_gpu(GraphStruct*, bool, bool, size_t, SpT&, DTensor<GPU, int>&) { return false; }

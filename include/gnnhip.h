@@ -98,8 +98,8 @@ int gnnhip_spmm_csr_f32(int m, int k, int n, int nnz, float alpha, const int* ro
  *      lists filled by GraphStruct::AddEdge / AddNode (src/util/graph_struct.cpp:62-75).
  *      key[e * key_stride], payload[e * payload_stride] (strides in ints, so an array of (x, y) pairs
  *      can be passed as it is).  val = 1, or 1 / row length when average != 0.  Stable radix sort without
- *      atomics on global memory, or, for up to 65,536 pairs whose rows (4 bytes each) and pairs (2.4 bytes
- *      each) fit 160 KB of LDS, one launch of one workgroup that puts every row back into input order:
+ *      atomics on global memory, or, for up to 65,536 pairs (2.35 bytes each, plus 4 bytes per row of a
+ *      sixteenth of the rows, have to fit 160 KB of LDS), one launch that puts every row back into input order:
  *      either way the result is a pure function of the input, bit-identical to the host construction.
  *      The outputs must not overlap key or payload. */
 int gnnhip_csr_group_i32(int rows, int n, const int* key, int key_stride, const int* payload, int payload_stride,

@@ -1639,12 +1639,13 @@ def _stable_group(rows, key, pay, average=False):
     return rp, pay[order], val
 
 
-@pytest.mark.parametrize("case", ["lengths_around_eight", "hub_in_a_window", "one_row_of_all", "past_one_workgroup", "many_rows", "ascending",
+@pytest.mark.parametrize("case", ["lengths_around_eight", "hub_in_a_window", "one_row_of_all", "largest", "past_the_largest", "many_rows", "ascending",
                                   "ascending_but_one", "long_rows_only", "two_pairs"])
 def test_device_csr_group_of_a_small_batch_in_one_launch(gpu, case):
-    """pairs and rows that fit 160 KB of LDS (4 bytes per row, 2.4 per pair, at most 65,536 pairs) are grouped by one
-    workgroup: rows of up to 8 entries ordered by a thread, longer rows by a wavefront with a bitmap (one bitmap only in
-    the largest cases), keys that already ascend copied through; bit-identical to the stable sort"""
+    """up to 65,536 pairs are grouped in one launch of up to 16 workgroups, each with a run of the rows (4 bytes per row of
+    the run and 2.35 per pair have to fit 160 KB of LDS): rows of up to 8 entries ordered by a thread, longer rows by a
+    wavefront with a bitmap (one bitmap only in the largest cases), keys that already ascend copied through;
+    bit-identical to the stable sort"""
     from graphnn_amd import ops
     rng = np.random.default_rng(sum(map(ord, case)))
     if case == "lengths_around_eight":
@@ -1659,8 +1660,10 @@ def test_device_csr_group_of_a_small_batch_in_one_launch(gpu, case):
     elif case == "one_row_of_all":
         rows = 5; key = np.full(65536, 3, np.int32)
         key[::1000] = 1                                           # not ascending, so that the row is really ordered
-    elif case == "past_one_workgroup":
+    elif case == "largest":
         rows = 32768; key = rng.integers(0, rows, 65536).astype(np.int32)
+    elif case == "past_the_largest":
+        rows = 45000; key = rng.integers(0, rows, 65536).astype(np.int32)
     elif case == "many_rows":
         rows = 21000; key = rng.integers(0, rows, 30000).astype(np.int32); key[5000:5400] = 20999
     elif case == "ascending":
