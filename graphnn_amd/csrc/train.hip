@@ -26,7 +26,8 @@ __global__ __launch_bounds__(kBlock) void loss_acc_partial_kernel(int B, int Q, 
                                                                   const int* __restrict__ lrow_ptr, const int* __restrict__ lcol,
                                                                   const float* __restrict__ lval, float* __restrict__ probs,
                                                                   float* __restrict__ loss_rows, int* __restrict__ hit_rows,
-                                                                  float* __restrict__ partial /* [2][gridDim.x] */)
+                                                                  float* __restrict__ partial /* [2][gridDim.x] */,
+                                                                  float* __restrict__ loss_mean, float* __restrict__ acc_mean)
 {
     __shared__ float sh_loss[kWavesPerBlock], sh_hit[kWavesPerBlock];
     const int per = (B + gridDim.x - 1) / gridDim.x;
@@ -67,6 +68,12 @@ __global__ __launch_bounds__(kBlock) void loss_acc_partial_kernel(int B, int Q, 
     if (threadIdx.x == 0) {
         float l = 0.f, h = 0.f;
         for (int w = 0; w < kWavesPerBlock; ++w) { l += sh_loss[w]; h += sh_hit[w]; }
+        if (gridDim.x == 1) {
+            // a single workgroup has the whole sums: the means leave from here, as loss_acc_final_kernel would form them
+            if (loss_mean) loss_mean[0] = l / (float)B;
+            if (acc_mean) acc_mean[0] = h / (float)B;
+            return;
+        }
         partial[blockIdx.x] = l;
         partial[gridDim.x + blockIdx.x] = h;
     }
@@ -207,8 +214,9 @@ int gnnhip_s2v_loss_acc_f32(int B, int Q, const float* logits, const int* lrow_p
     void* partial = nullptr;
     if (int rc = stream_scratch(s, sizeof(float) * 2 * (size_t)nb, &partial)) return rc;
     hipLaunchKernelGGL(loss_acc_partial_kernel, dim3((unsigned)nb), dim3(kBlock), 0, s, B, Q, logits, lrow_ptr, lcol, lval, probs,
-                       loss_rows, hit_rows, static_cast<float*>(partial));
+                       loss_rows, hit_rows, static_cast<float*>(partial), loss_mean, acc_mean);
     GNNHIP_LAUNCH_CHECK("loss_acc_partial");
+    if (nb == 1) return GNNHIP_OK;
     hipLaunchKernelGGL(loss_acc_final_kernel, dim3(1), dim3(kWave), 0, s, nb, B, static_cast<const float*>(partial), loss_mean, acc_mean);
     GNNHIP_LAUNCH_CHECK("loss_acc_final");
     return GNNHIP_OK;
