@@ -21,14 +21,14 @@ namespace {
 
 constexpr int BM = 64, BN = 64, BK = 16, kBlock = 256;
 
+// One 64 x 64 output tile (tile_x, tile_y) over k in [k_lo, k_hi).  part != nullptr: the raw sums go to
+// part[m][n]; otherwise the tile finishes C itself.
 template <bool TA, bool TB>
-__global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
-    int m, int n, int k, float alpha, const float* __restrict__ A, int lda,
-    const float* __restrict__ B, int ldb, float beta, float* C, int ldc, int k_chunk, float* __restrict__ partial)
+__device__ __forceinline__ void sgemm_tile_body(
+    int m, int n, float alpha, const float* __restrict__ A, int lda,
+    const float* __restrict__ B, int ldb, float beta, float* C, int ldc, int k_lo, int k_hi, float* __restrict__ part,
+    int tile_x, int tile_y)
 {
-    // partial != nullptr: workgroup z handles k in [z k_chunk, (z+1) k_chunk) and stores its raw sums to
-    // partial[z][m][n]; otherwise one workgroup walks all of k and finishes C itself.
-    //
     // Both tiles sit in LDS with k contiguous, so that a lane fetches its four k values of a step with one
     // 128-bit read.  Wavefront w owns the output rows 16 w .. 16 w + 15 of the tile and all 64 columns: four
     // accumulators of v_mfma_f32_16x16x4_f32 with the operand roles swapped (out^T = B^T * A^T), which leaves
@@ -40,15 +40,13 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1), wave = tid / kWave;
     const int q = lane >> 4, t = lane & 15;
-    const long long row0 = (long long)blockIdx.x * BM;
-    const int col0 = blockIdx.y * BN;
+    const long long row0 = (long long)tile_x * BM;
+    const int col0 = tile_y * BN;
 
     mfma_f4 acc[BN / 16];
 #pragma unroll
     for (int jb = 0; jb < BN / 16; ++jb) acc[jb] = mfma_f4{0.f, 0.f, 0.f, 0.f};
 
-    const int k_lo = partial ? (int)blockIdx.z * k_chunk : 0;
-    const int k_hi = partial ? min(k, k_lo + k_chunk) : k;
     // each lane moves 4 elements of each tile; the elements of step k0 + BK are requested before the
     // products of step k0 are formed, so a step costs the longer of the two instead of their sum
     float ra[4], rb[4];
@@ -111,8 +109,8 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
             for (int i = 0; i < 4; ++i) {
                 const int gj = col0 + jb * 16 + 4 * q + i;
                 if (gj >= n) continue;
-                if (partial) {
-                    partial[((size_t)blockIdx.z * m + gi) * n + gj] = acc[jb][i];
+                if (part) {
+                    part[(size_t)gi * n + gj] = acc[jb][i];
                     continue;
                 }
                 float* dst = C + (size_t)gi * ldc + gj;
@@ -123,12 +121,51 @@ __global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
     }
 }
 
+// partial != nullptr: workgroup z handles k in [z k_chunk, (z+1) k_chunk) and stores its raw sums to
+// partial[z][m][n]; otherwise one workgroup walks all of k and finishes C itself.
+template <bool TA, bool TB>
+__global__ __launch_bounds__(kBlock) void sgemm_tile_kernel(
+    int m, int n, int k, float alpha, const float* __restrict__ A, int lda,
+    const float* __restrict__ B, int ldb, float beta, float* C, int ldc, int k_chunk, float* __restrict__ partial)
+{
+    const int k_lo = partial ? (int)blockIdx.z * k_chunk : 0;
+    const int k_hi = partial ? min(k, k_lo + k_chunk) : k;
+    sgemm_tile_body<TA, TB>(m, n, alpha, A, lda, B, ldb, beta, C, ldc, k_lo, k_hi,
+                            partial ? partial + (size_t)blockIdx.z * m * n : nullptr, (int)blockIdx.x, (int)blockIdx.y);
+}
+
+// Several products C_p = alpha A_p^T B_p + beta C_p in one launch: the weight gradients at the end of a backward
+// pass, each a small output over a long k, none of which fills the GPU alone.  Product p owns the z range
+// [z0[p], z0[p+1]) of the grid, one range of k per z; tiles outside a product's own tile grid leave at once.
+constexpr int kGemmBatch = 8;
+struct GemmBatch {
+    const float* A[kGemmBatch];
+    const float* B[kGemmBatch];
+    float* C[kGemmBatch];
+    float* partial[kGemmBatch];
+    int m[kGemmBatch], n[kGemmBatch], k[kGemmBatch], lda[kGemmBatch], ldb[kGemmBatch], ldc[kGemmBatch];
+    int k_chunk[kGemmBatch], z0[kGemmBatch + 1];
+    int count;
+};
+
+__global__ __launch_bounds__(kBlock) void sgemm_tn_batch_kernel(GemmBatch b)
+{
+    int p = 0;
+    while (p + 1 < b.count && (int)blockIdx.z >= b.z0[p + 1]) ++p;
+    const int m = b.m[p], n = b.n[p];
+    if ((long long)blockIdx.x * BM >= m || (int)blockIdx.y * BN >= n) return;
+    const int z = (int)blockIdx.z - b.z0[p];
+    const int k_lo = z * b.k_chunk[p], k_hi = min(b.k[p], k_lo + b.k_chunk[p]);
+    sgemm_tile_body<true, false>(m, n, 1.0f, b.A[p], b.lda[p], b.B[p], b.ldb[p], 0.0f, b.C[p], b.ldc[p], k_lo, k_hi,
+                                 b.partial[p] + (size_t)z * m * n, (int)blockIdx.x, (int)blockIdx.y);
+}
+
 // C = alpha * (sum over z of partial[z]) + beta * C.  A workgroup takes 64 consecutive elements; wavefront w
 // adds the ranges z = w, w + 4, ... (up to sixteen loads in flight per lane) and the four sums are added in
 // wavefront order, so the result is the same on every run.
-__global__ __launch_bounds__(kBlock) void sgemm_splitk_reduce_kernel(int m, int n, int splits, float alpha,
-                                                                     const float* __restrict__ partial, float beta,
-                                                                     float* C, int ldc)
+__device__ __forceinline__ void sgemm_splitk_reduce_body(int m, int n, int splits, float alpha,
+                                                         const float* __restrict__ partial, float beta,
+                                                         float* C, int ldc)
 {
     __shared__ float part[kBlock / kWave][kWave];
     const size_t total = (size_t)m * n;
@@ -166,6 +203,20 @@ __global__ __launch_bounds__(kBlock) void sgemm_splitk_reduce_kernel(int m, int 
         }
         __syncthreads();
     }
+}
+
+__global__ __launch_bounds__(kBlock) void sgemm_splitk_reduce_kernel(int m, int n, int splits, float alpha,
+                                                                     const float* __restrict__ partial, float beta,
+                                                                     float* C, int ldc)
+{
+    sgemm_splitk_reduce_body(m, n, splits, alpha, partial, beta, C, ldc);
+}
+
+// the sums of product blockIdx.y of a batch
+__global__ __launch_bounds__(kBlock) void sgemm_splitk_reduce_batch_kernel(GemmBatch b, float alpha, float beta)
+{
+    const int p = blockIdx.y;
+    sgemm_splitk_reduce_body(b.m[p], b.n[p], b.z0[p + 1] - b.z0[p], alpha, b.partial[p], beta, b.C[p], b.ldc[p]);
 }
 
 }  // namespace
@@ -294,6 +345,57 @@ void launch_skinny(bool tb, int m, int k, float alpha, const float* A, int lda, 
 
 }  // namespace
 
+// length of the ranges of k when few output tiles share a long k: about two workgroups per CU, four steps at least
+inline long long splitk_chunk(long long tiles, long long k)
+{
+    const long long want = (2 * kNumCU) / tiles;                           // ranges per tile
+    long long chunk = (k + want - 1) / want;
+    if (chunk < 4 * BK) chunk = 4 * BK;
+    return (chunk + BK - 1) / BK * BK;
+}
+
+// count <= kGemmBatch products C_p = alpha A_p^T B_p + beta C_p (A_p stored [k_p, m_p], B_p [k_p, n_p]) in two launches
+int gemm_tn_batch_dispatch(int count, const int* m, const int* n, const int* k, const float* const* A, const int* lda,
+                           const float* const* B, const int* ldb, float alpha, float beta, float* const* C, const int* ldc, hipStream_t s)
+{
+    GemmBatch b;
+    b.count = 0;
+    size_t floats = 0;
+    unsigned gx = 1, gy = 1, red = 1;
+    size_t offset[kGemmBatch];
+    int z = 0;
+    for (int p = 0; p < count; ++p) {
+        if (m[p] == 0 || n[p] == 0) continue;
+        const int q = b.count++;
+        b.A[q] = A[p]; b.B[q] = B[p]; b.C[q] = C[p];
+        b.m[q] = m[p]; b.n[q] = n[p]; b.k[q] = k[p];
+        b.lda[q] = lda[p]; b.ldb[q] = ldb[p]; b.ldc[q] = ldc[p];
+        const unsigned tx = ceil_div_u((size_t)m[p], BM), ty = ceil_div_u((size_t)n[p], BN);
+        const long long tiles = (long long)tx * ty;
+        // the rule of the single product, so that a batch gives the bits of its products done one by one
+        long long chunk = (tiles <= kNumCU / 4 && k[p] >= 256) ? splitk_chunk(tiles, k[p]) : (k[p] > 0 ? k[p] : 1);
+        const int splits = k[p] > 0 ? (int)(((long long)k[p] + chunk - 1) / chunk) : 1;
+        b.k_chunk[q] = (int)chunk;
+        b.z0[q] = z;
+        z += splits;
+        offset[q] = floats;
+        floats += (size_t)splits * m[p] * n[p];
+        if (tx > gx) gx = tx;
+        if (ty > gy) gy = ty;
+        const unsigned r = ceil_div_u((size_t)m[p] * n[p], kWave) < 2048u ? ceil_div_u((size_t)m[p] * n[p], kWave) : 2048u;
+        if (r > red) red = r;
+    }
+    if (b.count == 0) return GNNHIP_OK;
+    b.z0[b.count] = z;
+    void* q = nullptr;
+    if (int rc = stream_scratch_slot(s, 2, sizeof(float) * floats, &q)) return rc;
+    for (int p = 0; p < b.count; ++p) b.partial[p] = static_cast<float*>(q) + offset[p];
+    hipLaunchKernelGGL(sgemm_tn_batch_kernel, dim3(gx, gy, (unsigned)z), dim3(kBlock), 0, s, b);
+    hipLaunchKernelGGL(sgemm_splitk_reduce_batch_kernel, dim3(red, (unsigned)b.count), dim3(kBlock), 0, s, b, alpha, beta);
+    GNNHIP_LAUNCH_CHECK("sgemm_tn_batch");
+    return GNNHIP_OK;
+}
+
 int gemm_dispatch(int transA, int transB, int m, int n, int k, float alpha, const float* A, int lda,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s)
 {
@@ -314,10 +416,7 @@ int gemm_dispatch(int transA, int transB, int m, int n, int k, float alpha, cons
     float* partial = nullptr;
     const long long tiles = (long long)grid.x * grid.y;
     if (tiles <= kNumCU / 4 && k >= 256) {
-        const long long want = (2 * kNumCU) / tiles;                       // ranges per tile
-        long long chunk = ((long long)k + want - 1) / want;
-        if (chunk < 4 * BK) chunk = 4 * BK;
-        chunk = (chunk + BK - 1) / BK * BK;
+        const long long chunk = splitk_chunk(tiles, k);
         const int splits = (int)(((long long)k + chunk - 1) / chunk);
         if (splits > 1) {
             void* q = nullptr;
@@ -363,4 +462,28 @@ extern "C" int gnnhip_gemm_f32(int transA, int transB, int m, int n, int k, floa
     GNNHIP_REQUIRE(ceil_div_u((size_t)n, 64) <= 65535u, "n=%d too wide for the gemm grid", n);
     if (int rc = require_ready()) return rc;
     return gemm_dispatch(transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, as_stream(stream));
+}
+
+extern "C" int gnnhip_gemm_tn_batch_f32(int count, const int* m, const int* n, const int* k, const float* const* A, const int* lda,
+                                        const float* const* B, const int* ldb, float alpha, float beta, float* const* C, const int* ldc,
+                                        void* stream)
+{
+    GNNHIP_REQUIRE(count >= 0, "negative count in gemm_tn_batch");
+    if (count == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(m && n && k && A && lda && B && ldb && C && ldc, "null array in gemm_tn_batch");
+    for (int p = 0; p < count; ++p) {
+        GNNHIP_REQUIRE(m[p] >= 0 && n[p] >= 0 && k[p] >= 0, "negative dimension in gemm_tn_batch (product %d: m=%d n=%d k=%d)", p, m[p], n[p], k[p]);
+        if (m[p] == 0 || n[p] == 0) continue;
+        GNNHIP_REQUIRE(C[p] != nullptr && ldc[p] >= n[p], "bad output in gemm_tn_batch (product %d: ldc=%d n=%d)", p, ldc[p], n[p]);
+        GNNHIP_REQUIRE(k[p] == 0 || (A[p] && B[p] && lda[p] >= m[p] && ldb[p] >= n[p]), "bad operand in gemm_tn_batch (product %d)", p);
+        GNNHIP_REQUIRE(ceil_div_u((size_t)n[p], 64) <= 65535u, "n=%d too wide for the gemm grid", n[p]);
+    }
+    if (int rc = require_ready()) return rc;
+    for (int at = 0; at < count; at += kGemmBatch) {
+        const int take = count - at < kGemmBatch ? count - at : kGemmBatch;
+        if (int rc = gemm_tn_batch_dispatch(take, m + at, n + at, k + at, A + at, lda + at, B + at, ldb + at, alpha, beta, C + at, ldc + at,
+                                            as_stream(stream)))
+            return rc;
+    }
+    return GNNHIP_OK;
 }

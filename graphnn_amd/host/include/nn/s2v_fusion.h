@@ -494,21 +494,24 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
                                                               hs + (size_t)(l - 1) * NC, dmsg, s));
                         std::swap(g, g2);
                     }
-                    if (!cWc)
-                        GNN_HIP(gnnhip_gemm_f32(1, 0, (int)C, (int)C, (int)((size_t)L * N), 1.0f, hs, (int)C, us, (int)C, 1.0f,
-                                                Wc->grad.Full().data->ptr, (int)C, s));
                 } else {
                     GNN_HIP(gnnhip_s2v_grad_gate_f32(NC, hs, g, nullptr, dmsg, 0, s));
                 }
-                if (!cWn)
-                    GNN_HIP(gnnhip_gemm_f32(1, 0, (int)K, (int)C, (int)N, 1.0f, X->value.data->ptr, (int)K, dmsg, (int)C, 1.0f,
-                                            Wn->grad.Full().data->ptr, (int)C, s));
-                if (!cW1)
-                    GNN_HIP(gnnhip_gemm_f32(1, 0, (int)C, (int)H, (int)B, 1.0f, Pool->value.data->ptr, (int)C, st->du.data->ptr, (int)H, 1.0f,
-                                            W1->grad.Full().data->ptr, (int)H, s));
-                if (!cW2)
-                    GNN_HIP(gnnhip_gemm_f32(1, 0, (int)H, (int)Q, (int)B, 1.0f, Hid->value.data->ptr, (int)H, st->dl.data->ptr, (int)Q, 1.0f,
-                                            W2->grad.Full().data->ptr, (int)Q, s));
+                // the weight gradients, x^T dy each and none of them large enough to fill the GPU: one batch
+                int gm[4], gn[4], gk[4], glda[4], gldb[4], gldc[4], count = 0;
+                const float* ga[4];
+                const float* gb[4];
+                float* gc[4];
+                auto product = [&](const float* x, size_t rows, size_t m, const float* dy, size_t n, float* grad) {
+                    ga[count] = x; gb[count] = dy; gc[count] = grad;
+                    gm[count] = glda[count] = (int)m; gn[count] = gldb[count] = gldc[count] = (int)n; gk[count] = (int)rows;
+                    ++count;
+                };
+                if (L > 0 && !cWc) product(hs, (size_t)L * N, C, st->ustack.data->ptr, C, Wc->grad.Full().data->ptr);
+                if (!cWn) product(X->value.data->ptr, N, K, dmsg, C, Wn->grad.Full().data->ptr);
+                if (!cW1) product(Pool->value.data->ptr, B, C, st->du.data->ptr, H, W1->grad.Full().data->ptr);
+                if (!cW2) product(Hid->value.data->ptr, B, H, st->dl.data->ptr, Q, W2->grad.Full().data->ptr);
+                GNN_HIP(gnnhip_gemm_tn_batch_f32(count, gm, gn, gk, ga, glda, gb, gldb, 1.0f, 1.0f, gc, gldc, s));
             };
         } else
         step->run = [=](Phase ph) {

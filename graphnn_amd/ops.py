@@ -92,6 +92,24 @@ def gemm(A, B, transA=False, transB=False, alpha=1.0, beta=0.0, out=None):
     return out
 
 
+def gemm_tn_batch(products, alpha=1.0, beta=0.0):
+    """products: list of (A [k,m], B [k,n], out [m,n]); out = alpha * A^T B + beta * out for all of them in two launches"""
+    import ctypes
+    count = len(products)
+    ints = lambda vals: (ctypes.c_int * count)(*vals)
+    ptrs = lambda ts: (ctypes.c_void_p * count)(*[t.data_ptr() for t in ts])
+    for A, B, out in products:
+        if A.shape[0] != B.shape[0] or tuple(out.shape) != (A.shape[1], B.shape[1]):
+            raise ValueError("mat dim doesn't match")
+        _f32(A, "A"), _f32(B, "B"), _f32(out, "out")
+    As, Bs, Cs = zip(*products) if count else ((), (), ())
+    check(_lib().gnnhip_gemm_tn_batch_f32(count, ints([a.shape[1] for a in As]), ints([b.shape[1] for b in Bs]),
+                                          ints([a.shape[0] for a in As]), ptrs(As), ints([a.shape[1] for a in As]),
+                                          ptrs(Bs), ints([b.shape[1] for b in Bs]), alpha, beta, ptrs(Cs),
+                                          ints([c.shape[1] for c in Cs]), _stream()))
+    return [c for c in Cs]
+
+
 def s2v_input(X, W_n2l):
     N, K = X.shape
     if W_n2l.shape[0] != K:

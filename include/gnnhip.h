@@ -117,6 +117,16 @@ int gnnhip_csr_transpose_f32(int m, int k, int nnz, const int* row_ptr, const in
 int gnnhip_gemm_f32(int transA, int transB, int m, int n, int k, float alpha, const float* A, int lda,
                     const float* B, int ldb, float beta, float* C, int ldc, void* stream);
 
+/* ---- count products C_p[m_p,n_p] = alpha * A_p^T * B_p + beta * C_p in two launches, with A_p stored [k_p,m_p]
+ *      and B_p [k_p,n_p]: the weight gradients that MatMul::Backward forms one by one at the end of a backward pass
+ *      (src/nn/matmul.cpp:35-76, x^T * dy through DTensor<GPU>::MM, src/tensor/gpu_dense_tensor.cu:192-224).
+ *      m, n, k, lda, ldb, ldc and the pointer tables A, B, C are HOST arrays of count entries; the matrices are
+ *      device memory.  Every product gives the bits gnnhip_gemm_f32(1, 0, ...) gives for it alone when that
+ *      call splits k (few output tiles, k >= 256). */
+int gnnhip_gemm_tn_batch_f32(int count, const int* m, const int* n, const int* k, const float* const* A, const int* lda,
+                             const float* const* B, const int* ldb, float alpha, float beta, float* const* C, const int* ldc,
+                             void* stream);
+
 /* ---- one mean-field level in a single pass:
  *      h_out = ReLU((A * h_in) * W + bias + msg)
  *      replaces MatMul(sparse) + MatMul(dense) + ElewiseAdd + ReLU

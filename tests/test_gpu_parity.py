@@ -210,6 +210,32 @@ def test_gemm_all_transposes(gpu, oracle, shape):
             assert_parity("gemm %d%d" % (ta, tb), got2, *_gemm_want(oracle, A, B, ta, tb, alpha=1.5, beta=-0.5, C=C0))
 
 
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (-0.75, 0.5)])
+def test_gemm_batch_of_weight_gradient_products(gpu, oracle, alpha, beta):
+    """the four x^T dy products at the end of a configuration-2 backward pass, a product too short to split, one that
+    covers several output tiles, an empty one and a single element, in two launches: each against the oracle, and
+    bit-identical to the same product through gnnhip_gemm_f32 where that call splits k too"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(77)
+    shapes = [(29800, 64, 64), (7450, 38, 64), (256, 64, 32), (256, 32, 2), (100, 20, 30), (3000, 150, 70), (40, 0, 5),
+              (1, 1, 1), (513, 64, 64)]                       # (k, m, n); nine products: more than one table
+    host = []
+    products = []
+    for k, m, n in shapes:
+        A = rng.standard_normal((k, m)).astype(np.float32); B = rng.standard_normal((k, n)).astype(np.float32)
+        C0 = rng.standard_normal((m, n)).astype(np.float32)
+        host.append((A, B, C0))
+        products.append((_t(A, gpu), _t(B, gpu), _t(C0, gpu)))
+    outs = ops.gemm_tn_batch(products, alpha=alpha, beta=beta)
+    for (k, m, n), (A, B, C0), got in zip(shapes, host, outs):
+        if m == 0:
+            continue
+        assert_parity("gemm batch k=%d m=%d n=%d" % (k, m, n), _n(got), *_gemm_want(oracle, A, B, True, False, alpha=alpha, beta=beta, C=C0))
+        alone = _n(ops.gemm(_t(A, gpu), _t(B, gpu), True, False, alpha=alpha, beta=beta, out=_t(C0, gpu)))
+        if k >= 256 and m <= 512 and n <= 512:
+            assert np.array_equal(_n(got), alone), (k, m, n)
+
+
 def test_gemm_reference_test_shape(gpu, oracle):
     """10x20 . (30x20)^T with |delta ASum| <= 1e-4 (test/gpu_tensor_test.cpp:131-149)"""
     from graphnn_amd import ops
