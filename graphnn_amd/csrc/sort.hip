@@ -325,10 +325,30 @@ __device__ __forceinline__ void order_pair(int& a, int& b)
     b = hi;
 }
 
-__global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(
-    int rows, int n, SmallLayout lay, const int* __restrict__ key, int key_stride, const int* __restrict__ payload, int payload_stride,
-    const float* __restrict__ val_in, int average, int* __restrict__ row_ptr, int* __restrict__ col_idx, float* __restrict__ val)
+// One grouping of the n pairs.  A launch carries one or two of them (the same pairs grouped by either member:
+// a matrix and its transpose); workgroup b works on job b / groups.
+struct SmallJob {
+    const int* key;
+    const int* payload;
+    const float* val_in;
+    int* row_ptr;
+    int* col_idx;
+    float* val;
+    int key_stride, payload_stride;
+};
+
+__global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(int rows, int n, SmallLayout lay, SmallJob job0, SmallJob job1, int average)
 {
+    const bool second = (int)blockIdx.x >= lay.groups;
+    const int run_index = (int)blockIdx.x - (second ? lay.groups : 0);
+    const int* __restrict__ key = second ? job1.key : job0.key;
+    const int* __restrict__ payload = second ? job1.payload : job0.payload;
+    const float* __restrict__ val_in = second ? job1.val_in : job0.val_in;
+    int* __restrict__ row_ptr = second ? job1.row_ptr : job0.row_ptr;
+    int* __restrict__ col_idx = second ? job1.col_idx : job0.col_idx;
+    float* __restrict__ val = second ? job1.val : job0.val;
+    const int key_stride = second ? job1.key_stride : job0.key_stride;
+    const int payload_stride = second ? job1.payload_stride : job0.payload_stride;
     extern __shared__ int small_lds[];
     int* cnt = small_lds;                          // one per row of this workgroup's run
     unsigned short* slots = reinterpret_cast<unsigned short*>(small_lds + lay.slots);
@@ -337,7 +357,7 @@ __global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int uwave = __builtin_amdgcn_readfirstlane(wave);
     const int top = rows - 1;
-    const int lo = (int)blockIdx.x * lay.run, mine = min(lay.run, rows - lo);      // this run: rows lo .. lo + mine - 1
+    const int lo = run_index * lay.run, mine = min(lay.run, rows - lo);            // this run: rows lo .. lo + mine - 1
 
     for (int r = tid; r < mine; r += kSmallBlock) cnt[r] = 0;
     if (tid < kSmallMisc) misc[tid] = 0;
@@ -569,6 +589,28 @@ int radix_order_by_digit(const unsigned* keys, long long n, int shift, unsigned*
     return GNNHIP_OK;
 }
 
+// The one-launch grouping where it fits; false: it does not (nothing launched).  With t_row_ptr the same launch
+// also groups the pairs by payload with the key as the payload: the transpose, its entries in pair order, values 1.
+bool csr_group_small(int rows, long long n, const int* key, int key_stride, const int* payload, int payload_stride, const float* val_in,
+                     int average, int* row_ptr, int* col_idx, float* val, int* t_row_ptr, int* t_col_idx, float* t_val, hipStream_t s)
+{
+    SmallLayout lay;
+    if (!small_layout(rows, n, &lay)) return false;
+    static LdsLimit limit;
+    if (limit.raise(reinterpret_cast<const void*>(csr_group_small_kernel), sizeof(int) * kSmallLdsInts) != hipSuccess) return false;
+    const SmallJob job0 = {key, payload, val_in, row_ptr, col_idx, val, key_stride, payload_stride};
+    const SmallJob job1 = {payload, key, nullptr, t_row_ptr, t_col_idx, t_val, payload_stride, key_stride};
+    hipLaunchKernelGGL(csr_group_small_kernel, dim3(lay.groups * (t_row_ptr ? 2 : 1)), dim3(kSmallBlock),
+                       sizeof(int) * (size_t)(lay.bitmaps + lay.words * lay.nbitmaps), s, rows, (int)n, lay, job0, job1, average);
+    return true;
+}
+
+inline int last_launch_status(const char* what)
+{
+    GNNHIP_LAUNCH_CHECK(what);
+    return GNNHIP_OK;
+}
+
 // Groups n pairs by key (0 <= key < rows) keeping input order inside a group:
 //   row_ptr[rows + 1], col_idx[i] = payload of the i-th pair in grouped order,
 //   val[i] = val_in of that pair (or 1), or 1 / group size when average is set.
@@ -576,16 +618,8 @@ int radix_order_by_digit(const unsigned* keys, long long n, int shift, unsigned*
 int csr_group_pairs(int rows, long long n, const int* key, int key_stride, const int* payload, int payload_stride,
                     const float* val_in, int average, int* row_ptr, int* col_idx, float* val, hipStream_t s)
 {
-    SmallLayout lay;
-    if (small_layout(rows, n, &lay)) {
-        static LdsLimit limit;
-        if (limit.raise(reinterpret_cast<const void*>(csr_group_small_kernel), sizeof(int) * kSmallLdsInts) != hipSuccess)
-            return set_error(GNNHIP_EHIP, "csr_group: %zu bytes of LDS refused", sizeof(int) * kSmallLdsInts);
-        hipLaunchKernelGGL(csr_group_small_kernel, dim3(lay.groups), dim3(kSmallBlock), sizeof(int) * (size_t)(lay.bitmaps + lay.words * lay.nbitmaps), s,
-                           rows, (int)n, lay, key, key_stride, payload, payload_stride, val_in, average, row_ptr, col_idx, val);
-        GNNHIP_LAUNCH_CHECK("csr_group_small");
-        return GNNHIP_OK;
-    }
+    if (csr_group_small(rows, n, key, key_stride, payload, payload_stride, val_in, average, row_ptr, col_idx, val, nullptr, nullptr, nullptr, s))
+        return last_launch_status("csr_group_small");
     const int ntiles = (int)((n + kTile - 1) / kTile);
     const long long nhist = (long long)kDigits * (ntiles > 0 ? ntiles : 1);
     size_t off = 0;
@@ -643,6 +677,21 @@ int gnnhip_csr_group_i32(int rows, int n, const int* key, int key_stride, const 
     GNNHIP_REQUIRE(n == 0 || rows >= 1, "pairs but no rows in csr_group");
     if (int rc = require_ready()) return rc;
     return csr_group_pairs(rows, n, key, key_stride, payload, payload_stride, nullptr, average, row_ptr, col_idx, val, as_stream(stream));
+}
+
+int gnnhip_csr_group_both_i32(int rows, int n, const int* x, int x_stride, const int* y, int y_stride,
+                              int* row_ptr, int* col_idx, float* val, int* t_row_ptr, int* t_col_idx, float* t_val, void* stream)
+{
+    GNNHIP_REQUIRE(rows >= 0 && n >= 0 && x_stride >= 1 && y_stride >= 1, "bad shape in csr_group_both (rows=%d n=%d)", rows, n);
+    GNNHIP_REQUIRE(row_ptr && t_row_ptr, "null row pointers in csr_group_both");
+    GNNHIP_REQUIRE(n == 0 || (x && y && col_idx && val && t_col_idx && t_val), "null array in csr_group_both");
+    GNNHIP_REQUIRE(n == 0 || rows >= 1, "pairs but no rows in csr_group_both");
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    if (csr_group_small(rows, n, y, y_stride, x, x_stride, nullptr, 0, row_ptr, col_idx, val, t_row_ptr, t_col_idx, t_val, s))
+        return last_launch_status("csr_group_small");
+    if (int rc = csr_group_pairs(rows, n, y, y_stride, x, x_stride, nullptr, 0, row_ptr, col_idx, val, s)) return rc;
+    return csr_group_pairs(rows, n, x, x_stride, y, y_stride, nullptr, 0, t_row_ptr, t_col_idx, t_val, s);
 }
 
 int gnnhip_csr_transpose_f32(int m, int k, int nnz, const int* row_ptr, const int* col_idx, const float* val,

@@ -60,7 +60,7 @@ public:
         auto* gv = dynamic_cast<GraphVar*>(operands[0].get());
         ASSERT(gv && gv->graph, "message passing needs a bound GraphVar");
         auto& out = detail::sparse_var<mode, Dtype>(outputs[0], "IMsgPass").value;
-        if (BuildOnDevice(gv->graph, out)) return;
+        if (BuildOnDevice(gv->graph, out, phase)) return;
         InitCPUWeight(gv->graph);
         out.CopyFrom(cpu_weight);          // host -> device (or host -> host) copy of the three CSR arrays
         // training multiplies by the transpose in the backward pass: the matrix is on the host right now,
@@ -76,7 +76,7 @@ protected:
     virtual void InitCPUWeight(GraphStruct* graph) = 0;
     // Operands that are a grouping of the flat edge list can be built on the device from one copy
     // of that list; returns false where the host construction is to be used.
-    virtual bool BuildOnDevice(GraphStruct*, SpTensor<mode, Dtype>&) { return false; }
+    virtual bool BuildOnDevice(GraphStruct*, SpTensor<mode, Dtype>&, Phase) { return false; }
     virtual bool TransposeForBackward() const { return false; }
     SpTensor<CPU, Dtype> cpu_weight, cpu_transpose;
     std::vector<int> cursor;
@@ -103,8 +103,10 @@ inline void fill_row_weights(const int* row_ptr, int rows, bool average, Dtype* 
 // CSR [num_rows, num_cols] on the device whose row y lists, in edge order, the tail x (payload_is_edge
 // false) or the index (true) of every edge x -> y: one copy of the (x, y) pairs, then a stable
 // grouping by y (gnnhip_csr_group_i32).
+// with_transpose (node-to-node operand of a training pass, unit values): the same call groups the pairs by x
+// as well and the result becomes the cached transpose of `out`.
 inline void group_edges_on_device(GraphStruct* graph, bool payload_is_edge, bool average, size_t num_cols,
-                                  SpTensor<GPU, float>& out, DTensor<GPU, int>& staging)
+                                  SpTensor<GPU, float>& out, DTensor<GPU, int>& staging, bool with_transpose = false)
 {
     static_assert(sizeof(std::pair<int, int>) == 2 * sizeof(int), "edge list is not a flat (x, y) array");
     const int E = (int)graph->num_edges, N = (int)graph->num_nodes;
@@ -122,6 +124,12 @@ inline void group_edges_on_device(GraphStruct* graph, bool payload_is_edge, bool
         if (E > 0) GNN_HIP(gnnhip_memcpy_h2d(pairs + 2 * (size_t)E, idx.data->ptr, sizeof(int) * (size_t)E, GpuHandle::Stream()));
         payload = pairs + 2 * (size_t)E;
         payload_stride = 1;
+    }
+    if (with_transpose && !payload_is_edge && !average && num_cols == (size_t)N) {
+        auto& t = out.AdoptTransposed();
+        GNN_HIP(gnnhip_csr_group_both_i32(N, E, pairs, 2, pairs + 1, 2, out.data->row_ptr, out.data->col_idx, out.data->val,
+                                          t.row_ptr, t.col_idx, t.val, GpuHandle::Stream()));
+        return;
     }
     GNN_HIP(gnnhip_csr_group_i32(N, E, pairs + 1, 2, payload, payload_stride, average ? 1 : 0,
                                  out.data->row_ptr, out.data->col_idx, out.data->val, GpuHandle::Stream()));
@@ -149,13 +157,13 @@ inline bool device_grouping_pays(size_t pairs, size_t rows)
     return pairs >= kRadixGroupingPairs || rows / 4 + 47 * pairs / 20 + 1024 <= 160 * 1024;
 }
 template<typename Dtype, typename SpT>
-inline bool group_edges_if_gpu(GraphStruct*, bool, bool, size_t, SpT&, DTensor<GPU, int>&) { return false; }
+inline bool group_edges_if_gpu(GraphStruct*, bool, bool, size_t, SpT&, DTensor<GPU, int>&, bool = false) { return false; }
 template<>
 inline bool group_edges_if_gpu<float, SpTensor<GPU, float> >(GraphStruct* graph, bool payload_is_edge, bool average, size_t num_cols,
-                                                             SpTensor<GPU, float>& out, DTensor<GPU, int>& staging)
+                                                             SpTensor<GPU, float>& out, DTensor<GPU, int>& staging, bool with_transpose)
 {
     if (!device_grouping_pays(graph->num_edges, graph->num_nodes)) return false;
-    group_edges_on_device(graph, payload_is_edge, average, num_cols, out, staging);
+    group_edges_on_device(graph, payload_is_edge, average, num_cols, out, staging, with_transpose);
     return true;
 }
 template<typename Dtype, typename SpT>
@@ -185,9 +193,10 @@ public:
 
 protected:
     virtual bool TransposeForBackward() const override { return true; }
-    virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out) override
+    virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out, Phase phase) override
     {
-        if (!detail::group_edges_if_gpu<Dtype>(graph, false, this->average, graph->num_nodes, out, edge_staging)) return false;
+        if (!detail::group_edges_if_gpu<Dtype>(graph, false, this->average, graph->num_nodes, out, edge_staging, phase == Phase::TRAIN))
+            return false;
         this->layout.block_diagonal = graph->num_nodes <= detail::kExamineBlocksMaxNodes && NoEdgeBetweenSubgraphs(graph);
         return true;
     }
@@ -229,7 +238,7 @@ public:
     Edge2NodeMsgPass(std::string _name, bool _average = false) : IMsgPass<mode, Dtype>(_name, _average) {}
 
 protected:
-    virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out) override
+    virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out, Phase phase) override
     {
         return detail::group_edges_if_gpu<Dtype>(graph, true, this->average, graph->num_edges, out, edge_staging);
     }
@@ -321,7 +330,7 @@ public:
 protected:
     // Nodes added subgraph after subgraph, each with the next index (GetBatch does): the matrix is then the
     // identity layout, its facts are known from one pass over the records, and the device groups it.
-    virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out) override
+    virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out, Phase phase) override
     {
         const int M = (int)graph->node_list.size();
         if (M != (int)graph->num_nodes) return false;

@@ -47,6 +47,18 @@ public:
         }
         return *t_data;
     }
+    // Storage for a transpose that the builder of the matrix fills on the device in the same launch; what it
+    // writes there counts as the transpose from now on (any order of the entries inside a row will do: the
+    // products with it sum a row in the order it is stored, the same on every run).
+    SparseData<GPU, Dtype>& AdoptTransposed()
+    {
+        if (!t_data) t_data = std::make_shared< SparseData<GPU, Dtype> >();
+        t_data->Reserve(data->nnz, (int)shape[1] + 1);
+        t_data->nnz = data->nnz;
+        t_data->len_ptr = (int)shape[1] + 1;
+        t_valid = true;
+        return *t_data;
+    }
     // The transpose handed over by a builder that had the matrix on the host anyway (three small copies instead
     // of the dozen launches of the device transposition); t must be the stable transpose of what this tensor
     // holds: row c of t lists the rows of the matrix that have an entry in column c, in ascending row order.

@@ -512,6 +512,21 @@ def csr_group(rows, key, payload, average=False, key_stride=1, payload_stride=1,
     return row_ptr, col_idx, val
 
 
+def csr_group_both(rows, x, y, x_stride=1, y_stride=1, n=None):
+    """the pairs (x, y) grouped by y (row i lists x) and by x (row i lists y): a matrix and its transpose, values 1"""
+    if n is None:
+        n = x.numel() // x_stride
+    dev = x.device
+    out = []
+    for _ in range(2):
+        out += [torch.empty(rows + 1, dtype=torch.int32, device=dev), torch.empty(n, dtype=torch.int32, device=dev),
+                torch.empty(n, dtype=torch.float32, device=dev)]
+    check(_lib().gnnhip_csr_group_both_i32(rows, n, _i32(x, "x"), x_stride, _i32(y, "y"), y_stride,
+                                           _i32(out[0], "row_ptr"), _i32(out[1], "col_idx"), _f32(out[2], "val"),
+                                           _i32(out[3], "t_row_ptr"), _i32(out[4], "t_col_idx"), _f32(out[5], "t_val"), _stream()))
+    return tuple(out[:3]), tuple(out[3:])
+
+
 def csr_transpose(row_ptr, col_idx, val, m, k):
     nnz = col_idx.numel()
     dev = row_ptr.device

@@ -105,6 +105,15 @@ int gnnhip_spmm_csr_f32(int m, int k, int n, int nnz, float alpha, const int* ro
 int gnnhip_csr_group_i32(int rows, int n, const int* key, int key_stride, const int* payload, int payload_stride,
                          int average, int* row_ptr, int* col_idx, float* val, void* stream);
 
+/* ---- the n pairs (x, y) grouped both ways at once, values 1: row i of (row_ptr, col_idx, val) lists the x of the
+ *      pairs with y = i, which is gnnhip_csr_group_i32(rows, n, y, .., x, .., 0, ..), the operand of
+ *      Node2NodeMsgPass (src/nn/msg_pass.cpp:46-67); row i of (t_row_ptr, t_col_idx, t_val) lists the y of the
+ *      pairs with x = i: its transpose, which the reference leaves to cuSPARSE csrmm with Trans::T in the backward
+ *      pass (src/tensor/gpu_dense_tensor.cu:271-296).  Both [rows, rows], entries in pair order; one launch where
+ *      the one-launch grouping fits, two groupings otherwise. */
+int gnnhip_csr_group_both_i32(int rows, int n, const int* x, int x_stride, const int* y, int y_stride,
+                              int* row_ptr, int* col_idx, float* val, int* t_row_ptr, int* t_col_idx, float* t_val, void* stream);
+
 /* ---- CSR of the transpose: A [m,k] with nnz entries -> A^T [k,m]; entries of a row of A^T keep the
  *      order of the rows of A they came from.  The reference transposes implicitly inside cuSPARSE
  *      csrmm for MM(SpTensor, DTensor, Trans::T) (src/tensor/gpu_dense_tensor.cu:271-296). */

@@ -1715,6 +1715,31 @@ def test_device_csr_group_of_a_small_batch_in_one_launch(gpu, case):
     assert np.array_equal(_n(rp), want[0]) and np.array_equal(_n(ci), want[1])
 
 
+@pytest.mark.parametrize("rows,n", [(7450, 16382), (300, 40_000), (50_000, 70_000), (9, 1), (5, 0)])
+def test_device_csr_group_both_ways(gpu, rows, n):
+    """an edge list grouped by head and by tail at once (a matrix and its transpose, entries in edge order): the one-launch
+    grouping with two jobs, the radix route past it; both equal the stable sorts, and the two are transposes of each other"""
+    import scipy.sparse as sp
+    from graphnn_amd import ops
+    rng = np.random.default_rng(rows + n)
+    x = rng.integers(0, rows, n).astype(np.int32); y = rng.integers(0, rows, n).astype(np.int32)
+    if n > 1000:
+        y[100:700] = 3                                            # a long row on one side, short ones on the other
+    pairs = _t(np.stack([x, y], axis=1).reshape(-1), gpu)
+    if n:
+        a, at = ops.csr_group_both(rows, pairs, pairs[1:], 2, 2, n=n)
+    else:
+        empty = _t(np.zeros(0, np.int32), gpu)
+        a, at = ops.csr_group_both(rows, empty, empty)
+    for got, want in ((a, _stable_group(rows, y, x)), (at, _stable_group(rows, x, y))):
+        for g, w in zip(got, want):
+            assert np.array_equal(_n(g), w)
+    if n:
+        A = sp.csr_matrix((_n(a[2]), _n(a[1]), _n(a[0])), shape=(rows, rows))
+        AT = sp.csr_matrix((_n(at[2]), _n(at[1]), _n(at[0])), shape=(rows, rows))
+        assert (A.T != AT).nnz == 0
+
+
 @pytest.mark.parametrize("m,k,nnz", [(411, 233, 3000), (5000, 7000, 120_000), (3, 70_000, 32_768), (1, 1, 1), (900, 20_000, 65_536),
                                      (32_768, 32_768, 65_537)])
 def test_device_csr_transpose(gpu, oracle, m, k, nnz):
