@@ -1154,6 +1154,41 @@ def test_packed_batch_refuses_a_graph_larger_than_a_bin(gpu, oracle):
     assert np.array_equal(_n(bufs.pred)[keep], want["pred"][keep])
 
 
+@pytest.mark.parametrize("B", [40, 300, 600, 1100])
+def test_batched_forward_with_graphs_of_no_nodes(gpu, oracle, B):
+    """graphs without nodes between the others (rows of S without entries; GetBatch never makes them, the operand
+    allows them): pooled features of zero and the logits of a zero vector, through every way the one-launch forward
+    hands out its graphs (in batch order, largest first, packed into bins), the first and the last graph among them"""
+    from graphnn_amd import ops
+    K, C, H, Q, L = 9, 32, 16, 3, 2
+    rng = np.random.default_rng(50 + B)
+    sizes = rng.integers(1, 31, B)
+    sizes[rng.random(B) < 0.2] = 0
+    sizes[[0, B - 1, B // 2, B // 2 + 1]] = 0
+    off = np.concatenate([[0], np.cumsum(sizes)])
+    ex, ey = [], []
+    for g, n in enumerate(sizes):
+        if n < 2:
+            continue
+        i = np.arange(n - 1) + off[g]
+        ex += [i, i + 1]; ey += [i + 1, i]
+    ex = np.concatenate(ex).astype(np.int32); ey = np.concatenate(ey).astype(np.int32)
+    N = int(off[-1])
+    a = batching.node2node_csr(N, ex, ey)
+    s = (off.astype(np.int32), np.arange(N, dtype=np.int32), np.ones(N, np.float32))
+    X = rng.standard_normal((N, K)).astype(np.float32)
+    w = synth.make_weights(synth.Stream(78), K, C, H, Q)
+    wts = (_t(w.W_n2l, gpu), _t(w.W_conv, gpu), _t(w.W_h1, gpu), _t(w.W_h2, gpu))
+    bufs = ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), *wts, L, 32)
+    assert int(_n(bufs.status)[0]) == 0
+    want = _forward_want(oracle, a, s, X, w, L)
+    keys = ("msg", "h_final", "pool", "hidden", "logits", "probs")
+    _assert_forward_parity({k: _n(getattr(bufs, k)) for k in keys}, want, L)
+    none = sizes == 0
+    assert np.all(_n(bufs.pool)[none] == 0) and np.all(_n(bufs.logits)[none] == 0)
+    assert np.array_equal(_n(bufs.pred)[none], want["pred"][none])
+
+
 @pytest.mark.parametrize("C,L,B", [(64, 4, 256), (16, 1, 37), (32, 3, 300), (64, 0, 9)])
 def test_batched_forward_keeps_every_level_for_training(gpu, oracle, C, L, B):
     """the one-launch forward of a training iteration: h_0 .. h_L as the per-level entry points give them (which
