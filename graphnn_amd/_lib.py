@@ -76,6 +76,7 @@ SIGNATURES = {
     "gnnhip_s2v_level_backward_f32": [_I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_s2v_grad_gate_f32": [_Z, _P, _P, _P, _P, _I, _P],
     "gnnhip_momentum_sgd_batch_f32": [_I, _P, _P, _P, _P, _F, _F, _F, _P],
+    "gnnhip_adam_batch_f32": [_I, _P, _P, _P, _P, _P, _F, _F, _F, _F, _F, _F, _F, _F, _P],
     "gnnhip_last_error": [],
     "gnnhip_version": [],
 }

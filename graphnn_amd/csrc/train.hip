@@ -187,6 +187,84 @@ __global__ __launch_bounds__(kBlock) void momentum_sgd_batch_kernel(UpdateBatch 
     }
 }
 
+// ------------------------------------------------------------------ Adam
+// Sum of squares of every gradient tensor, for the clipping factor: workgroup (x, y) adds its stride of tensor y in
+// double and leaves one partial; the update kernel adds the partials in index order.
+__global__ __launch_bounds__(kBlock) void sumsq_batch_kernel(UpdateBatch b, double* __restrict__ partial)
+{
+    __shared__ double sh[kWavesPerBlock];
+    const float* __restrict__ g = b.g[blockIdx.y];
+    const size_t n = b.n[blockIdx.y];
+    double acc = 0.0;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) acc += (double)g[i] * (double)g[i];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int d = kWave / 2; d >= 1; d >>= 1) acc += __shfl_xor(acc, d, kWave);
+    if (lane == 0) sh[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0.0;
+        for (int w = 0; w < kWavesPerBlock; ++w) t += sh[w];
+        partial[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = t;
+    }
+}
+
+struct AdamBatch {
+    float* w[kUpdateBatch];
+    float* g[kUpdateBatch];
+    float* m[kUpdateBatch];
+    float* v[kUpdateBatch];
+    size_t n[kUpdateBatch];
+};
+
+// AdamOptimizer::Update (src/nn/optimizer.cpp:105-160), tensor blockIdx.y, every step rounded as the reference's
+// sequence of tensor operations rounds it (Axpby = scale, then one fused multiply-add):
+//   g = l2 w + scale g ;  m = (1 - b1) g + b1 m ;  v = (1 - b2) g^2 + b2 v
+//   w = -(lr s1) m / (sqrt(v s2) + eps) + w ;  g = 0
+// scale = clip / norm when the norm of all gradients (nparts partial sums of squares) exceeds clip > 0, else 1.
+__global__ __launch_bounds__(kBlock) void adam_batch_kernel(AdamBatch b, const double* __restrict__ partial, int nparts, float clip,
+                                                            float lr_s1, float l2, float one_minus_b1, float b1, float one_minus_b2, float b2,
+                                                            float eps, float s2)
+{
+    __shared__ double sh[kWavesPerBlock];
+    __shared__ float sh_scale;
+    float scale = 1.0f;
+    if (nparts > 0) {
+        double acc = 0.0;
+        for (int i = threadIdx.x; i < nparts; i += kBlock) acc += partial[i];
+        const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+        for (int d = kWave / 2; d >= 1; d >>= 1) acc += __shfl_xor(acc, d, kWave);
+        if (lane == 0) sh[wave] = acc;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            double t = 0.0;
+            for (int w = 0; w < kWavesPerBlock; ++w) t += sh[w];
+            const float norm = (float)sqrt(t);
+            sh_scale = norm > clip ? clip / norm : 1.0f;
+        }
+        __syncthreads();
+        scale = sh_scale;
+    }
+    const int t = blockIdx.y;
+    float* __restrict__ w = b.w[t];
+    float* __restrict__ g = b.g[t];
+    float* __restrict__ m = b.m[t];
+    float* __restrict__ v = b.v[t];
+    const size_t n = b.n[t];
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const float wi = w[i];
+        const float gi = __fmaf_rn(l2, wi, __fmul_rn(scale, g[i]));
+        const float mi = __fmaf_rn(one_minus_b1, gi, __fmul_rn(b1, m[i]));
+        const float vi = __fmaf_rn(one_minus_b2, __fmul_rn(gi, gi), __fmul_rn(b2, v[i]));
+        m[i] = mi;
+        v[i] = vi;
+        const float step = __fmul_rn(__fdiv_rn(1.0f, __fadd_rn(__fsqrt_rn(__fmul_rn(vi, s2)), eps)), mi);
+        w[i] = __fmaf_rn(-lr_s1, step, wi);
+        g[i] = 0.f;
+    }
+}
+
 inline unsigned ew_grid(size_t n)
 {
     size_t b = (n + kBlock - 1) / kBlock;
@@ -276,6 +354,63 @@ int gnnhip_momentum_sgd_batch_f32(int n, float* const* w, float* const* g, float
         if (gx > 1024u) gx = 1024u;
         hipLaunchKernelGGL(momentum_sgd_batch_kernel, dim3(gx, (unsigned)m), dim3(kBlock), 0, as_stream(stream), b, lr, momentum, l2);
         GNNHIP_LAUNCH_CHECK("momentum_sgd_batch");
+    }
+    return GNNHIP_OK;
+}
+
+int gnnhip_adam_batch_f32(int n, float* const* w, float* const* g, float* const* m, float* const* v, const size_t* count,
+                          float lr, float l2, float clip_threshold, float beta1, float beta2, float eps, float s1, float s2, void* stream)
+{
+    GNNHIP_REQUIRE(n >= 0 && (n == 0 || (w && g && m && v && count)), "bad arguments in adam_batch");
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    constexpr unsigned kNormGrid = 64;
+    // the norm of ALL gradients comes first: one launch of partial sums per 16 tensors
+    int tensors = 0;
+    for (int i = 0; i < n; ++i) {
+        if (count[i] == 0) continue;
+        GNNHIP_REQUIRE(w[i] && g[i] && m[i] && v[i], "null tensor in adam_batch");
+        ++tensors;
+    }
+    if (tensors == 0) return GNNHIP_OK;
+    double* partial = nullptr;
+    int nparts = 0;
+    if (clip_threshold > 0.f) {
+        void* q = nullptr;
+        if (int rc = stream_scratch(s, sizeof(double) * (size_t)tensors * kNormGrid, &q)) return rc;
+        partial = static_cast<double*>(q);
+        int i = 0;
+        while (i < n) {
+            UpdateBatch b;
+            int k = 0;
+            for (; i < n && k < kUpdateBatch; ++i) {
+                if (count[i] == 0) continue;
+                b.w[k] = nullptr; b.v[k] = nullptr; b.g[k] = g[i]; b.n[k] = count[i];
+                ++k;
+            }
+            if (k == 0) break;
+            hipLaunchKernelGGL(sumsq_batch_kernel, dim3(kNormGrid, (unsigned)k), dim3(kBlock), 0, s, b, partial + nparts);
+            nparts += k * (int)kNormGrid;
+        }
+        GNNHIP_LAUNCH_CHECK("sumsq_batch");
+    }
+    int i = 0;
+    while (i < n) {
+        AdamBatch b;
+        int k = 0;
+        size_t largest = 0;
+        for (; i < n && k < kUpdateBatch; ++i) {
+            if (count[i] == 0) continue;
+            b.w[k] = w[i]; b.g[k] = g[i]; b.m[k] = m[i]; b.v[k] = v[i]; b.n[k] = count[i];
+            if (count[i] > largest) largest = count[i];
+            ++k;
+        }
+        if (k == 0) break;
+        unsigned gx = ew_grid(largest);
+        if (gx > 1024u) gx = 1024u;
+        hipLaunchKernelGGL(adam_batch_kernel, dim3(gx, (unsigned)k), dim3(kBlock), 0, s, b, partial, nparts, clip_threshold,
+                           lr * s1, l2, 1 - beta1, beta1, 1 - beta2, beta2, eps, s2);
+        GNNHIP_LAUNCH_CHECK("adam_batch");
     }
     return GNNHIP_OK;
 }

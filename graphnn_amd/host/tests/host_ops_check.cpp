@@ -146,6 +146,11 @@ int main(int argc, char** argv)
         auto g = p->grad.Full();
         append(out, g);
     }
+    // one Adam update from those gradients (threshold 0.5: the clipping factor is in play), then the parameters
+    AdamOptimizer<mode, Dtype> adam(&model, 0.01f, 0.001f);
+    adam.clip_threshold = 0.5f;
+    adam.Update();
+    for (auto& p : {w_n2l, fc, w_score}) append(out, p->value);
     FILE* f = fopen((dir + "/out.bin").c_str(), "wb");
     ASSERT(f, "cannot write out.bin");
     fwrite(out.data(), sizeof(float), out.size(), f);

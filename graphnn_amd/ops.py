@@ -5,6 +5,7 @@ Every helper validates dtype / device / contiguity on the host before a pointer
 reaches a kernel, and raises GnnHipError on a non-zero status.
 """
 import ctypes
+import numpy as np
 
 import torch
 
@@ -599,6 +600,20 @@ def momentum_sgd_batch(ws, gs, vs, lr, momentum, l2):
         _f32(t, "tensor")
     cnt = Z(*[t.numel() for t in ws])
     check(_lib().gnnhip_momentum_sgd_batch_f32(n, wp, gp, vp, cnt, float(lr), float(momentum), float(l2), _stream()))
+
+
+def adam_batch(ws, gs, ms, vs, lr, l2, clip_threshold, beta1, beta2, eps, t):
+    """one AdamOptimizer::Update over the tensors, t = the iteration count after the increment (1 for the first)"""
+    n = len(ws)
+    P = ctypes.c_void_p * n
+    Z = ctypes.c_size_t * n
+    for x in list(ws) + list(gs) + list(ms) + list(vs):
+        _f32(x, "tensor")
+    ptr = lambda ts: P(*[x.data_ptr() for x in ts])
+    s1 = np.float32(1.0 / (1 - float(np.float32(beta1)) ** t))
+    s2 = np.float32(1.0 / (1 - float(np.float32(beta2)) ** t))
+    check(_lib().gnnhip_adam_batch_f32(n, ptr(ws), ptr(gs), ptr(ms), ptr(vs), Z(*[x.numel() for x in ws]), float(lr), float(l2),
+                                       float(clip_threshold), float(beta1), float(beta2), float(eps), float(s1), float(s2), _stream()))
 
 
 def upload_sparse32(host_array, out=None):

@@ -385,6 +385,16 @@ int gnnhip_s2v_level_backward_f32(int N, int C, int nnz, const int* t_row_ptr, c
 int gnnhip_momentum_sgd_batch_f32(int n, float* const* w, float* const* g, float* const* v, const size_t* count,
                                   float lr, float momentum, float l2, void* stream);
 
+/* ---- AdamOptimizer::Update over n tensors (src/nn/optimizer.cpp:105-160), with the clipping factor of
+ *      IOptimizer::ClipGradients (src/nn/optimizer.cpp:16-32) formed on the device:
+ *      scale = clip_threshold / |all g| when that norm exceeds clip_threshold > 0, else 1 (clip_threshold <= 0: no clipping)
+ *      g = l2 w + scale g ; m = (1 - beta1) g + beta1 m ; v = (1 - beta2) g^2 + beta2 v
+ *      w -= lr s1 m / (sqrt(v s2) + eps) ; g = 0          s1 = 1 / (1 - beta1^t), s2 = 1 / (1 - beta2^t), formed by the caller
+ *      m, v: the optimizer's first_moments / second_moments.  w, g, m, v: host arrays of n device pointers;
+ *      count: host array of element counts. */
+int gnnhip_adam_batch_f32(int n, float* const* w, float* const* g, float* const* m, float* const* v, const size_t* count,
+                          float lr, float l2, float clip_threshold, float beta1, float beta2, float eps, float s1, float s2, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -357,6 +357,45 @@ void orc_momentum_sgd(size_t n, float* w, float* g, float* v, float lr, float mo
     for (size_t i = 0; i < n; ++i) g[i] = 0.0f;
 }
 
+/* IOptimizer::ClipGradients over the tensors of a parameter set (src/nn/optimizer.cpp:16-32): norm = sqrt of the
+ * sum of the squared 2-norms (each Norm2 a float), factor = threshold / norm when the norm exceeds it, else 1. */
+float orc_clip_factor(int tensors, const float* const* g, const size_t* n, float threshold)
+{
+    float norm = 0.0f;
+    for (int t = 0; t < tensors; ++t) {
+        double sq = 0.0;
+        for (size_t i = 0; i < n[t]; ++i) sq += (double)g[t][i] * (double)g[t][i];
+        const float norm2 = (float)sqrt(sq);
+        norm += norm2 * norm2;
+    }
+    norm = sqrtf(norm);
+    return norm > threshold ? threshold / norm : 1.0f;
+}
+
+/* One AdamOptimizer::Update on one tensor (src/nn/optimizer.cpp:105-160) as the calls it makes, gscale being
+ * what ClipGradients returned and t the iteration count after the increment:
+ * grad.RowSparseAxpby(l2, value, gscale); m.RowSparseAxpby(1 - b1, grad, b1); grad.Square();
+ * v.RowSparseAxpby(1 - b2, grad, b2); v_hat = v; Scale(s2); Sqrt; Add(eps); Inv; ElewiseMul(m);
+ * value.RowSparseAxpby(-lr * s1, v_hat, 1.0); grad.RowSpZeros()        s1 = 1 / (1 - b1^t), s2 = 1 / (1 - b2^t) */
+void orc_adam(size_t n, float* w, float* g, float* m, float* v, float lr, float l2, float gscale, float b1, float b2, float eps, int t)
+{
+    const float s1 = (float)(1.0 / (1 - pow(b1, t)));
+    const float s2 = (float)(1.0 / (1 - pow(b2, t)));
+    orc_axpby(n, l2, w, gscale, g);
+    orc_axpby(n, 1 - b1, g, b1, m);
+    for (size_t i = 0; i < n; ++i) g[i] = g[i] * g[i];
+    orc_axpby(n, 1 - b2, g, b2, v);
+    for (size_t i = 0; i < n; ++i) {
+        float h = v[i] * s2;
+        h = sqrtf(h);
+        h = h + eps;
+        h = 1.0f / h;
+        g[i] = h * m[i];                       /* v_hat, kept in the gradient's storage */
+    }
+    orc_axpby(n, -lr * s1, g, 1.0f, w);
+    for (size_t i = 0; i < n; ++i) g[i] = 0.0f;
+}
+
 /* Global sum / mean: sequential fp32 accumulation, mean = s / cnt
  * (src/tensor/cpu_dense_tensor.cpp:269-295). */
 float orc_sum(const float* x, size_t n)

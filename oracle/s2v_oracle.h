@@ -41,6 +41,8 @@ void orc_unary(int op, float* x, size_t n, float a0, float a1);
 void orc_row_softmax(float* x, int rows, int cols);
 void orc_jagged_softmax(float* x, const int* lens, int nseg);
 void orc_momentum_sgd(size_t n, float* w, float* g, float* v, float lr, float momentum, float l2);
+float orc_clip_factor(int tensors, const float* const* g, const size_t* n, float threshold);
+void orc_adam(size_t n, float* w, float* g, float* m, float* v, float lr, float l2, float gscale, float b1, float b2, float eps, int t);
 void orc_jagged_softmax_deriv(float* dst, const float* out, const float* grad, const int* lens, int nseg);
 float orc_sum(const float* x, size_t n);
 float orc_mean(const float* x, size_t n);

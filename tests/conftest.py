@@ -142,6 +142,20 @@ class Oracle:
                                   ctypes.c_float(momentum), ctypes.c_float(l2))
         return w, g, v
 
+    def clip_factor(self, grads, threshold):
+        gs = [np.ascontiguousarray(g, np.float32) for g in grads]
+        ptrs = (ctypes.c_void_p * len(gs))(*[g.ctypes.data for g in gs])
+        counts = (ctypes.c_size_t * len(gs))(*[g.size for g in gs])
+        self.lib.orc_clip_factor.restype = ctypes.c_float
+        return float(self.lib.orc_clip_factor(len(gs), ptrs, counts, ctypes.c_float(threshold)))
+
+    def adam(self, w, g, m, v, lr, l2, gscale, b1, b2, eps, t):
+        """one update of one tensor; returns the new (w, g, m, v)"""
+        w, g, m, v = (np.array(a, np.float32, copy=True) for a in (w, g, m, v))
+        self.lib.orc_adam(ctypes.c_size_t(w.size), _ptr(w), _ptr(g), _ptr(m), _ptr(v), ctypes.c_float(lr), ctypes.c_float(l2),
+                          ctypes.c_float(gscale), ctypes.c_float(b1), ctypes.c_float(b2), ctypes.c_float(eps), ctypes.c_int(t))
+        return w, g, m, v
+
     def sum(self, x):
         x = np.ascontiguousarray(x, np.float32)
         return float(self.lib.orc_sum(_ptr(x), ctypes.c_size_t(x.size)))

@@ -225,10 +225,21 @@ def test_host_api_bias_level_jagged_softmax_reduce(gpu, oracle, tmp_path):
     obj64 = (att64[:, None] * h64).sum()
     obj64.backward()
     assert abs(float(obj64) - obj) <= 1e-4 * abs(obj)
+    grads = {}
     for name, p64 in (("w_n2l", Wn), ("fc", Fc), ("w_score", Ws)):
         g64 = p64.grad.numpy()
         got = take(g64.size).reshape(g64.shape)
         assert max_rel(got, g64) < PARITY_TOL, name
+        grads[name] = got.copy()
+    # AdamOptimizer::Update from those gradients: the oracle's update of every tensor with the clipping factor of
+    # the whole set (threshold 0.5, l2 0.001, the reference's default rates)
+    scale = oracle.clip_factor(list(grads.values()), 0.5)
+    assert scale < 1.0
+    for name, w0 in (("w_n2l", w.W_n2l), ("fc", fc), ("w_score", w_score)):
+        zero = np.zeros(w0.size, np.float32)
+        want, _, _, _ = oracle.adam(w0.reshape(-1), grads[name].reshape(-1), zero, zero, 0.01, 0.001, scale, 0.9, 0.999, 1e-8, 1)
+        got = take(w0.size)
+        assert np.allclose(got, want, rtol=1e-6, atol=1e-6), name
     assert pos == out.size
 
 

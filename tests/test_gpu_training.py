@@ -163,6 +163,43 @@ def test_momentum_sgd_batch_two_steps(gpu, oracle, momentum):
                 assert np.allclose(_n(vd[i]), v[i], rtol=1e-6, atol=1e-7), (step, i)
 
 
+@pytest.mark.parametrize("clip,l2", [(5.0, 0.01), (0.0, 0.0), (1e6, 0.3)])
+def test_adam_batch_three_steps(gpu, oracle, clip, l2):
+    """AdamOptimizer::Update over a parameter set in two launches (the norm of all gradients, then the update with
+    the clipping factor formed on the device), three consecutive steps: gradients that are clipped (their norm is
+    far above 5), not clipped (threshold off or out of reach), 18 tensors (more than one table), one of them large"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(23)
+    shapes = [(38, 64), (64, 64), (64, 32), (32, 2), (1,), (300007,)] + [(5, 3)] * 12
+    lr, b1, b2, eps = 0.01, 0.9, 0.999, 1e-8
+    w = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+    m = [np.zeros(s, np.float32) for s in shapes]
+    v = [np.zeros(s, np.float32) for s in shapes]
+    wd, md, vd = [_t(a, gpu) for a in w], [_t(a, gpu) for a in m], [_t(a, gpu) for a in v]
+    for step in range(1, 4):
+        g = [(rng.standard_normal(s) * (0.02 if step == 3 else 1.0)).astype(np.float32) for s in shapes]
+        gd = [_t(a, gpu) for a in g]
+        ops.adam_batch(wd, gd, md, vd, lr, l2, clip, b1, b2, eps, step)
+        scale = oracle.clip_factor(g, clip) if clip > 0 else 1.0
+        if clip == 5.0:
+            assert (scale < 0.05) == (step < 3)
+        for i in range(len(shapes)):
+            # where weight decay and the scaled gradient cancel (l2 w = -scale g to four digits) the sum carries the
+            # last bits of the clipping factor, which the device forms in double: those elements are left out
+            parts = np.abs(l2 * w[i]) + np.abs(scale * g[i])
+            steady = np.abs(l2 * w[i] + scale * g[i]) > 1e-3 * parts
+            w[i], g0, m[i], v[i] = oracle.adam(w[i], g[i], m[i], v[i], lr, l2, scale, b1, b2, eps, step)
+            assert not _n(gd[i]).any()
+            assert steady.size < 1000 or steady.mean() > 0.99
+            # both sides round b m + (1 - b) g term by term, the device with one fused step: an ulp of the larger term
+            assert np.allclose(_n(md[i]), m[i], rtol=2e-6, atol=1e-6), (step, i)
+            assert np.allclose(_n(vd[i]), v[i], rtol=4e-6, atol=1e-6), (step, i)
+            assert np.allclose(_n(wd[i])[steady], w[i][steady], rtol=1e-6, atol=2e-7), (step, i)
+            assert np.allclose(_n(wd[i]), w[i], rtol=0, atol=2.1 * lr), (step, i)
+            # the device's own values go on, so that a left-out element does not carry into the next step
+            w[i], m[i], v[i] = _n(wd[i]).copy(), _n(md[i]).copy(), _n(vd[i]).copy()
+
+
 def _dense(csr, rows, cols):
     import scipy.sparse as sp
     return sp.csr_matrix((csr[2].astype(np.float64), csr[1], csr[0]), shape=(rows, cols)).toarray()

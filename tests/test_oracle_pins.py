@@ -381,6 +381,46 @@ def test_momentum_sgd_two_steps_closed_form(oracle):
     assert np.allclose(w_sgd, (1 - lr * l2) * W0 - lr * G1, rtol=1e-5, atol=1e-6) and not g_sgd.any()
 
 
+def test_adam_first_steps_closed_form(oracle):
+    """what the published algorithm fixes: after the first update from zero moments the bias-corrected moments are
+    g and g^2, so every weight moves by lr g / (|g| + eps), whatever the size of g; two updates against the
+    recurrence written out in float64; weight decay enters the gradient (a zero gradient still moves w by its
+    sign); clipping scales the gradient to the threshold norm before anything else (src/nn/optimizer.cpp:16-32,105-160)"""
+    rng = _rng(41)
+    lr, l2, b1, b2, eps = 0.01, 0.0, 0.9, 0.999, 1e-8
+    w0 = rng.standard_normal(500).astype(np.float32)
+    g1 = (rng.standard_normal(500) * np.logspace(-3, 3, 500)).astype(np.float32)
+    zero = np.zeros_like(w0)
+    w1, g, m1, v1 = oracle.adam(w0, g1, zero, zero, lr, l2, 1.0, b1, b2, eps, 1)
+    assert not g.any()
+    G1 = g1.astype(np.float64)
+    assert np.allclose(w1, w0 - lr * G1 / (np.abs(G1) + eps), rtol=1e-5, atol=1e-7)
+    # the decay rates as single precision holds them (1 - 0.999f is 1.0000467e-3)
+    B1, B2 = float(np.float32(b1)), float(np.float32(b2))
+    C1, C2 = float(np.float32(1) - np.float32(b1)), float(np.float32(1) - np.float32(b2))
+    assert np.allclose(m1, C1 * G1, rtol=1e-5) and np.allclose(v1, C2 * G1 * G1, rtol=1e-5)
+    # second update, with weight decay
+    l2 = 0.05
+    g2 = rng.standard_normal(500).astype(np.float32)
+    w2, _, m2, v2 = oracle.adam(w1, g2, m1, v1, lr, l2, 1.0, b1, b2, eps, 2)
+    W1, M1, V1 = (a.astype(np.float64) for a in (w1, m1, v1))
+    G2 = g2.astype(np.float64) + l2 * W1
+    M2 = B1 * M1 + C1 * G2
+    V2 = B2 * V1 + C2 * G2 * G2
+    W2 = W1 - lr / (1 - B1 ** 2) * M2 / (np.sqrt(V2 / (1 - B2 ** 2)) + eps)
+    assert np.allclose(m2, M2, rtol=1e-5, atol=1e-7) and np.allclose(v2, V2, rtol=1e-5, atol=1e-9)
+    assert np.allclose(w2, W2, rtol=1e-5, atol=1e-6)
+    # a zero gradient with weight decay: the first step is lr * sign(w)
+    w3, _, _, _ = oracle.adam(w0, zero, zero, zero, lr, 0.3, 1.0, b1, b2, eps, 1)
+    assert np.allclose(w3, w0 - lr * np.sign(w0), atol=1e-6)
+    # clipping: factor = threshold / global norm over all tensors, 1 below the threshold
+    ga, gb = rng.standard_normal(300).astype(np.float32), rng.standard_normal((20, 7)).astype(np.float32)
+    norm = np.sqrt((ga.astype(np.float64) ** 2).sum() + (gb.astype(np.float64) ** 2).sum())
+    assert abs(oracle.clip_factor([ga, gb], 5.0) - 5.0 / norm) <= 1e-6 and oracle.clip_factor([ga, gb], 1e3) == 1.0
+    w4, _, m4, _ = oracle.adam(w0[:300], ga, zero[:300], zero[:300], lr, 0.0, 0.25, b1, b2, eps, 1)
+    assert np.allclose(m4, C1 * 0.25 * ga.astype(np.float64), rtol=1e-5)
+
+
 def test_reductions(oracle):
     ints = np.arange(1, 1001, dtype=np.float32)
     assert oracle.sum(ints) == 500500.0 and oracle.mean(ints) == 500.5 and oracle.max(ints) == 1000.0
