@@ -60,6 +60,7 @@ SIGNATURES = {
     "gnnhip_jagged_softmax_f32": [_P, _P, _I, _P],
     "gnnhip_jagged_softmax_static_f32": [_P, _P, _I, _P],
     "gnnhip_jagged_softmax_deriv_f32": [_P, _P, _P, _P, _I, _P],
+    "gnnhip_row_softmax_deriv_f32": [_P, _P, _P, _I, _I, _P],
     "gnnhip_reduce_f32": [_I, _P, _Z, _P, _P],
     "gnnhip_row_argmax_f32": [_P, _I, _I, _P, _P],
     "gnnhip_csr_row_argmax_f32": [_P, _P, _P, _I, _P, _P],

@@ -166,6 +166,22 @@ __global__ __launch_bounds__(kBlock) void jagged_softmax_deriv_kernel(float* __r
     }
 }
 
+// ---- gradient of the row softmax: per row z = <grad, out>, dst += (grad - z) * out
+//      (SoftmaxDeriv, src/nn/softmax.cpp:8-29; on the GPU cunn_SoftMax_updateGradInput_kernel, src/nn/softmax.cu:10-59)
+__global__ __launch_bounds__(kBlock) void row_softmax_deriv_kernel(float* __restrict__ dst, const float* __restrict__ out,
+                                                                   const float* __restrict__ grad, int rows, int cols)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    for (long long r = (long long)blockIdx.x * kWavesPerBlock + wave; r < rows; r += (long long)gridDim.x * kWavesPerBlock) {
+        const size_t a = (size_t)r * cols;
+        float z = 0.f;
+        for (int j = lane; j < cols; j += kWave) z += grad[a + j] * out[a + j];
+        z = wave_sum(z);
+        for (int j = lane; j < cols; j += kWave) dst[a + j] += (grad[a + j] - z) * out[a + j];
+    }
+}
+
 // ---- global reductions: stage 1 writes one partial per workgroup, stage 2 combines
 // them in index order, so the result does not depend on scheduling.
 template <bool IS_MAX>
@@ -371,6 +387,17 @@ int gnnhip_jagged_softmax_deriv_f32(float* dst, const float* out, const float* g
     hipLaunchKernelGGL(jagged_softmax_deriv_kernel, dim3(wave_rows_grid(nseg)), dim3(kBlock), 0, s, dst, out, grad,
                        static_cast<const int*>(off), nseg);
     GNNHIP_LAUNCH_CHECK("jagged_softmax_deriv");
+    return GNNHIP_OK;
+}
+
+int gnnhip_row_softmax_deriv_f32(float* dst, const float* out, const float* grad, int rows, int cols, void* stream)
+{
+    GNNHIP_REQUIRE(rows >= 0 && cols >= 0, "negative shape in row_softmax_deriv");
+    if (rows == 0 || cols == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(dst && out && grad, "null tensor in row_softmax_deriv");
+    if (int rc = require_ready()) return rc;
+    hipLaunchKernelGGL(row_softmax_deriv_kernel, dim3(wave_rows_grid(rows)), dim3(kBlock), 0, as_stream(stream), dst, out, grad, rows, cols);
+    GNNHIP_LAUNCH_CHECK("row_softmax_deriv");
     return GNNHIP_OK;
 }
 

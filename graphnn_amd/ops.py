@@ -93,6 +93,13 @@ def gemm(A, B, transA=False, transB=False, alpha=1.0, beta=0.0, out=None):
     return out
 
 
+def row_softmax_deriv(dst, out, grad):
+    """dst += out * (grad - <grad, out> per row), in place on dst"""
+    rows, cols = out.shape
+    check(_lib().gnnhip_row_softmax_deriv_f32(_f32(dst, "dst"), _f32(out, "out"), _f32(grad, "grad"), rows, cols, _stream()))
+    return dst
+
+
 def gemm_tn_batch(products, alpha=1.0, beta=0.0):
     """products: list of (A [k,m], B [k,n], out [m,n]); out = alpha * A^T B + beta * out for all of them in two launches"""
     import ctypes

@@ -324,6 +324,11 @@ int gnnhip_relu_deriv_f32(size_t n, const float* out, const float* grad, float* 
 int gnnhip_jagged_softmax_deriv_f32(float* dst, const float* out, const float* grad, const int* lens, int nseg,
                                     void* stream);
 
+/* ---- gradient of the row softmax, per row: dst += out . (grad - <grad, out>)
+ *      (Softmax::Backward -> SoftmaxDeriv, src/nn/softmax.cpp:8-29,53-70; cunn_SoftMax_updateGradInput_kernel,
+ *      src/nn/softmax.cu:10-59).  dst, out, grad [rows, cols]; dst may not alias the others. */
+int gnnhip_row_softmax_deriv_f32(float* dst, const float* out, const float* grad, int rows, int cols, void* stream);
+
 /* ---- y[i] *= x[i] : DTensor<GPU>::ElewiseMul(DTensor) with equal shapes
  *      (src/tensor/gpu_dense_tensor.cu:611-628, include/tensor/gpu_binary_functor.h:40-95) */
 int gnnhip_mul_f32(size_t n, const float* x, float* y, void* stream);

@@ -308,3 +308,45 @@ def test_reference_example_runs_unchanged(gpu, tmp_path):
     # held-out accuracy, well above the 0.5 of a coin: the example seeds its weights and its shuffling from
     # the clock, so the exact figure differs from run to run (typically 0.8 to 0.95 on the 80 graphs)
     assert max(acc for _, acc in tests[-3:]) > 0.7
+
+
+def _write_idx(path_images, path_labels, images, labels):
+    """the MNIST files' layout: big-endian magic, count (and rows, cols), then bytes"""
+    with open(path_images, "wb") as f:
+        f.write(np.array([0x803, len(images), 28, 28], ">i4").tobytes())
+        f.write(np.ascontiguousarray(images, np.uint8).tobytes())
+    with open(path_labels, "wb") as f:
+        f.write(np.array([0x801, len(labels)], ">i4").tobytes())
+        f.write(np.ascontiguousarray(labels, np.uint8).tobytes())
+
+
+def test_reference_mnist_example_runs_unchanged(gpu, tmp_path):
+    """graphnn's other example, examples/mnist/mnist.cpp (785-1024-1024-10 perceptron: FullyConnected, ReLU, Softmax,
+    CrossEntropy on probabilities, ReduceMean, ArgMax, InTopK, TypeCast, MomentumSGDOptimizer, ParamSet::Save), not a
+    line changed, built against the host layer and run on files in the MNIST layout: ten noisy prototypes, one per
+    class (the MNIST files themselves are not in the image).  Ten epochs as the example hard-codes them: the test
+    loss falls and the error rate ends far below the 0.9 of a guess"""
+    exe = os.path.join(BUILD, "mnist")
+    if not os.path.exists(exe):
+        pytest.skip("the reference mnist example was not built (graphnn source tree absent at build time)")
+    rng = np.random.default_rng(1998)
+    proto = rng.integers(0, 256, (10, 784))
+    def make(n):
+        y = rng.integers(0, 10, n)
+        x = 0.45 * proto[y] + 0.55 * rng.integers(0, 256, (n, 784))
+        return np.clip(x, 0, 255).astype(np.uint8), y.astype(np.uint8)
+    d = str(tmp_path)
+    _write_idx(d + "/train-images", d + "/train-labels", *make(3000))
+    _write_idx(d + "/test-images", d + "/test-labels", *make(700))
+    r = subprocess.run([exe, "-train_feat", d + "/train-images", "-train_label", d + "/train-labels", "-test_feat", d + "/test-images",
+                        "-test_label", d + "/test-labels", "-device", "0"], capture_output=True, text=True, timeout=300, cwd=d)
+    assert r.returncode == 0, r.stderr[-3000:]
+    assert "3000 images for training" in r.stderr and "700 images for test" in r.stderr
+    rows = [(float(m.group(1)), float(m.group(2))) for m in re.finditer(r"test loss: ([0-9.eE+-]+)\s+error rate: ([0-9.eE+-]+)", r.stderr)]
+    assert len(rows) == 10
+    assert rows[0][0] > np.log(10) and rows[0][1] > 0.7                      # untrained: ten classes, a guess (pixels up to 255: not ln 10)
+    assert rows[-1][0] < 0.25 * rows[0][0] and rows[-1][1] < 0.05            # trained
+    # one checkpoint per epoch in graphnn's format: w1 [785,1024], w2 [1025,1024], wo [1025,10]
+    blob = open(d + "/epoch_9.model", "rb").read()
+    assert len(blob) == sum(8 * 4 + 4 * r_ * c_ for r_, c_ in ((785, 1024), (1025, 1024), (1025, 10)))
+    assert np.frombuffer(blob[:24], dtype=np.uint64).tolist() == [2, 785, 1024]

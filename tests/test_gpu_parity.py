@@ -388,6 +388,25 @@ def test_jagged_softmax_gradient(gpu, oracle):
     assert_parity("jagged softmax gradient", got, want, want64)
 
 
+@pytest.mark.parametrize("rows,cols", [(100, 10), (1, 1), (37, 300), (5000, 2), (3, 1025)])
+def test_row_softmax_gradient(gpu, oracle, rows, cols):
+    """dst += (grad - <grad, out>) * out per row (SoftmaxDeriv, src/nn/softmax.cpp:8-29): the segment rule of the
+    jagged softmax with equal segments, which is how the oracle states it; float64 settles a miss; and the
+    textbook property that a constant gradient passes nothing on (the probabilities of a row add up to 1)"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(rows + cols)
+    p = oracle.row_softmax((rng.standard_normal((rows, cols)) * 2).astype(np.float32))
+    g = rng.standard_normal((rows, cols)).astype(np.float32)
+    d0 = rng.standard_normal((rows, cols)).astype(np.float32)
+    lens = np.full(rows, cols, np.int32)
+    want = oracle.jagged_softmax_deriv(d0.reshape(-1), p.reshape(-1), g.reshape(-1), lens).reshape(rows, cols)
+    got = _n(ops.row_softmax_deriv(_t(d0, gpu), _t(p, gpu), _t(g, gpu)))
+    z = (g.astype(np.float64) * p).sum(axis=1, keepdims=True)
+    assert_parity("row softmax gradient", got, want, d0 + (g - z) * p.astype(np.float64))
+    flat = _n(ops.row_softmax_deriv(_t(np.zeros_like(d0), gpu), _t(p, gpu), _t(np.full_like(g, 3.5), gpu)))
+    assert np.abs(flat).max() < 1e-5
+
+
 # ------------------------------------------------------------------ reductions and index ops
 @pytest.mark.parametrize("n", [1, 63, 256, 4000, 16385, 3_000_001])
 def test_reduce(gpu, oracle, n):
