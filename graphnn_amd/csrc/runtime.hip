@@ -466,6 +466,48 @@ int gnnhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void
     return GNNHIP_OK;
 }
 
+int gnnhip_memcpy_d2h_batch(int count, void* const* dst_host, const void* const* src_device, const size_t* bytes, void* stream)
+{
+    GNNHIP_REQUIRE(count >= 0 && (count == 0 || (dst_host && src_device && bytes)), "bad arguments in memcpy_d2h_batch");
+    if (count == 0) return GNNHIP_OK;
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    // every piece at an 8-byte boundary of the pinned landing buffer
+    size_t total = 0;
+    for (int i = 0; i < count; ++i) {
+        GNNHIP_REQUIRE(bytes[i] == 0 || (dst_host[i] && src_device[i]), "null pointer in memcpy_d2h_batch");
+        total += (bytes[i] + 7) & ~(size_t)7;
+    }
+    void* pin = nullptr;
+    if (total <= kReadbackBytes) {
+        Runtime& r = rt();
+        std::lock_guard<std::mutex> lock(r.mu);
+        void*& slot = r.readback[s];
+        if (!slot && (hipHostMalloc(&slot, kReadbackBytes, hipHostMallocDefault) != hipSuccess || !slot)) {
+            (void)hipGetLastError();
+            slot = nullptr;
+        }
+        pin = slot;
+    }
+    if (!pin) {
+        for (int i = 0; i < count; ++i)
+            if (int rc = gnnhip_memcpy_d2h(dst_host[i], src_device[i], bytes[i], stream)) return rc;
+        return GNNHIP_OK;
+    }
+    size_t at = 0;
+    for (int i = 0; i < count; ++i) {
+        if (bytes[i]) GNNHIP_HIP(hipMemcpyAsync(static_cast<char*>(pin) + at, src_device[i], bytes[i], hipMemcpyDeviceToHost, s));
+        at += (bytes[i] + 7) & ~(size_t)7;
+    }
+    GNNHIP_HIP(hipStreamSynchronize(s));
+    at = 0;
+    for (int i = 0; i < count; ++i) {
+        if (bytes[i]) memcpy(dst_host[i], static_cast<char*>(pin) + at, bytes[i]);
+        at += (bytes[i] + 7) & ~(size_t)7;
+    }
+    return GNNHIP_OK;
+}
+
 int gnnhip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream)
 {
     if (bytes == 0) return GNNHIP_OK;

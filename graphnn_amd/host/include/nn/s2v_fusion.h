@@ -638,6 +638,12 @@ inline void FactorGraph::FoldLossTail(Plan& plan)
             GNN_HIP(gnnhip_s2v_loss_acc_f32((int)B, (int)Q, Logits->value.data->ptr, Y->value.data->row_ptr, Y->value.data->col_idx,
                                             Y->value.data->val, probs->data->ptr, Ce->value.data->ptr, nullptr,
                                             Loss->value.data->ptr, Acc ? Acc->value.data->ptr : nullptr, GpuHandle::Stream()));
+            if (Acc) {
+                // the caller reads the two numbers one after the other: the first read brings both
+                auto both = std::make_shared< detail::ScalarGroup<float> >();
+                Loss->value.JoinScalars(both);
+                Acc->value.JoinScalars(both);
+            }
         };
         int last = -1;
         for (size_t f : fs) { const int i = single_step_of(f); last = std::max(last, i); }

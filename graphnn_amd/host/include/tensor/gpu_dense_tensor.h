@@ -17,6 +17,16 @@ template<typename Dtype> class TensorTemplate<GPU, ROW_SPARSE, Dtype>;
 
 namespace detail
 {
+// One-element tensors that one launch writes and a caller reads one after the other (the loss and the accuracy):
+// the first AsScalar of any of them fetches all, behind one wait for the device.
+template<typename Dtype>
+struct ScalarGroup
+{
+    std::vector<const Dtype*> device;
+    std::vector<Dtype> host;
+    bool fetched = false;
+};
+
 // storage shared by the float and int specialisations
 template<typename Dtype>
 class GpuDenseBase : public Tensor
@@ -25,6 +35,7 @@ public:
     GpuDenseBase() : data(std::make_shared< DenseData<GPU, Dtype> >()) {}
     virtual void Reshape(std::vector<size_t> l) override
     {
+        scalars.reset();                   // whoever writes the tensor next reshapes it first
         shape.Reshape(l);
         if (!data) data = std::make_shared< DenseData<GPU, Dtype> >();
         data->Resize(shape.Count());
@@ -50,11 +61,34 @@ public:
     Dtype AsScalar()
     {
         ASSERT(shape.Count() == 1, "can only convert trivial tensor to scalar");
+        if (scalars && scalar_slot < scalars->device.size() && scalars->device[scalar_slot] == data->ptr) {
+            auto& g = *scalars;
+            if (!g.fetched) {
+                const size_t n = g.device.size();
+                g.host.resize(n);
+                std::vector<void*> dst(n);
+                std::vector<const void*> src(n);
+                std::vector<size_t> bytes(n, sizeof(Dtype));
+                for (size_t i = 0; i < n; ++i) { dst[i] = &g.host[i]; src[i] = g.device[i]; }
+                GNN_HIP(gnnhip_memcpy_d2h_batch((int)n, dst.data(), src.data(), bytes.data(), GpuHandle::Stream()));
+                g.fetched = true;
+            }
+            return g.host[scalar_slot];
+        }
         Dtype v;
         GNN_HIP(gnnhip_memcpy_d2h(&v, data->ptr, sizeof(Dtype), GpuHandle::Stream()));
         return v;
     }
+    // the tensor joins a group of scalars written together (the writer calls this after its launch)
+    void JoinScalars(const std::shared_ptr< ScalarGroup<Dtype> >& group)
+    {
+        scalar_slot = group->device.size();
+        group->device.push_back(data->ptr);
+        scalars = group;
+    }
     std::shared_ptr< DenseData<GPU, Dtype> > data;
+    std::shared_ptr< ScalarGroup<Dtype> > scalars;
+    size_t scalar_slot = 0;
 };
 }  // namespace detail
 

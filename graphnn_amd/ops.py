@@ -93,6 +93,16 @@ def gemm(A, B, transA=False, transB=False, alpha=1.0, beta=0.0, out=None):
     return out
 
 
+def read_scalars(tensors):
+    """the first element of each device tensor, all behind one wait for the stream"""
+    n = len(tensors)
+    outs = [np.zeros(1, np.float32 if t.dtype == torch.float32 else np.int32) for t in tensors]
+    P = ctypes.c_void_p * n
+    check(_lib().gnnhip_memcpy_d2h_batch(n, P(*[o.ctypes.data for o in outs]), P(*[t.data_ptr() for t in tensors]),
+                                         (ctypes.c_size_t * n)(*[4] * n), _stream()))
+    return [o[0] for o in outs]
+
+
 def row_softmax_deriv(dst, out, grad):
     """dst += out * (grad - <grad, out> per row), in place on dst"""
     rows, cols = out.shape

@@ -74,6 +74,11 @@ int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void
 int gnnhip_memcpy_h2d_sparse32(void* dst_device, const void* src_host, size_t words, void* stream);
 int gnnhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
 int gnnhip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream);
+/* ---- count small device-to-host reads behind ONE wait for the stream: the loss and the accuracy that the example
+ *      reads one after the other with DTensor<GPU>::AsScalar (src/tensor/gpu_dense_tensor.cu:129-137, read at
+ *      examples/graph_classification/include/nn_common.h:140-160).  dst_host, src_device, bytes: host arrays of count
+ *      entries; pieces of up to 4 KB together land in pinned memory, larger ones are read one by one. */
+int gnnhip_memcpy_d2h_batch(int count, void* const* dst_host, const void* const* src_device, const size_t* bytes, void* stream);
 int gnnhip_memset0(void* device_ptr, size_t bytes, void* stream);
 /* n buffers zeroed in one launch (the gradient tensors FactorGraph::BackPropagate clears one by one,
  * src/nn/factor_graph.cpp:190-196); entries with 0 bytes are skipped. */

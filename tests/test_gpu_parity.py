@@ -1817,6 +1817,25 @@ def test_device_csr_transpose(gpu, oracle, m, k, nnz):
     assert np.allclose(got, (A.T @ B), atol=1e-4)
 
 
+def test_scalars_read_behind_one_wait(gpu):
+    """gnnhip_memcpy_d2h_batch: the first elements of several device tensors (a loss, an accuracy, an int), queued
+    behind the kernels that wrote them, arrive together; pieces too large for the pinned landing buffer are read one by one"""
+    import ctypes
+    import torch
+    from graphnn_amd import ops
+    a = torch.full((1,), 2.5, device=gpu); b = torch.full((3,), -7.0, device=gpu); c = torch.full((1,), 41, dtype=torch.int32, device=gpu)
+    a.mul_(2.0)                                                   # still in the queue when the read is issued
+    got = ops.read_scalars([a, b, c])
+    assert got[0] == 5.0 and got[1] == -7.0 and got[2] == 41
+    assert ops.read_scalars([]) == []
+    big = torch.arange(3000, dtype=torch.float32, device=gpu)     # 12 KB: past the landing buffer
+    host = np.zeros(3000, np.float32); one = np.zeros(1, np.float32)
+    P = ctypes.c_void_p * 2
+    ops.check(ops._lib().gnnhip_memcpy_d2h_batch(2, P(host.ctypes.data, one.ctypes.data), P(big.data_ptr(), a.data_ptr()),
+                                                 (ctypes.c_size_t * 2)(12000, 4), None))
+    assert np.array_equal(host, np.arange(3000, dtype=np.float32)) and one[0] == 5.0
+
+
 @pytest.mark.parametrize("shape,density", [((7450, 38), "one_hot"), ((7450, 38), 0.5), ((100, 7), "one_hot"), ((300_000, 64), "one_hot"),
                                            ((16384,), 0.0), ((16385,), 1.0 / 17), ((40_000, 3), 1.0 / 15), ((5_000_000,), 0.001)])
 def test_sparse_upload_rebuilds_the_same_bits(gpu, shape, density):
