@@ -35,6 +35,7 @@ SIGNATURES = {
     "gnnhip_memcpy_d2h": [_P, _P, _Z, _P],
     "gnnhip_memcpy_d2d": [_P, _P, _Z, _P],
     "gnnhip_memcpy_d2h_batch": [_I, _P, _P, _P, _P],
+    "gnnhip_memcpy_h2d_batch": [_I, _P, _P, _P, _P],
     "gnnhip_memset0": [_P, _Z, _P],
     "gnnhip_memset0_batch": [_I, _P, _P, _P],
     "gnnhip_stream_sync": [_P],

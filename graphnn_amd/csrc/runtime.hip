@@ -339,6 +339,56 @@ __attribute__((target("avx2"))) bool collect_nonzero_avx2(const unsigned* w, siz
     return collect_nonzero(w, i, words, cap, idx, val, count);
 }
 
+// A staged upload leaves the pinned buffer through a kernel, not through hipMemcpyAsync: the runtime hands copies of
+// this size to a DMA engine, and the kernel that consumes the data then waits for that engine's completion signal to
+// cross over to the compute queue, 15 to 20 us per copy on an otherwise idle device.  A kernel of the stream's own
+// queue reads the pinned memory over the bus just as fast at these sizes (up to 2 MB) and orders itself.
+constexpr int kStageBlock = 256;
+template <typename T>
+__global__ __launch_bounds__(kStageBlock) void stage_copy_kernel(T* __restrict__ dst, const T* __restrict__ src, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * kStageBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kStageBlock) dst[i] = src[i];
+}
+
+// dst_device[0, bytes) = pinned[0, bytes) on stream s, in the widest pieces the three of them allow
+int stage_copy(void* dst_device, const void* pinned, size_t bytes, hipStream_t s)
+{
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(dst_device) | reinterpret_cast<uintptr_t>(pinned) | (uintptr_t)bytes;
+    auto grid_for = [](size_t n) {
+        size_t g = (n + kStageBlock * 4 - 1) / (kStageBlock * 4);          // four pieces per lane
+        return (unsigned)(g < 1 ? 1 : (g > 2048 ? 2048 : g));
+    };
+    if ((bits & 15) == 0) {
+        const size_t n = bytes / 16;
+        hipLaunchKernelGGL(stage_copy_kernel<uint4>, dim3(grid_for(n)), dim3(kStageBlock), 0, s, static_cast<uint4*>(dst_device),
+                           static_cast<const uint4*>(pinned), n);
+    } else if ((bits & 3) == 0) {
+        const size_t n = bytes / 4;
+        hipLaunchKernelGGL(stage_copy_kernel<unsigned>, dim3(grid_for(n)), dim3(kStageBlock), 0, s, static_cast<unsigned*>(dst_device),
+                           static_cast<const unsigned*>(pinned), n);
+    } else {
+        hipLaunchKernelGGL(stage_copy_kernel<unsigned char>, dim3(grid_for(bytes)), dim3(kStageBlock), 0, s,
+                           static_cast<unsigned char*>(dst_device), static_cast<const unsigned char*>(pinned), bytes);
+    }
+    GNNHIP_LAUNCH_CHECK("stage_copy");
+    return GNNHIP_OK;
+}
+
+// several staged pieces leaving in one launch: piece blockIdx.y, 32-bit words
+constexpr int kStagePieces = 8;
+struct StagePieces {
+    unsigned* dst[kStagePieces];
+    const unsigned* src[kStagePieces];
+    size_t words[kStagePieces];
+};
+__global__ __launch_bounds__(kStageBlock) void stage_copy_pieces_kernel(StagePieces p)
+{
+    unsigned* __restrict__ dst = p.dst[blockIdx.y];
+    const unsigned* __restrict__ src = p.src[blockIdx.y];
+    const size_t n = p.words[blockIdx.y];
+    for (size_t i = (size_t)blockIdx.x * kStageBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kStageBlock) dst[i] = src[i];
+}
+
 constexpr int kExpandBlock = 256;
 constexpr int kExpandTile = 1024;        // 32-bit words of the destination per workgroup
 
@@ -385,8 +435,7 @@ int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void
         if (int rc = staging_slot(r, s, bytes, &slot)) return rc;
         if (slot) {
             memcpy(slot, src_host, bytes);
-            GNNHIP_HIP(hipMemcpyAsync(dst_device, slot, bytes, hipMemcpyHostToDevice, s));
-            return GNNHIP_OK;
+            return stage_copy(dst_device, slot, bytes, s);
         }
     }
     GNNHIP_HIP(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, s));
@@ -397,6 +446,53 @@ int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void
 // Host-to-device copy of `words` 32-bit words that sends only the non-zero ones when they are few (one-hot
 // feature matrices: 1.1 MB of which 30 KB are ones).  Same promise as gnnhip_memcpy_h2d; the device ends up with
 // the same bits.
+// count host-to-device copies; pieces of whole, aligned 32-bit words that fit the staging buffer together leave in
+// one launch (the three arrays of a CSR matrix), anything else piece by piece.  Same promise as gnnhip_memcpy_h2d.
+int gnnhip_memcpy_h2d_batch(int count, void* const* dst_device, const void* const* src_host, const size_t* bytes, void* stream)
+{
+    GNNHIP_REQUIRE(count >= 0 && (count == 0 || (dst_device && src_host && bytes)), "bad arguments in memcpy_h2d_batch");
+    if (count == 0) return GNNHIP_OK;
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    size_t total = 0;
+    bool together = count <= kStagePieces;
+    for (int i = 0; i < count; ++i) {
+        GNNHIP_REQUIRE(bytes[i] == 0 || (dst_device[i] && src_host[i]), "null pointer in memcpy_h2d_batch");
+        together = together && bytes[i] % 4 == 0 && reinterpret_cast<uintptr_t>(dst_device[i]) % 4 == 0;
+        total += (bytes[i] + 255) & ~(size_t)255;
+    }
+    char* slot = nullptr;
+    if (together && total <= kStagingHalf) {
+        Runtime& r = rt();
+        std::lock_guard<std::mutex> lock(r.mu);
+        if (int rc = staging_slot(r, s, total, &slot)) return rc;
+    }
+    if (!slot) {
+        for (int i = 0; i < count; ++i)
+            if (int rc = gnnhip_memcpy_h2d(dst_device[i], src_host[i], bytes[i], stream)) return rc;
+        return GNNHIP_OK;
+    }
+    StagePieces p;
+    size_t at = 0, largest = 0;
+    int k = 0;
+    for (int i = 0; i < count; ++i) {
+        if (bytes[i] == 0) continue;
+        memcpy(slot + at, src_host[i], bytes[i]);
+        p.dst[k] = static_cast<unsigned*>(dst_device[i]);
+        p.src[k] = reinterpret_cast<const unsigned*>(slot + at);
+        p.words[k] = bytes[i] / 4;
+        if (p.words[k] > largest) largest = p.words[k];
+        at += (bytes[i] + 255) & ~(size_t)255;
+        ++k;
+    }
+    if (k == 0) return GNNHIP_OK;
+    size_t gx = (largest + kStageBlock * 4 - 1) / (kStageBlock * 4);
+    if (gx > 1024) gx = 1024;
+    hipLaunchKernelGGL(stage_copy_pieces_kernel, dim3((unsigned)gx, (unsigned)k), dim3(kStageBlock), 0, s, p);
+    GNNHIP_LAUNCH_CHECK("stage_copy_pieces");
+    return GNNHIP_OK;
+}
+
 int gnnhip_memcpy_h2d_sparse32(void* dst_device, const void* src_host, size_t words, void* stream)
 {
     constexpr size_t kMinWords = 16384;                  // below this the plain copy is one short DMA anyway
@@ -424,7 +520,8 @@ int gnnhip_memcpy_h2d_sparse32(void* dst_device, const void* src_host, size_t wo
     memmove(idx + count, val, count * 4);                // indices and values back to back: one copy
     void* dev = nullptr;
     if (int rc = stream_scratch_slot(s, 6, (count ? count : 1) * 8, &dev)) return rc;
-    if (count) GNNHIP_HIP(hipMemcpyAsync(dev, slot, count * 8, hipMemcpyHostToDevice, s));
+    if (count)
+        if (int rc = stage_copy(dev, slot, count * 8, s)) return rc;
     const unsigned* d_idx = static_cast<const unsigned*>(dev);
     const unsigned grid = (unsigned)((words + kExpandTile - 1) / kExpandTile);
     hipLaunchKernelGGL(expand_pairs_kernel, dim3(grid), dim3(kExpandBlock), 0, s, static_cast<unsigned*>(dst_device), words, d_idx,

@@ -69,21 +69,21 @@ public:
         t_data->Reserve(t.data->nnz, t.data->len_ptr);
         t_data->nnz = t.data->nnz;
         t_data->len_ptr = t.data->len_ptr;
-        void* s = GpuHandle::Stream();
-        GNN_HIP(gnnhip_memcpy_h2d(t_data->val, t.data->val, sizeof(Dtype) * (size_t)t.data->nnz, s));
-        GNN_HIP(gnnhip_memcpy_h2d(t_data->col_idx, t.data->col_idx, sizeof(int) * (size_t)t.data->nnz, s));
-        GNN_HIP(gnnhip_memcpy_h2d(t_data->row_ptr, t.data->row_ptr, sizeof(int) * (size_t)t.data->len_ptr, s));
+        void* dst[3] = {t_data->val, t_data->col_idx, t_data->row_ptr};
+        const void* from[3] = {t.data->val, t.data->col_idx, t.data->row_ptr};
+        const size_t bytes[3] = {sizeof(Dtype) * (size_t)t.data->nnz, sizeof(int) * (size_t)t.data->nnz, sizeof(int) * (size_t)t.data->len_ptr};
+        GNN_HIP(gnnhip_memcpy_h2d_batch(3, dst, from, bytes, GpuHandle::Stream()));
         t_valid = true;
     }
-    // three host-to-device copies, ordered on the layer's stream
+    // the three arrays in one batch of host-to-device copies, ordered on the layer's stream
     void CopyFrom(SpTensor<CPU, Dtype>& src)
     {
         shape = src.shape;
         ResizeSp(src.data->nnz, src.data->len_ptr);
-        void* s = GpuHandle::Stream();
-        GNN_HIP(gnnhip_memcpy_h2d(data->val, src.data->val, sizeof(Dtype) * (size_t)data->nnz, s));
-        GNN_HIP(gnnhip_memcpy_h2d(data->col_idx, src.data->col_idx, sizeof(int) * (size_t)data->nnz, s));
-        GNN_HIP(gnnhip_memcpy_h2d(data->row_ptr, src.data->row_ptr, sizeof(int) * (size_t)data->len_ptr, s));
+        void* dst[3] = {data->val, data->col_idx, data->row_ptr};
+        const void* from[3] = {src.data->val, src.data->col_idx, src.data->row_ptr};
+        const size_t bytes[3] = {sizeof(Dtype) * (size_t)data->nnz, sizeof(int) * (size_t)data->nnz, sizeof(int) * (size_t)data->len_ptr};
+        GNN_HIP(gnnhip_memcpy_h2d_batch(3, dst, from, bytes, GpuHandle::Stream()));
     }
     void CopyFrom(SpTensor<GPU, Dtype>& src)
     {

@@ -73,6 +73,10 @@ int gnnhip_pool_stats(size_t* bytes_in_use, size_t* bytes_parked, size_t* n_driv
 int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream);
 int gnnhip_memcpy_h2d_sparse32(void* dst_device, const void* src_host, size_t words, void* stream);
 int gnnhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
+/* ---- count host-to-device copies with the promise of gnnhip_memcpy_h2d, in one launch where the pieces allow it
+ *      (whole 32-bit words, up to 8 pieces, 2 MB together): the three arrays that SpTensor<GPU>::CopyFrom(CPU) sends
+ *      one by one (src/tensor/gpu_sparse_tensor.cu:55-63).  dst_device, src_host, bytes: host arrays of count entries. */
+int gnnhip_memcpy_h2d_batch(int count, void* const* dst_device, const void* const* src_host, const size_t* bytes, void* stream);
 int gnnhip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream);
 /* ---- count small device-to-host reads behind ONE wait for the stream: the loss and the accuracy that the example
  *      reads one after the other with DTensor<GPU>::AsScalar (src/tensor/gpu_dense_tensor.cu:129-137, read at

@@ -1817,6 +1817,36 @@ def test_device_csr_transpose(gpu, oracle, m, k, nnz):
     assert np.allclose(got, (A.T @ B), atol=1e-4)
 
 
+def test_uploads_in_one_batch(gpu):
+    """gnnhip_memcpy_h2d_batch: the three arrays of a CSR matrix in one launch, an empty piece among them; pieces that
+    are not whole words, or too many, or too large for the staging buffer, go one by one; the host buffers are free
+    as soon as the call returns"""
+    import ctypes
+    import torch
+    from graphnn_amd import ops
+    rng = np.random.default_rng(12)
+    def send(arrays):
+        outs = [torch.full((max(a.nbytes, 1),), 255, dtype=torch.uint8, device=gpu) for a in arrays]
+        n = len(arrays)
+        P = ctypes.c_void_p * n
+        ops.check(ops._lib().gnnhip_memcpy_h2d_batch(n, P(*[o.data_ptr() for o in outs]), P(*[a.ctypes.data for a in arrays]),
+                                                     (ctypes.c_size_t * n)(*[a.nbytes for a in arrays]), None))
+        for a in arrays:
+            a[...] = 0                                            # the call has read them
+        return [o.cpu().numpy()[:max(len(w), 0)] for o, w in zip(outs, wants)]
+    cases = [[rng.integers(0, 1 << 30, 16382).astype(np.int32), rng.standard_normal(16382).astype(np.float32),
+              rng.integers(0, 9, 7451).astype(np.int32)],
+             [np.zeros(0, np.int32), rng.integers(0, 99, 5).astype(np.int32)],
+             [rng.integers(0, 255, 7).astype(np.uint8), rng.integers(0, 99, 33).astype(np.int32)],
+             [rng.integers(0, 99, 3).astype(np.int32) for _ in range(11)],
+             [rng.integers(0, 99, 700_000).astype(np.int32), rng.integers(0, 99, 4).astype(np.int32)]]
+    for arrays in cases:
+        wants = [a.tobytes() for a in arrays]
+        got = send(arrays)
+        for g, w in zip(got, wants):
+            assert g.tobytes()[:len(w)] == w
+
+
 def test_scalars_read_behind_one_wait(gpu):
     """gnnhip_memcpy_d2h_batch: the first elements of several device tensors (a loss, an accuracy, an int), queued
     behind the kernels that wrote them, arrive together; pieces too large for the pinned landing buffer are read one by one"""
