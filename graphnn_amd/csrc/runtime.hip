@@ -355,7 +355,7 @@ int stage_copy(void* dst_device, const void* pinned, size_t bytes, hipStream_t s
 {
     const uintptr_t bits = reinterpret_cast<uintptr_t>(dst_device) | reinterpret_cast<uintptr_t>(pinned) | (uintptr_t)bytes;
     auto grid_for = [](size_t n) {
-        size_t g = (n + kStageBlock * 4 - 1) / (kStageBlock * 4);          // four pieces per lane
+        size_t g = (n + kStageBlock - 1) / kStageBlock;                    // one piece per lane: every read of a small copy in flight at once
         return (unsigned)(g < 1 ? 1 : (g > 2048 ? 2048 : g));
     };
     if ((bits & 15) == 0) {
@@ -486,7 +486,7 @@ int gnnhip_memcpy_h2d_batch(int count, void* const* dst_device, const void* cons
         ++k;
     }
     if (k == 0) return GNNHIP_OK;
-    size_t gx = (largest + kStageBlock * 4 - 1) / (kStageBlock * 4);
+    size_t gx = (largest + kStageBlock - 1) / kStageBlock;
     if (gx > 1024) gx = 1024;
     hipLaunchKernelGGL(stage_copy_pieces_kernel, dim3((unsigned)gx, (unsigned)k), dim3(kStageBlock), 0, s, p);
     GNNHIP_LAUNCH_CHECK("stage_copy_pieces");
