@@ -567,6 +567,21 @@ __global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(int rows, 
     }
 }
 
+// col_idx[j] = j and val[j] = 1 (or 1 / row length) for j in [row_ptr[i], row_ptr[i+1]): a wavefront per row
+__global__ __launch_bounds__(kBlock) void consecutive_rows_kernel(int rows, const int* __restrict__ row_ptr, int average,
+                                                                  int* __restrict__ col_idx, float* __restrict__ val)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const long long row = ((long long)blockIdx.x * kBlock + threadIdx.x) / kWave;
+    if (row >= rows) return;
+    const int a = row_ptr[row], b = row_ptr[row + 1];
+    const float w = (average && b > a) ? (float)(1.0 / (double)(b - a)) : 1.0f;       // as the reference: double divide, then narrowed
+    for (int j = a + lane; j < b; j += kWave) {
+        col_idx[j] = j;
+        val[j] = w;
+    }
+}
+
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 }  // namespace
@@ -677,6 +692,18 @@ int gnnhip_csr_group_i32(int rows, int n, const int* key, int key_stride, const 
     GNNHIP_REQUIRE(n == 0 || rows >= 1, "pairs but no rows in csr_group");
     if (int rc = require_ready()) return rc;
     return csr_group_pairs(rows, n, key, key_stride, payload, payload_stride, nullptr, average, row_ptr, col_idx, val, as_stream(stream));
+}
+
+int gnnhip_csr_consecutive_rows_f32(int rows, const int* row_ptr, int average, int* col_idx, float* val, void* stream)
+{
+    GNNHIP_REQUIRE(rows >= 0, "negative row count in csr_consecutive_rows");
+    if (rows == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(row_ptr && col_idx && val, "null array in csr_consecutive_rows");
+    if (int rc = require_ready()) return rc;
+    const unsigned grid = (unsigned)(((long long)rows * kWave + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(consecutive_rows_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), rows, row_ptr, average, col_idx, val);
+    GNNHIP_LAUNCH_CHECK("consecutive_rows");
+    return GNNHIP_OK;
 }
 
 int gnnhip_csr_group_both_i32(int rows, int n, const int* x, int x_stride, const int* y, int y_stride,

@@ -134,18 +134,19 @@ inline void group_edges_on_device(GraphStruct* graph, bool payload_is_edge, bool
     GNN_HIP(gnnhip_csr_group_i32(N, E, pairs + 1, 2, payload, payload_stride, average ? 1 : 0,
                                  out.data->row_ptr, out.data->col_idx, out.data->val, GpuHandle::Stream()));
 }
-// CSR [num_subgraph, num_nodes] on the device from one copy of the (subgraph, node) records
-inline void group_nodes_on_device(GraphStruct* graph, bool average, SpTensor<GPU, float>& out, DTensor<GPU, int>& staging)
+// CSR [num_subgraph, num_nodes] on the device for nodes that were added subgraph after subgraph, each with the next
+// index: the subgraph offsets (the host has just found them) travel, the device writes the entries.
+// offsets[q] is set for q <= last; the subgraphs behind the last one that has nodes are empty.
+inline void consecutive_rows_on_device(GraphStruct* graph, std::vector<int>& offsets, int last, int nodes, bool average,
+                                       SpTensor<GPU, float>& out)
 {
-    static_assert(sizeof(std::pair<int, int>) == 2 * sizeof(int), "node list is not a flat (subgraph, node) array");
-    const int M = (int)graph->node_list.size(), B = (int)graph->num_subgraph;
+    const int B = (int)graph->num_subgraph;
+    for (int q = last + 1; q <= B; ++q) offsets[q] = nodes;
     out.Reshape({(size_t)B, (size_t)graph->num_nodes});
-    out.ResizeSp(M, B + 1);
-    staging.Reshape({2 * (size_t)std::max(M, 1)});
-    int* pairs = staging.data->ptr;
-    if (M > 0) GNN_HIP(gnnhip_memcpy_h2d(pairs, graph->node_list.data(), sizeof(int) * 2 * (size_t)M, GpuHandle::Stream()));
-    GNN_HIP(gnnhip_csr_group_i32(B, M, pairs, 2, pairs + 1, 2, average ? 1 : 0, out.data->row_ptr, out.data->col_idx, out.data->val,
-                                 GpuHandle::Stream()));
+    out.ResizeSp(nodes, B + 1);
+    GNN_HIP(gnnhip_memcpy_h2d(out.data->row_ptr, offsets.data(), sizeof(int) * ((size_t)B + 1), GpuHandle::Stream()));
+    if (nodes > 0)
+        GNN_HIP(gnnhip_csr_consecutive_rows_f32(B, out.data->row_ptr, average ? 1 : 0, out.data->col_idx, out.data->val, GpuHandle::Stream()));
 }
 // The device groups a batch in one launch (up to 16 workgroups, each a run of the rows) when a run's counters
 // (4 bytes per row) and the slots of all pairs (2.35 bytes each, with the lists and one bitmap) fit 160 KB of
@@ -167,13 +168,12 @@ inline bool group_edges_if_gpu<float, SpTensor<GPU, float> >(GraphStruct* graph,
     return true;
 }
 template<typename Dtype, typename SpT>
-inline bool group_nodes_if_gpu(GraphStruct*, bool, SpT&, DTensor<GPU, int>&) { return false; }
+inline bool consecutive_rows_if_gpu(GraphStruct*, std::vector<int>&, int, int, bool, SpT&) { return false; }
 template<>
-inline bool group_nodes_if_gpu<float, SpTensor<GPU, float> >(GraphStruct* graph, bool average, SpTensor<GPU, float>& out,
-                                                             DTensor<GPU, int>& staging)
+inline bool consecutive_rows_if_gpu<float, SpTensor<GPU, float> >(GraphStruct* graph, std::vector<int>& offsets, int last, int nodes,
+                                                                  bool average, SpTensor<GPU, float>& out)
 {
-    if (!device_grouping_pays(graph->node_list.size(), graph->num_subgraph)) return false;
-    group_nodes_on_device(graph, average, out, staging);
+    consecutive_rows_on_device(graph, offsets, last, nodes, average, out);
     return true;
 }
 // Batches of up to this many nodes are examined on the host for edges between subgraphs (the one-launch
@@ -330,25 +330,29 @@ public:
 protected:
     // Nodes added subgraph after subgraph, each with the next index (GetBatch does): the matrix is then the
     // identity layout, its facts are known from one pass over the records, and the device groups it.
-    virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out, Phase phase) override
+    virtual bool BuildOnDevice(GraphStruct* graph, SpTensor<mode, Dtype>& out, Phase) override
     {
-        const int M = (int)graph->node_list.size();
+        const int M = (int)graph->node_list.size(), B = (int)graph->num_subgraph;
         if (M != (int)graph->num_nodes) return false;
-        int biggest = 0, run = 0, prev = 0;
+        offsets.assign((size_t)B + 1, 0);
+        int biggest = 0, prev = 0, start = 0;
         bool ordered = true;
         for (int i = 0; i < M && ordered; ++i) {
             const int g = graph->node_list[i].first;
-            ordered = graph->node_list[i].second == i && g >= prev && g < (int)graph->num_subgraph;
-            run = g == prev ? run + 1 : 1;
-            biggest = std::max(biggest, run);
-            prev = g;
+            ordered = graph->node_list[i].second == i && g >= prev && g < B;
+            if (g != prev && ordered) {
+                biggest = std::max(biggest, i - start);
+                for (int q = prev + 1; q <= g; ++q) offsets[q] = i;
+                prev = g;
+                start = i;
+            }
         }
-        if (!ordered || !detail::group_nodes_if_gpu<Dtype>(graph, this->average, out, node_staging)) return false;
+        if (!ordered || !detail::consecutive_rows_if_gpu<Dtype>(graph, offsets, prev, M, this->average, out)) return false;
         this->layout.contiguous_subgraphs = true;
-        this->layout.max_subgraph_nodes = biggest;
+        this->layout.max_subgraph_nodes = std::max(biggest, M - start);
         return true;
     }
-    DTensor<GPU, int> node_staging;
+    std::vector<int> offsets;
 
     virtual void InitCPUWeight(GraphStruct* graph) override
     {

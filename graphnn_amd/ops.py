@@ -545,6 +545,17 @@ def csr_group_both(rows, x, y, x_stride=1, y_stride=1, n=None):
     return tuple(out[:3]), tuple(out[3:])
 
 
+def csr_consecutive_rows(row_ptr, average=False):
+    """col_idx, val of the CSR matrix whose row i lists the columns row_ptr[i] .. row_ptr[i+1]-1 (row_ptr on the device)"""
+    rows = row_ptr.numel() - 1
+    n = int(row_ptr[-1].item())
+    col_idx = torch.empty(n, dtype=torch.int32, device=row_ptr.device)
+    val = torch.empty(n, dtype=torch.float32, device=row_ptr.device)
+    check(_lib().gnnhip_csr_consecutive_rows_f32(rows, _i32(row_ptr, "row_ptr"), int(average), _i32(col_idx, "col_idx"),
+                                                 _f32(val, "val"), _stream()))
+    return col_idx, val
+
+
 def csr_transpose(row_ptr, col_idx, val, m, k):
     nnz = col_idx.numel()
     dev = row_ptr.device

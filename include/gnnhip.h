@@ -114,6 +114,13 @@ int gnnhip_spmm_csr_f32(int m, int k, int n, int nnz, float alpha, const int* ro
 int gnnhip_csr_group_i32(int rows, int n, const int* key, int key_stride, const int* payload, int payload_stride,
                          int average, int* row_ptr, int* col_idx, float* val, void* stream);
 
+/* ---- the entries of a CSR matrix whose row i lists the consecutive columns row_ptr[i] .. row_ptr[i+1]-1 with value 1
+ *      (1 / row length when average != 0): the operand of SubgraphMsgPass (src/nn/msg_pass.cpp:156-177) for a batch
+ *      whose nodes were added subgraph after subgraph, as GetBatch adds them
+ *      (examples/graph_classification/include/nn_common.h:36-105).  row_ptr [rows+1] is on the device already (the
+ *      subgraph offsets, which the host knows); col_idx and val have row_ptr[rows] entries. */
+int gnnhip_csr_consecutive_rows_f32(int rows, const int* row_ptr, int average, int* col_idx, float* val, void* stream);
+
 /* ---- the n pairs (x, y) grouped both ways at once, values 1: row i of (row_ptr, col_idx, val) lists the x of the
  *      pairs with y = i, which is gnnhip_csr_group_i32(rows, n, y, .., x, .., 0, ..), the operand of
  *      Node2NodeMsgPass (src/nn/msg_pass.cpp:46-67); row i of (t_row_ptr, t_col_idx, t_val) lists the y of the

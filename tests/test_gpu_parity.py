@@ -1769,6 +1769,21 @@ def test_device_csr_group_of_a_small_batch_in_one_launch(gpu, case):
     assert np.array_equal(_n(rp), want[0]) and np.array_equal(_n(ci), want[1])
 
 
+@pytest.mark.parametrize("average", [False, True])
+def test_device_csr_of_consecutive_rows(gpu, oracle, average):
+    """the pooling operand of a batch whose nodes were added subgraph after subgraph, from the subgraph offsets alone:
+    bit-identical to what the host builder makes of the (subgraph, node) records, graphs without nodes and a graph of
+    3,000 nodes among them"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(5)
+    sizes = rng.integers(0, 60, 700); sizes[[0, 1, 350, 699]] = 0; sizes[77] = 3000
+    sid = np.repeat(np.arange(sizes.size), sizes).astype(np.int32)
+    nid = np.arange(sid.size, dtype=np.int32)
+    want = oracle.csr_subgraph(sizes.size, sid, nid, average)
+    ci, v = ops.csr_consecutive_rows(_t(want[0], gpu), average)
+    assert np.array_equal(_n(ci), want[1]) and np.array_equal(_n(v), want[2])
+
+
 @pytest.mark.parametrize("rows,n", [(7450, 16382), (300, 40_000), (50_000, 70_000), (9, 1), (5, 0)])
 def test_device_csr_group_both_ways(gpu, rows, n):
     """an edge list grouped by head and by tail at once (a matrix and its transpose, entries in edge order): the one-launch
