@@ -425,7 +425,8 @@ def end_to_end_host_layer(host, reps=300):
         return {"skipped": "host_forward_bench failed: " + (r.stderr or r.stdout)[-300:]}
     res = json.loads(r.stdout.strip().splitlines()[-1])
     res["graphs_per_s"] = res["graphs"] / (res["us_per_batch"] * 1e-6)
-    res["what"] = ("GetBatch-style host batch build + CSR build + H2D + FactorGraph::FeedForward (fused plan) + "
+    res["what"] = ("GetBatch-style host batch build + uploads (X, labels, edge records, subgraph offsets) + CSR operands "
+                   "grouped on the device + FactorGraph::FeedForward (fused plan) + "
                    "loss/accuracy read-back, per batch; PCIe-inclusive, never `value`")
     return res
 
