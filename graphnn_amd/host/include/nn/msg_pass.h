@@ -202,15 +202,29 @@ protected:
     }
     DTensor<GPU, int> edge_staging;
 
-    // does every edge stay inside one subgraph?  (node -> subgraph from the AddNode records)
+    // does every edge stay inside one subgraph?  (node -> subgraph from the AddNode records: read in place when the
+    // records came in node order, as GetBatch writes them, through a table otherwise)
     bool NoEdgeBetweenSubgraphs(GraphStruct* graph)
     {
-        node_subgraph.assign(graph->num_nodes, -1);
-        for (const auto& sn : graph->node_list)
-            if (sn.second >= 0 && sn.second < (int)graph->num_nodes) node_subgraph[sn.second] = sn.first;
-        const int* where = node_subgraph.data();
+        static_assert(sizeof(std::pair<int, int>) == 2 * sizeof(int), "node list is not a flat (subgraph, node) array");
+        const auto& records = graph->node_list;
+        const size_t N = graph->num_nodes;
+        bool in_order = records.size() == N;
+        for (size_t i = 0; in_order && i < N; ++i) in_order = (size_t)records[i].second == i;
+        const int* where;
+        size_t stride;
+        if (in_order && N > 0) {
+            where = &records[0].first;
+            stride = 2;
+        } else {
+            node_subgraph.assign(N, -1);
+            for (const auto& sn : records)
+                if (sn.second >= 0 && sn.second < (int)N) node_subgraph[sn.second] = sn.first;
+            where = node_subgraph.data();
+            stride = 1;
+        }
         int differ = 0;
-        for (const auto& e : graph->edge_list) differ |= where[e.first] ^ where[e.second];
+        for (const auto& e : graph->edge_list) differ |= where[(size_t)e.first * stride] ^ where[(size_t)e.second * stride];
         return differ == 0;
     }
 
