@@ -27,6 +27,8 @@ thread_local char g_err[512] = "";
 // and nothing waits for the device.  A half is reused only after the event recorded behind its last
 // copy has completed.
 constexpr size_t kStagingHalf = 2u << 20;
+constexpr int kExpandBlock = 256;
+constexpr int kExpandTile = 1024;        // sparse uploads: 32-bit words of the destination per workgroup
 constexpr size_t kReadbackBytes = 4096;
 struct Staging {
     char* base = nullptr;              // 2 * kStagingHalf bytes from hipHostMalloc
@@ -301,10 +303,13 @@ int staging_slot(Runtime& r, hipStream_t s, size_t bytes, char** out)
 }
 
 // Positions and values of the non-zero words of w[from, words), appended at *count; false when there are more than cap.
-bool collect_nonzero(const unsigned* w, size_t from, size_t words, size_t cap, unsigned* idx, unsigned* val, size_t* count)
+// starts[t] = how many of them lie ahead of word 1024 t (the tiles the device rebuilds the buffer by).
+bool collect_nonzero(const unsigned* w, size_t from, size_t words, size_t cap, unsigned* idx, unsigned* val, size_t* count,
+                     unsigned* starts)
 {
     size_t c = *count;
     for (size_t i = from; i < words; ++i) {
+        if ((i & (kExpandTile - 1)) == 0) starts[i / kExpandTile] = (unsigned)c;     // the tile of 1,024 words that begins here
         if (w[i]) {
             if (c == cap) return false;
             idx[c] = (unsigned)i;
@@ -321,13 +326,14 @@ bool collect_nonzero(const unsigned* w, size_t from, size_t words, size_t cap, u
 // word in every fifth group of 8, a pattern branch predictors lose against: 113 -> 25 us on a desktop-class core, and the whole upload of that matrix
 // 25 -> 21 us on the host of the GPU box.)
 __attribute__((target("avx2"))) bool collect_nonzero_avx2(const unsigned* w, size_t words, size_t cap, unsigned* idx, unsigned* val,
-                                                          size_t* count)
+                                                          size_t* count, unsigned* starts)
 {
     size_t c = 0, i = 0;
     const __m256i zero = _mm256_setzero_si256();
 #define GNNHIP_ZEROS_OF(at) \
     ((unsigned)_mm256_movemask_ps(_mm256_castsi256_ps(_mm256_cmpeq_epi32(_mm256_loadu_si256(reinterpret_cast<const __m256i*>(w + (at))), zero))))
     for (; i + 32 <= words; i += 32) {
+        if ((i & (kExpandTile - 1)) == 0) starts[i / kExpandTile] = (unsigned)c;
         unsigned nz = ~(GNNHIP_ZEROS_OF(i) | (GNNHIP_ZEROS_OF(i + 8) << 8) | (GNNHIP_ZEROS_OF(i + 16) << 16) | (GNNHIP_ZEROS_OF(i + 24) << 24));
         if (!nz) continue;
         if (c + (size_t)__builtin_popcount(nz) > cap) return false;
@@ -341,7 +347,7 @@ __attribute__((target("avx2"))) bool collect_nonzero_avx2(const unsigned* w, siz
     }
 #undef GNNHIP_ZEROS_OF
     *count = c;
-    return collect_nonzero(w, i, words, cap, idx, val, count);
+    return collect_nonzero(w, i, words, cap, idx, val, count, starts);
 }
 
 // A staged upload leaves the pinned buffer through a kernel, not through hipMemcpyAsync: the runtime hands copies of
@@ -394,28 +400,20 @@ __global__ __launch_bounds__(kStageBlock) void stage_copy_pieces_kernel(StagePie
     for (size_t i = (size_t)blockIdx.x * kStageBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kStageBlock) dst[i] = src[i];
 }
 
-constexpr int kExpandBlock = 256;
-constexpr int kExpandTile = 1024;        // 32-bit words of the destination per workgroup
 
 // dst[0..n) = 0 except dst[idx[i]] = val[i], idx ascending: a workgroup builds its tile of the destination in
-// LDS (zeros, then the entries that fall into it, found by bisection) and writes it out whole.
-__global__ __launch_bounds__(kExpandBlock) void expand_pairs_kernel(unsigned* __restrict__ dst, size_t n, const unsigned* __restrict__ idx,
-                                                                    const unsigned* __restrict__ val, int count)
+// LDS (zeros, then the entries that fall into it: numbers starts[tile] .. starts[tile + 1] - 1) and writes it out
+// whole.  starts, idx and val are read where the host left them, in pinned memory: two trips over the bus per
+// workgroup, no copy ahead of the kernel.
+__global__ __launch_bounds__(kExpandBlock) void expand_pairs_kernel(unsigned* __restrict__ dst, size_t n, const unsigned* __restrict__ starts,
+                                                                    const unsigned* __restrict__ idx, const unsigned* __restrict__ val)
 {
     __shared__ unsigned tile[kExpandTile];
     const size_t base = (size_t)blockIdx.x * kExpandTile;
+    const unsigned a = starts[blockIdx.x], b = starts[blockIdx.x + 1];
     for (int i = threadIdx.x; i < kExpandTile; i += kExpandBlock) tile[i] = 0u;
     __syncthreads();
-    int lo = 0, hi = count;                              // first entry with idx >= base
-    while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if ((size_t)idx[mid] < base) lo = mid + 1; else hi = mid;
-    }
-    for (int i = lo + threadIdx.x; i < count; i += kExpandBlock) {
-        const size_t at = idx[i];
-        if (at >= base + kExpandTile) break;
-        tile[at - base] = val[i];
-    }
+    for (unsigned i = a + threadIdx.x; i < b; i += kExpandBlock) tile[idx[i] - base] = val[i];
     __syncthreads();
     for (int i = threadIdx.x; i < kExpandTile; i += kExpandBlock)
         if (base + i < n) dst[base + i] = tile[i];
@@ -502,7 +500,8 @@ int gnnhip_memcpy_h2d_sparse32(void* dst_device, const void* src_host, size_t wo
 {
     constexpr size_t kMinWords = 16384;                  // below this the plain copy is one short DMA anyway
     const size_t cap = words / 16;                       // non-zero words beyond this: the plain copy
-    if (words < kMinWords || cap * 8 > kStagingHalf || words >= ((size_t)1 << 32))
+    const size_t tiles = (words + kExpandTile - 1) / kExpandTile;
+    if (words < kMinWords || cap * 8 + (tiles + 1) * 4 > kStagingHalf || words >= ((size_t)1 << 32))
         return gnnhip_memcpy_h2d(dst_device, src_host, words * 4, stream);
     GNNHIP_REQUIRE(dst_device && src_host, "null pointer in memcpy_h2d_sparse32");
     if (int rc = require_ready()) return rc;
@@ -511,26 +510,22 @@ int gnnhip_memcpy_h2d_sparse32(void* dst_device, const void* src_host, size_t wo
     {
         Runtime& r = rt();
         std::lock_guard<std::mutex> lock(r.mu);
-        if (int rc = staging_slot(r, s, cap * 8, &slot)) return rc;
+        if (int rc = staging_slot(r, s, cap * 8 + (tiles + 1) * 4, &slot)) return rc;
     }
     if (!slot) return gnnhip_memcpy_h2d(dst_device, src_host, words * 4, stream);
     // the slot belongs to this call from here on: scan without the lock
     const unsigned* w = static_cast<const unsigned*>(src_host);
     unsigned* idx = reinterpret_cast<unsigned*>(slot);
     unsigned* val = idx + cap;
+    unsigned* starts = val + cap;
     size_t count = 0;
-    const bool few = __builtin_cpu_supports("avx2") ? collect_nonzero_avx2(w, words, cap, idx, val, &count)
-                                                    : collect_nonzero(w, 0, words, cap, idx, val, &count);
+    const bool few = __builtin_cpu_supports("avx2") ? collect_nonzero_avx2(w, words, cap, idx, val, &count, starts)
+                                                    : collect_nonzero(w, 0, words, cap, idx, val, &count, starts);
     if (!few) return gnnhip_memcpy_h2d(dst_device, src_host, words * 4, stream);
-    memmove(idx + count, val, count * 4);                // indices and values back to back: one copy
-    void* dev = nullptr;
-    if (int rc = stream_scratch_slot(s, 6, (count ? count : 1) * 8, &dev)) return rc;
-    if (count)
-        if (int rc = stage_copy(dev, slot, count * 8, s)) return rc;
-    const unsigned* d_idx = static_cast<const unsigned*>(dev);
-    const unsigned grid = (unsigned)((words + kExpandTile - 1) / kExpandTile);
-    hipLaunchKernelGGL(expand_pairs_kernel, dim3(grid), dim3(kExpandBlock), 0, s, static_cast<unsigned*>(dst_device), words, d_idx,
-                       d_idx + count, (int)count);
+    starts[tiles] = (unsigned)count;
+    // the kernel reads the slot in place; the slot is not reused before the stream has run past it
+    hipLaunchKernelGGL(expand_pairs_kernel, dim3((unsigned)tiles), dim3(kExpandBlock), 0, s, static_cast<unsigned*>(dst_device), words,
+                       starts, idx, val);
     GNNHIP_LAUNCH_CHECK("expand_pairs");
     return GNNHIP_OK;
 }
