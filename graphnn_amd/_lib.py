@@ -43,6 +43,7 @@ SIGNATURES = {
     "gnnhip_csr_group_i32": [_I, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P],
     "gnnhip_csr_group_both_i32": [_I, _I, _P, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_csr_consecutive_rows_f32": [_I, _P, _I, _P, _P, _P],
+    "gnnhip_csr_consecutive_rows_host_f32": [_I, _P, _I, _P, _P, _P, _P],
     "gnnhip_csr_transpose_f32": [_I, _I, _I, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_gemm_f32": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P],
     "gnnhip_gemm_tn_batch_f32": [_I, _P, _P, _P, _P, _P, _P, _P, _F, _F, _P, _P, _P],

@@ -191,6 +191,8 @@ struct HubPlan {
 };
 int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
                 const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan = false, bool relu_in = false);
+// runtime.hip: host bytes placed in the stream's pinned staging buffer for a kernel to read in place (null: not to be had)
+int stage_in_pinned(hipStream_t s, const void* src_host, size_t bytes, const void** pinned);
 // spmm.hip: C = alpha*A*B + beta*C on stream s (A is [m,k]); reuse_plan as for hub_prepass
 int spmm_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
                   const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan = false);

@@ -421,6 +421,27 @@ __global__ __launch_bounds__(kExpandBlock) void expand_pairs_kernel(unsigned* __
 
 }  // namespace
 
+namespace gnnhip {
+
+// bytes of host memory placed in the stream's pinned staging buffer, for a kernel of that stream to read in place;
+// *pinned stays valid until the stream has run everything queued behind this call's next launch.  *pinned = null
+// where that cannot be had (no pinned memory, or more than the buffer takes): the caller copies instead.
+int stage_in_pinned(hipStream_t s, const void* src_host, size_t bytes, const void** pinned)
+{
+    *pinned = nullptr;
+    if (bytes == 0 || bytes > kStagingHalf) return GNNHIP_OK;
+    Runtime& r = rt();
+    std::lock_guard<std::mutex> lock(r.mu);
+    char* slot = nullptr;
+    if (int rc = staging_slot(r, s, bytes, &slot)) return rc;
+    if (!slot) return GNNHIP_OK;
+    memcpy(slot, src_host, bytes);
+    *pinned = slot;
+    return GNNHIP_OK;
+}
+
+}  // namespace gnnhip
+
 extern "C" {
 
 int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream)

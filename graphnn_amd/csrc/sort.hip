@@ -568,13 +568,19 @@ __global__ __launch_bounds__(kSmallBlock) void csr_group_small_kernel(int rows, 
 }
 
 // col_idx[j] = j and val[j] = 1 (or 1 / row length) for j in [row_ptr[i], row_ptr[i+1]): a wavefront per row
+// (row_ptr may be pinned host memory: then row_ptr_out, device memory, receives a copy for the kernels that follow)
 __global__ __launch_bounds__(kBlock) void consecutive_rows_kernel(int rows, const int* __restrict__ row_ptr, int average,
-                                                                  int* __restrict__ col_idx, float* __restrict__ val)
+                                                                  int* __restrict__ col_idx, float* __restrict__ val,
+                                                                  int* __restrict__ row_ptr_out)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const long long row = ((long long)blockIdx.x * kBlock + threadIdx.x) / kWave;
     if (row >= rows) return;
     const int a = row_ptr[row], b = row_ptr[row + 1];
+    if (row_ptr_out && lane == 0) {
+        row_ptr_out[row] = a;
+        if (row == rows - 1) row_ptr_out[rows] = b;
+    }
     const float w = (average && b > a) ? (float)(1.0 / (double)(b - a)) : 1.0f;       // as the reference: double divide, then narrowed
     for (int j = a + lane; j < b; j += kWave) {
         col_idx[j] = j;
@@ -701,7 +707,29 @@ int gnnhip_csr_consecutive_rows_f32(int rows, const int* row_ptr, int average, i
     GNNHIP_REQUIRE(row_ptr && col_idx && val, "null array in csr_consecutive_rows");
     if (int rc = require_ready()) return rc;
     const unsigned grid = (unsigned)(((long long)rows * kWave + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL(consecutive_rows_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), rows, row_ptr, average, col_idx, val);
+    hipLaunchKernelGGL(consecutive_rows_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), rows, row_ptr, average, col_idx, val,
+                       static_cast<int*>(nullptr));
+    GNNHIP_LAUNCH_CHECK("consecutive_rows");
+    return GNNHIP_OK;
+}
+
+int gnnhip_csr_consecutive_rows_host_f32(int rows, const int* offsets_host, int average, int* row_ptr, int* col_idx, float* val, void* stream)
+{
+    GNNHIP_REQUIRE(rows >= 0, "negative row count in csr_consecutive_rows_host");
+    GNNHIP_REQUIRE(offsets_host && row_ptr, "null row pointers in csr_consecutive_rows_host");
+    GNNHIP_REQUIRE(offsets_host[rows] == 0 || (col_idx && val), "null array in csr_consecutive_rows_host");
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    const void* pinned = nullptr;
+    if (rows > 0 && offsets_host[rows] > 0)
+        if (int rc = stage_in_pinned(s, offsets_host, sizeof(int) * ((size_t)rows + 1), &pinned)) return rc;
+    if (!pinned) {
+        if (int rc = gnnhip_memcpy_h2d(row_ptr, offsets_host, sizeof(int) * ((size_t)rows + 1), stream)) return rc;
+        return (rows > 0 && offsets_host[rows] > 0) ? gnnhip_csr_consecutive_rows_f32(rows, row_ptr, average, col_idx, val, stream) : GNNHIP_OK;
+    }
+    const unsigned grid = (unsigned)(((long long)rows * kWave + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(consecutive_rows_kernel, dim3(grid), dim3(kBlock), 0, s, rows, static_cast<const int*>(pinned), average, col_idx, val,
+                       row_ptr);
     GNNHIP_LAUNCH_CHECK("consecutive_rows");
     return GNNHIP_OK;
 }

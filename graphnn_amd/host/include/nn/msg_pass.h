@@ -144,9 +144,8 @@ inline void consecutive_rows_on_device(GraphStruct* graph, std::vector<int>& off
     for (int q = last + 1; q <= B; ++q) offsets[q] = nodes;
     out.Reshape({(size_t)B, (size_t)graph->num_nodes});
     out.ResizeSp(nodes, B + 1);
-    GNN_HIP(gnnhip_memcpy_h2d(out.data->row_ptr, offsets.data(), sizeof(int) * ((size_t)B + 1), GpuHandle::Stream()));
-    if (nodes > 0)
-        GNN_HIP(gnnhip_csr_consecutive_rows_f32(B, out.data->row_ptr, average ? 1 : 0, out.data->col_idx, out.data->val, GpuHandle::Stream()));
+    GNN_HIP(gnnhip_csr_consecutive_rows_host_f32(B, offsets.data(), average ? 1 : 0, out.data->row_ptr, out.data->col_idx, out.data->val,
+                                                 GpuHandle::Stream()));
 }
 // The device groups a batch in one launch (up to 16 workgroups, each a run of the rows) when a run's counters
 // (4 bytes per row) and the slots of all pairs (2.35 bytes each, with the lists and one bitmap) fit 160 KB of

@@ -556,6 +556,18 @@ def csr_consecutive_rows(row_ptr, average=False):
     return col_idx, val
 
 
+def csr_consecutive_rows_host(offsets, device, average=False):
+    """(row_ptr, col_idx, val) on the device from the row offsets in a host int32 array"""
+    offsets = np.ascontiguousarray(offsets, np.int32)
+    rows, n = offsets.size - 1, int(offsets[-1])
+    row_ptr = torch.empty(rows + 1, dtype=torch.int32, device=device)
+    col_idx = torch.empty(n, dtype=torch.int32, device=device)
+    val = torch.empty(n, dtype=torch.float32, device=device)
+    check(_lib().gnnhip_csr_consecutive_rows_host_f32(rows, ctypes.c_void_p(offsets.ctypes.data), int(average), _i32(row_ptr, "row_ptr"),
+                                                      _i32(col_idx, "col_idx") if n else None, _f32(val, "val") if n else None, _stream()))
+    return row_ptr, col_idx, val
+
+
 def csr_transpose(row_ptr, col_idx, val, m, k):
     nnz = col_idx.numel()
     dev = row_ptr.device

@@ -120,6 +120,11 @@ int gnnhip_csr_group_i32(int rows, int n, const int* key, int key_stride, const 
  *      (examples/graph_classification/include/nn_common.h:36-105).  row_ptr [rows+1] is on the device already (the
  *      subgraph offsets, which the host knows); col_idx and val have row_ptr[rows] entries. */
 int gnnhip_csr_consecutive_rows_f32(int rows, const int* row_ptr, int average, int* col_idx, float* val, void* stream);
+/* ---- the same operand of SubgraphMsgPass (src/nn/msg_pass.cpp:156-177) from the subgraph offsets in HOST memory
+ *      (offsets_host [rows+1], free again when the call returns): row_ptr [rows+1] on the device receives them, col_idx
+ *      and val the entries, in one launch. */
+int gnnhip_csr_consecutive_rows_host_f32(int rows, const int* offsets_host, int average, int* row_ptr, int* col_idx, float* val,
+                                         void* stream);
 
 /* ---- the n pairs (x, y) grouped both ways at once, values 1: row i of (row_ptr, col_idx, val) lists the x of the
  *      pairs with y = i, which is gnnhip_csr_group_i32(rows, n, y, .., x, .., 0, ..), the operand of

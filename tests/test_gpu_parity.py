@@ -1782,6 +1782,12 @@ def test_device_csr_of_consecutive_rows(gpu, oracle, average):
     want = oracle.csr_subgraph(sizes.size, sid, nid, average)
     ci, v = ops.csr_consecutive_rows(_t(want[0], gpu), average)
     assert np.array_equal(_n(ci), want[1]) and np.array_equal(_n(v), want[2])
+    # the same from the offsets in host memory, in one launch; and a batch without nodes
+    got = ops.csr_consecutive_rows_host(want[0], gpu, average)
+    for g, w_ in zip(got, want):
+        assert np.array_equal(_n(g), w_)
+    rp, ci, v = ops.csr_consecutive_rows_host(np.zeros(6, np.int32), gpu, average)
+    assert not _n(rp).any() and ci.numel() == 0
 
 
 @pytest.mark.parametrize("rows,n", [(7450, 16382), (300, 40_000), (50_000, 70_000), (9, 1), (5, 0)])
