@@ -11,6 +11,9 @@
  *     Calls are asynchronous on that stream except where stated.
  *   - the library keeps no caller pointer after the call's work on the stream
  *     has finished; outputs are caller-allocated.
+ *   - one host thread at a time feeds a stream: the scratch and the pinned
+ *     staging buffers that the library keeps per stream belong to the call in
+ *     progress.  Threads that work side by side use a stream each.
  *
  * Each declaration cites the reference interface it stands in for
  * (paths relative to the graphnn source tree).
