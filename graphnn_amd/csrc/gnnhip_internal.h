@@ -185,12 +185,16 @@ constexpr int kHubThreshold = 64;      // rows with more entries are summed by t
 constexpr int kHubChunk = 2048;        // entries per partial sum of the pre-pass
 constexpr int kHubMinRows = 32768;     // smaller matrices skip the pre-pass: its launches would cost more than a long row
 struct HubPlan {
-    const int* row_slot;               // [m], defined for rows longer than kHubThreshold only; -1: not summed
+    const int* row_slot;               // [m], defined for rows longer than the pass's threshold only; -1: not summed
     const float* agg;                  // [slots][ld]
     int ld;
 };
+// threshold / chunk_len: rows with more entries than `threshold` are summed, cut into chunks of `chunk_len`
+// (the consumer must apply the same threshold when it looks a row up in row_slot); max_hubs >= 0: the caller's
+// bound on the number of such rows
 int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
-                const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan = false, bool relu_in = false);
+                const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan = false, bool relu_in = false,
+                int threshold = kHubThreshold, int chunk_len = kHubChunk, long long max_hubs = -1);
 // runtime.hip: host bytes placed in the stream's pinned staging buffer for a kernel to read in place (null: not to be had)
 int stage_in_pinned(hipStream_t s, const void* src_host, size_t bytes, const void** pinned);
 // spmm.hip: C = alpha*A*B + beta*C on stream s (A is [m,k]); reuse_plan as for hub_prepass
@@ -217,7 +221,7 @@ struct PiecesOperand {
     bool plan_reused;
 };
 int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                     const float* B, int ldb, hipStream_t s, bool reuse_plan, PiecesOperand* out);
+                     const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan, PiecesOperand* out);
 int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
                          const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan);
 

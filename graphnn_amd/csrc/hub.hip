@@ -32,7 +32,7 @@ constexpr int kRowsPerBlock = 1024;          // count / fill: four consecutive r
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kFillScanBlocks = 4096;       // up to this many workgroups (4M rows) fill does the scan itself
 
-__device__ __forceinline__ int hub_chunks(int deg) { return (deg + kHubChunk - 1) / kHubChunk; }
+__device__ __forceinline__ int hub_chunks(int deg, int chunk) { return (deg + chunk - 1) / chunk; }
 
 // Exclusive prefix over the 256 lanes of the workgroup, in lane order; *total receives the sum.
 __device__ __forceinline__ int block_exclusive_scan(int v, int* sh, int* total)
@@ -58,7 +58,8 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* sh, int* total)
 }
 
 __global__ __launch_bounds__(kBlock) void hub_count_kernel(int m, const int* __restrict__ row_ptr,
-                                                            int* __restrict__ block_hubs, int* __restrict__ block_chunks)
+                                                            int* __restrict__ block_hubs, int* __restrict__ block_chunks,
+                                                            int threshold, int chunk_len)
 {
     __shared__ int sh[2][kWavesPerBlock];
     const long long r0 = (long long)blockIdx.x * kRowsPerBlock + threadIdx.x * 4;
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(kBlock) void hub_count_kernel(int m, const int* __r
         const long long r = r0 + i;
         if (r < m) {
             const int deg = row_ptr[r + 1] - row_ptr[r];
-            if (deg > kHubThreshold) { ++hubs; chunks += hub_chunks(deg); }
+            if (deg > threshold) { ++hubs; chunks += hub_chunks(deg, chunk_len); }
         }
     }
     hubs = wave_sum_i(hubs);
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(kBlock) void hub_fill_kernel(int m, int nb, const i
                                                            int hub_cap, int chunk_cap, int* __restrict__ row_slot,
                                                            int* __restrict__ hub_row, int* __restrict__ hub_chunk0,
                                                            int* __restrict__ chunk_hub, int* __restrict__ hub_done,
-                                                           int* __restrict__ counts)
+                                                           int* __restrict__ counts, int threshold, int chunk_len)
 {
     __shared__ int sh[kWavesPerBlock];
     __shared__ int base_sh[2];
@@ -157,15 +158,15 @@ __global__ __launch_bounds__(kBlock) void hub_fill_kernel(int m, int nb, const i
         const long long r = r0 + i;
         deg[i] = 0;
         if (r < m) deg[i] = row_ptr[r + 1] - row_ptr[r];
-        if (deg[i] > kHubThreshold) { ++hubs; chunks += hub_chunks(deg[i]); }
+        if (deg[i] > threshold) { ++hubs; chunks += hub_chunks(deg[i], chunk_len); }
     }
     int tot;
     int slot = slot0 + block_exclusive_scan(hubs, sh, &tot);
     int chunk = chunk0 + block_exclusive_scan(chunks, sh, &tot);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        if (deg[i] > kHubThreshold) {
-            const int nc = hub_chunks(deg[i]);
+        if (deg[i] > threshold) {
+            const int nc = hub_chunks(deg[i], chunk_len);
             // a hub past the capacity of the buffers keeps slot -1: its consumer sums it in place
             const bool fits = slot < hub_cap && chunk + nc <= chunk_cap;
             row_slot[r0 + i] = fits ? slot : -1;
@@ -209,7 +210,7 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
     const int* __restrict__ counts, int chunk_cap, int n, const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
     const float* __restrict__ val, const float* __restrict__ B, int ldb, int logG,
     const int* __restrict__ hub_row, const int* __restrict__ hub_chunk0, const int* __restrict__ chunk_hub,
-    float* part, int ldp, float* __restrict__ agg, int* hub_done, int relu_in)
+    float* part, int ldp, float* __restrict__ agg, int* hub_done, int relu_in, int chunk_len)
 {
     // relu_in: the rows of B are used as ReLU(B) (a first level that reads msg in place of h0)
     using V = HV<VEC>;
@@ -223,9 +224,9 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
         if (slot < 0) continue;                  // chunk of a hub that did not fit the buffers
         const int row = hub_row[slot];
         const int rb = row_ptr[row], re = row_ptr[row + 1];
-        const int nc = hub_chunks(re - rb);
-        const int cb = rb + (c - hub_chunk0[slot]) * kHubChunk;
-        const int ce = min(cb + kHubChunk, re);
+        const int nc = hub_chunks(re - rb, chunk_len);
+        const int cb = rb + (c - hub_chunk0[slot]) * chunk_len;
+        const int ce = min(cb + chunk_len, re);
         typename V::T acc[ITERS];
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) acc[it] = V::zero();
@@ -319,28 +320,30 @@ inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 template <int VEC, int ITERS>
 void launch_partial(hipStream_t s, const int* counts, int chunk_cap, int n, const int* row_ptr, const int* col_idx,
                     const float* val, const float* B, int ldb, int logG, const int* hub_row, const int* hub_chunk0,
-                    const int* chunk_hub, float* part, int ldp, float* agg, int* hub_done, int relu_in)
+                    const int* chunk_hub, float* part, int ldp, float* agg, int* hub_done, int relu_in, int chunk_len)
 {
     const unsigned grid = kNumCU * 8;
     hipLaunchKernelGGL((hub_partial_kernel<VEC, ITERS>), dim3(grid), dim3(kBlock), 0, s, counts, chunk_cap, n, row_ptr,
-                       col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in);
+                       col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in, chunk_len);
 }
 
 }  // namespace
 
-// Sums the hubs of A (rows longer than kHubThreshold) times B[:, 0..n) into plan->agg.
+// Sums the hubs of A (rows longer than `threshold` entries, cut into chunks of `chunk_len`) times B[:, 0..n) into
+// plan->agg.  max_hubs, when not negative, is the caller's bound on the number of such rows (it sizes the buffers).
 // n <= 1024.  The buffers live in the stream's plan scratch and stay valid until the next
 // hub_prepass on the same stream.
 // reuse_plan: the caller guarantees that the structure of A has not changed since the previous call on
 // this stream with the same arguments (the levels of one forward); the planning launches
 // (count, scan, fill) are then skipped and only the sums are recomputed.
 int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
-                const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan, bool relu_in)
+                const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan, bool relu_in, int threshold, int chunk_len,
+                long long max_hubs)
 {
     plan->row_slot = nullptr;
     plan->agg = nullptr;
     plan->ld = 0;
-    if (m < kHubMinRows || nnz <= kHubThreshold || n > kWave * 16) return GNNHIP_OK;
+    if (m < kHubMinRows || nnz <= threshold || n > kWave * 16) return GNNHIP_OK;
     const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && aligned16(B);
     const int vec = vec4 ? 4 : 1;
     const int units = (n + vec - 1) / vec;
@@ -350,8 +353,9 @@ int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_
     const int ldp = (int)round_up((size_t)n, 4);
 
     const int nb = (m + kRowsPerBlock - 1) / kRowsPerBlock;
-    const long long hub_cap_ll = nnz / (kHubThreshold + 1) + 1;
-    const long long chunk_cap_ll = nnz / kHubChunk + hub_cap_ll + 1;
+    long long hub_cap_ll = nnz / (threshold + 1) + 1;
+    if (max_hubs >= 0 && max_hubs < hub_cap_ll) hub_cap_ll = max_hubs;
+    const long long chunk_cap_ll = nnz / chunk_len + hub_cap_ll + 1;
     const int hub_cap = (int)(hub_cap_ll < m ? hub_cap_ll : m);
     const int chunk_cap = (int)chunk_cap_ll;
 
@@ -379,30 +383,31 @@ int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_
     float* part = reinterpret_cast<float*>(b + o_part);
     float* agg = reinterpret_cast<float*>(b + o_agg);
 
-    struct Memo { hipStream_t s; const int* row_ptr; int m, n; long long nnz; void* base; };
-    static thread_local Memo memo = {nullptr, nullptr, 0, 0, 0, nullptr};
+    struct Memo { hipStream_t s; const int* row_ptr; int m, n; long long nnz; void* base; int threshold, chunk_len, hub_cap; };
+    static thread_local Memo memo = {nullptr, nullptr, 0, 0, 0, nullptr, 0, 0, 0};
     const bool planned = reuse_plan && memo.row_ptr == row_ptr && memo.s == s && memo.m == m && memo.n == n &&
-                         memo.nnz == nnz && memo.base == base;
+                         memo.nnz == nnz && memo.base == base && memo.threshold == threshold && memo.chunk_len == chunk_len &&
+                         memo.hub_cap == hub_cap;
     if (!planned) {
-        hipLaunchKernelGGL(hub_count_kernel, dim3(nb), dim3(kBlock), 0, s, m, row_ptr, bh, bc);
+        hipLaunchKernelGGL(hub_count_kernel, dim3(nb), dim3(kBlock), 0, s, m, row_ptr, bh, bc, threshold, chunk_len);
         if (nb <= kFillScanBlocks) {
             hipLaunchKernelGGL(hub_fill_kernel<true>, dim3(nb), dim3(kBlock), 0, s, m, nb, row_ptr, bh, bc, hub_cap, chunk_cap,
-                               row_slot, hub_row, hub_chunk0, chunk_hub, hub_done, counts);
+                               row_slot, hub_row, hub_chunk0, chunk_hub, hub_done, counts, threshold, chunk_len);
         } else {
             hipLaunchKernelGGL(hub_scan_kernel, dim3(1), dim3(kScanBlock), 0, s, nb, bh, bc, counts);
             hipLaunchKernelGGL(hub_fill_kernel<false>, dim3(nb), dim3(kBlock), 0, s, m, nb, row_ptr, bh, bc, hub_cap, chunk_cap,
-                               row_slot, hub_row, hub_chunk0, chunk_hub, hub_done, counts);
+                               row_slot, hub_row, hub_chunk0, chunk_hub, hub_done, counts, threshold, chunk_len);
         }
-        memo = Memo{s, row_ptr, m, n, nnz, base};
+        memo = Memo{s, row_ptr, m, n, nnz, base, threshold, chunk_len, hub_cap};
     }
     if (vec4) {
-        if (iters <= 1) launch_partial<4, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
-        else if (iters == 2) launch_partial<4, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
-        else launch_partial<4, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
+        if (iters <= 1) launch_partial<4, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
+        else if (iters == 2) launch_partial<4, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
+        else launch_partial<4, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
     } else {
-        if (iters <= 1) launch_partial<1, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
-        else if (iters == 2) launch_partial<1, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
-        else launch_partial<1, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0);
+        if (iters <= 1) launch_partial<1, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
+        else if (iters == 2) launch_partial<1, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
+        else launch_partial<1, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
     }
     GNNHIP_LAUNCH_CHECK("hub_prepass");
     plan->row_slot = row_slot;

@@ -11,9 +11,12 @@
 //
 //   plan     pieces per row -> offsets (scan) -> piece records + keys -> order by first column ->
 //            entries copied in piece order (a CSR matrix whose rows are the pieces)
-//   sums     one lane group per piece, entries read front to back; the sums are stored in the order they are formed
-//   combine  C = P * sums + beta * C, P the 0/1 matrix that picks the pieces of a row in piece order
-//            (the plain row-group SpMM: rows without entries get beta * C, very long rows its hub pass)
+//   sums     one lane group per piece, entries read front to back; a row of one piece (most rows) gets its
+//            result, beta * C included, straight from here
+//   combine  the other rows: the sums are stored by piece id, so the pieces of a row, and of the rows after it, lie
+//            next to each other; a lane group takes a run of consecutive rows and adds up each row's pieces front
+//            to back (rows without entries get beta * C; rows of more than eight pieces come from the
+//            balanced pass over long rows, run on the 0/1 matrix P that picks the pieces of a row)
 //
 // Every sum is taken in an order fixed by the matrix (no atomics): the result does not depend on scheduling.
 // The plan depends on A only (structure and values) and is reused by the later levels of one forward.
@@ -28,14 +31,16 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kPiece = 32;              // entries per piece
 
-struct PieceRec { int start, end, id; };    // entries [start, end); id = first[row] + index of the piece in its row
+// entries [start, end); id = first[row] + index of the piece in its row; row: the row when the piece is all of it
+// and holds entries (then its sum is the row's result), else -1
+struct PieceRec { int start, end, id, row; };
 
 __device__ __forceinline__ int pieces_of(int deg) { return (deg + kPiece - 1) / kPiece; }
 
 // counts[r] = pieces of row r (counts[m] = 0, so that the scan leaves the total there).  The host's entry count
 // `cap` sizes every array of the plan; should the matrix hold more entries than that, a row that reaches past
 // entry `cap` (the last rows) is one piece whatever its length: no entries are copied for it, and
-// piece_tail_kernel forms its sum from the CSR arrays.
+// piece_tail_kernel forms the row's result from the CSR arrays.
 __global__ __launch_bounds__(kBlock) void piece_count_kernel(int m, const int* __restrict__ row_ptr, int cap, int* __restrict__ counts)
 {
     for (long long r = (long long)blockIdx.x * kBlock + threadIdx.x; r <= m; r += (long long)gridDim.x * kBlock) {
@@ -57,7 +62,7 @@ __global__ __launch_bounds__(kBlock) void piece_fill_kernel(int m, long long slo
     const int total = first[m];
     for (long long id = (long long)blockIdx.x * kBlock + threadIdx.x; id < slots; id += (long long)gridDim.x * kBlock) {
         if (id >= total) {
-            rec[id] = PieceRec{0, 0, (int)id};
+            rec[id] = PieceRec{0, 0, (int)id, -1};
             keys[id] = 0xFFFFu;
             continue;
         }
@@ -71,7 +76,7 @@ __global__ __launch_bounds__(kBlock) void piece_fill_kernel(int m, long long slo
         const int rb = row_ptr[row], re = row_ptr[row + 1];
         const int start = rb + k * kPiece;
         const int end = re <= cap ? min(start + kPiece, re) : start;     // a row past the host's count: an empty stand-in
-        rec[id] = PieceRec{start, end, (int)id};
+        rec[id] = PieceRec{start, end, (int)id, (end > start && first[row + 1] - first[row] == 1) ? row : -1};
         keys[id] = ((unsigned)col_idx[start] >> shift) & 0xFFFFu;
     }
 }
@@ -85,16 +90,20 @@ __global__ __launch_bounds__(kBlock) void piece_permute_kernel(long long slots, 
 }
 
 // lens[i] = entries of the i-th piece in order (lens[slots] = 0, so that the scan leaves the total there);
-// where[id] = i, the place of piece id in the order; ones[i] = 1 (the values of the matrix that picks pieces)
+// where[i] = i and ones[i] = 1: the matrix that picks the pieces of a row (the sums are stored by piece id, so the
+// pieces of a row lie next to each other and the combining pass reads them front to back);
+// target[i]: where the sum of the i-th piece in order goes: the row r >= 0 when the piece is all of that row,
+// else -1 - id, its place among the partial sums
 __global__ __launch_bounds__(kBlock) void piece_place_kernel(long long slots, const PieceRec* __restrict__ ordered, int* __restrict__ lens,
-                                                             int* __restrict__ where, float* __restrict__ ones)
+                                                             int* __restrict__ where, float* __restrict__ ones, int* __restrict__ target)
 {
     for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i <= slots; i += (long long)gridDim.x * kBlock) {
         if (i == slots) { lens[i] = 0; continue; }
         const PieceRec r = ordered[i];
         lens[i] = r.end - r.start;
-        where[r.id] = (int)i;
+        where[i] = (int)i;
         ones[i] = 1.f;
+        target[i] = r.row >= 0 ? r.row : -1 - r.id;
     }
 }
 
@@ -117,7 +126,7 @@ __global__ __launch_bounds__(kBlock) void piece_gather_kernel(const int* __restr
 #pragma unroll
         for (int u = 0; u < kTurn; ++u) {
             const bool live = i0 + u < total;
-            r[u] = live ? ordered[i0 + u] : PieceRec{0, 0, 0};
+            r[u] = live ? ordered[i0 + u] : PieceRec{0, 0, 0, -1};
             dst[u] = live ? at[i0 + u] : 0;
         }
 #pragma unroll
@@ -139,6 +148,7 @@ template <> struct PV<4> {
     static __device__ __forceinline__ T load(const float* p) { return *reinterpret_cast<const float4*>(p); }
     static __device__ __forceinline__ void store(float* p, T v) { *reinterpret_cast<float4*>(p) = v; }
     static __device__ __forceinline__ void fma(T& a, float s, T x) { a.x += s * x.x; a.y += s * x.y; a.z += s * x.z; a.w += s * x.w; }
+    static __device__ __forceinline__ T axpby(T a, float b, T c) { return make_float4(a.x + b * c.x, a.y + b * c.y, a.z + b * c.z, a.w + b * c.w); }
 };
 template <> struct PV<1> {
     using T = float;
@@ -146,6 +156,7 @@ template <> struct PV<1> {
     static __device__ __forceinline__ T load(const float* p) { return *p; }
     static __device__ __forceinline__ void store(float* p, T v) { *p = v; }
     static __device__ __forceinline__ void fma(T& a, float s, T x) { a += s * x; }
+    static __device__ __forceinline__ T axpby(T a, float b, T c) { return a + b * c; }
 };
 
 // One lane group (G lanes) per piece, pieces taken in order; die x (workgroups x, x + 8, ...) walks the
@@ -154,10 +165,13 @@ template <> struct PV<1> {
 // workgroup lets them drift apart and costs a quarter more fetched bytes).  The launch covers the host's bound
 // on the number of pieces; workgroups past the real count leave at once.  Inner loop as in the row-group SpMM:
 // the group reads G column indices and values at once and hands them round by shuffle, four gathers in flight.
+// The sum of a piece that is all of its row goes to C (as sum + beta * C, what the combining pass would make of
+// it), the others to the place of their piece id among the partial sums.
 template <int VEC, int ITERS>
 __global__ __launch_bounds__(kBlock) void piece_sum_kernel(
     const int* __restrict__ count, int n, float alpha, const int* __restrict__ at, const int* __restrict__ col_idx, const float* __restrict__ val,
-    const float* __restrict__ B, int ldb, float* __restrict__ part, int ldp, int logG)
+    const float* __restrict__ B, int ldb, float* __restrict__ part, int ldp, int logG, const int* __restrict__ target, float beta,
+    float* __restrict__ C, int ldc)
 {
     using V = PV<VEC>;
     const int G = 1 << logG;
@@ -203,22 +217,31 @@ __global__ __launch_bounds__(kBlock) void piece_sum_kernel(
                 }
             }
         }
+        const int row = target[i];
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
             const int col0 = (sub + it * G) * VEC;
-            if (col0 < n) V::store(part + (size_t)i * ldp + col0, acc[it]);
+            if (col0 >= n) continue;
+            if (row < 0) {
+                V::store(part + (size_t)(-1 - row) * ldp + col0, acc[it]);
+            } else {
+                float* dst = C + (size_t)row * ldc + col0;
+                if (beta == 0.f) V::store(dst, acc[it]);
+                else V::store(dst, V::axpby(acc[it], beta, V::load(dst)));
+            }
         }
     }
 }
 
-// The rows that reach past entry `cap` (none when the host's entry count is the matrix's own): the sum of the row,
-// alpha * A[row] * B, goes where the row's one stand-in piece has its place among the partial sums.  Rows are
-// taken from the last one down, a lane group each; the first row that ends inside the plan ends the walk.
+// The rows that reach past entry `cap` (none when the host's entry count is the matrix's own): such a row has one
+// stand-in piece without entries, so neither the sums nor the combining pass write it; its result,
+// alpha * A[row] * B + beta * C[row], is formed here.  Rows are taken from the last one down, a lane group each;
+// the first row that ends inside the plan ends the walk.
 template <int VEC, int ITERS>
 __global__ __launch_bounds__(kBlock) void piece_tail_kernel(int m, int n, float alpha, const int* __restrict__ row_ptr, int cap,
                                                             const int* __restrict__ col_idx, const float* __restrict__ val,
-                                                            const float* __restrict__ B, int ldb, const int* __restrict__ first,
-                                                            const int* __restrict__ where, float* __restrict__ part, int ldp, int logG)
+                                                            const float* __restrict__ B, int ldb, float beta, float* __restrict__ C,
+                                                            int ldc, int logG)
 {
     using V = PV<VEC>;
     const int G = 1 << logG;
@@ -242,11 +265,83 @@ __global__ __launch_bounds__(kBlock) void piece_tail_kernel(int m, int n, float 
                 if (col0 < n) V::fma(acc[it], v, V::load(B + (size_t)c * ldb + col0));
             }
         }
-        float* dst = part + (size_t)where[first[row]] * ldp;
+        float* dst = C + (size_t)row * ldc;
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
             const int col0 = (sub + it * G) * VEC;
-            if (col0 < n) V::store(dst + col0, acc[it]);
+            if (col0 >= n) continue;
+            if (beta == 0.f) V::store(dst + col0, acc[it]);
+            else V::store(dst + col0, V::axpby(acc[it], beta, V::load(dst + col0)));
+        }
+    }
+}
+
+// C[row] = sum of the row's partial sums + beta * C[row] for the rows of no piece or of several; a row of one piece
+// has its result already.  part holds the sums by piece id: row r owns part[first[r] .. first[r + 1]).  A lane group
+// takes kRun consecutive rows, whose pieces are one contiguous stretch of part, and adds each row's pieces in
+// piece order, eight loads in flight.  A row of more than kCombineLong pieces takes its sum from the balanced
+// pass (hub_slot / hub_agg) when that pass has one for it: on a power-law matrix the rows of many pieces sit next
+// to each other, and summed here they kept an eighth of the wavefronts busy for the whole launch.
+constexpr int kRun = 8;
+constexpr int kCombineLong = 8;         // pieces; the balanced pass cuts such rows into chunks of kCombineChunk pieces
+constexpr int kCombineChunk = 256;
+template <int VEC, int ITERS>
+__global__ __launch_bounds__(kBlock) void piece_combine_kernel(
+    int m, int n, const int* __restrict__ first, const float* __restrict__ part, int ldp, float beta, float* __restrict__ C, int ldc,
+    int logG, const int* __restrict__ hub_slot, const float* __restrict__ hub_agg, int hub_ld)
+{
+    using V = PV<VEC>;
+    constexpr int kFlight = 8;
+    const int G = 1 << logG;                       // at least 8 lanes (the route's narrowest operand): a lane per row of the run
+    const int sub = threadIdx.x & (G - 1);
+    const int grp = threadIdx.x >> logG;
+    const int ngroups = kBlock >> logG;
+    const long long row0 = ((long long)blockIdx.x * ngroups + grp) * kRun;
+    if (row0 >= m) return;
+    // lane j < kRun of the group holds the bounds of row row0 + j
+    const long long mine = row0 + (sub < kRun ? sub : 0);
+    const int my_b = first[mine < m ? mine : m], my_e = first[mine + 1 < m ? mine + 1 : m];
+    const int rows = (int)((long long)m - row0 < kRun ? (long long)m - row0 : kRun);
+    for (int j = 0; j < rows; ++j) {
+        const int b = __shfl(my_b, j, G), e = __shfl(my_e, j, G);
+        const int cnt = e - b;
+        if (cnt == 1) continue;
+        const long long row = row0 + j;
+        typename V::T acc[ITERS];
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) acc[it] = V::zero();
+        int hslot = -1;
+        if (hub_slot && cnt > kCombineLong) hslot = hub_slot[row];
+        if (hslot >= 0) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int col0 = (sub + it * G) * VEC;
+                if (col0 < n) acc[it] = V::load(hub_agg + (size_t)hslot * hub_ld + col0);
+            }
+        } else {
+            for (int p = b; p < e; p += kFlight) {
+#pragma unroll
+                for (int it = 0; it < ITERS; ++it) {
+                    const int col0 = (sub + it * G) * VEC;
+                    if (col0 < n) {
+                        typename V::T x[kFlight];
+#pragma unroll
+                        for (int u = 0; u < kFlight; ++u)
+                            x[u] = (p + u < e) ? V::load(part + (size_t)(p + u) * ldp + col0) : V::zero();
+#pragma unroll
+                        for (int u = 0; u < kFlight; ++u)
+                            if (p + u < e) V::fma(acc[it], 1.f, x[u]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int col0 = (sub + it * G) * VEC;
+            if (col0 >= n) continue;
+            float* dst = C + (size_t)row * ldc + col0;
+            if (beta == 0.f) V::store(dst, acc[it]);
+            else V::store(dst, V::axpby(acc[it], beta, V::load(dst)));
         }
     }
 }
@@ -274,13 +369,14 @@ inline long long pieces_degree()
 
 // The partial sums alpha * (piece of A) * B of every piece, in column order, and the matrix P that picks the pieces of
 // each row (out->first / where / ones: CSR arrays of P [m, out->slots], out->part: the sums, row stride out->ld);
-// A * B is P * part.  GNNHIP_EUNSUPPORTED (nothing launched) where the caller keeps its own route.
+// A * B is P * part.  The rows of exactly one piece are finished here (C[row] = sum + beta * C[row]); the caller
+// combines the others.  GNNHIP_EUNSUPPORTED (nothing launched) where the caller keeps its own route.
 int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                     const float* B, int ldb, hipStream_t s, bool reuse_plan, PiecesOperand* out)
+                     const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan, PiecesOperand* out)
 {
     const long long deg = pieces_degree();
     if (deg <= 0 || m < kHubMinRows || nnz < deg * (long long)m || nnz >= (1ll << 31) - 64) return GNNHIP_EUNSUPPORTED;
-    const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && aligned16(B);
+    const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && aligned16(B) && aligned16(C);
     const int vec = vec4 ? 4 : 1;
     const int units = (n + vec - 1) / vec;
     // a lane group covers at most 64 x 4 column units (wider operands stay with the caller's route, which cuts them into slabs)
@@ -303,6 +399,7 @@ int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int*
     auto carve = [&](size_t bytes) { const size_t o = off; off = round_up_p(off + bytes, 256); return o; };
     const size_t o_first = carve(sizeof(int) * ((size_t)m + 1)), o_where = carve(sizeof(int) * (size_t)slots);
     const size_t o_at = carve(sizeof(int) * ((size_t)slots + 1)), o_ones = carve(sizeof(float) * (size_t)slots);
+    const size_t o_target = carve(sizeof(int) * (size_t)slots);
     const size_t o_col = carve(sizeof(int) * (size_t)nnz), o_val = carve(sizeof(float) * (size_t)nnz);
     const size_t longest = (size_t)(slots + 1 > (long long)m + 1 ? slots + 1 : (long long)m + 1);
     const size_t o_seg = carve(sizeof(int) * (longest / 4096 + 2 + radix_seg_ints(slots)));
@@ -319,6 +416,7 @@ int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int*
     int* where = reinterpret_cast<int*>(b + o_where);
     int* at = reinterpret_cast<int*>(b + o_at);
     float* ones = reinterpret_cast<float*>(b + o_ones);
+    int* target = reinterpret_cast<int*>(b + o_target);
     int* col_ord = reinterpret_cast<int*>(b + o_col);
     float* val_ord = reinterpret_cast<float*>(b + o_val);
     int* seg = reinterpret_cast<int*>(b + o_seg);
@@ -347,7 +445,7 @@ int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int*
         hipLaunchKernelGGL(piece_permute_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, perm, rec, ordered);
         if (int rc = radix_order_by_digit(keys2, slots, 8, keys, perm, hist, seg, s)) return rc;
         hipLaunchKernelGGL(piece_permute_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, perm, ordered, rec);
-        hipLaunchKernelGGL(piece_place_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, rec, at, where, ones);
+        hipLaunchKernelGGL(piece_place_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, rec, at, where, ones, target);
         if (int rc = exclusive_scan_i32(at, slots + 1, seg, s)) return rc;
         hipLaunchKernelGGL(piece_gather_kernel, dim3(egrid), dim3(kBlock), 0, s, first + m, rec, at, col_idx, val, col_ord, val_ord);
         GNNHIP_LAUNCH_CHECK("spmm_pieces plan");
@@ -358,7 +456,7 @@ int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int*
     const unsigned sgrid = (unsigned)(((slots + kNumXCD - 1) / kNumXCD + 1 + sum_groups - 1) / sum_groups) * kNumXCD;
 #define GNNHIP_PIECES_LAUNCH(V, I)                                                                                               \
     hipLaunchKernelGGL((piece_sum_kernel<V, I>), dim3(sgrid), dim3(kBlock), 0, s, first + m, n, alpha, at, col_ord, val_ord, B, ldb, \
-                       part, ldp, logG)
+                       part, ldp, logG, target, beta, C, ldc)
     if (vec4) {
         if (iters <= 1) GNNHIP_PIECES_LAUNCH(4, 1);
         else if (iters == 2) GNNHIP_PIECES_LAUNCH(4, 2);
@@ -370,11 +468,11 @@ int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int*
     }
 #undef GNNHIP_PIECES_LAUNCH
     GNNHIP_LAUNCH_CHECK("spmm_pieces sums");
-    // rows past the host's entry count, if any: their sums go to the place of their stand-in piece
+    // rows past the host's entry count, if any
     const unsigned tgrid = kNumCU * 4;
 #define GNNHIP_PIECES_TAIL(V, I)                                                                                                  \
     hipLaunchKernelGGL((piece_tail_kernel<V, I>), dim3(tgrid), dim3(kBlock), 0, s, m, n, alpha, row_ptr, (int)nnz, col_idx, val, \
-                       B, ldb, first, where, part, ldp, logG)
+                       B, ldb, beta, C, ldc, logG)
     if (vec4) {
         if (iters <= 1) GNNHIP_PIECES_TAIL(4, 1);
         else if (iters == 2) GNNHIP_PIECES_TAIL(4, 2);
@@ -400,10 +498,35 @@ int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const 
                          const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
 {
     PiecesOperand po;
-    if (int rc = spmm_pieces_sums(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, s, reuse_plan, &po)) return rc;
-    // C = P * part + beta * C: row r of P has a one at where[first[r] + j] for each of its pieces j, in piece order.
-    // `slots` stands in for the number of entries of P (an upper bound is all the row-group route needs).
-    return spmm_plain_dispatch(m, (int)po.slots, n, po.slots, 1.f, po.first, po.where, po.ones, po.part, po.ld, beta, C, ldc, s, false);
+    if (int rc = spmm_pieces_sums(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, s, reuse_plan, &po)) return rc;
+    // the rows of very many pieces: the balanced pass over long rows, on P = (first, where, ones) times part
+    // (`slots` stands in for the number of entries of P: an upper bound is all that pass needs)
+    HubPlan hubs;
+    // (a row of more than kCombineLong pieces has more than kCombineLong * kPiece entries: that bounds their number)
+    if (int rc = hub_prepass(m, n, po.slots, po.first, po.where, po.ones, po.part, po.ld, s, &hubs, po.plan_reused, false, kCombineLong,
+                             kCombineChunk, nnz / ((long long)kCombineLong * kPiece + 1) + 1))
+        return rc;
+    const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && aligned16(B) && aligned16(C);
+    const int vec = vec4 ? 4 : 1;
+    const int units = (n + vec - 1) / vec;
+    const int logG = ilog2_ceil_p(units < kWave ? units : kWave);
+    const int iters = (units + (1 << logG) - 1) >> logG;
+    const unsigned grid = (unsigned)(((long long)m + (long long)(kBlock >> logG) * kRun - 1) / ((long long)(kBlock >> logG) * kRun));
+#define GNNHIP_PIECES_COMBINE(V, I)                                                                                           \
+    hipLaunchKernelGGL((piece_combine_kernel<V, I>), dim3(grid), dim3(kBlock), 0, s, m, n, po.first, po.part, po.ld, beta, C, ldc, \
+                       logG, hubs.row_slot, hubs.agg, hubs.ld)
+    if (vec4) {
+        if (iters <= 1) GNNHIP_PIECES_COMBINE(4, 1);
+        else if (iters == 2) GNNHIP_PIECES_COMBINE(4, 2);
+        else GNNHIP_PIECES_COMBINE(4, 4);
+    } else {
+        if (iters <= 1) GNNHIP_PIECES_COMBINE(1, 1);
+        else if (iters == 2) GNNHIP_PIECES_COMBINE(1, 2);
+        else GNNHIP_PIECES_COMBINE(1, 4);
+    }
+#undef GNNHIP_PIECES_COMBINE
+    GNNHIP_LAUNCH_CHECK("spmm_pieces combine");
+    return GNNHIP_OK;
 }
 
 }  // namespace gnnhip
