@@ -394,10 +394,10 @@ def kernel_rooflines(dev, forwards=None):
         forwards["one_launch_by_graphs"] = time_one_launch_by_graphs(dev)
     return [
         r4,
-        hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + spmm_rowgroup_kernel<4,1> (sums of a row's pieces) + "
+        hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + piece_combine_kernel<4,1> (sums of a row's pieces) + "
             "s2v_level_stream_kernel<64,true,...> (contraction over the summed rows)", w5 + ": one level, plan included",
             level_algorithmic_bytes(N, E, C), c5["level"]["avg_ms"], gather_GBps=c5["level"]["gather_GBps"]),
-        hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + spmm_rowgroup_kernel<4,1>", w5 + ": SpMM A*h, plan included",
+        hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + piece_combine_kernel<4,1>", w5 + ": SpMM A*h, plan included",
             spmm_algorithmic_bytes(N, N, E, C), c5["spmm"]["avg_ms"], gather_GBps=c5["spmm"]["gather_GBps"]),
         hbm("sgemm_skinny_rows_kernel<1>", w5 + ": node scores h*w", 4 * N * (C + 1), c5["score"]["avg_ms"]),
         hbm("jagged_softmax_fused_kernel", w5 + ": jagged softmax over %d segments of 1024" % B,
