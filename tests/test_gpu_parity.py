@@ -1466,7 +1466,7 @@ def test_spmm_few_long_rows_take_a_workgroup_each(gpu, oracle, m, n):
         assert np.all(got[1] == 0) and np.array_equal(got2[1], (1.5 * C0[1]).astype(np.float32))
 
 
-@pytest.mark.parametrize("n", [64, 128, 9, 36, 300, 32, 4])
+@pytest.mark.parametrize("n", [64, 128, 9, 36, 300, 32, 4, 520, 150])
 def test_spmm_column_ordered_pieces_on_a_power_law_matrix(gpu, oracle, n):
     """R-MAT, 65,536 rows, 16 entries per row on average (rows of up to 13,000 entries, a third of the rows
     empty): large and dense enough for the route that cuts rows into pieces of 32 entries and sums them in the
