@@ -206,7 +206,7 @@ int exclusive_scan_i32(int* x, long long n, int* seg_scratch, hipStream_t s);
 size_t radix_hist_ints(long long n);
 size_t radix_seg_ints(long long n);
 int radix_order_by_digit(const unsigned* keys, long long n, int shift, unsigned* keys_out, unsigned* perm_out, int* hist, int* seg,
-                         hipStream_t s);
+                         hipStream_t s, const unsigned* carried = nullptr);
 int spmm_plain_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
                         const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan = false);
 // pieces.hip: C = alpha*A*B + beta*C for large matrices with many entries per row, the rows cut into pieces that

@@ -9,7 +9,8 @@
 // contiguous eighth of it.  What runs together then starts in the same narrow band of B; measured on R-MAT
 // with 4M rows and 16 entries per row this brings the fetched bytes from 14 GB (pieces in row order) to 8 GB.
 //
-//   plan     pieces per row -> offsets (scan) -> piece records + keys -> order by first column ->
+//   plan     pieces per row -> offsets (scan) -> piece records + keys -> order by first column (the second radix
+//            pass carries the first one's order along, the records themselves stay where they are) ->
 //            entries copied in piece order (a CSR matrix whose rows are the pieces)
 //   sums     one lane group per piece, entries read front to back; a row of one piece (most rows) gets its
 //            result, beta * C included, straight from here
@@ -81,25 +82,20 @@ __global__ __launch_bounds__(kBlock) void piece_fill_kernel(int m, long long slo
     }
 }
 
-// ordered[i] = rec[perm[i]]
-__global__ __launch_bounds__(kBlock) void piece_permute_kernel(long long slots, const unsigned* __restrict__ perm,
-                                                               const PieceRec* __restrict__ rec, PieceRec* __restrict__ ordered)
-{
-    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < slots; i += (long long)gridDim.x * kBlock)
-        ordered[i] = rec[perm[i]];
-}
-
 // lens[i] = entries of the i-th piece in order (lens[slots] = 0, so that the scan leaves the total there);
 // where[i] = i and ones[i] = 1: the matrix that picks the pieces of a row (the sums are stored by piece id, so the
 // pieces of a row lie next to each other and the combining pass reads them front to back);
 // target[i]: where the sum of the i-th piece in order goes: the row r >= 0 when the piece is all of that row,
-// else -1 - id, its place among the partial sums
-__global__ __launch_bounds__(kBlock) void piece_place_kernel(long long slots, const PieceRec* __restrict__ ordered, int* __restrict__ lens,
-                                                             int* __restrict__ where, float* __restrict__ ones, int* __restrict__ target)
+// else -1 - id, its place among the partial sums.  order[i] = id of the i-th piece in order; ordered[i] = its record.
+__global__ __launch_bounds__(kBlock) void piece_place_kernel(long long slots, const unsigned* __restrict__ order,
+                                                             const PieceRec* __restrict__ rec, PieceRec* __restrict__ ordered,
+                                                             int* __restrict__ lens, int* __restrict__ where, float* __restrict__ ones,
+                                                             int* __restrict__ target)
 {
     for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i <= slots; i += (long long)gridDim.x * kBlock) {
         if (i == slots) { lens[i] = 0; continue; }
-        const PieceRec r = ordered[i];
+        const PieceRec r = rec[order[i]];
+        ordered[i] = r;
         lens[i] = r.end - r.start;
         where[i] = (int)i;
         ones[i] = 1.f;
@@ -109,6 +105,8 @@ __global__ __launch_bounds__(kBlock) void piece_place_kernel(long long slots, co
 
 // Entries copied into piece order: half a wavefront per piece (kPiece = 32 entries, one per lane), four pieces
 // per turn so that their dependent loads (record, place, entry) overlap.  The empty pieces at the end are skipped.
+// (Taken by id instead, so that the reads walk the CSR arrays front to back and the writes scatter, the copy is
+// slower: 0.44 against 0.37 ms.)
 __global__ __launch_bounds__(kBlock) void piece_gather_kernel(const int* __restrict__ count, const PieceRec* __restrict__ ordered,
                                                               const int* __restrict__ at, const int* __restrict__ col_idx,
                                                               const float* __restrict__ val, int* __restrict__ col_out,
@@ -405,7 +403,7 @@ int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int*
     const size_t o_seg = carve(sizeof(int) * (longest / 4096 + 2 + radix_seg_ints(slots)));
     const size_t o_rec = carve(sizeof(PieceRec) * (size_t)slots), o_ord = carve(sizeof(PieceRec) * (size_t)slots);
     const size_t o_keys = carve(sizeof(unsigned) * (size_t)slots), o_keys2 = carve(sizeof(unsigned) * (size_t)slots);
-    const size_t o_perm = carve(sizeof(unsigned) * (size_t)slots);
+    const size_t o_perm = carve(sizeof(unsigned) * (size_t)slots), o_perm2 = carve(sizeof(unsigned) * (size_t)slots);
     const size_t o_hist = carve(sizeof(int) * radix_hist_ints(slots));
     void* base = nullptr;
     if (int rc = stream_scratch_slot(s, 3, off, &base)) return rc;
@@ -425,6 +423,7 @@ int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int*
     unsigned* keys = reinterpret_cast<unsigned*>(b + o_keys);
     unsigned* keys2 = reinterpret_cast<unsigned*>(b + o_keys2);
     unsigned* perm = reinterpret_cast<unsigned*>(b + o_perm);
+    unsigned* order = reinterpret_cast<unsigned*>(b + o_perm2);
     int* hist = reinterpret_cast<int*>(b + o_hist);
     float* part = static_cast<float*>(pbase);
 
@@ -440,14 +439,12 @@ int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int*
         while (bits < 31 && (1ll << bits) < (long long)k) ++bits;
         const int shift = bits > 16 ? bits - 16 : 0;
         hipLaunchKernelGGL(piece_fill_kernel, dim3(egrid), dim3(kBlock), 0, s, m, slots, row_ptr, (int)nnz, col_idx, first, shift, rec, keys);
-        // two stable passes, low digit first: the pieces end up ordered by the top 16 bits of their first column
+        // two stable passes, low digit first: order[i] = id of the piece that comes i-th by the top 16 bits of its first column
         if (int rc = radix_order_by_digit(keys, slots, 0, keys2, perm, hist, seg, s)) return rc;
-        hipLaunchKernelGGL(piece_permute_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, perm, rec, ordered);
-        if (int rc = radix_order_by_digit(keys2, slots, 8, keys, perm, hist, seg, s)) return rc;
-        hipLaunchKernelGGL(piece_permute_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, perm, ordered, rec);
-        hipLaunchKernelGGL(piece_place_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, rec, at, where, ones, target);
+        if (int rc = radix_order_by_digit(keys2, slots, 8, keys, order, hist, seg, s, perm)) return rc;
+        hipLaunchKernelGGL(piece_place_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, order, rec, ordered, at, where, ones, target);
         if (int rc = exclusive_scan_i32(at, slots + 1, seg, s)) return rc;
-        hipLaunchKernelGGL(piece_gather_kernel, dim3(egrid), dim3(kBlock), 0, s, first + m, rec, at, col_idx, val, col_ord, val_ord);
+        hipLaunchKernelGGL(piece_gather_kernel, dim3(egrid), dim3(kBlock), 0, s, first + m, ordered, at, col_idx, val, col_ord, val_ord);
         GNNHIP_LAUNCH_CHECK("spmm_pieces plan");
         memo = Memo{s, row_ptr, col_idx, val, m, nnz, base};
     }

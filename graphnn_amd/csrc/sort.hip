@@ -594,18 +594,19 @@ inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 // One stable pass of the radix sort: perm_out[i] = index of the key that comes i-th when the n keys are ordered by
 // the 8-bit digit (key >> shift) & 255 (equal digits keep their input order); keys_out receives the keys in that
-// order.  hist needs radix_hist_ints(n) ints, seg radix_seg_ints(n).
+// order.  With `carried`, perm_out[i] = carried[that index] instead (the order of an earlier pass carried along).
+// hist needs radix_hist_ints(n) ints, seg radix_seg_ints(n).
 size_t radix_hist_ints(long long n) { return (size_t)kDigits * (size_t)((n + kTile - 1) / kTile > 0 ? (n + kTile - 1) / kTile : 1); }
 size_t radix_seg_ints(long long n) { return (radix_hist_ints(n) + kScanSeg - 1) / kScanSeg + 1; }
 int radix_order_by_digit(const unsigned* keys, long long n, int shift, unsigned* keys_out, unsigned* perm_out, int* hist, int* seg,
-                         hipStream_t s)
+                         hipStream_t s, const unsigned* carried)
 {
     if (n <= 0) return GNNHIP_OK;
     const int ntiles = (int)((n + kTile - 1) / kTile);
     hipLaunchKernelGGL(radix_hist_kernel, dim3(ntiles), dim3(kBlock), 0, s, keys, n, shift, ntiles, hist);
     if (int rc = exclusive_scan_i32(hist, (long long)kDigits * ntiles, seg, s)) return rc;
-    hipLaunchKernelGGL(radix_scatter_kernel, dim3(ntiles), dim3(kBlock), 0, s, keys, (const unsigned*)nullptr, n, shift, ntiles, hist,
-                       keys_out, perm_out, 1);
+    hipLaunchKernelGGL(radix_scatter_kernel, dim3(ntiles), dim3(kBlock), 0, s, keys, carried, n, shift, ntiles, hist,
+                       keys_out, perm_out, carried ? 0 : 1);
     GNNHIP_LAUNCH_CHECK("radix_order_by_digit");
     return GNNHIP_OK;
 }
