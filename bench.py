@@ -372,6 +372,14 @@ def time_cfg5(dev, scale=22):
     return res
 
 
+# HBM bytes of one configuration-5 product with its plan (all launches from piece_count_kernel to piece_combine_kernel:
+# fetched 11.62 GB, written 2.91 GB) and of the level on top of it (s2v_level_stream_kernel: 2.15 + 1.07 GB more)
+CFG5_SPMM_TRAFFIC = 14530000000
+CFG5_LEVEL_TRAFFIC = 17750000000
+CFG5_TRAFFIC_SOURCE = ("constant: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 summed over the launches of one call, from the rocprofv3 "
+                       "--pmc runs summarised in profiles/spmm_pieces_cfg5_fetch_write.md (not re-measured in this run)")
+
+
 def kernel_rooflines(dev, forwards=None):
     """The other kernels of the path at the sizes they are built for, each against the roofline that bounds
     it: the hidden-256 level of configuration 4 against the FP32 matrix peak, the configuration-5 kernels
@@ -396,9 +404,11 @@ def kernel_rooflines(dev, forwards=None):
         r4,
         hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + piece_combine_kernel<4,1> (sums of a row's pieces) + "
             "s2v_level_stream_kernel<64,true,...> (contraction over the summed rows)", w5 + ": one level, plan included",
-            level_algorithmic_bytes(N, E, C), c5["level"]["avg_ms"], gather_GBps=c5["level"]["gather_GBps"]),
+            level_algorithmic_bytes(N, E, C), c5["level"]["avg_ms"], gather_GBps=c5["level"]["gather_GBps"],
+            traffic=CFG5_LEVEL_TRAFFIC, traffic_source=CFG5_TRAFFIC_SOURCE),
         hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + piece_combine_kernel<4,1>", w5 + ": SpMM A*h, plan included",
-            spmm_algorithmic_bytes(N, N, E, C), c5["spmm"]["avg_ms"], gather_GBps=c5["spmm"]["gather_GBps"]),
+            spmm_algorithmic_bytes(N, N, E, C), c5["spmm"]["avg_ms"], gather_GBps=c5["spmm"]["gather_GBps"],
+            traffic=CFG5_SPMM_TRAFFIC, traffic_source=CFG5_TRAFFIC_SOURCE),
         hbm("sgemm_skinny_rows_kernel<1>", w5 + ": node scores h*w", 4 * N * (C + 1), c5["score"]["avg_ms"]),
         hbm("jagged_softmax_fused_kernel", w5 + ": jagged softmax over %d segments of 1024" % B,
             8 * N + 4 * B, c5["jagged_softmax"]["avg_ms"]),
