@@ -247,6 +247,100 @@ def rmat_csr(seed, scale, nnz, a=0.57, b=0.19, c=0.19, chunk=1 << 24):
     return _csr_from_sorted_rows(rows, n), cols, np.ones(nnz, dtype=np.float32)
 
 
+# ---- the same streams generated by torch (on the GPU for the large configurations) --------------------
+# SplitMix64 in two's-complement int64 arithmetic: products wrap exactly as the unsigned ones do, and a logical
+# right shift is an arithmetic one with the sign copies masked off, so every value equals the numpy stream's
+# bit for bit; tests assert it.
+def _i64(x):
+    x &= _MASK64
+    return x - (1 << 64) if x >= (1 << 63) else x
+
+
+def _lsr(z, s):
+    return (z >> s) & ((1 << (64 - s)) - 1)
+
+
+def torch_u64(seed, pos, n, device):
+    """int64 tensor with the bits of Stream(seed) outputs number pos + 1 .. pos + n"""
+    import torch
+    idx = torch.arange(pos + 1, pos + n + 1, dtype=torch.int64, device=device)
+    z = idx * _i64(int(_GOLDEN)) + _i64(int(seed))
+    z = (z ^ _lsr(z, 30)) * _i64(int(_M1))
+    z = (z ^ _lsr(z, 27)) * _i64(int(_M2))
+    return z ^ _lsr(z, 31)
+
+
+def torch_uniform(seed, pos, n, device):
+    """float64 tensor equal to Stream(seed).uniform at positions pos .. pos + n"""
+    return _lsr(torch_u64(seed, pos, n, device), 11).double() * (1.0 / 9007199254740992.0)
+
+
+def rmat_edges_torch(seed, scale, nnz, device, a=0.57, b=0.19, c=0.19, lo=0, hi=None, chunk=1 << 24):
+    """(rows, cols) int64 of edges lo .. hi of rmat_csr's edge list before sorting, generated on `device`"""
+    import torch
+    hi = nnz if hi is None else hi
+    root = Stream(seed)
+    seeds = [root.child(level).seed for level in range(scale)]
+    rows = torch.zeros(hi - lo, dtype=torch.int64, device=device)
+    cols = torch.zeros(hi - lo, dtype=torch.int64, device=device)
+    ab, abc = a + b, a + b + c
+    for p in range(lo, hi, chunk):
+        q = min(hi, p + chunk)
+        r = torch.zeros(q - p, dtype=torch.int64, device=device)
+        cc = torch.zeros(q - p, dtype=torch.int64, device=device)
+        for level in range(scale):
+            u = torch_uniform(seeds[level], p, q - p, device)
+            r = (r << 1) | (u >= ab).long()
+            cc = (cc << 1) | (((u >= a) & (u < ab)) | (u >= abc)).long()
+        rows[p - lo:q - lo] = r
+        cols[p - lo:q - lo] = cc
+    return rows, cols
+
+
+def rmat_csr_torch(seed, scale, nnz, device, a=0.57, b=0.19, c=0.19):
+    """rmat_csr on `device`: (row_ptr int32 [n + 1], col_idx int32 [nnz], val float32 [nnz]) as torch tensors, equal to
+    the numpy generator's arrays bit for bit"""
+    import torch
+    n = 1 << scale
+    rows, cols = rmat_edges_torch(seed, scale, nnz, device, a, b, c)
+    key = rows * n + cols
+    del rows, cols
+    key, _ = torch.sort(key)
+    r = key >> scale
+    col_idx = (key - (r << scale)).int()
+    cnt = torch.bincount(r, minlength=n)
+    del key, r
+    row_ptr = torch.zeros(n + 1, dtype=torch.int32, device=device)
+    row_ptr[1:] = torch.cumsum(cnt, 0).int()
+    return row_ptr, col_idx, torch.ones(nnz, dtype=torch.float32, device=device)
+
+
+def torch_uniform_f32(seed, n, device, lo=0.0, hi=1.0, chunk=1 << 25):
+    """float32 tensor of n values lo + (hi - lo) u, u the uniforms of Stream(seed) from its start, rounded to float32
+    once: equal to (lo + (hi - lo) * Stream(seed).uniform(n)).astype(float32)"""
+    import torch
+    out = torch.empty(n, dtype=torch.float32, device=device)
+    for p in range(0, n, chunk):
+        q = min(n, p + chunk)
+        out[p:q] = (lo + (hi - lo) * torch_uniform(seed, p, q - p, device)).float()
+    return out
+
+
+def torch_normal_f32(seed, n, device, std=1.0, chunk=1 << 24):
+    """float32 tensor of n Box-Muller normals from the uniforms of Stream(seed), as Stream(seed).normal(n, std): the
+    uniforms are the numpy stream's bit for bit; log1p / sqrt / cos are the device's float64 routines, whose last bit
+    may differ from the host library's, so a value may land on the neighbouring float32 (tests bound that on a prefix)"""
+    import math
+    import torch
+    out = torch.empty(n, dtype=torch.float32, device=device)
+    for p in range(0, n, chunk):
+        q = min(n, p + chunk)
+        u = torch_uniform(seed, 2 * p, 2 * (q - p), device)
+        z = torch.sqrt(-2.0 * torch.log1p(-u[0::2])) * torch.cos(2.0 * math.pi * u[1::2])
+        out[p:q] = (std * z).float()
+    return out
+
+
 def contiguous_subgraph_csr(num_nodes, num_subgraph):
     """S for subgraphs that are equal contiguous node ranges (row g lists its nodes)"""
     per = num_nodes // num_subgraph
@@ -263,11 +357,16 @@ CONFIGS = {
 }
 
 
-def make_config(config_id, B=None):
-    """(batch, weights, dims) for the molecule-style configurations 1, 2 and 4"""
+def make_config(config_id, B=None, size_mode=None):
+    """(batch, weights, dims) for the molecule-style configurations 1, 2 and 4.  size_mode="uniform" on configuration 2
+    takes its "nodes per graph ~ U[10,110]" literally (mean 60) instead of the right-skewed sizes with mean ~30."""
     cfg = dict(CONFIGS[config_id])
     if B is not None:
         cfg["B"] = B
+    if size_mode is not None and size_mode != cfg["size_mode"]:
+        cfg["size_mode"] = size_mode
+        if size_mode == "uniform" and "size_lo" not in cfg:
+            cfg["size_lo"], cfg["size_hi"] = 10, 110
     seed = config_seed(config_id)
     kw = {k: cfg[k] for k in ("size_lo", "size_hi") if k in cfg}
     batch = molecule_batch(seed, cfg["B"], cfg["K"], cfg["Q"], size_mode=cfg["size_mode"], **kw)

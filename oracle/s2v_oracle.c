@@ -182,6 +182,30 @@ void orc_spmm_csr(int m, int n, float alpha, const int* row_ptr, const int* col_
     }
 }
 
+/* Not a reference routine: the float64 arbiter of the parity tests at sizes where scipy's single-threaded product
+ * takes too long.  out[m,n] (double) = alpha * A * B with every product and sum in double; absolute != 0 gives the
+ * same sum over magnitudes (|alpha| |A| |B|), the condition tensor of the parity metric.  Pinned against scipy's
+ * float64 CSR product (tests/test_oracle_pins.py). */
+void orc_spmm_csr_f64(int m, int n, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+                      const float* B, int ldb, int absolute, double* out, int ldo)
+{
+#pragma omp parallel for schedule(dynamic, 256)
+    for (int i = 0; i < m; ++i) {
+        double* c = out + (size_t)i * ldo;
+        for (int j = 0; j < n; ++j) c[j] = 0.0;
+        for (int t = row_ptr[i]; t < row_ptr[i + 1]; ++t) {
+            double a = (double)alpha * (double)val[t];
+            const float* b = B + (size_t)col_idx[t] * ldb;
+            if (absolute) {
+                a = fabs(a);
+                for (int j = 0; j < n; ++j) c[j] += a * fabs((double)b[j]);
+            } else {
+                for (int j = 0; j < n; ++j) c[j] += a * (double)b[j];
+            }
+        }
+    }
+}
+
 /* C[k,n] = alpha * A^T * B + beta * C, A CSR with m rows and k columns, B [m,n].
  * Reference: same call with trans 'T' (used by MatMul::Backward, src/nn/matmul.cpp:35-76). */
 void orc_spmm_csr_T(int m, int n, int k, float alpha, const int* row_ptr, const int* col_idx,

@@ -31,6 +31,9 @@ void orc_csr_subgraph(int num_subgraph, int num_nodes, const int* subg_id, const
 /* ---- tensor ops ---- */
 void orc_spmm_csr(int m, int n, float alpha, const int* row_ptr, const int* col_idx,
                   const float* val, const float* B, int ldb, float beta, float* C, int ldc);
+/* float64 arbiter (not a reference routine): out = alpha * A * B in double, or the same sum over magnitudes */
+void orc_spmm_csr_f64(int m, int n, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+                      const float* B, int ldb, int absolute, double* out, int ldo);
 void orc_spmm_csr_T(int m, int n, int k, float alpha, const int* row_ptr, const int* col_idx,
                     const float* val, const float* B, int ldb, float beta, float* C, int ldc);
 void orc_gemm(int transA, int transB, int m, int n, int k, float alpha, const float* A, int lda,

@@ -11,7 +11,7 @@ import os
 import numpy as np
 import pytest
 
-from conftest import FLOOR_POOL, FLOOR_PROBS_ABS, PARITY_TOL, Lazy, assert_parity, forward_float64, max_rel
+from conftest import FLOOR_POOL, FLOOR_PROBS_ABS, PARITY_TOL, Lazy, assert_parity, assert_stages, forward_float64, max_rel
 from graphnn_amd import batching, synth
 
 pytestmark = pytest.mark.gpu
@@ -46,45 +46,47 @@ def _random_csr(rng, m, k, nnz, unit=False, sort_cols=False):
 
 # float64 models of the kernels: assert_parity consults them only when a device result misses the oracle
 # (both are then fp32 evaluations in different summation orders, and float64 tells which one is off)
-def _csr64(rp, ci, v, m, k):
+def _csr64(rp, v, m, k, ci):
     import scipy.sparse as sp
     return sp.csr_matrix((np.asarray(v, np.float64), ci, rp), shape=(m, k))
 
 
 def _spmm_want(oracle, rp, ci, v, B, m, alpha=1.0, beta=0.0, C=None):
     want = oracle.spmm(rp, ci, v, B, m, alpha=alpha, beta=beta, C=C)
-    def model():
-        y = alpha * (_csr64(rp, ci, v, m, B.shape[0]) @ B.astype(np.float64))
-        return y if C is None else y + beta * C.astype(np.float64)
-    return want, Lazy(model)
+    def model(mag=lambda x: x):
+        y = mag(alpha) * (_csr64(rp, mag(np.asarray(v, np.float64)), m, B.shape[0], ci) @ mag(B.astype(np.float64)))
+        return y if C is None else y + mag(beta) * mag(C.astype(np.float64))
+    return want, Lazy(model, Lazy(lambda: model(np.abs)))
 
 
 def _gemm_want(oracle, A, B, ta=False, tb=False, alpha=1.0, beta=0.0, C=None):
     want = oracle.gemm(A, B, ta, tb, alpha=alpha, beta=beta, C=C)
-    def model():
-        a64, b64 = A.astype(np.float64), B.astype(np.float64)
-        y = alpha * ((a64.T if ta else a64) @ (b64.T if tb else b64))
-        return y if C is None else y + beta * C.astype(np.float64)
-    return want, Lazy(model)
+    def model(mag=lambda x: x):
+        a64, b64 = mag(A.astype(np.float64)), mag(B.astype(np.float64))
+        y = mag(alpha) * ((a64.T if ta else a64) @ (b64.T if tb else b64))
+        return y if C is None else y + mag(beta) * mag(C.astype(np.float64))
+    return want, Lazy(model, Lazy(lambda: model(np.abs)))
 
 
 def _level_want(oracle, rp, ci, v, h_in, W, msg=None, bias=None):
     want = oracle.level(rp, ci, v, h_in, W, msg, bias)
-    def model():
+    def model(mag=None):
         N = h_in.shape[0]
-        z = (_csr64(rp, ci, v, N, N) @ h_in.astype(np.float64)) @ W.astype(np.float64)
+        f = mag or (lambda x: x)
+        z = (_csr64(rp, f(np.asarray(v, np.float64)), N, N, ci) @ f(h_in.astype(np.float64))) @ f(W.astype(np.float64))
         if bias is not None:
-            z = z + bias.astype(np.float64)
+            z = z + f(bias.astype(np.float64))
         if msg is not None:
-            z = z + msg.astype(np.float64)
-        return np.maximum(z, 0)
-    return want, Lazy(model)
+            z = z + f(msg.astype(np.float64))
+        return z if mag else np.maximum(z, 0)
+    return want, Lazy(model, Lazy(lambda: model(np.abs)))
 
 
 def _forward_want(oracle, a, s, X, w, L, lab=None):
-    """the oracle's forward; want["_f64"] is the lazily computed float64 model of the same network"""
+    """the oracle's forward; want["_f64"] is the lazily computed float64 model of the same network, and carries the
+    same network on absolute values as its condition tensors"""
     want = oracle.forward(a, s, X, w, L, lab)
-    want["_f64"] = Lazy(lambda: forward_float64(a, s, X, w, L))
+    want["_f64"] = Lazy(lambda: forward_float64(a, s, X, w, L), Lazy(lambda: forward_float64(a, s, X, w, L, magnitudes=True)))
     return want
 
 
@@ -761,6 +763,7 @@ def test_forward_matches_reference_path(gpu, oracle, config_id):
     from graphnn_amd import ops
     batch, cfg, a, s, X, w, lab, want, got, bufs = _forward_case(gpu, oracle, config_id)
     _assert_forward_parity(got, want, cfg["L"])
+    assert_stages("", a, s, X, w, {k: got[k] for k in ("msg", "h_final", "pool", "hidden", "logits", "probs")})
     # argmax predictions bit-exact with the reference path
     assert np.array_equal(got["pred"], want["pred"])
     # loss / accuracy tail of the graph, operator by operator on the device
@@ -918,9 +921,12 @@ def test_forward_every_level_matches(gpu, oracle):
     msg, h = ops.s2v_input(_t(X, gpu), _t(w.W_n2l, gpu))
     assert max_rel(_n(h), want["h"][0]) < PARITY_TOL
     Wc = _t(w.W_conv, gpu)
+    levels = [_n(h)]
     for lv in range(cfg["L"]):
         h = ops.s2v_level(*a_d, h, Wc, msg)
         assert max_rel(_n(h), want["h"][lv + 1]) < PARITY_TOL, lv
+        levels.append(_n(h))
+    assert_stages(" (level entry)", a, s, X, w, dict(msg=_n(msg), h=np.stack(levels)))
 
 
 def test_forward_unfused_operator_route_agrees(gpu, oracle):
@@ -988,6 +994,7 @@ def _batched_case(gpu, oracle, batch, w, L):
     s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
     X = batch.one_hot()
     want = _forward_want(oracle, a, s, X, w, L, batch.label_csr())
+    want["_inputs"] = (a, s, X, w)
     bufs = ops.s2v_forward_batched(_csr_t(a, gpu), _csr_t(s, gpu), _t(X, gpu), _t(w.W_n2l, gpu), _t(w.W_conv, gpu),
                                    _t(w.W_h1, gpu), _t(w.W_h2, gpu), L, int(batch.graph_sizes.max()))
     return want, bufs
@@ -995,7 +1002,10 @@ def _batched_case(gpu, oracle, batch, w, L):
 
 def _assert_batched_matches(want, bufs, L):
     assert int(_n(bufs.status)[0]) == 0
-    _assert_forward_parity({k: _n(getattr(bufs, k)) for k in ("msg", "h_final", "pool", "hidden", "logits", "probs")}, want, L)
+    got = {k: _n(getattr(bufs, k)) for k in ("msg", "h_final", "pool", "hidden", "logits", "probs")}
+    _assert_forward_parity(got, want, L)
+    if "_inputs" in want:
+        assert_stages(" (one launch)", *want["_inputs"], got)
     assert np.array_equal(_n(bufs.pred), want["pred"])
 
 
@@ -1230,6 +1240,8 @@ def test_batched_forward_keeps_every_level_for_training(gpu, oracle, C, L, B):
     for l in range(L + 1):
         assert max_rel(_n(hl[l]), want["h"][l]) < PARITY_TOL, l
     assert np.array_equal(_n(hl[0]), np.maximum(_n(bufs.msg), 0))
+    assert_stages(" (one launch, levels kept)", a, s, batch.one_hot(), w,
+                  dict(msg=_n(bufs.msg), h=_n(hl), pool=_n(bufs.pool), hidden=_n(bufs.hidden), logits=_n(bufs.logits), probs=_n(bufs.probs)))
 
 
 def test_batched_forward_dense_features_past_the_staging_registers(gpu, oracle):

@@ -537,6 +537,87 @@ def test_parity_floors_are_the_smallest_the_oracle_itself_survives(oracle, confi
         assert need["pool"] > FLOOR_POOL / 10
 
 
+@pytest.mark.parametrize("config_id,B", [(1, 50), (2, 256), (2, 1000)])
+def test_condition_metric_holds_for_the_oracle_and_has_no_blind_band(oracle, config_id, B):
+    """conftest.assert_condition: |x - float64| <= 1e-4 * (the same network on absolute values), element by element,
+    no floor.  A correct fp32 evaluation (the oracle) meets it with a wide margin on every tensor; an error planted on
+    an element far below the tensor's scale, which max_rel's floor hides, breaks it."""
+    from conftest import FLOOR_DEFAULT, condition_error, forward_float64
+    batch, w, cfg = synth.make_config(config_id, B=B)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    got = oracle.forward(a, s, X, w, cfg["L"], batch.label_csr())
+    want = forward_float64(a, s, X, w, cfg["L"])
+    cond = forward_float64(a, s, X, w, cfg["L"], magnitudes=True)
+    worst = {k: condition_error(got[k], want[k], cond[k])[0] for k in ("msg", "h", "pool", "hidden", "logits", "probs")}
+    print("configuration %d, %d graphs: oracle, worst |x - float64| / sum|terms|: " % (config_id, B)
+          + "  ".join("%s %.2e" % kv for kv in worst.items()))
+    assert max(worst.values()) < 2e-5            # an fp32 sum of n terms is within n * 2^-24 in these units
+    # the condition tensor dominates the value it belongs to (triangle inequality), so the metric is never laxer than
+    # an absolute error of 1e-4 of the element's own magnitude
+    for k in ("msg", "h", "pool", "hidden", "logits"):
+        assert np.all(cond[k] >= np.abs(want[k]) * (1 - 1e-12))
+    # plant an error of 1 % on the smallest non-zero logit: invisible to max_rel at its floor when that logit is
+    # far below the scale, caught by the condition metric whenever it exceeds 1e-4 of the element's terms
+    lg = got["logits"].copy()
+    flat = np.abs(want["logits"]).ravel()
+    i = int(np.argmin(np.where(flat > 0, flat, np.inf)))
+    lg.ravel()[i] *= 1.5
+    planted, at = condition_error(lg, want["logits"], cond["logits"])
+    if 0.5 * flat[i] > 1e-4 * cond["logits"].ravel()[i]:
+        assert planted > 1e-4 and at == i
+    if 0.5 * flat[i] < 1e-4 * FLOOR_DEFAULT * np.abs(want["logits"]).max():
+        assert max_rel(lg, got["logits"]) < 1e-4     # the floored metric does not see it
+
+
+def test_stage_checker_accepts_the_oracle_and_catches_a_planted_error(oracle):
+    """conftest.assert_stages on the oracle's own outputs (a correct fp32 evaluation passes every stage), then with one
+    embedding element moved by 1e-3 of its terms (the stage that produced it must fail)"""
+    from conftest import assert_stages
+    batch, w, cfg = synth.make_config(1)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    got = oracle.forward(a, s, X, w, cfg["L"], batch.label_csr())
+    dev = {k: got[k] for k in ("msg", "h", "pool", "hidden", "logits", "probs")}
+    assert_stages("", a, s, X, w, dev, tol=2e-6)
+    bad = dict(dev, h=got["h"].copy())
+    i = np.unravel_index(np.argmax(got["h"][2]), got["h"][2].shape)
+    bad["h"][2][i] *= 1.001
+    with pytest.raises(AssertionError, match="h2"):
+        assert_stages("", a, s, X, w, bad)
+
+
+def test_condition_metric_on_products(oracle):
+    """the same bound for the oracle's SpMM, GEMM and level on signed random operands (every output a cancelling
+    sum), and what it means at its edges: an element whose terms are all zero must be exactly zero"""
+    import scipy.sparse as sp
+    from conftest import condition_error
+    rng = _rng(77)
+    m, k, n, nnz = 300, 200, 64, 6000
+    rows = np.sort(rng.integers(0, m, nnz))
+    rp = np.zeros(m + 1, np.int32); np.cumsum(np.bincount(rows, minlength=m), out=rp[1:])
+    ci = rng.integers(0, k, nnz).astype(np.int32); v = rng.standard_normal(nnz).astype(np.float32)
+    Bm = rng.standard_normal((k, n)).astype(np.float32)
+    A64 = sp.csr_matrix((v.astype(np.float64), ci, rp), shape=(m, k))
+    A64_mag = sp.csr_matrix((np.abs(v.astype(np.float64)), ci, rp), shape=(m, k))
+    got = oracle.spmm(rp, ci, v, Bm, m)
+    worst, _ = condition_error(got, A64 @ Bm.astype(np.float64), A64_mag @ np.abs(Bm.astype(np.float64)))
+    assert worst < 1e-5
+    Am = rng.standard_normal((150, 333)).astype(np.float32); Bg = rng.standard_normal((333, 40)).astype(np.float32)
+    worst, _ = condition_error(oracle.gemm(Am, Bg), Am.astype(np.float64) @ Bg.astype(np.float64),
+                               np.abs(Am.astype(np.float64)) @ np.abs(Bg.astype(np.float64)))
+    assert worst < 1e-5
+    # the oracle's own float64 product (the arbiter at full sizes) against scipy's
+    f64 = oracle.spmm_f64(rp, ci, v, Bm, m, alpha=-0.75)
+    assert np.allclose(f64, -0.75 * (A64 @ Bm.astype(np.float64)), rtol=1e-13, atol=1e-13)
+    assert np.allclose(oracle.spmm_f64(rp, ci, v, Bm, m, alpha=-0.75, absolute=True), 0.75 * (A64_mag @ np.abs(Bm.astype(np.float64))), rtol=1e-13)
+    # all-zero terms: zero passes, anything else is infinitely wrong
+    assert condition_error(np.zeros(3), np.zeros(3), np.zeros(3))[0] == 0.0
+    assert condition_error(np.array([0.0, 1e-30, 0.0]), np.zeros(3), np.zeros(3)) == (np.inf, 1)
+
+
 def test_edge_based_operands_against_dense_definitions(oracle):
     """Edge2Node / Node2Edge / Edge2Edge (src/nn/msg_pass.cpp:72-152) against matrices written straight
     from their definitions, and the numpy builders against the oracle"""
