@@ -300,35 +300,24 @@ def training_step_host_layer(host, reps=100):
 
 
 def time_cfg5(dev, scale=22):
-    """Configuration 5: R-MAT (a=.57, b=c=.19), 16 entries per row, generated on the device with the
-    same recursive-quadrant rule as synth.rmat_csr (torch's generator, so not the parity inputs);
-    level, SpMM, jagged softmax over segments of 1024 node scores, sum-pool."""
+    """Configuration 5: R-MAT (a=.57, b=c=.19), 16 entries per row, from the SplitMix64 streams of the configuration
+    (seed 0x5EED0005; generated on the device by the torch twin of synth.rmat_csr, bit-identical to the host
+    generator): level, SpMM (each with the plan made in the call, and with a plan made once by gnnhip_csr_plan_create),
+    node scores, jagged softmax over segments of 1024 node scores, sum-pool, and the whole forward."""
     import torch
-    from graphnn_amd import ops
+    from graphnn_amd import ops, synth
     N, E, C, K = 1 << scale, 16 << scale, 64, 16
-    g = torch.Generator(device=dev)
-    g.manual_seed(5)
-    rows = torch.zeros(E, dtype=torch.int64, device=dev)
-    cols = torch.zeros(E, dtype=torch.int64, device=dev)
-    for _ in range(scale):
-        u = torch.rand(E, device=dev, generator=g)
-        rows = (rows << 1) | (u >= 0.76).long()
-        cols = (cols << 1) | (((u >= 0.57) & (u < 0.76)) | (u >= 0.95)).long()
-    key, _ = torch.sort(rows * N + cols)
-    del rows, cols
-    r = key // N
-    ci = (key - r * N).int()
-    cnt = torch.bincount(r, minlength=N)
-    del key, r
-    rp = torch.zeros(N + 1, dtype=torch.int32, device=dev)
-    rp[1:] = torch.cumsum(cnt, 0).int()
-    val = torch.ones(E, dtype=torch.float32, device=dev)
-    lab = torch.randint(0, K, (N,), device=dev, generator=g)
+    seed = synth.config_seed(5)
+    root = synth.Stream(seed)
+    rp, ci, val = synth.rmat_csr_torch(seed, scale, E, dev)
+    cnt = (rp[1:] - rp[:-1])
+    t = lambda arr: torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
+    lab = t(root.child(3).randint(N, 0, K))
     X = torch.zeros((N, K), dtype=torch.float32, device=dev)
     X[torch.arange(N, device=dev), lab] = 1.0
-    Wn = torch.randn((K, C), device=dev, generator=g) * 0.1
-    Wc = torch.randn((C, C), device=dev, generator=g) * 0.1
-    wsc = torch.randn((C, 1), device=dev, generator=g) * 0.1
+    w = synth.make_weights(root, K, C, 64, 2)
+    Wn, Wc, Wh1, Wh2 = t(w.W_n2l), t(w.W_conv), t(w.W_h1), t(w.W_h2)
+    wsc = t(root.child(104).normal(C, 0.1).reshape(C, 1))
     B = N // 1024
     s_rp = (torch.arange(B + 1, device=dev) * 1024).int()
     s_ci = torch.arange(N, device=dev).int()
@@ -339,20 +328,35 @@ def time_cfg5(dev, scale=22):
     agg = torch.empty_like(h0)
     score = torch.empty((N, 1), dtype=torch.float32, device=dev)
     pool = torch.empty((B, C), dtype=torch.float32, device=dev)
-    res = {"workload": "configuration 5: R-MAT scale %d, %d rows, %d entries, max row %d, %d rows over 256 entries, hidden %d"
-                       % (scale, N, E, int(cnt.max()), int((cnt > 256).sum()), C), "shape": (N, E, C, B)}
+    res = {"workload": "configuration 5: R-MAT scale %d, %d rows, %d entries, max row %d, %d rows over 256 entries, %d empty rows, hidden %d"
+                       % (scale, N, E, int(cnt.max()), int((cnt > 256).sum()), int((cnt == 0).sum()), C), "shape": (N, E, C, B)}
     ms = _event_ms(lambda: ops.s2v_level(rp, ci, val, h0, Wc, msg, out=h1), 5)
     res["level"] = {"avg_ms": ms, "algorithmic_GBps": level_algorithmic_bytes(N, E, C) / (ms * 1e-3) / 1e9,
                     "gather_GBps": (4.0 * E * C + 12.0 * N * C + 8.0 * E) / (ms * 1e-3) / 1e9}
     ms = _event_ms(lambda: ops.spmm(rp, ci, val, h0, N, out=agg), 5)
     res["spmm"] = {"avg_ms": ms, "algorithmic_GBps": spmm_algorithmic_bytes(N, N, E, C) / (ms * 1e-3) / 1e9,
                    "gather_GBps": (4.0 * E * C + 4.0 * N * C + 8.0 * E) / (ms * 1e-3) / 1e9}
+    # the same two with a plan made once (gnnhip_csr_plan_create): what a caller that keeps its matrix pays per product
+    unplanned_level, unplanned_agg = h1.clone(), agg.clone()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    plan = ops.CsrPlan(rp, ci, val, N, N)
+    torch.cuda.synchronize()
+    plan_ms = (time.perf_counter() - t0) * 1e3
+    ms = _event_ms(lambda: plan.level(h0, Wc, msg, out=h1), 10)
+    res["level_planned"] = {"avg_ms": ms, "algorithmic_GBps": level_algorithmic_bytes(N, E, C) / (ms * 1e-3) / 1e9}
+    ms = _event_ms(lambda: plan.spmm(h0, out=agg), 10)
+    res["spmm_planned"] = {"avg_ms": ms, "algorithmic_GBps": spmm_algorithmic_bytes(N, N, E, C) / (ms * 1e-3) / 1e9}
+    assert bool(torch.equal(h1, unplanned_level)) and bool(torch.equal(agg, unplanned_agg)), "planned and unplanned products differ"
+    res["plan"] = {"create_ms_wall": plan_ms, "device_bytes": plan.bytes(),
+                   "what": "gnnhip_csr_plan_create (blocking: it reads back the piece count) and the device memory the plan owns "
+                           "after a product of width 64, partial sums included"}
+    del unplanned_level, unplanned_agg
+    plan.close()
     ms = _event_ms(lambda: ops.gemm(h1, wsc, out=score), 5)
     res["score"] = {"avg_ms": ms}
     # the whole forward (input, 3 levels, readout): levels two and three reuse the plan that level one made for A
     H, Q, L = 64, 2, 3
-    Wh1 = torch.randn((C, H), device=dev, generator=g) * 0.1
-    Wh2 = torch.randn((H, Q), device=dev, generator=g) * 0.1
     bufs = ops.ForwardBuffers(N, B, C, H, Q, dev)
     ms = _event_ms(lambda: ops.s2v_forward((rp, ci, val), (s_rp, s_ci, s_v), X, Wn, Wc, Wh1, Wh2, L, bufs=bufs), 5)
     res["forward"] = {"avg_ms": ms, "levels": L, "graphs": B}
@@ -365,7 +369,7 @@ def time_cfg5(dev, scale=22):
     ones = torch.ones((N, 4), device=dev, dtype=torch.float32)
     deg = ops.spmm(rp, ci, val, ones, N)
     assert bool((deg[:, 0] == cnt.float()).all()), "row-length check failed on the R-MAT matrix"
-    sc = torch.randn((N, 1), device=dev, generator=g)
+    sc = synth.torch_uniform_f32(root.child(32).seed, N, dev, -6.0, 6.0).view(N, 1)
     ops.jagged_softmax(sc, lens)
     seg = sc.view(B, 1024).double().sum(dim=1)
     assert float((seg - 1.0).abs().max()) < 1e-5, "jagged softmax segments do not sum to 1"

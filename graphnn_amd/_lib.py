@@ -40,6 +40,12 @@ SIGNATURES = {
     "gnnhip_memset0_batch": [_I, _P, _P, _P],
     "gnnhip_stream_sync": [_P],
     "gnnhip_spmm_csr_f32": [_I, _I, _I, _I, _F, _P, _P, _P, _P, _I, _F, _P, _I, _P],
+    "gnnhip_csr_plan_create": [_I, _I, _P, _P, _P, _P, POINTER(_P)],
+    "gnnhip_csr_plan_destroy": [_P],
+    "gnnhip_csr_plan_bytes": [_P, POINTER(c_size_t)],
+    "gnnhip_spmm_csr_planned_f32": [_P, _I, _F, _P, _I, _F, _P, _I, _P],
+    "gnnhip_s2v_level_planned_f32": [_P, _I, _P, _P, _P, _P, _P, _P],
+    "gnnhip_release_scratch": [_P],
     "gnnhip_csr_group_i32": [_I, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P],
     "gnnhip_csr_group_both_i32": [_I, _I, _P, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_csr_consecutive_rows_f32": [_I, _P, _I, _P, _P, _P],

@@ -12,7 +12,7 @@ bool fused_hidden_supported(int C);
 int input_dispatch(int N, int K, int C, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s);
 int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
                    const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph = false,
-                   bool relu_in = false);
+                   bool relu_in = false, CsrPlan* plan = nullptr);
 bool level_accepts_relu_input(int N, int C, long long nnz);
 int level_backward_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* dz,
                             const float* W, float* u, float* g_prev, const float* gate, float* acc, hipStream_t s);
@@ -73,16 +73,16 @@ int input_any(int N, int K, int C, const float* X, const float* Wn2l, float* msg
 
 int level_any(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
               const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph = false,
-              bool relu_in = false)
+              bool relu_in = false, CsrPlan* plan = nullptr)
 {
-    int rc = level_dispatch(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s, same_graph, relu_in);
+    int rc = level_dispatch(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s, same_graph, relu_in, plan);
     if (rc != GNNHIP_EUNSUPPORTED) return rc;
     if (relu_in) return set_error(GNNHIP_EUNSUPPORTED, "no level kernel reads its input through ReLU for this shape");
     void* tmp = nullptr;
     const size_t total = (size_t)N * C;
     if ((rc = stream_scratch(s, sizeof(float) * total, &tmp))) return rc;
     float* agg = static_cast<float*>(tmp);
-    if ((rc = spmm_dispatch(N, N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, agg, C, s, same_graph))) return rc;
+    if ((rc = spmm_dispatch(N, N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, agg, C, s, same_graph, false, plan))) return rc;
     if ((rc = gemm_dispatch(0, 0, N, C, C, 1.f, agg, C, W, C, 0.f, h_out, C, s))) return rc;
     hipLaunchKernelGGL(bias_add_relu_kernel, dim3(ew_grid(total)), dim3(kBlock), 0, s,
                        h_out, bias, msg, h_out, (float*)nullptr, total, C, 1);
@@ -163,6 +163,20 @@ int gnnhip_s2v_level_f32(int N, int C, int nnz, const int* row_ptr, const int* c
     GNNHIP_REQUIRE(h_in != h_out, "s2v_level cannot run in place");
     if (int rc = require_ready()) return rc;
     return level_any(N, C, nnz, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, as_stream(stream));
+}
+
+int gnnhip_s2v_level_planned_f32(void* plan, int C, const float* h_in, const float* W, const float* msg, const float* bias, float* h_out,
+                                 void* stream)
+{
+    CsrPlan* p = as_csr_plan(plan);
+    GNNHIP_REQUIRE(p, "%p is not a live CSR plan", plan);
+    GNNHIP_REQUIRE(p->m == p->k, "s2v_level_planned needs the plan of a square matrix (it has %d rows and %d columns)", p->m, p->k);
+    GNNHIP_REQUIRE(C >= 1, "bad hidden size in s2v_level_planned (C=%d)", C);
+    if (p->m == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(h_in && W && h_out, "null tensor in s2v_level_planned");
+    GNNHIP_REQUIRE(h_in != h_out, "s2v_level_planned cannot run in place");
+    if (int rc = require_ready()) return rc;
+    return level_any(p->m, C, p->nnz, p->row_ptr, p->col_idx, p->val, h_in, W, msg, bias, h_out, as_stream(stream), false, false, p);
 }
 
 int gnnhip_s2v_level_backward_f32(int N, int C, int nnz, const int* t_row_ptr, const int* t_col_idx, const float* t_val,

@@ -163,6 +163,9 @@ __device__ __forceinline__ float4 relu_ref4(const float4& v)
 // Device memory from the library's pool (released with pool_release).
 int pool_acquire(void** p, size_t bytes);
 int pool_release(void* p);
+// a block of exactly this size straight from the driver, for long-lived blocks of hundreds of megabytes (pool_free
+// gives it back to the driver)
+int pool_acquire_exact(void** p, size_t bytes);
 
 // Grow-only scratch owned by the library, one buffer per stream, so that calls
 // ordered on one stream reuse it safely and calls on different streams never
@@ -174,6 +177,7 @@ int stream_scratch(hipStream_t s, size_t bytes, void** p);
 // takes slot 0; slot 2 holds the partial tiles of a GEMM split along k, whose operands
 // may sit in slot 0.
 constexpr int kScratchSlots = 7;     // 3: plan of the column-ordered SpMM, 4: its partial sums, 5: identity matrix of the wide level, 6: (index, value) pairs of a sparse upload
+constexpr int kExactScratchSlot = 3;  // slots from here on hold what one matrix needs (up to gigabytes): sized exactly, the old block freed first
 int stream_scratch_slot(hipStream_t s, int slot, size_t bytes, void** p);
 
 // reduce.hip: device address of the statically allocated segment offsets on the current device
@@ -189,17 +193,63 @@ struct HubPlan {
     const float* agg;                  // [slots][ld]
     int ld;
 };
+// A block of pool memory that holds the plan and the sums of one balanced pass for an owner that keeps it across
+// calls (a CSR plan); planned: the planning launches have run in it.
+struct HubStore {
+    void* base = nullptr;
+    size_t bytes = 0;
+    bool planned = false;
+};
 // threshold / chunk_len: rows with more entries than `threshold` are summed, cut into chunks of `chunk_len`
 // (the consumer must apply the same threshold when it looks a row up in row_slot); max_hubs >= 0: the caller's
-// bound on the number of such rows
+// bound on the number of such rows; store: where the pass keeps its arrays (null: the stream's scratch slot 1)
 int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
                 const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan = false, bool relu_in = false,
-                int threshold = kHubThreshold, int chunk_len = kHubChunk, long long max_hubs = -1);
+                int threshold = kHubThreshold, int chunk_len = kHubChunk, long long max_hubs = -1, HubStore* store = nullptr);
+// scratch bytes of that call (0 when the pass does not apply)
+size_t hub_scratch_bytes(int m, int n, long long nnz, int threshold = kHubThreshold, int chunk_len = kHubChunk, long long max_hubs = -1);
 // runtime.hip: host bytes placed in the stream's pinned staging buffer for a kernel to read in place (null: not to be had)
 int stage_in_pinned(hipStream_t s, const void* src_host, size_t bytes, const void** pinned);
-// spmm.hip: C = alpha*A*B + beta*C on stream s (A is [m,k]); reuse_plan as for hub_prepass
+// pieces.hip: what a caller prepares once for a CSR matrix it multiplies with many times (gnnhip_csr_plan_create).
+// For large matrices with many entries per row: the rows cut into pieces of consecutive entries, the pieces ordered by
+// their first column and the entries copied into that order; for every matrix: the plan of the balanced pass over
+// long rows.  All device memory of a plan is pool memory owned by it.
+struct CsrPlan {
+    unsigned magic = 0;
+    const int* row_ptr = nullptr;
+    const int* col_idx = nullptr;
+    const float* val = nullptr;
+    int m = 0, k = 0;
+    long long nnz = 0;            // entries of the matrix (an upper bound when the plan lives in stream scratch)
+    // ---- column-ordered pieces (has_pieces)
+    bool has_pieces = false;
+    long long slots = 0;          // capacity of the per-piece arrays (>= number of pieces)
+    long long pslots = 0;         // capacity of the partial sums (>= pieces of the rows of several pieces)
+    int* first = nullptr;         // [m + 1] pieces before row r
+    int* pfirst = nullptr;        // [m + 1] pieces of rows of several pieces before row r: row pointers of P
+    int* at = nullptr;            // [slots + 1] entries before the i-th piece in order
+    int* target = nullptr;        // [slots] row r >= 0 that the piece is all of, else -1 - (its place among the partial sums)
+    int* where = nullptr;         // [pslots] column indices of P (the identity)
+    float* ones = nullptr;        // [pslots] values of P
+    int* col_ord = nullptr;       // [nnz] entries in piece order
+    float* val_ord = nullptr;
+    void* head_block = nullptr;   // first, pfirst
+    void* body_block = nullptr;   // the other arrays
+    float* part = nullptr;        // partial sums [pslots, ldp], grown to the widest operand seen
+    size_t part_bytes = 0;
+    HubStore combine_hub;         // balanced pass over P (rows of many pieces)
+    // ---- balanced pass over the long rows of A itself (the route without pieces)
+    HubStore row_hub;
+    bool owned = false;           // blocks come from the pool and go back there with the plan
+};
+constexpr unsigned kCsrPlanMagic = 0x43535250u;
+
+// spmm.hip: C = alpha*A*B + beta*C on stream s (A is [m,k]); reuse_plan as for hub_prepass.
+// skip_empty_rows: rows of A without entries are left as they are in C (the caller treats them as zero; beta must be 0).
+// plan: a plan made for exactly these arrays (then nnz is exact and reuse_plan is ignored), or null.
 int spmm_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                  const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan = false);
+                  const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan = false,
+                  bool skip_empty_rows = false, CsrPlan* plan = nullptr);
 
 // sort.hip
 int exclusive_scan_i32(int* x, long long n, int* seg_scratch, hipStream_t s);
@@ -208,22 +258,20 @@ size_t radix_seg_ints(long long n);
 int radix_order_by_digit(const unsigned* keys, long long n, int shift, unsigned* keys_out, unsigned* perm_out, int* hist, int* seg,
                          hipStream_t s, const unsigned* carried = nullptr);
 int spmm_plain_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                        const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan = false);
+                        const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan = false,
+                        HubStore* row_hub = nullptr);
 // pieces.hip: C = alpha*A*B + beta*C for large matrices with many entries per row, the rows cut into pieces that
-// are summed in the order of their first column; GNNHIP_EUNSUPPORTED where the caller keeps its own route
-struct PiecesOperand {
-    const int* first;      // row pointers of P [m + 1]
-    const int* where;      // column indices of P: the place of each piece among the partial sums
-    const float* ones;     // values of P
-    const float* part;     // the partial sums [slots, ld]
-    int ld;
-    long long slots;       // columns of P (an upper bound of its entries)
-    bool plan_reused;
-};
-int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                     const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan, PiecesOperand* out);
+// are summed in the order of their first column; GNNHIP_EUNSUPPORTED (nothing launched, C untouched) where the caller
+// keeps its own route, GNNHIP_ENOMEM likewise when the device cannot give the scratch
 int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                         const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan);
+                         const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan, bool skip_empty_rows,
+                         CsrPlan* plan);
+// whether a matrix of this shape takes the pieces route at all (the width of the dense operand decides the rest)
+bool pieces_route_applies(int m, long long nnz);
+CsrPlan* as_csr_plan(void* handle);      // null unless handle is a live plan
+
+// runtime.hip: the pool's blocks given back to the driver (gnnhip_free), for scratch a plan no longer needs
+int pool_free(void* p);
 
 }  // namespace gnnhip
 

@@ -23,6 +23,8 @@
 // atomic counter per hub (hub_done) only elects the wavefront that adds the chunks' sums.
 #include "gnnhip_internal.h"
 
+#include <map>
+
 namespace gnnhip {
 
 namespace {
@@ -329,65 +331,122 @@ void launch_partial(hipStream_t s, const int* counts, int chunk_cap, int n, cons
 
 }  // namespace
 
+namespace {
+
+// Where the arrays of one pre-pass lie inside its block; everything up to `part` does not depend on the width n.
+struct HubLayout {
+    int nb, hub_cap, chunk_cap, ldp;
+    size_t o_counts, o_bh, o_bc, o_slot, o_hrow, o_hc0, o_chub, o_done, o_part, o_agg, bytes;
+};
+
+HubLayout hub_layout(int m, int n, long long nnz, int threshold, int chunk_len, long long max_hubs)
+{
+    HubLayout L;
+    L.ldp = (int)round_up((size_t)n, 4);
+    L.nb = (m + kRowsPerBlock - 1) / kRowsPerBlock;
+    long long hub_cap_ll = nnz / (threshold + 1) + 1;
+    if (max_hubs >= 0 && max_hubs < hub_cap_ll) hub_cap_ll = max_hubs;
+    const long long chunk_cap_ll = nnz / chunk_len + hub_cap_ll + 1;
+    L.hub_cap = (int)(hub_cap_ll < m ? hub_cap_ll : m);
+    L.chunk_cap = (int)chunk_cap_ll;
+    size_t off = 0;
+    auto carve = [&](size_t bytes) { const size_t o = off; off = round_up(off + bytes, 256); return o; };
+    L.o_counts = carve(sizeof(int) * 4);
+    L.o_bh = carve(sizeof(int) * L.nb);
+    L.o_bc = carve(sizeof(int) * L.nb);
+    L.o_slot = carve(sizeof(int) * (size_t)m);
+    L.o_hrow = carve(sizeof(int) * (size_t)L.hub_cap);
+    L.o_hc0 = carve(sizeof(int) * (size_t)L.hub_cap);
+    L.o_chub = carve(sizeof(int) * (size_t)L.chunk_cap);
+    L.o_done = carve(sizeof(int) * (size_t)L.hub_cap);
+    L.o_part = carve(sizeof(float) * (size_t)L.chunk_cap * L.ldp);
+    L.o_agg = carve(sizeof(float) * (size_t)L.hub_cap * L.ldp);
+    L.bytes = off;
+    return L;
+}
+
+inline bool hub_pass_applies(int m, int n, long long nnz, int threshold) { return !(m < kHubMinRows || nnz <= threshold || n > kWave * 16); }
+
+}  // namespace
+
+// Bytes of scratch a hub_prepass call with these arguments takes (0: the pass does not run).  A caller that must not
+// fail for lack of memory after its own first launch reserves them up front (stream_scratch_slot(s, 1, ...)).
+size_t hub_scratch_bytes(int m, int n, long long nnz, int threshold, int chunk_len, long long max_hubs)
+{
+    if (!hub_pass_applies(m, n, nnz, threshold)) return 0;
+    return hub_layout(m, n, nnz, threshold, chunk_len, max_hubs).bytes;
+}
+
 // Sums the hubs of A (rows longer than `threshold` entries, cut into chunks of `chunk_len`) times B[:, 0..n) into
 // plan->agg.  max_hubs, when not negative, is the caller's bound on the number of such rows (it sizes the buffers).
-// n <= 1024.  The buffers live in the stream's plan scratch and stay valid until the next
-// hub_prepass on the same stream.
-// reuse_plan: the caller guarantees that the structure of A has not changed since the previous call on
+// n <= 1024.  Without `store` the buffers live in the stream's scratch slot 1 and stay valid until the next
+// hub_prepass on the same stream; with it they live in a block the store's owner keeps (pool memory, grown when a
+// wider operand needs it), and the planning launches run only while store->planned is false.
+// reuse_plan (no store): the caller guarantees that the structure of A has not changed since the previous call on
 // this stream with the same arguments (the levels of one forward); the planning launches
 // (count, scan, fill) are then skipped and only the sums are recomputed.
 int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
                 const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan, bool relu_in, int threshold, int chunk_len,
-                long long max_hubs)
+                long long max_hubs, HubStore* store)
 {
     plan->row_slot = nullptr;
     plan->agg = nullptr;
     plan->ld = 0;
-    if (m < kHubMinRows || nnz <= threshold || n > kWave * 16) return GNNHIP_OK;
+    if (!hub_pass_applies(m, n, nnz, threshold)) return GNNHIP_OK;
     const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && aligned16(B);
     const int vec = vec4 ? 4 : 1;
     const int units = (n + vec - 1) / vec;
     const int logG = ilog2_ceil_(units < kWave ? units : kWave);
     const int G = 1 << logG;
     const int iters = (units + G - 1) / G;                   // 1..4
-    const int ldp = (int)round_up((size_t)n, 4);
+    const HubLayout L = hub_layout(m, n, nnz, threshold, chunk_len, max_hubs);
+    const int ldp = L.ldp, nb = L.nb, hub_cap = L.hub_cap, chunk_cap = L.chunk_cap;
 
-    const int nb = (m + kRowsPerBlock - 1) / kRowsPerBlock;
-    long long hub_cap_ll = nnz / (threshold + 1) + 1;
-    if (max_hubs >= 0 && max_hubs < hub_cap_ll) hub_cap_ll = max_hubs;
-    const long long chunk_cap_ll = nnz / chunk_len + hub_cap_ll + 1;
-    const int hub_cap = (int)(hub_cap_ll < m ? hub_cap_ll : m);
-    const int chunk_cap = (int)chunk_cap_ll;
-
-    size_t off = 0;
-    auto carve = [&](size_t bytes) { const size_t o = off; off = round_up(off + bytes, 256); return o; };
-    const size_t o_counts = carve(sizeof(int) * 4);
-    const size_t o_bh = carve(sizeof(int) * nb), o_bc = carve(sizeof(int) * nb);
-    const size_t o_slot = carve(sizeof(int) * (size_t)m);
-    const size_t o_hrow = carve(sizeof(int) * (size_t)hub_cap), o_hc0 = carve(sizeof(int) * (size_t)hub_cap);
-    const size_t o_chub = carve(sizeof(int) * (size_t)chunk_cap);
-    const size_t o_done = carve(sizeof(int) * (size_t)hub_cap);
-    const size_t o_part = carve(sizeof(float) * (size_t)chunk_cap * ldp);
-    const size_t o_agg = carve(sizeof(float) * (size_t)hub_cap * ldp);
     void* base = nullptr;
-    if (int rc = stream_scratch_slot(s, 1, off, &base)) return rc;
+    if (store) {
+        if (store->bytes < L.bytes) {
+            if (store->base) {
+                GNNHIP_HIP(hipStreamSynchronize(s));             // earlier launches may still read the old block
+                (void)pool_free(store->base);
+                store->base = nullptr;
+                store->bytes = 0;
+            }
+            if (int rc = pool_acquire_exact(&store->base, L.bytes)) return rc;
+            store->bytes = L.bytes;
+            store->planned = false;
+        }
+        base = store->base;
+    } else if (int rc = stream_scratch_slot(s, 1, L.bytes, &base)) {
+        return rc;
+    }
     char* b = static_cast<char*>(base);
-    int* counts = reinterpret_cast<int*>(b + o_counts);
-    int* bh = reinterpret_cast<int*>(b + o_bh);
-    int* bc = reinterpret_cast<int*>(b + o_bc);
-    int* row_slot = reinterpret_cast<int*>(b + o_slot);
-    int* hub_row = reinterpret_cast<int*>(b + o_hrow);
-    int* hub_chunk0 = reinterpret_cast<int*>(b + o_hc0);
-    int* chunk_hub = reinterpret_cast<int*>(b + o_chub);
-    int* hub_done = reinterpret_cast<int*>(b + o_done);
-    float* part = reinterpret_cast<float*>(b + o_part);
-    float* agg = reinterpret_cast<float*>(b + o_agg);
+    int* counts = reinterpret_cast<int*>(b + L.o_counts);
+    int* bh = reinterpret_cast<int*>(b + L.o_bh);
+    int* bc = reinterpret_cast<int*>(b + L.o_bc);
+    int* row_slot = reinterpret_cast<int*>(b + L.o_slot);
+    int* hub_row = reinterpret_cast<int*>(b + L.o_hrow);
+    int* hub_chunk0 = reinterpret_cast<int*>(b + L.o_hc0);
+    int* chunk_hub = reinterpret_cast<int*>(b + L.o_chub);
+    int* hub_done = reinterpret_cast<int*>(b + L.o_done);
+    float* part = reinterpret_cast<float*>(b + L.o_part);
+    float* agg = reinterpret_cast<float*>(b + L.o_agg);
 
-    struct Memo { hipStream_t s; const int* row_ptr; int m, n; long long nnz; void* base; int threshold, chunk_len, hub_cap; };
-    static thread_local Memo memo = {nullptr, nullptr, 0, 0, 0, nullptr, 0, 0, 0};
-    const bool planned = reuse_plan && memo.row_ptr == row_ptr && memo.s == s && memo.m == m && memo.n == n &&
-                         memo.nnz == nnz && memo.base == base && memo.threshold == threshold && memo.chunk_len == chunk_len &&
-                         memo.hub_cap == hub_cap;
+    // What the stream's scratch slot holds a plan for.  Kept per stream, next to the scratch it describes (any thread
+    // that plans on the stream replaces it), not per thread.
+    struct Memo { const int* row_ptr; int m, n; long long nnz; void* base; int threshold, chunk_len, hub_cap; };
+    static std::mutex memo_mu;
+    static std::map<hipStream_t, Memo> memos;
+    bool planned;
+    if (store) {
+        planned = store->planned;
+    } else {
+        std::lock_guard<std::mutex> lock(memo_mu);
+        auto it = memos.find(s);
+        planned = reuse_plan && it != memos.end() && it->second.row_ptr == row_ptr && it->second.m == m && it->second.n == n &&
+                  it->second.nnz == nnz && it->second.base == base && it->second.threshold == threshold &&
+                  it->second.chunk_len == chunk_len && it->second.hub_cap == hub_cap;
+        if (!planned) memos[s] = Memo{row_ptr, m, n, nnz, base, threshold, chunk_len, hub_cap};
+    }
     if (!planned) {
         hipLaunchKernelGGL(hub_count_kernel, dim3(nb), dim3(kBlock), 0, s, m, row_ptr, bh, bc, threshold, chunk_len);
         if (nb <= kFillScanBlocks) {
@@ -398,7 +457,7 @@ int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_
             hipLaunchKernelGGL(hub_fill_kernel<false>, dim3(nb), dim3(kBlock), 0, s, m, nb, row_ptr, bh, bc, hub_cap, chunk_cap,
                                row_slot, hub_row, hub_chunk0, chunk_hub, hub_done, counts, threshold, chunk_len);
         }
-        memo = Memo{s, row_ptr, m, n, nnz, base, threshold, chunk_len, hub_cap};
+        if (store) store->planned = true;
     }
     if (vec4) {
         if (iters <= 1) launch_partial<4, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);

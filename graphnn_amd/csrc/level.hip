@@ -511,16 +511,8 @@ __global__ __launch_bounds__(kBlock) void s2v_readout_kernel(
     }
 }
 
-// Mean entries per row from which the two-launch route is taken; GNNHIP_TWO_STEP_DEGREE overrides it
-// (read once), which is how the crossover was measured.
-inline long long two_step_degree()
-{
-    static const long long d = [] {
-        const char* e = getenv("GNNHIP_TWO_STEP_DEGREE");
-        return (e && *e) ? atoll(e) : (long long)kTwoStepMeanDegree;
-    }();
-    return d;
-}
+// Mean entries per row from which the two-launch route is taken.
+inline long long two_step_degree() { return (long long)kTwoStepMeanDegree; }
 
 template <int C, int RT>
 int launch_input(int N, int K, const float* X, const float* Wn2l, float* msg, float* h0, hipStream_t s)
@@ -613,8 +605,9 @@ __global__ __launch_bounds__(kBlock) void identity_csr_kernel(int n, int* __rest
 
 int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
                    const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s, bool same_graph,
-                   bool relu_in)
+                   bool relu_in, CsrPlan* plan)
 {
+    // plan: made by gnnhip_csr_plan_create for exactly these CSR arrays (then nnz is the matrix's own count), or null
     // relu_in: h_in is read as ReLU(h_in); only where level_accepts_relu_input says so
     // same_graph: the previous call on this stream had the same A (a later level of one forward), so the
     // plan of the long-row pass is still in place and only its sums are redone
@@ -631,7 +624,10 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
         const bool two_step = N >= kHubMinRows && nnz >= two_step_degree() * (long long)N;
         if (relu_in && (two_step || !level_stream_covers(N, C))) return GNNHIP_EUNSUPPORTED;
         if (two_step) {
-            if (int rc = spmm_dispatch(N, N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, h_out, C, s, same_graph)) return rc;
+            // the streaming kernel knows the rows without entries from row_ptr and takes them as zero without reading
+            // them, so the product need not write them (on R-MAT more than half of the rows)
+            const bool skip_empty = level_stream_covers(N, C);
+            if (int rc = spmm_dispatch(N, N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, h_out, C, s, same_graph, skip_empty, plan)) return rc;
             const HubPlan none{nullptr, nullptr, 0};
             if (int rc = level_stream_dispatch(N, C, true, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, none, false, s);
                 rc != GNNHIP_EUNSUPPORTED)
@@ -643,7 +639,9 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
             }
         }
         HubPlan hubs{nullptr, nullptr, 0};
-        if (int rc = hub_prepass(N, C, nnz, row_ptr, col_idx, val, h_in, C, s, &hubs, same_graph, relu_in)) return rc;
+        if (int rc = hub_prepass(N, C, nnz, row_ptr, col_idx, val, h_in, C, s, &hubs, same_graph, relu_in, kHubThreshold, kHubChunk, -1,
+                                 plan ? &plan->row_hub : nullptr))
+            return rc;
         // activations of 4 GiB and more keep the kernel with 64-bit addressing below
         if (int rc = level_stream_dispatch(N, C, false, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, hubs, relu_in, s);
             rc != GNNHIP_EUNSUPPORTED)
@@ -669,7 +667,7 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
         int* id_row_ptr = static_cast<int*>(idp);
         int* id_col = id_row_ptr + N + 1;
         float* id_val = reinterpret_cast<float*>(id_col + N);
-        if (int rc = spmm_dispatch(N, N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, agg, C, s, same_graph)) return rc;
+        if (int rc = spmm_dispatch(N, N, C, nnz, 1.f, row_ptr, col_idx, val, h_in, C, 0.f, agg, C, s, same_graph, false, plan)) return rc;
         hipLaunchKernelGGL(identity_csr_kernel, dim3((unsigned)(((long long)N + kBlock) / kBlock)), dim3(kBlock), 0, s, N, id_row_ptr,
                            id_col, id_val);
         GNNHIP_LAUNCH_CHECK("identity_csr");

@@ -27,7 +27,8 @@
 // the register count and doubles the wavefronts per SIMD.
 //
 // DENSE: A * h_in has already been written to h_out (by the SpMM); the tile is read from there
-// and overwritten in place.
+// and overwritten in place.  Rows of A without entries (known from row_ptr) are taken as zero and not read, so the
+// product may leave them unwritten.
 //
 // Algorithmic bytes: 4(N+1) + 8E + 12NC + 4C^2.
 #include "gnnhip_internal.h"
@@ -178,7 +179,7 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
     // lane's register: only that part is compared with the buffer size.
     auto load_rp = [&](int (&rpx)[RN], int tile_id) {
 #pragma unroll
-        for (int i = 0; i < RN; ++i) rpx[i] = DENSE ? 0 : buf_load_i(rp_rsrc, (tile_id * 16 + grp * ROUNDS + i) * 4, 0);
+        for (int i = 0; i < RN; ++i) rpx[i] = buf_load_i(rp_rsrc, (tile_id * 16 + grp * ROUNDS + i) * 4, 0);
     };
     // First batch of a row: lane tx takes entry tx.  offs = byte offset of the entry's row of h_in, w = its
     // weight; lanes past the end of the row, and all lanes of a row that is gathered cooperatively (too
@@ -225,12 +226,18 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
         float w0n[ROUNDS];
 
         if constexpr (DENSE) {
+            // a row of A without entries was not written by the product: it counts as zero and is not read (an
+            // offset past the end returns zeros without a memory access)
+            float4 xd[ROUNDS];
 #pragma unroll
-            for (int rd = 0; rd < ROUNDS; ++rd) {
-                const int lr = grp * ROUNDS + rd;
-                const float4 x = buf_load4(out_rsrc, row_off(row0 + lr), 0);
-                *reinterpret_cast<float4*>(tile + lr * LDT + tx * 4) = x;
-            }
+            for (int rd = 0; rd < ROUNDS; ++rd)
+                xd[rd] = buf_load4(out_rsrc, rp[rd + 1] > rp[rd] ? row_off(row0 + grp * ROUNDS + rd) : kPastEndRow, 0);
+            load_rp(rpnn, tile_n2 < ntiles ? tile_n2 : ntiles);      // behind the rows: the pointers of the tile after next
+#pragma unroll
+            for (int rd = 0; rd < ROUNDS; ++rd)
+                *reinterpret_cast<float4*>(tile + (grp * ROUNDS + rd) * LDT + tx * 4) = xd[rd];
+#pragma unroll
+            for (int i = 0; i < RN; ++i) { rp[i] = rpn[i]; rpn[i] = rpnn[i]; }
         } else {
             // ---- the first four neighbours of every row of the tile, fetched together
             if constexpr (!PIPE) {

@@ -24,7 +24,8 @@
 // Bound: HBM / L2.  Algorithmic bytes as for the plain SpMM, plus 8 bytes of partial sums per column and piece.
 #include "gnnhip_internal.h"
 
-#include <cstdlib>
+#include <map>
+#include <set>
 
 namespace gnnhip {
 namespace {
@@ -32,17 +33,19 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kPiece = 32;              // entries per piece
 
-// entries [start, end); id = first[row] + index of the piece in its row; row: the row when the piece is all of it
-// and holds entries (then its sum is the row's result), else -1
+// entries [start, end); id: the place of the piece's sum among the partial sums, -1 when its row has no other piece;
+// row: the row when the piece is all of it and holds entries (then its sum is the row's result), else -1
 struct PieceRec { int start, end, id, row; };
+constexpr int kNoPlace = (int)0x80000000;   // target of a piece whose sum nobody reads
 
 __device__ __forceinline__ int pieces_of(int deg) { return (deg + kPiece - 1) / kPiece; }
 
-// counts[r] = pieces of row r (counts[m] = 0, so that the scan leaves the total there).  The host's entry count
-// `cap` sizes every array of the plan; should the matrix hold more entries than that, a row that reaches past
-// entry `cap` (the last rows) is one piece whatever its length: no entries are copied for it, and
-// piece_tail_kernel forms the row's result from the CSR arrays.
-__global__ __launch_bounds__(kBlock) void piece_count_kernel(int m, const int* __restrict__ row_ptr, int cap, int* __restrict__ counts)
+// counts[r] = pieces of row r, pcounts[r] = the same for rows of several pieces and 0 for the others (entry m of both
+// is 0, so that the scans leave the totals there).  The host's entry count `cap` sizes every array of the plan; should
+// the matrix hold more entries than that, a row that reaches past entry `cap` (the last rows) is one piece whatever
+// its length: no entries are copied for it, and piece_tail_kernel forms the row's result from the CSR arrays.
+__global__ __launch_bounds__(kBlock) void piece_count_kernel(int m, const int* __restrict__ row_ptr, int cap, int* __restrict__ counts,
+                                                             int* __restrict__ pcounts)
 {
     for (long long r = (long long)blockIdx.x * kBlock + threadIdx.x; r <= m; r += (long long)gridDim.x * kBlock) {
         int c = 0;
@@ -51,19 +54,23 @@ __global__ __launch_bounds__(kBlock) void piece_count_kernel(int m, const int* _
             c = e1 <= cap ? pieces_of(e1 - e0) : (e1 > e0 ? 1 : 0);
         }
         counts[r] = c;
+        pcounts[r] = c > 1 ? c : 0;
     }
 }
 
 // One lane per piece slot: the row that owns piece id is found by bisection in the scanned counts.
 // Slots at or past the number of pieces get an empty record and the largest key (they sort to the end).
+// rec.id: the place of the piece's sum among the partial sums (pfirst[row] + index of the piece in its row) when its row
+// has several pieces, else -1.
 __global__ __launch_bounds__(kBlock) void piece_fill_kernel(int m, long long slots, const int* __restrict__ row_ptr, int cap,
                                                             const int* __restrict__ col_idx, const int* __restrict__ first,
-                                                            int shift, PieceRec* __restrict__ rec, unsigned* __restrict__ keys)
+                                                            const int* __restrict__ pfirst, int shift, PieceRec* __restrict__ rec,
+                                                            unsigned* __restrict__ keys)
 {
     const int total = first[m];
     for (long long id = (long long)blockIdx.x * kBlock + threadIdx.x; id < slots; id += (long long)gridDim.x * kBlock) {
         if (id >= total) {
-            rec[id] = PieceRec{0, 0, (int)id, -1};
+            rec[id] = PieceRec{0, 0, -1, -1};
             keys[id] = 0xFFFFu;
             continue;
         }
@@ -77,29 +84,30 @@ __global__ __launch_bounds__(kBlock) void piece_fill_kernel(int m, long long slo
         const int rb = row_ptr[row], re = row_ptr[row + 1];
         const int start = rb + k * kPiece;
         const int end = re <= cap ? min(start + kPiece, re) : start;     // a row past the host's count: an empty stand-in
-        rec[id] = PieceRec{start, end, (int)id, (end > start && first[row + 1] - first[row] == 1) ? row : -1};
+        const bool alone = first[row + 1] - first[row] == 1;
+        rec[id] = PieceRec{start, end, alone ? -1 : pfirst[row] + k, (end > start && alone) ? row : -1};
         keys[id] = ((unsigned)col_idx[start] >> shift) & 0xFFFFu;
     }
 }
 
 // lens[i] = entries of the i-th piece in order (lens[slots] = 0, so that the scan leaves the total there);
-// where[i] = i and ones[i] = 1: the matrix that picks the pieces of a row (the sums are stored by piece id, so the
-// pieces of a row lie next to each other and the combining pass reads them front to back);
 // target[i]: where the sum of the i-th piece in order goes: the row r >= 0 when the piece is all of that row,
-// else -1 - id, its place among the partial sums.  order[i] = id of the i-th piece in order; ordered[i] = its record.
-__global__ __launch_bounds__(kBlock) void piece_place_kernel(long long slots, const unsigned* __restrict__ order,
+// else -1 - (its place among the partial sums; a stand-in piece without entries and without place gets a place past the
+// end, which the sum kernel recognises).  order[i] = id of the i-th piece in order; ordered[i] = its record.
+// where[j] = j and ones[j] = 1 for j < pslots: the matrix P that picks the partial sums of a row (the sums of a row's
+// pieces lie next to each other, so the combining pass reads them front to back).
+__global__ __launch_bounds__(kBlock) void piece_place_kernel(long long slots, long long pslots, const unsigned* __restrict__ order,
                                                              const PieceRec* __restrict__ rec, PieceRec* __restrict__ ordered,
                                                              int* __restrict__ lens, int* __restrict__ where, float* __restrict__ ones,
                                                              int* __restrict__ target)
 {
     for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i <= slots; i += (long long)gridDim.x * kBlock) {
+        if (i < pslots) { where[i] = (int)i; ones[i] = 1.f; }
         if (i == slots) { lens[i] = 0; continue; }
         const PieceRec r = rec[order[i]];
         ordered[i] = r;
         lens[i] = r.end - r.start;
-        where[i] = (int)i;
-        ones[i] = 1.f;
-        target[i] = r.row >= 0 ? r.row : -1 - r.id;
+        target[i] = r.row >= 0 ? r.row : (r.id >= 0 ? -1 - r.id : kNoPlace);
     }
 }
 
@@ -216,6 +224,7 @@ __global__ __launch_bounds__(kBlock) void piece_sum_kernel(
             }
         }
         const int row = target[i];
+        if (row == kNoPlace) return;
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
             const int col0 = (sub + it * G) * VEC;
@@ -275,18 +284,22 @@ __global__ __launch_bounds__(kBlock) void piece_tail_kernel(int m, int n, float 
 }
 
 // C[row] = sum of the row's partial sums + beta * C[row] for the rows of no piece or of several; a row of one piece
-// has its result already.  part holds the sums by piece id: row r owns part[first[r] .. first[r + 1]).  A lane group
-// takes kRun consecutive rows, whose pieces are one contiguous stretch of part, and adds each row's pieces in
+// has its result already.  first: pieces before each row; pfirst: row pointers into part, which holds the sums of the
+// rows of several pieces, a row's sums next to each other: row r owns part[pfirst[r] .. pfirst[r + 1]).  A lane group
+// takes kRun consecutive rows, whose sums are one contiguous stretch of part, and adds each row's pieces in
 // piece order, eight loads in flight.  A row of more than kCombineLong pieces takes its sum from the balanced
 // pass (hub_slot / hub_agg) when that pass has one for it: on a power-law matrix the rows of many pieces sit next
 // to each other, and summed here they kept an eighth of the wavefronts busy for the whole launch.
+// skip_empty: rows without entries are not written (the consumer knows them from row_ptr and reads zeros instead);
+// otherwise they get beta * C.
 constexpr int kRun = 8;
 constexpr int kCombineLong = 8;         // pieces; the balanced pass cuts such rows into chunks of kCombineChunk pieces
 constexpr int kCombineChunk = 256;
 template <int VEC, int ITERS>
 __global__ __launch_bounds__(kBlock) void piece_combine_kernel(
-    int m, int n, const int* __restrict__ first, const float* __restrict__ part, int ldp, float beta, float* __restrict__ C, int ldc,
-    int logG, const int* __restrict__ hub_slot, const float* __restrict__ hub_agg, int hub_ld)
+    int m, int n, const int* __restrict__ first, const int* __restrict__ pfirst, const float* __restrict__ part, int ldp, float beta,
+    float* __restrict__ C, int ldc, int logG, const int* __restrict__ hub_slot, const float* __restrict__ hub_agg, int hub_ld,
+    int skip_empty)
 {
     using V = PV<VEC>;
     constexpr int kFlight = 8;
@@ -298,12 +311,15 @@ __global__ __launch_bounds__(kBlock) void piece_combine_kernel(
     if (row0 >= m) return;
     // lane j < kRun of the group holds the bounds of row row0 + j
     const long long mine = row0 + (sub < kRun ? sub : 0);
-    const int my_b = first[mine < m ? mine : m], my_e = first[mine + 1 < m ? mine + 1 : m];
+    const long long lo_i = mine < m ? mine : m, hi_i = mine + 1 < m ? mine + 1 : m;
+    const int my_pieces = first[hi_i] - first[lo_i];
+    const int my_b = pfirst[lo_i], my_e = pfirst[hi_i];
     const int rows = (int)((long long)m - row0 < kRun ? (long long)m - row0 : kRun);
     for (int j = 0; j < rows; ++j) {
+        const int pieces = __shfl(my_pieces, j, G);
+        if (pieces == 1 || (pieces == 0 && skip_empty)) continue;
         const int b = __shfl(my_b, j, G), e = __shfl(my_e, j, G);
         const int cnt = e - b;
-        if (cnt == 1) continue;
         const long long row = row0 + j;
         typename V::T acc[ITERS];
 #pragma unroll
@@ -352,109 +368,134 @@ inline int ilog2_ceil_p(int x)
 }
 inline size_t round_up_p(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
-// Mean entries per row from which a matrix of at least kHubMinRows rows takes this route;
-// GNNHIP_PIECES_DEGREE overrides it (read once; 0 switches the route off), which is how the crossover was measured.
-inline long long pieces_degree()
+// Mean entries per row from which a matrix of at least kHubMinRows rows takes this route.
+constexpr long long kPiecesMeanDegree = 12;
+
+struct Width {            // how a lane group covers the columns of an operand of width n
+    bool ok, vec4;
+    int logG, iters, ldp;
+};
+Width width_of(int n, const float* B, int ldb, const float* C, int ldc)
 {
-    static const long long d = [] {
-        const char* e = getenv("GNNHIP_PIECES_DEGREE");
-        return (e && *e) ? atoll(e) : 12ll;
-    }();
-    return d;
+    Width w;
+    w.vec4 = (n % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && aligned16(B) && aligned16(C);
+    const int vec = w.vec4 ? 4 : 1;
+    const int units = (n + vec - 1) / vec;
+    // A lane group covers at most 64 x 4 column units (wider operands stay with the caller's route, which cuts them into
+    // slabs).  Narrow operands stay with the row-group route too: with fewer than eight lanes per piece a wavefront reads
+    // the entries of more than eight pieces at once, 128 bytes apart, and fetches whole lines for a few bytes each
+    // (width 4 on the 4M-row R-MAT matrix: 16.6 GB fetched, 2.7 ms against 0.26 ms).
+    w.ok = units <= kWave * 4 && units >= 8;
+    w.logG = ilog2_ceil_p(units < kWave ? units : kWave);
+    w.iters = (units + (1 << w.logG) - 1) >> w.logG;               // 1..4 (3 runs as 4)
+    w.ldp = (int)round_up_p((size_t)n, 4);
+    return w;
 }
 
-}  // namespace
+// Every row has at most one piece that is not full, and a row of several pieces has at least kPiece + 1 entries.
+inline long long slots_bound(int m, long long nnz) { return nnz / kPiece + m; }
+inline long long pslots_bound(long long nnz) { return nnz / kPiece + nnz / (kPiece + 1) + 1; }
 
-// The partial sums alpha * (piece of A) * B of every piece, in column order, and the matrix P that picks the pieces of
-// each row (out->first / where / ones: CSR arrays of P [m, out->slots], out->part: the sums, row stride out->ld);
-// A * B is P * part.  The rows of exactly one piece are finished here (C[row] = sum + beta * C[row]); the caller
-// combines the others.  GNNHIP_EUNSUPPORTED (nothing launched) where the caller keeps its own route.
-int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                     const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan, PiecesOperand* out)
+struct Layout {           // offsets inside the head, body and temporary blocks of a plan
+    size_t o_first, o_pfirst, head_bytes;
+    size_t o_at, o_target, o_where, o_ones, o_col, o_val, body_bytes;
+    size_t o_seg, o_rec, o_ord, o_keys, o_keys2, o_perm, o_perm2, o_hist, temp_bytes;
+};
+Layout layout_of(int m, long long nnz, long long slots, long long pslots)
 {
-    const long long deg = pieces_degree();
-    if (deg <= 0 || m < kHubMinRows || nnz < deg * (long long)m || nnz >= (1ll << 31) - 64) return GNNHIP_EUNSUPPORTED;
-    const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && aligned16(B) && aligned16(C);
-    const int vec = vec4 ? 4 : 1;
-    const int units = (n + vec - 1) / vec;
-    // a lane group covers at most 64 x 4 column units (wider operands stay with the caller's route, which cuts them into slabs)
-    if (units > kWave * 4) return GNNHIP_EUNSUPPORTED;
-    // Narrow operands stay with the row-group route: with fewer than eight lanes per piece a wavefront reads the
-    // entries of more than eight pieces at once, 128 bytes apart, and fetches whole lines for a few bytes each
-    // (width 4 on the 4M-row R-MAT matrix: 16.6 GB fetched, 2.7 ms against 0.26 ms).
-    if (units < 8) return GNNHIP_EUNSUPPORTED;
-    const int logG = ilog2_ceil_p(units < kWave ? units : kWave);
-    const int G = 1 << logG;
-    const int iters = (units + G - 1) / G;                        // 1..4 (3 runs as 4)
-    const int ldp = (int)round_up_p((size_t)n, 4);
-
-    // Every row has at most one piece that is not full.  The host does not know how many pieces there are, so
-    // the arrays and the launches are sized for this bound; the slots past the real pieces hold empty pieces,
-    // ordered last, that no row picks.
-    const long long slots = nnz / kPiece + m;
-    if (slots >= (1ll << 31) - 64) return GNNHIP_EUNSUPPORTED;
+    Layout L;
     size_t off = 0;
     auto carve = [&](size_t bytes) { const size_t o = off; off = round_up_p(off + bytes, 256); return o; };
-    const size_t o_first = carve(sizeof(int) * ((size_t)m + 1)), o_where = carve(sizeof(int) * (size_t)slots);
-    const size_t o_at = carve(sizeof(int) * ((size_t)slots + 1)), o_ones = carve(sizeof(float) * (size_t)slots);
-    const size_t o_target = carve(sizeof(int) * (size_t)slots);
-    const size_t o_col = carve(sizeof(int) * (size_t)nnz), o_val = carve(sizeof(float) * (size_t)nnz);
+    L.o_first = carve(sizeof(int) * ((size_t)m + 1));
+    L.o_pfirst = carve(sizeof(int) * ((size_t)m + 1));
+    L.head_bytes = off;
+    off = 0;
+    L.o_at = carve(sizeof(int) * ((size_t)slots + 1));
+    L.o_target = carve(sizeof(int) * (size_t)slots);
+    L.o_where = carve(sizeof(int) * (size_t)pslots);
+    L.o_ones = carve(sizeof(float) * (size_t)pslots);
+    L.o_col = carve(sizeof(int) * (size_t)nnz);
+    L.o_val = carve(sizeof(float) * (size_t)nnz);
+    L.body_bytes = off;
+    off = 0;
     const size_t longest = (size_t)(slots + 1 > (long long)m + 1 ? slots + 1 : (long long)m + 1);
-    const size_t o_seg = carve(sizeof(int) * (longest / 4096 + 2 + radix_seg_ints(slots)));
-    const size_t o_rec = carve(sizeof(PieceRec) * (size_t)slots), o_ord = carve(sizeof(PieceRec) * (size_t)slots);
-    const size_t o_keys = carve(sizeof(unsigned) * (size_t)slots), o_keys2 = carve(sizeof(unsigned) * (size_t)slots);
-    const size_t o_perm = carve(sizeof(unsigned) * (size_t)slots), o_perm2 = carve(sizeof(unsigned) * (size_t)slots);
-    const size_t o_hist = carve(sizeof(int) * radix_hist_ints(slots));
-    void* base = nullptr;
-    if (int rc = stream_scratch_slot(s, 3, off, &base)) return rc;
-    void* pbase = nullptr;
-    if (int rc = stream_scratch_slot(s, 4, sizeof(float) * (size_t)slots * ldp, &pbase)) return rc;
-    char* b = static_cast<char*>(base);
-    int* first = reinterpret_cast<int*>(b + o_first);
-    int* where = reinterpret_cast<int*>(b + o_where);
-    int* at = reinterpret_cast<int*>(b + o_at);
-    float* ones = reinterpret_cast<float*>(b + o_ones);
-    int* target = reinterpret_cast<int*>(b + o_target);
-    int* col_ord = reinterpret_cast<int*>(b + o_col);
-    float* val_ord = reinterpret_cast<float*>(b + o_val);
-    int* seg = reinterpret_cast<int*>(b + o_seg);
-    PieceRec* rec = reinterpret_cast<PieceRec*>(b + o_rec);
-    PieceRec* ordered = reinterpret_cast<PieceRec*>(b + o_ord);
-    unsigned* keys = reinterpret_cast<unsigned*>(b + o_keys);
-    unsigned* keys2 = reinterpret_cast<unsigned*>(b + o_keys2);
-    unsigned* perm = reinterpret_cast<unsigned*>(b + o_perm);
-    unsigned* order = reinterpret_cast<unsigned*>(b + o_perm2);
-    int* hist = reinterpret_cast<int*>(b + o_hist);
-    float* part = static_cast<float*>(pbase);
+    L.o_seg = carve(sizeof(int) * (longest / 4096 + 2 + radix_seg_ints(slots)));
+    L.o_rec = carve(sizeof(PieceRec) * (size_t)slots);
+    L.o_ord = carve(sizeof(PieceRec) * (size_t)slots);
+    L.o_keys = carve(sizeof(unsigned) * (size_t)slots);
+    L.o_keys2 = carve(sizeof(unsigned) * (size_t)slots);
+    L.o_perm = carve(sizeof(unsigned) * (size_t)slots);
+    L.o_perm2 = carve(sizeof(unsigned) * (size_t)slots);
+    L.o_hist = carve(sizeof(int) * radix_hist_ints(slots));
+    L.temp_bytes = off;
+    return L;
+}
 
-    struct Memo { hipStream_t s; const int* row_ptr; const int* col_idx; const float* val; int m; long long nnz; void* base; };
-    static thread_local Memo memo = {nullptr, nullptr, nullptr, nullptr, 0, 0, nullptr};
-    const bool planned = reuse_plan && memo.row_ptr == row_ptr && memo.col_idx == col_idx && memo.val == val && memo.s == s &&
-                         memo.m == m && memo.nnz == nnz && memo.base == base;
-    const unsigned egrid = kNumCU * 16;
-    if (!planned) {
-        hipLaunchKernelGGL(piece_count_kernel, dim3(egrid), dim3(kBlock), 0, s, m, row_ptr, (int)nnz, first);
-        if (int rc = exclusive_scan_i32(first, (long long)m + 1, seg, s)) return rc;
-        int bits = 1;
-        while (bits < 31 && (1ll << bits) < (long long)k) ++bits;
-        const int shift = bits > 16 ? bits - 16 : 0;
-        hipLaunchKernelGGL(piece_fill_kernel, dim3(egrid), dim3(kBlock), 0, s, m, slots, row_ptr, (int)nnz, col_idx, first, shift, rec, keys);
-        // two stable passes, low digit first: order[i] = id of the piece that comes i-th by the top 16 bits of its first column
-        if (int rc = radix_order_by_digit(keys, slots, 0, keys2, perm, hist, seg, s)) return rc;
-        if (int rc = radix_order_by_digit(keys2, slots, 8, keys, order, hist, seg, s, perm)) return rc;
-        hipLaunchKernelGGL(piece_place_kernel, dim3(egrid), dim3(kBlock), 0, s, slots, order, rec, ordered, at, where, ones, target);
-        if (int rc = exclusive_scan_i32(at, slots + 1, seg, s)) return rc;
-        hipLaunchKernelGGL(piece_gather_kernel, dim3(egrid), dim3(kBlock), 0, s, first + m, ordered, at, col_idx, val, col_ord, val_ord);
-        GNNHIP_LAUNCH_CHECK("spmm_pieces plan");
-        memo = Memo{s, row_ptr, col_idx, val, m, nnz, base};
-    }
-    // workgroups for the bound on the pieces of one die, times the number of dies
+constexpr unsigned kElemGrid = kNumCU * 16;
+
+// pieces per row and their scans: first, pfirst (the totals end up in entry m of each)
+int count_pieces(CsrPlan* p, int cap, int* seg, hipStream_t s)
+{
+    hipLaunchKernelGGL(piece_count_kernel, dim3(kElemGrid), dim3(kBlock), 0, s, p->m, p->row_ptr, cap, p->first, p->pfirst);
+    if (int rc = exclusive_scan_i32(p->first, (long long)p->m + 1, seg, s)) return rc;
+    if (int rc = exclusive_scan_i32(p->pfirst, (long long)p->m + 1, seg, s)) return rc;
+    GNNHIP_LAUNCH_CHECK("spmm_pieces count");
+    return GNNHIP_OK;
+}
+
+// the rest of the plan, from the scanned counts: records, order by first column, entries copied into that order
+int order_pieces(CsrPlan* p, int cap, const Layout& L, char* temp, hipStream_t s)
+{
+    int* seg = reinterpret_cast<int*>(temp + L.o_seg);
+    PieceRec* rec = reinterpret_cast<PieceRec*>(temp + L.o_rec);
+    PieceRec* ordered = reinterpret_cast<PieceRec*>(temp + L.o_ord);
+    unsigned* keys = reinterpret_cast<unsigned*>(temp + L.o_keys);
+    unsigned* keys2 = reinterpret_cast<unsigned*>(temp + L.o_keys2);
+    unsigned* perm = reinterpret_cast<unsigned*>(temp + L.o_perm);
+    unsigned* order = reinterpret_cast<unsigned*>(temp + L.o_perm2);
+    int* hist = reinterpret_cast<int*>(temp + L.o_hist);
+    int bits = 1;
+    while (bits < 31 && (1ll << bits) < (long long)p->k) ++bits;
+    const int shift = bits > 16 ? bits - 16 : 0;
+    hipLaunchKernelGGL(piece_fill_kernel, dim3(kElemGrid), dim3(kBlock), 0, s, p->m, p->slots, p->row_ptr, cap, p->col_idx, p->first,
+                       p->pfirst, shift, rec, keys);
+    // two stable passes, low digit first: order[i] = id of the piece that comes i-th by the top 16 bits of its first column
+    if (int rc = radix_order_by_digit(keys, p->slots, 0, keys2, perm, hist, seg, s)) return rc;
+    if (int rc = radix_order_by_digit(keys2, p->slots, 8, keys, order, hist, seg, s, perm)) return rc;
+    hipLaunchKernelGGL(piece_place_kernel, dim3(kElemGrid), dim3(kBlock), 0, s, p->slots, p->pslots, order, rec, ordered, p->at, p->where,
+                       p->ones, p->target);
+    if (int rc = exclusive_scan_i32(p->at, p->slots + 1, seg, s)) return rc;
+    hipLaunchKernelGGL(piece_gather_kernel, dim3(kElemGrid), dim3(kBlock), 0, s, p->first + p->m, ordered, p->at, p->col_idx, p->val,
+                       p->col_ord, p->val_ord);
+    GNNHIP_LAUNCH_CHECK("spmm_pieces plan");
+    return GNNHIP_OK;
+}
+
+void point_plan(CsrPlan* p, const Layout& L, char* head, char* body)
+{
+    p->first = reinterpret_cast<int*>(head + L.o_first);
+    p->pfirst = reinterpret_cast<int*>(head + L.o_pfirst);
+    p->at = reinterpret_cast<int*>(body + L.o_at);
+    p->target = reinterpret_cast<int*>(body + L.o_target);
+    p->where = reinterpret_cast<int*>(body + L.o_where);
+    p->ones = reinterpret_cast<float*>(body + L.o_ones);
+    p->col_ord = reinterpret_cast<int*>(body + L.o_col);
+    p->val_ord = reinterpret_cast<float*>(body + L.o_val);
+}
+
+// The sums over a finished plan: C = alpha * A * B + beta * C.  `part` holds p->pslots rows of w.ldp floats;
+// hub_store: where the balanced pass over P keeps its arrays (null: stream scratch slot 1, which the caller has reserved).
+int run_pieces(const CsrPlan* p, const Width& w, int n, float alpha, const float* B, int ldb, float beta, float* C, int ldc, float* part,
+               bool hub_planned, HubStore* hub_store, bool skip_empty, hipStream_t s)
+{
+    const int m = p->m, logG = w.logG, iters = w.iters, ldp = w.ldp;
+    // workgroups for the bound on the pieces of one die, times the number of dies; those past the real count leave at once
     const int sum_groups = kBlock >> logG;
-    const unsigned sgrid = (unsigned)(((slots + kNumXCD - 1) / kNumXCD + 1 + sum_groups - 1) / sum_groups) * kNumXCD;
-#define GNNHIP_PIECES_LAUNCH(V, I)                                                                                               \
-    hipLaunchKernelGGL((piece_sum_kernel<V, I>), dim3(sgrid), dim3(kBlock), 0, s, first + m, n, alpha, at, col_ord, val_ord, B, ldb, \
-                       part, ldp, logG, target, beta, C, ldc)
-    if (vec4) {
+    const unsigned sgrid = (unsigned)(((p->slots + kNumXCD - 1) / kNumXCD + 1 + sum_groups - 1) / sum_groups) * kNumXCD;
+#define GNNHIP_PIECES_LAUNCH(V, I)                                                                                            \
+    hipLaunchKernelGGL((piece_sum_kernel<V, I>), dim3(sgrid), dim3(kBlock), 0, s, p->first + m, n, alpha, p->at, p->col_ord, p->val_ord, B, \
+                       ldb, part, ldp, logG, p->target, beta, C, ldc)
+    if (w.vec4) {
         if (iters <= 1) GNNHIP_PIECES_LAUNCH(4, 1);
         else if (iters == 2) GNNHIP_PIECES_LAUNCH(4, 2);
         else GNNHIP_PIECES_LAUNCH(4, 4);
@@ -465,54 +506,36 @@ int spmm_pieces_sums(int m, int k, int n, long long nnz, float alpha, const int*
     }
 #undef GNNHIP_PIECES_LAUNCH
     GNNHIP_LAUNCH_CHECK("spmm_pieces sums");
-    // rows past the host's entry count, if any
-    const unsigned tgrid = kNumCU * 4;
-#define GNNHIP_PIECES_TAIL(V, I)                                                                                                  \
-    hipLaunchKernelGGL((piece_tail_kernel<V, I>), dim3(tgrid), dim3(kBlock), 0, s, m, n, alpha, row_ptr, (int)nnz, col_idx, val, \
+    if (!p->owned) {
+        // rows past the host's entry count, if any (a plan of its own knows the matrix's count)
+        const unsigned tgrid = kNumCU * 4;
+#define GNNHIP_PIECES_TAIL(V, I)                                                                                                   \
+    hipLaunchKernelGGL((piece_tail_kernel<V, I>), dim3(tgrid), dim3(kBlock), 0, s, m, n, alpha, p->row_ptr, (int)p->nnz, p->col_idx, p->val, \
                        B, ldb, beta, C, ldc, logG)
-    if (vec4) {
-        if (iters <= 1) GNNHIP_PIECES_TAIL(4, 1);
-        else if (iters == 2) GNNHIP_PIECES_TAIL(4, 2);
-        else GNNHIP_PIECES_TAIL(4, 4);
-    } else {
-        if (iters <= 1) GNNHIP_PIECES_TAIL(1, 1);
-        else if (iters == 2) GNNHIP_PIECES_TAIL(1, 2);
-        else GNNHIP_PIECES_TAIL(1, 4);
-    }
+        if (w.vec4) {
+            if (iters <= 1) GNNHIP_PIECES_TAIL(4, 1);
+            else if (iters == 2) GNNHIP_PIECES_TAIL(4, 2);
+            else GNNHIP_PIECES_TAIL(4, 4);
+        } else {
+            if (iters <= 1) GNNHIP_PIECES_TAIL(1, 1);
+            else if (iters == 2) GNNHIP_PIECES_TAIL(1, 2);
+            else GNNHIP_PIECES_TAIL(1, 4);
+        }
 #undef GNNHIP_PIECES_TAIL
-    GNNHIP_LAUNCH_CHECK("spmm_pieces tail");
-    out->first = first;
-    out->where = where;
-    out->ones = ones;
-    out->part = part;
-    out->ld = ldp;
-    out->slots = slots;
-    out->plan_reused = planned;
-    return GNNHIP_OK;
-}
-
-int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                         const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
-{
-    PiecesOperand po;
-    if (int rc = spmm_pieces_sums(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, s, reuse_plan, &po)) return rc;
-    // the rows of very many pieces: the balanced pass over long rows, on P = (first, where, ones) times part
-    // (`slots` stands in for the number of entries of P: an upper bound is all that pass needs)
+        GNNHIP_LAUNCH_CHECK("spmm_pieces tail");
+    }
+    // the rows of very many pieces: the balanced pass over long rows, on P = (pfirst, where, ones) times part
+    // (`pslots` stands in for the number of entries of P: an upper bound is all that pass needs; a row of more than
+    // kCombineLong pieces has more than kCombineLong * kPiece entries, which bounds the number of such rows)
     HubPlan hubs;
-    // (a row of more than kCombineLong pieces has more than kCombineLong * kPiece entries: that bounds their number)
-    if (int rc = hub_prepass(m, n, po.slots, po.first, po.where, po.ones, po.part, po.ld, s, &hubs, po.plan_reused, false, kCombineLong,
-                             kCombineChunk, nnz / ((long long)kCombineLong * kPiece + 1) + 1))
+    if (int rc = hub_prepass(m, n, p->pslots, p->pfirst, p->where, p->ones, part, ldp, s, &hubs, hub_planned, false, kCombineLong,
+                             kCombineChunk, p->nnz / ((long long)kCombineLong * kPiece + 1) + 1, hub_store))
         return rc;
-    const bool vec4 = (n % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && aligned16(B) && aligned16(C);
-    const int vec = vec4 ? 4 : 1;
-    const int units = (n + vec - 1) / vec;
-    const int logG = ilog2_ceil_p(units < kWave ? units : kWave);
-    const int iters = (units + (1 << logG) - 1) >> logG;
     const unsigned grid = (unsigned)(((long long)m + (long long)(kBlock >> logG) * kRun - 1) / ((long long)(kBlock >> logG) * kRun));
-#define GNNHIP_PIECES_COMBINE(V, I)                                                                                           \
-    hipLaunchKernelGGL((piece_combine_kernel<V, I>), dim3(grid), dim3(kBlock), 0, s, m, n, po.first, po.part, po.ld, beta, C, ldc, \
-                       logG, hubs.row_slot, hubs.agg, hubs.ld)
-    if (vec4) {
+#define GNNHIP_PIECES_COMBINE(V, I)                                                                                             \
+    hipLaunchKernelGGL((piece_combine_kernel<V, I>), dim3(grid), dim3(kBlock), 0, s, m, n, p->first, p->pfirst, part, ldp, beta, C, ldc, \
+                       logG, hubs.row_slot, hubs.agg, hubs.ld, skip_empty ? 1 : 0)
+    if (w.vec4) {
         if (iters <= 1) GNNHIP_PIECES_COMBINE(4, 1);
         else if (iters == 2) GNNHIP_PIECES_COMBINE(4, 2);
         else GNNHIP_PIECES_COMBINE(4, 4);
@@ -526,4 +549,193 @@ int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const 
     return GNNHIP_OK;
 }
 
+// What the scratch of a stream holds a plan for: kept per stream, next to the scratch it describes, so that whichever
+// thread plans on the stream replaces it.
+std::mutex g_memo_mu;
+std::map<hipStream_t, CsrPlan> g_memo;
+
+std::mutex g_plans_mu;
+std::set<CsrPlan*> g_plans;
+
+}  // namespace
+
+bool pieces_route_applies(int m, long long nnz)
+{
+    return m >= kHubMinRows && nnz >= kPiecesMeanDegree * (long long)m && nnz < (1ll << 31) - 64 && slots_bound(m, nnz) < (1ll << 31) - 64;
+}
+
+CsrPlan* as_csr_plan(void* handle)
+{
+    CsrPlan* p = static_cast<CsrPlan*>(handle);
+    std::lock_guard<std::mutex> lock(g_plans_mu);
+    return (p && g_plans.count(p) && p->magic == kCsrPlanMagic) ? p : nullptr;
+}
+
+// C = alpha * A * B + beta * C through the column-ordered pieces.  With `plan` (made by gnnhip_csr_plan_create for these
+// arrays) nothing is planned here; without it the plan is made in the stream's scratch, sized for the host's bounds, and
+// reused when reuse_plan says the previous call on the stream had the same matrix (structure and values).
+// All scratch is taken before the first launch: GNNHIP_ENOMEM and GNNHIP_EUNSUPPORTED leave C untouched.
+int spmm_pieces_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
+                         const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan, bool skip_empty_rows,
+                         CsrPlan* plan)
+{
+    const Width w = width_of(n, B, ldb, C, ldc);
+    if (!w.ok) return GNNHIP_EUNSUPPORTED;
+    if (skip_empty_rows && beta != 0.f) return set_error(GNNHIP_EINVAL, "rows without entries can only be skipped when beta is 0");
+    if (plan) {
+        if (!plan->has_pieces) return GNNHIP_EUNSUPPORTED;
+        const size_t need = sizeof(float) * (size_t)(plan->pslots > 0 ? plan->pslots : 1) * w.ldp;
+        if (plan->part_bytes < need) {
+            if (plan->part) {
+                GNNHIP_HIP(hipStreamSynchronize(s));
+                (void)pool_free(plan->part);
+                plan->part = nullptr;
+                plan->part_bytes = 0;
+            }
+            void* q = nullptr;
+            if (int rc = pool_acquire_exact(&q, need)) return rc;
+            plan->part = static_cast<float*>(q);
+            plan->part_bytes = need;
+        }
+        // the balanced pass over P takes its block before anything is launched (it is the only other allocation)
+        const size_t hb = hub_scratch_bytes(m, n, plan->pslots, kCombineLong, kCombineChunk, plan->nnz / ((long long)kCombineLong * kPiece + 1) + 1);
+        if (hb > plan->combine_hub.bytes) {
+            if (plan->combine_hub.base) {
+                GNNHIP_HIP(hipStreamSynchronize(s));
+                (void)pool_free(plan->combine_hub.base);
+                plan->combine_hub = HubStore{};
+            }
+            if (int rc = pool_acquire_exact(&plan->combine_hub.base, hb)) return rc;
+            plan->combine_hub.bytes = hb;
+        }
+        return run_pieces(plan, w, n, alpha, B, ldb, beta, C, ldc, plan->part, true, &plan->combine_hub, skip_empty_rows, s);
+    }
+
+    if (!pieces_route_applies(m, nnz)) return GNNHIP_EUNSUPPORTED;
+    CsrPlan p;
+    p.row_ptr = row_ptr; p.col_idx = col_idx; p.val = val;
+    p.m = m; p.k = k; p.nnz = nnz;
+    p.slots = slots_bound(m, nnz);
+    p.pslots = pslots_bound(nnz) < p.slots ? pslots_bound(nnz) : p.slots;
+    p.has_pieces = true;
+    const Layout L = layout_of(m, nnz, p.slots, p.pslots);
+    void *base = nullptr, *pbase = nullptr, *hbase = nullptr;
+    if (int rc = stream_scratch_slot(s, 3, L.head_bytes + L.body_bytes + L.temp_bytes, &base)) return rc;
+    if (int rc = stream_scratch_slot(s, 4, sizeof(float) * (size_t)p.pslots * w.ldp, &pbase)) return rc;
+    // the balanced pass over P reserves its scratch now: past this point nothing can fail for lack of memory, so a
+    // caller that falls back to another route on GNNHIP_ENOMEM finds C untouched
+    if (const size_t hb = hub_scratch_bytes(m, n, p.pslots, kCombineLong, kCombineChunk, nnz / ((long long)kCombineLong * kPiece + 1) + 1))
+        if (int rc = stream_scratch_slot(s, 1, hb, &hbase)) return rc;
+    char* b = static_cast<char*>(base);
+    point_plan(&p, L, b, b + L.head_bytes);
+    char* temp = b + L.head_bytes + L.body_bytes;
+
+    bool planned = false;
+    {
+        std::lock_guard<std::mutex> lock(g_memo_mu);
+        auto it = g_memo.find(s);
+        planned = reuse_plan && it != g_memo.end() && it->second.row_ptr == row_ptr && it->second.col_idx == col_idx &&
+                  it->second.val == val && it->second.m == m && it->second.k == k && it->second.nnz == nnz && it->second.first == p.first;
+        if (!planned) g_memo[s] = p;
+    }
+    if (!planned) {
+        if (int rc = count_pieces(&p, (int)nnz, reinterpret_cast<int*>(temp + L.o_seg), s)) return rc;
+        if (int rc = order_pieces(&p, (int)nnz, L, temp, s)) return rc;
+    }
+    return run_pieces(&p, w, n, alpha, B, ldb, beta, C, ldc, static_cast<float*>(pbase), planned, nullptr, skip_empty_rows, s);
+}
+
 }  // namespace gnnhip
+
+using namespace gnnhip;
+
+extern "C" int gnnhip_csr_plan_create(int m, int k, const int* row_ptr, const int* col_idx, const float* val, void* stream, void** plan)
+{
+    GNNHIP_REQUIRE(plan, "null plan output");
+    *plan = nullptr;
+    GNNHIP_REQUIRE(m >= 0 && k >= 0, "negative dimension in csr_plan_create (m=%d k=%d)", m, k);
+    GNNHIP_REQUIRE(row_ptr, "null row_ptr in csr_plan_create");
+    if (int rc = require_ready()) return rc;
+    hipStream_t s = as_stream(stream);
+    // the matrix's own entry count
+    int nnz = 0;
+    GNNHIP_HIP(hipMemcpyAsync(&nnz, row_ptr + m, sizeof(int), hipMemcpyDeviceToHost, s));
+    GNNHIP_HIP(hipStreamSynchronize(s));
+    GNNHIP_REQUIRE(nnz >= 0, "row_ptr[m] is negative (%d)", nnz);
+    GNNHIP_REQUIRE(nnz == 0 || (col_idx && val), "null col_idx or val for a matrix with entries");
+    CsrPlan* p = new CsrPlan();
+    p->magic = kCsrPlanMagic;
+    p->row_ptr = row_ptr; p->col_idx = col_idx; p->val = val;
+    p->m = m; p->k = k; p->nnz = nnz;
+    p->owned = true;
+    auto fail = [&](int rc) {
+        if (p->head_block) (void)pool_free(p->head_block);
+        if (p->body_block) (void)pool_free(p->body_block);
+        delete p;
+        return rc;
+    };
+    if (pieces_route_applies(m, nnz)) {
+        // counts first (they need the head block only), then the arrays at the size the matrix really needs
+        Layout L = layout_of(m, nnz, 1, 1);
+        if (int rc = pool_acquire_exact(&p->head_block, L.head_bytes)) return fail(rc);
+        void* segp = nullptr;
+        if (int rc = stream_scratch(s, sizeof(int) * ((size_t)m / 4096 + 4), &segp)) return fail(rc);
+        point_plan(p, L, static_cast<char*>(p->head_block), nullptr);
+        if (int rc = count_pieces(p, nnz, static_cast<int*>(segp), s)) return fail(rc);
+        int totals[2] = {0, 0};
+        GNNHIP_HIP(hipMemcpyAsync(&totals[0], p->first + m, sizeof(int), hipMemcpyDeviceToHost, s));
+        GNNHIP_HIP(hipMemcpyAsync(&totals[1], p->pfirst + m, sizeof(int), hipMemcpyDeviceToHost, s));
+        GNNHIP_HIP(hipStreamSynchronize(s));
+        p->slots = totals[0] > 0 ? totals[0] : 1;
+        p->pslots = totals[1] > 0 ? totals[1] : 1;
+        L = layout_of(m, nnz, p->slots, p->pslots);
+        if (int rc = pool_acquire_exact(&p->body_block, L.body_bytes)) return fail(rc);
+        void* temp = nullptr;
+        if (int rc = pool_acquire_exact(&temp, L.temp_bytes)) return fail(rc);
+        point_plan(p, L, static_cast<char*>(p->head_block), static_cast<char*>(p->body_block));
+        int rc = order_pieces(p, nnz, L, static_cast<char*>(temp), s);
+        hipError_t e = hipStreamSynchronize(s);                    // the temporary arrays go back to the driver right away
+        (void)pool_free(temp);
+        if (rc) return fail(rc);
+        if (e != hipSuccess) return fail(set_error(GNNHIP_EHIP, "csr_plan_create: %s", hipGetErrorString(e)));
+        p->has_pieces = true;
+    }
+    {
+        std::lock_guard<std::mutex> lock(g_plans_mu);
+        g_plans.insert(p);
+    }
+    *plan = p;
+    return GNNHIP_OK;
+}
+
+extern "C" int gnnhip_csr_plan_destroy(void* plan)
+{
+    if (!plan) return GNNHIP_OK;
+    CsrPlan* p = static_cast<CsrPlan*>(plan);
+    {
+        std::lock_guard<std::mutex> lock(g_plans_mu);
+        if (!g_plans.erase(p)) return set_error(GNNHIP_EINVAL, "%p is not a live CSR plan", plan);
+    }
+    if (runtime_ready()) {
+        (void)hipDeviceSynchronize();                               // launches that read the plan's arrays may still be queued
+        for (void* q : {p->head_block, p->body_block, static_cast<void*>(p->part), p->combine_hub.base, p->row_hub.base})
+            if (q) (void)pool_free(q);
+    }
+    p->magic = 0;
+    delete p;
+    return GNNHIP_OK;
+}
+
+extern "C" int gnnhip_csr_plan_bytes(void* plan, size_t* bytes)
+{
+    GNNHIP_REQUIRE(bytes, "null output in csr_plan_bytes");
+    CsrPlan* p = as_csr_plan(plan);
+    GNNHIP_REQUIRE(p, "%p is not a live CSR plan", plan);
+    size_t total = p->part_bytes + p->combine_hub.bytes + p->row_hub.bytes;
+    if (p->has_pieces) {
+        const Layout L = layout_of(p->m, p->nnz, p->slots, p->pslots);
+        total += L.head_bytes + L.body_bytes;
+    }
+    *bytes = total;
+    return GNNHIP_OK;
+}

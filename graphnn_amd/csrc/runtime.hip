@@ -114,6 +114,33 @@ int pool_acquire(void** p, size_t bytes)
     return GNNHIP_OK;
 }
 
+// A block of exactly `bytes` (rounded to the granule) straight from the driver, known to the pool (pool_free or
+// shutdown returns it): for long-lived blocks of hundreds of megabytes, which must not take a larger parked block.
+int pool_acquire_exact(void** p, size_t bytes)
+{
+    if (!p) return set_error(GNNHIP_EINVAL, "null output pointer");
+    *p = nullptr;
+    Runtime& r = rt();
+    std::lock_guard<std::mutex> lock(r.mu);
+    if (!r.ready) return set_error(GNNHIP_ENOTINIT, "gnnhip_init has not been called");
+    if (bytes == 0) bytes = 1;
+    const size_t want = (bytes + kAllocGranule - 1) / kAllocGranule * kAllocGranule;
+    void* q = nullptr;
+    hipError_t e = hipMalloc(&q, want);
+    if (e != hipSuccess || q == nullptr) {
+        (void)hipGetLastError();
+        return set_error(GNNHIP_ENOMEM, "hipMalloc of %zu bytes failed: %s", want, hipGetErrorString(e));
+    }
+    r.all[q] = want;
+    r.live[q] = want;
+    r.bytes_in_use += want;
+    r.n_driver_allocs += 1;
+    *p = q;
+    return GNNHIP_OK;
+}
+
+int pool_free(void* p) { return gnnhip_free(p); }
+
 int pool_release(void* p)
 {
     if (!p) return GNNHIP_OK;
@@ -142,7 +169,16 @@ int stream_scratch_slot(hipStream_t s, int which, size_t bytes, void** p)
     auto& slot = r.scratch[std::make_pair(s, which)];
     if (slot.second < bytes) {
         size_t want = (bytes + 65535) / 65536 * 65536;
-        if (want < slot.second * 2) want = slot.second * 2;
+        const bool exact = which >= kExactScratchSlot;
+        if (!exact && want < slot.second * 2) want = slot.second * 2;
+        if (exact && slot.first) {
+            // these slots run to gigabytes: the old block goes before the new one comes, so that the peak is the need
+            // (kernels queued earlier on this stream may still read it)
+            (void)hipStreamSynchronize(s);
+            (void)hipFree(slot.first);
+            slot.first = nullptr;
+            slot.second = 0;
+        }
         void* q = nullptr;
         hipError_t e = hipMalloc(&q, want);
         if (e != hipSuccess || !q) {
@@ -217,6 +253,24 @@ int gnnhip_shutdown(void)
     r.bytes_in_use = r.bytes_parked = 0;
     r.ready = false;
     r.device = -1;
+    return GNNHIP_OK;
+}
+
+int gnnhip_release_scratch(void* stream)
+{
+    Runtime& r = rt();
+    std::lock_guard<std::mutex> lock(r.mu);
+    if (!r.ready) return GNNHIP_OK;
+    hipStream_t s = as_stream(stream);
+    GNNHIP_HIP(hipStreamSynchronize(s));
+    for (auto it = r.scratch.begin(); it != r.scratch.end();) {
+        if (it->first.first == s) {
+            (void)hipFree(it->second.first);
+            it = r.scratch.erase(it);
+        } else {
+            ++it;
+        }
+    }
     return GNNHIP_OK;
 }
 

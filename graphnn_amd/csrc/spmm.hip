@@ -229,20 +229,22 @@ int launch_slab(int m, int n, float alpha, const int* row_ptr, const int* col_id
 
 // Shared with the fused forward: C = alpha*A*B + beta*C on stream s.
 int spmm_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                  const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
+                  const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan, bool skip_empty_rows,
+                  CsrPlan* plan)
 {
-    // large matrices with many entries per row (power-law graphs): rows cut into pieces, summed in column order
-    // (its scratch, about 40 bytes per entry of A + 4 n bytes per piece, is taken before anything is launched: when
-    // the device cannot give it, the row-group route below, which needs far less, does the product)
-    if (int rc = spmm_pieces_dispatch(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, s, reuse_plan);
+    // large matrices with many entries per row (power-law graphs): rows cut into pieces, summed in column order.  That
+    // route takes all its scratch (about 40 bytes per entry of A + 4 n bytes per piece) before its first launch: when
+    // the device cannot give it, C is untouched and the row-group route below, which needs far less, does the product.
+    if (int rc = spmm_pieces_dispatch(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, s, reuse_plan, skip_empty_rows, plan);
         rc != GNNHIP_EUNSUPPORTED && rc != GNNHIP_ENOMEM)
         return rc;
-    return spmm_plain_dispatch(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, s, reuse_plan);
+    return spmm_plain_dispatch(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, s, reuse_plan, plan ? &plan->row_hub : nullptr);
 }
 
-// The row-group route alone (with its pass over very long rows); nnz may be an upper bound.
+// The row-group route alone (with its pass over very long rows); nnz may be an upper bound.  row_hub: where a plan's
+// owner keeps the pass's arrays across calls.
 int spmm_plain_dispatch(int m, int k, int n, long long nnz, float alpha, const int* row_ptr, const int* col_idx, const float* val,
-                        const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan)
+                        const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s, bool reuse_plan, HubStore* row_hub)
 {
     (void)k;
     // few rows of hundreds of entries each (sum-pooling into subgraphs): a workgroup per row instead of a lane group
@@ -261,7 +263,7 @@ int spmm_plain_dispatch(int m, int k, int n, long long nnz, float alpha, const i
         float* Cs = C + col0;
         int rc;
         HubPlan hubs;
-        if ((rc = hub_prepass(m, w, nnz, row_ptr, col_idx, val, Bs, ldb, s, &hubs, reuse_plan && n <= slab_max))) return rc;
+        if ((rc = hub_prepass(m, w, nnz, row_ptr, col_idx, val, Bs, ldb, s, &hubs, reuse_plan && n <= slab_max, false, kHubThreshold, kHubChunk, -1, row_hub))) return rc;
         if (vec4) {
             if (iters <= 1) rc = launch_slab<4, 1>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, one_row, s);
             else if (iters == 2) rc = launch_slab<4, 2>(m, w, alpha, row_ptr, col_idx, val, Bs, ldb, beta, Cs, ldc, logG, hubs, one_row, s);
@@ -291,4 +293,18 @@ extern "C" int gnnhip_spmm_csr_f32(int m, int k, int n, int nnz, float alpha, co
     GNNHIP_REQUIRE(k == 0 || B, "null dense operand in spmm");   // col_idx / val may be null when A has no entries
     if (int rc = require_ready()) return rc;
     return spmm_dispatch(m, k, n, nnz, alpha, row_ptr, col_idx, val, B, ldb, beta, C, ldc, as_stream(stream));
+}
+
+extern "C" int gnnhip_spmm_csr_planned_f32(void* plan, int n, float alpha, const float* B, int ldb, float beta, float* C, int ldc,
+                                           void* stream)
+{
+    CsrPlan* p = as_csr_plan(plan);
+    GNNHIP_REQUIRE(p, "%p is not a live CSR plan", plan);
+    GNNHIP_REQUIRE(n >= 0, "negative width in spmm_csr_planned (n=%d)", n);
+    if (p->m == 0 || n == 0) return GNNHIP_OK;
+    GNNHIP_REQUIRE(C, "null output in spmm_csr_planned");
+    GNNHIP_REQUIRE(ldb >= n && ldc >= n, "leading dimension smaller than n in spmm_csr_planned (ldb=%d ldc=%d n=%d)", ldb, ldc, n);
+    GNNHIP_REQUIRE(p->k == 0 || B, "null dense operand in spmm_csr_planned");
+    if (int rc = require_ready()) return rc;
+    return spmm_dispatch(p->m, p->k, n, p->nnz, alpha, p->row_ptr, p->col_idx, p->val, B, ldb, beta, C, ldc, as_stream(stream), false, false, p);
 }

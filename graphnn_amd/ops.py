@@ -77,6 +77,63 @@ def spmm(row_ptr, col_idx, val, B, m, alpha=1.0, beta=0.0, out=None, nnz_hint=No
     return out
 
 
+class CsrPlan:
+    """gnnhip_csr_plan_create for a CSR matrix [m, k] held in torch tensors, which the plan keeps alive; close() (or
+    the end of a `with` block) destroys it.  spmm / level run the planned entry points."""
+
+    def __init__(self, row_ptr, col_idx, val, m, k):
+        _check_csr(row_ptr, col_idx, val, m, "A")
+        self.m, self.k = int(m), int(k)
+        self._keep = (row_ptr, col_idx, val)
+        h = ctypes.c_void_p()
+        check(_lib().gnnhip_csr_plan_create(self.m, self.k, _i32(row_ptr, "row_ptr"), _i32(col_idx, "col_idx"), _f32(val, "val"),
+                                            _stream(), ctypes.byref(h)))
+        self.handle = h
+
+    def bytes(self):
+        n = ctypes.c_size_t()
+        check(_lib().gnnhip_csr_plan_bytes(self.handle, ctypes.byref(n)))
+        return int(n.value)
+
+    def spmm(self, B, alpha=1.0, beta=0.0, out=None):
+        k, n = B.shape
+        if k != self.k:
+            raise ValueError("B must have %d rows" % self.k)
+        if out is None:
+            out = torch.empty((self.m, n), dtype=torch.float32, device=B.device)
+        elif tuple(out.shape) != (self.m, n):
+            raise ValueError("out has the wrong shape")
+        check(_lib().gnnhip_spmm_csr_planned_f32(self.handle, n, alpha, _f32(B, "B"), n, beta, _f32(out, "out"), n, _stream()))
+        return out
+
+    def level(self, h_in, W, msg=None, bias=None, out=None):
+        N, C = h_in.shape
+        if N != self.m or tuple(W.shape) != (C, C):
+            raise ValueError("h_in must be [m,C] and W [C,C]")
+        if out is None:
+            out = torch.empty_like(h_in)
+        check(_lib().gnnhip_s2v_level_planned_f32(self.handle, C, _f32(h_in, "h_in"), _f32(W, "W"), _f32(msg, "msg"),
+                                                  _f32(bias, "bias"), _f32(out, "out"), _stream()))
+        return out
+
+    def close(self):
+        if self.handle is not None:
+            check(_lib().gnnhip_csr_plan_destroy(self.handle))
+            self.handle = None
+            self._keep = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+
+def release_scratch():
+    """gives the current stream's library scratch back to the driver"""
+    check(_lib().gnnhip_release_scratch(_stream()))
+
+
 def gemm(A, B, transA=False, transB=False, alpha=1.0, beta=0.0, out=None):
     m = A.shape[1] if transA else A.shape[0]
     k = A.shape[0] if transA else A.shape[1]

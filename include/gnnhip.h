@@ -17,6 +17,8 @@
  *
  * Each declaration cites the reference interface it stands in for
  * (paths relative to the graphnn source tree).
+ *
+ * The library reads no environment variable: which kernel a call takes depends on its arguments alone.
  */
 #ifndef GNNHIP_H
 #define GNNHIP_H
@@ -64,6 +66,10 @@ int gnnhip_malloc(void** device_ptr, size_t bytes);
 int gnnhip_recycle(void* device_ptr);
 int gnnhip_free(void* device_ptr);
 int gnnhip_pool_stats(size_t* bytes_in_use, size_t* bytes_parked, size_t* n_driver_allocs);
+/* Scratch the library keeps per stream (plans and partial sums of products with large matrices run to gigabytes; the
+ * reference's counterpart is the temporary storage its cuSPARSE / cuBLAS handles keep, src/tensor/gpu_handle.cu:17-70):
+ * waits for the stream and gives that stream's scratch back to the driver.  The next call that needs scratch takes it anew. */
+int gnnhip_release_scratch(void* stream);
 
 /* ---- copies: DTensor<GPU>::CopyFrom / AsScalar / Zeros
  *      (src/tensor/gpu_dense_tensor.cu:97-150), SpTensor<GPU>::CopyFrom
@@ -102,6 +108,26 @@ int gnnhip_stream_sync(void* stream);
 int gnnhip_spmm_csr_f32(int m, int k, int n, int nnz, float alpha, const int* row_ptr, const int* col_idx,
                         const float* val, const float* B, int ldb, float beta, float* C, int ldc,
                         void* stream);
+
+/* ---- a plan for a CSR matrix that is multiplied with many times: what DTensor<GPU>::MM(SpTensor, DTensor, N, N)
+ *      (src/tensor/gpu_dense_tensor.cu:227-239,257-270) would work out again on every call for the same operand
+ *      (the reference holds its sparse operand in SpTensor<GPU>, src/tensor/gpu_sparse_tensor.cu:25-63, across all the
+ *      levels of a batch and across batches of one big graph).  For large matrices with many entries per row
+ *      (power-law graphs) the plan holds the rows cut into pieces of consecutive entries, ordered by the column they
+ *      start at, and the entries copied into that order; for every matrix the plan of the balanced pass over long
+ *      rows.  plan_create reads the matrix on `stream`, blocks until the plan is built (it reads back the number of
+ *      pieces to size its arrays exactly), and owns pool memory of about 8 bytes per entry plus 16 per piece; the
+ *      partial sums of a product (4n bytes per piece of a row of several pieces) are added at the first use.
+ *      The CSR arrays must stay alive and unchanged (structure and values) while the plan is used; when they change,
+ *      destroy the plan and make a new one.  Calls that share a plan must be ordered one after the other (they share its partial
+ *      sums); plan_destroy waits for the device.  spmm_csr_planned / s2v_level_planned give bit-identical results to
+ *      gnnhip_spmm_csr_f32 / gnnhip_s2v_level_f32 on the same arrays (same kernels, same order of every sum).
+ *      plan_bytes: device bytes the plan owns at present. */
+int gnnhip_csr_plan_create(int m, int k, const int* row_ptr, const int* col_idx, const float* val, void* stream, void** plan);
+int gnnhip_csr_plan_destroy(void* plan);
+int gnnhip_csr_plan_bytes(void* plan, size_t* bytes);
+int gnnhip_spmm_csr_planned_f32(void* plan, int n, float alpha, const float* B, int ldb, float beta, float* C, int ldc,
+                                void* stream);
 
 /* ---- CSR from (key, payload) pairs on the device: row i lists the payloads of the pairs with key i in
  *      input order, i.e. what the message-pass factors build on the host from the per-node lists:
@@ -171,6 +197,11 @@ int gnnhip_gemm_tn_batch_f32(int count, const int* m, const int* n, const int* k
 int gnnhip_s2v_level_f32(int N, int C, int nnz, const int* row_ptr, const int* col_idx, const float* val,
                          const float* h_in, const float* W, const float* msg, const float* bias,
                          float* h_out, void* stream);
+
+/* ---- the same level with the plan of A (gnnhip_csr_plan_create; A must be square): the levels of
+ *      examples/graph_classification/src/kernel_mean_field.cpp:35-42 all multiply with the same n2nsum_param. */
+int gnnhip_s2v_level_planned_f32(void* plan, int C, const float* h_in, const float* W, const float* msg, const float* bias,
+                                 float* h_out, void* stream);
 
 /* ---- msg = X * W_n2l and h0 = ReLU(msg) in one pass
  *      (examples/graph_classification/src/kernel_mean_field.cpp:31-32: MatMul + ReLU).  X [N,K], W_n2l [K,C].

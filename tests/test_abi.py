@@ -66,6 +66,24 @@ def test_argument_validation_needs_no_gpu():
     assert lib.gnnhip_memset0(None, 0, None) == 0
 
 
+def test_plan_entries_reject_what_is_not_a_plan():
+    lib = binding.load_library()
+    x = np.zeros(8, np.float32)
+    p = x.ctypes.data_as(ctypes.c_void_p)
+    f = ctypes.c_float
+    assert lib.gnnhip_spmm_csr_planned_f32(p, 4, f(1), p, 4, f(0), p, 4, None) == -1
+    assert b"not a live CSR plan" in lib.gnnhip_last_error()
+    assert lib.gnnhip_s2v_level_planned_f32(None, 64, p, p, None, None, p, None) == -1
+    assert lib.gnnhip_csr_plan_destroy(None) == 0
+    assert lib.gnnhip_csr_plan_destroy(p) == -1
+    n = ctypes.c_size_t()
+    assert lib.gnnhip_csr_plan_bytes(p, ctypes.byref(n)) == -1
+    h = ctypes.c_void_p()
+    assert lib.gnnhip_csr_plan_create(-1, 1, p, p, p, None, ctypes.byref(h)) == -1
+    assert lib.gnnhip_csr_plan_create(1, 1, None, p, p, None, ctypes.byref(h)) == -1
+    assert lib.gnnhip_csr_plan_create(1, 1, p, p, p, None, None) == -1
+
+
 def test_compute_before_init_is_refused():
     import torch
     if torch.cuda.is_available():

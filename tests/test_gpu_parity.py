@@ -11,7 +11,7 @@ import os
 import numpy as np
 import pytest
 
-from conftest import FLOOR_POOL, FLOOR_PROBS_ABS, PARITY_TOL, Lazy, assert_parity, assert_stages, forward_float64, max_rel
+from conftest import FLOOR_POOL, FLOOR_PROBS_ABS, PARITY_TOL, Lazy, assert_condition, assert_parity, assert_stages, forward_float64, max_rel
 from graphnn_amd import batching, synth
 
 pytestmark = pytest.mark.gpu
@@ -1512,6 +1512,100 @@ def test_spmm_column_ordered_pieces_on_a_power_law_matrix(gpu, oracle, n):
         assert 0 < inside.sum() < N
         assert np.array_equal(got_h[inside], got2[inside]), hint
         assert_parity("spmm", got_h, *_spmm_want(oracle, *csr, B, N, alpha=-0.5, beta=1.5, C=C0))
+
+
+@pytest.mark.parametrize("n", [64, 128, 36, 9, 4, 300, 1100])
+def test_spmm_with_a_plan_has_the_bits_of_the_call_without(gpu, oracle, n):
+    """gnnhip_csr_plan_create + gnnhip_spmm_csr_planned_f32 on the power-law matrix of the test above: the plan sizes its
+    arrays for the pieces the matrix really has, the product runs the same kernels in the same order, so every bit
+    equals gnnhip_spmm_csr_f32's; also with beta, on a second and third call, at another width through the same plan
+    (its partial sums grow), and against the oracle"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(900 + n)
+    a = synth.rmat_csr(0x5EED0005, 16, 16 << 16)
+    N = 1 << 16
+    v = (rng.random(a[1].size) * 0.2 - 0.05).astype(np.float32)
+    csr = (a[0], a[1], v)
+    csr_d = _csr_t(csr, gpu)
+    B = rng.standard_normal((N, n)).astype(np.float32)
+    C0 = rng.standard_normal((N, n)).astype(np.float32)
+    B_d = _t(B, gpu)
+    plain = _n(ops.spmm(*csr_d, B_d, N))
+    plain2 = _n(ops.spmm(*csr_d, B_d, N, alpha=-0.5, beta=1.5, out=_t(C0, gpu)))
+    with ops.CsrPlan(*csr_d, N, N) as plan:
+        first_bytes = plan.bytes()
+        got = _n(plan.spmm(B_d))
+        assert np.array_equal(got, plain)
+        assert np.array_equal(_n(plan.spmm(B_d, alpha=-0.5, beta=1.5, out=_t(C0, gpu))), plain2)
+        assert np.array_equal(_n(plan.spmm(B_d)), plain)
+        # another width through the same plan, then the first one again
+        B8 = rng.standard_normal((N, 72)).astype(np.float32)
+        assert np.array_equal(_n(plan.spmm(_t(B8, gpu))), _n(ops.spmm(*csr_d, _t(B8, gpu), N)))
+        assert np.array_equal(_n(plan.spmm(B_d)), plain)
+        assert plan.bytes() >= first_bytes
+        # the plan's arrays: 8 bytes per entry, 8 per row, 16 per piece and less than that again for the balanced pass
+        pieces = int(np.ceil(np.diff(a[0]) / 32).sum())
+        assert first_bytes <= 8 * a[1].size + 8 * (N + 1) + 16 * pieces + (1 << 16)
+    want, w64 = _spmm_want(oracle, *csr, B, N)
+    assert_parity("spmm", got, want, w64)
+
+
+def test_plan_of_matrices_that_take_the_other_routes(gpu, oracle):
+    """a plan is made for any matrix: small ones, sparse ones and ones with a few very long rows keep the row-group
+    route (with the balanced pass over long rows, whose plan is then kept); no rows, no entries"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(901)
+    cases = [_random_csr(rng, 517, 389, 4000), _random_csr(rng, 40_000, 40_000, 90_000),
+             _hub_matrix(rng, 36_000, 36_000, [(0, 12000), (5, 300), (17, 65), (20000, 3000), (35_999, 1000)]),
+             (np.zeros(8, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32))]
+    for rp, ci, v in cases:
+        m = rp.size - 1
+        k = 389 if m == 517 else max(m, 1)
+        B = rng.standard_normal((k, 64)).astype(np.float32)
+        csr_d = _csr_t((rp, ci, v), gpu)
+        with ops.CsrPlan(*csr_d, m, k) as plan:
+            for _ in range(2):
+                got = _n(plan.spmm(_t(B, gpu)))
+                assert np.array_equal(got, _n(ops.spmm(*csr_d, _t(B, gpu), m)))
+            if m == k and m > 7:
+                h = np.maximum(B, 0)
+                W = (rng.standard_normal((64, 64)) * 0.1).astype(np.float32)
+                lv = _n(plan.level(_t(h, gpu), _t(W, gpu), _t(B, gpu)))
+                assert np.array_equal(lv, _n(ops.s2v_level(*csr_d, _t(h, gpu), _t(W, gpu), _t(B, gpu))))
+        assert_parity("spmm", got, *_spmm_want(oracle, rp, ci, v, B, m))
+    with ops.CsrPlan(*_csr_t((np.zeros(1, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32)), gpu), 0, 5) as plan:
+        assert plan.spmm(_t(np.ones((5, 3), np.float32), gpu)).shape == (0, 3)
+
+
+@pytest.mark.parametrize("C", [16, 32, 64, 128])
+def test_level_on_a_power_law_graph_leaves_no_trace_of_the_output_buffer(gpu, oracle, C):
+    """the two-launch level on the R-MAT matrix (a third of its rows empty): the product skips the rows without
+    entries and the contraction takes them as zero without reading them, so whatever the output buffer held before
+    the call (NaN here) must not show; with and without a plan, the same bits; against the oracle"""
+    import torch
+    from graphnn_amd import ops
+    rng = np.random.default_rng(910 + C)
+    a = synth.rmat_csr(0x5EED0005, 16, 16 << 16)
+    N = 1 << 16
+    v = (rng.random(a[1].size) * 0.1).astype(np.float32)
+    csr = (a[0], a[1], v)
+    csr_d = _csr_t(csr, gpu)
+    h_in = np.maximum(rng.standard_normal((N, C)), 0).astype(np.float32)
+    W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
+    msg = rng.standard_normal((N, C)).astype(np.float32)
+    out = torch.full((N, C), float("nan"), device=gpu)
+    got = _n(ops.s2v_level(*csr_d, _t(h_in, gpu), _t(W, gpu), _t(msg, gpu), out=out))
+    assert not np.isnan(got).any()
+    empty = np.diff(a[0]) == 0
+    assert empty.sum() > 1000 and np.array_equal(got[empty], np.maximum(msg[empty], 0))
+    with ops.CsrPlan(*csr_d, N, N) as plan:
+        out2 = torch.full((N, C), float("nan"), device=gpu)
+        assert np.array_equal(_n(plan.level(_t(h_in, gpu), _t(W, gpu), _t(msg, gpu), out=out2)), got)
+        assert np.array_equal(_n(plan.level(_t(h_in, gpu), _t(W, gpu), _t(msg, gpu), out=out2)), got)
+    want, w64 = _level_want(oracle, *csr, h_in, W, msg, None)
+    short = np.diff(a[0]) <= 256
+    assert_parity("level, rows of up to 256 entries", got[short], want[short], w64[short])
+    assert_condition("level, all rows", got, w64(), w64.cond())
 
 
 @pytest.mark.parametrize("C", [16, 64])
