@@ -352,14 +352,19 @@ def time_cfg5(dev, scale=22):
                    "what": "gnnhip_csr_plan_create (blocking: it reads back the piece count) and the device memory the plan owns "
                            "after a product of width 64, partial sums included"}
     del unplanned_level, unplanned_agg
-    plan.close()
     ms = _event_ms(lambda: ops.gemm(h1, wsc, out=score), 5)
     res["score"] = {"avg_ms": ms}
-    # the whole forward (input, 3 levels, readout): levels two and three reuse the plan that level one made for A
+    # the whole forward (input, 3 levels, readout): levels two and three reuse the plan that level one made for A;
+    # with the caller's plan none of them makes one
     H, Q, L = 64, 2, 3
     bufs = ops.ForwardBuffers(N, B, C, H, Q, dev)
     ms = _event_ms(lambda: ops.s2v_forward((rp, ci, val), (s_rp, s_ci, s_v), X, Wn, Wc, Wh1, Wh2, L, bufs=bufs), 5)
     res["forward"] = {"avg_ms": ms, "levels": L, "graphs": B}
+    logits = bufs.logits.clone()
+    ms = _event_ms(lambda: ops.s2v_forward_planned(plan, (s_rp, s_ci, s_v), X, Wn, Wc, Wh1, Wh2, L, bufs=bufs), 5)
+    res["forward_planned"] = {"avg_ms": ms, "levels": L, "graphs": B}
+    assert bool(torch.equal(bufs.logits, logits)), "planned and unplanned forwards differ"
+    plan.close()
     del bufs
     ms = _event_ms(lambda: ops.jagged_softmax(score, lens), 5)
     res["jagged_softmax"] = {"avg_ms": ms, "GBps": 8.0 * N / (ms * 1e-3) / 1e9}

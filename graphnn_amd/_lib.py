@@ -57,6 +57,7 @@ SIGNATURES = {
     "gnnhip_s2v_input_f32": [_I, _I, _I, _P, _P, _P, _P, _P],
     "gnnhip_s2v_readout_f32": [_I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "gnnhip_s2v_forward_f32": [_I] * 8 + [_P] * 11 + [_P] * 8 + [POINTER(c_int), _P],
+    "gnnhip_s2v_forward_planned_f32": [_P] + [_I] * 6 + [_P] * 8 + [_P] * 8 + [POINTER(c_int), _P],
     "gnnhip_s2v_forward_batched_f32": [_I] * 8 + [_P] * 11 + [_P] * 7 + [_P, _P],
     "gnnhip_s2v_forward_batched_train_f32": [_I] * 8 + [_P] * 11 + [_P] * 7 + [_P, _P],
     "gnnhip_s2v_forward_batched_labels_f32": [_I] * 8 + [_P] * 11 + [_P] * 7 + [_P, _P],

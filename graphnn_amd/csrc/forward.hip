@@ -137,6 +137,31 @@ int readout_any(int B, int N, int C, int H, int Q, const int* s_row_ptr, const i
     return GNNHIP_OK;
 }
 
+// input, L levels, readout on one stream; plan: of A, or null
+int forward_any(int N, int B, int K, int C, int H, int Q, int L, long long a_nnz, const int* a_row_ptr, const int* a_col_idx,
+                const float* a_val, const int* s_row_ptr, const int* s_col_idx, const float* s_val, const float* X, const float* W_n2l,
+                const float* W_conv, const float* W_h1, const float* W_h2, float* msg, float* h_a, float* h_b, float* pool, float* hidden,
+                float* logits, float* probs, int* pred, int* which_h, hipStream_t s, CsrPlan* plan)
+{
+    // With at least one level, and a level kernel that can read its input through ReLU, h0 = ReLU(msg) is
+    // never stored: the first level gathers from msg.
+    const bool lazy_h0 = L >= 1 && level_accepts_relu_input(N, C, a_nnz);
+    int rc = input_any(N, K, C, X, W_n2l, msg, lazy_h0 ? nullptr : h_a, s);
+    if (rc) return rc;
+    float* cur = lazy_h0 ? msg : h_a;
+    float* nxt = lazy_h0 ? h_a : h_b;
+    for (int lv = 0; lv < L; ++lv) {
+        if ((rc = level_any(N, C, a_nnz, a_row_ptr, a_col_idx, a_val, cur, W_conv, msg, nullptr, nxt, s, lv > 0,
+                            lazy_h0 && lv == 0, plan)))
+            return rc;
+        float* t = (cur == msg) ? h_b : cur;     // msg stays what it is; the other buffer takes the next level
+        cur = nxt;
+        nxt = t;
+    }
+    if (which_h) *which_h = (cur == h_a) ? 0 : 1;
+    return readout_any(B, N, C, H, Q, s_row_ptr, s_col_idx, s_val, cur, W_h1, W_h2, pool, hidden, logits, probs, pred, s);
+}
+
 }  // namespace
 }  // namespace gnnhip
 
@@ -230,24 +255,29 @@ int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L, int 
     GNNHIP_REQUIRE(msg && h_a && h_b && pool && hidden && logits, "null output in s2v_forward");
     GNNHIP_REQUIRE(h_a != h_b && msg != h_a && msg != h_b, "msg, h_a and h_b must be distinct buffers");
     if (int rc = require_ready()) return rc;
-    hipStream_t s = as_stream(stream);
-    // With at least one level, and a level kernel that can read its input through ReLU, h0 = ReLU(msg) is
-    // never stored: the first level gathers from msg.
-    const bool lazy_h0 = L >= 1 && level_accepts_relu_input(N, C, a_nnz);
-    int rc = input_any(N, K, C, X, W_n2l, msg, lazy_h0 ? nullptr : h_a, s);
-    if (rc) return rc;
-    float* cur = lazy_h0 ? msg : h_a;
-    float* nxt = lazy_h0 ? h_a : h_b;
-    for (int lv = 0; lv < L; ++lv) {
-        if ((rc = level_any(N, C, a_nnz, a_row_ptr, a_col_idx, a_val, cur, W_conv, msg, nullptr, nxt, s, lv > 0,
-                            lazy_h0 && lv == 0)))
-            return rc;
-        float* t = (cur == msg) ? h_b : cur;     // msg stays what it is; the other buffer takes the next level
-        cur = nxt;
-        nxt = t;
-    }
-    if (which_h) *which_h = (cur == h_a) ? 0 : 1;
-    return readout_any(B, N, C, H, Q, s_row_ptr, s_col_idx, s_val, cur, W_h1, W_h2, pool, hidden, logits, probs, pred, s);
+    return forward_any(N, B, K, C, H, Q, L, a_nnz, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, X, W_n2l, W_conv, W_h1, W_h2,
+                       msg, h_a, h_b, pool, hidden, logits, probs, pred, which_h, as_stream(stream), nullptr);
+}
+
+int gnnhip_s2v_forward_planned_f32(void* a_plan, int B, int K, int C, int H, int Q, int L,
+                                   const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                                   const float* X, const float* W_n2l, const float* W_conv,
+                                   const float* W_h1, const float* W_h2,
+                                   float* msg, float* h_a, float* h_b,
+                                   float* pool, float* hidden, float* logits, float* probs, int* pred,
+                                   int* which_h, void* stream)
+{
+    CsrPlan* p = as_csr_plan(a_plan);
+    GNNHIP_REQUIRE(p, "%p is not a live CSR plan", a_plan);
+    GNNHIP_REQUIRE(p->m == p->k && p->m >= 1, "s2v_forward_planned needs the plan of a square matrix with rows (it has %d rows and %d columns)", p->m, p->k);
+    GNNHIP_REQUIRE(B >= 1 && K >= 1 && C >= 1 && H >= 1 && Q >= 1 && L >= 0,
+                   "bad shape in s2v_forward_planned (B=%d K=%d C=%d H=%d Q=%d L=%d)", B, K, C, H, Q, L);
+    GNNHIP_REQUIRE(s_row_ptr && s_col_idx && s_val && X && W_n2l && W_conv && W_h1 && W_h2, "null input in s2v_forward_planned");
+    GNNHIP_REQUIRE(msg && h_a && h_b && pool && hidden && logits, "null output in s2v_forward_planned");
+    GNNHIP_REQUIRE(h_a != h_b && msg != h_a && msg != h_b, "msg, h_a and h_b must be distinct buffers");
+    if (int rc = require_ready()) return rc;
+    return forward_any(p->m, B, K, C, H, Q, L, p->nnz, p->row_ptr, p->col_idx, p->val, s_row_ptr, s_col_idx, s_val, X, W_n2l, W_conv, W_h1,
+                       W_h2, msg, h_a, h_b, pool, hidden, logits, probs, pred, which_h, as_stream(stream), p);
 }
 
 }  // extern "C"

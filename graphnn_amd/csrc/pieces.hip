@@ -551,11 +551,12 @@ int run_pieces(const CsrPlan* p, const Width& w, int n, float alpha, const float
 
 // What the scratch of a stream holds a plan for: kept per stream, next to the scratch it describes, so that whichever
 // thread plans on the stream replaces it.
-std::mutex g_memo_mu;
-std::map<hipStream_t, CsrPlan> g_memo;
+// (these registries are never destroyed: a caller's static objects may still hand plans back while the process exits)
+std::mutex& g_memo_mu = *new std::mutex;
+std::map<hipStream_t, CsrPlan>& g_memo = *new std::map<hipStream_t, CsrPlan>;
 
-std::mutex g_plans_mu;
-std::set<CsrPlan*> g_plans;
+std::mutex& g_plans_mu = *new std::mutex;
+std::set<CsrPlan*>& g_plans = *new std::set<CsrPlan*>;
 
 }  // namespace
 
@@ -690,12 +691,13 @@ extern "C" int gnnhip_csr_plan_create(int m, int k, const int* row_ptr, const in
         p->pslots = totals[1] > 0 ? totals[1] : 1;
         L = layout_of(m, nnz, p->slots, p->pslots);
         if (int rc = pool_acquire_exact(&p->body_block, L.body_bytes)) return fail(rc);
+        // the temporary arrays come from the pool and go back there (the next plan of a matrix of this size takes them)
         void* temp = nullptr;
-        if (int rc = pool_acquire_exact(&temp, L.temp_bytes)) return fail(rc);
+        if (int rc = pool_acquire(&temp, L.temp_bytes)) return fail(rc);
         point_plan(p, L, static_cast<char*>(p->head_block), static_cast<char*>(p->body_block));
         int rc = order_pieces(p, nnz, L, static_cast<char*>(temp), s);
-        hipError_t e = hipStreamSynchronize(s);                    // the temporary arrays go back to the driver right away
-        (void)pool_free(temp);
+        hipError_t e = hipStreamSynchronize(s);
+        (void)pool_release(temp);
         if (rc) return fail(rc);
         if (e != hipSuccess) return fail(set_error(GNNHIP_EHIP, "csr_plan_create: %s", hipGetErrorString(e)));
         p->has_pieces = true;

@@ -240,11 +240,17 @@ inline void FactorGraph::BuildSteps(Plan& plan, bool fold)
                                    A->value.rows() == H->value.rows(),
                                    "fused level: operand shapes do not chain");
                             O->value.Reshape(H->value.shape.dims);
-                            GNN_HIP(gnnhip_s2v_level_f32((int)H->value.rows(), (int)C, A->value.data->nnz, A->value.data->row_ptr,
-                                                         A->value.data->col_idx, A->value.data->val, H->value.data->ptr,
-                                                         W->value.data->ptr, M->value.data->ptr,
-                                                         bias ? W->value.data->ptr + C * C : nullptr,
-                                                         O->value.data->ptr, GpuHandle::Stream()));
+                            // a matrix large and dense enough for the library to plan keeps its plan across the levels
+                            if (void* plan = A->value.Plan())
+                                GNN_HIP(gnnhip_s2v_level_planned_f32(plan, (int)C, H->value.data->ptr, W->value.data->ptr, M->value.data->ptr,
+                                                                     bias ? W->value.data->ptr + C * C : nullptr, O->value.data->ptr,
+                                                                     GpuHandle::Stream()));
+                            else
+                                GNN_HIP(gnnhip_s2v_level_f32((int)H->value.rows(), (int)C, A->value.data->nnz, A->value.data->row_ptr,
+                                                             A->value.data->col_idx, A->value.data->val, H->value.data->ptr,
+                                                             W->value.data->ptr, M->value.data->ptr,
+                                                             bias ? W->value.data->ptr + C * C : nullptr,
+                                                             O->value.data->ptr, GpuHandle::Stream()));
                         };
                         for (size_t f : step->factors) taken[f] = true;
                         emit_at[f4] = step;                 // f4 reads f3 reads f2 reads f1: it is the last of the four
@@ -446,10 +452,16 @@ inline void FactorGraph::FoldWholeForward(Plan& plan)
                     ASSERT(rc == GNNHIP_EUNSUPPORTED, gnnhip_last_error());
                 }
                 GNN_HIP(gnnhip_s2v_input_f32((int)N, (int)K, (int)C, X->value.data->ptr, Wn->value.data->ptr, Msg->value.data->ptr, hs, s));
-                for (int l = 0; l < L; ++l)
-                    GNN_HIP(gnnhip_s2v_level_f32((int)N, (int)C, A->value.data->nnz, A->value.data->row_ptr, A->value.data->col_idx,
-                                                 A->value.data->val, hs + (size_t)l * NC, Wc->value.data->ptr, Msg->value.data->ptr,
-                                                 nullptr, hs + (size_t)(l + 1) * NC, s));
+                void* a_plan = A->value.Plan();
+                for (int l = 0; l < L; ++l) {
+                    if (a_plan)
+                        GNN_HIP(gnnhip_s2v_level_planned_f32(a_plan, (int)C, hs + (size_t)l * NC, Wc->value.data->ptr, Msg->value.data->ptr,
+                                                             nullptr, hs + (size_t)(l + 1) * NC, s));
+                    else
+                        GNN_HIP(gnnhip_s2v_level_f32((int)N, (int)C, A->value.data->nnz, A->value.data->row_ptr, A->value.data->col_idx,
+                                                     A->value.data->val, hs + (size_t)l * NC, Wc->value.data->ptr, Msg->value.data->ptr,
+                                                     nullptr, hs + (size_t)(l + 1) * NC, s));
+                }
                 GNN_HIP(gnnhip_s2v_readout_f32((int)B, (int)N, (int)C, (int)H, (int)Q, S->value.data->row_ptr, S->value.data->col_idx,
                                                S->value.data->val, hs + (size_t)L * NC, W1->value.data->ptr, W2->value.data->ptr,
                                                Pool->value.data->ptr, Hid->value.data->ptr, Logits->value.data->ptr, nullptr, nullptr, s));

@@ -9,6 +9,32 @@
 namespace gnn
 {
 
+// The library's plan for the products with one CSR matrix (gnnhip_csr_plan_create): made at the first product after
+// the matrix was (re)built when the matrix is large and dense enough for the library to plan at all (the thresholds
+// of its column-ordered route), kept for the later products with it (the levels of a forward multiply with the same
+// operand), destroyed with the matrix's contents.
+struct CsrPlanBox {
+    void* handle = nullptr;
+    bool tried = false;
+    ~CsrPlanBox() { Drop(); }
+    void Drop()
+    {
+        if (handle) (void)gnnhip_csr_plan_destroy(handle);
+        handle = nullptr;
+        tried = false;
+    }
+    // null when the matrix is not worth a plan
+    void* Get(int rows, int cols, int nnz, const int* row_ptr, const int* col_idx, const float* val)
+    {
+        if (!tried) {
+            tried = true;
+            if (rows >= 32768 && (long long)nnz >= 12ll * rows)
+                GNN_HIP(gnnhip_csr_plan_create(rows, cols, row_ptr, col_idx, val, GpuHandle::Stream(), &handle));
+        }
+        return handle;
+    }
+};
+
 template<typename Dtype>
 class TensorTemplate<GPU, CSR_SPARSE, Dtype> : public Tensor
 {
@@ -30,6 +56,24 @@ public:
         data->nnz = newNNZ;
         data->len_ptr = newNPtr;
         t_valid = false;                   // every builder resizes first: the cached transpose is stale
+        DropPlans();                       // ... and so are the plans of the products with the old contents
+    }
+    // plan of the products with this matrix / with its transpose (null: the plain entry points are as good)
+    void* Plan()
+    {
+        if (!plan) plan = std::make_shared<CsrPlanBox>();
+        return plan->Get((int)shape[0], (int)shape[1], data->nnz, data->row_ptr, data->col_idx, data->val);
+    }
+    void* TransposedPlan()
+    {
+        auto& t = Transposed();
+        if (!t_plan) t_plan = std::make_shared<CsrPlanBox>();
+        return t_plan->Get((int)shape[1], (int)shape[0], t.nnz, t.row_ptr, t.col_idx, t.val);
+    }
+    void DropPlans()
+    {
+        if (plan) plan->Drop();
+        if (t_plan) t_plan->Drop();
     }
     // CSR of the transpose, built on the device at the first use after the matrix was (re)built and kept
     // for the following ones (the backward pass multiplies by A^T once per level).  The product with it
@@ -94,7 +138,7 @@ public:
         GNN_HIP(gnnhip_memcpy_d2d(data->col_idx, src.data->col_idx, sizeof(int) * (size_t)data->nnz, s));
         GNN_HIP(gnnhip_memcpy_d2d(data->row_ptr, src.data->row_ptr, sizeof(int) * (size_t)data->len_ptr, s));
     }
-    void ShallowCopy(SpTensor<GPU, Dtype>& src) { shape = src.shape; data = src.data; t_valid = false; }
+    void ShallowCopy(SpTensor<GPU, Dtype>& src) { shape = src.shape; data = src.data; t_valid = false; plan = src.plan; t_plan.reset(); }
 
     void ArgMax(DTensor<GPU, int>& dst, uint axis = 0)
     {
@@ -109,6 +153,7 @@ public:
 private:
     std::shared_ptr< SparseData<GPU, Dtype> > t_data;   // transpose, see Transposed()
     bool t_valid = false;
+    std::shared_ptr<CsrPlanBox> plan, t_plan;           // see Plan(); shared with shallow copies, which share the arrays
 };
 
 // dense <- alpha * op(sparse) * dense + beta * dense
@@ -120,10 +165,18 @@ inline void TensorTemplate<GPU, DENSE, float>::MM(SpTensor<GPU, float>& a, DTens
     GetDims(a.rows(), a.cols(), transA, b.rows(), b.cols(), transB, m, n, k);
     Reshape({m, n});
     if (transA == Trans::N) {
+        if (void* plan = a.Plan()) {
+            GNN_HIP(gnnhip_spmm_csr_planned_f32(plan, (int)n, alpha, b.data->ptr, (int)b.cols(), beta, data->ptr, (int)n, GpuHandle::Stream()));
+            return;
+        }
         GNN_HIP(gnnhip_spmm_csr_f32((int)m, (int)k, (int)n, a.data->nnz, alpha, a.data->row_ptr, a.data->col_idx, a.data->val,
                                     b.data->ptr, (int)b.cols(), beta, data->ptr, (int)n, GpuHandle::Stream()));
     } else {
         auto& t = a.Transposed();
+        if (void* plan = a.TransposedPlan()) {
+            GNN_HIP(gnnhip_spmm_csr_planned_f32(plan, (int)n, alpha, b.data->ptr, (int)b.cols(), beta, data->ptr, (int)n, GpuHandle::Stream()));
+            return;
+        }
         GNN_HIP(gnnhip_spmm_csr_f32((int)m, (int)k, (int)n, t.nnz, alpha, t.row_ptr, t.col_idx, t.val,
                                     b.data->ptr, (int)b.cols(), beta, data->ptr, (int)n, GpuHandle::Stream()));
     }

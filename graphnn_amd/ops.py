@@ -289,6 +289,28 @@ def s2v_forward(a_csr, s_csr, X, W_n2l, W_conv, W_h1, W_h2, L, bufs=None):
     return bufs
 
 
+def s2v_forward_planned(plan, s_csr, X, W_n2l, W_conv, W_h1, W_h2, L, bufs=None):
+    """Whole forward with a CsrPlan of A (gnnhip_s2v_forward_planned_f32)."""
+    N, K = X.shape
+    C, H, Q = W_n2l.shape[1], W_h1.shape[1], W_h2.shape[1]
+    B = s_csr[0].numel() - 1
+    if N != plan.m or plan.m != plan.k:
+        raise ValueError("the plan must be of the [N,N] adjacency")
+    _check_csr(s_csr[0], s_csr[1], s_csr[2], B, "S")
+    if W_n2l.shape[0] != K or tuple(W_conv.shape) != (C, C) or W_h1.shape[0] != C or W_h2.shape[0] != H:
+        raise ValueError("weight shapes do not chain")
+    if bufs is None:
+        bufs = ForwardBuffers(N, B, C, H, Q, X.device)
+    check(_lib().gnnhip_s2v_forward_planned_f32(
+        plan.handle, B, K, C, H, Q, L,
+        _i32(s_csr[0], "s_row_ptr"), _i32(s_csr[1], "s_col_idx"), _f32(s_csr[2], "s_val"),
+        _f32(X, "X"), _f32(W_n2l, "W_n2l"), _f32(W_conv, "W_conv"), _f32(W_h1, "W_h1"), _f32(W_h2, "W_h2"),
+        _f32(bufs.msg, "msg"), _f32(bufs.h_a, "h_a"), _f32(bufs.h_b, "h_b"), _f32(bufs.pool, "pool"),
+        _f32(bufs.hidden, "hidden"), _f32(bufs.logits, "logits"), _f32(bufs.probs, "probs"),
+        _i32(bufs.pred, "pred"), ctypes.byref(bufs.which), _stream()))
+    return bufs
+
+
 class BatchedBuffers:
     """Caller-owned outputs of the graph-resident forward."""
 

@@ -245,6 +245,17 @@ int gnnhip_s2v_forward_f32(int N, int B, int K, int C, int H, int Q, int L, int 
                            float* pool, float* hidden, float* logits, float* probs, int* pred,
                            int* which_h, void* stream);
 
+/* ---- the same forward with the plan of A (gnnhip_csr_plan_create; N = the plan's rows): for callers that run the network
+ *      of examples/graph_classification/src/kernel_mean_field.cpp:31-56 over one large graph batch after batch, where
+ *      the reference rebuilds nothing but the features.  Same bits as gnnhip_s2v_forward_f32. */
+int gnnhip_s2v_forward_planned_f32(void* a_plan, int B, int K, int C, int H, int Q, int L,
+                                   const int* s_row_ptr, const int* s_col_idx, const float* s_val,
+                                   const float* X, const float* W_n2l, const float* W_conv,
+                                   const float* W_h1, const float* W_h2,
+                                   float* msg, float* h_a, float* h_b,
+                                   float* pool, float* hidden, float* logits, float* probs, int* pred,
+                                   int* which_h, void* stream);
+
 /* ---- the same forward for block-diagonal batches of small graphs, in ONE launch with the
  *      embeddings resident in LDS: the op sequence of
  *      examples/graph_classification/src/kernel_mean_field.cpp:31-49 on a batch laid out by GetBatch

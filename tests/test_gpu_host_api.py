@@ -10,7 +10,7 @@ import subprocess
 import numpy as np
 import pytest
 
-from conftest import PARITY_TOL, max_rel
+from conftest import PARITY_TOL, Lazy, assert_condition, assert_parity, max_rel
 from graphnn_amd import batching, synth
 
 pytestmark = pytest.mark.gpu
@@ -277,6 +277,71 @@ def test_host_api_large_batch_takes_the_separate_kernels(gpu, oracle, tmp_path):
     logits_t = out[pos + 4:pos + 4 + B * Q].reshape(B, Q)
     assert max_rel(logits_t, want["logits"]) < PARITY_TOL
     assert abs(loss_t - loss) <= 1e-5 * abs(loss) and acc_t == acc
+
+
+def test_host_api_large_dense_graph_keeps_the_plan_of_its_operand(gpu, oracle, tmp_path):
+    """one R-MAT graph of 65,536 nodes, 16 edges per node, through graphnn's tensor and FactorGraph API
+    (host/tests/host_big_graph_check.cpp): the sparse operand takes the library's planned products, the plan is kept
+    from the first product on and dropped when the matrix gets new contents; products with the matrix and its transpose
+    and three fused levels against the oracle"""
+    exe = os.path.join(BUILD, "host_big_graph_check")
+    assert os.path.exists(exe), "build the host layer first: make -C graphnn_amd/host"
+    scale, K, C, L = 16, 5, 64, 3
+    N, E = 1 << scale, 16 << scale
+    rng = np.random.default_rng(65)
+    rows, cols = (t.numpy() for t in synth.rmat_edges_torch(synth.config_seed(5), scale, E, "cpu"))
+    order = rng.permutation(E)                        # AddEdge order: any; the operand lists a row's entries in that order
+    x, y = cols[order].astype(np.int32), rows[order].astype(np.int32)       # edge x -> y adds x to row y
+    a = batching.node2node_csr(N, x, y)
+    val = (rng.random(E) * 0.2 - 0.05).astype(np.float32)
+    val2 = (rng.random(E) * 0.2 - 0.05).astype(np.float32)
+    B = rng.standard_normal((N, C)).astype(np.float32)
+    X = np.zeros((N, K), np.float32); X[np.arange(N), rng.integers(0, K, N)] = 1.0
+    Wn = (rng.standard_normal((K, C)) * 0.3).astype(np.float32)
+    W = (rng.standard_normal((C, C)) * 0.02).astype(np.float32)
+    d = str(tmp_path)
+    np.stack([x, y], axis=1).astype(np.int32).tofile(d + "/edges.bin")
+    for name, arr in (("val", val), ("val2", val2), ("b", B), ("x", X), ("w_n2l", Wn), ("w", W)):
+        arr.tofile(d + "/%s.bin" % name)
+    r = subprocess.run([exe, d, str(N), str(K), str(C), str(L)], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "planned 1, transpose planned 1" in r.stdout, r.stdout
+    assert int(re.search(r"fused steps (\d+)", r.stdout).group(1)) >= L, r.stdout        # every level is one fused step
+    out = np.fromfile(d + "/out.bin", dtype=np.float32).reshape(5, N, C)
+    c1, c2, ct, c3, h_l = out
+    assert np.array_equal(c1, c2)
+    lens = np.diff(a[0])
+    short = lens <= 256
+
+    def check(name, got, want, model, cond, rows_ok):
+        assert_condition(name + ", all rows", got, model, cond)
+        assert_parity(name + ", rows of up to 256 entries", got[rows_ok], want[rows_ok], Lazy(lambda: model[rows_ok]))
+
+    for name, got, v in (("spmm", c1, val), ("spmm new values", c3, val2)):
+        check(name, got, oracle.spmm(a[0], a[1], v, B, N), oracle.spmm_f64(a[0], a[1], v, B, N),
+              oracle.spmm_f64(a[0], a[1], v, B, N, absolute=True), short)
+    assert not np.array_equal(c1, c3)
+    # the stable transpose: row c lists the rows with an entry in column c, ascending
+    order_t = np.argsort(a[1], kind="stable")
+    t_rp = np.zeros(N + 1, np.int32)
+    np.cumsum(np.bincount(a[1], minlength=N), out=t_rp[1:])
+    t_csr = (t_rp, np.repeat(np.arange(N, dtype=np.int32), lens)[order_t], val[order_t])
+    check("spmm transposed", ct, oracle.spmm(*t_csr, B, N), oracle.spmm_f64(*t_csr, B, N), oracle.spmm_f64(*t_csr, B, N, absolute=True),
+          np.diff(t_csr[0]) <= 256)
+    # the levels: every row against float64 under the condition metric, level by level on the oracle's side
+    ones = np.ones(E, np.float32)
+    msg = oracle.gemm(X, Wn)
+    h = np.maximum(msg, 0)
+    h64, c64 = msg.astype(np.float64), np.abs(msg.astype(np.float64))
+    h64 = np.maximum(h64, 0)
+    import scipy.sparse as sp
+    A64 = sp.csr_matrix((ones.astype(np.float64), a[1], a[0]), shape=(N, N))
+    for _ in range(L):
+        h = oracle.level(a[0], a[1], ones, h, W, msg)
+        h64 = np.maximum((A64 @ h64) @ W.astype(np.float64) + msg, 0)
+        c64 = (A64 @ c64) @ np.abs(W.astype(np.float64)) + np.abs(msg)
+    assert_condition("h_final, all rows", h_l, h64, c64)
+    assert_parity("h_final, rows of up to 256 entries", h_l[short], h[short], Lazy(lambda: h64[short]))
 
 
 def test_reference_example_runs_unchanged(gpu, tmp_path):

@@ -1602,6 +1602,18 @@ def test_level_on_a_power_law_graph_leaves_no_trace_of_the_output_buffer(gpu, or
         out2 = torch.full((N, C), float("nan"), device=gpu)
         assert np.array_equal(_n(plan.level(_t(h_in, gpu), _t(W, gpu), _t(msg, gpu), out=out2)), got)
         assert np.array_equal(_n(plan.level(_t(h_in, gpu), _t(W, gpu), _t(msg, gpu), out=out2)), got)
+        if C == 64:
+            # the whole forward with the caller's plan: the bits of the forward that plans for itself
+            K, H, Q, L, B = 6, 16, 3, 2, 64
+            w = synth.make_weights(synth.Stream(910), K, C, H, Q)
+            X = np.zeros((N, K), np.float32); X[np.arange(N), rng.integers(0, K, N)] = 1.0
+            s_d = _csr_t(synth.contiguous_subgraph_csr(N, B), gpu)
+            dev_w = [_t(x, gpu) for x in (w.W_n2l, w.W_conv * 0.1, w.W_h1, w.W_h2)]
+            f1 = ops.s2v_forward(csr_d, s_d, _t(X, gpu), *dev_w, L)
+            f2 = ops.s2v_forward_planned(plan, s_d, _t(X, gpu), *dev_w, L)
+            for key in ("msg", "pool", "hidden", "logits", "probs", "pred"):
+                assert np.array_equal(_n(getattr(f1, key)), _n(getattr(f2, key))), key
+            assert np.array_equal(_n(f1.h_final), _n(f2.h_final))
     want, w64 = _level_want(oracle, *csr, h_in, W, msg, None)
     short = np.diff(a[0]) <= 256
     assert_parity("level, rows of up to 256 entries", got[short], want[short], w64[short])
