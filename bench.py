@@ -37,10 +37,10 @@ def level_algorithmic_bytes(N, E, C):
     return 4 * (N + 1) + 8 * E + 12 * N * C + 4 * C * C
 
 
-def build_forward_workload(dev):
+def build_forward_workload(dev, size_mode=None):
     import torch
     from graphnn_amd import batching, synth
-    batch, w, cfg = synth.make_config(2)
+    batch, w, cfg = synth.make_config(2, size_mode=size_mode)
     a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
     s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
     X = batch.one_hot()
@@ -50,8 +50,8 @@ def build_forward_workload(dev):
     return dev_args, host
 
 
-def time_forward(dev_args, cfg, batch, steps, warmup, route):
-    """Wall-clock seconds per forward.  route = "graph_resident" (one launch, embeddings in LDS; valid
+def time_forward(dev_args, cfg, batch, steps, warmup, route, device_times=None):
+    """Wall-clock seconds per forward (device_times, a dict, also receives the HIP-event time of one forward).  route = "graph_resident" (one launch, embeddings in LDS; valid
     because the batch is block diagonal, as GetBatch builds it) or "general" (input + L levels + readout
     launches that accept any CSR)."""
     import torch
@@ -80,7 +80,26 @@ def time_forward(dev_args, cfg, batch, steps, warmup, route):
     t1 = time.perf_counter()
     if route.startswith("graph_resident"):
         assert int(bufs.status.cpu()[0]) == 0, "graph-resident forward reported a layout violation"
+    if device_times is not None:
+        device_times[route] = _event_median_ms(run, max(50, min(steps, 500)))
     return (t1 - t0) / steps, bufs
+
+
+def _event_median_ms(fn, reps, warmup=5):
+    """Device time of one call of fn: a pair of HIP events around every one of `reps` calls on the stream the launches
+    go to (torch's current stream), after `warmup` untimed calls; returns {median, min, mean, runs} in milliseconds."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for e0, e1 in evs:
+        e0.record()
+        fn()
+        e1.record()
+    torch.cuda.synchronize()
+    ms = np.array([e0.elapsed_time(e1) for e0, e1 in evs])
+    return {"median_ms": float(np.median(ms)), "min_ms": float(ms.min()), "mean_ms": float(ms.mean()), "runs": int(reps)}
 
 
 def time_forward_pipelined(dev_args, cfg, batch, steps, warmup, nstreams=4):
@@ -121,34 +140,60 @@ def time_stream_copy(dev, n=1 << 28):
     return {"kernel": "map1_kernel<FReLU>", "bytes": 8 * n, "avg_ms": ms, "GBps": 8.0 * n / (ms * 1e-3) / 1e9}
 
 
-def time_spmm_cfg3(dev, reps=20, warmup=3):
-    """HIP-event time of the SpMM kernel alone on configuration 3."""
+def time_read_ceiling(dev, n=1 << 29):
+    """What this GPU's memory delivers to a kernel that only reads: the sum reduction (gnnhip_reduce_f32) over 2 GiB,
+    four times the memory-side cache, so every byte comes from HBM."""
+    import torch
+    from graphnn_amd import ops
+    x = torch.ones(n, device=dev, dtype=torch.float32)
+    t = _event_median_ms(lambda: ops.reduce("sum", x), 20, 3)
+    return {"kernel": "reduce_partial_kernel (gnnhip_reduce_f32, sum)", "bytes": 4 * n, "median_ms": t["median_ms"],
+            "GBps": 4.0 * n / (t["median_ms"] * 1e-3) / 1e9}
+
+
+def time_gather_ceiling(dev, m=1_000_000, per=10, d=128):
+    """The SpMM kernel of configuration 3 on a matrix of the same shape whose columns never repeat (m rows of `per`
+    entries over m * per columns, scattered by a multiplicative permutation): the dense operand is m * per rows of
+    512 bytes = 5.12 GB, twenty times the memory-side cache, and each of its rows is gathered exactly once, so all
+    gathered bytes come from HBM.  What this measures is the rate at which HBM serves this kernel's 512-byte gathers."""
+    import torch
+    from graphnn_amd import ops
+    k = m * per
+    idx = torch.arange(k, device=dev, dtype=torch.int64)
+    cols = (idx * 6_700_417) % k                      # a permutation of 0 .. k-1 (the multiplier is prime, k = 2^7 5^7)
+    cols, _ = torch.sort(cols.view(m, per), dim=1)    # ascending inside a row, as CSR rows are
+    ci = cols.reshape(-1).int()
+    rp = (torch.arange(m + 1, device=dev, dtype=torch.int64) * per).int()
+    v = torch.ones(k, device=dev, dtype=torch.float32)
+    del idx, cols
+    X = torch.ones((k, d), device=dev, dtype=torch.float32)
+    Y = torch.empty((m, d), device=dev, dtype=torch.float32)
+    t = _event_median_ms(lambda: ops.spmm(rp, ci, v, X, m, out=Y), 20, 3)
+    assert float(Y[12345, 7]) == float(per), "gather-ceiling product is wrong"
+    nbytes = 4 * (m + 1) + 8 * k + 4 * k * d + 4 * m * d
+    return {"kernel": "spmm_rowgroup_kernel<4,1>", "workload": "%d rows x %d entries, %d distinct columns, width %d" % (m, per, k, d),
+            "bytes": nbytes, "median_ms": t["median_ms"], "GBps": nbytes / (t["median_ms"] * 1e-3) / 1e9}
+
+
+def time_spmm_cfg3(dev, reps=50, warmup=5, regular=False):
+    """HIP-event time of the SpMM kernel alone on configuration 3 (SplitMix64 streams of the configuration; the dense
+    operand by the torch twin of the normal stream, on the device).  regular: exactly 10 entries in every row."""
     import torch
     from graphnn_amd import ops, synth
     n, nnz, d = 1_000_000, 10_000_000, 128
-    rp, ci, v = synth.erdos_renyi_csr(synth.config_seed(3), n, nnz)
+    seed = synth.config_seed(3)
+    rp, ci, v = synth.erdos_renyi_csr(seed, n, nnz, regular=regular)
     t = lambda arr: torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
     rp_d, ci_d, v_d = t(rp), t(ci), t(v)
-    gen = torch.Generator(device=dev)
-    gen.manual_seed(synth.config_seed(3))
-    X = torch.randn((n, d), generator=gen, device=dev, dtype=torch.float32)
+    X = synth.torch_normal_f32(synth.Stream(seed).child(2).seed, n * d, dev).view(n, d)
     Y = torch.empty((n, d), device=dev, dtype=torch.float32)
-    for _ in range(warmup):
-        ops.spmm(rp_d, ci_d, v_d, X, n, out=Y)
-    torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
-    for e0, e1 in evs:
-        e0.record()
-        ops.spmm(rp_d, ci_d, v_d, X, n, out=Y)
-        e1.record()
-    torch.cuda.synchronize()
-    ms = np.array([e0.elapsed_time(e1) for e0, e1 in evs])
+    ev = _event_median_ms(lambda: ops.spmm(rp_d, ci_d, v_d, X, n, out=Y), reps, warmup)
     # property check at full size: A * ones = row lengths, exactly
     ones = torch.ones((n, 4), device=dev, dtype=torch.float32)
     deg = ops.spmm(rp_d, ci_d, v_d, ones, n)
     torch.cuda.synchronize()
     assert np.array_equal(deg[:, 0].cpu().numpy(), np.diff(rp).astype(np.float32)), "SpMM row-length check failed"
-    return float(ms.mean()), float(ms.min()), spmm_algorithmic_bytes(n, n, nnz, d), (n, nnz, d)
+    return ev, spmm_algorithmic_bytes(n, n, nnz, d), (n, nnz, d)
 
 
 FP32_MFMA_PEAK_TFLOPS = 157.3   # MI355X dense FP32 matrix, published
@@ -594,7 +639,12 @@ def main():
     ap.add_argument("--no-rooflines", action="store_true",
                     help="skip the configuration-4 / configuration-5 kernel rooflines")
     ap.add_argument("--only", default="", help="comma-separated legs to run alone (for profiling): "
-                                                "forward, spmm, cfg4, cfg5, train, e2e, sizes")
+                                                "forward, spmm, ceilings, cfg4, cfg5, train, e2e, sizes")
+    ap.add_argument("--regular", action="store_true",
+                    help="configuration 3 with exactly 10 entries in every row (the other reading of its \"uniform degree\")")
+    ap.add_argument("--uniform", action="store_true",
+                    help="configuration 2 with graph sizes drawn uniformly from 10..110 (mean 60) instead of the right-skewed "
+                         "sizes with mean ~30")
     ap.add_argument("--mkl-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one element-wise copy kernel of known size (1 GiB read, 1 GiB written) "
@@ -618,11 +668,15 @@ def main():
         legs = set(args.only.split(","))
         res = {}
         if "forward" in legs:
-            dev_args, host = build_forward_workload(dev)
+            dev_args, host = build_forward_workload(dev, "uniform" if args.uniform else None)
             sec, _ = time_forward(dev_args, host["cfg"], host["batch"], args.steps, args.warmup, "graph_resident")
             res["forward_ms"] = sec * 1e3
         if "spmm" in legs:
-            res["spmm_cfg3_ms"] = time_spmm_cfg3(dev)[0]
+            res["spmm_cfg3"] = time_spmm_cfg3(dev, regular=args.regular)[0]
+        if "ceilings" in legs:
+            res["read_ceiling"] = time_read_ceiling(dev)
+            res["gather_ceiling"] = time_gather_ceiling(dev)
+            res["stream_copy"] = time_stream_copy(dev)
         if "cfg4" in legs:
             res["cfg4_level"] = time_level_cfg4(dev)
         if "cfg5" in legs:
@@ -645,11 +699,12 @@ def main():
         print(json.dumps(res))
         return
 
-    dev_args, host = build_forward_workload(dev)
+    dev_args, host = build_forward_workload(dev, "uniform" if args.uniform else None)
     batch, cfg = host["batch"], host["cfg"]
-    sec_general, bufs_general = time_forward(dev_args, cfg, batch, args.steps, args.warmup, "general")
-    sec, bufs = time_forward(dev_args, cfg, batch, args.steps, args.warmup, "graph_resident")
-    sec_labels, bufs_labels = time_forward(dev_args, cfg, batch, args.steps, args.warmup, "graph_resident_labels")
+    dev_ms = {}
+    sec_general, bufs_general = time_forward(dev_args, cfg, batch, args.steps, args.warmup, "general", dev_ms)
+    sec, bufs = time_forward(dev_args, cfg, batch, args.steps, args.warmup, "graph_resident", dev_ms)
+    sec_labels, bufs_labels = time_forward(dev_args, cfg, batch, args.steps, args.warmup, "graph_resident_labels", dev_ms)
     assert bool(torch.equal(bufs_labels.logits, bufs.logits)) and bool(torch.equal(bufs_labels.pred, bufs.pred)), \
         "label input and one-hot input disagree"
     # the two routes must agree on what they computed
@@ -669,6 +724,10 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": sec * 1e3,
+        # the same launch between two HIP events, median over the runs: what the device spends on one forward (the wall
+        # figure above also carries the host's launch work and one synchronisation per `steps` forwards)
+        "device_ms_per_step": dev_ms["graph_resident"]["median_ms"],
+        "device_ms": dev_ms["graph_resident"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -676,11 +735,14 @@ def main():
         "data": "synthetic",
         "config": {"workload": "s2v mean-field forward, configuration 2: 256 graphs, %d nodes, %d directed edges, "
                                "38 label types, hidden 64, 4 levels, MLP 64-32-2, softmax + argmax"
-                               % (batch.num_nodes, batch.num_edges),
+                               % (batch.num_nodes, batch.num_edges)
+                               + ("; graph sizes uniform in 10..110 (--uniform)" if args.uniform else
+                                  "; graph sizes right-skewed with mean ~30 (10 + min(100, floor(-20 ln(1-u))))"),
                    "graphs": batch.num_graphs, "nodes": batch.num_nodes, "edges": batch.num_edges},
         "nodes_per_s": batch.num_nodes / sec,
         "route": "graph-resident forward, one launch (gnnhip_s2v_forward_batched_f32)",
         "label_input_route": {"graphs_per_s": batch.num_graphs / sec_labels, "ms_per_step": sec_labels * 1e3,
+                              "device_ms_per_step": dev_ms["graph_resident_labels"]["median_ms"],
                               "what": "gnnhip_s2v_forward_batched_labels_f32: the same launch fed one int label per node "
                                       "instead of the one-hot matrix X (bit-identical outputs); `value` keeps the "
                                       "reference's dense X"},
@@ -689,6 +751,7 @@ def main():
                                            "bit-identical outputs): compute units that finish their graph early start on the next "
                                            "batch; `value` keeps one batch at a time"},
         "general_route": {"graphs_per_s": batch.num_graphs / sec_general, "ms_per_step": sec_general * 1e3,
+                          "device_ms_per_step": dev_ms["general"]["median_ms"],
                           "what": "gnnhip_s2v_forward_f32: input + 4 fused levels + readout, any CSR"},
     }
 
@@ -698,21 +761,43 @@ def main():
         out["training_step"] = training_step_host_layer(host)
 
     if not args.no_spmm:
-        mean_ms, min_ms, bytes_alg, (n, nnz, d) = time_spmm_cfg3(dev)
-        achieved = bytes_alg / (mean_ms * 1e-3) / 1e9
+        ev, bytes_alg, (n, nnz, d) = time_spmm_cfg3(dev, regular=args.regular)
+        med_ms = ev["median_ms"]
+        achieved = bytes_alg / (med_ms * 1e-3) / 1e9
+        traffic = MEASURED_TRAFFIC_BYTES["spmm_cfg3"]
+        read_c, gather_c, copy_c = time_read_ceiling(dev), time_gather_ceiling(dev), time_stream_copy(dev)
         out["roofline"] = {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES["spmm_cfg3"],
+            "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
             "traffic_source": "constant: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 of spmm_rowgroup_kernel<4,1> from the rocprofv3 "
-                              "--pmc runs summarised in profiles/bench_forward_cfg2_spmm_cfg3.md (not re-measured in this run)",
+                              "--pmc runs summarised in profiles/bench_forward_cfg2_spmm_cfg3.md (not re-measured in this run). "
+                              "These counters count what the L2 asks of the fabric; the 256 MB memory-side cache sits behind that "
+                              "point and no counter this profiler exposes tells its hits from HBM reads",
             "kernel": "spmm_rowgroup_kernel<4,1>",
-            "workload": "configuration 3: CSR SpMM, %d rows, %d entries, width %d" % (n, nnz, d),
-            "algorithmic_bytes": bytes_alg, "avg_ms": mean_ms, "min_ms": min_ms,
-            # the counted traffic over the same launch time: what the memory system actually moves
-            "traffic_GBps": MEASURED_TRAFFIC_BYTES["spmm_cfg3"] / (mean_ms * 1e-3) / 1e9,
-            "traffic_frac": MEASURED_TRAFFIC_BYTES["spmm_cfg3"] / (mean_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            # what a plain streaming kernel reaches on this GPU, measured in this run
-            "stream_copy": time_stream_copy(dev),
+            "workload": "configuration 3: CSR SpMM, %d rows, %d entries%s, width %d"
+                        % (n, nnz, " (exactly 10 per row, --regular)" if args.regular else "", d),
+            "algorithmic_bytes": bytes_alg, "avg_ms": med_ms, "median_ms": med_ms, "min_ms": ev["min_ms"], "mean_ms": ev["mean_ms"],
+            "runs": ev["runs"],
+            # the counted L2-miss traffic over the same launch time: requests to the fabric, NOT all of them HBM reads
+            "l2_miss_traffic_GBps": traffic / (med_ms * 1e-3) / 1e9,
+            "l2_miss_traffic_frac": traffic / (med_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            # what this GPU's HBM delivers, measured in this run: a read-only kernel over 2 GiB, a copy of 1 GiB, and this
+            # same SpMM kernel on a matrix whose 10M columns never repeat (5.12 GB operand: every gathered byte from HBM)
+            "read_ceiling": read_c, "stream_copy": copy_c, "gather_ceiling": gather_c,
+            # north-star target ">= 60 % of HBM peak": stated separately for the fabric side (counted L2 misses, which the
+            # memory-side cache partly serves: the 512 MB operand is twice its size and every row is gathered ten times)
+            # and for bytes that provably come from HBM (the no-reuse gather above)
+            "hbm_target": {
+                "target_frac": 0.6,
+                "fabric_side_frac": traffic / (med_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                "met_on_fabric_side": bool(traffic / (med_ms * 1e-3) / 1e9 / HBM_PEAK_GBS >= 0.6),
+                "hbm_side_gather_frac": gather_c["GBps"] / HBM_PEAK_GBS,
+                "met_on_hbm_side": bool(gather_c["GBps"] / HBM_PEAK_GBS >= 0.6),
+                "read_only_frac": read_c["GBps"] / HBM_PEAK_GBS,
+                "gather_vs_read_only": gather_c["GBps"] / read_c["GBps"],
+                "dram_counters": "none: the profiler's TCC_EA0_RDREQ_DRAM counts requests bound for the memory controllers, "
+                                 "ahead of the memory-side cache, and equals the fabric figure",
+            },
         }
     else:
         out["roofline"] = None

@@ -197,16 +197,47 @@ __device__ __forceinline__ float block_combine(float v, float* sh)
     return r;
 }
 
+// The array is read as 128-bit words from its first 16-byte aligned element on (the few elements before it and after
+// the last whole word go to workgroup 0), grid-strided, four words in flight per lane and sixteen running values per
+// lane, which are combined in a fixed order: the result depends on n and the grid alone.  For max every running value
+// starts from x[0], so that a NaN there, and only there, survives (the reference's strict comparison).
 template <bool IS_MAX, bool SQUARE = false>
 __global__ __launch_bounds__(kBlock) void reduce_partial_kernel(const float* __restrict__ x, size_t n, float* __restrict__ partial)
 {
     __shared__ float sh[kWavesPerBlock];
-    const size_t per = (n + gridDim.x - 1) / gridDim.x;
-    const size_t lo = (size_t)blockIdx.x * per;
-    const size_t hi = lo + per < n ? lo + per : n;
-    float v = IS_MAX ? -INFINITY : 0.f;
-    if (IS_MAX && lo < hi) v = x[lo];
-    for (size_t i = lo + threadIdx.x; i < hi; i += kBlock) v = IS_MAX ? max_keep(v, x[i]) : v + (SQUARE ? x[i] * x[i] : x[i]);
+    auto comb = [](float a, float b) { return IS_MAX ? max_keep(a, b) : a + (SQUARE ? b * b : b); };
+    size_t head = ((16 - (reinterpret_cast<uintptr_t>(x) & 15)) & 15) / 4;
+    if (head > n) head = n;
+    const float4* __restrict__ x4 = reinterpret_cast<const float4*>(x + head);
+    const size_t n4 = (n - head) / 4;
+    const size_t tail0 = head + n4 * 4;
+    const float init = IS_MAX ? x[0] : 0.f;
+    float4 a[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) a[u] = make_float4(init, init, init, init);
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    for (; i + 3 * stride < n4; i += 4 * stride) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = x4[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            a[u].x = comb(a[u].x, v[u].x); a[u].y = comb(a[u].y, v[u].y);
+            a[u].z = comb(a[u].z, v[u].z); a[u].w = comb(a[u].w, v[u].w);
+        }
+    }
+    for (; i < n4; i += stride) {
+        const float4 v = x4[i];
+        a[0].x = comb(a[0].x, v.x); a[0].y = comb(a[0].y, v.y); a[0].z = comb(a[0].z, v.z); a[0].w = comb(a[0].w, v.w);
+    }
+    if (blockIdx.x == 0) {
+        for (size_t j = threadIdx.x; j < head; j += kBlock) a[0].x = comb(a[0].x, x[j]);
+        for (size_t j = tail0 + threadIdx.x; j < n; j += kBlock) a[0].x = comb(a[0].x, x[j]);
+    }
+    auto join = [](float p, float q) { return IS_MAX ? max_keep(p, q) : p + q; };
+    float v = join(join(join(a[0].x, a[0].y), join(a[0].z, a[0].w)), join(join(a[1].x, a[1].y), join(a[1].z, a[1].w)));
+    v = join(v, join(join(join(a[2].x, a[2].y), join(a[2].z, a[2].w)), join(join(a[3].x, a[3].y), join(a[3].z, a[3].w))));
     v = block_combine<IS_MAX>(v, sh);
     if (threadIdx.x == 0) partial[blockIdx.x] = v;
 }
@@ -429,9 +460,9 @@ int gnnhip_reduce_f32(int op, const float* x, size_t n, float* out, void* stream
     if (int rc = require_ready()) return rc;
     hipStream_t s = as_stream(stream);
     size_t nb = (n + 16383) / 16384;                   // >= 16K elements per workgroup
-    if (nb > 1024) nb = 1024;
+    if (nb > 2048) nb = 2048;                          // eight workgroups per compute unit
     void* partial = nullptr;
-    if (int rc = stream_scratch(s, sizeof(float) * 1024, &partial)) return rc;
+    if (int rc = stream_scratch(s, sizeof(float) * 2048, &partial)) return rc;
     float* pp = static_cast<float*>(partial);
     const float div = (op == GNNHIP_REDUCE_MEAN) ? (float)n : 0.f;
     if (op == GNNHIP_REDUCE_MAX) {

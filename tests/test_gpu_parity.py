@@ -422,6 +422,22 @@ def test_reduce(gpu, oracle, n):
     assert float(_n(ops.reduce("max", xd))[0]) == oracle.max(x)
     ints = rng.integers(-50, 50, min(n, 100000)).astype(np.float32)
     assert float(_n(ops.reduce("sum", _t(ints, gpu)))[0]) == float(ints.astype(np.float64).sum())   # exact in fp32
+    # views that start 4, 8 and 12 bytes past a 16-byte boundary (the kernel reads 128-bit words from the first aligned one)
+    for off in (1, 2, 3):
+        if n > off:
+            v = xd[off:]
+            assert v.data_ptr() % 16 == 4 * off
+            assert abs(float(_n(ops.reduce("sum", v))[0]) - ref64[off:].sum()) <= 1e-5 * ref64[off:].sum()
+            assert float(_n(ops.reduce("max", v))[0]) == oracle.max(x[off:])
+            assert float(_n(ops.reduce("sum", _t(ints, gpu)[min(off, ints.size - 1):]))[0]) == float(ints[min(off, ints.size - 1):].astype(np.float64).sum())
+    sq = float(_n(ops.reduce("sumsq", xd))[0])
+    assert abs(sq - (ref64 ** 2).sum()) <= 1e-5 * (ref64 ** 2).sum()
+    # max keeps the reference's rule for NaN: one in the first place is the result, one anywhere else is never selected
+    if n > 1:
+        y = x.copy(); y[n // 2] = np.nan
+        assert float(_n(ops.reduce("max", _t(y, gpu)))[0]) == oracle.max(y) == np.nanmax(y)
+    y = x.copy(); y[0] = np.nan
+    assert np.isnan(float(_n(ops.reduce("max", _t(y, gpu)))[0])) and np.isnan(oracle.max(y))
 
 
 def test_row_argmax(gpu, oracle):
