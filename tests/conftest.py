@@ -306,13 +306,15 @@ class Lazy:
 
 
 # Two correct fp32 evaluations of one sum are each a few 1e-5 to 1e-4 from float64 on the worst element of a
-# large tensor, and which of the two is further is a coin toss (observed device/oracle ratios on the tests of
-# this suite: 0.3 to 2.6; the matrix cores do not round partial sums the way a serial fp32 loop does).  The
-# float64 arbiter therefore accepts a device result up to this factor further from float64 than the oracle,
-# and one that is further from float64 than the oracle itself only up to ARBITER_CEILING times the tolerance;
-# a wrong index, a dropped term or reduced precision is off by orders of magnitude.
-ARBITER_SLACK = 4.0
-ARBITER_CEILING = 2.0
+# large tensor under the floored metric, and which of the two is further is a coin toss (observed device/oracle
+# ratios on the tests of this suite: 0.3 to 2.6; the matrix cores do not round partial sums the way a serial fp32
+# loop does).  Where the device misses the oracle under the floors, the float64 arbiter accepts it when it is within
+# the tolerance of float64, or at most this factor further from float64 than the oracle itself is.  (A fixed ceiling
+# on top of that, say twice the tolerance, does not hold: on tensors whose floor is tight the oracle itself is three
+# tolerances from float64.)  The arbiter is the weaker of two guards: every comparison that carries a float64 model
+# is also held to the condition bound (assert_condition), which has neither floor nor slack, and a wrong index, a
+# dropped term or reduced precision is off by orders of magnitude under either.
+ARBITER_SLACK = 3.0
 
 # What the run decided how: name -> worst |device - float64| / condition over the run (condition-aware check),
 # and the comparisons that the float64 arbiter settled.  Printed at the end of the session.
@@ -355,8 +357,7 @@ def assert_parity(name, got, want, want64=None, tol=PARITY_TOL, floor=None, floo
     """got (device) against want (oracle) under max_rel; prints the worst element under the fixed 1e-6 floor.
 
     With want64 (a float64 model of the same computation, or a callable giving it) a miss is still a pass
-    when the device is about as close to float64 as the oracle is (ARBITER_SLACK; further than the oracle only
-    up to ARBITER_CEILING * tol): both are then correct fp32 evaluations that differ in summation order on an element the
+    when the device is about as close to float64 as the oracle is (ARBITER_SLACK): both are then correct fp32 evaluations that differ in summation order on an element the
     floor does not cover.  When want64 carries a condition tensor (Lazy.cond), the device result is in addition
     held to |device - float64| <= tol * sum|terms| on every element (assert_condition), which has no floor."""
     cond = getattr(want64, "cond", None)
@@ -375,9 +376,7 @@ def assert_parity(name, got, want, want64=None, tol=PARITY_TOL, floor=None, floo
         e_ref = max_rel(want, want64, floor, floor_frac)
         print("       %-10s vs float64: device %.2e, oracle %.2e" % (name, e_dev, e_ref))
         ARBITER_DECIDED.append((os.environ.get("PYTEST_CURRENT_TEST", "?").split(" ")[0], name, err, e_dev, e_ref))
-        # within tol of float64: pass.  Otherwise at most ARBITER_SLACK times the oracle's own distance, and further from
-        # float64 than the oracle itself only while under ARBITER_CEILING * tol.
-        assert e_dev <= tol or (e_dev <= ARBITER_SLACK * e_ref and e_dev <= max(ARBITER_CEILING * tol, e_ref)), \
+        assert e_dev <= max(ARBITER_SLACK * e_ref, tol), \
             "%s: device %.3e from float64, oracle %.3e (device vs oracle %.3e)" % (name, e_dev, e_ref, err)
         return err
     raise AssertionError("%s differs from the oracle: max_rel %.3e >= %.1e" % (name, err, tol))
