@@ -323,7 +323,7 @@ def time_device_batch_assembly(dev):
 
 def training_step_host_layer(host, reps=100):
     """One training iteration of graphnn's example loop through the C++ host layer (FeedForward in the TRAIN
-    phase, BackPropagate, momentum-SGD update) on the configuration-2 batch; child process as end_to_end."""
+    phase, BackPropagate, momentum-SGD update) on the batch in `host`; child process as end_to_end."""
     import subprocess
     import tempfile
     from graphnn_amd import synth
@@ -341,6 +341,19 @@ def training_step_host_layer(host, reps=100):
     res["what"] = ("GetBatch-style host batch build + FactorGraph::FeedForward(TRAIN) + BackPropagate + "
                    "MomentumSGDOptimizer::Update per batch; the training plan folds the forward (levels kept), the loss "
                    "tail, the backward pass and the update of all tensors")
+    return res
+
+
+def training_step_cfg4(reps=10):
+    """The same training iteration on the configuration-4 batch (10,000 graphs, hidden 256, 5 levels): the folded training
+    plan on the wide kernels (level on the matrix cores with every level kept, backward of a level as A^T dz and a
+    product with W^T, the four weight gradients as one batch of products)."""
+    from graphnn_amd import synth
+    batch, w, cfg = synth.make_config(4)
+    res = training_step_host_layer(dict(batch=batch, cfg=cfg), reps)
+    if "us_per_batch" in res:
+        res["graphs_per_s"] = res["graphs"] / (res["us_per_batch"] * 1e-6)
+        res["ms_per_iteration"] = res["us_per_batch"] * 1e-3
     return res
 
 
@@ -426,10 +439,13 @@ def time_cfg5(dev, scale=22):
     return res
 
 
-# HBM bytes of one configuration-5 product with its plan (all launches from piece_count_kernel to piece_combine_kernel:
-# fetched 11.62 GB, written 2.91 GB) and of the level on top of it (s2v_level_stream_kernel: 2.15 + 1.07 GB more)
-CFG5_SPMM_TRAFFIC = 14530000000
-CFG5_LEVEL_TRAFFIC = 17750000000
+# Bytes the L2 exchanges with the fabric per call on configuration 5 (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 summed over the
+# launches of one call; rocprofv3 --pmc runs summarised in profiles/spmm_pieces_cfg5_fetch_write.md):
+#   sums 8.48 + 0.94, balanced pass over rows of many pieces 0.36 + 0.01, combining pass 0.24 + 0.63 (SpMM: zeros for the
+#   empty rows) or 0.24 + 0.07 (level: empty rows skipped), contraction 1.62 + 1.07, plan 2.60 + 1.34
+CFG5_TRAFFIC = {"spmm_planned": 10_658_000_000, "level_planned": 12_793_000_000, "plan": 3_940_000_000}
+CFG5_TRAFFIC["spmm"] = CFG5_TRAFFIC["spmm_planned"] + CFG5_TRAFFIC["plan"]
+CFG5_TRAFFIC["level"] = CFG5_TRAFFIC["level_planned"] + CFG5_TRAFFIC["plan"]
 CFG5_TRAFFIC_SOURCE = ("constant: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 summed over the launches of one call, from the rocprofv3 "
                        "--pmc runs summarised in profiles/spmm_pieces_cfg5_fetch_write.md (not re-measured in this run)")
 
@@ -452,17 +468,25 @@ def kernel_rooflines(dev, forwards=None):
     w5 = c5["workload"]
     if forwards is not None:
         forwards["configuration 4"] = {"forward": c4["forward"], "readout": c4["readout"]}
-        forwards["configuration 5"] = {"forward": c5["forward"]}
+        forwards["configuration 5"] = {"forward": c5["forward"], "forward_planned": c5["forward_planned"], "plan": c5["plan"]}
         forwards["one_launch_by_graphs"] = time_one_launch_by_graphs(dev)
     return [
         r4,
         hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + piece_combine_kernel<4,1> (sums of a row's pieces) + "
             "s2v_level_stream_kernel<64,true,...> (contraction over the summed rows)", w5 + ": one level, plan included",
             level_algorithmic_bytes(N, E, C), c5["level"]["avg_ms"], gather_GBps=c5["level"]["gather_GBps"],
-            traffic=CFG5_LEVEL_TRAFFIC, traffic_source=CFG5_TRAFFIC_SOURCE),
+            traffic=CFG5_TRAFFIC["level"], traffic_source=CFG5_TRAFFIC_SOURCE),
         hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + piece_combine_kernel<4,1>", w5 + ": SpMM A*h, plan included",
             spmm_algorithmic_bytes(N, N, E, C), c5["spmm"]["avg_ms"], gather_GBps=c5["spmm"]["gather_GBps"],
-            traffic=CFG5_SPMM_TRAFFIC, traffic_source=CFG5_TRAFFIC_SOURCE),
+            traffic=CFG5_TRAFFIC["spmm"], traffic_source=CFG5_TRAFFIC_SOURCE),
+        hbm("piece_sum_kernel<4,1> + hub_partial_kernel<4,1> + piece_combine_kernel<4,1> + s2v_level_stream_kernel<64,true,...>",
+            w5 + ": one level with the caller's plan (gnnhip_s2v_level_planned_f32)",
+            level_algorithmic_bytes(N, E, C), c5["level_planned"]["avg_ms"], traffic=CFG5_TRAFFIC["level_planned"],
+            traffic_source=CFG5_TRAFFIC_SOURCE),
+        hbm("piece_sum_kernel<4,1> + hub_partial_kernel<4,1> + piece_combine_kernel<4,1>",
+            w5 + ": SpMM A*h with the caller's plan (gnnhip_spmm_csr_planned_f32)",
+            spmm_algorithmic_bytes(N, N, E, C), c5["spmm_planned"]["avg_ms"], traffic=CFG5_TRAFFIC["spmm_planned"],
+            traffic_source=CFG5_TRAFFIC_SOURCE),
         hbm("sgemm_skinny_rows_kernel<1>", w5 + ": node scores h*w", 4 * N * (C + 1), c5["score"]["avg_ms"]),
         hbm("jagged_softmax_fused_kernel", w5 + ": jagged softmax over %d segments of 1024" % B,
             8 * N + 4 * B, c5["jagged_softmax"]["avg_ms"]),
@@ -639,7 +663,7 @@ def main():
     ap.add_argument("--no-rooflines", action="store_true",
                     help="skip the configuration-4 / configuration-5 kernel rooflines")
     ap.add_argument("--only", default="", help="comma-separated legs to run alone (for profiling): "
-                                                "forward, spmm, ceilings, cfg4, cfg5, train, e2e, sizes")
+                                                "forward, spmm, ceilings, cfg4, cfg5, train, train4, e2e, sizes")
     ap.add_argument("--regular", action="store_true",
                     help="configuration 3 with exactly 10 entries in every row (the other reading of its \"uniform degree\")")
     ap.add_argument("--uniform", action="store_true",
@@ -684,6 +708,8 @@ def main():
         if "train" in legs:
             _, host = build_forward_workload(dev)
             res["training_step"] = training_step_host_layer(host)
+        if "train4" in legs:
+            res["training_step_cfg4"] = training_step_cfg4()
         if "e2e" in legs:
             _, host = build_forward_workload(dev)
             res["end_to_end"] = end_to_end_host_layer(host)
@@ -759,6 +785,7 @@ def main():
     out["end_to_end"] = end_to_end_host_layer(host)
     if not args.no_rooflines:
         out["training_step"] = training_step_host_layer(host)
+        out["training_step_cfg4"] = training_step_cfg4()
 
     if not args.no_spmm:
         ev, bytes_alg, (n, nnz, d) = time_spmm_cfg3(dev, regular=args.regular)

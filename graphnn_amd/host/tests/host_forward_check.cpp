@@ -4,7 +4,9 @@
 // the CPU oracle:  inference pass (fused plan), training pass (folded forward + backward, then factor by
 // factor), gradients, two optimizer steps, checkpoint.
 //
-//   host_forward_check <dir> K C H Q L
+//   host_forward_check <dir> K C H Q L [bridges]
+//   bridges: that many extra undirected edges, node 0 of graph g to node 0 of graph g + 1 for g = 0 .. bridges - 1, added after
+//   the graphs' own edges: the batch is then not block diagonal and takes the routes that accept any adjacency
 //   <dir>/graphs.txt            dataset in graphnn's txt layout (all graphs form the batch)
 //   <dir>/w_n2l.bin w_conv.bin w_h1.bin w_h2.bin   row-major fp32
 //   -> <dir>/out.bin            see the write() calls at the bottom
@@ -46,10 +48,11 @@ static void append(std::vector<float>& out, DTensor<mode, Dtype>& t)
 
 int main(int argc, char** argv)
 {
-    ASSERT(argc == 7, "usage: host_forward_check <dir> K C H Q L");
+    ASSERT(argc == 7 || argc == 8, "usage: host_forward_check <dir> K C H Q L [bridges]");
     const std::string dir = argv[1];
     const size_t K = atoi(argv[2]), C = atoi(argv[3]), H = atoi(argv[4]), Q = atoi(argv[5]);
     const int L = atoi(argv[6]);
+    const int bridges = argc == 8 ? atoi(argv[7]) : 0;
     GpuHandle::Init(0, 1);
 
     // ---- the batch: every graph of the file
@@ -99,6 +102,14 @@ int main(int argc, char** argv)
         base += sizes[g];
     }
     y_cpu.data->row_ptr[num_graph] = num_graph;
+    {
+        std::vector<size_t> first(num_graph + 1, 0);
+        for (int g = 0; g < num_graph; ++g) first[g + 1] = first[g] + sizes[g];
+        for (int g = 0; g < bridges && g + 1 < num_graph; ++g) {
+            graph.AddEdge(edge++, (int)first[g], (int)first[g + 1]);
+            graph.AddEdge(edge++, (int)first[g + 1], (int)first[g]);
+        }
+    }
     DTensor<mode, Dtype> input;
     SpTensor<mode, Dtype> label;
     input.CopyFrom(x_cpu);
