@@ -299,6 +299,33 @@ def time_one_launch_by_graphs(dev, sizes=(256, 400, 600, 1024, 2000)):
     return res
 
 
+def time_forward_hidden128(dev):
+    """The configuration-2 batch (256 graphs) with hidden size 128: the one-launch forward (eight wavefronts per graph)
+    beside the general route (input + 4 levels on the matrix-core kernel + readout)."""
+    import torch
+    from graphnn_amd import batching, ops, synth
+    batch, _, cfg = synth.make_config(2)
+    C = 128
+    w = synth.make_weights(synth.Stream(synth.config_seed(2) + C), cfg["K"], C, cfg["H"], cfg["Q"])
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    t = lambda arr: torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
+    a_d, s_d = tuple(map(t, a)), tuple(map(t, s))
+    X, Wn, Wc, W1, W2 = t(batch.one_hot()), t(w.W_n2l), t(w.W_conv), t(w.W_h1), t(w.W_h2)
+    N, B, H, Q, L = batch.num_nodes, batch.num_graphs, cfg["H"], cfg["Q"], cfg["L"]
+    bb = ops.BatchedBuffers(N, B, C, H, Q, dev)
+    fb = ops.ForwardBuffers(N, B, C, H, Q, dev)
+    nmax = int(batch.graph_sizes.max())
+    one = _event_median_ms(lambda: ops.s2v_forward_batched(a_d, s_d, X, Wn, Wc, W1, W2, L, nmax, bufs=bb), 100)
+    gen = _event_median_ms(lambda: ops.s2v_forward(a_d, s_d, X, Wn, Wc, W1, W2, L, bufs=fb), 100)
+    assert int(bb.status.cpu()[0]) == 0
+    assert bool((bb.pred == fb.pred).all()), "routes disagree on predictions at hidden 128"
+    assert float((bb.logits - fb.logits).abs().max()) <= 1e-4 * float(fb.logits.abs().max()), "routes disagree on logits at hidden 128"
+    return {"workload": "configuration-2 batch with hidden 128: %d graphs, %d nodes, %d levels" % (B, N, L),
+            "one_launch": {"median_us": one["median_ms"] * 1e3, "graphs_per_s": B / (one["median_ms"] * 1e-3)},
+            "general_route": {"median_us": gen["median_ms"] * 1e3, "graphs_per_s": B / (gen["median_ms"] * 1e-3)}}
+
+
 def time_device_batch_assembly(dev):
     """CSR of A from the flat edge list of configuration 4 on the device (stable radix sort) and the CSR
     transposition used by the backward pass, beside the numpy host builder for the same edge list."""
@@ -470,6 +497,7 @@ def kernel_rooflines(dev, forwards=None):
         forwards["configuration 4"] = {"forward": c4["forward"], "readout": c4["readout"]}
         forwards["configuration 5"] = {"forward": c5["forward"], "forward_planned": c5["forward_planned"], "plan": c5["plan"]}
         forwards["one_launch_by_graphs"] = time_one_launch_by_graphs(dev)
+        forwards["hidden_128"] = time_forward_hidden128(dev)
     return [
         r4,
         hbm("plan of the column-ordered pieces + piece_sum_kernel<4,1> + piece_combine_kernel<4,1> (sums of a row's pieces) + "
@@ -663,7 +691,7 @@ def main():
     ap.add_argument("--no-rooflines", action="store_true",
                     help="skip the configuration-4 / configuration-5 kernel rooflines")
     ap.add_argument("--only", default="", help="comma-separated legs to run alone (for profiling): "
-                                                "forward, spmm, ceilings, cfg4, cfg5, train, train4, e2e, sizes")
+                                                "forward, spmm, ceilings, cfg4, cfg5, train, train4, e2e, sizes, h128")
     ap.add_argument("--regular", action="store_true",
                     help="configuration 3 with exactly 10 entries in every row (the other reading of its \"uniform degree\")")
     ap.add_argument("--uniform", action="store_true",
@@ -715,6 +743,8 @@ def main():
             res["end_to_end"] = end_to_end_host_layer(host)
         if "sizes" in legs:
             res["one_launch_by_graphs"] = time_one_launch_by_graphs(dev)
+        if "h128" in legs:
+            res["hidden_128"] = time_forward_hidden128(dev)
         if args.calibrate:
             n = 1 << 28
             src = torch.ones(n, device=dev, dtype=torch.float32)

@@ -717,41 +717,58 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_graph_forward_kernel(
             continue;
         }
         // ---- readout: weighted sum-pool over the graph's rows, then the two small dense layers.
-        // Pooling: a lane owns one column and walks rows, so at C = 64 nothing crosses lanes; one partial
-        // per wavefront goes to LDS.
+        // Pooling: a lane owns one column (two at C = 128: lane and lane + 64) and walks rows, so from C = 64 on
+        // nothing crosses lanes; one partial per wavefront goes to LDS.
+        constexpr int CPL = (C + kWave - 1) / kWave;         // columns per lane
         {
             constexpr int GP = (C < kWave) ? C : kWave;      // lanes per row
             constexpr int RS = kWave / GP;                   // rows per wavefront per step
             const int pc = lane % GP, pr = lane / GP;
-            float acc = 0.f;
-            for (int lr = wave * RS + pr; lr < n; lr += kWavesPerBlock * RS)
-                acc = fmaf(l_sv[lr], hbuf[(size_t)lr * LDT + pc], acc);
+            float acc[CPL];
 #pragma unroll
-            for (int off = GP; off < kWave; off <<= 1) acc += __shfl_xor(acc, off, kWave);
-            if (lane < GP) part[(size_t)wave * C + pc] = acc;
+            for (int u = 0; u < CPL; ++u) acc[u] = 0.f;
+            for (int lr = wave * RS + pr; lr < n; lr += kWavesPerBlock * RS)
+#pragma unroll
+                for (int u = 0; u < CPL; ++u) acc[u] = fmaf(l_sv[lr], hbuf[(size_t)lr * LDT + pc + u * kWave], acc[u]);
+            if constexpr (CPL == 1) {
+#pragma unroll
+                for (int off = GP; off < kWave; off <<= 1) acc[0] += __shfl_xor(acc[0], off, kWave);
+            }
+            if (lane < GP) {
+#pragma unroll
+                for (int u = 0; u < CPL; ++u) part[(size_t)wave * C + pc + u * kWave] = acc[u];
+            }
         }
         __syncthreads();
         GNNHIP_PHASE_MARK(12);
-        // every wavefront adds up its own copy of the pooled row (lane c holds column c; C <= 64)
-        float plv = 0.f;
-        if (lane < C) {
+        // every wavefront adds up its own copy of the pooled row (lane c holds column c, and c + 64 at C = 128)
+        float plv[CPL];
 #pragma unroll
-            for (int p = 0; p < kWavesPerBlock; ++p) plv += part[(size_t)p * C + lane];
+        for (int u = 0; u < CPL; ++u) {
+            plv[u] = 0.f;
+            if (lane + u * kWave < C) {
+#pragma unroll
+                for (int p = 0; p < kWavesPerBlock; ++p) plv[u] += part[(size_t)p * C + lane + u * kWave];
+            }
+            if (wave == 0 && lane + u * kWave < C) pool[(size_t)g * C + lane + u * kWave] = plv[u];
         }
-        if (wave == 0 && lane < C) pool[(size_t)g * C + lane] = plv;
         GNNHIP_PHASE_MARK(13);
         // hidden layer: one wavefront per output, two outputs per step so that their reductions overlap
         for (int j = wave; j < H; j += 2 * kWavesPerBlock) {
             const int j1 = j + kWavesPerBlock;
             const bool two = j1 < H;
             float s0 = 0.f, s1 = 0.f;
-            if (lane < C) {
-                if (ro_staged) {
-                    s0 = plv * w1s[j * C + lane];
-                    if (two) s1 = plv * w1s[j1 * C + lane];
-                } else {
-                    s0 = plv * Wh1[(size_t)lane * H + j];
-                    if (two) s1 = plv * Wh1[(size_t)lane * H + j1];
+#pragma unroll
+            for (int u = 0; u < CPL; ++u) {
+                const int c = lane + u * kWave;
+                if (c < C) {
+                    if (ro_staged) {
+                        s0 = fmaf(plv[u], w1s[j * C + c], s0);
+                        if (two) s1 = fmaf(plv[u], w1s[j1 * C + c], s1);
+                    } else {
+                        s0 = fmaf(plv[u], Wh1[(size_t)c * H + j], s0);
+                        if (two) s1 = fmaf(plv[u], Wh1[(size_t)c * H + j1], s1);
+                    }
                 }
             }
             s0 = relu_ref(wave_sum(s0));
@@ -853,7 +870,7 @@ int launch_graph_forward(int B, int K, int H, int Q, int L, int n16max,
     const size_t smem = sizeof(float) * (GraphLds::fixed_floats(n16max, C, K, H, Q, kBlock, LABELS) + 2 * (size_t)ecap);
     constexpr bool kKeepBuilt = !LABELS;    // the variant that keeps all levels exists for the dense input only
     // the variant that packs graphs into bins exists for the workgroup shapes bins of 128 nodes and more select
-    constexpr bool kPackBuilt = (WAVES == 16) || (C == 16 && WAVES == 8);
+    constexpr bool kPackBuilt = C <= 64 && ((WAVES == 16) || (C == 16 && WAVES == 8));
     const bool keep = h_levels != nullptr;
     if (keep && !kKeepBuilt) return GNNHIP_EUNSUPPORTED;
     if (pack && (!kPackBuilt || keep)) return GNNHIP_EUNSUPPORTED;
@@ -928,10 +945,16 @@ int dispatch_waves(bool labels, int B, int K, int H, int Q, int L, int n16max,
 {
 #define GNNHIP_GF_ARGS B, K, H, Q, L, n16max, a_row_ptr, a_col_idx, a_val, s_row_ptr, s_col_idx, s_val, \
                        X, Wn2l, Wc, Wh1, Wh2, msg, h_final, pool, hidden, logits, probs, pred, status, h_levels, level_stride, pack, s
-    const int tasks = (C / 16) * (n16max / 16);         // (column block x row tile) tasks of the largest graph
-    if (tasks <= 4) return dispatch_ksx<C, 4>(labels, GNNHIP_GF_ARGS);
-    if (tasks <= 8) return dispatch_ksx<C, 8>(labels, GNNHIP_GF_ARGS);
-    return dispatch_ksx<C, 16>(labels, GNNHIP_GF_ARGS);
+    // hidden 128: eight wavefronts, one per 16-column block (64 registers of a lane hold W^T and the tile operand of
+    // a contraction; sixteen wavefronts would leave a lane 128 registers in all)
+    if constexpr (C == 128) {
+        return dispatch_ksx<C, 8>(labels, GNNHIP_GF_ARGS);
+    } else {
+        const int tasks = (C / 16) * (n16max / 16);         // (column block x row tile) tasks of the largest graph
+        if (tasks <= 4) return dispatch_ksx<C, 4>(labels, GNNHIP_GF_ARGS);
+        if (tasks <= 8) return dispatch_ksx<C, 8>(labels, GNNHIP_GF_ARGS);
+        return dispatch_ksx<C, 16>(labels, GNNHIP_GF_ARGS);
+    }
 #undef GNNHIP_GF_ARGS
 }
 
@@ -957,8 +980,8 @@ int forward_batched_entry(bool labels, int N, int B, int K, int C, int H, int Q,
                    "null input in s2v_forward_batched");
     GNNHIP_REQUIRE(msg && h_final && pool && hidden && logits, "null output in s2v_forward_batched");
     if (int rc = require_ready()) return rc;
-    if (!(C == 16 || C == 32 || C == 64) || (!labels && K > 64))
-        return set_error(GNNHIP_EUNSUPPORTED, "graph-resident forward supports hidden 16/32/64 and at most 64 dense feature columns (C=%d K=%d)", C, K);
+    if (!(C == 16 || C == 32 || C == 64 || C == 128) || (!labels && K > 64))
+        return set_error(GNNHIP_EUNSUPPORTED, "graph-resident forward supports hidden 16/32/64/128 and at most 64 dense feature columns (C=%d K=%d)", C, K);
     if (!(aligned16(msg) && aligned16(h_final)))
         return set_error(GNNHIP_EUNSUPPORTED, "msg and h_final must be 16-byte aligned");
     if (labels && !aligned16(W_n2l))
@@ -976,6 +999,7 @@ int forward_batched_entry(bool labels, int N, int B, int K, int C, int H, int Q,
         switch (C) {
         case 16: return dispatch_waves<16>(GNNHIP_GF_ARGS);
         case 32: return dispatch_waves<32>(GNNHIP_GF_ARGS);
+        case 128: return dispatch_waves<128>(GNNHIP_GF_ARGS);
         default: return dispatch_waves<64>(GNNHIP_GF_ARGS);
         }
 #undef GNNHIP_GF_ARGS

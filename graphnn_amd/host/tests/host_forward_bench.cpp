@@ -9,6 +9,7 @@
 // FeedForward in the TRAIN phase, BackPropagate from the loss, one momentum-SGD update; the loss is read
 // back once at the end, as the example only reads it on report iterations.
 #include <chrono>
+#include <cmath>
 #include <cstdio>
 #include <fstream>
 #include <map>
@@ -66,7 +67,9 @@ int main(int argc, char** argv)
     auto w_conv = add_diff<DTensorVar>(model, "w_conv", {C, C});
     auto w_h1 = add_diff<DTensorVar>(model, "w_h1", {C, H});
     auto w_h2 = add_diff<DTensorVar>(model, "w_h2", {H, Q});
-    for (auto& p : {w_n2l, w_conv, w_h1, w_h2}) { p->value.SetRandN(0, 0.1f); fg.AddParam(p); }
+    // (standard deviation 0.1 at hidden 64, scaled down with the width so that the embeddings of wide networks stay finite)
+    const float w_std = 0.1f * std::sqrt(64.0f / (float)(C > 64 ? C : 64));
+    for (auto& p : {w_n2l, w_conv, w_h1, w_h2}) { p->value.SetRandN(0, w_std); fg.AddParam(p); }
     auto x_var = add_const< DTensorVar<mode, Dtype> >(fg, "data", true);
     auto y_var = add_const< SpTensorVar<mode, Dtype> >(fg, "label", true);
     auto msg = af<MatMul>(fg, {x_var, w_n2l});
@@ -146,6 +149,6 @@ int main(int argc, char** argv)
            "\"%s\": %.2f, \"fused_factors\": %d, \"plan_steps\": %d, \"checksum\": %.6f}\n",
            num_graph, N, reps, train ? "train" : "test", (t_build + t_device) / reps, t_build / reps,
            train ? "us_csr_copy_forward_backward_update" : "us_csr_copy_forward_readback", t_device / reps,
-           (int)fg.LastPlanFusedCount(), (int)fg.LastPlanFactorCount(), checksum);
+           (int)fg.LastPlanFusedCount(), (int)fg.LastPlanFactorCount(), std::isfinite(checksum) ? checksum : -1.0f);
     return 0;
 }

@@ -1035,7 +1035,9 @@ def test_batched_forward_matches_reference_path(gpu, oracle, config_id):
 @pytest.mark.parametrize("C,K,H,Q,L", [(16, 7, 8, 3, 2), (32, 20, 16, 2, 3), (64, 64, 32, 5, 1), (64, 3, 100, 70, 0),
                                        (32, 48, 8, 2, 5), (16, 33, 4, 2, 1),
                                        # label counts around the steps of the input stage (two columns per 64-bit read)
-                                       (64, 1, 8, 2, 2), (32, 2, 8, 2, 1), (64, 17, 16, 3, 2), (16, 49, 8, 2, 1)])
+                                       (64, 1, 8, 2, 2), (32, 2, 8, 2, 1), (64, 17, 16, 3, 2), (16, 49, 8, 2, 1),
+                                       # hidden 128: eight wavefronts, a lane carries two columns through the readout
+                                       (128, 7, 16, 2, 2), (128, 38, 32, 2, 4), (128, 64, 100, 70, 1), (128, 3, 8, 2, 0)])
 def test_batched_forward_shapes(gpu, oracle, C, K, H, Q, L):
     seed = 1000 + C + K + L
     batch = synth.molecule_batch(seed, 37, K, Q, size_mode="uniform", size_lo=1, size_hi=70)
@@ -1234,7 +1236,7 @@ def test_batched_forward_with_graphs_of_no_nodes(gpu, oracle, B):
     assert np.array_equal(_n(bufs.pred)[none], want["pred"][none])
 
 
-@pytest.mark.parametrize("C,L,B", [(64, 4, 256), (16, 1, 37), (32, 3, 300), (64, 0, 9)])
+@pytest.mark.parametrize("C,L,B", [(64, 4, 256), (16, 1, 37), (32, 3, 300), (64, 0, 9), (128, 3, 100), (128, 4, 256)])
 def test_batched_forward_keeps_every_level_for_training(gpu, oracle, C, L, B):
     """the one-launch forward of a training iteration: h_0 .. h_L as the per-level entry points give them (which
     have their own parity tests), every other output with the bits of the inference entry"""
@@ -1252,9 +1254,9 @@ def test_batched_forward_keeps_every_level_for_training(gpu, oracle, C, L, B):
     for k in ("msg", "pool", "hidden", "logits", "probs", "pred"):
         assert np.array_equal(_n(getattr(bufs, k)), _n(getattr(plain, k))), k
     assert np.array_equal(_n(hl[L]), _n(plain.h_final))
-    want = oracle.forward(a, s, batch.one_hot(), w, L, None)
+    want = _forward_want(oracle, a, s, batch.one_hot(), w, L, None)
     for l in range(L + 1):
-        assert max_rel(_n(hl[l]), want["h"][l]) < PARITY_TOL, l
+        assert_parity("h%d" % l, _n(hl[l]), want["h"][l], want["_f64"]["h"][l])
     assert np.array_equal(_n(hl[0]), np.maximum(_n(bufs.msg), 0))
     assert_stages(" (one launch, levels kept)", a, s, batch.one_hot(), w,
                   dict(msg=_n(bufs.msg), h=_n(hl), pool=_n(bufs.pool), hidden=_n(bufs.hidden), logits=_n(bufs.logits), probs=_n(bufs.probs)))
@@ -1352,7 +1354,7 @@ def test_batched_forward_from_labels_has_the_bits_of_the_one_hot_route(gpu, orac
 
 
 @pytest.mark.parametrize("C,K,H,Q,L,B", [(16, 7, 8, 3, 2, 37), (32, 200, 16, 2, 3, 300), (64, 64, 32, 5, 1, 1025), (64, 1, 8, 2, 0, 9),
-                                         (64, 130, 32, 2, 2, 40)])
+                                         (64, 130, 32, 2, 2, 40), (128, 38, 32, 2, 4, 256), (128, 100, 16, 3, 2, 300)])
 def test_batched_forward_from_labels_shapes(gpu, oracle, C, K, H, Q, L, B):
     """label tables that fit LDS (K C <= 8192 floats) and ones read from L2, more than 64 label types (the dense
     route stops at 64 columns), no level, more graphs than workgroups; a label out of range sets status bit 3"""
