@@ -81,13 +81,15 @@ def time_forward(dev_args, cfg, batch, steps, warmup, route, device_times=None):
     if route.startswith("graph_resident"):
         assert int(bufs.status.cpu()[0]) == 0, "graph-resident forward reported a layout violation"
     if device_times is not None:
-        device_times[route] = _event_median_ms(run, max(50, min(steps, 500)))
+        device_times[route] = _event_median_ms(run, 50, inner=20)
     return (t1 - t0) / steps, bufs
 
 
-def _event_median_ms(fn, reps, warmup=5):
-    """Device time of one call of fn: a pair of HIP events around every one of `reps` calls on the stream the launches
-    go to (torch's current stream), after `warmup` untimed calls; returns {median, min, mean, runs} in milliseconds."""
+def _event_median_ms(fn, reps, warmup=5, inner=1):
+    """Device time of one call of fn: a pair of HIP events around every group of `inner` back-to-back calls on the stream
+    the launches go to (torch's current stream), `reps` groups after `warmup` untimed calls; {median, min, mean, runs}
+    in milliseconds per call.  A pair of events around a single launch of a few microseconds mostly measures the events
+    (about 17 us on this GPU), so short kernels are timed in groups."""
     import torch
     for _ in range(warmup):
         fn()
@@ -95,11 +97,13 @@ def _event_median_ms(fn, reps, warmup=5):
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
     for e0, e1 in evs:
         e0.record()
-        fn()
+        for _ in range(inner):
+            fn()
         e1.record()
     torch.cuda.synchronize()
-    ms = np.array([e0.elapsed_time(e1) for e0, e1 in evs])
-    return {"median_ms": float(np.median(ms)), "min_ms": float(ms.min()), "mean_ms": float(ms.mean()), "runs": int(reps)}
+    ms = np.array([e0.elapsed_time(e1) for e0, e1 in evs]) / inner
+    return {"median_ms": float(np.median(ms)), "min_ms": float(ms.min()), "mean_ms": float(ms.mean()), "runs": int(reps),
+            "launches_per_event_pair": int(inner)}
 
 
 def time_forward_pipelined(dev_args, cfg, batch, steps, warmup, nstreams=4):
@@ -316,8 +320,8 @@ def time_forward_hidden128(dev):
     bb = ops.BatchedBuffers(N, B, C, H, Q, dev)
     fb = ops.ForwardBuffers(N, B, C, H, Q, dev)
     nmax = int(batch.graph_sizes.max())
-    one = _event_median_ms(lambda: ops.s2v_forward_batched(a_d, s_d, X, Wn, Wc, W1, W2, L, nmax, bufs=bb), 100)
-    gen = _event_median_ms(lambda: ops.s2v_forward(a_d, s_d, X, Wn, Wc, W1, W2, L, bufs=fb), 100)
+    one = _event_median_ms(lambda: ops.s2v_forward_batched(a_d, s_d, X, Wn, Wc, W1, W2, L, nmax, bufs=bb), 30, inner=20)
+    gen = _event_median_ms(lambda: ops.s2v_forward(a_d, s_d, X, Wn, Wc, W1, W2, L, bufs=fb), 30, inner=20)
     assert int(bb.status.cpu()[0]) == 0
     assert bool((bb.pred == fb.pred).all()), "routes disagree on predictions at hidden 128"
     assert float((bb.logits - fb.logits).abs().max()) <= 1e-4 * float(fb.logits.abs().max()), "routes disagree on logits at hidden 128"
@@ -780,8 +784,9 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": sec * 1e3,
-        # the same launch between two HIP events, median over the runs: what the device spends on one forward (the wall
-        # figure above also carries the host's launch work and one synchronisation per `steps` forwards)
+        # the same launch between HIP events (20 forwards per pair of events, median over 50 pairs): what the device
+        # spends on one forward with the launches queued back to back (the wall figure above also carries the host's
+        # launch work and one synchronisation per `steps` forwards)
         "device_ms_per_step": dev_ms["graph_resident"]["median_ms"],
         "device_ms": dev_ms["graph_resident"],
         "higher_is_better": True,

@@ -11,6 +11,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <atomic>
 #include <map>
 #include <string.h>
 #include <mutex>
@@ -160,12 +161,20 @@ int pool_release(void* p)
 
 int stream_scratch(hipStream_t s, size_t bytes, void** p) { return stream_scratch_slot(s, 0, bytes, p); }
 
+// Test hook (exported, not part of the public header): the next request for this scratch slot fails as if the device
+// were out of memory, so that the tests can walk the fallback paths that a full device would take.  -1: off.
+static std::atomic<int> g_fail_scratch_slot{-1};
+extern "C" void gnnhip_test_fail_next_scratch(int slot) { g_fail_scratch_slot.store(slot); }
+
 int stream_scratch_slot(hipStream_t s, int which, size_t bytes, void** p)
 {
     Runtime& r = rt();
     std::lock_guard<std::mutex> lock(r.mu);
     if (!r.ready) return set_error(GNNHIP_ENOTINIT, "gnnhip_init has not been called");
     if (which < 0 || which >= kScratchSlots) return set_error(GNNHIP_EINVAL, "bad scratch slot %d", which);
+    int expected = which;
+    if (g_fail_scratch_slot.compare_exchange_strong(expected, -1))
+        return set_error(GNNHIP_ENOMEM, "scratch slot %d: allocation failure injected by gnnhip_test_fail_next_scratch", which);
     auto& slot = r.scratch[std::make_pair(s, which)];
     if (slot.second < bytes) {
         size_t want = (bytes + 65535) / 65536 * 65536;

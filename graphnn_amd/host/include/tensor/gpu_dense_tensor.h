@@ -55,8 +55,11 @@ public:
         Reshape(src.shape.dims);
         GNN_HIP(gnnhip_memcpy_d2d(data->ptr, src.data->ptr, sizeof(Dtype) * shape.Count(), GpuHandle::Stream()));
     }
-    void ShallowCopy(DTensor<GPU, Dtype>& src) { shape = src.shape; data = src.data; }
-    void Zeros() { GNN_HIP(gnnhip_memset0(data->ptr, sizeof(Dtype) * shape.Count(), GpuHandle::Stream())); }
+    void ShallowCopy(DTensor<GPU, Dtype>& src) { Touched(); shape = src.shape; data = src.data; }
+    void Zeros() { Touched(); GNN_HIP(gnnhip_memset0(data->ptr, sizeof(Dtype) * shape.Count(), GpuHandle::Stream())); }
+    // every method that writes the tensor in place calls this: a host copy of its value fetched earlier (AsScalar of a
+    // grouped scalar) no longer stands for it, and the next AsScalar reads the device again, as graphnn's does every time
+    void Touched() { scalars.reset(); }
     // blocking read of a one-element tensor: the forward's only synchronisation point
     Dtype AsScalar()
     {
@@ -181,11 +184,13 @@ public:
     void Softmax()
     {
         ASSERT(rank() == 2, "Softmax is assumed to exec on matrix");
+        Touched();
         GNN_HIP(gnnhip_row_softmax_f32(data->ptr, (int)rows(), (int)cols(), GpuHandle::Stream()));
     }
     void JaggedSoftmax(DTensor<GPU, int>& lens)
     {
         ASSERT(rows() == shape.Count(), "input must be a column vector");
+        Touched();
         GNN_HIP(gnnhip_jagged_softmax_f32(data->ptr, lens.data->ptr, (int)lens.shape.Count(), GpuHandle::Stream()));
     }
     void Sum(DTensor<GPU, Dtype>& a, int axis = -1)
@@ -210,12 +215,14 @@ public:
     void Axpy(Dtype a, DTensor<GPU, Dtype>& x)
     {
         ASSERT(shape == x.shape, "shape doesn't match in Axpy");
+        Touched();
         GNN_HIP(gnnhip_axpy_f32(shape.Count(), a, x.data->ptr, data->ptr, GpuHandle::Stream()));
     }
     void Axpy(Dtype a, SpTensor<GPU, Dtype>& x);
     void Axpby(Dtype a, DTensor<GPU, Dtype>& x, Dtype b)
     {
         ASSERT(shape == x.shape, "shape doesn't match in Axpby");
+        Touched();
         GNN_HIP(gnnhip_axpby_f32(shape.Count(), a, x.data->ptr, b, data->ptr, GpuHandle::Stream()));
     }
     void ElewiseMul(DTensor<GPU, Dtype>& src);
@@ -255,6 +262,7 @@ public:
 private:
     void Unary(int op, Dtype a0 = 0, Dtype a1 = 0)
     {
+        Touched();
         GNN_HIP(gnnhip_unary_f32(op, data->ptr, shape.Count(), a0, a1, GpuHandle::Stream()));
     }
 };

@@ -76,6 +76,7 @@ public:
 // ---- dense methods that take the types above
 inline void TensorTemplate<GPU, DENSE, float>::ElewiseMul(DTensor<GPU, float>& src)
 {
+    Touched();
     if (src.shape == shape) {
         GNN_HIP(gnnhip_mul_f32(shape.Count(), src.data->ptr, data->ptr, GpuHandle::Stream()));
         return;

@@ -186,6 +186,7 @@ inline void TensorTemplate<GPU, DENSE, float>::MM(SpTensor<GPU, float>& a, DTens
 inline void TensorTemplate<GPU, DENSE, float>::Axpy(float a, SpTensor<GPU, float>& x)
 {
     ASSERT(shape == x.shape, "shape doesn't match in Axpy");
+    Touched();
     GNN_HIP(gnnhip_csr_axpy_f32((int)x.rows(), (int)x.cols(), a, x.data->row_ptr, x.data->col_idx, x.data->val,
                                 data->ptr, GpuHandle::Stream()));
 }

@@ -164,6 +164,15 @@ int main(int argc, char** argv)
     out.push_back(loss->AsScalar());
     out.push_back(acc->AsScalar());
     append(out, logits->value);
+    {
+        // loss and accuracy were fetched together behind one wait; a tensor written in place afterwards must be read
+        // from the device again (graphnn's AsScalar reads the device every time)
+        const float l0 = loss->AsScalar();
+        loss->value.Scale(2.0f);
+        ASSERT(loss->value.AsScalar() == 2.0f * l0, "AsScalar returned a value fetched before the tensor was rewritten");
+        loss->value.Scale(0.5f);
+        ASSERT(loss->value.AsScalar() == l0, "AsScalar after the second in-place write");
+    }
     // 2. training pass: the plan folds the forward (keeping every level for its backward pass) and the loss tail
     fg.FeedForward(targets, feed, Phase::TRAIN);
     out.push_back((float)fg.LastPlanFactorCount());

@@ -1568,6 +1568,42 @@ def test_spmm_with_a_plan_has_the_bits_of_the_call_without(gpu, oracle, n):
     assert_parity("spmm", got, want, w64)
 
 
+@pytest.mark.parametrize("slot", [1, 3, 4])
+def test_spmm_falls_back_with_the_output_untouched_when_scratch_cannot_be_had(gpu, oracle, slot):
+    """The column-ordered route takes all its scratch (slot 3: plan, 4: partial sums, 1: the balanced pass over rows of
+    many pieces) before its first launch.  When one of the requests fails (injected through the library's test hook, as
+    a full device would fail it), the product falls back to the row-group route with C as the caller left it: with
+    beta != 0, beta is applied exactly once."""
+    import ctypes
+    from graphnn_amd import ops
+    from graphnn_amd._lib import load_library
+    rng = np.random.default_rng(950 + slot)
+    a = synth.rmat_csr(0x5EED0005, 16, 16 << 16)
+    N, n = 1 << 16, 64
+    v = (rng.random(a[1].size) * 0.2 - 0.05).astype(np.float32)
+    csr = (a[0], a[1], v)
+    csr_d = _csr_t(csr, gpu)
+    B = rng.standard_normal((N, n)).astype(np.float32)
+    C0 = rng.standard_normal((N, n)).astype(np.float32)
+    normal = _n(ops.spmm(*csr_d, _t(B, gpu), N, alpha=-0.5, beta=1.5, out=_t(C0, gpu)))
+    lib = load_library()
+    lib.gnnhip_test_fail_next_scratch.argtypes = [ctypes.c_int]
+    lib.gnnhip_test_fail_next_scratch.restype = None
+    lib.gnnhip_test_fail_next_scratch(slot)
+    try:
+        got = _n(ops.spmm(*csr_d, _t(B, gpu), N, alpha=-0.5, beta=1.5, out=_t(C0, gpu)))
+    finally:
+        lib.gnnhip_test_fail_next_scratch(-1)
+    want, w64 = _spmm_want(oracle, *csr, B, N, alpha=-0.5, beta=1.5, C=C0)
+    assert_parity("spmm after a failed scratch request", got, want, w64)
+    # the fallback is another route (its sums run in another order), so the bits differ from the normal call's somewhere,
+    # while a beta applied twice would be off by |0.75 C0| ~ 1 everywhere
+    assert not np.array_equal(got, normal)
+    assert np.abs(got - normal).max() < 1e-3
+    # and the next call takes the normal route again
+    assert np.array_equal(_n(ops.spmm(*csr_d, _t(B, gpu), N, alpha=-0.5, beta=1.5, out=_t(C0, gpu))), normal)
+
+
 def test_plan_of_matrices_that_take_the_other_routes(gpu, oracle):
     """a plan is made for any matrix: small ones, sparse ones and ones with a few very long rows keep the row-group
     route (with the balanced pass over long rows, whose plan is then kept); no rows, no entries"""
