@@ -832,7 +832,7 @@ def main():
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
             "traffic_source": "constant: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 of spmm_rowgroup_kernel<4,1> from the rocprofv3 "
-                              "--pmc runs summarised in profiles/bench_forward_cfg2_spmm_cfg3.md (not re-measured in this run). "
+                              "--pmc runs summarised in profiles/spmm_cfg3_fetch_write_and_hbm_ceilings.md (not re-measured in this run). "
                               "These counters count what the L2 asks of the fabric; the 256 MB memory-side cache sits behind that "
                               "point and no counter this profiler exposes tells its hits from HBM reads",
             "kernel": "spmm_rowgroup_kernel<4,1>",
