@@ -44,6 +44,12 @@ __device__ __forceinline__ void buf_store4(rsrc_t r, int voff, int soff, const f
     __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, soff, 0);
 }
 
+__device__ __forceinline__ void buf_store2(rsrc_t r, int voff, int soff, const float2& x)
+{
+    const u32x2 v = {__float_as_uint(x.x), __float_as_uint(x.y)};
+    __builtin_amdgcn_raw_buffer_store_b64(v, r, voff, soff, 0);
+}
+
 }  // namespace gnnhip
 
 #endif

@@ -345,6 +345,18 @@ void launch_skinny(bool tb, int m, int k, float alpha, const float* A, int lda, 
 
 }  // namespace
 
+// gemm_tn_tall.hip: square outputs of 128 / 256 over a very long k
+bool gemm_tn_tall_applies(int m, int n, int k, const float* A, int lda, const float* B, int ldb);
+int gemm_tn_tall_dispatch(int m, int n, int k, float alpha, const float* A, int lda, const float* B, int ldb, float beta, float* C,
+                          int ldc, hipStream_t s);
+
+void launch_splitk_reduce(int m, int n, int splits, float alpha, const float* partial, float beta, float* C, int ldc, hipStream_t s)
+{
+    const size_t total = (size_t)m * n;
+    const unsigned rgrid = ceil_div_u(total, kWave) < 2048u ? ceil_div_u(total, kWave) : 2048u;
+    hipLaunchKernelGGL(sgemm_splitk_reduce_kernel, dim3(rgrid), dim3(kBlock), 0, s, m, n, splits, alpha, partial, beta, C, ldc);
+}
+
 // length of the ranges of k when few output tiles share a long k: about two workgroups per CU, four steps at least
 inline long long splitk_chunk(long long tiles, long long k)
 {
@@ -366,6 +378,11 @@ int gemm_tn_batch_dispatch(int count, const int* m, const int* n, const int* k, 
     int z = 0;
     for (int p = 0; p < count; ++p) {
         if (m[p] == 0 || n[p] == 0) continue;
+        // the rule of the single product here too: a wide square output over a very long k has a kernel of its own
+        if (gemm_tn_tall_applies(m[p], n[p], k[p], A[p], lda[p], B[p], ldb[p])) {
+            if (int rc = gemm_tn_tall_dispatch(m[p], n[p], k[p], alpha, A[p], lda[p], B[p], ldb[p], beta, C[p], ldc[p], s)) return rc;
+            continue;
+        }
         const int q = b.count++;
         b.A[q] = A[p]; b.B[q] = B[p]; b.C[q] = C[p];
         b.m[q] = m[p]; b.n[q] = n[p]; b.k[q] = k[p];
@@ -408,6 +425,9 @@ int gemm_dispatch(int transA, int transB, int m, int n, int k, float alpha, cons
         }
         GNNHIP_LAUNCH_CHECK("sgemm_skinny");
         return GNNHIP_OK;
+    }
+    if (transA && !transB) {
+        if (int rc = gemm_tn_tall_dispatch(m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, s); rc != GNNHIP_EUNSUPPORTED) return rc;
     }
     dim3 grid(ceil_div_u((size_t)m, BM), ceil_div_u((size_t)n, BN));
     dim3 block(kBlock);

@@ -47,6 +47,8 @@ int level_wide_dispatch(int N, int C, long long nnz, const int* row_ptr, const i
                         const float* h_in, const float* W, const float* msg, const float* bias, float* h_out, bool relu_in,
                         hipStream_t s);
 bool level_wide_covers(int N, int C);
+int level_wide_backward_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* dz, const float* W,
+                                 float* u, float* g_prev, const float* gate, float* acc, hipStream_t s);
 
 namespace {
 
@@ -681,6 +683,15 @@ int level_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* c
 int level_backward_dispatch(int N, int C, long long nnz, const int* row_ptr, const int* col_idx, const float* val, const float* dz,
                             const float* W, float* u, float* g_prev, const float* gate, float* acc, hipStream_t s)
 {
+    if (C == 128 || C == 256) {
+        // hidden 128 / 256: the wide kernel's backward variant, except where the forward takes two steps too (large
+        // graphs with many entries per row: the wide kernel sums a row of any length inside one wavefront)
+        if (!level_wide_covers(N, C)) return GNNHIP_EUNSUPPORTED;
+        if (N >= kHubMinRows && nnz >= two_step_degree() * (long long)N) return GNNHIP_EUNSUPPORTED;
+        if (!(aligned16(dz) && aligned16(W) && aligned16(u) && aligned16(g_prev) && (!gate || aligned16(gate)) && (!acc || aligned16(acc))))
+            return GNNHIP_EUNSUPPORTED;
+        return level_wide_backward_dispatch(N, C, row_ptr, col_idx, val, dz, W, u, g_prev, gate, acc, s);
+    }
     if (!(C == 16 || C == 32 || C == 64) || !level_stream_covers(N, C)) return GNNHIP_EUNSUPPORTED;
     if (!(aligned16(dz) && aligned16(W) && aligned16(u) && aligned16(g_prev) && (!gate || aligned16(gate)) && (!acc || aligned16(acc))))
         return GNNHIP_EUNSUPPORTED;

@@ -72,6 +72,9 @@ template <> struct VecT<4> { using type = float4; };
 template <int VEC> struct BufLoad;
 template <> struct BufLoad<4> { static __device__ __forceinline__ float4 get(rsrc_t r, int v, int s) { return buf_load4(r, v, s); } };
 template <> struct BufLoad<2> { static __device__ __forceinline__ float2 get(rsrc_t r, int v, int s) { return buf_load2(r, v, s); } };
+template <int VEC> struct BufStore;
+template <> struct BufStore<4> { static __device__ __forceinline__ void put(rsrc_t r, int v, int s, const float4& x) { buf_store4(r, v, s, x); } };
+template <> struct BufStore<2> { static __device__ __forceinline__ void put(rsrc_t r, int v, int s, const float2& x) { buf_store2(r, v, s, x); } };
 
 // A batch of kInFlight consecutive entries of a CSR array (column indices, or edge weights as bit
 // patterns) in scalar registers.  The two scalar loads are written as inline assembly with the batch as a
@@ -126,11 +129,17 @@ __device__ __forceinline__ void vec_fma(float (&acc)[VEC], float a, const typena
 // either wavefront of a SIMD takes time away from its matrix pipe.
 // RELU_IN: the gathered rows count as ReLU(row) (the first level reading msg where h0 was not stored)
 // TR: rows per pass (16, 32 or 64)
-template <int C, int WAVES, bool RELU_IN, int TR>
+// BWD: the backward pass of a level through the same machinery.  The CSR arrays are those of A^T, h_in is dz, the
+//      summed rows u = A^T dz are also stored to u_out as each one is finished (they are the other factor of the
+//      weight gradient), the contraction takes W transposed (g = u W^T), and the epilogue, instead of adding msg and
+//      applying ReLU, lets g through where the rows of `msg` (here: the embedding whose ReLU the gradient passes next,
+//      or null for no gate) are positive and adds what it stores to acc_io (or null).
+template <int C, int WAVES, bool RELU_IN, int TR, bool BWD = false>
 __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     int N, int tiles_per_block, const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
     const float* __restrict__ val, const float* __restrict__ h_in, const float* __restrict__ W,
-    const float* __restrict__ msg, const float* __restrict__ bias, float* __restrict__ h_out)
+    const float* __restrict__ msg, const float* __restrict__ bias, float* __restrict__ h_out,
+    float* __restrict__ u_out, float* __restrict__ acc_io)
 {
     constexpr int KS = C / 4;                    // contraction steps
     constexpr int kWideBlock = WAVES * kWave;
@@ -153,17 +162,17 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     if (bias)
         for (int i = threadIdx.x; i < C; i += kWideBlock) bias_lds[i] = bias[i];
 
-    // W^T operand: wreg[jb][s] = W[KS q + s][col0 + 16 jb + t]
+    // W^T operand: wreg[jb][s] = W[KS q + s][col0 + 16 jb + t]; BWD: W itself, wreg[jb][s] = W[col0 + 16 jb + t][KS q + s]
     // (buffer loads: one lane offset, the steps as scalar offsets, so no 64-bit address per element is formed)
     float wreg[NB][KS];
     {
         const rsrc_t w_rsrc = make_rsrc(W, (unsigned)(C * C * 4));
-        const int w_lane_off = ((KS * q) * C + col0 + t) * 4;
+        const int w_lane_off = BWD ? ((col0 + t) * C + KS * q) * 4 : ((KS * q) * C + col0 + t) * 4;
 #pragma unroll
         for (int jb = 0; jb < NB; ++jb)
 #pragma unroll
             for (int s = 0; s < KS; ++s)
-                wreg[jb][s] = buf_load_f(w_rsrc, w_lane_off + 64 * jb, s * (C * 4));
+                wreg[jb][s] = buf_load_f(w_rsrc, w_lane_off + (BWD ? 16 * C * 4 : 64) * jb, s * (BWD ? 4 : C * 4));
     }
 
     const int ntiles = (int)(((long long)N + kTileRows - 1) / kTileRows);
@@ -214,16 +223,24 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     int e = 0, ee = 0, lr = 0, row_end = 0, rpv = 0;
     float* dstp = nullptr;
     float acc[VEC];
-    auto begin = [&](int rp_lanes, int eb, int eend, float* dst) {
+    rsrc_t u_rsrc = make_rsrc(u_out, 0);         // BWD: the rows of u_out that the pass being gathered covers
+    auto begin = [&](int rp_lanes, int eb, int eend, float* dst, int tile_id) {
         rpv = rp_lanes;
         e = eb; ee = eend; lr = 0;
         row_end = __builtin_amdgcn_readlane(rpv, 1);
         dstp = dst;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+        if constexpr (BWD) {
+            const long long r0 = (long long)tile_id * kTileRows;
+            const long long rows = max(min((long long)N - r0, (long long)kTileRows), 0ll);      // none past the last pass
+            u_rsrc = make_rsrc(u_out + (size_t)min(r0, (long long)N) * C, (unsigned)(rows * (C * 4)));
+        }
     };
     auto flush_row = [&]() {
         *reinterpret_cast<vec_t*>(dstp) = *reinterpret_cast<vec_t*>(acc);
+        if constexpr (BWD)                        // rows past N lie outside the descriptor
+            BufStore<VEC>::put(u_rsrc, lane * (VEC * 4), (wave * RPW + lr) * (C * 4), *reinterpret_cast<vec_t*>(acc));
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
         dstp += LDT;
@@ -251,7 +268,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
 #pragma unroll
     for (int jb = 0; jb < NB; ++jb) outv[jb] = f4_zero();
     const int lane_off = (t * C + col0 + 4 * q) * 4;              // byte offset of this lane inside a 16-row block
-    rsrc_t msg_rsrc = make_rsrc(msg, 0), out_rsrc = make_rsrc(h_out, 0);
+    rsrc_t msg_rsrc = make_rsrc(msg, 0), out_rsrc = make_rsrc(h_out, 0), acc_rsrc = make_rsrc(acc_io, 0);
     auto store_pending = [&]() {
         if (out_rt >= 0) {
 #pragma unroll
@@ -269,7 +286,7 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     // ---- first pass: its gather has nothing to hide behind
     int rp_next = load_rowptrs(tile_begin);      // row pointers of the next pass to gather
     int ebN = __builtin_amdgcn_readlane(rp_next, 0), eeN = __builtin_amdgcn_readlane(rp_next, RPW);
-    begin(rp_next, ebN, eeN, tiles + gather_off);
+    begin(rp_next, ebN, eeN, tiles + gather_off, tile_begin);
     while (e < ee) {
         vec_t x[kInFlight];
         cShift = load_batch(col_idx, e, cC);
@@ -296,12 +313,13 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
         const float* cur = tiles + parity * (kTileRows * LDT);
         const bool has_next = tile_id + 1 < tile_end;
         const bool has_next2 = tile_id + 2 < tile_end;
-        begin(rp_next, ebN, eeN, tiles + (parity ^ 1) * (kTileRows * LDT) + gather_off);   // empty when !has_next
+        begin(rp_next, ebN, eeN, tiles + (parity ^ 1) * (kTileRows * LDT) + gather_off, tile_id + 1);   // empty when !has_next
         {
             const long long left = (long long)N - row0;
             const unsigned bytes = (unsigned)(min(left, (long long)kTileRows) * (C * 4));
             out_rsrc = make_rsrc(h_out + (size_t)row0 * C, bytes);
             msg_rsrc = make_rsrc(msg ? msg + (size_t)row0 * C : nullptr, msg ? bytes : 0u);   // no msg: every load reads 0
+            if constexpr (BWD) acc_rsrc = make_rsrc(acc_io ? acc_io + (size_t)row0 * C : nullptr, acc_io ? bytes : 0u);
         }
         if (has_next2) rp_next = load_rowptrs(tile_id + 2);
 
@@ -311,12 +329,18 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
         for (int rt = 0; rt < kTileRows / 16; ++rt) {
             // msg is asked for now and added after the contraction (as the accumulators' initial value it
             // would have to arrive before the first matrix instruction)
-            float4 mm[NB];
+            float4 mm[NB], aa[BWD ? NB : 1];
             mfma_f4 acc_m[NB];
 #pragma unroll
             for (int jb = 0; jb < NB; ++jb) {
                 mm[jb] = buf_load4(msg_rsrc, lane_off + rt * (16 * C * 4) + 64 * jb, 0);
                 acc_m[jb] = mfma_f4{0.f, 0.f, 0.f, 0.f};
+            }
+            if constexpr (BWD) {
+                if (acc_io) {
+#pragma unroll
+                    for (int jb = 0; jb < NB; ++jb) aa[jb] = buf_load4(acc_rsrc, lane_off + rt * (16 * C * 4) + 64 * jb, 0);
+                }
             }
             vec_t x[kInFlight];
             const bool batch = e < ee;
@@ -380,18 +404,34 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
                 }
             }
             GNNHIP_PHASE_ACC(3);
+            if constexpr (BWD) {
 #pragma unroll
-            for (int jb = 0; jb < NB; ++jb) {
-                acc_m[jb][0] += mm[jb].x; acc_m[jb][1] += mm[jb].y; acc_m[jb][2] += mm[jb].z; acc_m[jb][3] += mm[jb].w;
-            }
-#pragma unroll
-            for (int jb = 0; jb < NB; ++jb) {
-                float4 v = make_float4(acc_m[jb][0], acc_m[jb][1], acc_m[jb][2], acc_m[jb][3]);
-                if (bias) {
-                    const float4 b4 = *reinterpret_cast<const float4*>(bias_lds + col0 + 16 * jb + 4 * q);
-                    v.x += b4.x; v.y += b4.y; v.z += b4.z; v.w += b4.w;
+                for (int jb = 0; jb < NB; ++jb) {
+                    float4 v = make_float4(acc_m[jb][0], acc_m[jb][1], acc_m[jb][2], acc_m[jb][3]);
+                    if (msg) {                   // past the ReLU whose output these rows are
+                        v.x = mm[jb].x > 0.f ? v.x : 0.f; v.y = mm[jb].y > 0.f ? v.y : 0.f;
+                        v.z = mm[jb].z > 0.f ? v.z : 0.f; v.w = mm[jb].w > 0.f ? v.w : 0.f;
+                    }
+                    if (acc_io) {                // every row belongs to one pass: nobody else touches it during the launch
+                        const float4 a = make_float4(aa[jb].x + v.x, aa[jb].y + v.y, aa[jb].z + v.z, aa[jb].w + v.w);
+                        buf_store4(acc_rsrc, lane_off + rt * (16 * C * 4) + 64 * jb, 0, a);
+                    }
+                    outv[jb] = v;
                 }
-                outv[jb] = make_float4(relu_ref(v.x), relu_ref(v.y), relu_ref(v.z), relu_ref(v.w));
+            } else {
+#pragma unroll
+                for (int jb = 0; jb < NB; ++jb) {
+                    acc_m[jb][0] += mm[jb].x; acc_m[jb][1] += mm[jb].y; acc_m[jb][2] += mm[jb].z; acc_m[jb][3] += mm[jb].w;
+                }
+#pragma unroll
+                for (int jb = 0; jb < NB; ++jb) {
+                    float4 v = make_float4(acc_m[jb][0], acc_m[jb][1], acc_m[jb][2], acc_m[jb][3]);
+                    if (bias) {
+                        const float4 b4 = *reinterpret_cast<const float4*>(bias_lds + col0 + 16 * jb + 4 * q);
+                        v.x += b4.x; v.y += b4.y; v.z += b4.z; v.w += b4.w;
+                    }
+                    outv[jb] = make_float4(relu_ref(v.x), relu_ref(v.y), relu_ref(v.z), relu_ref(v.w));
+                }
             }
             out_rt = rt;
             GNNHIP_PHASE_ACC(4);
@@ -417,9 +457,10 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     GNNHIP_PHASE_FINI
 }
 
-template <int C, int WAVES, bool RELU_IN, int TR>
+template <int C, int WAVES, bool RELU_IN, int TR, bool BWD = false>
 int launch_level_wide_t(int N, const int* row_ptr, const int* col_idx, const float* val, const float* h_in,
-                      const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s)
+                      const float* W, const float* msg, const float* bias, float* h_out, hipStream_t s,
+                      float* u_out = nullptr, float* acc_io = nullptr)
 {
     if ((unsigned long long)N * C * 4ull >= (1ull << 32)) return GNNHIP_EUNSUPPORTED;   // 32-bit buffer offsets
     constexpr int kTileRows = TR;
@@ -431,10 +472,10 @@ int launch_level_wide_t(int N, const int* row_ptr, const int* col_idx, const flo
     const long long blocks = (ntiles + per - 1) / per;
     const size_t smem = sizeof(float) * (2 * kTileRows * (C + 4) + C);
     static LdsLimit lds_limit;                                       // one per kernel instantiation
-    GNNHIP_HIP(lds_limit.raise(reinterpret_cast<const void*>(&s2v_level_wide_kernel<C, WAVES, RELU_IN, TR>), smem));
-    hipLaunchKernelGGL((s2v_level_wide_kernel<C, WAVES, RELU_IN, TR>), dim3((unsigned)blocks), dim3(WAVES * kWave), smem, s,
-                       N, (int)per, row_ptr, col_idx, val, h_in, W, msg, bias, h_out);
-    GNNHIP_LAUNCH_CHECK("s2v_level_wide");
+    GNNHIP_HIP(lds_limit.raise(reinterpret_cast<const void*>(&s2v_level_wide_kernel<C, WAVES, RELU_IN, TR, BWD>), smem));
+    hipLaunchKernelGGL((s2v_level_wide_kernel<C, WAVES, RELU_IN, TR, BWD>), dim3((unsigned)blocks), dim3(WAVES * kWave), smem, s,
+                       N, (int)per, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, u_out, acc_io);
+    GNNHIP_LAUNCH_CHECK(BWD ? "s2v_level_wide backward" : "s2v_level_wide");
     return GNNHIP_OK;
 }
 
@@ -448,6 +489,17 @@ int launch_level_wide(int N, const int* row_ptr, const int* col_idx, const float
     if (N >= 2 * kSlots * 64) return launch_level_wide_t<C, WAVES, RELU_IN, 64>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
     if (N >= 2 * kSlots * 32) return launch_level_wide_t<C, WAVES, RELU_IN, 32>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
     return launch_level_wide_t<C, WAVES, RELU_IN, 16>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+}
+
+// The backward pass: same choice of rows per pass.
+template <int C, int WAVES>
+int launch_level_wide_backward(int N, const int* row_ptr, const int* col_idx, const float* val, const float* dz, const float* W,
+                               float* u, float* g_prev, const float* gate, float* acc, hipStream_t s)
+{
+    constexpr int kSlots = kNumCU * ((C == 128) ? 2 : 1);
+    if (N >= 2 * kSlots * 64) return launch_level_wide_t<C, WAVES, false, 64, true>(N, row_ptr, col_idx, val, dz, W, gate, nullptr, g_prev, s, u, acc);
+    if (N >= 2 * kSlots * 32) return launch_level_wide_t<C, WAVES, false, 32, true>(N, row_ptr, col_idx, val, dz, W, gate, nullptr, g_prev, s, u, acc);
+    return launch_level_wide_t<C, WAVES, false, 16, true>(N, row_ptr, col_idx, val, dz, W, gate, nullptr, g_prev, s, u, acc);
 }
 
 }  // namespace
@@ -470,6 +522,18 @@ int level_wide_dispatch(int N, int C, long long nnz, const int* row_ptr, const i
     case 256:
         return relu_in ? launch_level_wide<256, 8, true>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s)
                        : launch_level_wide<256, 8, false>(N, row_ptr, col_idx, val, h_in, W, msg, bias, h_out, s);
+    }
+    return GNNHIP_EUNSUPPORTED;
+}
+
+// u = A' dz (stored) and g_prev = u W^T past the gate of `gate` (may be null), added to acc (may be null): the wide
+// kernel's backward variant over the CSR arrays of A' = A^T.
+int level_wide_backward_dispatch(int N, int C, const int* row_ptr, const int* col_idx, const float* val, const float* dz, const float* W,
+                                 float* u, float* g_prev, const float* gate, float* acc, hipStream_t s)
+{
+    switch (C) {
+    case 128: return launch_level_wide_backward<128, 8>(N, row_ptr, col_idx, val, dz, W, u, g_prev, gate, acc, s);
+    case 256: return launch_level_wide_backward<256, 8>(N, row_ptr, col_idx, val, dz, W, u, g_prev, gate, acc, s);
     }
     return GNNHIP_EUNSUPPORTED;
 }

@@ -212,6 +212,29 @@ def test_gemm_all_transposes(gpu, oracle, shape):
             assert_parity("gemm %d%d" % (ta, tb), got2, *_gemm_want(oracle, A, B, ta, tb, alpha=1.5, beta=-0.5, C=C0))
 
 
+@pytest.mark.parametrize("k,c", [(8192, 128), (20_003, 128), (8191, 256), (8192, 256), (40_001, 256), (300_007, 256)])
+def test_gemm_wide_weight_gradient_over_a_long_k(gpu, oracle, k, c):
+    """h^T u with a 128 x 128 or 256 x 256 output and k in the thousands to hundreds of thousands (the level weight gradient
+    at hidden 128 / 256): from k = 8,192 the whole output lives in one workgroup's registers, each workgroup a range of k
+    (ranges that end inside a step of 16 rows, one row short of the threshold, a last range shorter than the others);
+    alone and inside a batch: same bits"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(k + c)
+    A = (rng.standard_normal((k, c)) * (rng.random((k, c)) < 0.6)).astype(np.float32)      # embeddings past a ReLU: many zeros
+    B = rng.standard_normal((k, c)).astype(np.float32)
+    C0 = rng.standard_normal((c, c)).astype(np.float32)
+    got = _n(ops.gemm(_t(A, gpu), _t(B, gpu), True, False))
+    assert_parity("gemm 10", got, *_gemm_want(oracle, A, B, True, False))
+    assert np.array_equal(got, _n(ops.gemm(_t(A, gpu), _t(B, gpu), True, False)))           # fixed order of the ranges
+    got2 = _n(ops.gemm(_t(A, gpu), _t(B, gpu), True, False, alpha=0.5, beta=1.0, out=_t(C0, gpu)))
+    assert_parity("gemm 10", got2, *_gemm_want(oracle, A, B, True, False, alpha=0.5, beta=1.0, C=C0))
+    small = lambda: (_t(A[:300, :64].copy(), gpu), _t(B[:300, :32].copy(), gpu), _t(C0[:64, :32].copy(), gpu))
+    outs = ops.gemm_tn_batch([small(), (_t(A, gpu), _t(B, gpu), _t(C0, gpu)), small()], alpha=0.5, beta=1.0)
+    assert np.array_equal(_n(outs[1]), got2)
+    assert np.array_equal(_n(outs[0]), _n(outs[2]))
+    assert_parity("gemm batch", _n(outs[0]), *_gemm_want(oracle, A[:300, :64], B[:300, :32], True, False, alpha=0.5, beta=1.0, C=C0[:64, :32]))
+
+
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (-0.75, 0.5)])
 def test_gemm_batch_of_weight_gradient_products(gpu, oracle, alpha, beta):
     """the four x^T dy products at the end of a configuration-2 backward pass, a product too short to split, one that

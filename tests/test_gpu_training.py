@@ -87,11 +87,11 @@ def test_readout_backward(gpu, oracle, C, H, Q, B):
     assert_parity("g_h", _n(gh), w_gh, gh64)
 
 
-@pytest.mark.parametrize("C", [16, 32, 64, 128])
-@pytest.mark.parametrize("N", [77, 7450, 40_000])
+@pytest.mark.parametrize("N,C", [(N, C) for C in (16, 32, 64, 128, 256) for N in (77, 7450, 40_000)] + [(70_001, 128), (70_001, 256), (16_400, 256)])
 def test_level_backward(gpu, oracle, C, N):
-    """u = A^T dz and g_prev = u W^T in one pass (hidden 16/32/64; hidden 128 takes SpMM + GEMM inside the entry):
-    ragged rows, two long rows (the larger matrix sends them through the balanced pass), signed dz"""
+    """u = A^T dz and g_prev = u W^T in one pass (hidden 16/32/64: the streaming kernel; hidden 128/256: the wide kernel's
+    backward variant in passes of 16, 32 and 64 rows, which the row counts select): ragged rows, two long rows (the larger
+    matrices send them through the balanced pass at the narrow sizes), signed dz"""
     from graphnn_amd import ops
     rng = np.random.default_rng(C + N)
     lens = rng.integers(0, 7, N); lens[N // 3] = min(N, 3000); lens[N - 1] = 70
