@@ -179,6 +179,29 @@ def time_gather_ceiling(dev, m=1_000_000, per=10, d=128):
             "bytes": nbytes, "median_ms": t["median_ms"], "GBps": nbytes / (t["median_ms"] * 1e-3) / 1e9}
 
 
+def time_cached_gather_ceiling(dev, m=1_000_000, per=10, d=128, k=393_216):
+    """The same kernel and shape again with uniform random columns over a dense operand of 201 MB: twenty-five times the
+    eight L2s together, but inside the 256 MB memory-side cache, so nearly every gather misses its L2 and is served
+    without an HBM read.  What this measures is the rate of the path between the L2s and the fabric for 512-byte gathers,
+    which is the bound of configuration 3 itself once its operand sits behind that path."""
+    import torch
+    from graphnn_amd import ops
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    cols, _ = torch.sort(torch.randint(0, k, (m, per), device=dev, dtype=torch.int32, generator=g), dim=1)
+    ci = cols.reshape(-1).contiguous()
+    rp = (torch.arange(m + 1, device=dev, dtype=torch.int64) * per).int()
+    v = torch.ones(m * per, device=dev, dtype=torch.float32)
+    X = torch.ones((k, d), device=dev, dtype=torch.float32)
+    Y = torch.empty((m, d), device=dev, dtype=torch.float32)
+    t = _event_median_ms(lambda: ops.spmm(rp, ci, v, X, m, out=Y), 20, 3)
+    assert float(Y[12345, 7]) == float(per), "cached-gather product is wrong"
+    nbytes = 4 * (m + 1) + 8 * m * per + 4 * m * per * d + 4 * m * d
+    return {"kernel": "spmm_rowgroup_kernel<4,1>", "workload": "%d rows x %d entries, uniform random over %d columns (operand %.0f MB), width %d"
+                                                               % (m, per, k, k * d * 4 / 1e6, d),
+            "bytes_gathered_and_written": nbytes, "median_ms": t["median_ms"], "GBps": nbytes / (t["median_ms"] * 1e-3) / 1e9}
+
+
 def time_spmm_cfg3(dev, reps=50, warmup=5, regular=False):
     """HIP-event time of the SpMM kernel alone on configuration 3 (SplitMix64 streams of the configuration; the dense
     operand by the torch twin of the normal stream, on the device).  regular: exactly 10 entries in every row."""
@@ -732,6 +755,7 @@ def main():
         if "ceilings" in legs:
             res["read_ceiling"] = time_read_ceiling(dev)
             res["gather_ceiling"] = time_gather_ceiling(dev)
+            res["cached_gather_ceiling"] = time_cached_gather_ceiling(dev)
             res["stream_copy"] = time_stream_copy(dev)
         if "cfg4" in legs:
             res["cfg4_level"] = time_level_cfg4(dev)
@@ -828,6 +852,7 @@ def main():
         achieved = bytes_alg / (med_ms * 1e-3) / 1e9
         traffic = MEASURED_TRAFFIC_BYTES["spmm_cfg3"]
         read_c, gather_c, copy_c = time_read_ceiling(dev), time_gather_ceiling(dev), time_stream_copy(dev)
+        cached_c = time_cached_gather_ceiling(dev)
         out["roofline"] = {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
@@ -846,6 +871,10 @@ def main():
             # what this GPU's HBM delivers, measured in this run: a read-only kernel over 2 GiB, a copy of 1 GiB, and this
             # same SpMM kernel on a matrix whose 10M columns never repeat (5.12 GB operand: every gathered byte from HBM)
             "read_ceiling": read_c, "stream_copy": copy_c, "gather_ceiling": gather_c,
+            # and what the path between L2 and fabric delivers to the same kernel when HBM is out of the picture (operand
+            # inside the memory-side cache): configuration 3's counted traffic runs at this rate
+            "cached_gather_ceiling": cached_c,
+            "l2_miss_traffic_vs_cached_gather_ceiling": (traffic / (med_ms * 1e-3) / 1e9) / cached_c["GBps"],
             # north-star target ">= 60 % of HBM peak": stated separately for the fabric side (counted L2 misses, which the
             # memory-side cache partly serves: the 512 MB operand is twice its size and every row is gathered ten times)
             # and for bytes that provably come from HBM (the no-reuse gather above)

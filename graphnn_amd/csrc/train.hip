@@ -12,6 +12,10 @@
 #include "gnnhip_internal.h"
 
 namespace gnnhip {
+// gemm.hip
+int gemm_dispatch(int transA, int transB, int m, int n, int k, float alpha, const float* A, int lda,
+                  const float* B, int ldb, float beta, float* C, int ldc, hipStream_t s);
+
 namespace {
 
 constexpr int kBlock = 256;
@@ -99,7 +103,7 @@ __global__ __launch_bounds__(kBlock) void readout_backward_kernel(
     int B, int C, int H, int Q, const int* __restrict__ s_row_ptr, const int* __restrict__ s_col_idx, const float* __restrict__ s_val,
     const float* __restrict__ probs, const int* __restrict__ lrow_ptr, const int* __restrict__ lcol, const float* __restrict__ lval,
     float scale, const float* __restrict__ hidden, const float* __restrict__ Wh1, const float* __restrict__ Wh2,
-    float* __restrict__ dlogits, float* __restrict__ du, float* __restrict__ g_h)
+    float* __restrict__ dlogits, float* __restrict__ du, float* __restrict__ g_h, int head_only)
 {
     extern __shared__ float smem[];
     float* dl = smem;
@@ -126,6 +130,7 @@ __global__ __launch_bounds__(kBlock) void readout_backward_kernel(
             du[(size_t)g * H + j] = v;
         }
         __syncthreads();
+        if (head_only) continue;                // large batches: dpool for all graphs as one product, rows by the kernel below
         // dpool = du W_h1^T
         for (int c = tid; c < C; c += kBlock) {
             float s = 0.f;
@@ -141,6 +146,38 @@ __global__ __launch_bounds__(kBlock) void readout_backward_kernel(
             g_h[(size_t)s_col_idx[a + r] * C + c] = s_val[a + r] * dp[c];
         }
         __syncthreads();
+    }
+}
+
+// Large batches: g_h[node] = s_val * dpool[graph of node], one workgroup per graph, a wavefront per node row (the
+// graph's dpool row is read once per wavefront and stays in registers while its node rows are written).
+__global__ __launch_bounds__(kBlock) void readout_backward_rows_kernel(int B, int C, const int* __restrict__ s_row_ptr,
+                                                                       const int* __restrict__ s_col_idx, const float* __restrict__ s_val,
+                                                                       const float* __restrict__ dpool, float* __restrict__ g_h)
+{
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    constexpr int kWaves = kBlock / kWave;
+    for (int g = blockIdx.x; g < B; g += gridDim.x) {
+        const int a = s_row_ptr[g], e = s_row_ptr[g + 1];
+        const float* dp = dpool + (size_t)g * C;
+        if ((C & 3) == 0 && C <= 4 * kWave * 2) {
+            // up to 512 columns: two 128-bit pieces per lane
+            const int c0 = 4 * lane, c1 = 4 * (lane + kWave);
+            const float4 p0 = c0 < C ? *reinterpret_cast<const float4*>(dp + c0) : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 p1 = c1 < C ? *reinterpret_cast<const float4*>(dp + c1) : make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int r = a + wave; r < e; r += kWaves) {
+                const float w = s_val[r];
+                float* dst = g_h + (size_t)s_col_idx[r] * C;
+                if (c0 < C) *reinterpret_cast<float4*>(dst + c0) = make_float4(w * p0.x, w * p0.y, w * p0.z, w * p0.w);
+                if (c1 < C) *reinterpret_cast<float4*>(dst + c1) = make_float4(w * p1.x, w * p1.y, w * p1.z, w * p1.w);
+            }
+        } else {
+            for (int r = a + wave; r < e; r += kWaves) {
+                const float w = s_val[r];
+                float* dst = g_h + (size_t)s_col_idx[r] * C;
+                for (int c = lane; c < C; c += kWave) dst[c] = w * dp[c];
+            }
+        }
     }
 }
 
@@ -315,9 +352,22 @@ int gnnhip_s2v_readout_backward_f32(int B, int N, int C, int H, int Q,
         return set_error(GNNHIP_EUNSUPPORTED, "readout backward keeps Q + H + C = %d floats per graph in LDS; too many", Q + H + C);
     long long blocks = B;
     if (blocks > (long long)kNumCU * 16) blocks = (long long)kNumCU * 16;
-    hipLaunchKernelGGL(readout_backward_kernel, dim3((unsigned)blocks), dim3(kBlock), smem, as_stream(stream), B, C, H, Q,
-                       s_row_ptr, s_col_idx, s_val, probs, lrow_ptr, lcol, lval, scale, hidden, W_h1, W_h2, dlogits, du, g_h);
+    hipStream_t s = as_stream(stream);
+    // From 1,024 graphs on the per-graph product du W_h1^T (every lane walking its own row of W_h1) becomes one GEMM
+    // over all graphs, and the node rows are written by a kernel of their own; below, one launch does everything.
+    const bool split = B >= 1024 && aligned16(g_h);
+    void* dpool = nullptr;
+    if (split)
+        if (int rc = stream_scratch(s, sizeof(float) * (size_t)B * C, &dpool)) return rc;
+    hipLaunchKernelGGL(readout_backward_kernel, dim3((unsigned)blocks), dim3(kBlock), smem, s, B, C, H, Q,
+                       s_row_ptr, s_col_idx, s_val, probs, lrow_ptr, lcol, lval, scale, hidden, W_h1, W_h2, dlogits, du, g_h, split ? 1 : 0);
     GNNHIP_LAUNCH_CHECK("readout_backward");
+    if (split) {
+        if (int rc = gemm_dispatch(0, 1, B, C, H, 1.f, du, H, W_h1, H, 0.f, static_cast<float*>(dpool), C, s)) return rc;
+        hipLaunchKernelGGL(readout_backward_rows_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, B, C, s_row_ptr, s_col_idx, s_val,
+                           static_cast<const float*>(dpool), g_h);
+        GNNHIP_LAUNCH_CHECK("readout_backward rows");
+    }
     return GNNHIP_OK;
 }
 

@@ -58,7 +58,9 @@ def test_loss_tail_with_weighted_and_empty_label_rows(gpu, oracle):
     assert np.array_equal(_n(hit), oracle.in_top_k(logits, oracle.csr_row_argmax(*lab), 1))
 
 
-@pytest.mark.parametrize("C,H,Q,B", [(64, 32, 2, 256), (16, 8, 3, 5), (256, 128, 2, 700), (48, 100, 70, 33)])
+@pytest.mark.parametrize("C,H,Q,B", [(64, 32, 2, 256), (16, 8, 3, 5), (256, 128, 2, 700), (48, 100, 70, 33),
+                                     # from 1,024 graphs: du W_h1^T as one product over all graphs, node rows by a kernel of their own
+                                     (256, 128, 2, 1024), (64, 32, 2, 3000), (130, 20, 3, 1100), (600, 16, 2, 1030)])
 def test_readout_backward(gpu, oracle, C, H, Q, B):
     from graphnn_amd import ops
     rng = np.random.default_rng(C + H + B)
