@@ -203,6 +203,8 @@ struct HubStore {
 // threshold / chunk_len: rows with more entries than `threshold` are summed, cut into chunks of `chunk_len`
 // (the consumer must apply the same threshold when it looks a row up in row_slot); max_hubs >= 0: the caller's
 // bound on the number of such rows; store: where the pass keeps its arrays (null: the stream's scratch slot 1)
+// reuse_plan: the caller states that the previous call on this stream had the very same matrix: same arrays, same structure
+// AND same values (the column-ordered pieces keep a copy of the values), nothing rewritten in between.
 int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_idx, const float* val,
                 const float* B, int ldb, hipStream_t s, HubPlan* plan, bool reuse_plan = false, bool relu_in = false,
                 int threshold = kHubThreshold, int chunk_len = kHubChunk, long long max_hubs = -1, HubStore* store = nullptr);

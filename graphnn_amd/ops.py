@@ -134,11 +134,16 @@ def release_scratch():
     check(_lib().gnnhip_release_scratch(_stream()))
 
 
-def gemm(A, B, transA=False, transB=False, alpha=1.0, beta=0.0, out=None):
-    m = A.shape[1] if transA else A.shape[0]
-    k = A.shape[0] if transA else A.shape[1]
-    kb = B.shape[1] if transB else B.shape[0]
-    n = B.shape[0] if transB else B.shape[1]
+def gemm(A, B, transA=False, transB=False, alpha=1.0, beta=0.0, out=None, cols_a=None, cols_b=None):
+    """cols_a / cols_b: use only the first so many columns of the stored A / B (the row stride stays the tensor's)"""
+    ca = A.shape[1] if cols_a is None else int(cols_a)
+    cb = B.shape[1] if cols_b is None else int(cols_b)
+    if not (0 <= ca <= A.shape[1] and 0 <= cb <= B.shape[1]):
+        raise ValueError("cols_a / cols_b out of range")
+    m = ca if transA else A.shape[0]
+    k = A.shape[0] if transA else ca
+    kb = cb if transB else B.shape[0]
+    n = B.shape[0] if transB else cb
     if k != kb:
         raise ValueError("mat dim doesn't match")
     if out is None:

@@ -228,6 +228,11 @@ def test_gemm_wide_weight_gradient_over_a_long_k(gpu, oracle, k, c):
     assert np.array_equal(got, _n(ops.gemm(_t(A, gpu), _t(B, gpu), True, False)))           # fixed order of the ranges
     got2 = _n(ops.gemm(_t(A, gpu), _t(B, gpu), True, False, alpha=0.5, beta=1.0, out=_t(C0, gpu)))
     assert_parity("gemm 10", got2, *_gemm_want(oracle, A, B, True, False, alpha=0.5, beta=1.0, C=C0))
+    if k == 20_003 or k == 40_001:
+        # the operands as the leading columns of wider matrices (row strides of c + 64 and c + 4 floats)
+        Aw = np.concatenate([A, rng.standard_normal((k, 64)).astype(np.float32)], axis=1)
+        Bw = np.concatenate([B, rng.standard_normal((k, 4)).astype(np.float32)], axis=1)
+        assert np.array_equal(_n(ops.gemm(_t(Aw, gpu), _t(Bw, gpu), True, False, cols_a=c, cols_b=c)), got)
     small = lambda: (_t(A[:300, :64].copy(), gpu), _t(B[:300, :32].copy(), gpu), _t(C0[:64, :32].copy(), gpu))
     outs = ops.gemm_tn_batch([small(), (_t(A, gpu), _t(B, gpu), _t(C0, gpu)), small()], alpha=0.5, beta=1.0)
     assert np.array_equal(_n(outs[1]), got2)
