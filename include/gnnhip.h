@@ -181,7 +181,9 @@ int gnnhip_gemm_f32(int transA, int transB, int m, int n, int k, float alpha, co
  *      (src/nn/matmul.cpp:35-76, x^T * dy through DTensor<GPU>::MM, src/tensor/gpu_dense_tensor.cu:192-224).
  *      m, n, k, lda, ldb, ldc and the pointer tables A, B, C are HOST arrays of count entries; the matrices are
  *      device memory.  Every product gives the bits gnnhip_gemm_f32(1, 0, ...) gives for it alone when that
- *      call splits k (few output tiles, k >= 256). */
+ *      call splits k (few output tiles, k >= 256).  A product with a 128 x 128 or 256 x 256 output and k >= 8192 (the
+ *      level weight gradient at hidden 128 / 256) is taken out of the batch and gets the two launches of its own that
+ *      the single call gives it (the whole output in one workgroup's registers over a range of k). */
 int gnnhip_gemm_tn_batch_f32(int count, const int* m, const int* n, const int* k, const float* const* A, const int* lda,
                              const float* const* B, const int* ldb, float alpha, float beta, float* const* C, const int* ldc,
                              void* stream);
@@ -444,7 +446,9 @@ int gnnhip_s2v_grad_gate_f32(size_t n, const float* h, const float* g, float* dz
  *      gate_h (may be NULL): the embedding h_prev [N,C] whose ReLU the gradient passes next; g_prev is then stored
  *      past that gate (g_prev where h_prev > 0, else 0: ReLUDeriv, src/nn/relu.cu:18-37), ready to be the dz of the
  *      level below.  acc (may be NULL): acc += g_prev as stored (the gradient ElewiseAdd::Backward hands to msg,
- *      src/nn/elewise_add.cpp:35-52, summed over the levels). */
+ *      src/nn/elewise_add.cpp:35-52, summed over the levels).
+ *      One launch at C = 16, 32, 64 and at C = 128, 256 (N * C * 4 < 4 GiB); other widths, and matrices of 32,768 rows
+ *      and more with 12 entries per row and more, run SpMM, GEMM and gate one after the other. */
 int gnnhip_s2v_level_backward_f32(int N, int C, int nnz, const int* t_row_ptr, const int* t_col_idx, const float* t_val,
                                   const float* dz, const float* W, float* u, float* g_prev, const float* gate_h, float* acc,
                                   void* stream);
