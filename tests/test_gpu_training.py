@@ -127,6 +127,34 @@ def test_level_backward(gpu, oracle, C, N):
     assert np.array_equal(_n(g3), _n(g)) and np.array_equal(_n(acc), acc0 + _n(g))
 
 
+@pytest.mark.parametrize("C", [128, 256])
+@pytest.mark.parametrize("nnz", [0, 3, 6])
+def test_level_backward_wide_with_hardly_any_entries(gpu, oracle, C, nnz):
+    """the wide kernel's backward variant on a transposed adjacency with fewer entries than one index batch (and none)"""
+    from graphnn_amd import ops
+    rng = np.random.default_rng(C + nnz)
+    N = 40
+    rows = np.sort(rng.integers(0, N, nnz))
+    rp = np.zeros(N + 1, np.int32); np.cumsum(np.bincount(rows, minlength=N), out=rp[1:])
+    ci = rng.integers(0, N, nnz).astype(np.int32)
+    v = (0.5 + rng.random(nnz)).astype(np.float32)
+    dz = rng.standard_normal((N, C)).astype(np.float32)
+    W = (rng.standard_normal((C, C)) * 0.1).astype(np.float32)
+    h_prev = rng.standard_normal((N, C)).astype(np.float32)
+    acc0 = rng.standard_normal((N, C)).astype(np.float32)
+    acc = _t(acc0, gpu)
+    pad = lambda a, dt: _t(np.concatenate([a, np.zeros(1, dt)]), gpu)[:a.size]      # never a null pointer for an empty array
+    u, g = ops.s2v_level_backward(_t(rp, gpu), pad(ci, np.int32), pad(v, np.float32), _t(dz, gpu), _t(W, gpu), gate_h=_t(h_prev, gpu), acc=acc)
+    import scipy.sparse as sp
+    u64 = sp.csr_matrix((v.astype(np.float64), ci, rp), shape=(N, N)) @ dz.astype(np.float64)
+    g64 = (u64 @ W.astype(np.float64).T) * (h_prev > 0)
+    w_u = oracle.spmm(rp, ci, v, dz, N)
+    w_g = (oracle.gemm(w_u, W, transB=True) * (h_prev > 0)).astype(np.float32)
+    assert_parity("u", _n(u), w_u, u64)
+    assert_parity("g_prev", _n(g), w_g, g64)
+    assert np.array_equal(_n(acc), acc0 + _n(g))
+
+
 def test_grad_gate_is_exact(gpu):
     import torch
     from graphnn_amd import ops
