@@ -125,9 +125,10 @@ def _sizes_skewed(stream, B):
     return 10 + np.minimum(100, np.floor(-20.0 * np.log1p(-u))).astype(np.int64)
 
 
-def molecule_batch(seed, B, K, Q=2, size_mode="uniform", size_lo=10, size_hi=28):
+def molecule_batch(seed, B, K, Q=2, size_mode="uniform", size_lo=10, size_hi=28, edge_factor=1.1):
     """B random molecule-like graphs: spanning tree parent(v) ~ U{0..v-1}, plus
-    round(1.1 n) - (n - 1) distinct extra non-tree, non-self pairs; every undirected
+    round(edge_factor n) - (n - 1) distinct extra non-tree, non-self pairs (1.1 n undirected
+    edges: mean degree 2.2, what the molecule datasets have); every undirected
     edge is stored in both directions and adjacency lists are ascending, which is
     the order the dataset files (and therefore GetBatch) present them in."""
     root = Stream(seed)
@@ -152,7 +153,7 @@ def molecule_batch(seed, B, K, Q=2, size_mode="uniform", size_lo=10, size_hi=28)
     tree_b = (g_off + local)[child_mask]
 
     # extra edges by rejection, graph by graph (few per graph)
-    n_extra = np.maximum(0, np.rint(1.1 * sizes).astype(np.int64) - (sizes - 1))
+    n_extra = np.maximum(0, np.rint(edge_factor * sizes).astype(np.int64) - (sizes - 1))
     extra_a, extra_b = [], []
     tree_parent_local = parent
     for g in range(B):
@@ -357,9 +358,11 @@ CONFIGS = {
 }
 
 
-def make_config(config_id, B=None, size_mode=None):
+def make_config(config_id, B=None, size_mode=None, edge_factor=None):
     """(batch, weights, dims) for the molecule-style configurations 1, 2 and 4.  size_mode="uniform" on configuration 2
-    takes its "nodes per graph ~ U[10,110]" literally (mean 60) instead of the right-skewed sizes with mean ~30."""
+    takes its "nodes per graph ~ U[10,110]" literally (mean 60) instead of the right-skewed sizes with mean ~30.
+    edge_factor: undirected edges per node (default 1.1, mean degree 2.2; 2.2 reads configuration 4's "~660k undirected
+    edges" on ~300k nodes literally)."""
     cfg = dict(CONFIGS[config_id])
     if B is not None:
         cfg["B"] = B
@@ -369,6 +372,8 @@ def make_config(config_id, B=None, size_mode=None):
             cfg["size_lo"], cfg["size_hi"] = 10, 110
     seed = config_seed(config_id)
     kw = {k: cfg[k] for k in ("size_lo", "size_hi") if k in cfg}
+    if edge_factor is not None:
+        kw["edge_factor"] = edge_factor
     batch = molecule_batch(seed, cfg["B"], cfg["K"], cfg["Q"], size_mode=cfg["size_mode"], **kw)
     weights = make_weights(Stream(seed), cfg["K"], cfg["C"], cfg["H"], cfg["Q"])
     return batch, weights, cfg
