@@ -231,8 +231,6 @@ struct CsrPlan {
     int* pfirst = nullptr;        // [m + 1] pieces of rows of several pieces before row r: row pointers of P
     int* at = nullptr;            // [slots + 1] entries before the i-th piece in order
     int* target = nullptr;        // [slots] row r >= 0 that the piece is all of, else -1 - (its place among the partial sums)
-    int* where = nullptr;         // [pslots] column indices of P (the identity)
-    float* ones = nullptr;        // [pslots] values of P
     int* col_ord = nullptr;       // [nnz] entries in piece order
     float* val_ord = nullptr;
     void* head_block = nullptr;   // first, pfirst

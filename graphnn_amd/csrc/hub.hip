@@ -14,13 +14,15 @@
 //           counts before its own)
 //   fill    row_slot[row] (written for hubs only), per hub its first chunk, per chunk its hub
 //   partial one wavefront per chunk: sum of val * B[col, :] over the chunk; a hub of one chunk is
-//           finished with that, for a longer one the wavefront that delivers the last chunk adds the
-//           chunks' sums in chunk order: agg[slot][n]
+//           finished with that: agg[slot][n]
+//   finish  a hub of several chunks: its chunks' sums added in chunk order by a lane group, in a launch
+//           of its own.  (One launch, with the wavefront that delivers a hub's last chunk adding the
+//           sums, was the first version: the release / acquire fences it needs between wavefronts on
+//           different dies write the L2 back, and 4,600 of them made up most of a 0.14 ms launch.)
 //
 // The consumer reads agg[row_slot[row]] for a row whose length exceeds the
 // threshold.  Every sum is taken in an order fixed by the matrix structure, so the
-// result does not depend on scheduling: no value is accumulated with atomics.  The one
-// atomic counter per hub (hub_done) only elects the wavefront that adds the chunks' sums.
+// result does not depend on scheduling: no atomics, no communication inside a launch.
 #include "gnnhip_internal.h"
 
 #include <map>
@@ -175,7 +177,8 @@ __global__ __launch_bounds__(kBlock) void hub_fill_kernel(int m, int nb, const i
             if (fits) {
                 hub_row[slot] = (int)(r0 + i);
                 hub_chunk0[slot] = chunk;
-                hub_done[slot] = 0;
+            } else if (slot < hub_cap) {
+                hub_row[slot] = -1;                  // the finishing pass skips it
             }
             for (int j = 0; j < nc && chunk + j < chunk_cap; ++j) chunk_hub[chunk + j] = fits ? slot : -1;
             ++slot;
@@ -212,7 +215,7 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
     const int* __restrict__ counts, int chunk_cap, int n, const int* __restrict__ row_ptr, const int* __restrict__ col_idx,
     const float* __restrict__ val, const float* __restrict__ B, int ldb, int logG,
     const int* __restrict__ hub_row, const int* __restrict__ hub_chunk0, const int* __restrict__ chunk_hub,
-    float* part, int ldp, float* __restrict__ agg, int* hub_done, int relu_in, int chunk_len)
+    float* __restrict__ part, int ldp, float* __restrict__ agg, int relu_in, int chunk_len)
 {
     // relu_in: the rows of B are used as ReLU(B) (a first level that reads msg in place of h0)
     using V = HV<VEC>;
@@ -232,31 +235,32 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
         typename V::T acc[ITERS];
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) acc[it] = V::zero();
-        int t = cb + grp;
-        for (; t + 7 * ngroups < ce; t += 8 * ngroups) {
+        // eight entries of the group at a time, the last ones of the chunk under a predicate (a serial tail would
+        // walk up to seven dependent index -> row loads one after the other, and most chunks of the matrices that
+        // pick partial sums are shorter than one such block); the order of the additions is the entries' order
+        for (int t = cb + grp; t < ce; t += 8 * ngroups) {
             int c8[8];
             float v8[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) { c8[u] = col_idx[t + u * ngroups]; v8[u] = val[t + u * ngroups]; }
+            for (int u = 0; u < 8; ++u) {
+                const bool ok = t + u * ngroups < ce;
+                // no index array: entry t of the row is column t with weight 1 (a matrix that picks consecutive rows of B,
+                // whose row loads then wait for no index load)
+                c8[u] = !ok ? 0 : col_idx ? col_idx[t + u * ngroups] : t + u * ngroups;
+                v8[u] = !ok ? 0.f : val ? val[t + u * ngroups] : 1.f;
+            }
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
                 const int col0 = (sub + it * G) * VEC;
                 if (col0 < n) {
                     typename V::T x[8];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) x[u] = V::load(B + (size_t)c8[u] * ldb + col0, relu_in);
+                    for (int u = 0; u < 8; ++u)
+                        x[u] = (t + u * ngroups < ce) ? V::load(B + (size_t)c8[u] * ldb + col0, relu_in) : V::zero();
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) V::fma(acc[it], v8[u], x[u]);
+                    for (int u = 0; u < 8; ++u)
+                        if (t + u * ngroups < ce) V::fma(acc[it], v8[u], x[u]);
                 }
-            }
-        }
-        for (; t < ce; t += ngroups) {
-            const int c0 = col_idx[t];
-            const float v0 = val[t];
-#pragma unroll
-            for (int it = 0; it < ITERS; ++it) {
-                const int col0 = (sub + it * G) * VEC;
-                if (col0 < n) V::fma(acc[it], v0, V::load(B + (size_t)c0 * ldb + col0, relu_in));
             }
         }
 #pragma unroll
@@ -274,38 +278,40 @@ __global__ __launch_bounds__(kBlock) void hub_partial_kernel(
                 }
             }
         }
-        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-        if (nc > 1) {
-            // The wavefront that delivers the last chunk of the hub adds the chunks' sums, always in chunk
-            // order.  Release: this chunk's sum is visible before the count; acquire: the other sums are
-            // read from L2 after the count said they are there.
-            __threadfence();
-            int last = 0;
-            if (lane == 0) last = (atomicAdd(hub_done + slot, 1) == nc - 1);
-            last = __shfl(last, 0, kWave);
-            if (last) {
-                __threadfence();
-                const int c0 = hub_chunk0[slot];
-                if (grp == 0) {
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");       // red[wave] is rewritten by the next chunk
+    }
+}
+
+// agg[slot] = sum of the chunks' sums, in chunk order, for every hub of several chunks; one lane group per hub.
+template <int VEC, int ITERS>
+__global__ __launch_bounds__(kBlock) void hub_finish_kernel(
+    const int* __restrict__ counts, int hub_cap, int n, const int* __restrict__ row_ptr, int logG,
+    const int* __restrict__ hub_row, const int* __restrict__ hub_chunk0, const float* __restrict__ part, int ldp,
+    float* __restrict__ agg, int chunk_len)
+{
+    using V = HV<VEC>;
+    const int G = 1 << logG, sub = threadIdx.x & (G - 1), grp = threadIdx.x >> logG, ngroups = kBlock >> logG;
+    const int nhubs = min(counts[0], hub_cap);
+    for (int slot = blockIdx.x * ngroups + grp; slot < nhubs; slot += gridDim.x * ngroups) {
+        const int row = hub_row[slot];
+        if (row < 0) continue;                   // did not fit the buffers: its consumer sums it in place
+        const int nc = hub_chunks(row_ptr[row + 1] - row_ptr[row], chunk_len);
+        if (nc <= 1) continue;
+        const int c0 = hub_chunk0[slot];
 #pragma unroll
-                    for (int it = 0; it < ITERS; ++it) {
-                        const int col0 = (sub + it * G) * VEC;
-                        if (col0 < n) {
-                            float sum[VEC];
+        for (int it = 0; it < ITERS; ++it) {
+            const int col0 = (sub + it * G) * VEC;
+            if (col0 >= n) continue;
+            typename V::T sum = V::zero();
+            for (int j0 = 0; j0 < nc; j0 += 8) {
+                typename V::T p[8];
 #pragma unroll
-                            for (int e = 0; e < VEC; ++e) sum[e] = 0.f;
-                            for (int j = 0; j < nc; ++j)
+                for (int u = 0; u < 8; ++u) p[u] = (j0 + u < nc) ? V::load(part + (size_t)(c0 + j0 + u) * ldp + col0) : V::zero();
 #pragma unroll
-                                for (int e = 0; e < VEC; ++e)
-                                    sum[e] += __hip_atomic_load(part + (size_t)(c0 + j) * ldp + col0 + e, __ATOMIC_RELAXED,
-                                                                __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-                            for (int e = 0; e < VEC; ++e) agg[(size_t)slot * ldp + col0 + e] = sum[e];
-                        }
-                    }
-                }
-                if (lane == 0) __hip_atomic_store(hub_done + slot, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next pass over this plan
+                for (int u = 0; u < 8; ++u)
+                    if (j0 + u < nc) sum = V::add(sum, p[u]);
             }
+            V::store(agg + (size_t)slot * ldp + col0, sum);
         }
     }
 }
@@ -322,11 +328,18 @@ inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 template <int VEC, int ITERS>
 void launch_partial(hipStream_t s, const int* counts, int chunk_cap, int n, const int* row_ptr, const int* col_idx,
                     const float* val, const float* B, int ldb, int logG, const int* hub_row, const int* hub_chunk0,
-                    const int* chunk_hub, float* part, int ldp, float* agg, int* hub_done, int relu_in, int chunk_len)
+                    const int* chunk_hub, float* part, int ldp, float* agg, int hub_cap, int relu_in, int chunk_len)
 {
-    const unsigned grid = kNumCU * 8;
+    const unsigned grid = kNumCU * 32;
     hipLaunchKernelGGL((hub_partial_kernel<VEC, ITERS>), dim3(grid), dim3(kBlock), 0, s, counts, chunk_cap, n, row_ptr,
-                       col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in, chunk_len);
+                       col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, relu_in, chunk_len);
+    // the hubs of several chunks (few): a lane group each
+    const int groups = kBlock >> logG;
+    unsigned fgrid = (unsigned)((hub_cap + groups - 1) / groups);
+    if (fgrid > (unsigned)kNumCU * 4) fgrid = kNumCU * 4;
+    if (fgrid < 1) fgrid = 1;
+    hipLaunchKernelGGL((hub_finish_kernel<VEC, ITERS>), dim3(fgrid), dim3(kBlock), 0, s, counts, hub_cap, n, row_ptr, logG, hub_row,
+                       hub_chunk0, part, ldp, agg, chunk_len);
 }
 
 }  // namespace
@@ -378,7 +391,7 @@ size_t hub_scratch_bytes(int m, int n, long long nnz, int threshold, int chunk_l
 }
 
 // Sums the hubs of A (rows longer than `threshold` entries, cut into chunks of `chunk_len`) times B[:, 0..n) into
-// plan->agg.  max_hubs, when not negative, is the caller's bound on the number of such rows (it sizes the buffers).
+// plan->agg.  col_idx == nullptr: entry t is column t; val == nullptr: every weight is 1.  max_hubs, when not negative, is the caller's bound on the number of such rows (it sizes the buffers).
 // n <= 1024.  Without `store` the buffers live in the stream's scratch slot 1 and stay valid until the next
 // hub_prepass on the same stream; with it they live in a block the store's owner keeps (pool memory, grown when a
 // wider operand needs it), and the planning launches run only while store->planned is false.
@@ -460,13 +473,13 @@ int hub_prepass(int m, int n, long long nnz, const int* row_ptr, const int* col_
         if (store) store->planned = true;
     }
     if (vec4) {
-        if (iters <= 1) launch_partial<4, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
-        else if (iters == 2) launch_partial<4, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
-        else launch_partial<4, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
+        if (iters <= 1) launch_partial<4, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_cap, relu_in ? 1 : 0, chunk_len);
+        else if (iters == 2) launch_partial<4, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_cap, relu_in ? 1 : 0, chunk_len);
+        else launch_partial<4, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_cap, relu_in ? 1 : 0, chunk_len);
     } else {
-        if (iters <= 1) launch_partial<1, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
-        else if (iters == 2) launch_partial<1, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
-        else launch_partial<1, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_done, relu_in ? 1 : 0, chunk_len);
+        if (iters <= 1) launch_partial<1, 1>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_cap, relu_in ? 1 : 0, chunk_len);
+        else if (iters == 2) launch_partial<1, 2>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_cap, relu_in ? 1 : 0, chunk_len);
+        else launch_partial<1, 4>(s, counts, chunk_cap, n, row_ptr, col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, hub_cap, relu_in ? 1 : 0, chunk_len);
     }
     GNNHIP_LAUNCH_CHECK("hub_prepass");
     plan->row_slot = row_slot;

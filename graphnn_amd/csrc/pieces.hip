@@ -94,15 +94,11 @@ __global__ __launch_bounds__(kBlock) void piece_fill_kernel(int m, long long slo
 // target[i]: where the sum of the i-th piece in order goes: the row r >= 0 when the piece is all of that row,
 // else -1 - (its place among the partial sums; a stand-in piece without entries and without place gets a place past the
 // end, which the sum kernel recognises).  order[i] = id of the i-th piece in order; ordered[i] = its record.
-// where[j] = j and ones[j] = 1 for j < pslots: the matrix P that picks the partial sums of a row (the sums of a row's
-// pieces lie next to each other, so the combining pass reads them front to back).
 __global__ __launch_bounds__(kBlock) void piece_place_kernel(long long slots, long long pslots, const unsigned* __restrict__ order,
                                                              const PieceRec* __restrict__ rec, PieceRec* __restrict__ ordered,
-                                                             int* __restrict__ lens, int* __restrict__ where, float* __restrict__ ones,
-                                                             int* __restrict__ target)
+                                                             int* __restrict__ lens, int* __restrict__ target)
 {
     for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i <= slots; i += (long long)gridDim.x * kBlock) {
-        if (i < pslots) { where[i] = (int)i; ones[i] = 1.f; }
         if (i == slots) { lens[i] = 0; continue; }
         const PieceRec r = rec[order[i]];
         ordered[i] = r;
@@ -398,7 +394,7 @@ inline long long pslots_bound(long long nnz) { return nnz / kPiece + nnz / (kPie
 
 struct Layout {           // offsets inside the head, body and temporary blocks of a plan
     size_t o_first, o_pfirst, head_bytes;
-    size_t o_at, o_target, o_where, o_ones, o_col, o_val, body_bytes;
+    size_t o_at, o_target, o_col, o_val, body_bytes;
     size_t o_seg, o_rec, o_ord, o_keys, o_keys2, o_perm, o_perm2, o_hist, temp_bytes;
 };
 Layout layout_of(int m, long long nnz, long long slots, long long pslots)
@@ -412,8 +408,6 @@ Layout layout_of(int m, long long nnz, long long slots, long long pslots)
     off = 0;
     L.o_at = carve(sizeof(int) * ((size_t)slots + 1));
     L.o_target = carve(sizeof(int) * (size_t)slots);
-    L.o_where = carve(sizeof(int) * (size_t)pslots);
-    L.o_ones = carve(sizeof(float) * (size_t)pslots);
     L.o_col = carve(sizeof(int) * (size_t)nnz);
     L.o_val = carve(sizeof(float) * (size_t)nnz);
     L.body_bytes = off;
@@ -462,8 +456,7 @@ int order_pieces(CsrPlan* p, int cap, const Layout& L, char* temp, hipStream_t s
     // two stable passes, low digit first: order[i] = id of the piece that comes i-th by the top 16 bits of its first column
     if (int rc = radix_order_by_digit(keys, p->slots, 0, keys2, perm, hist, seg, s)) return rc;
     if (int rc = radix_order_by_digit(keys2, p->slots, 8, keys, order, hist, seg, s, perm)) return rc;
-    hipLaunchKernelGGL(piece_place_kernel, dim3(kElemGrid), dim3(kBlock), 0, s, p->slots, p->pslots, order, rec, ordered, p->at, p->where,
-                       p->ones, p->target);
+    hipLaunchKernelGGL(piece_place_kernel, dim3(kElemGrid), dim3(kBlock), 0, s, p->slots, p->pslots, order, rec, ordered, p->at, p->target);
     if (int rc = exclusive_scan_i32(p->at, p->slots + 1, seg, s)) return rc;
     hipLaunchKernelGGL(piece_gather_kernel, dim3(kElemGrid), dim3(kBlock), 0, s, p->first + p->m, ordered, p->at, p->col_idx, p->val,
                        p->col_ord, p->val_ord);
@@ -477,8 +470,6 @@ void point_plan(CsrPlan* p, const Layout& L, char* head, char* body)
     p->pfirst = reinterpret_cast<int*>(head + L.o_pfirst);
     p->at = reinterpret_cast<int*>(body + L.o_at);
     p->target = reinterpret_cast<int*>(body + L.o_target);
-    p->where = reinterpret_cast<int*>(body + L.o_where);
-    p->ones = reinterpret_cast<float*>(body + L.o_ones);
     p->col_ord = reinterpret_cast<int*>(body + L.o_col);
     p->val_ord = reinterpret_cast<float*>(body + L.o_val);
 }
@@ -524,11 +515,12 @@ int run_pieces(const CsrPlan* p, const Width& w, int n, float alpha, const float
 #undef GNNHIP_PIECES_TAIL
         GNNHIP_LAUNCH_CHECK("spmm_pieces tail");
     }
-    // the rows of very many pieces: the balanced pass over long rows, on P = (pfirst, where, ones) times part
+    // the rows of very many pieces: the balanced pass over long rows, on P times part (P: row pointers pfirst, entry j
+    // = column j with weight 1, which that pass takes when it is handed no index and value arrays)
     // (`pslots` stands in for the number of entries of P: an upper bound is all that pass needs; a row of more than
     // kCombineLong pieces has more than kCombineLong * kPiece entries, which bounds the number of such rows)
     HubPlan hubs;
-    if (int rc = hub_prepass(m, n, p->pslots, p->pfirst, p->where, p->ones, part, ldp, s, &hubs, hub_planned, false, kCombineLong,
+    if (int rc = hub_prepass(m, n, p->pslots, p->pfirst, nullptr, nullptr, part, ldp, s, &hubs, hub_planned, false, kCombineLong,
                              kCombineChunk, p->nnz / ((long long)kCombineLong * kPiece + 1) + 1, hub_store))
         return rc;
     const unsigned grid = (unsigned)(((long long)m + (long long)(kBlock >> logG) * kRun - 1) / ((long long)(kBlock >> logG) * kRun));
