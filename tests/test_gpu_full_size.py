@@ -1,10 +1,10 @@
-"""Checks at the full sizes of the named configurations: the whole device outputs of configurations 3 and 5 against
+"""Checks at the full sizes of the named configurations: the whole device outputs of configurations 3, 4 and 5 against
 the CPU oracle on the same seeded inputs, and properties that need no CPU run of the whole problem: exact row
 counts, linearity, independence of the graphs of a batch (a few graphs recomputed alone by the oracle), determinism."""
 import numpy as np
 import pytest
 
-from conftest import FLOOR_POOL, FLOOR_PROBS_ABS, PARITY_TOL, Lazy, assert_condition, assert_parity, condition_error, max_rel
+from conftest import FLOOR_POOL, FLOOR_PROBS_ABS, PARITY_TOL, Lazy, assert_condition, assert_parity, condition_error, forward_float64, max_rel
 from graphnn_amd import batching, synth
 
 pytestmark = pytest.mark.gpu
@@ -97,6 +97,36 @@ def test_forward_configuration_4_sampled_graphs(gpu, oracle):
         margin = abs(float(ref["logits"][0][0] - ref["logits"][0][1]))
         if margin > 1e-3 * scale:
             assert pred[gidx] == ref["pred"][0]
+
+
+def test_forward_configuration_4_whole_outputs_against_the_oracle(gpu, oracle):
+    """10,000 graphs, 299,536 nodes, hidden 256, 5 levels (the FP32 matrix-core level kernel, the tile readout): every
+    output of the whole batch against the CPU oracle's forward on the same seeded inputs (about ten seconds of CPU), with
+    the float64 model of the network behind it where two fp32 orders disagree, and its condition bound on every element"""
+    from graphnn_amd import ops
+    batch, w, cfg = synth.make_config(4)
+    a = batching.node2node_csr(batch.num_nodes, batch.edge_x, batch.edge_y)
+    s = batching.subgraph_csr(batch.num_graphs, batch.subg_id, batch.node_idx)
+    X = batch.one_hot()
+    L = cfg["L"]
+    bufs = ops.s2v_forward(tuple(_t(x, gpu) for x in a), tuple(_t(x, gpu) for x in s), _t(X, gpu), _t(w.W_n2l, gpu),
+                           _t(w.W_conv, gpu), _t(w.W_h1, gpu), _t(w.W_h2, gpu), L)
+    got = {"msg": bufs.msg, "h_final": bufs.h_b if bufs.which.value else bufs.h_a, "pool": bufs.pool, "hidden": bufs.hidden,
+           "logits": bufs.logits, "probs": bufs.probs}
+    got = {k: v.cpu().numpy() for k, v in got.items()}
+    pred = bufs.pred.cpu().numpy()
+    want = oracle.forward(a, s, X, w, L, None)
+    f64 = Lazy(lambda: forward_float64(a, s, X, w, L), Lazy(lambda: forward_float64(a, s, X, w, L, magnitudes=True)))
+    for key in ("msg", "h_final", "pool", "hidden", "logits", "probs"):
+        ref = want["h"][L] if key == "h_final" else want[key]
+        ref64 = f64["h"][L] if key == "h_final" else f64[key]
+        kw = {"floor_frac": FLOOR_POOL} if key == "pool" else {"floor": FLOOR_PROBS_ABS} if key == "probs" else {}
+        assert_parity("%s configuration 4" % key, got[key], ref, ref64, **kw)
+    # predictions: identical wherever the two logits are not a near tie
+    margin = np.abs(want["logits"][:, 0] - want["logits"][:, 1])
+    clear = margin > 1e-3 * np.abs(want["logits"]).max()
+    assert clear.mean() > 0.9
+    assert np.array_equal(pred[clear], want["pred"][clear])
 
 
 def test_skewed_configuration_5_whole_outputs_against_the_oracle(gpu, oracle):
