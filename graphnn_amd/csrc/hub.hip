@@ -330,13 +330,13 @@ void launch_partial(hipStream_t s, const int* counts, int chunk_cap, int n, cons
                     const float* val, const float* B, int ldb, int logG, const int* hub_row, const int* hub_chunk0,
                     const int* chunk_hub, float* part, int ldp, float* agg, int hub_cap, int relu_in, int chunk_len)
 {
-    const unsigned grid = kNumCU * 32;
+    const unsigned grid = kNumCU * 16;
     hipLaunchKernelGGL((hub_partial_kernel<VEC, ITERS>), dim3(grid), dim3(kBlock), 0, s, counts, chunk_cap, n, row_ptr,
                        col_idx, val, B, ldb, logG, hub_row, hub_chunk0, chunk_hub, part, ldp, agg, relu_in, chunk_len);
     // the hubs of several chunks (few): a lane group each
     const int groups = kBlock >> logG;
     unsigned fgrid = (unsigned)((hub_cap + groups - 1) / groups);
-    if (fgrid > (unsigned)kNumCU * 4) fgrid = kNumCU * 4;
+    if (fgrid > (unsigned)kNumCU) fgrid = kNumCU;
     if (fgrid < 1) fgrid = 1;
     hipLaunchKernelGGL((hub_finish_kernel<VEC, ITERS>), dim3(fgrid), dim3(kBlock), 0, s, counts, hub_cap, n, row_ptr, logG, hub_row,
                        hub_chunk0, part, ldp, agg, chunk_len);
