@@ -278,7 +278,7 @@ def time_level_cfg4(dev):
              "frac": flops2 / (ms2 * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS, "forward_ms": ms_fw2}
     return {"workload": "configuration 4: one level, %d nodes, %d entries, hidden %d" % (N, E, C),
             "variant_660k_undirected_edges": dense,
-            "kernel": "s2v_level_wide_kernel<256,8,false,64>", "avg_ms": ms, "flops": flops,
+            "kernel": "s2v_level_wide_kernel<256,8,false,64,false>", "avg_ms": ms, "flops": flops,
             "readout": {"avg_ms": ms_ro, "kernel": "s2v_readout_tile_kernel<256>", "graphs": B,
                         "algorithmic_GBps": (4.0 * N * C + 8.0 * N + 4.0 * B * (C + H + 2 * Q) + 4.0 * (C * H + H * Q)) / (ms_ro * 1e-3) / 1e9},
             "forward": {"avg_ms": ms_fw, "levels": L, "graphs_per_s": B / (ms_fw * 1e-3)},
