@@ -14,8 +14,11 @@
 #include <atomic>
 #include <map>
 #include <string.h>
+#include <functional>
 #include <mutex>
+#include <thread>
 #include <unordered_map>
+#include <vector>
 
 namespace gnnhip {
 
@@ -39,6 +42,15 @@ struct Staging {
     size_t used = 0;
 };
 
+// One pinned buffer per stream for the sparse form of a large upload (the positions and values of its non-zero words:
+// about half a byte per word of the tensor), sized to the largest one seen; reused once the kernel that read it has run.
+struct BigStaging {
+    char* base = nullptr;
+    size_t bytes = 0;
+    hipEvent_t done = nullptr;
+    bool pending = false;
+};
+
 struct Runtime {
     std::mutex mu;
     bool ready = false;
@@ -52,6 +64,7 @@ struct Runtime {
     std::map<std::pair<hipStream_t, int>, std::pair<void*, size_t>> scratch;   // library scratch per (stream, slot)
     std::map<hipStream_t, struct Staging> staging;  // pinned upload buffers per stream
     std::map<hipStream_t, void*> readback;          // pinned landing buffer for small device-to-host reads, per stream
+    std::map<hipStream_t, struct BigStaging> big_staging;
 };
 
 Runtime& rt()
@@ -256,6 +269,11 @@ int gnnhip_shutdown(void)
     r.staging.clear();
     for (auto& kv : r.readback) if (kv.second) (void)hipHostFree(kv.second);
     r.readback.clear();
+    for (auto& kv : r.big_staging) {
+        if (kv.second.base) (void)hipHostFree(kv.second.base);
+        if (kv.second.done) (void)hipEventDestroy(kv.second.done);
+    }
+    r.big_staging.clear();
     r.all.clear();
     r.live.clear();
     r.parked.clear();
@@ -413,6 +431,33 @@ __attribute__((target("avx2"))) bool collect_nonzero_avx2(const unsigned* w, siz
     return collect_nonzero(w, i, words, cap, idx, val, count, starts);
 }
 
+// Words [from, to) only (from a multiple of the tile size), for one of several threads that share a large tensor: positions
+// are absolute, *count and the starts are relative to this thread's own idx / val region.
+__attribute__((target("avx2"))) bool collect_range_avx2(const unsigned* w, size_t from, size_t to, size_t cap, unsigned* idx, unsigned* val,
+                                                        size_t* count, unsigned* starts)
+{
+    size_t c = 0, i = from;
+    const __m256i zero = _mm256_setzero_si256();
+#define GNNHIP_ZEROS_OF(at) \
+    ((unsigned)_mm256_movemask_ps(_mm256_castsi256_ps(_mm256_cmpeq_epi32(_mm256_loadu_si256(reinterpret_cast<const __m256i*>(w + (at))), zero))))
+    for (; i + 32 <= to; i += 32) {
+        if ((i & (kExpandTile - 1)) == 0) starts[i / kExpandTile] = (unsigned)c;
+        unsigned nz = ~(GNNHIP_ZEROS_OF(i) | (GNNHIP_ZEROS_OF(i + 8) << 8) | (GNNHIP_ZEROS_OF(i + 16) << 16) | (GNNHIP_ZEROS_OF(i + 24) << 24));
+        if (!nz) continue;
+        if (c + (size_t)__builtin_popcount(nz) > cap) return false;
+        while (nz) {
+            const unsigned j = (unsigned)__builtin_ctz(nz);
+            nz &= nz - 1;
+            idx[c] = (unsigned)(i + j);
+            val[c] = w[i + j];
+            ++c;
+        }
+    }
+#undef GNNHIP_ZEROS_OF
+    *count = c;
+    return collect_nonzero(w, i, to, cap, idx, val, count, starts);
+}
+
 // A staged upload leaves the pinned buffer through a kernel, not through hipMemcpyAsync: the runtime hands copies of
 // this size to a DMA engine, and the kernel that consumes the data then waits for that engine's completion signal to
 // cross over to the compute queue, 15 to 20 us per copy on an otherwise idle device.  A kernel of the stream's own
@@ -505,6 +550,99 @@ int stage_in_pinned(hipStream_t s, const void* src_host, size_t bytes, const voi
 
 }  // namespace gnnhip
 
+namespace {
+
+// dst_device[0, words) = w[0, words) for a tensor past the staging halves (the dense one-hot feature matrix of a batch of
+// ten thousand graphs is 77 MB): the scan for non-zero words is cut into tile-aligned ranges, one per thread, each
+// thread collecting into its own part of the pinned buffer; the parts are then pushed together and one kernel rebuilds
+// the tensor.  GNNHIP_EUNSUPPORTED (nothing queued) when more than one word in sixteen of some range is non-zero or no
+// pinned memory is to be had: the caller copies the tensor as it is.
+int sparse_upload_large(void* dst_device, const unsigned* w, size_t words, hipStream_t s)
+{
+    const size_t tiles = (words + kExpandTile - 1) / kExpandTile;
+    const size_t cap = words / 16;
+    const size_t bytes = cap * 8 + (tiles + 1) * 4;
+    char* base = nullptr;
+    hipEvent_t done = nullptr;
+    {
+        Runtime& r = rt();
+        std::lock_guard<std::mutex> lock(r.mu);
+        BigStaging& st = r.big_staging[s];
+        if (st.pending) {                          // the kernel of the previous large upload still reads the buffer
+            GNNHIP_HIP(hipEventSynchronize(st.done));
+            st.pending = false;
+        }
+        if (st.bytes < bytes) {
+            if (st.base) (void)hipHostFree(st.base);
+            st.base = nullptr;
+            st.bytes = 0;
+            void* q = nullptr;
+            if (hipHostMalloc(&q, bytes, hipHostMallocDefault) != hipSuccess || !q) {
+                (void)hipGetLastError();
+                return GNNHIP_EUNSUPPORTED;
+            }
+            st.base = static_cast<char*>(q);
+            st.bytes = bytes;
+        }
+        if (!st.done) GNNHIP_HIP(hipEventCreateWithFlags(&st.done, hipEventDisableTiming));
+        base = st.base;
+        done = st.done;
+    }
+    // one host thread at a time feeds a stream: the buffer is this call's from here on
+    unsigned* idx = reinterpret_cast<unsigned*>(base);
+    unsigned* val = idx + cap;
+    unsigned* starts = val + cap;
+    const bool avx2 = __builtin_cpu_supports("avx2");
+    unsigned hw = std::thread::hardware_concurrency();
+    size_t nthreads = hw >= 16 ? 8 : hw >= 4 ? hw / 2 : 1;
+    const size_t per_min = (size_t)1 << 20;        // a thread is worth starting for a million words
+    if (nthreads > (words + per_min - 1) / per_min) nthreads = (words + per_min - 1) / per_min;
+    if (nthreads < 1) nthreads = 1;
+    const size_t tiles_per = (tiles + nthreads - 1) / nthreads;
+    struct Part { size_t t0, t1, off, count; bool ok; };
+    std::vector<Part> parts;
+    for (size_t t0 = 0; t0 < tiles; t0 += tiles_per) {
+        const size_t t1 = t0 + tiles_per < tiles ? t0 + tiles_per : tiles;
+        parts.push_back(Part{t0, t1, t0 * kExpandTile / 16, 0, true});      // its share of cap starts where its words do, over 16
+    }
+    auto scan = [&](Part& p) {
+        const size_t from = p.t0 * kExpandTile, to = p.t1 * kExpandTile < words ? p.t1 * kExpandTile : words;
+        const size_t room = (to - from) / 16;
+        p.ok = avx2 ? collect_range_avx2(w, from, to, room, idx + p.off, val + p.off, &p.count, starts)
+                    : collect_nonzero(w, from, to, room, idx + p.off, val + p.off, &(p.count = 0), starts);
+    };
+    {
+        std::vector<std::thread> workers;
+        for (size_t i = 1; i < parts.size(); ++i) workers.emplace_back(scan, std::ref(parts[i]));
+        scan(parts[0]);
+        for (auto& t : workers) t.join();
+    }
+    size_t total = 0;
+    for (Part& p : parts) {
+        if (!p.ok) return GNNHIP_EUNSUPPORTED;
+        if (p.off != total) {                      // push the part up against the one before it (it only ever moves down)
+            memmove(idx + total, idx + p.off, p.count * sizeof(unsigned));
+            memmove(val + total, val + p.off, p.count * sizeof(unsigned));
+        }
+        if (total)                                 // the part's tile starts were counted from its own first entry
+            for (size_t t = p.t0; t < p.t1; ++t) starts[t] += (unsigned)total;
+        total += p.count;
+    }
+    starts[tiles] = (unsigned)total;
+    hipLaunchKernelGGL(expand_pairs_kernel, dim3((unsigned)tiles), dim3(kExpandBlock), 0, s, static_cast<unsigned*>(dst_device), words,
+                       starts, idx, val);
+    GNNHIP_LAUNCH_CHECK("expand_pairs (large)");
+    GNNHIP_HIP(hipEventRecord(done, s));
+    {
+        Runtime& r = rt();
+        std::lock_guard<std::mutex> lock(r.mu);
+        r.big_staging[s].pending = true;
+    }
+    return GNNHIP_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream)
@@ -585,11 +723,15 @@ int gnnhip_memcpy_h2d_sparse32(void* dst_device, const void* src_host, size_t wo
     constexpr size_t kMinWords = 16384;                  // below this the plain copy is one short DMA anyway
     const size_t cap = words / 16;                       // non-zero words beyond this: the plain copy
     const size_t tiles = (words + kExpandTile - 1) / kExpandTile;
-    if (words < kMinWords || cap * 8 + (tiles + 1) * 4 > kStagingHalf || words >= ((size_t)1 << 32))
-        return gnnhip_memcpy_h2d(dst_device, src_host, words * 4, stream);
+    if (words < kMinWords || words >= ((size_t)1 << 32)) return gnnhip_memcpy_h2d(dst_device, src_host, words * 4, stream);
     GNNHIP_REQUIRE(dst_device && src_host, "null pointer in memcpy_h2d_sparse32");
     if (int rc = require_ready()) return rc;
     hipStream_t s = as_stream(stream);
+    if (cap * 8 + (tiles + 1) * 4 > kStagingHalf) {
+        // too large for the staging halves: a pinned buffer of its own, the scan shared by a few threads
+        if (int rc = sparse_upload_large(dst_device, static_cast<const unsigned*>(src_host), words, s); rc != GNNHIP_EUNSUPPORTED) return rc;
+        return gnnhip_memcpy_h2d(dst_device, src_host, words * 4, stream);
+    }
     char* slot = nullptr;
     {
         Runtime& r = rt();
