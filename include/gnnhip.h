@@ -78,7 +78,9 @@ int gnnhip_release_scratch(void* stream);
  *      host memory; d2d and memset0 are asynchronous on the stream.
  *      h2d_sparse32 is h2d for `words` 32-bit words that are mostly zero (the one-hot feature matrix GetBatch
  *      fills, examples/graph_classification/include/nn_common.h:60-75): it sends the non-zero words with their
- *      positions and rebuilds the buffer on the device (same bits, same promise); dense data takes the plain copy. */
+ *      positions and rebuilds the buffer on the device (same bits, same promise); dense data takes the plain copy.
+ *      From about four million words on the scan for non-zero words is shared by up to eight host threads, started and
+ *      joined inside the call. */
 int gnnhip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream);
 int gnnhip_memcpy_h2d_sparse32(void* dst_device, const void* src_host, size_t words, void* stream);
 int gnnhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
