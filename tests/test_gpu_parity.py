@@ -1659,6 +1659,38 @@ def test_plan_of_matrices_that_take_the_other_routes(gpu, oracle):
         assert plan.spmm(_t(np.ones((5, 3), np.float32), gpu)).shape == (0, 3)
 
 
+def test_plans_give_their_memory_back(gpu):
+    """plans of a power-law matrix made, used at two widths (the partial sums and the balanced pass grow with the width) and
+    destroyed, several times over: the pool holds what it held before, and the bytes a plan reports are what it took"""
+    import ctypes
+    from graphnn_amd import ops
+    lib = ops._lib()
+    rng = np.random.default_rng(77)
+    a = synth.rmat_csr(0x5EED0005, 16, 16 << 16)
+    N = 1 << 16
+    csr_d = _csr_t((a[0], a[1], np.ones(a[1].size, np.float32)), gpu)
+    B32, B128 = _t(rng.standard_normal((N, 32)).astype(np.float32), gpu), _t(rng.standard_normal((N, 128)).astype(np.float32), gpu)
+    def in_use():
+        z = [ctypes.c_size_t() for _ in range(3)]
+        ops.check(lib.gnnhip_pool_stats(*[ctypes.byref(c) for c in z]))
+        return z[0].value
+    import torch
+    torch.cuda.synchronize()
+    before = in_use()
+    first = None
+    for _ in range(4):
+        with ops.CsrPlan(*csr_d, N, N) as plan:
+            held = plan.bytes()
+            assert in_use() - before == held
+            got = plan.spmm(B32)
+            got128 = plan.spmm(B128)
+            assert plan.bytes() > held and in_use() - before == plan.bytes()
+            if first is None:
+                first = (got.clone(), got128.clone())
+            assert torch.equal(got, first[0]) and torch.equal(got128, first[1])
+        assert in_use() == before
+
+
 @pytest.mark.parametrize("C", [16, 32, 64, 128])
 def test_level_on_a_power_law_graph_leaves_no_trace_of_the_output_buffer(gpu, oracle, C):
     """the two-launch level on the R-MAT matrix (a third of its rows empty): the product skips the rows without
