@@ -168,11 +168,23 @@ __global__ __launch_bounds__(WAVES * kWave) void s2v_level_wide_kernel(
     {
         const rsrc_t w_rsrc = make_rsrc(W, (unsigned)(C * C * 4));
         const int w_lane_off = BWD ? ((col0 + t) * C + KS * q) * 4 : ((KS * q) * C + col0 + t) * 4;
+        if constexpr (BWD) {
+            // a lane's steps are consecutive floats of one row of W: 128-bit loads (with one float per load, lanes
+            // 1 KB apart, the start-up of a launch on 7,450 rows took longer than its passes)
 #pragma unroll
-        for (int jb = 0; jb < NB; ++jb)
+            for (int jb = 0; jb < NB; ++jb)
 #pragma unroll
-            for (int s = 0; s < KS; ++s)
-                wreg[jb][s] = buf_load_f(w_rsrc, w_lane_off + (BWD ? 16 * C * 4 : 64) * jb, s * (BWD ? 4 : C * 4));
+                for (int s4 = 0; s4 < KS / 4; ++s4) {
+                    const float4 v = buf_load4(w_rsrc, w_lane_off + 16 * C * 4 * jb, s4 * 16);
+                    wreg[jb][4 * s4 + 0] = v.x; wreg[jb][4 * s4 + 1] = v.y; wreg[jb][4 * s4 + 2] = v.z; wreg[jb][4 * s4 + 3] = v.w;
+                }
+        } else {
+#pragma unroll
+            for (int jb = 0; jb < NB; ++jb)
+#pragma unroll
+                for (int s = 0; s < KS; ++s)
+                    wreg[jb][s] = buf_load_f(w_rsrc, w_lane_off + 64 * jb, s * (C * 4));
+        }
     }
 
     const int ntiles = (int)(((long long)N + kTileRows - 1) / kTileRows);
