@@ -137,20 +137,31 @@ __global__ __launch_bounds__(kBlock, MINW) void s2v_level_stream_kernel(
                 const int col = KS * (t >> 2) + 4 * jb + (t & 3);
                 const int k0 = KS * q + 4 * s4;
                 // element (k, col) of the operand: W[k][col], or W[col][k] when the level runs backward
-                w4.x = BWD ? W[(size_t)col * C + k0 + 0] : W[(size_t)(k0 + 0) * C + col];
-                w4.y = BWD ? W[(size_t)col * C + k0 + 1] : W[(size_t)(k0 + 1) * C + col];
-                w4.z = BWD ? W[(size_t)col * C + k0 + 2] : W[(size_t)(k0 + 2) * C + col];
-                w4.w = BWD ? W[(size_t)col * C + k0 + 3] : W[(size_t)(k0 + 3) * C + col];
+                if constexpr (BWD) {
+                    w4 = *reinterpret_cast<const float4*>(W + (size_t)col * C + k0);     // four steps: consecutive floats of a row (W is 16-byte aligned, host-checked)
+                } else {
+                    w4.x = W[(size_t)(k0 + 0) * C + col];
+                    w4.y = W[(size_t)(k0 + 1) * C + col];
+                    w4.z = W[(size_t)(k0 + 2) * C + col];
+                    w4.w = W[(size_t)(k0 + 3) * C + col];
+                }
                 wl[(jb * (KS / 4) + s4) * kWave + lane] = w4;
             }
         __syncthreads();
     } else {
 #pragma unroll
-        for (int jb = 0; jb < NJB; ++jb)
+        for (int jb = 0; jb < NJB; ++jb) {
+            if constexpr (BWD) {
 #pragma unroll
-            for (int s = 0; s < KS; ++s)
-                wreg[jb][s] = BWD ? W[(size_t)(KS * (t >> 2) + 4 * jb + (t & 3)) * C + KS * q + s]
-                                  : W[(size_t)(KS * q + s) * C + KS * (t >> 2) + 4 * jb + (t & 3)];
+                for (int s4 = 0; s4 < KS / 4; ++s4) {
+                    const float4 v = *reinterpret_cast<const float4*>(W + (size_t)(KS * (t >> 2) + 4 * jb + (t & 3)) * C + KS * q + 4 * s4);
+                    wreg[jb][4 * s4 + 0] = v.x; wreg[jb][4 * s4 + 1] = v.y; wreg[jb][4 * s4 + 2] = v.z; wreg[jb][4 * s4 + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int s = 0; s < KS; ++s) wreg[jb][s] = W[(size_t)(KS * q + s) * C + KS * (t >> 2) + 4 * jb + (t & 3)];
+            }
+        }
     }
 
     int E = 0;
